@@ -1,0 +1,210 @@
+"""Deterministic synthetic structures, model parameters and labels for the benchmark
+configurations and the parity tests.
+
+Random numbers come from a counter-based generator written here (SplitMix64 finaliser over
+``seed * 2**32 + counter``), so the same seed gives the same structure on any NumPy version
+and on any machine.  Nothing here touches the GPU.
+"""
+import math
+
+import numpy as np
+
+_M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def _mix(x):
+    """SplitMix64 output function on a uint64 array (wrapping arithmetic)."""
+    with np.errstate(over="ignore"):
+        x = (x + np.uint64(0x9E3779B97F4A7C15)) & _M64
+        x = ((x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)) & _M64
+        x = ((x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)) & _M64
+        return x ^ (x >> np.uint64(31))
+
+
+def rng_bits(seed, n, offset=0):
+    with np.errstate(over="ignore"):
+        ctr = np.arange(offset, offset + n, dtype=np.uint64)
+        return _mix(_mix(np.uint64(seed) * np.uint64(0x100000001B3) + np.uint64(0x51ED27)) ^ ctr)
+
+
+def rng_uniform(seed, n, lo=0.0, hi=1.0, offset=0):
+    """n doubles uniform in [lo, hi)."""
+    u = (rng_bits(seed, n, offset) >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+    return lo + (hi - lo) * u
+
+
+def rng_normal(seed, n, mean=0.0, sigma=1.0, offset=0):
+    """n doubles from N(mean, sigma^2) by Box-Muller on two uniform streams."""
+    u1 = rng_uniform(seed, n, offset=2 * offset)
+    u2 = rng_uniform(seed ^ 0x5DEECE66D, n, offset=2 * offset)
+    r = np.sqrt(-2.0 * np.log(1.0 - u1))
+    return mean + sigma * r * np.cos(2.0 * math.pi * u2)
+
+
+def rng_randint(seed, n, k, offset=0):
+    return (rng_bits(seed, n, offset) % np.uint64(k)).astype(np.int32)
+
+
+# ----------------------------------------------------------------------------------------
+# structures
+# ----------------------------------------------------------------------------------------
+def mos2_fixture():
+    """The 12-atom MoS2 cell the reference's unit tests use
+    (source/descriptor/nep/tests/test_nep.cc:100-158): lattice rows, type indices (0 = Mo,
+    1 = S), fractional coordinates."""
+    lattice = np.array([[3.1903157348, 5.5257885468, 0.0],
+                        [-6.3806307800, 0.0, 0.0],
+                        [0.0, 0.0, 23.1297687334]])
+    types = np.array([0, 1, 1] * 4, np.int32)
+    z = (0.500000000000, 0.432343276548, 0.567656723452)
+    frac = []
+    for mo, s in (((0.333333333333, 0.166666666667), (0.166666666667, 0.333333333333)),
+                  ((0.333333333333, 0.666666666667), (0.166666666667, 0.833333333333)),
+                  ((0.833333333333, 0.166666666667), (0.666666666667, 0.333333333333)),
+                  ((0.833333333333, 0.666666666667), (0.666666666667, 0.833333333333))):
+        frac += [[mo[0], mo[1], z[0]], [s[0], s[1], z[1]], [s[0], s[1], z[2]]]
+    return lattice, types, np.array(frac)
+
+
+def diamond_cell(reps=3, a=5.43, sigma=0.1, seed=1002):
+    """Config 1: reps^3 conventional diamond cells, Gaussian displacements, wrapped."""
+    base = np.array([[0, 0, 0], [0, .5, .5], [.5, 0, .5], [.5, .5, 0],
+                     [.25, .25, .25], [.25, .75, .75], [.75, .25, .75], [.75, .75, .25]])
+    cells = np.array([[i, j, k] for i in range(reps) for j in range(reps) for k in range(reps)], float)
+    pos = (cells[:, None, :] + base[None, :, :]).reshape(-1, 3) * a
+    L = reps * a
+    pos = pos + rng_normal(seed, pos.size, 0.0, sigma).reshape(-1, 3)
+    pos = np.mod(pos, L)
+    return np.eye(3) * L, pos
+
+
+def random_packed(n, box, dmin, seed):
+    """n points in an orthorhombic periodic box by sequential rejection sampling with a
+    minimum-image distance of at least dmin (cell-list accelerated)."""
+    box = np.asarray(box, float)
+    ncell = np.maximum((box / dmin).astype(int), 1)
+    csize = box / ncell
+    grid = {}
+    pos = np.zeros((n, 3))
+    placed = 0
+    drawn = 0
+    chunk = 4096
+    d2min = dmin * dmin
+    while placed < n:
+        cand = rng_uniform(seed, 3 * chunk, offset=drawn).reshape(chunk, 3) * box
+        drawn += 3 * chunk
+        for p in cand:
+            c = np.minimum((p / csize).astype(int), ncell - 1)
+            ok = True
+            for dx in (-1, 0, 1):
+                for dy in (-1, 0, 1):
+                    for dz in (-1, 0, 1):
+                        key = ((c[0] + dx) % ncell[0], (c[1] + dy) % ncell[1], (c[2] + dz) % ncell[2])
+                        for q in grid.get(key, ()):
+                            d = p - pos[q]
+                            d -= box * np.round(d / box)
+                            if d[0] * d[0] + d[1] * d[1] + d[2] * d[2] < d2min:
+                                ok = False
+                                break
+                        if not ok:
+                            break
+                    if not ok:
+                        break
+                if not ok:
+                    break
+            if ok:
+                pos[placed] = p
+                grid.setdefault((c[0], c[1], c[2]), []).append(placed)
+                placed += 1
+                if placed == n:
+                    break
+    return np.diag(box), pos
+
+
+def fcc_cell(reps, a, sigma, seed):
+    """Config 5: reps^3 conventional FCC cells (4 atoms each) with Gaussian jitter, wrapped.
+    Atoms are ordered cell by cell (x outer, z inner), so neighbours are close in memory."""
+    base = np.array([[0, 0, 0], [0, .5, .5], [.5, 0, .5], [.5, .5, 0]])
+    r = np.arange(reps, dtype=np.float64)
+    cx, cy, cz = np.meshgrid(r, r, r, indexing="ij")
+    cells = np.stack([cx.ravel(), cy.ravel(), cz.ravel()], axis=1)
+    pos = (cells[:, None, :] + base[None, :, :]).reshape(-1, 3) * a
+    L = reps * a
+    pos = pos + rng_normal(seed, pos.size, 0.0, sigma).reshape(-1, 3)
+    pos = np.mod(pos, L)
+    return np.eye(3) * L, pos
+
+
+# ----------------------------------------------------------------------------------------
+# model parameters
+# ----------------------------------------------------------------------------------------
+def nep_model(ntypes=3, n_radial_basis=6, n_angular_basis=4, l_max=4, chebyshev_size=8,
+              num_neurons=50, rmax_radial=7.0, rmax_angular=4.0, seed=3002, sigma=0.1,
+              type_map=(32, 51, 52)):
+    D = n_radial_basis + n_angular_basis * l_max
+    ncoef = ntypes * ntypes * (n_radial_basis + n_angular_basis) * chebyshev_size
+    return dict(chebyshev_size=chebyshev_size, n_radial_basis=n_radial_basis,
+                n_angular_basis=n_angular_basis, l_max=l_max, rmax_radial=rmax_radial,
+                rmax_angular=rmax_angular,
+                coeffs=rng_normal(seed, ncoef, 0, sigma),
+                w0=rng_normal(seed + 1, ntypes * num_neurons * D, 0, sigma),
+                b0=rng_normal(seed + 2, ntypes * num_neurons, 0, sigma),
+                w1=rng_normal(seed + 3, ntypes * num_neurons, 0, sigma),
+                type_bias=rng_normal(seed + 4, ntypes, 0, sigma),
+                q_scaler=np.ones(D), type_map=np.array(type_map[:ntypes], np.int32))
+
+
+def nep_model_closed_form():
+    """Parameter fill of the reference's NEP unit test
+    (source/descriptor/nep/tests/test_nep.cc:197-255), for the MoS2 known answer."""
+    ntypes, H, n_r, n_a, l_max, K = 2, 30, 6, 4, 3, 8
+    D = n_r + n_a * l_max
+    return dict(chebyshev_size=K, n_radial_basis=n_r, n_angular_basis=n_a, l_max=l_max,
+                rmax_radial=5.0, rmax_angular=4.0,
+                coeffs=0.01 + 0.001 * np.arange(ntypes * ntypes * (n_r + n_a) * K),
+                w0=0.1 + 0.001 * np.arange(ntypes * H * D),
+                b0=0.1 + 0.001 * np.arange(ntypes * H),
+                w1=0.1 + 0.001 * np.arange(ntypes * H),
+                type_bias=np.array([-0.1, -0.2]),
+                q_scaler=0.67 + 0.05 * np.arange(D), type_map=np.array([42, 16], np.int32))
+
+
+def mtp_model(tables, ntypes, chebyshev_size, rmax, rmin, seed, lo=-0.1, hi=0.1, type_map=None):
+    """Linear-MTP parameters drawn uniformly in [lo, hi); `tables` is the dict returned by
+    ai2pot_amd.mtp_param.mtp_param(level)."""
+    nmus = tables["nmus"]
+    S = len(tables["alpha_moment_mapping"])
+    ncoef = ntypes * ntypes * nmus * chebyshev_size
+    m = dict(tables)
+    m.update(chebyshev_size=chebyshev_size, scaling=1.0, rmax=rmax, rmin=rmin,
+             coeffs=rng_uniform(seed, ncoef, lo, hi),
+             linear_coeffs=rng_uniform(seed + 1, S, lo, hi),
+             type_bias=rng_uniform(seed + 2, ntypes, lo, hi),
+             q_scaler=np.ones(S),
+             type_map=np.array(type_map if type_map is not None else range(1, ntypes + 1), np.int32))
+    return m
+
+
+# ----------------------------------------------------------------------------------------
+# batching (the 7-tensor contract of the E/F/V operators)
+# ----------------------------------------------------------------------------------------
+def pack_batch(lists, natoms_pad=None):
+    """Stack per-structure neighbor-list tuples (inum, ilist, numneigh, firstneigh, rcs,
+    types, nghost) into the padded batch the operators take.  Rows of atoms beyond inum
+    are zero-filled, as the reference's dataset code does."""
+    B = len(lists)
+    P = natoms_pad or max(l[0] for l in lists)
+    U = lists[0][3].shape[1]
+    dt = lists[0][4].dtype
+    nb = dict(binum=np.zeros(B, np.int32), bilist=np.zeros((B, P), np.int32),
+              bnumneigh=np.zeros((B, P), np.int32), bfirstneigh=np.zeros((B, P, U), np.int32),
+              brcs=np.zeros((B, P, U, 3), dt), btypes=np.zeros((B, P), np.int32), nghost=0)
+    for b, (inum, ilist, numneigh, firstneigh, rcs, types, nghost) in enumerate(lists):
+        assert nghost == 0
+        nb["binum"][b] = inum
+        nb["bilist"][b, :inum] = ilist
+        nb["bnumneigh"][b, :inum] = numneigh
+        nb["bfirstneigh"][b, :inum] = firstneigh
+        nb["brcs"][b, :inum] = rcs
+        nb["btypes"][b, :inum] = types
+    return nb

@@ -1,0 +1,333 @@
+"""CPU checkers for the energy / force / virial hot path.  TEST INFRASTRUCTURE ONLY.
+
+Only the tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
+may import this package; the product (``ai2pot_amd``) never does.
+
+Two families of functions with identical NumPy signatures:
+
+* ``nblist``, ``nep_efv``, ``mtp_efv``, ``mtp_loss_step``, ``fvt_force``, ``fvt_virial`` --
+  this repository's own C++ restatement of the reference algorithm (``oracle/src``,
+  ``liboracle.so``), each function citing the reference file:line it follows;
+* ``ref_*`` -- the reference's own headers compiled where they lie (``oracle/_ref/*.so``,
+  built by ``oracle/Makefile`` when the reference tree is present).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_C = ctypes
+_libs = {}
+
+
+def build(ref=True):
+    """Compile liboracle.so and, when the reference tree is present, oracle/_ref."""
+    subprocess.check_call(["make", "-s", "-C", _HERE, "oracle"])
+    if ref:
+        subprocess.check_call(["make", "-s", "-C", _HERE, "ref"])
+
+
+def _load(name):
+    if name in _libs:
+        return _libs[name]
+    path = os.path.join(_HERE, name)
+    lib = _C.CDLL(path) if os.path.exists(path) else None
+    _libs[name] = lib
+    return lib
+
+
+def oracle_lib():
+    lib = _load("liboracle.so")
+    if lib is None:
+        build(ref=False)
+        _libs.pop("liboracle.so")
+        lib = _load("liboracle.so")
+    return lib
+
+
+def ref_available(which="nep"):
+    return _load("_ref/libref_%s.so" % which) is not None
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_C.c_void_p)
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+_I = _C.c_int
+_D = _C.c_double
+
+
+# ----------------------------------------------------------------------------------------
+# neighbor list
+# ----------------------------------------------------------------------------------------
+def _nblist(lib, prefix, lattice, types, coords, rcut, umax, is_cart, pbc, sort):
+    coords = np.ascontiguousarray(coords)
+    dt = coords.dtype
+    assert dt in (np.float32, np.float64)
+    suffix = "f32" if dt == np.float32 else "f64"
+    lattice = _c(lattice, dt).reshape(9)
+    types = _c(types, np.int32)
+    n = coords.shape[0]
+    pbc_i = _c([int(bool(x)) for x in pbc], np.int32)
+    ilist = np.zeros(n, np.int32)
+    numneigh = np.zeros(n, np.int32)
+    firstneigh = np.zeros((n, umax), np.int32)
+    rcs = np.zeros((n, umax, 3), dt)
+    types_out = np.zeros(n, np.int32)
+    max_nn = _I(0)
+    fn = getattr(lib, "%s_%s" % (prefix, suffix))
+    fn.restype = _I
+    rc = fn(_p(lattice), _p(types), _p(coords), _I(n), _D(float(rcut)), _I(umax), _I(int(is_cart)),
+            _p(pbc_i), _I(int(sort)), _p(ilist), _p(numneigh), _p(firstneigh), _p(rcs),
+            _p(types_out), _C.byref(max_nn))
+    if rc != 0:
+        raise RuntimeError("neighbor count %d exceeds umax_num_neigh_atoms %d" % (max_nn.value, umax))
+    return n, ilist, numneigh, firstneigh, rcs, types_out, 0
+
+
+def ref_nblist(lattice, types, coords, rcut, umax, is_cart=True, pbc=(True, True, True), sort=False):
+    return _nblist(_load("_ref/libref_nblist.so"), "ref_nblist", lattice, types, coords, rcut, umax,
+                   is_cart, pbc, sort)
+
+
+def nblist(lattice, types, coords, rcut, umax, is_cart=True, pbc=(True, True, True), sort=False):
+    return _nblist(oracle_lib(), "orc_nblist", lattice, types, coords, rcut, umax, is_cart, pbc, sort)
+
+
+# ----------------------------------------------------------------------------------------
+# shared unpacking of the 7-tensor neighbor batch
+# ----------------------------------------------------------------------------------------
+def _batch(nb, dt):
+    binum = _c(nb["binum"], np.int32)
+    bilist = _c(nb["bilist"], np.int32)
+    bnumneigh = _c(nb["bnumneigh"], np.int32)
+    bfirst = _c(nb["bfirstneigh"], np.int32)
+    brcs = _c(nb["brcs"], dt)
+    btypes = _c(nb["btypes"], np.int32)
+    nghost = int(nb.get("nghost", 0))
+    B, P = bilist.shape
+    U = bfirst.shape[2]
+    assert brcs.shape == (B, P, U, 3) and btypes.shape == (B, P + nghost)
+    return binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U
+
+
+# ----------------------------------------------------------------------------------------
+# NEP
+# ----------------------------------------------------------------------------------------
+def _nep_efv(lib, prefix, model, nb, dtype):
+    dt = np.dtype(dtype)
+    suffix = "f32" if dt == np.float32 else "f64"
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, dt)
+    coeffs = _c(model["coeffs"], dt)
+    w0 = _c(model["w0"], dt)
+    b0 = _c(model["b0"], dt)
+    w1 = _c(model["w1"], dt)
+    bias = _c(model["type_bias"], dt)
+    q_scaler = _c(model["q_scaler"], dt)
+    type_map = _c(model["type_map"], np.int32)
+    ntypes = type_map.size
+    H = w1.size // ntypes
+    e = np.zeros(B, dt)
+    f = np.zeros((B, P + nghost, 3), dt)
+    v = np.zeros((B, 9), dt)
+    fn = getattr(lib, "%s_efv_%s" % (prefix, suffix))
+    fn.restype = None
+    fn(_p(e), _p(f), _p(v), _I(model["chebyshev_size"]), _I(model["n_radial_basis"]),
+       _I(model["n_angular_basis"]), _I(model["l_max"]), _I(H), _p(coeffs), _p(w0), _p(b0), _p(w1),
+       _p(bias), _I(B), _I(P), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs),
+       _p(btypes), _I(ntypes), _p(type_map), _I(U), _I(nghost), _D(model["rmax_radial"]),
+       _D(model["rmax_angular"]), _p(q_scaler))
+    return e, f, v
+
+
+def _nep_desc(lib, prefix, model, nb, dtype):
+    dt = np.dtype(dtype)
+    suffix = "f32" if dt == np.float32 else "f64"
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, dt)
+    assert nghost == 0
+    coeffs = _c(model["coeffs"], dt)
+    type_map = _c(model["type_map"], np.int32)
+    n_r, n_a, l_max = model["n_radial_basis"], model["n_angular_basis"], model["l_max"]
+    D = n_r + n_a * l_max
+    d = np.zeros((B, P, D), dt)
+    fn = getattr(lib, "%s_desc_%s" % (prefix, suffix))
+    fn.restype = None
+    fn(_p(d), _I(model["chebyshev_size"]), _I(n_r), _I(n_a), _I(l_max), _p(coeffs), _I(B), _I(P),
+       _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes), _I(type_map.size),
+       _p(type_map), _I(U), _I(nghost), _D(model["rmax_radial"]), _D(model["rmax_angular"]))
+    return d
+
+
+def ref_nep_efv(model, nb, dtype=np.float64):
+    return _nep_efv(_load("_ref/libref_nep.so"), "ref_nep", model, nb, dtype)
+
+
+def nep_efv(model, nb, dtype=np.float64):
+    return _nep_efv(oracle_lib(), "orc_nep", model, nb, dtype)
+
+
+def ref_nep_descriptors(model, nb, dtype=np.float64):
+    return _nep_desc(_load("_ref/libref_nep.so"), "ref_nep", model, nb, dtype)
+
+
+def nep_descriptors(model, nb, dtype=np.float64):
+    return _nep_desc(oracle_lib(), "orc_nep", model, nb, dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# linear MTP
+# ----------------------------------------------------------------------------------------
+def ref_mtp_param(level, ai2pot_path="/root/reference"):
+    """Contraction tables of one level, parsed by the reference's own MtpParam."""
+    lib = _load("_ref/libref_mtpr.so")
+    saved = os.environ.get("AI2POT_PATH")
+    os.environ["AI2POT_PATH"] = ai2pot_path     # the reference reads it with getenv
+    try:
+        counts = np.zeros(5, np.int32)
+        lib.ref_mtp_param.restype = _I
+        if lib.ref_mtp_param(_I(level), _p(counts), None, None, None) != 0:
+            raise RuntimeError("reference MtpParam failed for level %d" % level)
+        basic = np.zeros((counts[1], 4), np.int32)
+        times = np.zeros((counts[2], 4), np.int32)
+        mapping = np.zeros(counts[3], np.int32)
+        lib.ref_mtp_param(_I(level), _p(counts), _p(basic), _p(times), _p(mapping))
+    finally:
+        if saved is None:
+            del os.environ["AI2POT_PATH"]
+        else:
+            os.environ["AI2POT_PATH"] = saved
+    return dict(alpha_moments_count=int(counts[0]), alpha_index_basic=basic,
+                alpha_index_times=times, alpha_moment_mapping=mapping, nmus=int(counts[4]))
+
+
+def _mtp_model_args(model):
+    coeffs = _c(model["coeffs"], np.float64)
+    lin = _c(model["linear_coeffs"], np.float64)
+    bias = _c(model["type_bias"], np.float64)
+    basic = _c(model["alpha_index_basic"], np.int32)
+    times = _c(model["alpha_index_times"], np.int32)
+    mapping = _c(model["alpha_moment_mapping"], np.int32)
+    keep = (coeffs, lin, bias, basic, times, mapping)
+    args = [_I(model["chebyshev_size"]), _D(model.get("scaling", 1.0)), _p(coeffs), _p(lin), _p(bias),
+            _I(model["alpha_moments_count"]), _I(basic.shape[0]), _p(basic), _I(times.shape[0]),
+            _p(times), _I(mapping.size), _p(mapping), _I(model["nmus"])]
+    return args, keep
+
+
+def _mtp_list_args(model, nb):
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    type_map = _c(model["type_map"], np.int32)
+    q_scaler = _c(model["q_scaler"], np.float64)
+    keep = (binum, bilist, bnumneigh, bfirst, brcs, btypes, type_map, q_scaler)
+    args = [_I(B), _I(P), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes),
+            _I(type_map.size), _p(type_map), _I(U), _I(nghost), _D(model["rmax"]), _D(model["rmin"]),
+            _p(q_scaler)]
+    return args, keep, (B, P, U, nghost, type_map.size)
+
+
+def _mtp_efv(lib, prefix, model, nb):
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    e = np.zeros(B)
+    f = np.zeros((B, P + nghost, 3))
+    v = np.zeros((B, 9))
+    fn = getattr(lib, prefix + "_efv_f64")
+    fn.restype = None
+    fn(_p(e), _p(f), _p(v), *margs, *largs)
+    return e, f, v
+
+
+def _mtp_loss_step(lib, prefix, model, nb, weights, labels):
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    assert nghost == 0
+    K, nmus = model["chebyshev_size"], model["nmus"]
+    S = np.asarray(model["alpha_moment_mapping"]).size
+    ncoef = ntypes * ntypes * nmus * K
+    e_dft = _c(labels["energy"], np.float64)
+    f_dft = _c(labels["force"], np.float64)
+    v_dft = _c(labels["virial"], np.float64)
+    assert e_dft.shape == (B,) and f_dft.shape == (B, P, 3) and v_dft.shape == (B, 9)
+    out = dict(bloss=np.zeros(B), rmse=np.zeros(3), energy=np.zeros(B), force=np.zeros((B, P, 3)),
+               virial=np.zeros((B, 9)), dcoeffs=np.zeros((B, ncoef)), dlinear=np.zeros((B, S)),
+               dbias=np.zeros((B, ntypes)))
+    fn = getattr(lib, prefix + "_loss_step_f64")
+    fn.restype = None
+    fn(_p(out["bloss"]), _p(out["rmse"]), _p(out["energy"]), _p(out["force"]), _p(out["virial"]),
+       _p(out["dcoeffs"]), _p(out["dlinear"]), _p(out["dbias"]), _D(weights[0]), _D(weights[1]),
+       _D(weights[2]), _p(e_dft), _p(f_dft), _p(v_dft), *margs, *largs)
+    return out
+
+
+def ref_mtp_efv(model, nb):
+    return _mtp_efv(_load("_ref/libref_mtpr.so"), "ref_mtp", model, nb)
+
+
+def mtp_efv(model, nb):
+    return _mtp_efv(oracle_lib(), "orc_mtp", model, nb)
+
+
+def ref_mtp_loss_step(model, nb, weights, labels):
+    return _mtp_loss_step(_load("_ref/libref_mtpr.so"), "ref_mtp", model, nb, weights, labels)
+
+
+def mtp_loss_step(model, nb, weights, labels):
+    return _mtp_loss_step(oracle_lib(), "orc_mtp", model, nb, weights, labels)
+
+
+# ----------------------------------------------------------------------------------------
+# fvt (single structure, fp64)
+# ----------------------------------------------------------------------------------------
+def _fvt_force(lib, prefix, ilist, numneigh, firstneigh, nghost, dei_drij, grad_in=None):
+    ilist = _c(ilist, np.int32)
+    numneigh = _c(numneigh, np.int32)
+    firstneigh = _c(firstneigh, np.int32)
+    dei = _c(dei_drij, np.float64)
+    inum, umax = firstneigh.shape
+    force = np.zeros((inum + nghost, 3))
+    gout = None
+    gin = None
+    if grad_in is not None:
+        gin = _c(grad_in, np.float64)
+        gout = np.zeros((inum, umax, 3))
+    fn = getattr(lib, prefix + "_force_f64")
+    fn.restype = None
+    fn(_p(force), _p(gout), _p(gin), _I(inum), _p(ilist), _p(numneigh), _p(firstneigh), _I(nghost),
+       _I(umax), _p(dei))
+    return force, gout
+
+
+def _fvt_virial(lib, prefix, numneigh, rcs, dei_drij, ders=False):
+    numneigh = _c(numneigh, np.int32)
+    rcs = _c(rcs, np.float64)
+    dei = _c(dei_drij, np.float64)
+    inum, umax = rcs.shape[:2]
+    v = np.zeros(9)
+    d1 = np.zeros((9, inum, umax)) if ders else None
+    d2 = np.zeros((9, inum, umax)) if ders else None
+    fn = getattr(lib, prefix + "_virial_f64")
+    fn.restype = None
+    fn(_p(v), _p(d1), _p(d2), _I(inum), _p(numneigh), _p(rcs), _I(umax), _p(dei))
+    return v, d1, d2
+
+
+def ref_fvt_force(*a, **k):
+    return _fvt_force(_load("_ref/libref_fvt.so"), "ref_fvt", *a, **k)
+
+
+def fvt_force(*a, **k):
+    return _fvt_force(oracle_lib(), "orc_fvt", *a, **k)
+
+
+def ref_fvt_virial(*a, **k):
+    return _fvt_virial(_load("_ref/libref_fvt.so"), "ref_fvt", *a, **k)
+
+
+def fvt_virial(*a, **k):
+    return _fvt_virial(oracle_lib(), "orc_fvt", *a, **k)

@@ -1,0 +1,84 @@
+// TEST INFRASTRUCTURE ONLY. extern "C" driver around the reference's linear-MTP CPU
+// launchers (REF_ROOT/source/descriptor/mtpr/include/linearMtp_cpu_launcher.h:128-203,
+// linearMtpLoss_cpu_launcher.h:151-194, 233-337, 477-527) and its template parser
+// (src/mtpParam.cc, compiled alongside), built into oracle/_ref/libref_mtpr.so.
+// The loss-step entry follows LinearMtpToLossFunction::{forward,backward}
+// (src/linearMtpOp.cc:621-1181, 1184-1765): E/F/V, per-structure loss, RMSEs, then the
+// per-structure parameter gradients [B, n] before the grad_output matmul.
+#include <cstring>
+#include <string>
+#include "descriptor/mtpr/include/mtpParam.h"
+#include "descriptor/mtpr/include/linearMtp_cpu_launcher.h"
+#include "descriptor/mtpr/include/linearMtpLoss_cpu_launcher.h"
+
+using namespace ai2pot::mtpr;
+
+extern "C" {
+
+// Two-call protocol: with out pointers null only the counts are returned.
+// counts = {alpha_moments_count, basic_count, times_count, scalar_moments, nmus}
+int ref_mtp_param(int level, int* counts, int* basic, int* times, int* mapping)
+{
+    try {
+        MtpParam p(level);
+        counts[0] = p.alpha_moments_count();
+        counts[1] = p.alpha_index_basic_count();
+        counts[2] = p.alpha_index_times_count();
+        counts[3] = p.alpha_scalar_moments();
+        counts[4] = p.nmus();
+        if (basic) std::memcpy(basic, p.alpha_index_basic(), sizeof(int) * 4 * counts[1]);
+        if (times) std::memcpy(times, p.alpha_index_times(), sizeof(int) * 4 * counts[2]);
+        if (mapping) std::memcpy(mapping, p.alpha_moment_mapping(), sizeof(int) * counts[3]);
+        return 0;
+    } catch (MtpException& e) {
+        return 1;
+    }
+}
+
+#define MTP_MODEL_ARGS int K, double scaling, const double* coeffs, const double* lin, \
+    const double* bias, int n_moms, int n_basic, const int* basic, int n_times, const int* times, \
+    int n_scalar, const int* mapping, int nmus
+#define MTP_LIST_ARGS int B, int P, const int* binum, const int* bilist, const int* bnumneigh, \
+    const int* bfirstneigh, const double* brcs, const int* btypes, int ntypes, \
+    const int* type_map, int U, int nghost, double rmax, double rmin, const double* q_scaler
+
+#define MTP_MODEL_PASS K, scaling, const_cast<double*>(coeffs), const_cast<double*>(lin), \
+    const_cast<double*>(bias), n_moms, n_basic, (const int(*)[4])basic, n_times, \
+    (const int(*)[4])times, n_scalar, mapping, nmus
+#define MTP_LIST_PASS B, P, const_cast<int*>(binum), const_cast<int*>(bilist), \
+    const_cast<int*>(bnumneigh), const_cast<int*>(bfirstneigh), \
+    (double(*)[3])const_cast<double*>(brcs), const_cast<int*>(btypes), ntypes, \
+    const_cast<int*>(type_map), U, nghost, rmax, rmin, const_cast<double*>(q_scaler)
+
+void ref_mtp_efv_f64(double* betot, double* bforce, double* bvirial, MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    find_efv_cpu_launcher<double>(betot, (double(*)[3])bforce, bvirial, MTP_MODEL_PASS, MTP_LIST_PASS);
+}
+
+// forward + backward of the training-loss op. Outputs: bloss[B], rmse[3] (e,f,v),
+// E/F/V of the model, and per-structure gradients dcoeffs[B,ncoef], dlin[B,S], dbias[B,ntypes].
+void ref_mtp_loss_step_f64(double* bloss, double* rmse, double* betot, double* bforce, double* bvirial,
+                           double* dcoeffs, double* dlin, double* dbias, double e_w, double f_w,
+                           double v_w, const double* e_dft, const double* f_dft, const double* v_dft,
+                           MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    find_efv_cpu_launcher<double>(betot, (double(*)[3])bforce, bvirial, MTP_MODEL_PASS, MTP_LIST_PASS);
+    find_loss_cpu_launcher<double>(bloss, B, P, const_cast<int*>(binum), const_cast<int*>(bilist),
+                                   e_w, f_w, v_w, betot, const_cast<double*>(e_dft),
+                                   (double(*)[3])bforce, (double(*)[3])const_cast<double*>(f_dft),
+                                   bvirial, const_cast<double*>(v_dft));
+    find_efv_rmse_cpu_launcher<double>(rmse[0], rmse[1], rmse[2], B, P, const_cast<int*>(binum),
+                                       const_cast<int*>(bilist), betot, const_cast<double*>(e_dft),
+                                       (double(*)[3])bforce, (double(*)[3])const_cast<double*>(f_dft),
+                                       bvirial, const_cast<double*>(v_dft));
+    int ncoef = ntypes * ntypes * nmus * K;
+    std::memset(dcoeffs, 0, sizeof(double) * B * ncoef);
+    std::memset(dlin, 0, sizeof(double) * B * n_scalar);
+    std::memset(dbias, 0, sizeof(double) * B * ntypes);
+    find_loss_backward_cpu_launcher<double>(dcoeffs, dlin, dbias, e_w, f_w, v_w, betot,
+                                            const_cast<double*>(e_dft), (double(*)[3])bforce,
+                                            (double(*)[3])const_cast<double*>(f_dft), bvirial,
+                                            const_cast<double*>(v_dft), MTP_MODEL_PASS, MTP_LIST_PASS);
+}
+
+}

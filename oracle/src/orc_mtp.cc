@@ -1,0 +1,281 @@
+// TEST INFRASTRUCTURE ONLY -- CPU restatement (fp64) of the reference's linear Moment
+// Tensor Potential: energy / force / virial and one training-loss step (forward loss,
+// RMSEs and the per-structure gradients w.r.t. coeffs, linear_coeffs and type_bias).
+// Citations are to files under the reference's source/descriptor/mtpr/include.
+//
+// The E/F/V part follows the reference's formulas (mtpBasis.h:400-534, linearMtp.h:190-352).
+// The loss gradient is NOT the reference's hand-derived tangent/adjoint sweeps
+// (linearMtpLoss.h:212-569): it is obtained here by forward-mode differentiation of the
+// E/F/V evaluation itself with dual numbers, one parameter direction at a time, which is
+// slow but independent, so an error in either derivation shows up as a mismatch.
+//
+// Pinned by: the compiled reference (oracle/_ref/libref_mtpr.so) to 1e-12 relative on the
+// test fixtures; the reference unit test's known answer E = -0.938157350795572
+// (tests/test_linearMtp.cc, efv_force_accuracy set-up); finite differences of E; switch
+// function end values (tests/test_basis.cc:106-111); linearity of E in linear_coeffs.
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+// minimal dual number: value + one directional derivative
+struct Dual {
+    double v, d;
+    Dual(double v_ = 0, double d_ = 0) : v(v_), d(d_) {}
+};
+inline Dual operator+(Dual a, Dual b) { return {a.v + b.v, a.d + b.d}; }
+inline Dual operator-(Dual a, Dual b) { return {a.v - b.v, a.d - b.d}; }
+inline Dual operator*(Dual a, Dual b) { return {a.v * b.v, a.d * b.v + a.v * b.d}; }
+inline Dual operator/(Dual a, Dual b) { return {a.v / b.v, (a.d * b.v - a.v * b.d) / (b.v * b.v)}; }
+inline Dual& operator+=(Dual& a, Dual b) { a = a + b; return a; }
+inline Dual& operator-=(Dual& a, Dual b) { a = a - b; return a; }
+inline double val(double x) { return x; }
+inline double val(Dual x) { return x.v; }
+
+struct Tables {
+    int n_moms, n_basic, n_times, n_scalar, nmus;
+    const int *basic, *times, *mapping;
+};
+
+// f_k(r) = scaling * s(u) * T_k(x) and its r-derivative (basis.h:154-196, 351-381, 620-637)
+void radial_basis(int K, double rmax, double rmin, double scaling, double r, double* f, double* df)
+{
+    double x = (2 * r - (rmax + rmin)) / (rmax - rmin);
+    double dx = 2 / (rmax - rmin);
+    double u = (r - rmin) / (rmax - rmin);
+    double s = 0, ds = 0;
+    if (r >= rmin && r < rmax) {
+        s = u * u * u * (-6 * u * u + 15 * u - 10) + 1;
+        ds = 1 / (rmax - rmin) * (-30 * u * u * u * u + 60 * u * u * u - 30 * u * u);
+    }
+    std::vector<double> T(K), dT(K);
+    for (int k = 0; k < K; k++) {
+        if (k == 0) { T[k] = 1; dT[k] = 0; }
+        else if (k == 1) { T[k] = x; dT[k] = 1; }
+        else {
+            T[k] = 2 * x * T[k - 1] - T[k - 2];
+            dT[k] = 2 * T[k - 1] + 2 * x * dT[k - 1] - dT[k - 2];
+        }
+        f[k] = scaling * s * T[k];
+        df[k] = scaling * (ds * T[k] + s * dT[k] * dx);
+    }
+}
+
+// E/F/V of one structure, generic in the scalar type of the parameters (double or Dual).
+template <typename S>
+void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeffs, const S* lin,
+             const S* bias, const Tables& t, int inum, const int* ilist, const int* numneigh,
+             const int* firstneigh, const double* rcs, const int* types, int ntypes, int U,
+             int nforce, double rmax, double rmin, const double* q_scaler)
+{
+    etot = S(0);
+    for (int i = 0; i < nforce * 3; i++) force[i] = S(0);   // linearMtp.h:228-230
+    for (int i = 0; i < 9; i++) virial[i] = S(0);
+    int kmax = 0;
+    for (int i = 0; i < t.n_basic; i++) {
+        int k = t.basic[i * 4 + 1] + t.basic[i * 4 + 2] + t.basic[i * 4 + 3];
+        if (k > kmax) kmax = k;
+    }
+    std::vector<S> M(t.n_moms), adj(t.n_moms), g(K * t.nmus), dg(K * t.nmus);
+    std::vector<double> f(K), df(K), pw((kmax + 1) * 3), rp(kmax + 1);
+    for (int ii = 0; ii < inum; ii++) {
+        const int ci = ilist[ii], ti = types[ci], nn = numneigh[ii];
+        std::fill(M.begin(), M.end(), S(0));
+        // basic moments, mtpBasis.h:449-519
+        for (int jj = 0; jj < nn; jj++) {
+            const double* v = &rcs[((size_t)ii * U + jj) * 3];
+            double r = std::sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
+            if (r > rmax) continue;
+            int tj = types[firstneigh[(size_t)ii * U + jj]];
+            radial_basis(K, rmax, rmin, scaling, r, f.data(), df.data());
+            rp[0] = 1; pw[0] = pw[1] = pw[2] = 1;
+            for (int k = 1; k <= kmax; k++) {
+                rp[k] = rp[k - 1] * r;
+                for (int a = 0; a < 3; a++) pw[k * 3 + a] = pw[(k - 1) * 3 + a] * v[a];
+            }
+            const S* c = &coeffs[(size_t)(ti * ntypes + tj) * t.nmus * K];
+            for (int mu = 0; mu < t.nmus; mu++) {
+                S s(0);
+                for (int k = 0; k < K; k++) s += c[mu * K + k] * S(f[k]);
+                g[mu] = s;
+            }
+            for (int i = 0; i < t.n_basic; i++) {
+                const int* b = &t.basic[i * 4];
+                int k = b[1] + b[2] + b[3];
+                double ang = pw[b[1] * 3 + 0] * pw[b[2] * 3 + 1] * pw[b[3] * 3 + 2] / rp[k];
+                M[i] += g[b[0]] * S(ang);
+            }
+        }
+        for (int i = 0; i < t.n_times; i++) {                 // mtpBasis.h:522-528
+            const int* q = &t.times[i * 4];
+            M[q[3]] += S((double)q[2]) * M[q[0]] * M[q[1]];
+        }
+        S e = bias[ti];                                        // linearMtp.h:281-285
+        for (int s = 0; s < t.n_scalar; s++) e += lin[s] * M[t.mapping[s]] / S(q_scaler[s]);
+        etot += e;
+        std::fill(adj.begin(), adj.end(), S(0));               // linearMtp.h:292-306
+        for (int s = 0; s < t.n_scalar; s++) adj[t.mapping[s]] = lin[s] / S(q_scaler[s]);
+        for (int i = t.n_times - 1; i >= 0; i--) {
+            const int* q = &t.times[i * 4];
+            S w = adj[q[3]] * S((double)q[2]);
+            adj[q[1]] += w * M[q[0]];
+            adj[q[0]] += w * M[q[1]];
+        }
+        // pair derivative and scatter, linearMtp.h:308-342
+        for (int jj = 0; jj < nn; jj++) {
+            const double* v = &rcs[((size_t)ii * U + jj) * 3];
+            double r = std::sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
+            if (r > rmax) continue;
+            int nj = firstneigh[(size_t)ii * U + jj], tj = types[nj];
+            radial_basis(K, rmax, rmin, scaling, r, f.data(), df.data());
+            rp[0] = 1; pw[0] = pw[1] = pw[2] = 1;
+            for (int k = 1; k <= kmax; k++) {
+                rp[k] = rp[k - 1] * r;
+                for (int a = 0; a < 3; a++) pw[k * 3 + a] = pw[(k - 1) * 3 + a] * v[a];
+            }
+            const S* c = &coeffs[(size_t)(ti * ntypes + tj) * t.nmus * K];
+            for (int mu = 0; mu < t.nmus; mu++) {
+                S s(0), ds(0);
+                for (int k = 0; k < K; k++) {
+                    s += c[mu * K + k] * S(f[k]);
+                    ds += c[mu * K + k] * S(df[k]);
+                }
+                g[mu] = s;
+                dg[mu] = ds;
+            }
+            S gr[3] = {S(0), S(0), S(0)};
+            for (int i = 0; i < t.n_basic; i++) {
+                const int* b = &t.basic[i * 4];
+                int k = b[1] + b[2] + b[3];
+                double mono = pw[b[1] * 3 + 0] * pw[b[2] * 3 + 1] * pw[b[3] * 3 + 2];
+                double ang = mono / rp[k];
+                for (int a = 0; a < 3; a++) {
+                    double dmono = 0;
+                    if (b[1 + a] > 0) {
+                        int e[3] = {b[1], b[2], b[3]};
+                        e[a]--;
+                        dmono = b[1 + a] * pw[e[0] * 3 + 0] * pw[e[1] * 3 + 1] * pw[e[2] * 3 + 2];
+                    }
+                    double dang = dmono / rp[k] - k * mono / (rp[k] * r * r) * v[a];
+                    gr[a] += adj[i] * (dg[b[0]] * S(ang * v[a] / r) + g[b[0]] * S(dang));
+                }
+            }
+            for (int a = 0; a < 3; a++) {
+                force[ci * 3 + a] += gr[a];
+                force[nj * 3 + a] -= gr[a];
+                for (int bb = 0; bb < 3; bb++) virial[a * 3 + bb] -= gr[a] * S(v[bb]);
+            }
+        }
+    }
+}
+
+// per-structure loss, linearMtpLoss.h:138-176
+template <typename S>
+S loss_one(int inum, const int* ilist, double e_w, double f_w, double v_w, S etot, double e_dft,
+           const S* force, const double* f_dft, const S* virial, const double* v_dft)
+{
+    S fl(0), vl(0);
+    for (int ii = 0; ii < inum; ii++)
+        for (int a = 0; a < 3; a++) {
+            S d = force[ilist[ii] * 3 + a] - S(f_dft[ilist[ii] * 3 + a]);
+            fl += d * d;
+        }
+    for (int i = 0; i < 9; i++) {
+        S d = virial[i] - S(v_dft[i]);
+        vl += d * d;
+    }
+    S de = etot - S(e_dft);
+    return S(f_w / (3 * inum)) * fl + S(v_w / (9 * inum)) * vl + S(e_w / inum) * de * de;
+}
+
+}  // namespace
+
+#define MTP_MODEL_ARGS int K, double scaling, const double* coeffs, const double* lin, \
+    const double* bias, int n_moms, int n_basic, const int* basic, int n_times, const int* times, \
+    int n_scalar, const int* mapping, int nmus
+#define MTP_LIST_ARGS int B, int P, const int* binum, const int* bilist, const int* bnumneigh, \
+    const int* bfirstneigh, const double* brcs, const int* btypes, int ntypes, \
+    const int* type_map, int U, int nghost, double rmax, double rmin, const double* q_scaler
+
+extern "C" {
+
+void orc_mtp_efv_f64(double* betot, double* bforce, double* bvirial, MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+#pragma omp parallel for schedule(dynamic)
+    for (int b = 0; b < B; b++)
+        efv_one<double>(betot[b], &bforce[(size_t)b * (P + nghost) * 3], &bvirial[b * 9], K, scaling,
+                        coeffs, lin, bias, t, binum[b], &bilist[(size_t)b * P],
+                        &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                        &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * (P + nghost)], ntypes, U,
+                        P + nghost, rmax, rmin, q_scaler);
+}
+
+void orc_mtp_loss_step_f64(double* bloss, double* rmse, double* betot, double* bforce, double* bvirial,
+                           double* dcoeffs, double* dlin, double* dbias, double e_w, double f_w,
+                           double v_w, const double* e_dft, const double* f_dft, const double* v_dft,
+                           MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int ncoef = ntypes * ntypes * nmus * K;
+    const int npar = ncoef + n_scalar + ntypes;
+    // forward values and loss
+    for (int b = 0; b < B; b++) {
+        efv_one<double>(betot[b], &bforce[(size_t)b * P * 3], &bvirial[b * 9], K, scaling, coeffs, lin,
+                        bias, t, binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P],
+                        &bfirstneigh[(size_t)b * P * U], &brcs[(size_t)b * P * U * 3],
+                        &btypes[(size_t)b * P], ntypes, U, P, rmax, rmin, q_scaler);
+        bloss[b] = loss_one<double>(binum[b], &bilist[(size_t)b * P], e_w, f_w, v_w, betot[b], e_dft[b],
+                                    &bforce[(size_t)b * P * 3], &f_dft[(size_t)b * P * 3],
+                                    &bvirial[b * 9], &v_dft[b * 9]);
+    }
+    // RMSEs, linearMtpLoss_cpu_launcher.h:477-527
+    double es = 0, fs = 0, vs = 0;
+    long nf = 0;
+    for (int b = 0; b < B; b++) {
+        double de = (betot[b] - e_dft[b]) / binum[b];
+        es += de * de;
+        for (int ii = 0; ii < binum[b]; ii++) {
+            int ci = bilist[(size_t)b * P + ii];
+            for (int a = 0; a < 3; a++) {
+                double d = bforce[((size_t)b * P + ci) * 3 + a] - f_dft[((size_t)b * P + ci) * 3 + a];
+                fs += d * d;
+            }
+            nf += 3;
+        }
+        for (int i = 0; i < 9; i++) {
+            double d = (bvirial[b * 9 + i] - v_dft[b * 9 + i]) / binum[b];
+            vs += d * d;
+        }
+    }
+    rmse[0] = std::sqrt(es / B);
+    rmse[1] = std::sqrt(fs / nf);
+    rmse[2] = std::sqrt(vs / (9.0 * B));
+
+    // gradient by forward-mode AD, one parameter direction per pass
+#pragma omp parallel
+    {
+        std::vector<Dual> c(ncoef), l(n_scalar), bi(ntypes), force((size_t)P * 3), virial(9);
+#pragma omp for schedule(dynamic) collapse(2)
+        for (int b = 0; b < B; b++)
+            for (int p = 0; p < npar; p++) {
+                for (int i = 0; i < ncoef; i++) c[i] = Dual(coeffs[i], i == p);
+                for (int i = 0; i < n_scalar; i++) l[i] = Dual(lin[i], ncoef + i == p);
+                for (int i = 0; i < ntypes; i++) bi[i] = Dual(bias[i], ncoef + n_scalar + i == p);
+                Dual e;
+                efv_one<Dual>(e, force.data(), virial.data(), K, scaling, c.data(), l.data(), bi.data(),
+                              t, binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P],
+                              &bfirstneigh[(size_t)b * P * U], &brcs[(size_t)b * P * U * 3],
+                              &btypes[(size_t)b * P], ntypes, U, P, rmax, rmin, q_scaler);
+                Dual L = loss_one<Dual>(binum[b], &bilist[(size_t)b * P], e_w, f_w, v_w, e, e_dft[b],
+                                        force.data(), &f_dft[(size_t)b * P * 3], virial.data(),
+                                        &v_dft[b * 9]);
+                if (p < ncoef) dcoeffs[(size_t)b * ncoef + p] = L.d;
+                else if (p < ncoef + n_scalar) dlin[(size_t)b * n_scalar + p - ncoef] = L.d;
+                else dbias[(size_t)b * ntypes + p - ncoef - n_scalar] = L.d;
+            }
+    }
+}
+
+}
