@@ -1,0 +1,122 @@
+// Internal helpers shared by the HIP translation units of libai2pot_hip.so:
+// error reporting, a per-device growable workspace, launch checks and wave-level
+// primitives for 64-wide wavefronts (gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdarg>
+#include <string>
+
+#include "../../include/ai2pot_hip.h"
+
+namespace a2p {
+
+// ---- error state (thread local, read back through a2p_last_error) ---------------------
+void set_error(const char* fmt, ...);
+const char* last_error();
+
+#define A2P_HIP_CHECK(expr)                                                              \
+    do {                                                                                 \
+        hipError_t e_ = (expr);                                                          \
+        if (e_ != hipSuccess) {                                                          \
+            a2p::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),        \
+                           __FILE__, __LINE__);                                          \
+            return A2P_ERR_HIP;                                                          \
+        }                                                                                \
+    } while (0)
+
+#define A2P_REQUIRE(cond, code, ...)                                                     \
+    do {                                                                                 \
+        if (!(cond)) {                                                                   \
+            a2p::set_error(__VA_ARGS__);                                                 \
+            return code;                                                                 \
+        }                                                                                \
+    } while (0)
+
+// ---- workspace: a few named device buffers per device, grown on demand -----------------
+enum WsSlot {
+    WS_PAIR_G = 0,     // per-pair derivative buffer [rows, U, 3]
+    WS_CSR,            // counts / offsets / cursors / incoming pair ids
+    WS_PARTIAL,        // per-block partial sums (energy, virial, loss terms)
+    WS_NBL_A,          // neighbor-list: images, bins
+    WS_NBL_B,
+    WS_MTP,            // MTP per-atom scratch
+    WS_FLAGS,          // device-side status words
+    WS_MISC,
+    WS_NSLOTS
+};
+// Returns a device pointer valid until the next ws_get on the same slot with a larger size.
+// Growth synchronises the device (hipFree); steady-state calls do not allocate.
+int ws_get(int slot, size_t bytes, void** out);
+
+// Device status word bits written by kernels when inputs violate the contract.
+enum StatusBits {
+    ST_BAD_NEIGHBOR = 1,   // neighbour index outside [0, natoms_pad + nghost)
+    ST_BAD_TYPE = 2,       // type index outside [0, ntypes)
+    ST_NEIGH_OVERFLOW = 4, // numneigh larger than the row capacity
+};
+
+inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// ---- wave64 primitives -------------------------------------------------------------------
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63); }
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_max(T v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        T o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+__device__ __forceinline__ long long shfl_xor_ll(long long v, int off)
+{
+    int lo = __shfl_xor((int)(v & 0xffffffffll), off, 64);
+    int hi = __shfl_xor((int)(v >> 32), off, 64);
+    return ((long long)hi << 32) | (unsigned int)lo;
+}
+
+// inclusive prefix sum across the 64 lanes of a wave
+__device__ __forceinline__ int wave_inclusive_scan(int v)
+{
+    int lane = lane_id();
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int o = __shfl_up(v, off, 64);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+// ---- shared device routines (pair_reduce.hip) --------------------------------------------
+// Deterministic reduction of per-pair derivatives g[row, slot, 3] onto atoms:
+//   force[b, j] = own[b, j] - sum over pairs (row, slot) of structure b whose neighbour is j.
+// `force` must already hold the `own` part (zero for atoms without a row).  Integer atomics
+// build the incoming lists; the floating-point sums are order-independent (exact fixed-point
+// accumulation against the per-target maximum), so results are reproducible run to run.
+template <typename T>
+int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
+                const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
+
+// out[b*out_stride + c] = sum over blocks of partial[(b*nblocks + block)*src_stride + c], c < ncomp,
+// with a fixed summation tree (fp64).
+template <typename T>
+int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
+                    int out_stride, hipStream_t stream);
+
+int fill_zero(void* ptr, size_t bytes, hipStream_t stream);
+
+}  // namespace a2p

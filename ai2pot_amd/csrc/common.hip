@@ -1,0 +1,135 @@
+// Error state, per-device workspace and small utility kernels of libai2pot_hip.so.
+#include "a2p_common.h"
+
+#include <mutex>
+#include <vector>
+
+namespace a2p {
+
+static thread_local std::string g_err;
+
+void set_error(const char* fmt, ...)
+{
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_err = buf;
+}
+
+const char* last_error() { return g_err.c_str(); }
+
+namespace {
+struct Buf {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+struct DeviceWs {
+    Buf slot[WS_NSLOTS];
+};
+std::mutex g_ws_mutex;
+std::vector<DeviceWs> g_ws;
+}  // namespace
+
+int ws_get(int slot, size_t bytes, void** out)
+{
+    int dev = 0;
+    A2P_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if ((int)g_ws.size() <= dev) g_ws.resize(dev + 1);
+    Buf& b = g_ws[dev].slot[slot];
+    if (bytes > b.bytes) {
+        if (b.ptr) A2P_HIP_CHECK(hipFree(b.ptr));   // synchronises: no kernel still uses it
+        b.ptr = nullptr;
+        b.bytes = 0;
+        size_t want = bytes + bytes / 8 + 256;      // head-room so small growth does not realloc
+        A2P_HIP_CHECK(hipMalloc(&b.ptr, want));
+        b.bytes = want;
+        if (slot == WS_FLAGS) A2P_HIP_CHECK(hipMemset(b.ptr, 0, want));
+    }
+    *out = b.ptr;
+    return A2P_OK;
+}
+
+__global__ void fill_zero_kernel(uint32_t* p, size_t nwords)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < nwords; i += stride) p[i] = 0u;
+}
+
+int fill_zero(void* ptr, size_t bytes, hipStream_t stream)
+{
+    if (bytes == 0) return A2P_OK;
+    A2P_REQUIRE(bytes % 4 == 0, A2P_ERR_INVALID, "fill_zero: size not a multiple of 4");
+    size_t nwords = bytes / 4;
+    int blocks = (int)std::min<size_t>((nwords + 255) / 256, 256 * 32);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t*)ptr, nwords);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+// One block per (structure, component): sums the per-block partials in block order.
+template <typename T>
+__global__ void finish_partials_kernel(T* out, const double* partial, int nblocks, int src_stride,
+                                       int out_stride)
+{
+    __shared__ double sh[256];
+    const int b = blockIdx.y, c = blockIdx.x;
+    const double* src = partial + ((size_t)b * nblocks) * src_stride + c;
+    // fixed assignment of blocks to threads, fixed tree: the result does not depend on timing
+    double acc = 0.0;
+    for (int k = threadIdx.x; k < nblocks; k += 256) acc += src[(size_t)k * src_stride];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[(size_t)b * out_stride + c] = (T)sh[0];
+}
+
+template <typename T>
+int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
+                    int out_stride, hipStream_t stream)
+{
+    hipLaunchKernelGGL(finish_partials_kernel<T>, dim3(ncomp, B), dim3(256), 0, stream, out, partial,
+                       nblocks, src_stride, out_stride);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+template int finish_partials<float>(float*, const double*, int, int, int, int, int, hipStream_t);
+template int finish_partials<double>(double*, const double*, int, int, int, int, int, hipStream_t);
+
+}  // namespace a2p
+
+extern "C" {
+
+const char* a2p_last_error(void) { return a2p::last_error(); }
+
+int a2p_abi_version(void) { return 1; }
+
+int a2p_check_status(void* stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    void* flags = nullptr;
+    int rc = a2p::ws_get(a2p::WS_FLAGS, 64, &flags);
+    if (rc) return rc;
+    int host = 0;
+    A2P_HIP_CHECK(hipMemcpyAsync(&host, flags, sizeof(int), hipMemcpyDeviceToHost, stream));
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    if (host == 0) return A2P_OK;
+    rc = a2p::fill_zero(flags, 64, stream);
+    if (rc) return rc;
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    if (host & a2p::ST_NEIGH_OVERFLOW) {
+        a2p::set_error("a neighbour count exceeds umax_num_neigh_atoms");
+        return A2P_ERR_OVERFLOW;
+    }
+    a2p::set_error("device-side input check failed:%s%s",
+                   (host & a2p::ST_BAD_NEIGHBOR) ? " neighbour index outside [0, natoms_pad+nghost)" : "",
+                   (host & a2p::ST_BAD_TYPE) ? " type index outside [0, ntypes)" : "");
+    return A2P_ERR_INPUT;
+}
+}

@@ -1,0 +1,73 @@
+/* libai2pot_hip.so -- C ABI of the MI355X (gfx950) energy / force / virial hot path.
+ *
+ * Every entry point takes plain pointers and sizes.  Unless a parameter is documented as
+ * "host", pointers are DEVICE pointers on the current HIP device; the caller owns every
+ * input and output buffer.  Work is enqueued on `stream` (a hipStream_t passed as void*;
+ * NULL = the default stream) and, unless stated otherwise, the call returns without
+ * synchronising.  Scratch memory is a per-device workspace the library grows on demand
+ * (steady-state calls allocate nothing).  Return value: A2P_OK or an A2P_ERR_* code; the
+ * message of the last error on the calling thread is returned by a2p_last_error().
+ *
+ * "Reference" below is lhycms/AI2Pot; paths are relative to its root.
+ */
+#ifndef AI2POT_HIP_H
+#define AI2POT_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define A2P_OK 0
+#define A2P_ERR_INVALID 1   /* argument violates the contract (message says which)          */
+#define A2P_ERR_HIP 2       /* a HIP runtime call failed                                     */
+#define A2P_ERR_OVERFLOW 3  /* a neighbour count exceeds the row capacity umax               */
+#define A2P_ERR_INPUT 4     /* device-side input check failed (bad neighbour / type index)   */
+
+const char* a2p_last_error(void);
+
+/* Version of this ABI (bumped on incompatible change). */
+int a2p_abi_version(void);
+
+/* Reads and clears the device status word that kernels set when an input violates the
+ * contract (neighbour index outside [0, natoms_pad+nghost), type index outside
+ * [0, ntypes), numneigh > umax).  Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT or
+ * A2P_ERR_OVERFLOW.  The reference has no such check: it asserts or overflows
+ * (source/nblist/include/neighborList.h:550, commented-out assert). */
+int a2p_check_status(void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * NEP energy / force / virial -- replaces the compute of torch.ops.nep.nepToEFVOp /
+ * nepToEFOp / nepToDescriptorsOp (source/descriptor/nep/bind/nep_bind.cc:26-135, 278-311;
+ * source/descriptor/nep/src/nepOp.cc:947-1284 -> include/nep_cpu_launcher.h:186-255 ->
+ * include/nep.h:320-529, include/nepBasis.h:57-196).
+ *
+ * Model: coeffs[ntypes][ntypes][n_radial+n_angular][K], w0[ntypes][H][D], b0[ntypes][H],
+ * w1[ntypes][H], type_bias[ntypes], q_scaler[D], D = n_radial + n_angular*l_max.
+ * Batch (the 7-tensor contract): binum[B], bilist[B][P], bnumneigh[B][P],
+ * bfirstneigh[B][P][U], brcs[B][P][U][3] (r_j - r_i), btypes[B][P+nghost] (type indices).
+ * Outputs (each may be NULL to skip): etot[B], force[B][P+nghost][3], virial[B][9]
+ * (row-major a*3+b, V = -sum g_a r_b), descriptors[B][P][D].  Outputs are overwritten.
+ * Sign convention as the reference: force[i] += dE_i/dr_ij, force[j] -= dE_i/dr_ij.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nep_efv_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
+                    int ntypes, const float* coeffs, const float* w0, const float* b0,
+                    const float* w1, const float* type_bias, const float* q_scaler,
+                    double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
+                    int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                    const int* bfirstneigh, const float* brcs, const int* btypes, float* etot,
+                    float* force, float* virial, float* descriptors, void* stream);
+
+int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
+                    int ntypes, const double* coeffs, const double* w0, const double* b0,
+                    const double* w1, const double* type_bias, const double* q_scaler,
+                    double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
+                    int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                    const int* bfirstneigh, const double* brcs, const int* btypes, double* etot,
+                    double* force, double* virial, double* descriptors, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

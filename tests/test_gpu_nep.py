@@ -1,0 +1,211 @@
+"""GPU parity of the NEP energy / force / virial path against the CPU oracle.
+
+Bars: fp64 results within 1e-10 relative of the oracle; fp32 energies and virials within
+1e-5 relative, fp32 forces within 1e-4 eV/A absolute + 1e-5 relative (the oracle evaluates
+the fp32 inputs in double, i.e. it is the exactly rounded answer)."""
+import numpy as np
+import pytest
+
+from ai2pot_amd import synth
+from conftest import to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _model_to_device(m, dtype, device="cuda:0"):
+    import torch
+    out = dict(m)
+    for k in ("coeffs", "w0", "b0", "w1", "type_bias", "q_scaler"):
+        out[k] = torch.from_numpy(np.ascontiguousarray(m[k], np.float64)).to(dtype).to(device)
+    out["type_map"] = torch.from_numpy(np.ascontiguousarray(m["type_map"], np.int32)).to(device)
+    return out
+
+
+def run_gpu(m, nb, np_dtype, virial=True):
+    import torch
+    from ai2pot_amd import ops
+    dtype = torch.float32 if np_dtype == np.float32 else torch.float64
+    md = _model_to_device(m, dtype)
+    d = to_device(nb, dtype)
+    fn = ops.nepToEFVOp if virial else ops.nepToEFOp
+    out = fn(m["chebyshev_size"], m["n_radial_basis"], m["n_angular_basis"], m["l_max"], md["coeffs"],
+             md["w0"], md["b0"], md["w1"], md["type_bias"], d["binum"], d["bilist"], d["bnumneigh"],
+             d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], d["nghost"], m["rmax_radial"],
+             m["rmax_angular"], md["q_scaler"], 0.0, 0.0, None, None)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in out]
+
+
+def check(out, ref, np_dtype):
+    e, f, v = out
+    er, fr, vr = ref
+    if np_dtype == np.float64:
+        assert np.allclose(e, er, rtol=1e-10, atol=0)
+        assert np.abs(f - fr).max() <= 1e-10 * max(np.abs(fr).max(), 1e-30)
+        assert np.abs(v - vr).max() <= 1e-10 * max(np.abs(vr).max(), 1e-30)
+    else:
+        assert np.allclose(e, er, rtol=1e-5, atol=0)
+        assert np.all(np.abs(f - fr) <= 1e-4 + 1e-5 * np.abs(fr))
+        assert np.abs(v - vr).max() <= 1e-5 * np.abs(vr).max()
+
+
+def small_structure(oracle, n=300, box=(18.0, 19.0, 20.0), ntypes=3, seed=11, dtype=np.float64,
+                    rcut=7.0, umax=200, sort=False):
+    lat, pos = synth.random_packed(n, list(box), 2.2, seed)
+    types = synth.rng_randint(seed + 1, n, ntypes)
+    return oracle.nblist(lat.astype(dtype), types, pos.astype(dtype), rcut, umax, sort=sort)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_mos2_known_answer(oracle, np_dtype):
+    """Set-up of the reference's own unit test (tests/test_nep.cc:100-255): l_max = 3,
+    30 neurons, sorted list, umax 20.  Known answer E = 46.363417549065026."""
+    lat, types, frac = synth.mos2_fixture()
+    out = oracle.nblist(lat.astype(np_dtype), types, frac.astype(np_dtype), 5.0, 20, is_cart=False, sort=True)
+    nb = synth.pack_batch([out])
+    m = synth.nep_model_closed_form()
+    e, f, v = run_gpu(m, nb, np_dtype)
+    tol = 1e-10 if np_dtype == np.float64 else 1e-5
+    assert abs(e[0] - 46.363417549065026) <= tol * 46.4
+    check((e, f, v), oracle.nep_efv(m, nb, np_dtype), np_dtype)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_random_cell_fast_path(oracle, np_dtype):
+    nb = synth.pack_batch([small_structure(oracle, dtype=np_dtype)])
+    m = synth.nep_model()
+    check(run_gpu(m, nb, np_dtype), oracle.nep_efv(m, nb, np_dtype), np_dtype)
+    # energy + force operator gives the same E and F
+    e2, f2 = run_gpu(m, nb, np_dtype, virial=False)
+    er, fr, _ = oracle.nep_efv(m, nb, np_dtype)
+    check((e2, f2, np.ones(9)), (er, fr, np.ones(9)), np_dtype)
+
+
+def test_batch_padding_permuted_ilist(oracle):
+    """Three structures of different size in one padded batch, rows listed in a permuted
+    order through ilist (row ii describes atom ilist[ii])."""
+    a = small_structure(oracle, 120, (14.0, 15.0, 13.0), seed=31)
+    b = small_structure(oracle, 200, (17.0, 15.0, 16.0), seed=32)
+    c = small_structure(oracle, 37, (11.0, 15.0, 9.0), seed=33)
+    nb = synth.pack_batch([a, b, c])
+    rng = np.random.default_rng(5)
+    for s, inum in enumerate(nb["binum"]):
+        perm = rng.permutation(inum)
+        for key in ("bnumneigh", "bfirstneigh", "brcs"):
+            nb[key][s, :inum] = nb[key][s, perm]
+        nb["bilist"][s, :inum] = perm
+    m = synth.nep_model()
+    check(run_gpu(m, nb, np.float64), oracle.nep_efv(m, nb, np.float64), np.float64)
+    check(run_gpu(m, nb, np.float32), oracle.nep_efv(m, nb, np.float32), np.float32)
+
+
+def test_ghost_atoms(oracle):
+    """The LAMMPS contract: neighbour indices point into [0, P + nghost); ghosts have a type
+    and receive forces but own no row (interface/lammps/AI2POT/pair_ai2pot.cpp:175-249)."""
+    full = small_structure(oracle, 150, (15.0, 15.0, 14.0), seed=41)
+    inum, ilist, numneigh, firstneigh, rcs, types, _ = full
+    nlocal = 100                       # atoms >= nlocal become ghosts of a smaller "rank"
+    nb = dict(binum=np.array([nlocal], np.int32), bilist=ilist[None, :nlocal].copy(),
+              bnumneigh=numneigh[None, :nlocal].copy(), bfirstneigh=firstneigh[None, :nlocal].copy(),
+              brcs=rcs[None, :nlocal].copy(), btypes=types[None, :].copy(), nghost=inum - nlocal)
+    nb["bfirstneigh"][nb["bfirstneigh"] < 0] = 0
+    m = synth.nep_model()
+    out = run_gpu(m, nb, np.float64)
+    assert out[1].shape == (1, inum, 3)
+    check(out, oracle.nep_efv(m, nb, np.float64), np.float64)
+
+
+@pytest.mark.parametrize("cfg", [dict(K=10, n_r=7, n_a=5, l_max=2, H=17, ntypes=2),
+                                 dict(K=6, n_r=4, n_a=3, l_max=0, H=8, ntypes=1),
+                                 dict(K=14, n_r=10, n_a=7, l_max=4, H=5, ntypes=2),
+                                 dict(K=8, n_r=6, n_a=4, l_max=4, H=200, ntypes=4)])
+def test_general_shapes(oracle, cfg):
+    """Sizes that do not hit the compile-time fast path, including l_max = 0 (radial only,
+    nep_utilities.h:43-44) and a network too large for LDS."""
+    nb = synth.pack_batch([small_structure(oracle, 90, (12.0, 13.0, 12.5), ntypes=cfg["ntypes"], seed=51,
+                                           rcut=6.0)])
+    m = synth.nep_model(ntypes=cfg["ntypes"], n_radial_basis=cfg["n_r"], n_angular_basis=cfg["n_a"],
+                        l_max=cfg["l_max"], chebyshev_size=cfg["K"], num_neurons=cfg["H"],
+                        rmax_radial=6.0, rmax_angular=4.5, seed=77, type_map=(1, 2, 3, 4))
+    if cfg["l_max"] == 0:
+        D = cfg["n_r"]
+        m["w0"] = m["w0"][:cfg["ntypes"] * cfg["H"] * D]
+        m["q_scaler"] = np.linspace(0.5, 1.5, D)
+    else:
+        m["q_scaler"] = np.linspace(0.5, 1.5, m["q_scaler"].size)
+    check(run_gpu(m, nb, np.float64), oracle.nep_efv(m, nb, np.float64), np.float64)
+
+
+def test_descriptors(oracle):
+    import torch
+    from ai2pot_amd import ops
+    nb = synth.pack_batch([small_structure(oracle, 80, (12.0, 13.0, 12.5), seed=61)])
+    m = synth.nep_model()
+    md = _model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    out = ops.nepToDescriptorsOp(8, 6, 4, 4, md["coeffs"], d["binum"], d["bilist"], d["bnumneigh"],
+                                 d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], 0, 7.0, 4.0)
+    ref = oracle.nep_descriptors(m, nb, np.float64)
+    assert np.abs(out[0].cpu().numpy() - ref).max() <= 1e-10 * np.abs(ref).max()
+
+
+def test_config2_full_size(oracle):
+    """Benchmark configuration 2 at full size: 4096 atoms, 3 species, fp32, list cutoff 7 A."""
+    lat, pos = synth.random_packed(4096, [49.8848] * 3, 2.2, 1003)
+    types = synth.rng_randint(2003, 4096, 3)
+    nb = synth.pack_batch([oracle.nblist(lat.astype(np.float32), types, pos.astype(np.float32), 7.0, 200)])
+    m = synth.nep_model(seed=3003)
+    out = run_gpu(m, nb, np.float32)
+    check(out, oracle.nep_efv(m, nb, np.float32), np.float32)
+    # size-independent properties: a symmetric full list gives zero net force and a
+    # symmetric virial up to rounding
+    f, v = out[1][0].astype(np.float64), out[2][0].reshape(3, 3)
+    assert np.abs(f.sum(0)).max() < 1e-3
+    assert np.abs(v - v.T).max() <= 2e-5 * np.abs(v).max()
+
+
+def test_reproducible(oracle):
+    """Two runs give bit-identical forces (no floating-point atomics anywhere)."""
+    nb = synth.pack_batch([small_structure(oracle, 300, dtype=np.float32)])
+    m = synth.nep_model()
+    a = run_gpu(m, nb, np.float32)
+    b = run_gpu(m, nb, np.float32)
+    for x, y in zip(a, b):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+
+
+def test_errors(oracle):
+    import torch
+    from ai2pot_amd import ops, _lib
+    nb = synth.pack_batch([small_structure(oracle, 60, (11.0, 11.0, 11.0), seed=71, umax=100)])
+    m = synth.nep_model()
+    md = _model_to_device(m, torch.float32)
+    d = to_device(nb, torch.float32)
+
+    def call(**over):
+        a = dict(d)
+        a.update(over)
+        return ops.nepToEFVOp(8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"],
+                              a["binum"], a["bilist"], a["bnumneigh"], a["bfirstneigh"], a["brcs"],
+                              a["btypes"], md["type_map"], 0, 7.0, 4.0, md["q_scaler"], 0.0, 0.0, None, None)
+
+    call()
+    with pytest.raises(RuntimeError):                       # wrong dtype
+        call(brcs=d["brcs"].double())
+    with pytest.raises(RuntimeError):                       # non-contiguous
+        call(bfirstneigh=d["bfirstneigh"].transpose(1, 2).contiguous().transpose(1, 2))
+    with pytest.raises(RuntimeError):                       # host tensor: no CPU path
+        call(brcs=d["brcs"].cpu())
+    with pytest.raises(RuntimeError):                       # neighbour count beyond the row
+        call(bnumneigh=d["bnumneigh"] + 1000)
+    bad = d["bfirstneigh"].clone()
+    bad[0, 0, 0] = 10 ** 6
+    with pytest.raises(_lib.A2PError):                      # neighbour index out of range
+        call(bfirstneigh=bad)
+    with pytest.raises(_lib.A2PError):                      # type index out of range
+        call(btypes=d["btypes"] + 7)
+    with pytest.raises(RuntimeError):                       # ZBL not built
+        ops.nepToEFVOp(8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"],
+                       d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"],
+                       md["type_map"], 0, 7.0, 4.0, md["q_scaler"], 1.0, 0.5, None, None)
+    call()                                                  # the library is still usable
