@@ -119,4 +119,9 @@ int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp
 
 int fill_zero(void* ptr, size_t bytes, hipStream_t stream);
 
+// out[i] = in[0] + ... + in[i-1] for i < n (out must not alias in); tmp holds
+// scan_tmp_ints(n) ints, and tmp[ceil(n/2048)] receives the total.
+int scan_tmp_ints(int n);
+int exclusive_scan_i32(const int* in, int* out, int n, int* tmp, hipStream_t stream);
+
 }  // namespace a2p

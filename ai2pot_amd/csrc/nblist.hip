@@ -1,0 +1,730 @@
+// Periodic neighbour list for gfx950, bit-exact to the reference's
+// source/nblist/include/{structure.h, binLinkedList.h, neighborList.h}.
+//
+// The reference replicates the cell into an explicit supercell of (2*ceil(rcut/d_a)+1)
+// images per periodic axis, bins every image atom into rcut/2 bins by head insertion and,
+// per centre atom, walks 5x5x5 bins (dx outer, dz inner), each bin in descending supercell
+// index.  Only image atoms that fall into the bins around the centre cell can ever be
+// visited, so here the supercell is never materialised:
+//   1. coords   : Cartesian coordinates; min / max of ALL image coordinates (they define
+//                 the reference's bin origin) and of the centre atoms, by reduction
+//   2. count    : every (atom, image) pair computes its reference bin with the reference's
+//                 rounding; those inside the bin box around the centre atoms are counted
+//   3. scan     : prefix sum over the box's bins (z fastest, so the five dz bins of one
+//                 (dx, dy) column are contiguous)
+//   4. fill     : image atoms copied into their bin segment
+//   5. binsort  : each bin ordered by descending supercell index (= the head-insertion order)
+//   6. lists    : one wavefront per centre atom walks the 25 (dx, dy) columns in reference
+//                 order; 64 candidates are distance-tested at a time with the reference's
+//                 mixed float/double arithmetic and compacted in order with a wave ballot
+//                 and prefix popcount; the padded row (-1 / 0 fill) is written in the same pass
+//   7. sort     : (sort = true) per atom, the same introsort + insertion sort sequence as
+//                 libstdc++'s std::sort on float-rounded distances, so ties land where the
+//                 reference puts them
+// This translation unit is compiled with -ffp-contract=off and spells the critical
+// operations with the *_rn intrinsics: no fused multiply-add may change a rounding.
+#include "a2p_common.h"
+
+#include <climits>
+#include <cmath>
+#include <vector>
+
+namespace a2p {
+namespace {
+
+constexpr double kMargin = 0.5;      // NBLIST_MARGIN, structure.h:27
+constexpr double kEpsilon = 1e-3;    // EPSILON, binLinkedList.h:28
+constexpr int NBL_BLOCK = 256;
+
+__device__ __forceinline__ float add_rn(float a, float b) { return __fadd_rn(a, b); }
+__device__ __forceinline__ float sub_rn(float a, float b) { return __fsub_rn(a, b); }
+__device__ __forceinline__ float mul_rn(float a, float b) { return __fmul_rn(a, b); }
+__device__ __forceinline__ float div_rn(float a, float b) { return __fdiv_rn(a, b); }
+__device__ __forceinline__ double add_rn(double a, double b) { return __dadd_rn(a, b); }
+__device__ __forceinline__ double sub_rn(double a, double b) { return __dsub_rn(a, b); }
+__device__ __forceinline__ double mul_rn(double a, double b) { return __dmul_rn(a, b); }
+__device__ __forceinline__ double div_rn(double a, double b) { return __ddiv_rn(a, b); }
+
+template <typename T>
+struct Grid {
+    T b[3][3];        // lattice rows
+    T mn[3];          // bin origin: min over all image coordinates - 0.5
+    T bin_size;       // rcut / 2
+    T rcut;
+    double rcut2;     // std::pow(rcut, 2) evaluated in double
+    int nbin[3];      // the reference's bin counts
+    int rlo[3];       // bin box kept here: [rlo, rlo + rdim)
+    int rdim[3];
+    int img_lo[3];    // image index ranges
+    int img_dim[3];
+    int nimg;
+    int N;
+    int ext_bins;     // ceil(rcut / bin_size) = 2
+    int is_cart;
+};
+
+// image coordinate x + b0*ii + b1*jj + b2*kk, left to right (structure.h:659-676)
+template <typename T>
+__device__ __forceinline__ T image_coord(T x, T b0, T b1, T b2, int ii, int jj, int kk)
+{
+    T v = add_rn(x, mul_rn(b0, (T)ii));
+    v = add_rn(v, mul_rn(b1, (T)jj));
+    return add_rn(v, mul_rn(b2, (T)kk));
+}
+
+template <typename T>
+__device__ __forceinline__ int bin_of(T c, T mn, T bin_size)      // binLinkedList.h:824-826
+{
+    return (int)floor(div_rn(sub_rn(c, mn), bin_size));
+}
+
+// ---- 1. coordinates and extents --------------------------------------------------------------
+template <typename T>
+__global__ void coords_minmax_kernel(const Grid<T> g, const T* __restrict__ coords, T* __restrict__ x,
+                                     T* __restrict__ partial)
+{
+    __shared__ T sh[NBL_BLOCK / 64][12];
+    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    T v[12];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        v[a] = (T)INT_MAX; v[3 + a] = (T)INT_MIN;       // structure.h:1018-1022
+        v[6 + a] = (T)INT_MAX; v[9 + a] = (T)INT_MIN;
+    }
+    if (p < g.N) {
+        T c[3];
+        if (g.is_cart) {
+#pragma unroll
+            for (int a = 0; a < 3; a++) c[a] = coords[(size_t)p * 3 + a];
+        } else {                                         // calc_cart_coords, structure.h:561-579
+            const T f0 = coords[(size_t)p * 3], f1 = coords[(size_t)p * 3 + 1], f2 = coords[(size_t)p * 3 + 2];
+#pragma unroll
+            for (int a = 0; a < 3; a++)
+                c[a] = add_rn(add_rn(mul_rn(f0, g.b[0][a]), mul_rn(f1, g.b[1][a])), mul_rn(f2, g.b[2][a]));
+        }
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            x[(size_t)p * 3 + a] = c[a];
+            v[6 + a] = c[a];
+            v[9 + a] = c[a];
+        }
+        for (int i = 0; i < g.img_dim[0]; i++)
+            for (int j = 0; j < g.img_dim[1]; j++)
+                for (int k = 0; k < g.img_dim[2]; k++) {
+#pragma unroll
+                    for (int a = 0; a < 3; a++) {
+                        T s = image_coord(c[a], g.b[0][a], g.b[1][a], g.b[2][a], g.img_lo[0] + i,
+                                          g.img_lo[1] + j, g.img_lo[2] + k);
+                        if (s < v[a]) v[a] = s;
+                        if (s > v[3 + a]) v[3 + a] = s;
+                    }
+                }
+    }
+#pragma unroll
+    for (int q = 0; q < 12; q++) {
+        const bool is_min = (q % 6) < 3;
+        T r = v[q];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            T o = __shfl_xor(r, off, 64);
+            r = is_min ? (o < r ? o : r) : (o > r ? o : r);
+        }
+        if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6][q] = r;
+    }
+    __syncthreads();
+    if (threadIdx.x < 12) {
+        const int q = threadIdx.x;
+        const bool is_min = (q % 6) < 3;
+        T r = sh[0][q];
+        for (int w = 1; w < NBL_BLOCK / 64; w++) {
+            T o = sh[w][q];
+            r = is_min ? (o < r ? o : r) : (o > r ? o : r);
+        }
+        partial[(size_t)blockIdx.x * 12 + q] = r;
+    }
+}
+
+template <typename T>
+__global__ void minmax_finish_kernel(const T* __restrict__ partial, int nblocks, T* __restrict__ out)
+{
+    __shared__ T sh[256];
+    for (int q = 0; q < 12; q++) {
+        const bool is_min = (q % 6) < 3;
+        T r = is_min ? (T)INT_MAX : (T)INT_MIN;
+        for (int k = threadIdx.x; k < nblocks; k += 256) {
+            T o = partial[(size_t)k * 12 + q];
+            r = is_min ? (o < r ? o : r) : (o > r ? o : r);
+        }
+        sh[threadIdx.x] = r;
+        __syncthreads();
+        for (int s = 128; s > 0; s >>= 1) {
+            if ((int)threadIdx.x < s) {
+                T o = sh[threadIdx.x + s];
+                T m = sh[threadIdx.x];
+                sh[threadIdx.x] = is_min ? (o < m ? o : m) : (o > m ? o : m);
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) out[q] = sh[0];
+        __syncthreads();
+    }
+}
+
+// ---- 2 / 4. binning of (atom, image) pairs ---------------------------------------------------
+// Returns the storage index of the pair's bin inside the box, or -1 when it lies outside.
+template <typename T>
+__device__ __forceinline__ int locate(const Grid<T>& g, const T* __restrict__ x, long long pair, T* c,
+                                      int* sidx)
+{
+    const int m = (int)(pair / g.N);
+    const int p = (int)(pair - (long long)m * g.N);
+    const int k = m % g.img_dim[2];
+    const int j = (m / g.img_dim[2]) % g.img_dim[1];
+    const int i = m / (g.img_dim[2] * g.img_dim[1]);
+    int bin[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        c[a] = image_coord(x[(size_t)p * 3 + a], g.b[0][a], g.b[1][a], g.b[2][a], g.img_lo[0] + i,
+                           g.img_lo[1] + j, g.img_lo[2] + k);
+        bin[a] = bin_of(c[a], g.mn[a], g.bin_size) - g.rlo[a];
+        if (bin[a] < 0 || bin[a] >= g.rdim[a]) return -1;
+    }
+    *sidx = m * g.N + p;      // supercell index: image-major, x outer / z inner (structure.h:654-681)
+    return (bin[0] * g.rdim[1] + bin[1]) * g.rdim[2] + bin[2];
+}
+
+template <typename T>
+__global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __restrict__ counts)
+{
+    const long long pair = (long long)blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (pair >= (long long)g.N * g.nimg) return;
+    T c[3];
+    int sidx;
+    const int bin = locate(g, x, pair, c, &sidx);
+    if (bin >= 0) atomicAdd(&counts[bin], 1);
+}
+
+template <typename T>
+__global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ offsets,
+                            int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x)
+{
+    const long long pair = (long long)blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (pair >= (long long)g.N * g.nimg) return;
+    T c[3];
+    int sidx;
+    const int bin = locate(g, x, pair, c, &sidx);
+    if (bin < 0) return;
+    const int pos = offsets[bin] + atomicAdd(&cursor[bin], 1);
+    s_idx[pos] = sidx;
+    s_x[(size_t)pos * 3 + 0] = c[0];
+    s_x[(size_t)pos * 3 + 1] = c[1];
+    s_x[(size_t)pos * 3 + 2] = c[2];
+}
+
+// ---- 5. order inside a bin: descending supercell index (head insertion, binLinkedList.h:833) -
+template <typename T>
+__global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* __restrict__ s_idx,
+                               T* __restrict__ s_x)
+{
+    const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (b >= nbins) return;
+    const int beg = offsets[b], end = offsets[b + 1];
+    for (int i = beg + 1; i < end; i++) {
+        const int key = s_idx[i];
+        const T kx = s_x[(size_t)i * 3], ky = s_x[(size_t)i * 3 + 1], kz = s_x[(size_t)i * 3 + 2];
+        int j = i - 1;
+        while (j >= beg && s_idx[j] < key) {
+            s_idx[j + 1] = s_idx[j];
+            s_x[(size_t)(j + 1) * 3] = s_x[(size_t)j * 3];
+            s_x[(size_t)(j + 1) * 3 + 1] = s_x[(size_t)j * 3 + 1];
+            s_x[(size_t)(j + 1) * 3 + 2] = s_x[(size_t)j * 3 + 2];
+            j--;
+        }
+        s_idx[j + 1] = key;
+        s_x[(size_t)(j + 1) * 3] = kx;
+        s_x[(size_t)(j + 1) * 3 + 1] = ky;
+        s_x[(size_t)(j + 1) * 3 + 2] = kz;
+    }
+}
+
+// squared distance as the reference forms it: differences in T, squares and sum in double,
+// result rounded to T (binLinkedList.h:1008-1012, neighborList.h:318-322)
+template <typename T>
+__device__ __forceinline__ double dist2_double(T dx, T dy, T dz)
+{
+    const double a = (double)dx, b = (double)dy, c = (double)dz;
+    return __dadd_rn(__dadd_rn(__dmul_rn(a, a), __dmul_rn(b, b)), __dmul_rn(c, c));
+}
+
+// ---- 6. per-atom lists: one wavefront per centre atom ----------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(NBL_BLOCK)
+lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
+             const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
+             int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
+             T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
+             int* __restrict__ status)
+{
+    __shared__ int sh_start[NBL_BLOCK / 64][64];
+    __shared__ int sh_base[NBL_BLOCK / 64][64];
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int p = blockIdx.x * (NBL_BLOCK / 64) + wv;
+    if (p >= g.N) return;                         // whole wave leaves together
+    T c[3];
+    int cb[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        c[a] = x[(size_t)p * 3 + a];
+        cb[a] = bin_of(c[a], g.mn[a], g.bin_size);
+    }
+    const int e = g.ext_bins, side = 2 * e + 1, nruns = side * side;
+    // column `lane` = (dx, dy): binLinkedList.h:925-927 order, dz innermost
+    int start = 0, len = 0;
+    if (lane < nruns) {
+        const int bx = cb[0] + lane / side - e, by = cb[1] + lane % side - e;
+        int zlo = cb[2] - e, zhi = cb[2] + e;
+        // bins outside the reference's grid are skipped (binLinkedList.h:952-968); inside it the
+        // box kept here covers every bin within `e` of a centre atom
+        const bool ok = bx >= 0 && bx < g.nbin[0] && by >= 0 && by < g.nbin[1] &&
+                        bx >= g.rlo[0] && bx < g.rlo[0] + g.rdim[0] && by >= g.rlo[1] &&
+                        by < g.rlo[1] + g.rdim[1];
+        zlo = max(zlo, max(0, g.rlo[2]));
+        zhi = min(zhi, min(g.nbin[2] - 1, g.rlo[2] + g.rdim[2] - 1));
+        if (ok && zlo <= zhi) {
+            const int col = ((bx - g.rlo[0]) * g.rdim[1] + (by - g.rlo[1])) * g.rdim[2] - g.rlo[2];
+            start = offsets[col + zlo];
+            len = offsets[col + zhi + 1] - start;
+        }
+    }
+    const int incl = wave_inclusive_scan(len);
+    const int total = __shfl(incl, 63, 64);
+    sh_start[wv][lane] = start;
+    sh_base[wv][lane] = incl - len;
+    __builtin_amdgcn_wave_barrier();
+
+    int cnt = 0;
+    const size_t rowi = (size_t)p * umax;
+    for (int c0 = 0; c0 < total; c0 += 64) {
+        const int ci = c0 + lane;
+        bool in = false;
+        T dx = 0, dy = 0, dz = 0;
+        int sj = 0;
+        double d2d = 0.0;
+        if (ci < total) {
+            // last column whose base is <= ci
+            int lo = 0, hi = nruns - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+            }
+            const int ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
+            sj = s_idx[ent];
+            dx = sub_rn(s_x[(size_t)ent * 3 + 0], c[0]);
+            dy = sub_rn(s_x[(size_t)ent * 3 + 1], c[1]);
+            dz = sub_rn(s_x[(size_t)ent * 3 + 2], c[2]);
+            d2d = dist2_double(dx, dy, dz);
+            const T d2 = (T)d2d;                                   // `CoordType relative_distance2`
+            in = ((double)d2 < g.rcut2) && ((double)d2 > kEpsilon);   // binLinkedList.h:1014-1017
+        }
+        const unsigned long long mask = __ballot(in);
+        const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+        const int slot = cnt + rank;
+        if (in && slot < umax) {
+            firstneigh[rowi + slot] = sj % g.N;                     // neighborList.h:561
+            rcs[(rowi + slot) * 3 + 0] = dx;
+            rcs[(rowi + slot) * 3 + 1] = dy;
+            rcs[(rowi + slot) * 3 + 2] = dz;
+            if (keys) keys[rowi + slot] = (T)__dsqrt_rn(d2d);            // neighborList.h:318-322
+        }
+        cnt += __popcll(mask);
+    }
+    if (lane == 0) {
+        ilist[p] = p;
+        numneigh[p] = cnt;
+        types_out[p] = types[p];
+        if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
+        atomicMax(status + 1, cnt);
+    }
+    // padding: -1 / 0 (neighborList.h:557, 563)
+    const int first_pad = min(cnt, umax);
+    for (int s = first_pad + lane; s < umax; s += 64) firstneigh[rowi + s] = -1;
+    for (int s = first_pad * 3 + lane; s < umax * 3; s += 64) rcs[rowi * 3 + s] = (T)0;
+}
+
+// ---- 7. distance sort, emulating libstdc++ std::sort(indices, cmp = d[a] < d[b]) --------------
+// Introsort: median-of-three quicksort down to partitions of 16, heap sort beyond depth
+// 2*floor(log2 n), then one insertion sort pass.  Only the sequence of comparisons and moves
+// decides where equal keys end up, so the published algorithm is followed step by step.
+template <typename T>
+struct IdxSorter {
+    int* v;          // index array being sorted
+    const T* d;      // keys
+    __device__ bool less(int a, int b) const { return d[a] < d[b]; }
+    __device__ void iter_swap(int i, int j) { int t = v[i]; v[i] = v[j]; v[j] = t; }
+
+    __device__ void move_median_to_first(int result, int a, int b, int c)
+    {
+        if (less(v[a], v[b])) {
+            if (less(v[b], v[c])) iter_swap(result, b);
+            else if (less(v[a], v[c])) iter_swap(result, c);
+            else iter_swap(result, a);
+        } else if (less(v[a], v[c])) iter_swap(result, a);
+        else if (less(v[b], v[c])) iter_swap(result, c);
+        else iter_swap(result, b);
+    }
+    __device__ int unguarded_partition(int first, int last, int pivot)
+    {
+        while (true) {
+            while (less(v[first], v[pivot])) ++first;
+            --last;
+            while (less(v[pivot], v[last])) --last;
+            if (!(first < last)) return first;
+            iter_swap(first, last);
+            ++first;
+        }
+    }
+    __device__ void push_heap(int first, int hole, int top, int value)
+    {
+        int parent = (hole - 1) / 2;
+        while (hole > top && less(v[first + parent], value)) {
+            v[first + hole] = v[first + parent];
+            hole = parent;
+            parent = (hole - 1) / 2;
+        }
+        v[first + hole] = value;
+    }
+    __device__ void adjust_heap(int first, int hole, int len, int value)
+    {
+        const int top = hole;
+        int child = hole;
+        while (child < (len - 1) / 2) {
+            child = 2 * (child + 1);
+            if (less(v[first + child], v[first + (child - 1)])) child--;
+            v[first + hole] = v[first + child];
+            hole = child;
+        }
+        if ((len & 1) == 0 && child == (len - 2) / 2) {
+            child = 2 * (child + 1);
+            v[first + hole] = v[first + (child - 1)];
+            hole = child - 1;
+        }
+        push_heap(first, hole, top, value);
+    }
+    __device__ void heap_sort(int first, int last)      // __partial_sort(first, last, last)
+    {
+        const int len = last - first;
+        if (len >= 2) {                                  // __make_heap
+            int parent = (len - 2) / 2;
+            while (true) {
+                int value = v[first + parent];
+                adjust_heap(first, parent, len, value);
+                if (parent == 0) break;
+                parent--;
+            }
+        }
+        while (last - first > 1) {                       // __sort_heap / __pop_heap
+            --last;
+            int value = v[last];
+            v[last] = v[first];
+            adjust_heap(first, 0, last - first, value);
+        }
+    }
+    __device__ void unguarded_linear_insert(int last)
+    {
+        int val = v[last];
+        int next = last - 1;
+        while (less(val, v[next])) {
+            v[last] = v[next];
+            last = next;
+            --next;
+        }
+        v[last] = val;
+    }
+    __device__ void insertion_sort(int first, int last)
+    {
+        if (first == last) return;
+        for (int i = first + 1; i != last; ++i) {
+            if (less(v[i], v[first])) {
+                int val = v[i];
+                for (int k = i; k > first; --k) v[k] = v[k - 1];   // move_backward
+                v[first] = val;
+            } else unguarded_linear_insert(i);
+        }
+    }
+    __device__ void sort(int n)
+    {
+        if (n <= 1) return;
+        int depth = 2 * (31 - __clz(n));
+        // __introsort_loop, recursion on the right part turned into an explicit stack
+        int stack_first[64], stack_last[64], stack_depth[64];
+        int sp = 0;
+        int first = 0, last = n;
+        while (true) {
+            while (last - first > 16) {
+                if (depth == 0) { heap_sort(first, last); break; }
+                --depth;
+                const int mid = first + (last - first) / 2;
+                move_median_to_first(first, first + 1, mid, last - 1);
+                const int cut = unguarded_partition(first + 1, last, first);
+                // the reference recurses into [cut, last) first, then continues with [first, cut)
+                stack_first[sp] = first; stack_last[sp] = cut; stack_depth[sp] = depth; sp++;
+                first = cut;
+            }
+            if (sp == 0) break;
+            sp--;
+            first = stack_first[sp]; last = stack_last[sp]; depth = stack_depth[sp];
+        }
+        if (n > 16) {                                    // __final_insertion_sort
+            insertion_sort(0, 16);
+            for (int i = 16; i < n; ++i) unguarded_linear_insert(i);
+        } else insertion_sort(0, n);
+    }
+};
+
+template <typename T>
+__global__ void sort_rows_kernel(int N, int umax, const int* __restrict__ numneigh,
+                                 const T* __restrict__ keys, int* __restrict__ order)
+{
+    const int p = blockIdx.x * 64 + threadIdx.x;
+    if (p >= N) return;
+    const int n = min(numneigh[p], umax);
+    int* v = order + (size_t)p * umax;
+    for (int j = 0; j < n; j++) v[j] = j;
+    IdxSorter<T> s{v, keys + (size_t)p * umax};
+    s.sort(n);
+}
+
+// out row = tmp row gathered through `order` (SingleNeighborListArrangement, neighborList.h:46-67)
+template <typename T>
+__global__ void gather_rows_kernel(int N, int umax, const int* __restrict__ numneigh,
+                                   const int* __restrict__ order, const int* __restrict__ tmp_first,
+                                   const T* __restrict__ tmp_rcs, int* __restrict__ firstneigh,
+                                   T* __restrict__ rcs)
+{
+    const int p = (blockIdx.x * NBL_BLOCK + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    if (p >= N) return;
+    const int n = min(numneigh[p], umax);
+    const size_t row = (size_t)p * umax;
+    for (int s = lane; s < umax; s += 64) {
+        if (s < n) {
+            const int src = order[row + s];
+            firstneigh[row + s] = tmp_first[row + src];
+            rcs[(row + s) * 3 + 0] = tmp_rcs[(row + src) * 3 + 0];
+            rcs[(row + s) * 3 + 1] = tmp_rcs[(row + src) * 3 + 1];
+            rcs[(row + s) * 3 + 2] = tmp_rcs[(row + src) * 3 + 2];
+        } else {
+            firstneigh[row + s] = -1;
+            rcs[(row + s) * 3 + 0] = (T)0;
+            rcs[(row + s) * 3 + 1] = (T)0;
+            rcs[(row + s) * 3 + 2] = (T)0;
+        }
+    }
+}
+
+// ---- host ------------------------------------------------------------------------------------
+template <typename T>
+void host_cross(const T* a, const T* b, T* o)        // source/core/include/vec3Operation.h:87-93
+{
+    o[0] = a[1] * b[2] - a[2] * b[1];
+    o[1] = a[2] * b[0] - a[0] * b[2];
+    o[2] = a[0] * b[1] - a[1] * b[0];
+}
+
+template <typename T>
+T host_plane_distance(const T* v, const T* n)        // structure.h:818-842, vec3Operation.h:97-104
+{
+    // squares and their sum in double, square root rounded to T, division and dot product in T
+    T len = (T)std::sqrt((double)n[0] * (double)n[0] + (double)n[1] * (double)n[1] +
+                         (double)n[2] * (double)n[2]);
+    T u[3] = {(T)(n[0] / len), (T)(n[1] / len), (T)(n[2] / len)};
+    T d = v[0] * u[0] + v[1] * u[1] + v[2] * u[2];
+    return std::abs(d);
+}
+
+template <typename T>
+int nblist_build(const T* lattice, const int* types, const T* coords, int N, double rcut_in, int umax,
+                 int is_cart, const int* pbc, int sort, int* ilist, int* numneigh, int* firstneigh,
+                 T* rcs, int* types_out, int* max_nn_host, hipStream_t stream)
+{
+    A2P_REQUIRE(lattice && pbc, A2P_ERR_INVALID, "nblist: lattice and pbc must be host pointers");
+    A2P_REQUIRE(N > 0, A2P_ERR_INVALID, "nblist: the structure has no atoms");   // binLinkedList.h:659
+    A2P_REQUIRE(umax > 0 && rcut_in > 0, A2P_ERR_INVALID, "nblist: rcut and umax must be positive");
+    A2P_REQUIRE(types && coords && ilist && numneigh && firstneigh && rcs && types_out, A2P_ERR_INVALID,
+                "nblist: null device pointer");
+    A2P_REQUIRE((long long)N * umax < (1ll << 31), A2P_ERR_INVALID, "nblist: natoms*umax exceeds 2^31");
+
+    Grid<T> g;
+    g.N = N;
+    g.is_cart = is_cart;
+    g.rcut = (T)rcut_in;
+    g.rcut2 = (double)g.rcut * (double)g.rcut;
+    g.bin_size = g.rcut / 2;                                   // binLinkedList.h:664
+    for (int i = 0; i < 3; i++)
+        for (int j = 0; j < 3; j++) g.b[i][j] = lattice[i * 3 + j];
+    T nyz[3], nxz[3], nxy[3];
+    host_cross(g.b[1], g.b[2], nyz);
+    host_cross(g.b[0], g.b[2], nxz);
+    host_cross(g.b[0], g.b[1], nxy);
+    const T dplane[3] = {host_plane_distance(g.b[0], nyz), host_plane_distance(g.b[1], nxz),
+                         host_plane_distance(g.b[2], nxy)};
+    long long nimg = 1;
+    for (int a = 0; a < 3; a++) {
+        A2P_REQUIRE(dplane[a] > 0 && std::isfinite((double)dplane[a]), A2P_ERR_INVALID,
+                    "nblist: degenerate lattice");
+        const int ext = (int)std::ceil(g.rcut / dplane[a]);    // binLinkedList.h:672-676
+        const int scaling = pbc[a] ? ext * 2 + 1 : 1;
+        g.img_dim[a] = scaling;
+        g.img_lo[a] = -(scaling - 1) / 2;                      // structure.h:597-606 (odd scaling)
+        nimg *= scaling;
+    }
+    A2P_REQUIRE(nimg * N < (1ll << 31), A2P_ERR_INVALID,
+                "nblist: %lld images x %d atoms exceeds the reference's int supercell index", nimg, N);
+    g.nimg = (int)nimg;
+    g.ext_bins = (int)std::ceil(g.rcut / g.bin_size);          // binLinkedList.h:914-915
+    A2P_REQUIRE(g.ext_bins >= 1 && g.ext_bins <= 3, A2P_ERR_INVALID, "nblist: unsupported bin stencil");
+
+    // workspace A: x[N*3] | partial[nblocks*12] | ext[12]
+    const int nblocks = ceil_div(N, NBL_BLOCK);
+    void* wsA = nullptr;
+    size_t bytesA = ((size_t)N * 3 + (size_t)nblocks * 12 + 16) * sizeof(T);
+    int rc = ws_get(WS_NBL_A, bytesA, &wsA);
+    if (rc) return rc;
+    T* x = (T*)wsA;
+    T* partial = x + (size_t)N * 3;
+    T* ext_dev = partial + (size_t)nblocks * 12;
+    void* flags = nullptr;
+    rc = ws_get(WS_FLAGS, 64, &flags);
+    if (rc) return rc;
+    int* status = (int*)flags;
+
+    for (int a = 0; a < 3; a++) { g.mn[a] = 0; g.nbin[a] = 0; g.rlo[a] = 0; g.rdim[a] = 0; }
+    hipLaunchKernelGGL(coords_minmax_kernel<T>, dim3(nblocks), dim3(NBL_BLOCK), 0, stream, g, coords, x,
+                       partial);
+    hipLaunchKernelGGL(minmax_finish_kernel<T>, dim3(1), dim3(256), 0, stream, partial, nblocks, ext_dev);
+    T ext[12];
+    A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+
+    // find_pl_info4nblist + bin counts (structure.h:1013-1061, binLinkedList.h:685-688)
+    long long nregion = 1;
+    for (int a = 0; a < 3; a++) {
+        A2P_REQUIRE(std::isfinite((double)ext[a]) && std::isfinite((double)ext[3 + a]), A2P_ERR_INVALID,
+                    "nblist: non-finite coordinates");
+        const T mn = ext[a] - (T)kMargin;
+        const T mx = ext[3 + a] + (T)kMargin;
+        const T pl = mx - mn;
+        g.mn[a] = mn;
+        g.nbin[a] = (int)std::ceil(pl / g.bin_size);
+        const int cb_lo = (int)std::floor((ext[6 + a] - mn) / g.bin_size);
+        const int cb_hi = (int)std::floor((ext[9 + a] - mn) / g.bin_size);
+        g.rlo[a] = std::max(cb_lo - g.ext_bins, 0);
+        const int rhi = std::min(cb_hi + g.ext_bins, g.nbin[a] - 1);
+        g.rdim[a] = rhi - g.rlo[a] + 1;
+        A2P_REQUIRE(g.rdim[a] > 0, A2P_ERR_INVALID, "nblist: empty bin box");
+        nregion *= g.rdim[a];
+    }
+    A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID,
+                "nblist: %lld bins around the centre atoms; are the coordinates far outside the cell?",
+                nregion);
+    const int nb1 = (int)nregion + 1;
+
+    // workspace B: counts[nb1] | offsets[nb1] | cursor[nb1] | scan tmp, then (after the count is
+    // known) s_idx[total] | s_x[total*3], and for sort: keys[N*umax] | order[N*umax] | tmp rows
+    const int ntmp = scan_tmp_ints(nb1);
+    size_t ints = (size_t)nb1 * 3 + ntmp;
+    void* wsB = nullptr;
+    rc = ws_get(WS_NBL_B, ints * sizeof(int), &wsB);
+    if (rc) return rc;
+    int* counts = (int*)wsB;
+    int* offsets = counts + nb1;
+    int* cursor = offsets + nb1;
+    int* tmp = cursor + nb1;
+    rc = fill_zero(counts, (size_t)nb1 * sizeof(int), stream);
+    if (rc) return rc;
+    rc = fill_zero(cursor, (size_t)nb1 * sizeof(int), stream);
+    if (rc) return rc;
+    const long long npairs = (long long)N * g.nimg;
+    const int pair_blocks = ceil_div(npairs, NBL_BLOCK);
+    hipLaunchKernelGGL(count_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, counts);
+    rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
+    if (rc) return rc;
+    int total = 0;
+    A2P_HIP_CHECK(hipMemcpyAsync(&total, offsets + nregion, sizeof(int), hipMemcpyDeviceToHost, stream));
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+
+    size_t sorted_bytes = (size_t)total * (sizeof(int) + 3 * sizeof(T)) + 256;
+    size_t sort_bytes = sort ? (size_t)N * umax * (2 * sizeof(int) + 4 * sizeof(T)) + 256 : 0;
+    void* wsC = nullptr;
+    rc = ws_get(WS_MISC, sorted_bytes + sort_bytes, &wsC);
+    if (rc) return rc;
+    T* s_x = (T*)wsC;                                   // T first keeps double alignment
+    int* s_idx = (int*)(s_x + (size_t)total * 3);
+    char* sort_base = (char*)wsC + (sorted_bytes / 256) * 256;   // 256-byte aligned, inside the slack
+    T* tmp_rcs = nullptr;
+    T* keys = nullptr;
+    int* order = nullptr;
+    int* tmp_first = nullptr;
+    if (sort) {
+        tmp_rcs = (T*)sort_base;
+        keys = tmp_rcs + (size_t)N * umax * 3;
+        order = (int*)(keys + (size_t)N * umax);
+        tmp_first = order + (size_t)N * umax;
+    }
+
+    hipLaunchKernelGGL(fill_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
+                       s_idx, s_x);
+    hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
+                       (int)nregion, offsets, s_idx, s_x);
+    rc = fill_zero(status + 1, sizeof(int), stream);     // running maximum of the neighbour counts
+    if (rc) return rc;
+    const int list_blocks = ceil_div(N, NBL_BLOCK / 64);
+    hipLaunchKernelGGL(lists_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types, offsets,
+                       s_idx, s_x, umax, ilist, numneigh, sort ? tmp_first : firstneigh,
+                       sort ? tmp_rcs : rcs, types_out, keys, status);
+    if (sort) {
+        hipLaunchKernelGGL(sort_rows_kernel<T>, dim3(ceil_div(N, 64)), dim3(64), 0, stream, N, umax, numneigh,
+                           keys, order);
+        hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, N, umax,
+                           numneigh, order, tmp_first, tmp_rcs, firstneigh, rcs);
+    }
+    A2P_HIP_CHECK(hipGetLastError());
+
+    if (max_nn_host) {
+        int st[2] = {0, 0};
+        A2P_HIP_CHECK(hipMemcpyAsync(st, status, sizeof(st), hipMemcpyDeviceToHost, stream));
+        A2P_HIP_CHECK(hipStreamSynchronize(stream));
+        *max_nn_host = st[1];
+        if (st[1] > umax) {
+            rc = fill_zero(status, sizeof(int), stream);
+            if (rc) return rc;
+            set_error("nblist: an atom has %d neighbours, more than umax_num_neigh_atoms = %d", st[1], umax);
+            return A2P_ERR_OVERFLOW;
+        }
+    }
+    return A2P_OK;
+}
+
+}  // namespace
+}  // namespace a2p
+
+extern "C" {
+
+int a2p_nblist_build_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                         double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                         int* numneigh, int* firstneigh, float* rcs, int* types_out, int* max_numneigh,
+                         void* stream)
+{
+    return a2p::nblist_build<float>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
+                                    numneigh, firstneigh, rcs, types_out, max_numneigh, (hipStream_t)stream);
+}
+
+int a2p_nblist_build_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                         double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                         int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
+                         void* stream)
+{
+    return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
+                                     numneigh, firstneigh, rcs, types_out, max_numneigh,
+                                     (hipStream_t)stream);
+}
+}

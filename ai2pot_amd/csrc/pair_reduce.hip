@@ -200,6 +200,19 @@ __global__ void reduce_kernel(T* __restrict__ force, const T* __restrict__ seg_g
 
 }  // namespace
 
+int scan_tmp_ints(int n) { return ceil_div(n, SCAN_TILE) + 8; }
+
+int exclusive_scan_i32(const int* in, int* out, int n, int* tmp, hipStream_t stream)
+{
+    if (n <= 0) return A2P_OK;
+    const int ntiles = ceil_div(n, SCAN_TILE);
+    hipLaunchKernelGGL(scan_tile_sums, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, in, tmp, n);
+    hipLaunchKernelGGL(scan_tile_offsets, dim3(1), dim3(1024), 0, stream, tmp, ntiles, tmp + ntiles);
+    hipLaunchKernelGGL(scan_apply, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, in, out, tmp, n);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 template <typename T>
 int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
                 const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
@@ -225,7 +238,6 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
     int* offsets = counts + n;
     int* cursor = offsets + n;
     int* tiles = cursor + n;
-    int* total = tiles + ntiles;
     T* seg_g = (T*)((char*)ws + bytes);
 
     // counts and cursor start at zero (offsets is fully overwritten)
@@ -237,9 +249,8 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
     const int wave_blocks = ceil_div(rows * 64, 256);
     hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, counts, B, P, U, NF, binum,
                        bnumneigh, bfirstneigh, (int*)flags);
-    hipLaunchKernelGGL(scan_tile_sums, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, counts, tiles, n);
-    hipLaunchKernelGGL(scan_tile_offsets, dim3(1), dim3(1024), 0, stream, tiles, ntiles, total);
-    hipLaunchKernelGGL(scan_apply, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, counts, offsets, tiles, n);
+    rc = exclusive_scan_i32(counts, offsets, n, tiles, stream);
+    if (rc) return rc;
     hipLaunchKernelGGL(fill_kernel<T>, dim3(wave_blocks), dim3(256), 0, stream, seg_g, cursor, offsets,
                        pair_g, B, P, U, NF, binum, bnumneigh, bfirstneigh);
     hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)n * 16, 256)), dim3(256), 0, stream,

@@ -67,6 +67,32 @@ int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, 
                     const int* bfirstneigh, const double* brcs, const int* btypes, double* etot,
                     double* force, double* virial, double* descriptors, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Neighbour list -- replaces the compute of the CPython module function
+ * nblist.find_info4mlff(lattice, types, coords, rcut, umax, is_cart, pbc_xyz, sort)
+ * (source/nblist/bind/nblist_bind.cc:35-189 -> source/nblist/include/structure.h,
+ * binLinkedList.h:658-696, 808-836, 900-1031, neighborList.h:274-338, 532-578).
+ *
+ * lattice[9] (rows) and pbc[3] are HOST pointers; types[natoms], coords[natoms][3] and all
+ * outputs are device pointers: ilist[natoms], numneigh[natoms], firstneigh[natoms][umax]
+ * (-1 padded, indices modulo natoms), rcs[natoms][umax][3] (r_j - r_i, 0 padded),
+ * types_out[natoms].  Results are bit-identical to the reference's, in both sort modes.
+ * The call synchronises `stream` twice (extents and image count are read back to size the
+ * bin grid).  max_numneigh (HOST int, may be NULL): when given, the call synchronises once
+ * more, stores the largest neighbour count and returns A2P_ERR_OVERFLOW if it exceeds umax
+ * (rows are then truncated, never overrun; the reference overruns, neighborList.h:550).
+ * When NULL the check is left to a2p_check_status.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nblist_build_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                         double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                         int* numneigh, int* firstneigh, float* rcs, int* types_out, int* max_numneigh,
+                         void* stream);
+
+int a2p_nblist_build_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                         double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                         int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,112 @@
+"""GPU neighbour list against the CPU oracle: numneigh, firstneigh bit-exact and rcs bitwise
+identical in the same precision, in both sort modes (the sorted mode includes the tie order
+of libstdc++'s std::sort, which perfect lattices exercise heavily)."""
+import numpy as np
+import pytest
+
+from ai2pot_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_list(lattice, types, coords, rcut, umax, is_cart=True, pbc=(True, True, True), sort=False):
+    from ai2pot_amd import nblist
+    return nblist.find_info4mlff(np.ascontiguousarray(lattice), np.ascontiguousarray(types),
+                                 np.ascontiguousarray(coords), float(rcut), int(umax), bool(is_cart),
+                                 [bool(x) for x in pbc], bool(sort))
+
+
+def assert_same(a, b):
+    assert a[0] == b[0] and a[6] == b[6]
+    names = ("inum", "ilist", "numneigh", "firstneigh", "rcs", "types")
+    for i in (1, 2, 5):
+        assert np.array_equal(a[i], b[i]), names[i]
+    bad = np.nonzero((a[3] != b[3]).any(axis=1))[0]
+    assert bad.size == 0, "firstneigh differs in rows %s" % bad[:10]
+    assert a[4].dtype == b[4].dtype
+    assert np.array_equal(a[4].view(np.uint8), b[4].view(np.uint8)), "rcs not bitwise identical"
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("sort", [False, True])
+@pytest.mark.parametrize("rcut", [3.2, 5.0, 7.0])
+def test_mos2(oracle, dt, sort, rcut):
+    lat, types, frac = synth.mos2_fixture()
+    a = gpu_list(lat.astype(dt), types, frac.astype(dt), rcut, 200, is_cart=False, sort=sort)
+    b = oracle.nblist(lat.astype(dt), types, frac.astype(dt), rcut, 200, is_cart=False, sort=sort)
+    assert_same(a, b)
+    if rcut == 3.2:     # the reference's own assertion, source/nblist/tests/test_neighborList.cc:244
+        assert a[2].max() == 12
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("sort", [False, True])
+@pytest.mark.parametrize("pbc", [(True, True, True), (True, False, True), (False, False, False)])
+def test_triclinic(oracle, dt, sort, pbc):
+    L = np.array([[9.0, 0.3, -0.2], [1.1, 8.2, 0.4], [-0.7, 0.9, 10.1]])
+    fr = synth.rng_uniform(7, 3 * 60).reshape(60, 3)
+    ty = synth.rng_randint(8, 60, 3)
+    a = gpu_list(L.astype(dt), ty, fr.astype(dt), 5.5, 250, is_cart=False, pbc=pbc, sort=sort)
+    b = oracle.nblist(L.astype(dt), ty, fr.astype(dt), 5.5, 250, is_cart=False, pbc=pbc, sort=sort)
+    assert_same(a, b)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_unwrapped_coordinates_small_cell(oracle, dt):
+    """Atoms outside the cell (the reference never wraps) and a cell smaller than the cutoff,
+    so several images of the same atom are neighbours."""
+    L = np.array([[4.1, 0.0, 0.0], [0.5, 3.9, 0.0], [0.2, -0.3, 4.4]])
+    fr = synth.rng_uniform(17, 3 * 7).reshape(7, 3) * 3.0 - 1.0
+    ty = synth.rng_randint(18, 7, 2).astype(np.int64)      # int64 types are accepted
+    a = gpu_list(L.astype(dt), ty, fr.astype(dt), 6.0, 400, is_cart=False, sort=True)
+    b = oracle.nblist(L.astype(dt), ty, fr.astype(dt), 6.0, 400, is_cart=False, sort=True)
+    assert_same(a, b)
+    assert a[5].dtype == np.int32
+
+
+@pytest.mark.parametrize("sort", [False, True])
+def test_config2_size(oracle, sort):
+    lat, pos = synth.random_packed(4096, [49.8848] * 3, 2.2, 1003)
+    types = synth.rng_randint(2003, 4096, 3)
+    a = gpu_list(lat.astype(np.float32), types, pos.astype(np.float32), 7.0, 200, sort=sort)
+    b = oracle.nblist(lat.astype(np.float32), types, pos.astype(np.float32), 7.0, 200, sort=sort)
+    assert_same(a, b)
+
+
+def test_fcc_lattice_ties(oracle):
+    """A perfect FCC crystal: every shell is a set of exactly tied distances."""
+    lat, pos = synth.fcc_cell(6, 4.949, 0.0, 1)
+    types = synth.rng_randint(3, pos.shape[0], 3)
+    for dt in (np.float32, np.float64):
+        a = gpu_list(lat.astype(dt), types, pos.astype(dt), 7.0, 200, sort=True)
+        b = oracle.nblist(lat.astype(dt), types, pos.astype(dt), 7.0, 200, sort=True)
+        assert_same(a, b)
+
+
+def test_config5_recipe_reduced(oracle):
+    """Configuration 5's recipe (jittered FCC, 0.033 atoms/A^3, rcut 7) at 32^3 x 4 atoms."""
+    lat, pos = synth.fcc_cell(32, 316.7 / 64, 0.15, 1006)
+    types = synth.rng_randint(2006, pos.shape[0], 3)
+    a = gpu_list(lat.astype(np.float32), types, pos.astype(np.float32), 7.0, 200)
+    b = oracle.nblist(lat.astype(np.float32), types, pos.astype(np.float32), 7.0, 200)
+    assert_same(a, b)
+    # symmetry of a full list: j in N(i) <=> i in N(j), as a checksum of pair counts
+    inum, _, numneigh, first, rcs, _, _ = a
+    assert numneigh.sum() % 2 == 0
+    counts = np.bincount(first[first >= 0], minlength=inum)
+    assert np.array_equal(counts, numneigh)
+
+
+def test_overflow_and_type_errors(oracle):
+    lat, types, frac = synth.mos2_fixture()
+    with pytest.raises(RuntimeError):
+        gpu_list(lat, types, frac, 7.0, 20, is_cart=False)      # 54 neighbours > umax 20
+    from ai2pot_amd import nblist
+    with pytest.raises(TypeError):
+        nblist.find_info4mlff(lat, types, frac, 5, 20, False, [True] * 3, False)       # rcut not float
+    with pytest.raises(TypeError):
+        nblist.find_info4mlff(lat, types, frac, 5.0, 20, False, (True, True, True), False)  # pbc not list
+    with pytest.raises(TypeError):
+        nblist.find_info4mlff(lat.tolist(), types, frac, 5.0, 20, False, [True] * 3, False)
+    a = gpu_list(lat, types, frac, 5.0, 20, is_cart=False, sort=True)               # still usable
+    assert_same(a, oracle.nblist(lat, types, frac, 5.0, 20, is_cart=False, sort=True))
