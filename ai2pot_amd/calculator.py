@@ -1,0 +1,92 @@
+"""Device-resident molecular-dynamics step: neighbour-list rebuild followed by NEP energy /
+force / virial, with every buffer allocated once.
+
+This is the GPU counterpart of the reference's inference call stack
+(ai2pot/models/potential_utils.py:217-268 -> ai2pot/utils/usepot.py:76-97 ->
+nblist.find_info4mlff -> ai2pot/models/nep/nep.py:298-357 -> torch.ops.nep.nepToEFVOp), minus
+the host round trip: positions stay in HBM, the padded 7-tensor neighbour contract is
+produced and consumed on the device.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_c = ctypes
+
+
+def _vp(t):
+    return _c.c_void_p(0 if t is None else t.data_ptr())
+
+
+class NepCalculator:
+    """Holds one NEP model and the neighbour buffers of one structure size."""
+
+    def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
+                 sort=False, dtype=torch.float32, device="cuda:0"):
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.n = int(natoms)
+        self.umax = int(umax)
+        self.sort = bool(sort)
+        self.m = model
+        self.rcut = float(rcut if rcut is not None else model["rmax_radial"])   # nep.py:66
+        npdt = np.float32 if dtype == torch.float32 else np.float64
+        self.lattice = np.ascontiguousarray(lattice, npdt).reshape(9)
+        self.pbc = np.ascontiguousarray([1 if p else 0 for p in pbc], np.int32)
+        dev = self.device
+        f = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64)).to(dtype).to(dev)
+        self.coeffs, self.w0, self.b0, self.w1 = f(model["coeffs"]), f(model["w0"]), f(model["b0"]), f(model["w1"])
+        self.bias, self.q_scaler = f(model["type_bias"]), f(model["q_scaler"])
+        self.ntypes = int(np.asarray(model["type_map"]).size)
+        self.H = self.w1.numel() // self.ntypes
+        self.types = torch.from_numpy(np.ascontiguousarray(types, np.int32)).to(dev)
+        n, U = self.n, self.umax
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.binum = torch.full((1,), n, **i32)
+        self.ilist = torch.empty(n, **i32)
+        self.numneigh = torch.empty(n, **i32)
+        self.firstneigh = torch.empty((n, U), **i32)
+        self.rcs = torch.empty((n, U, 3), dtype=dtype, device=dev)
+        self.types_out = torch.empty(n, **i32)
+        self.etot = torch.empty(1, dtype=dtype, device=dev)
+        self.force = torch.empty((n, 3), dtype=dtype, device=dev)
+        self.virial = torch.empty(9, dtype=dtype, device=dev)
+        L = _lib.lib()
+        f32 = dtype == torch.float32
+        self._nbl = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
+        self._efv = L.a2p_nep_efv_f32 if f32 else L.a2p_nep_efv_f64
+
+    def rebuild(self, coords, stream):
+        rc = self._nbl(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
+                       _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
+                       self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self.sort else 0),
+                       _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
+                       _vp(self.types_out), None, stream)
+        _lib.check(rc)
+
+    def evaluate(self, stream):
+        m = self.m
+        rc = self._efv(_c.c_int(m["chebyshev_size"]), _c.c_int(m["n_radial_basis"]),
+                       _c.c_int(m["n_angular_basis"]), _c.c_int(m["l_max"]), _c.c_int(self.H),
+                       _c.c_int(self.ntypes), _vp(self.coeffs), _vp(self.w0), _vp(self.b0), _vp(self.w1),
+                       _vp(self.bias), _vp(self.q_scaler), _c.c_double(m["rmax_radial"]),
+                       _c.c_double(m["rmax_angular"]), _c.c_int(1), _c.c_int(self.n), _c.c_int(self.umax),
+                       _c.c_int(0), _vp(self.binum), _vp(self.ilist), _vp(self.numneigh),
+                       _vp(self.firstneigh), _vp(self.rcs), _vp(self.types_out), _vp(self.etot),
+                       _vp(self.force), _vp(self.virial), None, stream)
+        _lib.check(rc)
+
+    def step(self, coords):
+        """coords: [N, 3] Cartesian tensor on the device.  Returns (E[1], F[N,3], V[9]) views of
+        the calculator's own output buffers (overwritten by the next step)."""
+        stream = _c.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        self.rebuild(coords, stream)
+        self.evaluate(stream)
+        return self.etot, self.force, self.virial
+
+    def check(self):
+        """Raise if any kernel since the last check flagged a contract violation (synchronises)."""
+        _lib.check_status(torch.cuda.current_stream(self.device).cuda_stream)

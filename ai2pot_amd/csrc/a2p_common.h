@@ -60,6 +60,18 @@ enum StatusBits {
 
 inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+// ---- optional per-kernel timing with HIP events on the launching stream --------------------
+// While profiling is enabled (a2p_profile_enable), a ProfScope around a launch records an
+// event before and after it on `stream`; a2p_profile_report resolves them into per-label
+// totals.  Disabled (the default) it costs one branch.
+void prof_begin(const char* label, hipStream_t stream);
+void prof_end(hipStream_t stream);
+struct ProfScope {
+    hipStream_t s;
+    ProfScope(const char* label, hipStream_t stream) : s(stream) { prof_begin(label, stream); }
+    ~ProfScope() { prof_end(s); }
+};
+
 // ---- wave64 primitives -------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63); }
 

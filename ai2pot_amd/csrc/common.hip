@@ -52,6 +52,36 @@ int ws_get(int slot, size_t bytes, void** out)
     return A2P_OK;
 }
 
+// ---- per-kernel timing ---------------------------------------------------------------------
+namespace {
+struct ProfRec {
+    const char* label;
+    hipEvent_t start, stop;
+};
+bool g_prof_on = false;
+std::mutex g_prof_mutex;
+std::vector<ProfRec> g_prof_recs;
+thread_local hipEvent_t g_prof_pending_stop = nullptr;
+}  // namespace
+
+void prof_begin(const char* label, hipStream_t stream)
+{
+    if (!g_prof_on) return;
+    ProfRec r{label, nullptr, nullptr};
+    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
+    hipEventRecord(r.start, stream);
+    g_prof_pending_stop = r.stop;
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    g_prof_recs.push_back(r);
+}
+
+void prof_end(hipStream_t stream)
+{
+    if (!g_prof_on || !g_prof_pending_stop) return;
+    hipEventRecord(g_prof_pending_stop, stream);
+    g_prof_pending_stop = nullptr;
+}
+
 __global__ void fill_zero_kernel(uint32_t* p, size_t nwords)
 {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -65,7 +95,9 @@ int fill_zero(void* ptr, size_t bytes, hipStream_t stream)
     A2P_REQUIRE(bytes % 4 == 0, A2P_ERR_INVALID, "fill_zero: size not a multiple of 4");
     size_t nwords = bytes / 4;
     int blocks = (int)std::min<size_t>((nwords + 255) / 256, 256 * 32);
+    prof_begin("fill_zero", stream);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t*)ptr, nwords);
+    prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
@@ -94,8 +126,10 @@ template <typename T>
 int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
                     int out_stride, hipStream_t stream)
 {
+    prof_begin("finish_partials", stream);
     hipLaunchKernelGGL(finish_partials_kernel<T>, dim3(ncomp, B), dim3(256), 0, stream, out, partial,
                        nblocks, src_stride, out_stride);
+    prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
@@ -109,6 +143,40 @@ extern "C" {
 const char* a2p_last_error(void) { return a2p::last_error(); }
 
 int a2p_abi_version(void) { return 1; }
+
+void a2p_profile_enable(int on)
+{
+    std::lock_guard<std::mutex> lock(a2p::g_prof_mutex);
+    a2p::g_prof_on = on != 0;
+}
+
+int a2p_profile_report(char* buf, size_t buflen)
+{
+    A2P_HIP_CHECK(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lock(a2p::g_prof_mutex);
+    struct Acc { const char* label; double ms; long count; };
+    std::vector<Acc> acc;
+    for (auto& r : a2p::g_prof_recs) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+            bool found = false;
+            for (auto& a : acc)
+                if (std::string(a.label) == r.label) { a.ms += ms; a.count++; found = true; break; }
+            if (!found) acc.push_back({r.label, (double)ms, 1});
+        }
+        hipEventDestroy(r.start);
+        hipEventDestroy(r.stop);
+    }
+    a2p::g_prof_recs.clear();
+    size_t used = 0;
+    if (buf && buflen) buf[0] = 0;
+    for (auto& a : acc) {
+        int n = snprintf(buf + used, used < buflen ? buflen - used : 0, "%s %ld %.6f\n", a.label, a.count, a.ms);
+        if (n < 0 || used + (size_t)n >= buflen) break;
+        used += (size_t)n;
+    }
+    return A2P_OK;
+}
 
 int a2p_check_status(void* stream_)
 {

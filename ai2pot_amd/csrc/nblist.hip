@@ -343,7 +343,6 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         numneigh[p] = cnt;
         types_out[p] = types[p];
         if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
-        atomicMax(status + 1, cnt);
     }
     // padding: -1 / 0 (neighborList.h:557, 563)
     const int first_pad = min(cnt, umax);
@@ -521,6 +520,17 @@ __global__ void gather_rows_kernel(int N, int umax, const int* __restrict__ numn
     }
 }
 
+__global__ void int_max_kernel(const int* __restrict__ v, int n, int* __restrict__ out)
+{
+    __shared__ int sh[4];
+    int m = 0;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) m = max(m, v[i]);
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(out, max(max(sh[0], sh[1]), max(sh[2], sh[3])));
+}
+
 // ---- host ------------------------------------------------------------------------------------
 template <typename T>
 void host_cross(const T* a, const T* b, T* o)        // source/core/include/vec3Operation.h:87-93
@@ -598,9 +608,13 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     int* status = (int*)flags;
 
     for (int a = 0; a < 3; a++) { g.mn[a] = 0; g.nbin[a] = 0; g.rlo[a] = 0; g.rdim[a] = 0; }
+    prof_begin("nbl_coords_minmax", stream);
     hipLaunchKernelGGL(coords_minmax_kernel<T>, dim3(nblocks), dim3(NBL_BLOCK), 0, stream, g, coords, x,
                        partial);
+    prof_end(stream);
+    prof_begin("nbl_coords_minmax", stream);
     hipLaunchKernelGGL(minmax_finish_kernel<T>, dim3(1), dim3(256), 0, stream, partial, nblocks, ext_dev);
+    prof_end(stream);
     T ext[12];
     A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
     A2P_HIP_CHECK(hipStreamSynchronize(stream));
@@ -645,7 +659,9 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (rc) return rc;
     const long long npairs = (long long)N * g.nimg;
     const int pair_blocks = ceil_div(npairs, NBL_BLOCK);
+    prof_begin("nbl_count", stream);
     hipLaunchKernelGGL(count_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, counts);
+    prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
     int total = 0;
@@ -671,25 +687,42 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         tmp_first = order + (size_t)N * umax;
     }
 
+    prof_begin("nbl_fill", stream);
+
     hipLaunchKernelGGL(fill_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
                        s_idx, s_x);
+
+    prof_end(stream);
+    prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
                        (int)nregion, offsets, s_idx, s_x);
-    rc = fill_zero(status + 1, sizeof(int), stream);     // running maximum of the neighbour counts
-    if (rc) return rc;
+    prof_end(stream);
     const int list_blocks = ceil_div(N, NBL_BLOCK / 64);
+    prof_begin("nbl_lists", stream);
     hipLaunchKernelGGL(lists_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types, offsets,
                        s_idx, s_x, umax, ilist, numneigh, sort ? tmp_first : firstneigh,
                        sort ? tmp_rcs : rcs, types_out, keys, status);
+    prof_end(stream);
     if (sort) {
+        prof_begin("nbl_sort_rows", stream);
         hipLaunchKernelGGL(sort_rows_kernel<T>, dim3(ceil_div(N, 64)), dim3(64), 0, stream, N, umax, numneigh,
                            keys, order);
+        prof_end(stream);
+        prof_begin("nbl_gather_rows", stream);
         hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, N, umax,
                            numneigh, order, tmp_first, tmp_rcs, firstneigh, rcs);
+        prof_end(stream);
     }
     A2P_HIP_CHECK(hipGetLastError());
 
     if (max_nn_host) {
+        // largest neighbour count: block-wise maxima, one integer atomic per block
+        rc = fill_zero(status + 1, sizeof(int), stream);
+        if (rc) return rc;
+        prof_begin("nbl_max", stream);
+        hipLaunchKernelGGL(int_max_kernel, dim3(std::min(ceil_div(N, 256), 1024)), dim3(256), 0, stream,
+                           numneigh, N, status + 1);
+        prof_end(stream);
         int st[2] = {0, 0};
         A2P_HIP_CHECK(hipMemcpyAsync(st, status, sizeof(st), hipMemcpyDeviceToHost, stream));
         A2P_HIP_CHECK(hipStreamSynchronize(stream));

@@ -521,7 +521,9 @@ int launch(const NepArgs<T>& a, size_t lds, hipStream_t stream)
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
+    prof_begin("nep_efv_kernel", stream);
     hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(NEP_BLOCK), lds, stream, a);
+    prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }

@@ -206,9 +206,15 @@ int exclusive_scan_i32(const int* in, int* out, int n, int* tmp, hipStream_t str
 {
     if (n <= 0) return A2P_OK;
     const int ntiles = ceil_div(n, SCAN_TILE);
+    prof_begin("scan", stream);
     hipLaunchKernelGGL(scan_tile_sums, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, in, tmp, n);
+    prof_end(stream);
+    prof_begin("scan", stream);
     hipLaunchKernelGGL(scan_tile_offsets, dim3(1), dim3(1024), 0, stream, tmp, ntiles, tmp + ntiles);
+    prof_end(stream);
+    prof_begin("scan", stream);
     hipLaunchKernelGGL(scan_apply, dim3(ntiles), dim3(SCAN_BLOCK), 0, stream, in, out, tmp, n);
+    prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
@@ -247,14 +253,20 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
     if (rc) return rc;
 
     const int wave_blocks = ceil_div(rows * 64, 256);
+    prof_begin("reduce_count", stream);
     hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, counts, B, P, U, NF, binum,
                        bnumneigh, bfirstneigh, (int*)flags);
+    prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, n, tiles, stream);
     if (rc) return rc;
+    prof_begin("reduce_fill", stream);
     hipLaunchKernelGGL(fill_kernel<T>, dim3(wave_blocks), dim3(256), 0, stream, seg_g, cursor, offsets,
                        pair_g, B, P, U, NF, binum, bnumneigh, bfirstneigh);
+    prof_end(stream);
+    prof_begin("reduce_sum", stream);
     hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)n * 16, 256)), dim3(256), 0, stream,
                        force, seg_g, offsets, counts, n);
+    prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }

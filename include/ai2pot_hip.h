@@ -37,6 +37,15 @@ int a2p_abi_version(void);
  * (source/nblist/include/neighborList.h:550, commented-out assert). */
 int a2p_check_status(void* stream);
 
+/* Per-kernel timing for benchmarks (no counterpart in the reference, which leaves timing to
+ * commented-out std::chrono calls, interface/lammps/AI2POT/pair_ai2pot.cpp:392-442).  While
+ * enabled, every kernel launch of the library is bracketed by HIP events on its stream.
+ * a2p_profile_report synchronises the device and writes one line per kernel label,
+ * "<label> <launch count> <total milliseconds>\n", into buf (truncated to buflen), then
+ * clears the records. */
+void a2p_profile_enable(int on);
+int a2p_profile_report(char* buf, size_t buflen);
+
 /* ------------------------------------------------------------------------------------------
  * NEP energy / force / virial -- replaces the compute of torch.ops.nep.nepToEFVOp /
  * nepToEFOp / nepToDescriptorsOp (source/descriptor/nep/bind/nep_bind.cc:26-135, 278-311;

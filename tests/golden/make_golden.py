@@ -1,0 +1,127 @@
+"""Writes tests/golden/*.npz: inputs and the outputs of the reference's own C++ code
+(compiled from /root/reference by oracle/Makefile into oracle/_ref) for small cases.
+
+    make -C oracle ref && python tests/golden/make_golden.py
+
+The fixtures are data only (arrays); they let the CPU test-suite pin this repository's
+oracle, and the GPU tests pin the HIP path, where the reference tree is absent.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "..", ".."))
+import oracle  # noqa: E402
+from ai2pot_amd import mtp_param, synth  # noqa: E402
+
+
+def trim(out):
+    """Drop the padding columns beyond the longest row to keep the files small."""
+    inum, ilist, numneigh, first, rcs, types, nghost = out
+    w = max(int(numneigh.max()), 1)
+    return dict(ilist=ilist, numneigh=numneigh, firstneigh=first[:, :w], rcs=rcs[:, :w], types=types)
+
+
+def nblist_cases():
+    cases = {}
+    lat, types, frac = synth.mos2_fixture()
+    L = np.array([[9.0, 0.3, -0.2], [1.1, 8.2, 0.4], [-0.7, 0.9, 10.1]])
+    fr = synth.rng_uniform(7, 3 * 60).reshape(60, 3)
+    ty = synth.rng_randint(8, 60, 3)
+    for dt in (np.float32, np.float64):
+        for sort in (0, 1):
+            for rc in (3.2, 5.0):
+                cases["mos2_%s_s%d_rc%.1f" % (dt.__name__, sort, rc)] = (
+                    lat.astype(dt), types, frac.astype(dt), rc, 64, False, (1, 1, 1), sort)
+            for pbc in ((1, 1, 1), (1, 0, 1), (0, 0, 0)):
+                cases["tri_%s_s%d_p%d%d%d" % ((dt.__name__, sort) + pbc)] = (
+                    L.astype(dt), ty, fr.astype(dt), 5.5, 80, False, pbc, sort)
+    out = {}
+    for name, (la, t, c, rc, umax, cart, pbc, sort) in cases.items():
+        res = oracle.ref_nblist(la, t, c, rc, umax, is_cart=cart, pbc=pbc, sort=bool(sort))
+        out[name + "/in_lattice"] = la
+        out[name + "/in_types"] = t
+        out[name + "/in_coords"] = c
+        out[name + "/in_params"] = np.array([rc, umax, int(cart), pbc[0], pbc[1], pbc[2], sort], np.float64)
+        for k, v in trim(res).items():
+            out[name + "/" + k] = v
+    np.savez_compressed(os.path.join(HERE, "nblist.npz"), **out)
+    print("nblist.npz", len(cases), "cases")
+
+
+def nep_cases():
+    out = {}
+    lat, types, frac = synth.mos2_fixture()
+    nb = synth.pack_batch([oracle.ref_nblist(lat, types, frac, 5.0, 20, is_cart=False, sort=True)])
+    m = synth.nep_model_closed_form()
+    e, f, v = oracle.ref_nep_efv(m, nb, np.float64)
+    d = oracle.ref_nep_descriptors(m, nb, np.float64)
+    out.update({"mos2/E": e, "mos2/F": f, "mos2/V": v, "mos2/D": d})
+    lat2, pos2 = synth.random_packed(96, [12.0, 13.0, 12.5], 2.2, 11)
+    ty2 = synth.rng_randint(12, 96, 3)
+    m2 = synth.nep_model()
+    for dt in (np.float64, np.float32):
+        o = oracle.ref_nblist(lat2.astype(dt), ty2, pos2.astype(dt), 7.0, 160)
+        nb2 = synth.pack_batch([o])
+        e, f, v = oracle.ref_nep_efv(m2, nb2, dt)
+        tag = "rand_" + dt.__name__
+        out.update({tag + "/E": e, tag + "/F": f, tag + "/V": v,
+                    tag + "/D": oracle.ref_nep_descriptors(m2, nb2, dt)})
+    np.savez_compressed(os.path.join(HERE, "nep.npz"), **out)
+    print("nep.npz")
+
+
+def mtp_cases():
+    out = {}
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    for level, nt in ((8, 2), (10, 1), (16, 3)):
+        ty = synth.rng_randint(22, 48, nt)
+        t = mtp_param.mtp_param(level)
+        ref_t = oracle.ref_mtp_param(level)
+        for k in ("alpha_index_basic", "alpha_index_times", "alpha_moment_mapping"):
+            assert np.array_equal(t[k], ref_t[k])
+        m = synth.mtp_model(t, nt, 8, 5.0, 0.5 if level == 10 else 1.8, 3000 + level)
+        o = oracle.ref_nblist(lat, ty, pos, 5.0, 100)
+        nb = synth.pack_batch([o, o])
+        nb["brcs"][1] *= 1.01
+        e, f, v = oracle.ref_mtp_efv(m, nb)
+        B, P = nb["bilist"].shape
+        labels = dict(energy=synth.rng_normal(1, B, -4 * 48, 3),
+                      force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                      virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+        r = oracle.ref_mtp_loss_step(m, nb, (1.0, 0.7, 0.3), labels)
+        tag = "L%02d" % level
+        out.update({tag + "/E": e, tag + "/F": f, tag + "/V": v})
+        for k, val in r.items():
+            out[tag + "/loss_" + k] = val
+        out[tag + "/table_sizes"] = np.array([t["alpha_moments_count"], t["alpha_index_basic"].shape[0],
+                                              t["alpha_index_times"].shape[0],
+                                              t["alpha_moment_mapping"].size, t["nmus"]])
+    np.savez_compressed(os.path.join(HERE, "mtp.npz"), **out)
+    print("mtp.npz")
+
+
+def fvt_cases():
+    rng = np.random.default_rng(0)
+    inum, U, ng = 10, 6, 3
+    nn = rng.integers(0, U + 1, inum).astype(np.int32)
+    fn = rng.integers(0, inum + ng, (inum, U)).astype(np.int32)
+    il = rng.permutation(inum).astype(np.int32)
+    dei = rng.normal(size=(inum, U, 3))
+    rcs = rng.normal(size=(inum, U, 3))
+    gin = rng.normal(size=(inum + ng, 3))
+    f, g = oracle.ref_fvt_force(il, nn, fn, ng, dei, gin)
+    v, d1, d2 = oracle.ref_fvt_virial(nn, rcs, dei, True)
+    np.savez_compressed(os.path.join(HERE, "fvt.npz"), ilist=il, numneigh=nn, firstneigh=fn, nghost=ng,
+                        dei_drij=dei, rcs=rcs, grad_in=gin, force=f, grad_out=g, virial=v, der1=d1, der2=d2)
+    print("fvt.npz")
+
+
+if __name__ == "__main__":
+    assert oracle.ref_available("nblist"), "build oracle/_ref first: make -C oracle ref"
+    nblist_cases()
+    nep_cases()
+    mtp_cases()
+    fvt_cases()
