@@ -185,6 +185,20 @@ def mtp_model(tables, ntypes, chebyshev_size, rmax, rmin, seed, lo=-0.1, hi=0.1,
     return m
 
 
+def mtp_model_closed_form(tables):
+    """Parameter fill of the reference's linear-MTP unit test
+    (source/descriptor/mtpr/tests/test_linearMtp.cc:142-156, 272-279, 317-324; level 16,
+    two species, rmax 5, rmin 2), for the MoS2 known answer E = -0.938157350795572."""
+    S = len(tables["alpha_moment_mapping"])
+    ncoef = 2 * 2 * tables["nmus"] * 8
+    m = dict(tables)
+    m.update(chebyshev_size=8, scaling=1.0, rmax=5.0, rmin=2.0,
+             coeffs=0.01 + 0.001 * np.arange(ncoef), linear_coeffs=0.01 + 0.001 * np.arange(S),
+             type_bias=np.array([-0.1, -0.2]), q_scaler=0.67 + 0.05 * np.arange(S),
+             type_map=np.array([42, 16], np.int32))
+    return m
+
+
 # ----------------------------------------------------------------------------------------
 # batching (the 7-tensor contract of the E/F/V operators)
 # ----------------------------------------------------------------------------------------
