@@ -1,0 +1,877 @@
+// Linear Moment Tensor Potential for gfx950: energy / force / virial, and the analytic
+// gradient of the training loss w.r.t. coeffs, linear_coeffs and type_bias.
+//
+// One wavefront (a 64-thread workgroup) per centre atom; the moment vector M, its adjoint
+// and (for the loss gradient) the tangent and mixed vectors live in LDS.  Neighbours are
+// processed in chunks of 32: a per-neighbour table (powers of the unit vector, contracted
+// radial functions g_mu(r) = sum_k c[ti,tj,mu,k] f_k(r) and their r-derivatives) is staged
+// in LDS, then
+//   basic moments : lane <- basic moment i,  M_i += sum_j g_mu(r_j) ux^a uy^b uz^c
+//                   (x^a y^b z^c / r^(a+b+c) of the reference, include/mtpBasis.h:472-519,
+//                    written with the unit vector u = r_ij / r)
+//   products      : level-ordered gather over the host-built plan (mtp_plan.h)
+//   energy        : E_i = bias[t] + sum_s lin[s] M[map[s]] / q_scaler[s]  (linearMtp.h:281-285)
+//   adjoint       : seed + reverse gather                                  (linearMtp.h:292-306)
+//   pair forces   : lane <- (neighbour, half of the basic moments):
+//                   dE_i/dr_ij = u sum_i adj_i m_i (g' - k g / r) + (1/r) sum_i adj_i g grad_u m_i
+//                   -> pair buffer, folded onto neighbours by a2p::pair_reduce (no float atomics)
+// The loss gradient adds the tangent sweep (include/linearMtpLoss.h:371-398), the mixed
+// adjoint (:417-434) and the coefficient-gradient pass (:438-536) in the same structure;
+// per-structure gradients are accumulated per workgroup and summed by a second kernel.
+#include "a2p_common.h"
+#include "mtp_plan.h"
+
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+#include <set>
+
+namespace a2p {
+namespace {
+
+constexpr int MTP_NC = 32;        // neighbours per chunk
+constexpr int MTP_KMAX = 16;      // radial basis size limit
+constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
+
+template <typename T>
+struct MtpArgs {
+    MtpPlanDevice p;
+    int K, ntypes;
+    T scaling, rmax, rmin;
+    const T *coeffs, *lin, *bias, *q_scaler;
+    int B, P, U, nghost;
+    const int *binum, *bilist, *bnumneigh, *bfirstneigh;
+    const T* brcs;
+    const int* btypes;
+    T* force;          // [B, P+nghost, 3]
+    T* pair_g;         // [B*P, U, 3]
+    double* partial;   // [B, P, 10]  energy + virial per atom
+    int* status;
+    int E;             // table entries per neighbour
+    // loss gradient mode
+    const T* cE;       // [B]        2 e_w / N (E - E_dft)
+    const T* dFs;      // [B, P, 3]  2 f_w / (3N) (F - F_dft)
+    const T* dVs;      // [B, 9]     2 v_w / (9N) (V - V_dft)
+    T* gpart;          // [B, P, ngrad] per-atom gradient rows (ngrad = ncoef + n_scalar + ntypes)
+    int ngrad;
+};
+
+__device__ __forceinline__ float sqrt_t(float x) { return sqrtf(x); }
+__device__ __forceinline__ double sqrt_t(double x) { return sqrt(x); }
+
+// Per-neighbour table for neighbours [c0, c0+nc) of the row, built by lanes j < nc.
+// Layout per neighbour (E entries of T): ux^0..kmax | uy^.. | uz^.. | g[nmus] | dg[nmus] |
+// ux uy uz 1/r | (loss mode) wx wy wz w.u | f[K] | df[K]
+template <typename T, bool LOSS>
+__device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, int lane, int nc, int c0,
+                                            const T* rcs, const int* first, const int* types, int ti,
+                                            int center, int b, int NF, int* nj_out, bool* valid_out,
+                                            T* d_out)
+{
+    const int kmax = a.p.kmax, nmus = a.p.nmus, K = a.K;
+    const int OX = 0, OY = kmax + 1, OZ = 2 * (kmax + 1), OG = 3 * (kmax + 1), ODG = OG + nmus,
+              OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
+    *valid_out = false;
+    *nj_out = center;
+    if (lane < nc) {
+        const int jj = c0 + lane;
+        const T x = rcs[jj * 3 + 0], y = rcs[jj * 3 + 1], z = rcs[jj * 3 + 2];
+        d_out[0] = x; d_out[1] = y; d_out[2] = z;
+        const T r = sqrt_t(x * x + y * y + z * z);
+        int nj = first[jj];
+        if ((unsigned)nj >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); nj = center; }
+        int tj = types[nj];
+        if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
+        *nj_out = nj;
+        const bool valid = !(r > a.rmax);                // mtpBasis.h:457, linearMtp.h:316
+        *valid_out = valid;
+        T* t = tab + lane * a.E;
+        const T rinv = (T)1 / r;
+        const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+        T px = (T)1, py = (T)1, pz = (T)1;
+        for (int k = 0; k <= kmax; k++) {
+            t[OX + k] = px; t[OY + k] = py; t[OZ + k] = pz;
+            px *= ux; py *= uy; pz *= uz;
+        }
+        t[OU + 0] = ux; t[OU + 1] = uy; t[OU + 2] = uz; t[OU + 3] = rinv;
+        // radial functions, basis.h:154-196, 351-381, 620-637
+        const T span = a.rmax - a.rmin;
+        const T xx = ((T)2 * r - (a.rmax + a.rmin)) / span;
+        const T dxx = (T)2 / span;
+        const T u = (r - a.rmin) / span;
+        T s = (T)0, ds = (T)0;
+        if (valid && r >= a.rmin && r < a.rmax) {
+            s = u * u * u * ((T)-6 * u * u + (T)15 * u - (T)10) + (T)1;
+            ds = (T)1 / span * ((T)-30 * u * u * u * u + (T)60 * u * u * u - (T)30 * u * u);
+        }
+        T g[MTP_NMUS_MAX], dg[MTP_NMUS_MAX];
+#pragma unroll
+        for (int m = 0; m < MTP_NMUS_MAX; m++) { g[m] = (T)0; dg[m] = (T)0; }
+        const T* c = a.coeffs + (size_t)(ti * a.ntypes + tj) * nmus * K;
+        T t0 = (T)1, t1 = xx, d0 = (T)0, d1 = (T)1;
+        for (int k = 0; k < K; k++) {
+            T tv, dv;
+            if (k == 0) { tv = t0; dv = d0; }
+            else if (k == 1) { tv = t1; dv = d1; }
+            else {
+                tv = (T)2 * xx * t1 - t0;
+                dv = (T)2 * t1 + (T)2 * xx * d1 - d0;
+                t0 = t1; t1 = tv; d0 = d1; d1 = dv;
+            }
+            const T f = a.scaling * s * tv;
+            const T df = a.scaling * (ds * tv + s * dv * dxx);
+            if (LOSS) { t[OF + k] = f; t[ODF + k] = df; }
+#pragma unroll
+            for (int m = 0; m < MTP_NMUS_MAX; m++)
+                if (m < nmus) { g[m] += c[m * K + k] * f; dg[m] += c[m * K + k] * df; }
+        }
+#pragma unroll
+        for (int m = 0; m < MTP_NMUS_MAX; m++)
+            if (m < nmus) { t[OG + m] = g[m]; t[ODG + m] = dg[m]; }
+        if (LOSS) {
+            // w_a = dFs[centre]_a - dFs[neighbour]_a - sum_b dVs[a,b] r_b   (linearMtpLoss.h:371-386)
+            const T* fc = a.dFs + ((size_t)b * a.P + center) * 3;
+            const T* fn = a.dFs + ((size_t)b * a.P + nj) * 3;
+            const T* dv = a.dVs + (size_t)b * 9;
+            T w[3];
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+                w[q] = fc[q] - fn[q] - (dv[q * 3 + 0] * x + dv[q * 3 + 1] * y + dv[q * 3 + 2] * z);
+            t[OW + 0] = w[0]; t[OW + 1] = w[1]; t[OW + 2] = w[2];
+            t[OW + 3] = w[0] * ux + w[1] * uy + w[2] * uz;
+        }
+    }
+}
+
+// forward products: M[dst] = sum mult M[m0] M[m1]; with TANGENT also the product rule on Tg
+template <typename T, bool TANGENT>
+__device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, int lane)
+{
+    for (int l = 0; l < p.n_levels; l++) {
+        for (int s = p.f_level[l] + lane; s < p.f_level[l + 1]; s += 64) {
+            T acc = (T)0, tacc = (T)0;
+            for (int t = p.f_begin[s]; t < p.f_begin[s + 1]; t++) {
+                const int m0 = p.f_m0[t], m1 = p.f_m1[t];
+                const T mult = (T)p.f_mult[t];
+                const T v0 = M[m0], v1 = M[m1];
+                acc += mult * v0 * v1;
+                if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+            }
+            const int dst = p.f_dst[s];
+            M[dst] = acc;
+            if (TANGENT) Tg[dst] = tacc;
+        }
+        __syncthreads();
+    }
+}
+
+// reverse gather: X[m] += sum mult (X[dst] M[other] (+ A[dst] Tg[other] when MIXED))
+template <typename T, bool MIXED>
+__device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M, T* X, const T* A,
+                                              const T* Tg, int lane)
+{
+    for (int l = p.n_levels - 1; l >= 0; l--) {
+        for (int s = p.r_level[l] + lane; s < p.r_level[l + 1]; s += 64) {
+            const int m = p.r_src[s];
+            T acc = X[m];
+            for (int t = p.r_begin[s]; t < p.r_begin[s + 1]; t++) {
+                const int dst = p.r_dst[t], other = p.r_other[t];
+                const T mult = (T)p.r_mult[t];
+                acc += X[dst] * mult * M[other];
+                if (MIXED) acc += mult * A[dst] * Tg[other];
+            }
+            X[m] = acc;
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T, bool LOSS>
+__global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const MtpPlanDevice& p = a.p;
+    const int lane = threadIdx.x;
+    const int ii = blockIdx.x, b = blockIdx.y;
+    const int NF = a.P + a.nghost;
+    const size_t row = (size_t)b * a.P + ii;
+    const int n_moms = p.n_moms, n_basic = p.n_basic, nmus = p.nmus, kmax = p.kmax, K = a.K, E = a.E;
+    const int OX = 0, OY = kmax + 1, OZ = 2 * (kmax + 1), OG = 3 * (kmax + 1), ODG = OG + nmus,
+              OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
+    const int ncoef = a.ntypes * a.ntypes * nmus * K;
+
+    T* M = (T*)smem_raw;
+    T* A = M + n_moms;
+    T* Tg = A + n_moms;                      // loss mode only
+    T* Bm = Tg + (LOSS ? n_moms : 0);        // loss mode only
+    T* tab = Bm + (LOSS ? n_moms : 0);
+    T* pq = tab + MTP_NC * E;                // loss mode: P[nc][nmus] | Q[nc][nmus]
+
+    if (ii >= a.binum[b]) {                  // padded row: contributes nothing
+        if (!LOSS && lane < 10) a.partial[row * 10 + lane] = 0.0;
+        if (LOSS)
+            for (int q = lane; q < a.ngrad; q += 64) a.gpart[row * a.ngrad + q] = (T)0;
+        return;
+    }
+    int center = a.bilist[row];
+    int nn = a.bnumneigh[row];
+    if (nn > a.U) { if (lane == 0) atomicOr(a.status, ST_NEIGH_OVERFLOW); nn = a.U; }
+    if ((unsigned)center >= (unsigned)NF) { if (lane == 0) atomicOr(a.status, ST_BAD_NEIGHBOR); center = 0; nn = 0; }
+    const int* types = a.btypes + (size_t)b * NF;
+    int ti = types[center];
+    if ((unsigned)ti >= (unsigned)a.ntypes) { if (lane == 0) atomicOr(a.status, ST_BAD_TYPE); ti = 0; nn = 0; }
+    const int* first = a.bfirstneigh + row * a.U;
+    const T* rcs = a.brcs + row * a.U * 3;
+
+    for (int i = lane; i < n_moms; i += 64) {
+        M[i] = (T)0; A[i] = (T)0;
+        if (LOSS) { Tg[i] = (T)0; Bm[i] = (T)0; }
+    }
+    __syncthreads();
+
+    // ---- basic moments (and their tangents) --------------------------------------------------
+    for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
+        const int nc = min(MTP_NC, nn - c0);
+        int nj; bool valid; T d[3];
+        build_table<T, LOSS>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+        __syncthreads();
+        for (int i = lane; i < n_basic; i += 64) {
+            const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
+                      ec = p.basic[i * 4 + 3];
+            const T kk = (T)(ea + eb + ec);
+            T acc = (T)0, tacc = (T)0;
+            for (int j = 0; j < nc; j++) {
+                const T* t = tab + j * E;
+                const T g = t[OG + mu];
+                const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
+                const T m = xa * yb * zc;
+                acc += g * m;
+                if (LOSS) {
+                    const T dg = t[ODG + mu], rinv = t[OU + 3], wu = t[OW + 3];
+                    const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
+                                 (T)eb * xa * t[OY + max(eb - 1, 0)] * zc * t[OW + 1] +
+                                 (T)ec * xa * yb * t[OZ + max(ec - 1, 0)] * t[OW + 2];
+                    tacc += wu * m * (dg - kk * g * rinv) + g * rinv * gm;
+                }
+            }
+            M[i] += acc;
+            if (LOSS) Tg[i] += tacc;
+        }
+        __syncthreads();
+    }
+
+    // ---- products, energy, adjoint ------------------------------------------------------------
+    sweep_forward<T, LOSS>(p, M, Tg, lane);
+    T e_part = (T)0;
+    for (int s = lane; s < p.n_scalar; s += 64) {
+        e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
+        A[p.mapping[s]] = a.lin[s] / a.q_scaler[s];
+    }
+    __syncthreads();
+    sweep_reverse<T, false>(p, M, A, nullptr, nullptr, lane);
+
+    if (!LOSS) {
+        // ---- pair derivatives: lane = half * 32 + neighbour ------------------------------------
+        const int j = lane & 31, h = lane >> 5;
+        T fx = (T)0, fy = (T)0, fz = (T)0;
+        T vir[9];
+#pragma unroll
+        for (int q = 0; q < 9; q++) vir[q] = (T)0;
+        T* grow = a.pair_g + row * a.U * 3;
+        for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
+            const int nc = min(MTP_NC, nn - c0);
+            int nj; bool valid; T d[3] = {(T)0, (T)0, (T)0};
+            __syncthreads();
+            build_table<T, false>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+            __syncthreads();
+            T gs = (T)0, wx = (T)0, wy = (T)0, wz = (T)0;
+            if (j < nc) {
+                const T* t = tab + j * E;
+                const T rinv = t[OU + 3];
+                for (int i = h; i < n_basic; i += 2) {
+                    const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
+                              ec = p.basic[i * 4 + 3];
+                    const T adj = A[i];
+                    const T g = t[OG + mu], dg = t[ODG + mu];
+                    const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
+                    const T m = xa * yb * zc;
+                    gs += adj * m * (dg - (T)(ea + eb + ec) * g * rinv);
+                    const T ag = adj * g;
+                    wx += ag * (T)ea * t[OX + max(ea - 1, 0)] * yb * zc;
+                    wy += ag * (T)eb * xa * t[OY + max(eb - 1, 0)] * zc;
+                    wz += ag * (T)ec * xa * yb * t[OZ + max(ec - 1, 0)];
+                }
+            }
+            gs += __shfl_xor(gs, 32, 64);
+            wx += __shfl_xor(wx, 32, 64);
+            wy += __shfl_xor(wy, 32, 64);
+            wz += __shfl_xor(wz, 32, 64);
+            if (h == 0 && j < nc) {
+                const T* t = tab + j * E;
+                const T rinv = t[OU + 3];
+                T gx = gs * t[OU + 0] + wx * rinv;
+                T gy = gs * t[OU + 1] + wy * rinv;
+                T gz = gs * t[OU + 2] + wz * rinv;
+                if (!valid) { gx = (T)0; gy = (T)0; gz = (T)0; }
+                const int jj = c0 + j;
+                grow[jj * 3 + 0] = gx; grow[jj * 3 + 1] = gy; grow[jj * 3 + 2] = gz;
+                fx += gx; fy += gy; fz += gz;
+                vir[0] -= gx * d[0]; vir[1] -= gx * d[1]; vir[2] -= gx * d[2];
+                vir[3] -= gy * d[0]; vir[4] -= gy * d[1]; vir[5] -= gy * d[2];
+                vir[6] -= gz * d[0]; vir[7] -= gz * d[1]; vir[8] -= gz * d[2];
+            }
+        }
+        fx = wave_sum(fx); fy = wave_sum(fy); fz = wave_sum(fz);
+        double e_atom = (double)wave_sum(e_part);
+        double out[10];
+        out[0] = e_atom + (double)a.bias[ti];
+#pragma unroll
+        for (int q = 0; q < 9; q++) out[1 + q] = (double)wave_sum(vir[q]);
+        if (lane == 0) {
+            T* fo = a.force + ((size_t)b * NF + center) * 3;
+            fo[0] = fx; fo[1] = fy; fo[2] = fz;
+#pragma unroll
+            for (int q = 0; q < 10; q++) a.partial[row * 10 + q] = out[q];
+        }
+        return;
+    }
+
+    // ---- loss gradient ------------------------------------------------------------------------
+    if (LOSS) {
+        const T cE = a.cE[b];
+        sweep_reverse<T, true>(p, M, Bm, A, Tg, lane);      // linearMtpLoss.h:417-434
+        T* grow = a.gpart + row * a.ngrad;
+        for (int q = lane; q < a.ngrad; q += 64) grow[q] = (T)0;
+        const int j = lane & 31, h = lane >> 5;
+        T* Pm = pq;
+        T* Qm = pq + MTP_NC * nmus;
+        int* tjs = (int*)(pq + 2 * MTP_NC * nmus);
+        T* gacc = pq + 2 * MTP_NC * nmus + MTP_NC;          // [ntypes][nmus][K] for this centre type
+        for (int q = lane; q < a.ntypes * nmus * K; q += 64) gacc[q] = (T)0;
+        for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
+            const int nc = min(MTP_NC, nn - c0);
+            int nj; bool valid; T d[3];
+            __syncthreads();
+            build_table<T, true>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+            __syncthreads();
+            // P_mu(j), Q_mu(j): linearMtpLoss.h:438-536 with the k-sum factored out
+            for (int mu = 0; mu < nmus; mu++) {
+                T Pv = (T)0, Qv = (T)0;
+                if (j < nc) {
+                    const T* t = tab + j * E;
+                    const T rinv = t[OU + 3], wu = t[OW + 3];
+                    for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += 2) {
+                        const int ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2], ec = p.basic[i * 4 + 3];
+                        const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
+                        const T m = xa * yb * zc;
+                        const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
+                                     (T)eb * xa * t[OY + max(eb - 1, 0)] * zc * t[OW + 1] +
+                                     (T)ec * xa * yb * t[OZ + max(ec - 1, 0)] * t[OW + 2];
+                        const T adj = A[i];
+                        Pv += (cE * adj + Bm[i]) * m + adj * rinv * (gm - (T)(ea + eb + ec) * m * wu);
+                        Qv += adj * m * wu;
+                    }
+                }
+                Pv += __shfl_xor(Pv, 32, 64);
+                Qv += __shfl_xor(Qv, 32, 64);
+                if (h == 0 && j < nc) { Pm[j * nmus + mu] = Pv; Qm[j * nmus + mu] = Qv; }
+            }
+            // tj of each neighbour of the chunk, for the accumulation below
+            if (h == 0 && j < nc) tjs[j] = valid ? types[nj] : -1;
+            __syncthreads();
+            // lanes <- (mu, k): sequential over neighbours keeps the sum order fixed
+            for (int q = lane; q < nmus * K; q += 64) {
+                const int mu = q / K, k = q - mu * K;
+                for (int jn = 0; jn < nc; jn++) {
+                    const int tj = tjs[jn];
+                    if (tj < 0) continue;
+                    const T* t = tab + jn * E;
+                    gacc[tj * nmus * K + q] += t[OF + k] * Pm[jn * nmus + mu] + t[ODF + k] * Qm[jn * nmus + mu];
+                }
+            }
+        }
+        __syncthreads();
+        for (int q = lane; q < a.ntypes * nmus * K; q += 64)
+            grow[(size_t)ti * a.ntypes * nmus * K + q] = gacc[q];
+        // linear coefficients and bias: linearMtpLoss.h:539-554
+        for (int s = lane; s < p.n_scalar; s += 64)
+            grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
+        if (lane == 0) grow[ncoef + p.n_scalar + ti] = cE;
+    }
+}
+
+// ---- loss forward pieces ------------------------------------------------------------------------
+// One block per structure: loss (linearMtpLoss.h:138-176), the scaled residuals the gradient
+// kernel needs, and the per-structure squared errors for the RMSEs
+// (linearMtpLoss_cpu_launcher.h:477-527).
+template <typename T>
+__global__ void __launch_bounds__(256)
+mtp_loss_forward_kernel(int P, const int* __restrict__ binum, const int* __restrict__ bilist, T e_w, T f_w,
+                        T v_w, const T* __restrict__ etot, const T* __restrict__ e_dft,
+                        const T* __restrict__ force, const T* __restrict__ f_dft,
+                        const T* __restrict__ virial, const T* __restrict__ v_dft, T* __restrict__ bloss,
+                        T* __restrict__ cE, T* __restrict__ dFs, T* __restrict__ dVs,
+                        double* __restrict__ sq)   // [B, 3]: (dE/N)^2, sum dF^2, sum (dV/N)^2
+{
+    __shared__ double sh[4];
+    const int b = blockIdx.x;
+    const int inum = binum[b];
+    const T fscale = (T)2 * f_w / (T)(3 * inum);
+    for (int q = threadIdx.x; q < P * 3; q += 256) dFs[(size_t)b * P * 3 + q] = (T)0;
+    __syncthreads();
+    double fl = 0.0;
+    for (int ii = threadIdx.x; ii < inum; ii += 256) {
+        const int c = bilist[(size_t)b * P + ii];
+        for (int q = 0; q < 3; q++) {
+            const T dlt = force[((size_t)b * P + c) * 3 + q] - f_dft[((size_t)b * P + c) * 3 + q];
+            fl += (double)dlt * (double)dlt;
+            dFs[((size_t)b * P + c) * 3 + q] = fscale * dlt;
+        }
+    }
+    fl = wave_sum(fl);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = fl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const double fsum = sh[0] + sh[1] + sh[2] + sh[3];
+        double vsum = 0.0;
+        for (int q = 0; q < 9; q++) {
+            const T dlt = virial[b * 9 + q] - v_dft[b * 9 + q];
+            vsum += (double)dlt * (double)dlt;
+            dVs[b * 9 + q] = (T)2 * v_w / (T)(9 * inum) * dlt;
+        }
+        const T de = etot[b] - e_dft[b];
+        cE[b] = (T)2 * e_w / (T)inum * de;
+        bloss[b] = (T)((double)f_w / (3.0 * inum) * fsum + (double)v_w / (9.0 * inum) * vsum +
+                       (double)e_w / inum * (double)de * (double)de);
+        sq[b * 3 + 0] = ((double)de / inum) * ((double)de / inum);
+        sq[b * 3 + 1] = fsum;
+        sq[b * 3 + 2] = vsum / ((double)inum * inum);
+    }
+}
+
+template <typename T>
+__global__ void mtp_rmse_kernel(int B, const int* __restrict__ binum, const double* __restrict__ sq,
+                                T* __restrict__ rmse)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    double e = 0, f = 0, v = 0;
+    long nf = 0;
+    for (int b = 0; b < B; b++) { e += sq[b * 3]; f += sq[b * 3 + 1]; v += sq[b * 3 + 2]; nf += 3L * binum[b]; }
+    rmse[0] = (T)sqrt(e / B);
+    rmse[1] = (T)sqrt(f / (double)nf);
+    rmse[2] = (T)sqrt(v / (9.0 * B));
+}
+
+// out[b, q] = sum over atoms ii < binum[b] of gpart[b, ii, q], in atom order
+template <typename T>
+__global__ void __launch_bounds__(256)
+mtp_grad_reduce_kernel(int P, int ncoef, int nlin, int nbias, const int* __restrict__ binum,
+                       const T* __restrict__ gpart, T* __restrict__ dcoeffs, T* __restrict__ dlin,
+                       T* __restrict__ dbias)
+{
+    const int b = blockIdx.y;
+    const int ngrad = ncoef + nlin + nbias;
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= ngrad) return;
+    const int inum = binum[b];
+    T acc = (T)0;
+    for (int ii = 0; ii < inum; ii++) acc += gpart[((size_t)b * P + ii) * ngrad + q];
+    if (q < ncoef) { if (dcoeffs) dcoeffs[(size_t)b * ncoef + q] = acc; }
+    else if (q < ncoef + nlin) { if (dlin) dlin[(size_t)b * nlin + q - ncoef] = acc; }
+    else if (dbias) dbias[(size_t)b * nbias + q - ncoef - nlin] = acc;
+}
+
+// ---- plan construction ---------------------------------------------------------------------------
+std::mutex g_plan_mutex;
+std::set<MtpPlan*> g_plans;
+
+int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const int* times, int n_scalar,
+                const int* mapping, MtpPlan** out)
+{
+    A2P_REQUIRE(n_moms > 0 && n_basic > 0 && n_basic <= n_moms && n_times >= 0 && n_scalar > 0,
+                A2P_ERR_INVALID, "mtp plan: bad table sizes");
+    A2P_REQUIRE(basic && mapping && (times || n_times == 0), A2P_ERR_INVALID, "mtp plan: null table");
+    int nmus = 0, kmax = 0;
+    for (int i = 0; i < n_basic; i++) {
+        const int* q = basic + i * 4;
+        A2P_REQUIRE(q[0] >= 0 && q[1] >= 0 && q[2] >= 0 && q[3] >= 0, A2P_ERR_INVALID,
+                    "mtp plan: negative entry in alpha_index_basic");
+        A2P_REQUIRE(i == 0 || q[0] >= basic[(i - 1) * 4], A2P_ERR_INVALID,
+                    "mtp plan: alpha_index_basic is not grouped by radial function index");
+        nmus = std::max(nmus, q[0] + 1);
+        kmax = std::max(kmax, q[1] + q[2] + q[3]);
+    }
+    A2P_REQUIRE(nmus <= MTP_NMUS_MAX, A2P_ERR_INVALID, "mtp plan: more than %d radial functions", MTP_NMUS_MAX);
+    A2P_REQUIRE(kmax <= 24, A2P_ERR_INVALID, "mtp plan: monomial degree %d too large", kmax);
+    std::vector<int> level(n_moms, 0), last_write(n_moms, -1);
+    for (int e = 0; e < n_times; e++) {
+        const int* q = times + e * 4;
+        A2P_REQUIRE(q[0] >= 0 && q[0] < n_moms && q[1] >= 0 && q[1] < n_moms && q[3] >= n_basic &&
+                        q[3] < n_moms,
+                    A2P_ERR_INVALID, "mtp plan: alpha_index_times entry %d out of range", e);
+        last_write[q[3]] = e;
+    }
+    int n_levels = 0;
+    for (int e = 0; e < n_times; e++) {
+        const int* q = times + e * 4;
+        for (int s = 0; s < 2; s++)
+            A2P_REQUIRE(last_write[q[s]] < e, A2P_ERR_INVALID,
+                        "mtp plan: moment %d is read by product %d before its last contribution (%d); "
+                        "the table cannot be executed level by level", q[s], e, last_write[q[s]]);
+        level[q[3]] = std::max(level[q[3]], 1 + std::max(level[q[0]], level[q[1]]));
+        n_levels = std::max(n_levels, level[q[3]]);
+    }
+    std::vector<char> seen(n_moms, 0);
+    for (int s = 0; s < n_scalar; s++) {
+        A2P_REQUIRE(mapping[s] >= 0 && mapping[s] < n_moms, A2P_ERR_INVALID, "mtp plan: mapping out of range");
+        A2P_REQUIRE(!seen[mapping[s]], A2P_ERR_INVALID, "mtp plan: alpha_moment_mapping repeats a moment");
+        seen[mapping[s]] = 1;
+    }
+    // forward gather lists
+    std::vector<std::vector<int>> terms_of(n_moms);          // product entries per dst, file order
+    for (int e = 0; e < n_times; e++) terms_of[times[e * 4 + 3]].push_back(e);
+    std::vector<int> f_level(n_levels + 1, 0), f_dst, f_begin(1, 0), f_m0, f_m1;
+    std::vector<double> f_mult;
+    for (int l = 1; l <= n_levels; l++) {
+        std::vector<int> dsts;
+        for (int m = n_basic; m < n_moms; m++)
+            if (level[m] == l && !terms_of[m].empty()) dsts.push_back(m);
+        std::stable_sort(dsts.begin(), dsts.end(),
+                         [&](int x, int y) { return terms_of[x].size() > terms_of[y].size(); });
+        for (int m : dsts) {
+            f_dst.push_back(m);
+            for (int e : terms_of[m]) {
+                f_m0.push_back(times[e * 4]);
+                f_m1.push_back(times[e * 4 + 1]);
+                f_mult.push_back((double)times[e * 4 + 2]);
+            }
+            f_begin.push_back((int)f_m0.size());
+        }
+        f_level[l] = (int)f_dst.size();
+    }
+    // reverse gather lists: terms per source in reverse file order
+    std::vector<std::vector<int>> uses(n_moms);              // encoded 2*e + which
+    for (int e = n_times - 1; e >= 0; e--) {
+        uses[times[e * 4 + 1]].push_back(2 * e + 1);         // adj[m1] += adj[dst] mult M[m0]
+        uses[times[e * 4 + 0]].push_back(2 * e + 0);         // adj[m0] += adj[dst] mult M[m1]
+    }
+    std::vector<int> r_level(n_levels + 1, 0), r_src, r_begin(1, 0), r_dst, r_other;
+    std::vector<double> r_mult;
+    for (int l = 0; l < n_levels; l++) {
+        std::vector<int> srcs;
+        for (int m = 0; m < n_moms; m++)
+            if (level[m] == l && !uses[m].empty()) srcs.push_back(m);
+        std::stable_sort(srcs.begin(), srcs.end(), [&](int x, int y) { return uses[x].size() > uses[y].size(); });
+        for (int m : srcs) {
+            r_src.push_back(m);
+            for (int code : uses[m]) {
+                const int e = code >> 1, which = code & 1;
+                r_dst.push_back(times[e * 4 + 3]);
+                r_other.push_back(which ? times[e * 4 + 0] : times[e * 4 + 1]);
+                r_mult.push_back((double)times[e * 4 + 2]);
+            }
+            r_begin.push_back((int)r_dst.size());
+        }
+        r_level[l + 1] = (int)r_src.size();
+    }
+    std::vector<int> mu_begin(nmus + 1, n_basic);
+    for (int i = n_basic - 1; i >= 0; i--) mu_begin[basic[i * 4]] = i;
+    for (int m = nmus - 1; m >= 0; m--) mu_begin[m] = std::min(mu_begin[m], mu_begin[m + 1]);
+    mu_begin[0] = 0;
+
+    // one device block
+    struct Seg { const void* src; size_t bytes; size_t off; };
+    std::vector<Seg> segs;
+    size_t total = 0;
+    auto add = [&](const void* src, size_t bytes) {
+        size_t off = total;
+        segs.push_back({src, bytes, off});
+        total += (bytes + 15) / 16 * 16;
+        return off;
+    };
+    const size_t o_basic = add(basic, sizeof(int) * 4 * n_basic);
+    const size_t o_mu = add(mu_begin.data(), sizeof(int) * mu_begin.size());
+    const size_t o_map = add(mapping, sizeof(int) * n_scalar);
+    const size_t o_fl = add(f_level.data(), sizeof(int) * f_level.size());
+    const size_t o_fd = add(f_dst.data(), sizeof(int) * f_dst.size());
+    const size_t o_fb = add(f_begin.data(), sizeof(int) * f_begin.size());
+    const size_t o_f0 = add(f_m0.data(), sizeof(int) * f_m0.size());
+    const size_t o_f1 = add(f_m1.data(), sizeof(int) * f_m1.size());
+    const size_t o_fm = add(f_mult.data(), sizeof(double) * f_mult.size());
+    const size_t o_rl = add(r_level.data(), sizeof(int) * r_level.size());
+    const size_t o_rs = add(r_src.data(), sizeof(int) * r_src.size());
+    const size_t o_rb = add(r_begin.data(), sizeof(int) * r_begin.size());
+    const size_t o_rd = add(r_dst.data(), sizeof(int) * r_dst.size());
+    const size_t o_ro = add(r_other.data(), sizeof(int) * r_other.size());
+    const size_t o_rm = add(r_mult.data(), sizeof(double) * r_mult.size());
+    std::vector<unsigned char> host(total + 16, 0);
+    for (auto& s : segs)
+        if (s.bytes) std::memcpy(host.data() + s.off, s.src, s.bytes);
+    MtpPlan* plan = new MtpPlan();
+    A2P_HIP_CHECK(hipGetDevice(&plan->device));
+    A2P_HIP_CHECK(hipMalloc(&plan->device_block, total + 16));
+    A2P_HIP_CHECK(hipMemcpy(plan->device_block, host.data(), total + 16, hipMemcpyHostToDevice));
+    char* base = (char*)plan->device_block;
+    MtpPlanDevice& d = plan->d;
+    d.n_moms = n_moms; d.n_basic = n_basic; d.n_times = n_times; d.n_scalar = n_scalar;
+    d.nmus = nmus; d.kmax = kmax; d.n_levels = n_levels;
+    d.basic = (const int*)(base + o_basic); d.mu_begin = (const int*)(base + o_mu);
+    d.mapping = (const int*)(base + o_map);
+    d.f_level = (const int*)(base + o_fl); d.f_dst = (const int*)(base + o_fd);
+    d.f_begin = (const int*)(base + o_fb); d.f_m0 = (const int*)(base + o_f0);
+    d.f_m1 = (const int*)(base + o_f1); d.f_mult = (const double*)(base + o_fm);
+    d.r_level = (const int*)(base + o_rl); d.r_src = (const int*)(base + o_rs);
+    d.r_begin = (const int*)(base + o_rb); d.r_dst = (const int*)(base + o_rd);
+    d.r_other = (const int*)(base + o_ro); d.r_mult = (const double*)(base + o_rm);
+    {
+        std::lock_guard<std::mutex> lock(g_plan_mutex);
+        g_plans.insert(plan);
+    }
+    *out = plan;
+    return A2P_OK;
+}
+
+int plan_check(void* handle, MtpPlan** out)
+{
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    A2P_REQUIRE(handle && g_plans.count((MtpPlan*)handle), A2P_ERR_INVALID, "mtp: invalid plan handle");
+    *out = (MtpPlan*)handle;
+    return A2P_OK;
+}
+
+template <typename T>
+int table_entries(const MtpPlanDevice& p, int K, bool loss)
+{
+    int E = 3 * (p.kmax + 1) + 2 * p.nmus + 4;
+    if (loss) E += 4 + 2 * K;
+    if ((E & 1) == 0) E++;            // odd stride: neighbours land in different LDS banks
+    return E;
+}
+
+template <typename T>
+size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K)
+{
+    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + (size_t)MTP_NC * E;
+    // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
+    if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
+    return n * sizeof(T) + 64;
+}
+
+template <typename T>
+int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coeffs, const T* lin,
+              const T* bias, int nmus, int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P,
+              int U, int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+              const int* bfirstneigh, const T* brcs, const int* btypes)
+{
+    A2P_REQUIRE(K >= 1 && K <= MTP_KMAX, A2P_ERR_INVALID, "mtp: chebyshev_size %d outside [1, %d]", K, MTP_KMAX);
+    A2P_REQUIRE(nmus == plan->d.nmus, A2P_ERR_INVALID, "mtp: nmus %d does not match the tables (%d)", nmus,
+                plan->d.nmus);
+    A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0 && U >= 1 && nghost >= 0, A2P_ERR_INVALID, "mtp: bad shape");
+    A2P_REQUIRE(rmax > rmin && rmin >= 0, A2P_ERR_INVALID, "mtp: need 0 <= rmin < rmax");
+    A2P_REQUIRE(coeffs && lin && bias && q_scaler && binum && bilist && bnumneigh && bfirstneigh && brcs &&
+                    btypes, A2P_ERR_INVALID, "mtp: null input pointer");
+    A2P_REQUIRE((long long)B * P * U < (1ll << 31), A2P_ERR_INVALID, "mtp: batch too large");
+    a.p = plan->d;
+    a.K = K; a.ntypes = ntypes; a.scaling = (T)scaling; a.rmax = (T)rmax; a.rmin = (T)rmin;
+    a.coeffs = coeffs; a.lin = lin; a.bias = bias; a.q_scaler = q_scaler;
+    a.B = B; a.P = P; a.U = U; a.nghost = nghost;
+    a.binum = binum; a.bilist = bilist; a.bnumneigh = bnumneigh; a.bfirstneigh = bfirstneigh;
+    a.brcs = brcs; a.btypes = btypes;
+    a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
+    a.force = nullptr; a.pair_g = nullptr; a.partial = nullptr;
+    void* ws = nullptr;
+    int rc = ws_get(WS_FLAGS, 64, &ws);
+    if (rc) return rc;
+    a.status = (int*)ws;
+    return A2P_OK;
+}
+
+template <typename T, bool LOSS>
+int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
+{
+    const size_t lds = lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K);
+    A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
+                "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
+    auto kern = mtp_atom_kernel<T, LOSS>;
+    if (lds > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)lds));
+    prof_begin(LOSS ? "mtp_loss_bwd_kernel" : "mtp_efv_kernel", stream);
+    hipLaunchKernelGGL(kern, dim3(a.P, a.B), dim3(64), lds, stream, a);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+template <typename T>
+int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus,
+            int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
+            const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
+            const int* btypes, T* etot, T* force, T* virial, hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
+                   binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    a.E = table_entries<T>(a.p, K, false);
+    void* ws = nullptr;
+    rc = ws_get(WS_PARTIAL, (size_t)B * P * 10 * sizeof(double), &ws);
+    if (rc) return rc;
+    a.partial = (double*)ws;
+    const size_t force_bytes = (size_t)B * (P + nghost) * 3 * sizeof(T);
+    a.force = force;
+    if (!force) {
+        rc = ws_get(WS_MISC, force_bytes, &ws);
+        if (rc) return rc;
+        a.force = (T*)ws;
+    }
+    rc = ws_get(WS_PAIR_G, (size_t)B * P * U * 3 * sizeof(T), &ws);
+    if (rc) return rc;
+    a.pair_g = (T*)ws;
+    rc = fill_zero(a.force, force_bytes, stream);      // the reference zeroes on entry, linearMtp.h:228-230
+    if (rc) return rc;
+    rc = launch_atoms<T, false>(a, stream);
+    if (rc) return rc;
+    if (force) {
+        rc = pair_reduce<T>(force, a.pair_g, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+        if (rc) return rc;
+    }
+    if (etot) {
+        rc = finish_partials<T>(etot, a.partial, B, P, 1, 10, 1, stream);
+        if (rc) return rc;
+    }
+    if (virial) {
+        rc = finish_partials<T>(virial, a.partial + 1, B, P, 9, 10, 9, stream);
+        if (rc) return rc;
+    }
+    return A2P_OK;
+}
+
+template <typename T>
+int mtp_loss(void* handle, double e_w, double f_w, double v_w, const T* e_dft, const T* f_dft, const T* v_dft,
+             int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus, int ntypes,
+             const T* q_scaler, double rmax, double rmin, int B, int P, int U, const int* binum,
+             const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs, const int* btypes,
+             T* bloss, T* rmse, T* etot, T* force, T* virial, T* dcoeffs, T* dlin, T* dbias,
+             hipStream_t stream)
+{
+    A2P_REQUIRE(e_dft && f_dft && v_dft && bloss && etot && force && virial, A2P_ERR_INVALID,
+                "mtp loss: null label or output pointer");
+    int rc = mtp_efv<T>(handle, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, 0,
+                        binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, stream);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    MtpPlan* plan = nullptr;
+    rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, 0,
+                   binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    const int ncoef = ntypes * ntypes * nmus * K;
+    const int ngrad = ncoef + a.p.n_scalar + ntypes;
+    const bool want_grad = dcoeffs || dlin || dbias;
+    // workspace: cE[B] | dVs[B*9] | dFs[B*P*3] | gpart[B*P*ngrad] | sq[B*3] (double)
+    size_t nT = (size_t)B + (size_t)B * 9 + (size_t)B * P * 3 + (want_grad ? (size_t)B * P * ngrad : 0);
+    size_t bytesT = (nT * sizeof(T) + 15) / 16 * 16;
+    void* ws = nullptr;
+    rc = ws_get(WS_MTP, bytesT + (size_t)B * 3 * sizeof(double), &ws);
+    if (rc) return rc;
+    T* cE = (T*)ws;
+    T* dVs = cE + B;
+    T* dFs = dVs + (size_t)B * 9;
+    T* gpart = dFs + (size_t)B * P * 3;
+    double* sq = (double*)((char*)ws + bytesT);
+    prof_begin("mtp_loss_forward", stream);
+    hipLaunchKernelGGL(mtp_loss_forward_kernel<T>, dim3(B), dim3(256), 0, stream, P, binum, bilist, (T)e_w,
+                       (T)f_w, (T)v_w, etot, e_dft, force, f_dft, virial, v_dft, bloss, cE, dFs, dVs, sq);
+    if (rmse) hipLaunchKernelGGL(mtp_rmse_kernel<T>, dim3(1), dim3(64), 0, stream, B, binum, sq, rmse);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    if (!want_grad) return A2P_OK;
+    a.E = table_entries<T>(a.p, K, true);
+    a.cE = cE; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = ngrad;
+    rc = launch_atoms<T, true>(a, stream);
+    if (rc) return rc;
+    prof_begin("mtp_grad_reduce", stream);
+    hipLaunchKernelGGL(mtp_grad_reduce_kernel<T>, dim3(ceil_div(ngrad, 256), B), dim3(256), 0, stream, P, ncoef,
+                       a.p.n_scalar, ntypes, binum, gpart, dcoeffs, dlin, dbias);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+}  // namespace
+}  // namespace a2p
+
+extern "C" {
+
+int a2p_mtp_plan_create(int n_moms, int n_basic, const int* basic, int n_times, const int* times,
+                        int n_scalar, const int* mapping, void** plan)
+{
+    A2P_REQUIRE(plan, A2P_ERR_INVALID, "mtp plan: null output");
+    a2p::MtpPlan* p = nullptr;
+    int rc = a2p::plan_create(n_moms, n_basic, basic, n_times, times, n_scalar, mapping, &p);
+    if (rc) return rc;
+    *plan = p;
+    return A2P_OK;
+}
+
+int a2p_mtp_plan_destroy(void* handle)
+{
+    a2p::MtpPlan* p = nullptr;
+    int rc = a2p::plan_check(handle, &p);
+    if (rc) return rc;
+    {
+        std::lock_guard<std::mutex> lock(a2p::g_plan_mutex);
+        a2p::g_plans.erase(p);
+    }
+    A2P_HIP_CHECK(hipFree(p->device_block));
+    delete p;
+    return A2P_OK;
+}
+
+#define MTP_MODEL(T) int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus, \
+    int ntypes, const T* q_scaler, double rmax, double rmin
+#define MTP_MODEL_PASS K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin
+#define MTP_BATCH(T) const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, \
+    const T* brcs, const int* btypes
+
+int a2p_mtp_efv_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
+                    double* etot, double* force, double* virial, void* stream)
+{
+    return a2p::mtp_efv<double>(plan, MTP_MODEL_PASS, B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh,
+                                brcs, btypes, etot, force, virial, (hipStream_t)stream);
+}
+
+int a2p_mtp_efv_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int nghost, MTP_BATCH(float),
+                    float* etot, float* force, float* virial, void* stream)
+{
+    return a2p::mtp_efv<float>(plan, MTP_MODEL_PASS, B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh,
+                               brcs, btypes, etot, force, virial, (hipStream_t)stream);
+}
+
+int a2p_mtp_loss_f64(void* plan, double e_weight, double f_weight, double v_weight, const double* e_dft,
+                     const double* f_dft, const double* v_dft, MTP_MODEL(double), int B, int P, int U,
+                     MTP_BATCH(double), double* bloss, double* rmse, double* etot, double* force,
+                     double* virial, double* dcoeffs, double* dlinear, double* dbias, void* stream)
+{
+    return a2p::mtp_loss<double>(plan, e_weight, f_weight, v_weight, e_dft, f_dft, v_dft, MTP_MODEL_PASS, B, P,
+                                 U, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, bloss, rmse, etot,
+                                 force, virial, dcoeffs, dlinear, dbias, (hipStream_t)stream);
+}
+
+int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weight, const float* e_dft,
+                     const float* f_dft, const float* v_dft, MTP_MODEL(float), int B, int P, int U,
+                     MTP_BATCH(float), float* bloss, float* rmse, float* etot, float* force, float* virial,
+                     float* dcoeffs, float* dlinear, float* dbias, void* stream)
+{
+    return a2p::mtp_loss<float>(plan, e_weight, f_weight, v_weight, e_dft, f_dft, v_dft, MTP_MODEL_PASS, B, P,
+                                U, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, bloss, rmse, etot, force,
+                                virial, dcoeffs, dlinear, dbias, (hipStream_t)stream);
+}
+}

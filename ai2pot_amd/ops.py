@@ -163,3 +163,225 @@ def nepToDescriptorsOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, c
                            bfirstneigh, brcs, btypes, type_map, nghost, rmax_radial, rmax_angular, None,
                            validate)
     return [d]
+
+
+# --------------------------------------------------------------------------------------------
+# linear MTP  (source/descriptor/mtpr/bind/mtpr_bind.cc:30-457)
+# --------------------------------------------------------------------------------------------
+_plans = {}
+
+
+def set_ai2pot_path(path):
+    """torch.ops.mtpr.set_ai2pot_path (mtpr_bind.cc:31-36): where the MTP templates live."""
+    from . import mtp_param
+    mtp_param.set_ai2pot_path(path)
+
+
+def mtpParamOp(mtp_level, device="cpu"):
+    """The seven int32 tensors of the reference's mtpParamOp (src/mtpParamOp.cc:25-63):
+    [alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping,
+    num_mus4moms, mus4moms, nmus]."""
+    from . import mtp_param
+    t = mtp_param.mtp_param(int(mtp_level))
+    f = lambda a: torch.from_numpy(a.astype("int32")).to(device)
+    return [torch.tensor(t["alpha_moments_count"], dtype=torch.int32, device=device),
+            f(t["alpha_index_basic"]), f(t["alpha_index_times"]), f(t["alpha_moment_mapping"]),
+            f(t["num_mus4moms"]), f(t["mus4moms"]), torch.tensor(t["nmus"], dtype=torch.int32, device=device)]
+
+
+def _mtp_plan(alpha_moments_count, basic_t, times_t, mapping_t, device):
+    """Plan handle for a set of table tensors.  The tables are model constants (registered
+    buffers in the reference, ai2pot/models/mtp/linear_mtp.py:63-69): they are read back to
+    the host once and cached by storage address, shape and version."""
+    key = (device.index, int(alpha_moments_count),
+           basic_t.data_ptr(), tuple(basic_t.shape), basic_t._version,
+           times_t.data_ptr(), tuple(times_t.shape), times_t._version,
+           mapping_t.data_ptr(), tuple(mapping_t.shape), mapping_t._version)
+    if key in _plans:
+        return _plans[key]
+    for name, t in (("alpha_index_basic", basic_t), ("alpha_index_times", times_t),
+                    ("alpha_moment_mapping", mapping_t)):
+        _req(isinstance(t, torch.Tensor) and t.dtype == torch.int32, "%s must be an int32 tensor" % name)
+    _req(basic_t.dim() == 2 and basic_t.shape[1] == 4, "alpha_index_basic must have shape [n, 4]")
+    _req(times_t.numel() == 0 or (times_t.dim() == 2 and times_t.shape[1] == 4),
+         "alpha_index_times must have shape [n, 4]")
+    basic = basic_t.detach().cpu().contiguous().numpy()
+    times = times_t.detach().cpu().contiguous().numpy().reshape(-1, 4)
+    mapping = mapping_t.detach().cpu().contiguous().numpy()
+    handle = _c.c_void_p()
+    with torch.cuda.device(device):
+        rc = _lib.lib().a2p_mtp_plan_create(
+            _c.c_int(int(alpha_moments_count)), _c.c_int(basic.shape[0]), basic.ctypes.data_as(_c.c_void_p),
+            _c.c_int(times.shape[0]), times.ctypes.data_as(_c.c_void_p), _c.c_int(mapping.size),
+            mapping.ctypes.data_as(_c.c_void_p), _c.byref(handle))
+    _lib.check(rc)
+    if len(_plans) > 64:
+        _, old = _plans.popitem()
+        _lib.lib().a2p_mtp_plan_destroy(old[0])
+    _plans[key] = (handle, mapping.size)
+    return _plans[key]
+
+
+def _mtp_common(coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic,
+                alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                btypes, type_map, nghost, q_scaler, chebyshev_size, validate):
+    _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
+         "brcs must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = brcs.dtype, brcs.device
+    _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
+    _req(brcs.is_contiguous(), "brcs must be contiguous")
+    for name, t in (("coeffs", coeffs), ("linear_coeffs", linear_coeffs), ("type_bias", type_bias),
+                    ("q_scaler", q_scaler)):
+        _check_float(name, t, dtype, device)
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh), ("btypes", btypes)):
+        _check_int(name, t, device)
+    nghost = int(nghost)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost)
+    ntypes = int(type_map.numel())
+    _req(ntypes > 0, "type_map is empty")
+    plan, n_scalar = _mtp_plan(alpha_moments_count, alpha_index_basic, alpha_index_times,
+                               alpha_moment_mapping, device)
+    _req(coeffs.numel() == ntypes * ntypes * int(nmus) * int(chebyshev_size), "coeffs size mismatch")
+    _req(linear_coeffs.numel() == n_scalar and q_scaler.numel() == n_scalar,
+         "linear_coeffs and q_scaler must have alpha_scalar_moments = %d elements" % n_scalar)
+    _req(type_bias.numel() == ntypes, "type_bias size mismatch")
+    if validate:
+        _validate_batch(binum, bnumneigh, U, P)
+    return dtype, device, B, P, U, nghost, ntypes, plan, n_scalar
+
+
+def _mtp_efv(want_virial, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh,
+             bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax, validate):
+    _no_zbl(zbl_rmax)
+    dtype, device, B, P, U, nghost, ntypes, plan, _ = _mtp_common(
+        coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+        q_scaler, chebyshev_size, validate)
+    etot = torch.zeros((B,), dtype=dtype, device=device)
+    force = torch.zeros((B, P + nghost, 3), dtype=dtype, device=device)
+    virial = torch.zeros((B, 9), dtype=dtype, device=device) if want_virial else None
+    L = _lib.lib()
+    fn = L.a2p_mtp_efv_f32 if dtype == torch.float32 else L.a2p_mtp_efv_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
+                _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax),
+                _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
+                _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(etot),
+                _ptr(force), _ptr(virial), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return etot, force, virial
+
+
+def linearMtpToEFVOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                     alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                     bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
+                     zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
+    """[E[B], F[B, P+nghost, 3], V[B, 9]]; mtpr_bind.cc:333-394, linearMtpOp.cc:2834-3180."""
+    e, f, v = _mtp_efv(True, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                       alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax,
+                       validate)
+    return [e, f, v]
+
+
+def linearMtpToEFOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                    alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                    bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
+                    zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
+    """[E[B], F[B, P+nghost, 3]]; mtpr_bind.cc:396-457."""
+    e, f, _ = _mtp_efv(False, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                       alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax,
+                       validate)
+    return [e, f]
+
+
+def mtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, scaling,
+                  coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+                  alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+                  nghost, rmax, rmin, q_scaler, want_grad=True, validate=True):
+    """Forward and (optionally) the per-structure parameter gradients of the training loss in
+    one call.  Returns a dict with bloss[B], rmse[3], energy, force, virial and, with
+    want_grad, dcoeffs[B, ncoef], dlinear[B, S], dbias[B, ntypes]."""
+    _req(int(nghost) == 0, "the loss operator requires nghost == 0, as the reference does")
+    dtype, device, B, P, U, nghost, ntypes, plan, n_scalar = _mtp_common(
+        coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+        q_scaler, chebyshev_size, validate)
+    for name, t, shape in (("betot_dft", betot_dft, (B,)), ("bforce_dft", bforce_dft, (B, P, 3)),
+                           ("bvirial_dft", bvirial_dft, (B, 9))):
+        _check_float(name, t, dtype, device)
+        n_expected = 1
+        for s_ in shape:
+            n_expected *= s_
+        _req(t.numel() == n_expected, "%s must have shape %s" % (name, shape))
+    ncoef = coeffs.numel()
+    z = lambda *s: torch.zeros(s, dtype=dtype, device=device)
+    out = dict(bloss=z(B), rmse=z(3), energy=z(B), force=z(B, P, 3), virial=z(B, 9))
+    if want_grad:
+        out.update(dcoeffs=z(B, ncoef), dlinear=z(B, n_scalar), dbias=z(B, ntypes))
+    L = _lib.lib()
+    fn = L.a2p_mtp_loss_f32 if dtype == torch.float32 else L.a2p_mtp_loss_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+                _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_double(scaling),
+                _ptr(coeffs), _ptr(linear_coeffs), _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes),
+                _ptr(q_scaler), _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U),
+                _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes),
+                _ptr(out["bloss"]), _ptr(out["rmse"]), _ptr(out["energy"]), _ptr(out["force"]),
+                _ptr(out["virial"]), _ptr(out.get("dcoeffs")), _ptr(out.get("dlinear")),
+                _ptr(out.get("dbias")), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return out
+
+
+class _LinearMtpToLoss(torch.autograd.Function):
+    """Autograd wrapper with the reference's contract (linearMtpOp.cc:621-1181, 1184-1765):
+    gradients flow to coeffs, linear_coeffs and type_bias only, as grad_output[B] @ dloss/dtheta."""
+
+    @staticmethod
+    def forward(ctx, coeffs, linear_coeffs, type_bias, args):
+        (e_w, f_w, v_w, e_dft, f_dft, v_dft, K, scaling, n_moms, basic, times, mapping, nmus, binum, bilist,
+         bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, validate) = args
+        need = coeffs.requires_grad or linear_coeffs.requires_grad or type_bias.requires_grad
+        r = mtp_loss_step(e_w, f_w, v_w, e_dft, f_dft, v_dft, K, scaling, coeffs.detach(),
+                          linear_coeffs.detach(), type_bias.detach(), n_moms, basic, times, mapping, nmus,
+                          binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin,
+                          q_scaler, want_grad=need, validate=validate)
+        if need:
+            # unlike the reference, which recomputes E/F/V in backward, the gradients are produced by
+            # the same call and kept
+            ctx.save_for_backward(r["dcoeffs"], r["dlinear"], r["dbias"])
+        ctx.shapes = (coeffs.shape, linear_coeffs.shape, type_bias.shape)
+        ctx.have = need
+        rm = r["rmse"]
+        return r["bloss"], rm[0:1].clone(), rm[1:2].clone(), rm[2:3].clone()
+
+    @staticmethod
+    def backward(ctx, gl, ge, gf, gv):
+        if not ctx.have:
+            return None, None, None, None
+        dc, dl, db = ctx.saved_tensors
+        sc, sl, sb = ctx.shapes
+        return (torch.matmul(gl, dc).reshape(sc), torch.matmul(gl, dl).reshape(sl),
+                torch.matmul(gl, db).reshape(sb), None)
+
+
+def linearMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size,
+                      scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic,
+                      alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh,
+                      brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
+                      zbl_cks=None, zbl_dks=None, validate=True):
+    """[bloss[B], e_rmse[1], f_rmse[1], v_rmse[1]], differentiable w.r.t. coeffs, linear_coeffs and
+    type_bias; mtpr_bind.cc:189-261."""
+    _no_zbl(zbl_rmax)
+    args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, scaling,
+            alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
+            bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, validate)
+    return list(_LinearMtpToLoss.apply(coeffs, linear_coeffs, type_bias, args))

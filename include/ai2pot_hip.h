@@ -102,6 +102,70 @@ int a2p_nblist_build_f64(const double* lattice, const int* types, const double* 
                          int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
                          void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Linear Moment Tensor Potential.
+ *
+ * a2p_mtp_plan_create takes the three HOST tables the reference's mtpParamOp returns
+ * (source/descriptor/mtpr/src/mtpParamOp.cc:25-63, parsed from NN.almtp by
+ * src/mtpParam.cc:82-214): alpha_index_basic[n_basic][4] = (mu, a, b, c),
+ * alpha_index_times[n_times][4] = (m0, m1, mult, dst), alpha_moment_mapping[n_scalar];
+ * it validates them, orders the products by dependency level and keeps the result on the
+ * current device.  The handle is passed to the calls below and freed by
+ * a2p_mtp_plan_destroy.  Levels whose moment vector does not fit LDS (above 24) are refused.
+ *
+ * a2p_mtp_efv_* replaces the compute of torch.ops.mtpr.linearMtpToEFVOp / linearMtpToEFOp
+ * (source/descriptor/mtpr/bind/mtpr_bind.cc:333-457; src/linearMtpOp.cc:2834-3180 ->
+ * include/linearMtp_cpu_launcher.h:128-203 -> include/linearMtp.h:190-352,
+ * include/mtpBasis.h:400-534).  coeffs[ntypes][ntypes][nmus][K], linear_coeffs[n_scalar],
+ * type_bias[ntypes], q_scaler[n_scalar]; batch and outputs as for a2p_nep_efv_*.
+ *
+ * a2p_mtp_loss_* replaces the compute of torch.ops.mtpr.linearMtpToLossOp, forward and
+ * backward (mtpr_bind.cc:189-261; src/linearMtpOp.cc:621-1181, 1184-1765 ->
+ * include/linearMtpLoss.h:138-176, 212-569, include/linearMtpLoss_cpu_launcher.h:151-194,
+ * 233-337, 477-527).  Labels e_dft[B], f_dft[B][P][3], v_dft[B][9].  Outputs: bloss[B],
+ * rmse[3] = (e, f, v) (may be NULL), the model's etot[B], force[B][P][3], virial[B][9]
+ * (required), and the per-structure gradients dcoeffs[B][ntypes*ntypes*nmus*K],
+ * dlinear[B][n_scalar], dbias[B][ntypes] (all three NULL = forward only).  The reference's
+ * backward then returns grad_output[B] @ these matrices (linearMtpOp.cc:1740-1742); that
+ * product is left to the caller.  nghost must be 0 for the loss, as in the reference
+ * (linearMtpLoss_cpu_launcher.h:174, 285 index forces with stride natoms_pad).
+ * ------------------------------------------------------------------------------------------ */
+int a2p_mtp_plan_create(int n_moms, int n_basic, const int* basic, int n_times, const int* times,
+                        int n_scalar, const int* mapping, void** plan);
+int a2p_mtp_plan_destroy(void* plan);
+
+int a2p_mtp_efv_f64(void* plan, int chebyshev_size, double scaling, const double* coeffs,
+                    const double* linear_coeffs, const double* type_bias, int nmus, int ntypes,
+                    const double* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                    int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                    const int* bfirstneigh, const double* brcs, const int* btypes, double* etot,
+                    double* force, double* virial, void* stream);
+
+int a2p_mtp_efv_f32(void* plan, int chebyshev_size, double scaling, const float* coeffs,
+                    const float* linear_coeffs, const float* type_bias, int nmus, int ntypes,
+                    const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                    int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                    const int* bfirstneigh, const float* brcs, const int* btypes, float* etot,
+                    float* force, float* virial, void* stream);
+
+int a2p_mtp_loss_f64(void* plan, double e_weight, double f_weight, double v_weight, const double* e_dft,
+                     const double* f_dft, const double* v_dft, int chebyshev_size, double scaling,
+                     const double* coeffs, const double* linear_coeffs, const double* type_bias, int nmus,
+                     int ntypes, const double* q_scaler, double rmax, double rmin, int batch,
+                     int natoms_pad, int umax, const int* binum, const int* bilist, const int* bnumneigh,
+                     const int* bfirstneigh, const double* brcs, const int* btypes, double* bloss,
+                     double* rmse, double* etot, double* force, double* virial, double* dcoeffs,
+                     double* dlinear, double* dbias, void* stream);
+
+int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weight, const float* e_dft,
+                     const float* f_dft, const float* v_dft, int chebyshev_size, double scaling,
+                     const float* coeffs, const float* linear_coeffs, const float* type_bias, int nmus,
+                     int ntypes, const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad,
+                     int umax, const int* binum, const int* bilist, const int* bnumneigh,
+                     const int* bfirstneigh, const float* brcs, const int* btypes, float* bloss,
+                     float* rmse, float* etot, float* force, float* virial, float* dcoeffs, float* dlinear,
+                     float* dbias, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
