@@ -385,3 +385,156 @@ def linearMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bviri
             alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
             bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, validate)
     return list(_LinearMtpToLoss.apply(coeffs, linear_coeffs, type_bias, args))
+
+
+# --------------------------------------------------------------------------------------------
+# fvt  (source/fvt/bind/fvt_sr_op_bind.cc:9-46)
+# --------------------------------------------------------------------------------------------
+def _fvt_fn(name, dtype):
+    return getattr(_lib.lib(), "a2p_fvt_%s_%s" % (name, "f32" if dtype == torch.float32 else "f64"))
+
+
+def _fvt_force_raw(binum, bilist, bnumneigh, bfirstneigh, nghost, dei):
+    B, P, U, _ = dei.shape
+    force = torch.empty((B, P + nghost, 3), dtype=dei.dtype, device=dei.device)
+    with torch.cuda.device(dei.device):
+        _lib.check(_fvt_fn("force_fwd", dei.dtype)(
+            _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum), _ptr(bilist),
+            _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(dei), _ptr(force), _stream(dei.device)))
+    return force
+
+
+def _fvt_force_bwd_raw(binum, bilist, bnumneigh, bfirstneigh, nghost, U, gF):
+    B, P = bilist.shape
+    out = torch.empty((B, P, U, 3), dtype=gF.dtype, device=gF.device)
+    with torch.cuda.device(gF.device):
+        _lib.check(_fvt_fn("force_bwd", gF.dtype)(
+            _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum), _ptr(bilist),
+            _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(gF), _ptr(out), _stream(gF.device)))
+    return out
+
+
+class _ForceSr(torch.autograd.Function):
+    """dei -> force.  The map is linear, so its backward is the adjoint gather and the
+    backward of that is this map again: any order of differentiation stays on the kernels."""
+
+    @staticmethod
+    def forward(ctx, dei, lists):
+        ctx.lists = lists
+        binum, bilist, bnumneigh, bfirstneigh, nghost = lists
+        return _fvt_force_raw(binum, bilist, bnumneigh, bfirstneigh, nghost, dei.contiguous())
+
+    @staticmethod
+    def backward(ctx, gF):
+        return _ForceSrAdjoint.apply(gF, ctx.lists), None
+
+
+class _ForceSrAdjoint(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gF, lists):
+        ctx.lists = lists
+        binum, bilist, bnumneigh, bfirstneigh, nghost = lists
+        return _fvt_force_bwd_raw(binum, bilist, bnumneigh, bfirstneigh, nghost, bfirstneigh.shape[2],
+                                  gF.contiguous())
+
+    @staticmethod
+    def backward(ctx, gg):
+        return _ForceSr.apply(gg, ctx.lists), None
+
+
+def ForceSrOp(binum, bilist, bnumneigh, bfirstneigh, nghost, umax_num_neighs, bdei_drij):
+    """[force[B, nlocal+nghost, 3]], differentiable w.r.t. bdei_drij to any order;
+    fvt_sr_op_bind.cc:9-29, src/force_sr_op.cc:11-179."""
+    _req(isinstance(bdei_drij, torch.Tensor) and bdei_drij.is_cuda,
+         "bdei_drij must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = bdei_drij.dtype, bdei_drij.device
+    _req(dtype in (torch.float32, torch.float64), "bdei_drij must be float32 or float64")
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh)):
+        _check_int(name, t, device)
+    _req(bdei_drij.dim() == 4 and bdei_drij.shape[3] == 3, "bdei_drij must have shape [B, nlocal, umax, 3]")
+    B, P, U, _ = bdei_drij.shape
+    _req(int(umax_num_neighs) == U, "umax_num_neighs does not match bdei_drij")
+    _req(tuple(bfirstneigh.shape) == (B, P, U) and tuple(bilist.shape) == (B, P) and
+         tuple(bnumneigh.shape) == (B, P) and tuple(binum.shape) == (B,), "neighbour tensors do not match")
+    _validate_batch(binum, bnumneigh, U, P)
+    out = _ForceSr.apply(bdei_drij, (binum, bilist, bnumneigh, bfirstneigh, int(nghost)))
+    _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return [out]
+
+
+def _fvt_virial_raw(bnumneigh, rcs, dei):
+    B, P, U, _ = dei.shape
+    v = torch.empty((B, 9), dtype=dei.dtype, device=dei.device)
+    with torch.cuda.device(dei.device):
+        _lib.check(_fvt_fn("virial_fwd", dei.dtype)(
+            _c.c_int(B), _c.c_int(P), _c.c_int(U), _ptr(bnumneigh), _ptr(rcs), _ptr(dei), _ptr(v),
+            _stream(dei.device)))
+    return v.view(B, 3, 3)
+
+
+def _fvt_virial_bwd_raw(bnumneigh, rcs, dei, gV, want_dei, want_rcs):
+    B, P, U, _ = dei.shape
+    gd = torch.empty_like(dei) if want_dei else None
+    gr = torch.empty_like(rcs) if want_rcs else None
+    with torch.cuda.device(dei.device):
+        _lib.check(_fvt_fn("virial_bwd", dei.dtype)(
+            _c.c_int(B), _c.c_int(P), _c.c_int(U), _ptr(bnumneigh), _ptr(rcs), _ptr(dei),
+            _ptr(gV.contiguous()), _ptr(gd), _ptr(gr), _stream(dei.device)))
+    return gd, gr
+
+
+class _VirialSr(torch.autograd.Function):
+    """(rcs, dei) -> virial, bilinear.  Backward is itself a Function of (gV, rcs, dei), so
+    create_graph=True callers (ai2pot/models/deepmd/se_r.py:316-330) differentiate again."""
+
+    @staticmethod
+    def forward(ctx, rcs, dei, bnumneigh):
+        ctx.save_for_backward(rcs, dei)
+        ctx.bnumneigh = bnumneigh
+        return _fvt_virial_raw(bnumneigh, rcs.contiguous(), dei.contiguous())
+
+    @staticmethod
+    def backward(ctx, gV):
+        rcs, dei = ctx.saved_tensors
+        grcs, gdei = _VirialSrBackward.apply(gV, rcs, dei, ctx.bnumneigh)
+        return grcs, gdei, None
+
+
+class _VirialSrBackward(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gV, rcs, dei, bnumneigh):
+        ctx.save_for_backward(gV, rcs, dei)
+        ctx.bnumneigh = bnumneigh
+        gd, gr = _fvt_virial_bwd_raw(bnumneigh, rcs.contiguous(), dei.contiguous(), gV, True, True)
+        return gr, gd
+
+    @staticmethod
+    def backward(ctx, ggr, ggd):
+        gV, rcs, dei = ctx.saved_tensors
+        nn = ctx.bnumneigh
+        # d/dgV: - sum ggd (x) rcs - sum dei (x) ggr, i.e. two forward virials
+        d_gV = _VirialSr.apply(rcs, ggd, nn) + _VirialSr.apply(ggr, dei, nn)
+        # d/drcs[.,b] = - sum_a gV[a,b] ggd[.,a];  d/ddei[.,a] = - sum_b gV[a,b] ggr[.,b]
+        d_rcs, _ = _VirialSrBackward.apply(gV, rcs, ggd, nn)
+        _, d_dei = _VirialSrBackward.apply(gV, ggr, dei, nn)
+        return d_gV, d_rcs, d_dei, None
+
+
+def VirialSrOp(bnumneigh, brcs, umax_num_neighs, bdei_drij):
+    """[virial[B, 3, 3]], differentiable w.r.t. brcs and bdei_drij;
+    fvt_sr_op_bind.cc:31-46, src/virial_sr_op.cc:10-164."""
+    _req(isinstance(bdei_drij, torch.Tensor) and bdei_drij.is_cuda,
+         "bdei_drij must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = bdei_drij.dtype, bdei_drij.device
+    _req(dtype in (torch.float32, torch.float64), "bdei_drij must be float32 or float64")
+    _check_int("bnumneigh", bnumneigh, device)
+    _req(isinstance(brcs, torch.Tensor) and brcs.dtype == dtype and brcs.device == device,
+         "brcs must match bdei_drij in dtype and device")
+    _req(bdei_drij.dim() == 4 and bdei_drij.shape[3] == 3 and brcs.shape == bdei_drij.shape,
+         "brcs and bdei_drij must have shape [B, nlocal, umax, 3]")
+    B, P, U, _ = bdei_drij.shape
+    _req(int(umax_num_neighs) == U and tuple(bnumneigh.shape) == (B, P), "shapes do not match")
+    if bnumneigh.numel():
+        _req(int(bnumneigh.max().item()) <= U, "a neighbour count exceeds umax_num_neighs")
+    return [_VirialSr.apply(brcs, bdei_drij, bnumneigh)]

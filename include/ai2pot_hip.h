@@ -166,6 +166,43 @@ int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weig
                      float* rmse, float* etot, float* force, float* virial, float* dcoeffs, float* dlinear,
                      float* dbias, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Short-range force / virial from per-pair derivatives -- replaces the compute of
+ * torch.ops.fvt.ForceSrOp and torch.ops.fvt.VirialSrOp, forward and backward
+ * (source/fvt/bind/fvt_sr_op_bind.cc:9-46; src/force_sr_op.cc:11-179, src/virial_sr_op.cc:10-164
+ * -> include/force_sr.h:50-124, include/virial_sr.h:24-51).
+ * dei_drij[B][nlocal][umax][3]; force[B][nlocal+nghost][3]; virial[B][9]; rows ii < binum[b]
+ * (force) or all nlocal rows (virial, as the reference) and slots s < bnumneigh[b][ii] count.
+ *   force_fwd : force[c] = sum_s dei[ii,s] - sum_{pairs with neighbour c} dei   (c = bilist[ii])
+ *   force_bwd : grad_dei[ii,s,k] = grad_force[c,k] - grad_force[j,k], zero on padding
+ *   virial_fwd: virial[a*3+b] = - sum dei[ii,s,a] rcs[ii,s,b]
+ *   virial_bwd: grad_dei[ii,s,a] = - sum_b grad_virial[a*3+b] rcs[ii,s,b];
+ *               grad_rcs[ii,s,b] = - sum_a grad_virial[a*3+b] dei[ii,s,a]   (either may be NULL)
+ * The dense Jacobians the reference builds are never formed.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_fvt_force_fwd_f32(int batch, int nlocal, int umax, int nghost, const int* binum, const int* bilist,
+                          const int* bnumneigh, const int* bfirstneigh, const float* dei_drij, float* force,
+                          void* stream);
+int a2p_fvt_force_fwd_f64(int batch, int nlocal, int umax, int nghost, const int* binum, const int* bilist,
+                          const int* bnumneigh, const int* bfirstneigh, const double* dei_drij, double* force,
+                          void* stream);
+int a2p_fvt_force_bwd_f32(int batch, int nlocal, int umax, int nghost, const int* binum, const int* bilist,
+                          const int* bnumneigh, const int* bfirstneigh, const float* grad_force,
+                          float* grad_dei, void* stream);
+int a2p_fvt_force_bwd_f64(int batch, int nlocal, int umax, int nghost, const int* binum, const int* bilist,
+                          const int* bnumneigh, const int* bfirstneigh, const double* grad_force,
+                          double* grad_dei, void* stream);
+int a2p_fvt_virial_fwd_f32(int batch, int nlocal, int umax, const int* bnumneigh, const float* rcs,
+                           const float* dei_drij, float* virial, void* stream);
+int a2p_fvt_virial_fwd_f64(int batch, int nlocal, int umax, const int* bnumneigh, const double* rcs,
+                           const double* dei_drij, double* virial, void* stream);
+int a2p_fvt_virial_bwd_f32(int batch, int nlocal, int umax, const int* bnumneigh, const float* rcs,
+                           const float* dei_drij, const float* grad_virial, float* grad_dei, float* grad_rcs,
+                           void* stream);
+int a2p_fvt_virial_bwd_f64(int batch, int nlocal, int umax, const int* bnumneigh, const double* rcs,
+                           const double* dei_drij, const double* grad_virial, double* grad_dei,
+                           double* grad_rcs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
