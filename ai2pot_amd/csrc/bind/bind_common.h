@@ -1,0 +1,99 @@
+// Shared helpers of the operator bind libraries (libnep_bind.so, libmtpr_bind.so,
+// libfvt_sr_op_bind.so): argument checks with TORCH_CHECK, raw pointers, the current HIP
+// stream, and translation of libai2pot_hip status codes into c10::Error.
+#pragma once
+#include <torch/extension.h>
+#include <torch/library.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include "../../../include/ai2pot_hip.h"
+
+namespace a2p_bind {
+
+// Makes the tensor's device current for the duration of a call: libai2pot_hip keeps its
+// workspace per current device.
+struct DeviceGuard {
+    int prev = -1;
+    explicit DeviceGuard(const at::Tensor& t)
+    {
+        TORCH_CHECK(hipGetDevice(&prev) == hipSuccess, "hipGetDevice failed");
+        const int want = t.device().index();
+        if (want >= 0 && want != prev) {
+            TORCH_CHECK(hipSetDevice(want) == hipSuccess, "hipSetDevice failed");
+        } else {
+            prev = -1;
+        }
+    }
+    ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
+};
+
+inline void* current_stream(const at::Tensor& t)
+{
+    return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream();
+}
+
+inline void check_rc(int rc)
+{
+    TORCH_CHECK(rc == A2P_OK, "libai2pot_hip error ", rc, ": ", a2p_last_error());
+}
+
+inline void check_device_float(const at::Tensor& ref, const at::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.defined(), name, " is undefined");
+    TORCH_CHECK(t.scalar_type() == ref.scalar_type(), name, " must have the dtype of brcs (", ref.scalar_type(),
+                "), got ", t.scalar_type());
+    TORCH_CHECK(t.device() == ref.device(), name, " must be on the device of brcs");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+inline void check_device_int(const at::Tensor& ref, const at::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.defined(), name, " is undefined");
+    TORCH_CHECK(t.scalar_type() == at::kInt, name, " must be int32");
+    TORCH_CHECK(t.device() == ref.device(), name, " must be on the device of brcs");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+struct Batch {
+    int B, P, U, nghost;
+};
+
+// The 7-tensor neighbour contract (source/descriptor/mtpr/README.md:4-9).
+inline Batch check_batch(const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                         const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                         int64_t nghost)
+{
+    TORCH_CHECK(brcs.is_cuda(), "brcs must be on a HIP device: this build has no CPU path");
+    TORCH_CHECK(brcs.scalar_type() == at::kFloat || brcs.scalar_type() == at::kDouble,
+                "brcs must be float32 or float64");
+    TORCH_CHECK(brcs.is_contiguous() && brcs.dim() == 4 && brcs.size(3) == 3, "brcs must be contiguous [B, P, U, 3]");
+    check_device_int(brcs, binum, "binum");
+    check_device_int(brcs, bilist, "bilist");
+    check_device_int(brcs, bnumneigh, "bnumneigh");
+    check_device_int(brcs, bfirstneigh, "bfirstneigh");
+    check_device_int(brcs, btypes, "btypes");
+    Batch s{(int)brcs.size(0), (int)brcs.size(1), (int)brcs.size(2), (int)nghost};
+    TORCH_CHECK(nghost >= 0, "nghost must be non-negative");
+    TORCH_CHECK(bfirstneigh.dim() == 3 && bfirstneigh.size(0) == s.B && bfirstneigh.size(1) == s.P &&
+                    bfirstneigh.size(2) == s.U, "bfirstneigh must have shape [B, P, U]");
+    TORCH_CHECK(bilist.numel() == (int64_t)s.B * s.P && bnumneigh.numel() == (int64_t)s.B * s.P,
+                "bilist and bnumneigh must have shape [B, P]");
+    TORCH_CHECK(binum.numel() == s.B, "binum must have shape [B]");
+    TORCH_CHECK(btypes.numel() == (int64_t)s.B * (s.P + s.nghost), "btypes must have shape [B, P + nghost]");
+    return s;
+}
+
+// Errors the reference leaves to a commented-out assert (source/nblist/include/neighborList.h:550)
+// or to out-of-bounds reads; one device status read per call.
+inline void check_device_status(const at::Tensor& t)
+{
+    check_rc(a2p_check_status(current_stream(t)));
+}
+
+inline void require_no_zbl(double zbl_rmax)
+{
+    TORCH_CHECK(zbl_rmax == 0.0, "the ZBL correction (zbl_rmax > 0) is not implemented in this build");
+}
+
+}  // namespace a2p_bind

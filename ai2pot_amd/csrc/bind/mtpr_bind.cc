@@ -1,0 +1,323 @@
+// libmtpr_bind.so -- registers torch.ops.mtpr.* with the reference's schemas
+// (source/descriptor/mtpr/bind/mtpr_bind.cc:30-569) on top of libai2pot_hip.so:
+// set_ai2pot_path, mtpParamOp, linearMtpToEFVOp, linearMtpToEFOp, linearMtpToLossOp and
+// linearMtpToEFLossOp (autograd to coeffs, linear_coeffs, type_bias only, as
+// src/linearMtpOp.cc:1732-1765).  The legacy and solver operators of the reference
+// (mtpBasisOp, LinMatrixLinVectorOp, CoeffsSchmidtOrthOp, linearMtpToEsitesOp,
+// linearMtpToDescriptorsOp) are not part of this build.
+#include "bind_common.h"
+
+#include <cstdlib>
+#include <fstream>
+#include <map>
+#include <mutex>
+#include <regex>
+#include <set>
+#include <sstream>
+#include <tuple>
+
+using namespace a2p_bind;
+using torch::autograd::AutogradContext;
+using torch::autograd::variable_list;
+
+namespace {
+
+std::string g_ai2pot_path;
+
+// ---- template files (source/descriptor/mtpr/src/mtpParam.cc:32-43, 65-214) ---------------------
+std::string template_dir()
+{
+    const char* env = std::getenv("AI2POT_PATH");
+    if (env) return std::string(env) + "/source/descriptor/mtpr/MTP_templates/";
+    return g_ai2pot_path + "/_data/MTP_templates/";
+}
+
+struct Tables {
+    int n_moms = 0;
+    std::vector<int> basic, times, mapping;     // flattened [n,4], [n,4], [n]
+};
+
+std::vector<int> ints_after(const std::string& body, const std::string& key)
+{
+    std::regex re("(^|\\n)\\s*" + key + "\\s*=\\s*([^\\n]*)");
+    std::smatch m;
+    TORCH_CHECK(std::regex_search(body, m, re), "Cannot read ", key, ".");
+    std::vector<int> out;
+    const std::string line = m[2];
+    std::regex num("-?\\d+");
+    for (auto it = std::sregex_iterator(line.begin(), line.end(), num); it != std::sregex_iterator(); ++it)
+        out.push_back(std::stoi(it->str()));
+    return out;
+}
+
+Tables load_tables(int level)
+{
+    TORCH_CHECK(level >= 2 && level <= 28 && level % 2 == 0, "mtp level must be an even number in 2..28");
+    std::string name = level <= 4 ? "depreciated-0" + std::to_string(level) + ".almtp"
+                                  : (level < 10 ? "0" : "") + std::to_string(level) + ".almtp";
+    const std::string path = template_dir() + name;
+    std::ifstream ifs(path);
+    TORCH_CHECK(ifs.is_open(), "Cannot open file ", path);
+    std::string line, body;
+    for (int i = 0; i < 10; i++) std::getline(ifs, line);        // header is ignored, mtpParam.cc:92-93
+    std::stringstream ss;
+    ss << ifs.rdbuf();
+    body = ss.str();
+    Tables t;
+    auto one = [&](const char* key) {
+        auto v = ints_after(body, key);
+        TORCH_CHECK(v.size() == 1, "Cannot read ", key, ".");
+        return v[0];
+    };
+    t.n_moms = one("alpha_moments_count");
+    const int nb = one("alpha_index_basic_count"), nt = one("alpha_index_times_count"),
+              ns = one("alpha_scalar_moments");
+    t.basic = ints_after(body, "alpha_index_basic");
+    t.times = nt ? ints_after(body, "alpha_index_times") : std::vector<int>();
+    t.mapping = ints_after(body, "alpha_moment_mapping");
+    TORCH_CHECK((int)t.basic.size() == 4 * nb, "Cannot read alpha_index_basic.");
+    TORCH_CHECK((int)t.times.size() == 4 * nt, "Cannot read alpha_index_times.");
+    TORCH_CHECK((int)t.mapping.size() == ns, "Cannot read alpha_moment_mapping.");
+    return t;
+}
+
+variable_list mtp_param_op(int64_t level)
+{
+    Tables t = load_tables((int)level);
+    const int nb = (int)t.basic.size() / 4, nt = (int)t.times.size() / 4;
+    // radial-function indices each moment depends on (mtpParam.cc:435-469)
+    std::vector<std::set<int>> mus(t.n_moms);
+    for (int i = 0; i < nb && i < t.n_moms; i++) mus[i].insert(t.basic[i * 4]);
+    for (int i = nb; i < t.n_moms; i++)
+        for (int e = 0; e < nt; e++)
+            if (t.times[e * 4 + 3] == i) {
+                const auto &a = mus[t.times[e * 4]], &b = mus[t.times[e * 4 + 1]];
+                mus[i].insert(a.begin(), a.end());
+                mus[i].insert(b.begin(), b.end());
+            }
+    size_t width = 0;
+    int nmus = 1;
+    for (auto& s : mus) width = std::max(width, s.size());
+    for (int i = 0; i < nb; i++) nmus = std::max(nmus, t.basic[i * 4] + 1);
+    auto iopt = at::TensorOptions().dtype(at::kInt);
+    at::Tensor basic = at::from_blob(t.basic.data(), {nb, 4}, iopt).clone();
+    at::Tensor times = nt ? at::from_blob(t.times.data(), {nt, 4}, iopt).clone() : at::zeros({0, 4}, iopt);
+    at::Tensor mapping = at::from_blob(t.mapping.data(), {(int64_t)t.mapping.size()}, iopt).clone();
+    at::Tensor num = at::zeros({t.n_moms}, iopt);
+    at::Tensor m4m = at::zeros({t.n_moms, (int64_t)width}, iopt) - 1;
+    for (int i = 0; i < t.n_moms; i++) {
+        num.data_ptr<int>()[i] = (int)mus[i].size();
+        int c = 0;
+        for (int v : mus[i]) m4m.data_ptr<int>()[i * width + (c++)] = v;
+    }
+    return {torch::tensor(t.n_moms, iopt), basic, times, mapping, num, m4m, torch::tensor(nmus, iopt)};
+}
+
+// ---- plan cache ---------------------------------------------------------------------------------
+struct PlanEntry {
+    void* handle;
+    int n_scalar;
+};
+std::mutex g_plan_mutex;
+std::map<std::tuple<int, int64_t, const void*, int64_t, uint32_t, const void*, int64_t, uint32_t, const void*,
+                    int64_t, uint32_t>, PlanEntry> g_plans;
+
+PlanEntry get_plan(int device, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times,
+                   const at::Tensor& mapping)
+{
+    // the tables are model constants (registered buffers, ai2pot/models/mtp/linear_mtp.py:63-69):
+    // read back once, cached by storage address, size and version
+    auto key = std::make_tuple(device, n_moms, basic.data_ptr(), basic.numel(), basic._version(),
+                               times.data_ptr(), times.numel(), times._version(), mapping.data_ptr(),
+                               mapping.numel(), mapping._version());
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) return it->second;
+    for (auto* t : {&basic, &times, &mapping})
+        TORCH_CHECK(t->scalar_type() == at::kInt, "the MTP index tensors must be int32");
+    TORCH_CHECK(basic.dim() == 2 && basic.size(1) == 4, "alpha_index_basic must have shape [n, 4]");
+    TORCH_CHECK(times.numel() == 0 || (times.dim() == 2 && times.size(1) == 4),
+                "alpha_index_times must have shape [n, 4]");
+    at::Tensor hb = basic.cpu().contiguous(), ht = times.cpu().contiguous(), hm = mapping.cpu().contiguous();
+    PlanEntry e;
+    e.n_scalar = (int)hm.numel();
+    check_rc(a2p_mtp_plan_create((int)n_moms, (int)hb.size(0), hb.data_ptr<int>(), (int)(ht.numel() / 4),
+                                 ht.numel() ? ht.data_ptr<int>() : nullptr, e.n_scalar, hm.data_ptr<int>(),
+                                 &e.handle));
+    g_plans[key] = e;
+    return e;
+}
+
+struct MtpCtx {
+    Batch s;
+    int ntypes;
+    PlanEntry plan;
+};
+
+MtpCtx check_mtp(int64_t K, const at::Tensor& coeffs, const at::Tensor& lin, const at::Tensor& bias,
+                 int64_t n_moms, const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping,
+                 int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                 const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                 const at::Tensor& type_map, int64_t nghost, const at::Tensor& q_scaler)
+{
+    MtpCtx c;
+    c.s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+    c.ntypes = (int)type_map.numel();
+    TORCH_CHECK(c.ntypes > 0, "type_map is empty");
+    check_device_float(brcs, coeffs, "coeffs");
+    check_device_float(brcs, lin, "linear_coeffs");
+    check_device_float(brcs, bias, "type_bias");
+    check_device_float(brcs, q_scaler, "q_scaler");
+    a2p_bind::DeviceGuard guard(brcs);
+    c.plan = get_plan(brcs.device().index(), n_moms, basic, times, mapping);
+    TORCH_CHECK(coeffs.numel() == (int64_t)c.ntypes * c.ntypes * nmus * K, "coeffs size mismatch");
+    TORCH_CHECK(lin.numel() == c.plan.n_scalar && q_scaler.numel() == c.plan.n_scalar,
+                "linear_coeffs and q_scaler must have alpha_scalar_moments elements");
+    TORCH_CHECK(bias.numel() == c.ntypes, "type_bias size mismatch");
+    return c;
+}
+
+variable_list mtp_efv(bool want_virial, int64_t K, double scaling, const at::Tensor& coeffs,
+                      const at::Tensor& lin, const at::Tensor& bias, int64_t n_moms, const at::Tensor& basic,
+                      const at::Tensor& times, const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum,
+                      const at::Tensor& bilist, const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
+                      const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost,
+                      double rmax, double rmin, const at::Tensor& q_scaler, double zbl_rmax)
+{
+    require_no_zbl(zbl_rmax);
+    MtpCtx c = check_mtp(K, coeffs, lin, bias, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                         bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
+    a2p_bind::DeviceGuard guard(brcs);
+    auto opt = brcs.options();
+    at::Tensor e = at::zeros({c.s.B}, opt), f = at::zeros({c.s.B, c.s.P + c.s.nghost, 3}, opt), v;
+    if (want_virial) v = at::zeros({c.s.B, 9}, opt);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble)
+        rc = a2p_mtp_efv_f64(c.plan.handle, (int)K, scaling, coeffs.data_ptr<double>(), lin.data_ptr<double>(),
+                             bias.data_ptr<double>(), (int)nmus, c.ntypes, q_scaler.data_ptr<double>(), rmax, rmin,
+                             c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                             bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(),
+                             btypes.data_ptr<int>(), e.data_ptr<double>(), f.data_ptr<double>(),
+                             v.defined() ? v.data_ptr<double>() : nullptr, st);
+    else
+        rc = a2p_mtp_efv_f32(c.plan.handle, (int)K, scaling, coeffs.data_ptr<float>(), lin.data_ptr<float>(),
+                             bias.data_ptr<float>(), (int)nmus, c.ntypes, q_scaler.data_ptr<float>(), rmax, rmin,
+                             c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                             bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(),
+                             btypes.data_ptr<int>(), e.data_ptr<float>(), f.data_ptr<float>(),
+                             v.defined() ? v.data_ptr<float>() : nullptr, st);
+    check_rc(rc);
+    check_device_status(brcs);
+    if (want_virial) return {e, f, v};
+    return {e, f};
+}
+
+// forward: [bloss, e_rmse, f_rmse(, v_rmse)]; backward: grad_output @ per-structure gradients
+struct LossFunction : public torch::autograd::Function<LossFunction> {
+    static variable_list forward(AutogradContext* ctx, bool with_virial, double e_w, double f_w, double v_w,
+                                 const at::Tensor& e_dft, const at::Tensor& f_dft, const at::Tensor& v_dft_in,
+                                 int64_t K, double scaling, const at::Tensor& coeffs, const at::Tensor& lin,
+                                 const at::Tensor& bias, int64_t n_moms, const at::Tensor& basic,
+                                 const at::Tensor& times, const at::Tensor& mapping, int64_t nmus,
+                                 const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                                 const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                                 const at::Tensor& type_map, int64_t nghost, double rmax, double rmin,
+                                 const at::Tensor& q_scaler)
+    {
+        TORCH_CHECK(nghost == 0, "the loss operator requires nghost == 0, as the reference does");
+        MtpCtx c = check_mtp(K, coeffs, lin, bias, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                             bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
+        a2p_bind::DeviceGuard guard(brcs);
+        auto opt = brcs.options();
+        const int B = c.s.B, P = c.s.P;
+        at::Tensor v_dft = with_virial ? v_dft_in : at::zeros({B, 9}, opt);
+        check_device_float(brcs, e_dft, "betot_dft");
+        check_device_float(brcs, f_dft, "bforce_dft");
+        check_device_float(brcs, v_dft, "bvirial_dft");
+        TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
+                    "label tensors must have shapes [B], [B, P, 3], [B, 9]");
+        const bool need = coeffs.requires_grad() || lin.requires_grad() || bias.requires_grad();
+        at::Tensor bloss = at::zeros({B}, opt), rmse = at::zeros({3}, opt), e = at::zeros({B}, opt),
+                   f = at::zeros({B, P, 3}, opt), v = at::zeros({B, 9}, opt), dc, dl, db;
+        if (need) {
+            dc = at::zeros({B, coeffs.numel()}, opt);
+            dl = at::zeros({B, lin.numel()}, opt);
+            db = at::zeros({B, bias.numel()}, opt);
+        }
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_mtp_loss_f64(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
+                                  (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
+                                  rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                  bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                  btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
+                                  st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_mtp_loss_f32(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
+                                  (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
+                                  rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                  bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                  btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
+                                  st);
+        }
+        check_rc(rc);
+        check_device_status(brcs);
+        ctx->saved_data["need"] = need;
+        if (need) ctx->save_for_backward({dc, dl, db});
+        ctx->saved_data["shape_c"] = coeffs.sizes().vec();
+        ctx->saved_data["shape_l"] = lin.sizes().vec();
+        ctx->saved_data["shape_b"] = bias.sizes().vec();
+        if (with_virial) return {bloss, rmse.slice(0, 0, 1).clone(), rmse.slice(0, 1, 2).clone(), rmse.slice(0, 2, 3).clone()};
+        return {bloss, rmse.slice(0, 0, 1).clone(), rmse.slice(0, 1, 2).clone()};
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(28);                   // one slot per forward argument after ctx
+        if (!ctx->saved_data["need"].toBool()) return out;
+        auto saved = ctx->get_saved_variables();
+        at::Tensor gl = grads[0].contiguous();
+        out[9] = torch::matmul(gl, saved[0]).reshape(ctx->saved_data["shape_c"].toIntVector());
+        out[10] = torch::matmul(gl, saved[1]).reshape(ctx->saved_data["shape_l"].toIntVector());
+        out[11] = torch::matmul(gl, saved[2]).reshape(ctx->saved_data["shape_b"].toIntVector());
+        return out;
+    }
+};
+
+}  // namespace
+
+#define MTP_EFV_ARGS int64_t K, double scaling, const at::Tensor& coeffs, const at::Tensor& lin, \
+    const at::Tensor& bias, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times, \
+    const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist, \
+    const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs, \
+    const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax, double rmin, \
+    const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin, const at::Tensor& zbl_cks, \
+    const at::Tensor& zbl_dks
+#define MTP_EFV_PASS K, scaling, coeffs, lin, bias, n_moms, basic, times, mapping, nmus, binum, bilist, \
+    bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler
+
+TORCH_LIBRARY(mtpr, m)
+{
+    m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
+    m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
+    m.def("linearMtpToEFVOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(true, MTP_EFV_PASS, zbl_rmax); });
+    m.def("linearMtpToEFOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(false, MTP_EFV_PASS, zbl_rmax); });
+    m.def("linearMtpToLossOp",
+          [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
+             const at::Tensor& v_dft, MTP_EFV_ARGS) -> variable_list {
+              require_no_zbl(zbl_rmax);
+              return LossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, MTP_EFV_PASS);
+          });
+    m.def("linearMtpToEFLossOp",
+          [](double e_w, double f_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
+             MTP_EFV_ARGS) -> variable_list {
+              require_no_zbl(zbl_rmax);
+              // no virial labels in this variant: zero weight, zero labels
+              return LossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
+                                         at::zeros({e_dft.numel(), 9}, e_dft.options()), MTP_EFV_PASS);
+          });
+}

@@ -131,6 +131,25 @@ def mtp_param(level):
     return out
 
 
+def write_almtp(path, t):
+    """Write tables in the template text format (ten header lines, then the six table
+    entries), e.g. to materialise a template directory from the packaged archive."""
+    def rows(a):
+        return "{" + ", ".join("{" + ", ".join(str(int(v)) for v in r) + "}" for r in a) + "}"
+    header = ["MTP", "version = 1.1.0", "potential_name = MTP1m", "species_count = 1", "potential_tag = ",
+              "radial_basis_type = RBChebyshev", "\tmin_dist = 2", "\tmax_dist = 5", "\tradial_basis_size = 8",
+              "\tradial_funcs_count = %d" % t["nmus"]]
+    body = ["alpha_moments_count = %d" % t["alpha_moments_count"],
+            "alpha_index_basic_count = %d" % t["alpha_index_basic"].shape[0],
+            "alpha_index_basic = " + rows(t["alpha_index_basic"]),
+            "alpha_index_times_count = %d" % t["alpha_index_times"].shape[0],
+            "alpha_index_times = " + rows(t["alpha_index_times"]),
+            "alpha_scalar_moments = %d" % t["alpha_moment_mapping"].size,
+            "alpha_moment_mapping = {" + ", ".join(str(int(v)) for v in t["alpha_moment_mapping"]) + "}"]
+    with open(path, "w") as fh:
+        fh.write("\n".join(header + body) + "\n")
+
+
 def validate_tables(t):
     """Host-side checks the kernels rely on; raises MtpError on violation."""
     n = t["alpha_moments_count"]

@@ -1,0 +1,187 @@
+"""The drop-in libraries a reference installation would load in place of its own
+(ai2pot/fromcc/__init__.py:53-134): torch.ops.nep / mtpr / fvt registered by
+ai2pot_amd/_lib/lib*_bind.so and the CPython module `nblist`.  They must give the same
+results as the Python mirror of the operators (which the oracle parity tests cover) and be
+callable from TorchScript by name, as the exported models do (ai2pot/models/nep/nep.py:297-324)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+from ai2pot_amd import mtp_param, synth
+from conftest import to_device
+
+pytestmark = pytest.mark.gpu
+
+LIBDIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ai2pot_amd", "_lib")
+
+
+@pytest.fixture(scope="module")
+def dropin():
+    import torch
+    for name in ("libnep_bind.so", "libmtpr_bind.so", "libfvt_sr_op_bind.so"):
+        path = os.path.join(LIBDIR, name)
+        assert os.path.exists(path), "%s missing: run python -m ai2pot_amd.build --bind" % path
+        torch.ops.load_library(path)
+    if LIBDIR not in sys.path:
+        sys.path.append(LIBDIR)
+    import nblist
+    return nblist
+
+
+def small(oracle, n=120, nt=3, rcut=7.0, seed=11, dtype=np.float32):
+    lat, pos = synth.random_packed(n, [14.0, 15.0, 13.0], 2.2, seed)
+    ty = synth.rng_randint(seed + 1, n, nt)
+    return lat, pos, ty, oracle.nblist(lat.astype(dtype), ty, pos.astype(dtype), rcut, 200)
+
+
+def test_nblist_module(oracle, dropin):
+    lat, pos, ty, ref = small(oracle)
+    out = dropin.find_info4mlff(lat.astype(np.float32), ty, pos.astype(np.float32), 7.0, 200, True,
+                                [True, True, True], False)
+    assert out[0] == ref[0] and out[6] == 0
+    for a, b in zip(out[1:6], ref[1:6]):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    out64 = dropin.find_info4mlff(lat, ty.astype(np.int64), pos, 7.0, 200, True, [True, True, True], True)
+    ref64 = oracle.nblist(lat, ty, pos, 7.0, 200, sort=True)
+    for a, b in zip(out64[1:6], ref64[1:6]):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    with pytest.raises(TypeError):
+        dropin.find_info4mlff(lat, ty, pos, 7, 200, True, [True, True, True], False)
+    with pytest.raises(RuntimeError):
+        dropin.find_info4mlff(lat, ty, pos, 7.0, 10, True, [True, True, True], False)
+
+
+def nep_args(oracle, dtype):
+    import torch
+    from test_gpu_nep import _model_to_device
+    _, _, _, o = small(oracle)
+    nb = synth.pack_batch([o])
+    m = synth.nep_model()
+    md = _model_to_device(m, dtype)
+    d = to_device(nb, dtype)
+    return (8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"], d["binum"], d["bilist"],
+            d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], 0, 7.0, 4.0, md["q_scaler"],
+            0.0, 0.0, torch.zeros(36, dtype=dtype, device="cuda:0"), torch.zeros(36, dtype=dtype, device="cuda:0"))
+
+
+def test_nep_ops_and_torchscript(oracle, dropin):
+    import torch
+    from ai2pot_amd import ops
+    args = nep_args(oracle, torch.float32)
+    got = torch.ops.nep.nepToEFVOp(*args)
+    want = ops.nepToEFVOp(*args)
+    assert len(got) == 3
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    ef = torch.ops.nep.nepToEFOp(*args)
+    assert len(ef) == 2 and torch.equal(ef[0], want[0]) and torch.equal(ef[1], want[1])
+    d = torch.ops.nep.nepToDescriptorsOp(*(args[:5] + args[9:19]))
+    assert d[0].shape == (1, 120, 22)
+    assert torch.equal(d[0], ops.nepToDescriptorsOp(*(args[:5] + args[9:19]))[0])
+
+    class Wrapper(torch.nn.Module):
+        def __init__(self, consts):
+            super().__init__()
+            self.coeffs, self.w0, self.b0, self.w1, self.bias, self.type_map, self.qs, self.z = consts
+
+        @torch.jit.export
+        def predict_efv(self, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes):
+            return torch.ops.nep.nepToEFVOp(8, 6, 4, 4, self.coeffs, self.w0, self.b0, self.w1, self.bias, binum,
+                                            bilist, bnumneigh, bfirstneigh, brcs, btypes, self.type_map, 0, 7.0, 4.0,
+                                            self.qs, 0.0, 0.0, self.z, self.z)
+
+        def forward(self, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes):
+            return self.predict_efv(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes)
+
+    mod = torch.jit.script(Wrapper((args[4], args[5], args[6], args[7], args[8], args[15], args[19], args[22])))
+    out = mod.predict_efv(*args[9:15])
+    for a, b in zip(out, want):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError):                      # wrong dtype is an error, not a crash
+        torch.ops.nep.nepToEFVOp(*(args[:13] + (args[13].double(),) + args[14:]))
+    with pytest.raises(RuntimeError):
+        torch.ops.nep.nepToLossOp(1.0, 1.0, 1.0, args[4], args[4], args[4], *args)
+
+
+def test_mtpr_ops(oracle, dropin, tmp_path):
+    import torch
+    from ai2pot_amd import ops
+    from test_gpu_mtp import model_to_device
+    # template directory materialised from the packaged tables; the library parses the text file
+    d = tmp_path / "_data" / "MTP_templates"
+    d.mkdir(parents=True)
+    mtp_param.write_almtp(str(d / "10.almtp"), mtp_param.mtp_param(10))
+    os.environ.pop("AI2POT_PATH", None)
+    torch.ops.mtpr.set_ai2pot_path(str(tmp_path))
+    p = torch.ops.mtpr.mtpParamOp(10)
+    want = ops.mtpParamOp(10)
+    assert len(p) == 7
+    for a, b in zip(p, want):
+        assert a.dtype == torch.int32 and torch.equal(a, b)
+    with pytest.raises(RuntimeError):
+        torch.ops.mtpr.mtpParamOp(12)                      # no such template file in that directory
+
+    lat, pos, ty, o = small(oracle, n=60, nt=2, rcut=5.0, dtype=np.float64)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.02
+    m = synth.mtp_model(mtp_param.mtp_param(10), 2, 8, 5.0, 1.0, 77)
+    md = model_to_device(m, torch.float64)
+    dv = to_device(nb, torch.float64)
+    z = torch.zeros(16, dtype=torch.float64, device="cuda:0")
+    efv_args = (8, 1.0, md["coeffs"], md["linear_coeffs"], md["type_bias"], int(p[0]), p[1].cuda(), p[2].cuda(),
+                p[3].cuda(), int(p[6]), dv["binum"], dv["bilist"], dv["bnumneigh"], dv["bfirstneigh"], dv["brcs"],
+                dv["btypes"], md["type_map"], 0, 5.0, 1.0, md["q_scaler"], 0.0, 0.0, z, z)
+    got = torch.ops.mtpr.linearMtpToEFVOp(*efv_args)
+    ref = oracle.mtp_efv(m, nb)
+    for a, b in zip(got, ref):
+        assert np.abs(a.cpu().numpy() - b).max() <= 1e-10 * np.abs(b).max()
+    assert len(torch.ops.mtpr.linearMtpToEFOp(*efv_args)) == 2
+
+    B, P = nb["bilist"].shape
+    lab = dict(energy=synth.rng_normal(1, B, -200, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+               virial=synth.rng_normal(3, B * 9).reshape(B, 9))
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    params = [md[k].clone().requires_grad_(True) for k in ("coeffs", "linear_coeffs", "type_bias")]
+    out = torch.ops.mtpr.linearMtpToLossOp(1.0, 0.7, 0.3, t(lab["energy"]), t(lab["force"]), t(lab["virial"]), 8, 1.0,
+                                           params[0], params[1], params[2], *efv_args[5:])
+    assert len(out) == 4 and out[0].shape == (B,)
+    out[0].sum().backward()
+    r = oracle.mtp_loss_step(m, nb, (1.0, 0.7, 0.3), lab)
+    close = lambda a, b: np.abs(a - b).max() <= 1e-10 * np.abs(b).max()
+    assert close(out[0].detach().cpu().numpy(), r["bloss"])
+    assert close(torch.cat(out[1:]).detach().cpu().numpy(), r["rmse"])
+    assert close(params[0].grad.cpu().numpy(), r["dcoeffs"].sum(0))
+    assert close(params[1].grad.cpu().numpy(), r["dlinear"].sum(0))
+    assert close(params[2].grad.cpu().numpy(), r["dbias"].sum(0))
+    # energy + force loss: the same with the virial weight switched off
+    params2 = [md[k].clone().requires_grad_(True) for k in ("coeffs", "linear_coeffs", "type_bias")]
+    out2 = torch.ops.mtpr.linearMtpToEFLossOp(1.0, 0.7, t(lab["energy"]), t(lab["force"]), 8, 1.0, params2[0],
+                                              params2[1], params2[2], *efv_args[5:])
+    assert len(out2) == 3
+    out2[0].sum().backward()
+    r2 = oracle.mtp_loss_step(m, nb, (1.0, 0.7, 0.0), lab)
+    assert close(out2[0].detach().cpu().numpy(), r2["bloss"]) and close(params2[0].grad.cpu().numpy(), r2["dcoeffs"].sum(0))
+
+
+def test_fvt_ops(oracle, dropin):
+    import torch
+    from test_gpu_fvt import dev, random_case
+    binum, bilist, nn, fn, dei, rcs = random_case(B=2, P=5, U=4, nghost=2, seed=3)
+    U = fn.shape[2]
+    lists = (dev(binum), dev(bilist), dev(nn), dev(fn))
+    d = dev(dei).requires_grad_(True)
+    r = dev(rcs).requires_grad_(True)
+    force = lambda x: torch.ops.fvt.ForceSrOp(lists[0], lists[1], lists[2], lists[3], 2, U, x)[0]
+    virial = lambda rr, x: torch.ops.fvt.VirialSrOp(lists[2], rr, U, x)[0]
+    f = force(d)
+    for b in range(2):
+        n = binum[b]
+        fr, _ = oracle.fvt_force(bilist[b, :n], nn[b, :n], fn[b, :n], 2 + 5 - n, dei[b, :n])
+        assert np.abs(f[b].detach().cpu().numpy() - fr).max() < 1e-12
+    assert virial(r, d).shape == (2, 3, 3)
+    assert torch.autograd.gradcheck(force, (d,), eps=1e-6, atol=1e-7)
+    assert torch.autograd.gradgradcheck(force, (d,), eps=1e-6, atol=1e-7)
+    assert torch.autograd.gradcheck(virial, (r, d), eps=1e-6, atol=1e-7)
+    assert torch.autograd.gradgradcheck(virial, (r, d), eps=1e-6, atol=1e-7)
