@@ -2,11 +2,13 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
 
-A step is one pass of the hot path over one synthetic structure resident in HBM:
-neighbour-list rebuild + NEP descriptors + per-species network + force / virial.  Prints one
-JSON line (metric: atom-steps/s) with a `roofline` object for the kernel that takes the most
-time and a `cpu_baseline` object (the reference's CPU code, or this repository's CPU
-restatement, timed on the host cores on a bounded sample of the same recipe).
+A step is one pass of the hot path over one batch of synthetic input resident in HBM.  The
+default workload is the configuration the headline target is quoted on (1,048,576-atom NEP
+molecular-dynamics step: neighbour-list rebuild + descriptors + per-species network + force /
+virial); the other workloads are the remaining benchmark configurations.  Prints one JSON
+line (metric: atom-steps/s) with a `roofline` object for the kernel that takes the most time
+and a `cpu_baseline` object (the reference's CPU code compiled into oracle/_ref when present,
+else this repository's CPU restatement) timed on the host cores on a bounded sample.
 """
 import argparse
 import ctypes
@@ -21,42 +23,140 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
-PEAK_FP32_TFLOPS = 157.3       # MI355X fp32 (vector and matrix share this figure)
-
-WORKLOADS = {
-    # BASELINE.json configs[4]: the configuration the headline target is quoted on
-    "nep_md_1048576": dict(reps=64, natoms=1048576),
-    # BASELINE.json configs[1] recipe is a random packing; this is the same model on the
-    # lattice recipe at 4096 atoms (a quick run)
-    "nep_md_4096": dict(reps=10, natoms=4000),
-    "nep_md_131072": dict(reps=32, natoms=131072),
-}
+PEAK_FP32_TFLOPS = 157.3       # MI355X fp32
+PEAK_FP64_TFLOPS = 78.6        # MI355X fp64
 
 
+# ------------------------------------------------------------------------------------------------
+# algorithmic work (FMA = 2 flops), per centre atom
+# ------------------------------------------------------------------------------------------------
 def nep_flops_per_atom(nr_mean, na_mean, K=8, n_r=6, n_a=4, D=22, H=50):
-    """Algorithmic flop count of the factored NEP E/F/V evaluation per centre atom (FMA = 2):
-    per radial neighbour 14 + c(K) + 4K n_r + 3 n_r, per angular neighbour
+    """Factored NEP E/F/V: per radial neighbour 14 + c(K) + 4K n_r + 3 n_r, per angular neighbour
     c(K) + 4K n_a + 210 + 480 n_a, per atom 144 n_a + 4 D H + 15 H, with c(K) = 14K + 24."""
     cK = 14 * K + 24
     return (nr_mean * (14 + cK + 4 * K * n_r + 3 * n_r) +
             na_mean * (cK + 4 * K * n_a + 210 + 48 * n_a + 432 * n_a) + 144 * n_a + 4 * D * H + 15 * H)
 
 
-def build_structure(reps):
+def mtp_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar):
+    """Linear-MTP E/F/V: per neighbour 8 + 8K + 30 + 4K nmus + 4 kmax + 29 n_basic, per atom
+    9 n_times + 4 n_scalar."""
+    return nn_mean * (8 + 8 * K + 30 + 4 * K * nmus + 4 * kmax + 29 * n_basic) + 9 * n_times + 4 * n_scalar
+
+
+def mtp_loss_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar):
+    """Training step (E/F/V + loss gradient): F_efv + per neighbour 2 (8K + 30 + 4 kmax + 4K nmus)
+    + 70 n_basic, per atom 24 n_times + 6 n_scalar."""
+    return (mtp_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar) +
+            nn_mean * (2 * (8 * K + 30 + 4 * kmax + 4 * K * nmus) + 70 * n_basic) + 24 * n_times + 6 * n_scalar)
+
+
+def profile_report(L):
+    from ai2pot_amd import _lib
+    buf = ctypes.create_string_buffer(1 << 16)
+    _lib.check(L.a2p_profile_report(buf, ctypes.c_size_t(len(buf))))
+    kernels = {}
+    for line in buf.value.decode().splitlines():
+        name, count, ms = line.split()
+        kernels[name] = dict(launches=int(count), total_ms=float(ms), avg_ms=float(ms) / int(count))
+    return kernels
+
+
+def timed(step, steps, warmup, L):
+    import torch
+    for k in range(warmup):
+        step(k)
+    torch.cuda.synchronize()
+    L.a2p_profile_enable(1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(warmup + k)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kernels = profile_report(L)
+    L.a2p_profile_enable(0)
+    return t1 - t0, kernels
+
+
+def roofline_of(kernels, work):
+    """work: {label: (bound, amount per launch, unit, peak, scale, engine)}; picks the label with
+    the largest total time."""
+    cands = [k for k in kernels if k in work]
+    if not cands:
+        return None
+    dom = max(cands, key=lambda k: kernels[k]["total_ms"])
+    bound, amount, unit, peak, scale, engine = work[dom]
+    achieved = amount / (kernels[dom]["avg_ms"] * 1e-3) / scale
+    return dict(kernel=dom, bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
+                traffic=None, avg_ms=kernels[dom]["avg_ms"], engine=engine)
+
+
+# ------------------------------------------------------------------------------------------------
+# NEP molecular-dynamics step (configurations 2 and 5)
+# ------------------------------------------------------------------------------------------------
+def nep_structure(kind, n_or_reps):
     from ai2pot_amd import synth
-    a = 316.7 / 64.0                      # 0.033 atoms / A^3
-    lattice, pos = synth.fcc_cell(reps, a, 0.15, 1006)
-    types = synth.rng_randint(2006, pos.shape[0], 3)
+    if kind == "fcc":
+        a = 316.7 / 64.0                      # 0.033 atoms / A^3
+        lattice, pos = synth.fcc_cell(n_or_reps, a, 0.15, 1006)
+        seed = 2006
+    else:                                     # configuration 2: random packing, d_min 2.2
+        L = (n_or_reps / 0.033) ** (1.0 / 3.0)
+        lattice, pos = synth.random_packed(n_or_reps, [L, L, L], 2.2, 1003)
+        seed = 2003
+    types = synth.rng_randint(seed, pos.shape[0], 3)
     disp = synth.rng_normal(5006, pos.size, 0.0, 0.01).reshape(-1, 3)
     return lattice, pos, types, disp
 
 
-def cpu_baseline(sample_reps=32, repeats=2):
-    """Reference CPU path (oracle/_ref when built, else the restatement) on a 131072-atom
-    sample of the same recipe: single-threaded neighbour list + OpenMP E/F/V."""
+def run_nep_md(args, kind, size, rebuild=True):
+    import torch
+    from ai2pot_amd import _lib, synth
+    from ai2pot_amd.calculator import NepCalculator
+    dev = torch.device("cuda:0")
+    lattice, pos, types, disp = nep_structure(kind, size)
+    n = pos.shape[0]
+    model = synth.nep_model(seed=3006)
+    calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev)
+    coords0 = torch.from_numpy(pos.astype(np.float32)).to(dev)
+    disp_t = torch.from_numpy(disp.astype(np.float32)).to(dev)
+    coords = torch.empty_like(coords0)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    calc.rebuild(coords0, stream)
+
+    def step(k):
+        if rebuild:     # a small deterministic displacement: every step builds a different list
+            torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
+            return calc.step(coords)
+        calc.evaluate(stream)
+
+    L = _lib.lib()
+    elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    calc.check()
+    if not np.isfinite(float(calc.etot.item())):
+        sys.exit("bench.py: non-finite energy")
+    nn_r = float(calc.numneigh.float().mean().item())
+    r = calc.rcs.norm(dim=2)
+    nn_a = float(((r > 0) & (r <= model["rmax_angular"])).sum().item()) / n
+    s, U = 4, 200
+    work = {
+        "nep_efv_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
+        "nbl_lists": ("hbm", ((3 * s + 4) + 12 + U * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
+        "reduce_fill": ("hbm", (nn_r * (3 * s + 4) + nn_r * 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
+    }
+    config = {"workload": args.workload, "natoms": n, "species": 3,
+              "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 7.0, "rcut_angular": 4.0,
+              "umax": 200, "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
+              "per_step": ("neighbor rebuild + " if rebuild else "") + "descriptors + ANN + force/virial"}
+    return n, elapsed, kernels, roofline_of(kernels, work), config, "f32"
+
+
+def cpu_baseline_nep(sample_reps=32, repeats=2):
+    """131072-atom sample of the same recipe: single-threaded list + OpenMP E/F/V, as the reference."""
     import oracle
     from ai2pot_amd import synth
-    lattice, pos, types, _ = build_structure(sample_reps)
+    lattice, pos, types, _ = nep_structure("fcc", sample_reps)
     m = synth.nep_model(seed=3006)
     use_ref = oracle.ref_available("nep") and oracle.ref_available("nblist")
     nbl = oracle.ref_nblist if use_ref else oracle.nblist
@@ -66,15 +166,141 @@ def cpu_baseline(sample_reps=32, repeats=2):
     for _ in range(repeats):
         t0 = time.time()
         out = nbl(lattice.astype(np.float32), types, pos.astype(np.float32), 7.0, 200)
-        nb = synth.pack_batch([out])
-        efv(m, nb, np.float32)
+        efv(m, synth.pack_batch([out]), np.float32)
         dt = time.time() - t0
         best = dt if best is None else min(best, dt)
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return dict(value=n / best, unit="atom-steps/s", cores=threads,
-                kind="reference" if use_ref else "port",
-                sample="%d atoms (FCC %d^3 x 4, same recipe), list rebuild (1 thread) + NEP E/F/V "
-                       "(OpenMP, %d threads), best of %d" % (n, sample_reps, threads, repeats))
+    return dict(value=n / best, unit="atom-steps/s", cores=threads, kind="reference" if use_ref else "port",
+                sample="%d atoms (FCC %d^3 x 4, same recipe), list rebuild (1 thread) + NEP E/F/V (OpenMP, "
+                       "%d threads), best of %d" % (n, sample_reps, threads, repeats))
+
+
+# ------------------------------------------------------------------------------------------------
+# linear MTP (configurations 1, 3, 4)
+# ------------------------------------------------------------------------------------------------
+def mtp_setup(cfg):
+    """Structures, lists (built on the GPU once, outside the timed region) and model of a config."""
+    import torch
+    from ai2pot_amd import mtp_param, nblist, synth
+    dev = torch.device("cuda:0")
+    if cfg == 1:
+        lat, pos = synth.diamond_cell()
+        structs = [(lat, pos, np.zeros(216, np.int32))]
+        level, nt, K, rmax, rmin, lohi, seed = 10, 1, 8, 5.0, 0.5, (-0.1, 0.1), 3001
+    elif cfg == 3:
+        lat, pos = synth.random_packed(8192, [64.0, 51.2, 50.0], 2.0, 1004)
+        structs = [(lat, pos, synth.rng_randint(2004, 8192, 4))]
+        level, nt, K, rmax, rmin, lohi, seed = 20, 4, 10, 5.5, 1.8, (-0.05, 0.05), 3004
+    else:
+        rho = synth.rng_uniform(1005, 64, 0.03, 0.05)
+        structs = []
+        for b in range(64):
+            Lb = (128.0 / rho[b]) ** (1.0 / 3.0)
+            lat, pos = synth.random_packed(128, [Lb, Lb, Lb], 2.0, 11005 + b)
+            structs.append((lat, pos, synth.rng_randint(21005 + b, 128, 3)))
+        level, nt, K, rmax, rmin, lohi, seed = 16, 3, 8, 5.0, 0.0, None, 3005
+    tables = mtp_param.mtp_param(level)
+    if lohi is not None:
+        m = synth.mtp_model(tables, nt, K, rmax, rmin, seed, lo=lohi[0], hi=lohi[1])
+    else:   # the distributions of the reference's LinearMtp.__init__ (linear_mtp.py:74-88)
+        m = synth.mtp_model(tables, nt, K, rmax, rmin, seed)
+        S = m["linear_coeffs"].size
+        m["coeffs"] = synth.rng_normal(seed, m["coeffs"].size, 0, 0.1) + synth.rng_uniform(seed + 7, m["coeffs"].size)
+        m["linear_coeffs"] = synth.rng_normal(seed + 1, S, 0, np.sqrt(2.0 / (S + 1)))
+        m["type_bias"] = synth.rng_normal(seed + 2, nt, 0, 1.0)
+    lists = []
+    for lat, pos, ty in structs:
+        out = nblist.find_info4mlff_device(lat, torch.from_numpy(ty).to(dev), torch.from_numpy(pos).to(dev), rmax, 200)
+        lists.append(tuple(o.cpu().numpy() if hasattr(o, "cpu") else o for o in out))
+    nb = synth.pack_batch(lists)
+    return m, nb, tables
+
+
+def run_mtp(args, cfg):
+    import torch
+    from ai2pot_amd import _lib, ops, synth
+    dev = torch.device("cuda:0")
+    m, nb, tables = mtp_setup(cfg)
+    f64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64)).to(dev)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(dev)
+    md = {k: f64(m[k]) for k in ("coeffs", "linear_coeffs", "type_bias", "q_scaler")}
+    tb = {k: i32(m[k]) for k in ("alpha_index_basic", "alpha_index_times", "alpha_moment_mapping", "type_map")}
+    d = {k: i32(nb[k]) for k in ("binum", "bilist", "bnumneigh", "bfirstneigh", "btypes")}
+    d["brcs"] = f64(nb["brcs"])
+    B, P = nb["bilist"].shape
+    natoms = int(nb["binum"].sum())
+    nn = float(nb["bnumneigh"].sum()) / natoms
+    common = (m["chebyshev_size"], 1.0, md["coeffs"], md["linear_coeffs"], md["type_bias"],
+              m["alpha_moments_count"], tb["alpha_index_basic"], tb["alpha_index_times"], tb["alpha_moment_mapping"],
+              m["nmus"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"],
+              tb["type_map"], 0, m["rmax"], m["rmin"], md["q_scaler"])
+    kmax = int(tables["alpha_index_basic"][:, 1:].sum(1).max())
+    sizes = (m["chebyshev_size"], m["nmus"], kmax, tables["alpha_index_basic"].shape[0],
+             tables["alpha_index_times"].shape[0], tables["alpha_moment_mapping"].size)
+    if cfg == 4:
+        lab = (f64(synth.rng_normal(4005, B * P, -4.0, 0.2).reshape(B, P).sum(1)),
+               f64(synth.rng_normal(4006, B * P * 3, 0.0, 1.0).reshape(B, P, 3)),
+               f64(synth.rng_normal(4007, B * 9, 0.0, 0.5).reshape(B, 9)))
+        out = {}
+
+        def step(k):    # forward + analytic backward w.r.t. all parameters, as one training step
+            out["r"] = ops.mtp_loss_step(1.0, 1.0, 1.0, lab[0], lab[1], lab[2], *common, want_grad=True,
+                                         validate=False)
+        flops = mtp_loss_flops_per_atom(nn, *sizes) * natoms
+        label = "mtp_loss_bwd_kernel"
+    else:
+        def step(k):
+            ops.linearMtpToEFVOp(*common, 0.0, 0.0, None, None, validate=False)
+        flops = mtp_flops_per_atom(nn, *sizes) * natoms
+        label = "mtp_efv_kernel"
+    L = _lib.lib()
+    elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
+    work = {label: ("mfma", flops if cfg != 4 else flops - mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s",
+                    PEAK_FP64_TFLOPS, 1e12, "valu_fp64"),
+            "mtp_efv_kernel": ("mfma", mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s", PEAK_FP64_TFLOPS, 1e12,
+                               "valu_fp64")}
+    config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P,
+              "model": "linear MTP level %d K=%d" % ({1: 10, 3: 20, 4: 16}[cfg], m["chebyshev_size"]),
+              "species": int(m["type_map"].size), "rmax": m["rmax"], "rmin": m["rmin"], "mean_neighbors": nn,
+              "per_step": "loss forward + analytic gradient w.r.t. coeffs/linear/bias" if cfg == 4 else
+                          "energy + force + virial (list built once, outside the timed region)"}
+    return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f64"
+
+
+def cpu_baseline_mtp(cfg):
+    import oracle
+    from ai2pot_amd import synth
+    m, nb, _ = mtp_setup(cfg)
+    use_ref = oracle.ref_available("mtpr")
+    natoms = int(nb["binum"].sum())
+    t0 = time.time()
+    if cfg == 4:
+        if not use_ref:
+            raise RuntimeError("the restatement's forward-mode gradient is too slow to serve as a baseline")
+        B, P = nb["bilist"].shape
+        lab = dict(energy=synth.rng_normal(4005, B * P, -4.0, 0.2).reshape(B, P).sum(1),
+                   force=synth.rng_normal(4006, B * P * 3, 0.0, 1.0).reshape(B, P, 3),
+                   virial=synth.rng_normal(4007, B * 9, 0.0, 0.5).reshape(B, 9))
+        oracle.ref_mtp_loss_step(m, nb, (1.0, 1.0, 1.0), lab)
+        what = "loss forward + backward (the reference's backward recomputes E/F/V once more; not included)"
+    else:
+        (oracle.ref_mtp_efv if use_ref else oracle.mtp_efv)(m, nb)
+        what = "E/F/V"
+    dt = time.time() - t0
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return dict(value=natoms / dt, unit="atom-steps/s", cores=threads, kind="reference" if use_ref else "port",
+                sample="the full workload (%d atoms), %s, OpenMP %d threads, one run" % (natoms, what, threads))
+
+
+WORKLOADS = {
+    "nep_md_1048576": lambda a: run_nep_md(a, "fcc", 64),         # BASELINE.json configs[4] (headline)
+    "nep_md_131072": lambda a: run_nep_md(a, "fcc", 32),
+    "nep_efv_4096": lambda a: run_nep_md(a, "random", 4096, rebuild=False),   # configs[1]
+    "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]
+    "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
+    "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]
+}
 
 
 def main():
@@ -88,95 +314,27 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
                  "(no collectives or sharding in this round)" % args.gpus)
-
     import torch
-    from ai2pot_amd import _lib, synth
-    from ai2pot_amd.calculator import NepCalculator
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
+    torch.cuda.set_device(0)
 
-    wl = WORKLOADS[args.workload]
-    lattice, pos, types, disp = build_structure(wl["reps"])
-    n = pos.shape[0]
-    model = synth.nep_model(seed=3006)
-    calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev)
-    coords0 = torch.from_numpy(pos.astype(np.float32)).to(dev)
-    disp_t = torch.from_numpy(disp.astype(np.float32)).to(dev)
-    coords = torch.empty_like(coords0)
-
-    def step(k):
-        # a small deterministic displacement, so that every step rebuilds a different list
-        torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
-        return calc.step(coords)
-
-    L = _lib.lib()
-    for k in range(args.warmup):
-        step(k)
-    torch.cuda.synchronize()
-    calc.check()
-    nn_r = float(calc.numneigh.float().mean().item())
-    r = calc.rcs.norm(dim=2)
-    nn_a = float(((r > 0) & (r <= model["rmax_angular"])).sum().item()) / n
-    del r
-
-    L.a2p_profile_enable(1)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        step(args.warmup + k)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    buf = ctypes.create_string_buffer(1 << 16)
-    _lib.check(L.a2p_profile_report(buf, ctypes.c_size_t(len(buf))))
-    L.a2p_profile_enable(0)
-    calc.check()
-    e = float(calc.etot.item())
-    if not np.isfinite(e):
-        sys.exit("bench.py: non-finite energy")
-
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = n * args.steps / (t1 - t0)
-
-    kernels = {}
-    for line in buf.value.decode().splitlines():
-        name, count, ms = line.split()
-        kernels[name] = dict(launches=int(count), total_ms=float(ms), avg_ms=float(ms) / int(count))
-    # algorithmic work per launch of the candidates for "dominant kernel"
-    s = 4
-    U = 200
-    work = {
-        "nep_efv_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12),
-        "nbl_lists": ("hbm", ((3 * s + 4) + 12 + U * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9),
-        "reduce_fill": ("hbm", (nn_r * (3 * s + 4) + nn_r * 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9),
-        "reduce_sum": ("hbm", (nn_r * 3 * s + 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9),
-    }
-    dominant = max(kernels, key=lambda k: kernels[k]["total_ms"]) if kernels else None
-    roofline = None
-    if dominant in work:
-        bound, amount, unit, peak, scale = work[dominant]
-        achieved = amount / (kernels[dominant]["avg_ms"] * 1e-3) / scale
-        roofline = dict(kernel=dominant, bound=bound, achieved=achieved, peak=peak, unit=unit,
-                        frac=achieved / peak, traffic=None,
-                        avg_ms=kernels[dominant]["avg_ms"],
-                        engine="valu_fp32" if bound == "mfma" else "hbm")
+    n, elapsed, kernels, roofline, config, dtype = WORKLOADS[args.workload](args)
+    ms_per_step = elapsed * 1e3 / args.steps
     out = {
-        "metric": "atom-steps/s (E+F+virial) on 1 MI355X", "value": value, "unit": "atom-steps/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "us_per_atom_step": ms_per_step * 1e3 / n,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": args.workload, "natoms": n, "species": 3, "model": "NEP radial+3-body "
-                   "K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 7.0, "rcut_angular": 4.0, "umax": 200,
-                   "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
-                   "per_step": "neighbor rebuild + descriptors + ANN + force/virial"},
-        "roofline": roofline,
-        "kernels": kernels,
+        "metric": "atom-steps/s (E+F+virial) on 1 MI355X", "value": n * args.steps / elapsed,
+        "unit": "atom-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "us_per_atom_step": ms_per_step * 1e3 / n, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": config,
+        "roofline": roofline, "kernels": kernels,
     }
     if not args.no_cpu_baseline:
         try:
-            out["cpu_baseline"] = cpu_baseline()
+            if args.workload.startswith("nep"):
+                out["cpu_baseline"] = cpu_baseline_nep()
+            else:
+                out["cpu_baseline"] = cpu_baseline_mtp({"mtp10_efv_216": 1, "mtp20_efv_8192": 3,
+                                                        "mtp16_train_64x128": 4}[args.workload])
         except Exception as ex:       # the baseline is a report, never a reason to lose the GPU line
             out["cpu_baseline"] = {"error": repr(ex)}
     print(json.dumps(out))
