@@ -123,6 +123,25 @@ template <typename T>
 int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
                 const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
 
+// The same reduction for a producer that stores each pair derivative straight into its
+// target's segment, without the intermediate [row, slot, 3] array:
+//   pair_csr_begin   counts the incoming pairs per target and scans them into segment offsets;
+//   the producer     claims a place with  pos = offsets[t] + atomicAdd(&cursor[t], 1)  and
+//                    stores seg_g[pos*3 .. pos*3+2] (it may skip pairs whose derivative is zero);
+//   pair_csr_finish  sums the filled part of every segment onto `force` as above.
+struct PairCsr {
+    int* counts;
+    int* offsets;
+    int* cursor;
+    void* seg_g;
+    int n;          // B * (P + nghost) targets
+};
+template <typename T>
+int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* binum,
+                   const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
+template <typename T>
+int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);
+
 // out[b*out_stride + c] = sum over blocks of partial[(b*nblocks + block)*src_stride + c], c < ncomp,
 // with a fixed summation tree (fp64).
 template <typename T>

@@ -504,6 +504,450 @@ nep_efv_kernel(const NepArgs<T> a)
     }
 }
 
+// ---- staged kernel for the common model shape (K=8, n_r=6, n_a=4, l_max=4, <= 4 species) ----
+// The generic kernel above lets every thread walk its own neighbour row, so each wave-wide
+// load touches 64 different cache lines.  Here the workgroup stages FCH slots of its FB rows
+// through LDS per round with row-contiguous loads (FCH lanes per row), the neighbour's species
+// is gathered by the loading lane and packed next to its index, and every thread then reads its
+// own FCH entries from LDS without bank conflicts.  Two passes over the rounds:
+//   pass 1: per-species sums of the radial functions (contracted with the coefficients once
+//           per atom afterwards) and the angular moments of the neighbours inside the angular
+//           cutoff; hidden layer, dE/dq, dE/dS
+//   pass 2: pair derivatives (radial and angular part of a pair together), stored straight
+//           into the target atom's reduction segment (a2p::PairCsr), own force, virial.
+// Inside a round a thread first processes the entries within the angular cutoff, then the
+// radial-only ones, each as a compacted bit-mask loop, so lanes of a wave work on the same kind
+// of entry.
+constexpr int FB = 256;        // atoms (threads) per workgroup
+constexpr int FCH = 8;         // neighbour slots staged per round
+constexpr int FLS = FB + 8;    // padded row length of the staging arrays
+constexpr int FDP = 24;        // padded descriptor count (22)
+
+__device__ __forceinline__ void lds_load4(const float* p, float (&o)[4])
+{
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void lds_load4(const double* p, double (&o)[4])
+{
+    const double2 v0 = *reinterpret_cast<const double2*>(p);
+    const double2 v1 = *reinterpret_cast<const double2*>(p + 2);
+    o[0] = v0.x; o[1] = v0.y; o[2] = v1.x; o[3] = v1.y;
+}
+
+template <typename T>
+struct StagedLds {
+    T *w0, *coef, *b0, *w1, *qs, *acc, *x, *y, *z;
+    int *w, *nn, *red;
+};
+
+__host__ __device__ __forceinline__ size_t lds_round16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
+
+// LDS layout of the staged kernel; 16-byte aligned vector rows first.  Returns the total size.
+template <typename T>
+__host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
+                                                             StagedLds<T>& L)
+{
+    size_t off = 0;
+    L.w0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * FDP * sizeof(T));
+    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * 10 * 8 * sizeof(T));
+    L.b0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
+    L.w1 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
+    L.qs = (T*)(base + off);   off += lds_round16((size_t)FDP * sizeof(T));
+    L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * 8 * FB * sizeof(T));
+    L.x = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.y = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.z = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.w = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
+    L.nn = (int*)(base + off); off += lds_round16((size_t)FB * sizeof(int));
+    L.red = (int*)(base + off); off += lds_round16((size_t)(FB / 64) * 10 * sizeof(double));
+    return off;
+}
+
+// Stage slots [c0, c0 + FCH) of the workgroup's rows: thread e handles row e / FCH, slot e % FCH,
+// so FCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
+// row's end (or with an index out of range) are stored far outside every cutoff.
+template <typename T>
+__device__ __forceinline__ void staged_load(const NepArgs<T>& a, const StagedLds<T>& L, int tid, int c0,
+                                            size_t rowbase, const int* __restrict__ types, int NF)
+{
+#pragma unroll
+    for (int it = 0; it < FCH; it++) {
+        const int e = it * FB + tid;
+        const int la = e / FCH, s = e % FCH;
+        const int slot = c0 + s;
+        T x = (T)1.0e18, y = (T)0, z = (T)0;
+        int w = 0;
+        if (slot < L.nn[la]) {
+            const size_t pr = (rowbase + la) * a.U + slot;
+            const T* p = a.brcs + pr * 3;
+            const int nj = a.bfirstneigh[pr];
+            if ((unsigned)nj >= (unsigned)NF) {
+                atomicOr(a.status, ST_BAD_NEIGHBOR);
+            } else {
+                x = p[0]; y = p[1]; z = p[2];
+                int tj = types[nj];
+                if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
+                w = nj | (tj << 28);
+            }
+        }
+        L.x[s * FLS + la] = x; L.y[s * FLS + la] = y; L.z[s * FLS + la] = z; L.w[s * FLS + la] = w;
+    }
+}
+
+// Bit masks of a thread's staged entries: bits 0..FCH-1 inside the angular cutoff, bits
+// 16..16+FCH-1 radial only.
+template <typename T>
+__device__ __forceinline__ unsigned staged_classify(const StagedLds<T>& L, int tid, T rr, T ra)
+{
+    unsigned m = 0;
+#pragma unroll
+    for (int s = 0; s < FCH; s++) {
+        const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+        const T r = sqrt_t(x * x + y * y + z * z);
+        if (r <= ra) m |= 1u << s;
+        else if (r <= rr) m |= 0x10000u << s;
+    }
+    return m;
+}
+
+template <typename T, int NTC>
+__global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
+nep_staged_kernel(const NepArgs<T> a, const int* __restrict__ seg_offsets, int* __restrict__ seg_cursor,
+                  T* __restrict__ seg_g)
+{
+    constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int tid = threadIdx.x;
+    const int b = blockIdx.y;
+    const int ii = blockIdx.x * FB + tid;
+    const int H = a.H, nt = a.ntypes;
+    const int NF = a.P + a.nghost;
+    StagedLds<T> L;
+    staged_lds_layout<T>(nt, H, NTC, smem_raw, L);
+
+    // ---- model tables ------------------------------------------------------------------------
+    for (int i = tid; i < nt * H * FDP; i += FB) {
+        const int r = i / FDP, j = i - r * FDP;
+        L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
+    }
+    for (int i = tid; i < nt * nt * NB * KC; i += FB) L.coef[i] = a.coeffs[i];
+    for (int i = tid; i < nt * H; i += FB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
+    if (tid < FDP) L.qs[tid] = tid < DC ? (T)1 / a.q_scaler[tid] : (T)0;
+#pragma unroll
+    for (int i = 0; i < NTC * KC; i++) L.acc[i * FB + tid] = (T)0;
+
+    const int inum = a.binum[b];
+    const bool active = ii < inum;
+    const size_t rowbase = (size_t)b * a.P + (size_t)blockIdx.x * FB;
+    const size_t row = rowbase + tid;
+    int center = 0, ti = 0, nn = 0;
+    if (active) {
+        center = a.bilist[row];
+        nn = a.bnumneigh[row];
+        if (nn > a.U) { atomicOr(a.status, ST_NEIGH_OVERFLOW); nn = a.U; }
+        if ((unsigned)center >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); center = 0; nn = 0; }
+        ti = a.btypes[(size_t)b * NF + center];
+        if ((unsigned)ti >= (unsigned)nt) { atomicOr(a.status, ST_BAD_TYPE); ti = 0; nn = 0; }
+    }
+    L.nn[tid] = nn;
+    {
+        int m = nn;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+        if ((tid & 63) == 0) L.red[tid >> 6] = m;
+    }
+    __syncthreads();
+    int maxnn = 0;
+#pragma unroll
+    for (int w = 0; w < FB / 64; w++) maxnn = max(maxnn, L.red[w]);
+
+    const int* types = a.btypes + (size_t)b * NF;
+    const T rr = a.rr, ra = a.ra;
+    const T rr_inv = (T)1 / rr, ra_inv = (T)1 / ra;
+
+    T S[NAC][NLM];
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
+
+    // ---- pass 1 -------------------------------------------------------------------------------
+    for (int c0 = 0; c0 < maxnn; c0 += FCH) {
+        __syncthreads();
+        staged_load<T>(a, L, tid, c0, rowbase, types, NF);
+        __syncthreads();
+        const unsigned cls = staged_classify<T>(L, tid, rr, ra);
+        unsigned am = cls & 0xffffu, rm = cls >> 16;
+        while (am) {
+            const int s = __ffs(am) - 1;
+            am &= am - 1;
+            const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+            const int tj = L.w[s * FLS + tid] >> 28;
+            const T r = sqrt_t(x * x + y * y + z * z);
+            const T rinv = (T)1 / r;
+            T f[KC], df[KC];
+            if (r <= rr) {
+                radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+                for (int k = 0; k < KC; k++) L.acc[(tj * KC + k) * FB + tid] += f[k];
+            }
+            radial_basis<T, KC, false>(r, ra_inv, KC, f, df);
+            const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
+            T bl[NLM];
+            blm_values<T, LC>(x * rinv, y * rinv, z * rinv, bl);
+#pragma unroll
+            for (int n = 0; n < NAC; n++) {
+                T c0v[4], c1v[4];
+                lds_load4(c + n * KC, c0v);
+                lds_load4(c + n * KC + 4, c1v);
+                T g = (T)0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) g += c0v[k] * f[k];
+#pragma unroll
+                for (int k = 0; k < 4; k++) g += c1v[k] * f[4 + k];
+#pragma unroll
+                for (int m = 0; m < NLM; m++) S[n][m] += g * bl[m];
+            }
+        }
+        while (rm) {
+            const int s = __ffs(rm) - 1;
+            rm &= rm - 1;
+            const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+            const int tj = L.w[s * FLS + tid] >> 28;
+            const T r = sqrt_t(x * x + y * y + z * z);
+            T f[KC], df[KC];
+            radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+            for (int k = 0; k < KC; k++) L.acc[(tj * KC + k) * FB + tid] += f[k];
+        }
+    }
+
+    // ---- descriptors --------------------------------------------------------------------------
+    T q[DC];
+#pragma unroll
+    for (int j = 0; j < DC; j++) q[j] = (T)0;
+    for (int t = 0; t < nt; t++) {
+        const T* c = L.coef + (ti * nt + t) * NB * KC;
+        T fs[KC];
+#pragma unroll
+        for (int k = 0; k < KC; k++) fs[k] = L.acc[(t * KC + k) * FB + tid];
+#pragma unroll
+        for (int n = 0; n < NRC; n++) {
+            T c0v[4], c1v[4];
+            lds_load4(c + n * KC, c0v);
+            lds_load4(c + n * KC + 4, c1v);
+#pragma unroll
+            for (int k = 0; k < 4; k++) q[n] += c0v[k] * fs[k];
+#pragma unroll
+            for (int k = 0; k < 4; k++) q[n] += c1v[k] * fs[4 + k];
+        }
+    }
+    // q_{n,l} = sum_m w_m C_lm S^2  (nepBasis.h:174-190)
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int l = 1; l <= LC; l++) {
+            T acc = (T)0;
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                acc += (T)(mp == 0 ? 1.0 : 2.0) * (T)kC3B[m] * S[n][m] * S[n][m];
+            }
+            q[NRC + n * LC + (l - 1)] = acc;
+        }
+    if (active && a.desc) {
+        T* dst = a.desc + row * DC;
+#pragma unroll
+        for (int j = 0; j < DC; j++) dst[j] = q[j];
+    }
+
+    // ---- hidden layer (nep.h:415-447) ----------------------------------------------------------
+    T dEdq[DC];
+    T e_site = active ? a.bias[ti] : (T)0;
+    {
+        T qn[DC];
+#pragma unroll
+        for (int j = 0; j < DC; j++) { qn[j] = q[j] * L.qs[j]; dEdq[j] = (T)0; }
+        for (int p = 0; p < H; p++) {
+            const T* wrow = L.w0 + (size_t)(ti * H + p) * FDP;
+            T wv[FDP];
+#pragma unroll
+            for (int j = 0; j < FDP; j += 4) {
+                T v[4];
+                lds_load4(wrow + j, v);
+                wv[j] = v[0]; wv[j + 1] = v[1]; wv[j + 2] = v[2]; wv[j + 3] = v[3];
+            }
+            T h = L.b0[ti * H + p];
+#pragma unroll
+            for (int j = 0; j < DC; j++) h += wv[j] * qn[j];
+            const T t = tanh_t(h);
+            const T w1p = L.w1[ti * H + p];
+            e_site += w1p * t;
+            const T sde = w1p * ((T)1 - t * t);
+#pragma unroll
+            for (int j = 0; j < DC; j++) dEdq[j] += sde * wv[j];
+        }
+#pragma unroll
+        for (int j = 0; j < DC; j++) dEdq[j] *= L.qs[j];
+    }
+    // dE/dS (nep.h:450-466), overwriting S
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int l = 1; l <= LC; l++)
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                S[n][m] *= dEdq[NRC + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+            }
+
+    // ---- pass 2: pair derivatives ---------------------------------------------------------------
+    T fx = (T)0, fy = (T)0, fz = (T)0;
+    T vir[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vir[i] = (T)0;
+    if (a.force != nullptr || a.want_virial) {
+        // radial coefficients contracted with dE/dq, per neighbour species (thread-private cells)
+        for (int t = 0; t < nt; t++) {
+            const T* c = L.coef + (ti * nt + t) * NB * KC;
+            T cc[KC];
+#pragma unroll
+            for (int k = 0; k < KC; k++) cc[k] = (T)0;
+#pragma unroll
+            for (int n = 0; n < NRC; n++) {
+                T c0v[4], c1v[4];
+                lds_load4(c + n * KC, c0v);
+                lds_load4(c + n * KC + 4, c1v);
+#pragma unroll
+                for (int k = 0; k < 4; k++) { cc[k] += dEdq[n] * c0v[k]; cc[4 + k] += dEdq[n] * c1v[k]; }
+            }
+#pragma unroll
+            for (int k = 0; k < KC; k++) L.acc[(t * KC + k) * FB + tid] = cc[k];
+        }
+        const size_t tbase = (size_t)b * NF;
+        auto emit = [&](int w, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
+            if (seg_g) {
+                const size_t t = tbase + (size_t)(w & 0x0fffffff);
+                const int pos = seg_offsets[t] + atomicAdd(&seg_cursor[t], 1);
+                T* dst = seg_g + (size_t)pos * 3;
+                dst[0] = gx; dst[1] = gy; dst[2] = gz;
+            }
+            fx += gx; fy += gy; fz += gz;
+            vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
+            vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
+            vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
+        };
+        for (int c0 = 0; c0 < maxnn; c0 += FCH) {
+            __syncthreads();
+            staged_load<T>(a, L, tid, c0, rowbase, types, NF);
+            __syncthreads();
+            const unsigned cls = staged_classify<T>(L, tid, rr, ra);
+            unsigned am = cls & 0xffffu, rm = cls >> 16;
+            while (am) {
+                const int s = __ffs(am) - 1;
+                am &= am - 1;
+                const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+                const int w = L.w[s * FLS + tid];
+                const int tj = w >> 28;
+                const T r = sqrt_t(x * x + y * y + z * z);
+                const T rinv = (T)1 / r;
+                const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+                T f[KC], df[KC];
+                T srad = (T)0;
+                if (r <= rr) {
+                    radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+#pragma unroll
+                    for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * FB + tid] * df[k];
+                }
+                radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+                const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
+                T A[NLM], Ad[NLM];
+#pragma unroll
+                for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
+#pragma unroll
+                for (int n = 0; n < NAC; n++) {
+                    T c0v[4], c1v[4];
+                    lds_load4(c + n * KC, c0v);
+                    lds_load4(c + n * KC + 4, c1v);
+                    T g = (T)0, dg = (T)0;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
+#pragma unroll
+                    for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
+                }
+                T bl[NLM];
+                blm_values<T, LC>(ux, uy, uz, bl);
+#pragma unroll
+                for (int l = 1; l <= LC; l++)
+#pragma unroll
+                    for (int mp = 0; mp < 2 * l + 1; mp++) {
+                        const int m = l * l - 1 + mp;
+                        srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+                    }
+                T wx = (T)0, wy = (T)0, wz = (T)0;
+                blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
+                emit(w, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
+            }
+            while (rm) {
+                const int s = __ffs(rm) - 1;
+                rm &= rm - 1;
+                const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+                const int w = L.w[s * FLS + tid];
+                const int tj = w >> 28;
+                const T r = sqrt_t(x * x + y * y + z * z);
+                T f[KC], df[KC];
+                radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+                T sr = (T)0;
+#pragma unroll
+                for (int k = 0; k < KC; k++) sr += L.acc[(tj * KC + k) * FB + tid] * df[k];
+                sr /= r;
+                emit(w, x, y, z, sr * x, sr * y, sr * z);
+            }
+        }
+        if (active && a.force) {
+            T* fo = a.force + ((size_t)b * NF + center) * 3;
+            fo[0] = fx; fo[1] = fy; fo[2] = fz;
+        }
+    }
+
+    // ---- workgroup partial sums of energy and virial (fp64) ---------------------------------
+    __syncthreads();
+    double* s_red = (double*)L.red;
+    double vals[10];
+    vals[0] = active ? (double)e_site : 0.0;
+#pragma unroll
+    for (int i = 0; i < 9; i++) vals[1 + i] = active ? (double)vir[i] : 0.0;
+#pragma unroll
+    for (int i = 0; i < 10; i++) {
+        double v = wave_sum(vals[i]);
+        if ((tid & 63) == 0) s_red[(tid >> 6) * 10 + i] = v;
+    }
+    __syncthreads();
+    if (tid < 10) {
+        double v = 0.0;
+        for (int w = 0; w < FB / 64; w++) v += s_red[w * 10 + tid];
+        a.partial[((size_t)b * a.nblocks + blockIdx.x) * 10 + tid] = v;
+    }
+}
+
+template <typename T, int NTC>
+int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
+{
+    auto kern = nep_staged_kernel<T, NTC>;
+    if (lds > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)lds));
+    prof_begin("nep_staged_kernel", stream);
+    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, (const int*)csr.offsets,
+                       csr.cursor, (T*)csr.seg_g);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 template <typename T>
 size_t nep_lds_bytes(const NepArgs<T>& a)
 {
@@ -566,6 +1010,15 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     A2P_REQUIRE(lds <= 150 * 1024, A2P_ERR_INVALID,
                 "nep: coefficient table (%zu bytes with neighbour masks) does not fit in LDS", lds);
 
+    // staged kernel: the common model shape with up to four species
+    const long long NF = (long long)P + nghost;
+    const int ntc = ntypes <= 1 ? 1 : ntypes == 2 ? 2 : ntypes == 3 ? 3 : 4;
+    StagedLds<T> lds_unused;
+    const size_t lds_staged = staged_lds_layout<T>(ntypes, H, ntc, nullptr, lds_unused);
+    const bool staged = K == 8 && n_r == 6 && n_a == 4 && l_max == 4 && ntypes <= 4 &&
+                        NF < (1ll << 28) && lds_staged <= 150 * 1024;
+    if (staged) a.nblocks = ceil_div(P, FB);
+
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
     if (rc) return rc;
@@ -576,34 +1029,52 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     a.pair_g = nullptr;
     a.force = force;
     const size_t force_bytes = (size_t)B * (P + nghost) * 3 * sizeof(T);
-    if (!force && virial) {         // the virial needs the pair derivatives: use a scratch force
-        rc = ws_get(WS_MISC, force_bytes, &ws);
-        if (rc) return rc;
-        a.force = (T*)ws;
-    }
-    if (a.force) {
-        rc = ws_get(WS_PAIR_G, (size_t)B * P * U * 3 * sizeof(T), &ws);
-        if (rc) return rc;
-        a.pair_g = (T*)ws;
-        rc = fill_zero(a.force, force_bytes, stream);
-        if (rc) return rc;
-    }
 
-    if (K == 8 && n_r == 6 && n_a == 4 && l_max == 4 && a.w_in_lds)
-        rc = launch<T, 8, 6, 4, 4, true>(a, lds, stream);
-    else if (K <= 8 && n_r <= 6 && n_a <= 4 && l_max <= 3)
-        rc = launch<T, 8, 6, 4, 3, false>(a, lds, stream);
-    else if (K <= 8 && n_r <= 6 && n_a <= 4)
-        rc = launch<T, 8, 6, 4, 4, false>(a, lds, stream);
-    else if (K <= 12 && n_r <= 8 && n_a <= 6)
-        rc = launch<T, 12, 8, 6, 4, false>(a, lds, stream);
-    else
-        rc = launch<T, 16, 12, 8, 4, false>(a, lds, stream);
-    if (rc) return rc;
-
-    if (force) {
-        rc = pair_reduce<T>(force, a.pair_g, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+    if (staged) {
+        PairCsr csr{};
+        if (force) {
+            rc = fill_zero(force, force_bytes, stream);
+            if (rc) return rc;
+            rc = pair_csr_begin<T>(&csr, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+            if (rc) return rc;
+        }
+        switch (ntc) {
+        case 1: rc = launch_staged<T, 1>(a, lds_staged, csr, stream); break;
+        case 2: rc = launch_staged<T, 2>(a, lds_staged, csr, stream); break;
+        case 3: rc = launch_staged<T, 3>(a, lds_staged, csr, stream); break;
+        default: rc = launch_staged<T, 4>(a, lds_staged, csr, stream); break;
+        }
         if (rc) return rc;
+        if (force) {
+            rc = pair_csr_finish<T>(force, csr, stream);
+            if (rc) return rc;
+        }
+    } else {
+        if (!force && virial) {     // the virial needs the pair derivatives: use a scratch force
+            rc = ws_get(WS_MISC, force_bytes, &ws);
+            if (rc) return rc;
+            a.force = (T*)ws;
+        }
+        if (a.force) {
+            rc = ws_get(WS_PAIR_G, (size_t)B * P * U * 3 * sizeof(T), &ws);
+            if (rc) return rc;
+            a.pair_g = (T*)ws;
+            rc = fill_zero(a.force, force_bytes, stream);
+            if (rc) return rc;
+        }
+        if (K <= 8 && n_r <= 6 && n_a <= 4 && l_max <= 3)
+            rc = launch<T, 8, 6, 4, 3, false>(a, lds, stream);
+        else if (K <= 8 && n_r <= 6 && n_a <= 4)
+            rc = launch<T, 8, 6, 4, 4, false>(a, lds, stream);
+        else if (K <= 12 && n_r <= 8 && n_a <= 6)
+            rc = launch<T, 12, 8, 6, 4, false>(a, lds, stream);
+        else
+            rc = launch<T, 16, 12, 8, 4, false>(a, lds, stream);
+        if (rc) return rc;
+        if (force) {
+            rc = pair_reduce<T>(force, a.pair_g, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+            if (rc) return rc;
+        }
     }
     if (etot) {
         rc = finish_partials<T>(etot, a.partial, B, a.nblocks, 1, 10, 1, stream);

@@ -220,8 +220,8 @@ int exclusive_scan_i32(const int* in, int* out, int n, int* tmp, hipStream_t str
 }
 
 template <typename T>
-int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
-                const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
+int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* binum,
+                   const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
 {
     const int NF = P + nghost;
     const long long NT = (long long)B * NF;
@@ -240,37 +240,59 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
     void* flags = nullptr;
     rc = ws_get(WS_FLAGS, 64, &flags);
     if (rc) return rc;
-    int* counts = (int*)ws;
-    int* offsets = counts + n;
-    int* cursor = offsets + n;
-    int* tiles = cursor + n;
-    T* seg_g = (T*)((char*)ws + bytes);
+    csr->n = n;
+    csr->counts = (int*)ws;
+    csr->offsets = csr->counts + n;
+    csr->cursor = csr->offsets + n;
+    int* tiles = csr->cursor + n;
+    csr->seg_g = (void*)((char*)ws + bytes);
 
-    // counts and cursor start at zero (offsets is fully overwritten)
-    rc = fill_zero(counts, (size_t)n * sizeof(int), stream);
+    // counts and cursor are adjacent and start at zero (offsets is fully overwritten)
+    rc = fill_zero(csr->counts, (size_t)n * sizeof(int), stream);
     if (rc) return rc;
-    rc = fill_zero(cursor, (size_t)n * sizeof(int), stream);
+    rc = fill_zero(csr->cursor, (size_t)n * sizeof(int), stream);
     if (rc) return rc;
 
     const int wave_blocks = ceil_div(rows * 64, 256);
     prof_begin("reduce_count", stream);
-    hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, counts, B, P, U, NF, binum,
-                       bnumneigh, bfirstneigh, (int*)flags);
+    hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, csr->counts, B, P, U, NF,
+                       binum, bnumneigh, bfirstneigh, (int*)flags);
     prof_end(stream);
-    rc = exclusive_scan_i32(counts, offsets, n, tiles, stream);
-    if (rc) return rc;
-    prof_begin("reduce_fill", stream);
-    hipLaunchKernelGGL(fill_kernel<T>, dim3(wave_blocks), dim3(256), 0, stream, seg_g, cursor, offsets,
-                       pair_g, B, P, U, NF, binum, bnumneigh, bfirstneigh);
-    prof_end(stream);
+    return exclusive_scan_i32(csr->counts, csr->offsets, n, tiles, stream);
+}
+
+template <typename T>
+int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream)
+{
+    // the cursor holds how many entries of each segment were filled
     prof_begin("reduce_sum", stream);
-    hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)n * 16, 256)), dim3(256), 0, stream,
-                       force, seg_g, offsets, counts, n);
+    hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)csr.n * 16, 256)), dim3(256), 0, stream,
+                       force, (const T*)csr.seg_g, csr.offsets, csr.cursor, csr.n);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
 
+template <typename T>
+int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
+                const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
+{
+    PairCsr csr;
+    int rc = pair_csr_begin<T>(&csr, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+    if (rc) return rc;
+    const long long rows = (long long)B * P;
+    const int wave_blocks = ceil_div(rows * 64, 256);
+    prof_begin("reduce_fill", stream);
+    hipLaunchKernelGGL(fill_kernel<T>, dim3(wave_blocks), dim3(256), 0, stream, (T*)csr.seg_g, csr.cursor,
+                       csr.offsets, pair_g, B, P, U, P + nghost, binum, bnumneigh, bfirstneigh);
+    prof_end(stream);
+    return pair_csr_finish<T>(force, csr, stream);
+}
+
+template int pair_csr_begin<float>(PairCsr*, int, int, int, int, const int*, const int*, const int*, hipStream_t);
+template int pair_csr_begin<double>(PairCsr*, int, int, int, int, const int*, const int*, const int*, hipStream_t);
+template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
+template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,
                                 const int*, hipStream_t);
 template int pair_reduce<double>(double*, const double*, int, int, int, int, const int*, const int*,
