@@ -126,18 +126,22 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 // The same reduction for a producer that stores each pair derivative straight into its
 // target's segment, without the intermediate [row, slot, 3] array:
 //   pair_csr_begin   counts the incoming pairs per target and scans them into segment offsets;
-//   the producer     claims a place with  pos = offsets[t] + atomicAdd(&cursor[t], 1)  and
-//                    stores seg_g[pos*3 .. pos*3+2] (it may skip pairs whose derivative is zero);
+//                    with_rank: every valid pair (row, slot) also gets rank[row*U + slot], its
+//                    place inside its target's segment (-1 for an index out of range);
+//   the producer     stores seg_g[pos*3 .. pos*3+2] at  pos = offsets[t] + rank[row*U + slot]
+//                    for EVERY valid pair (zeros where the derivative vanishes), or, without
+//                    ranks, claims  pos = offsets[t] + atomicAdd(&cursor[t], 1)  and may skip pairs;
 //   pair_csr_finish  sums the filled part of every segment onto `force` as above.
 struct PairCsr {
     int* counts;
     int* offsets;
     int* cursor;
+    int* rank;      // [B*P, U] or null
     void* seg_g;
     int n;          // B * (P + nghost) targets
 };
 template <typename T>
-int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* binum,
+int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost, const int* binum,
                    const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
 template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);

@@ -1,0 +1,579 @@
+// NEP energy / force / virial, staged kernel for the common model shape
+// (chebyshev_size 8, n_radial 6, n_angular 4, l_max 4, up to 4 species).
+//
+// The generic kernel (nep.hip) lets every thread walk its own neighbour row four times, so each
+// wave-wide load touches 64 different cache lines, and it holds the pair derivatives in a
+// [row, slot, 3] buffer that a separate pass copies into the reduction segments.  Here
+//   * the neighbour rows are read ONCE: the workgroup stages FCH slots of its FB rows through
+//     LDS per round with row-contiguous loads (FCH consecutive lanes per row); the loading lane
+//     also gathers the neighbour's species and the pair's place in its target's reduction
+//     segment (a2p::PairCsr ranks);
+//   * every thread copies its staged entries into two compact per-thread lists in global
+//     scratch, laid out [entry][thread] so that the k-th entries of a wave are contiguous:
+//     radial-only neighbours from the front, neighbours inside the angular cutoff from the back.
+//     All later loops run over these dense lists with coalesced 16-byte loads, equal trip counts
+//     across a wave, no barriers and the next entry prefetched;
+//   * the radial functions are summed per neighbour species and contracted with the
+//     coefficients once per atom (pass 1), and the coefficients are contracted with dE/dq once
+//     per atom before the radial derivative loop (pass 2);
+//   * pair derivatives are stored straight into the reduction segments.
+// Pass 1: rounds (radial sums, lists), angular moments over the back list; then descriptors,
+// hidden layer, dE/dq, dE/dS.  Pass 2: pair derivatives of the radial-only pairs (front list)
+// and of the pairs inside the angular cutoff, both parts together (back list); own force, virial.
+//
+// Formulas: source/descriptor/nep/include/{nepBasis.h:57-196; nep.h:320-529}.
+#include "a2p_common.h"
+#include "nep_device.h"
+
+namespace a2p {
+using namespace nepdev;
+namespace {
+
+constexpr int FB = 256;        // atoms (threads) per workgroup
+constexpr int FCH = 8;         // neighbour slots staged per round
+constexpr int FLS = FB + 8;    // padded row length of the staging arrays
+constexpr int FDP = 24;        // padded descriptor count (22)
+constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
+
+__device__ __forceinline__ void lds_load4(const float* p, float (&o)[4])
+{
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void lds_load4(const double* p, double (&o)[4])
+{
+    const double2 v0 = *reinterpret_cast<const double2*>(p);
+    const double2 v1 = *reinterpret_cast<const double2*>(p + 2);
+    o[0] = v0.x; o[1] = v0.y; o[2] = v1.x; o[3] = v1.y;
+}
+
+template <typename T>
+struct StagedLds {
+    T *coef, *acc;
+    T *x, *y, *z;            // staging arrays [FCH][FLS] ...
+    int *w, *p;              // ... species of the neighbour, place in the reduction segment
+    T *w0, *b0, *w1, *qs;    // network tables; they share the staging arrays' memory
+    int *nn, *red;
+};
+
+__host__ __device__ __forceinline__ size_t lds_round16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
+
+// LDS layout; returns the total size.  The network tables are only needed between the two
+// passes and overlay the staging arrays.
+template <typename T>
+__host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
+                                                             StagedLds<T>& L)
+{
+    size_t off = 0;
+    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * NB * KC * sizeof(T));
+    L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * KC * FB * sizeof(T));
+    const size_t u0 = off;
+    L.x = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.y = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.z = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
+    L.w = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
+    L.p = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
+    const size_t u1 = off;
+    off = u0;
+    L.w0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * FDP * sizeof(T));
+    L.b0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
+    L.w1 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
+    L.qs = (T*)(base + off);   off += lds_round16((size_t)FDP * sizeof(T));
+    off = off > u1 ? off : u1;
+    L.nn = (int*)(base + off); off += lds_round16((size_t)FB * sizeof(int));
+    L.red = (int*)(base + off); off += lds_round16((size_t)(FB / 64) * 10 * sizeof(double));
+    return off;
+}
+
+struct SegArgs {
+    const int* offsets;   // [B * NF] start of each target's segment, or null (no forces wanted)
+    const int* rank;      // [B*P, U] place of each pair inside its target's segment
+};
+
+// Stage slots [c0, c0 + FCH) of the workgroup's rows: thread e handles row e / FCH, slot e % FCH,
+// so FCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
+// row's end (or with an index out of range) are stored far outside every cutoff.
+template <typename T>
+__device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StagedLds<T>& L,
+                                            int tid, int c0, size_t rowbase, int b, int NF)
+{
+    const int* types = a.btypes + (size_t)b * NF;
+#pragma unroll
+    for (int it = 0; it < FCH; it++) {
+        const int e = it * FB + tid;
+        const int la = e / FCH, s = e % FCH;
+        const int slot = c0 + s;
+        T x = (T)1.0e18, y = (T)0, z = (T)0;
+        int w = 0, pos = 0;
+        if (slot < L.nn[la]) {
+            const size_t pr = (rowbase + la) * a.U + slot;
+            const T* p = a.brcs + pr * 3;
+            const int nj = a.bfirstneigh[pr];
+            if ((unsigned)nj >= (unsigned)NF) {
+                atomicOr(a.status, ST_BAD_NEIGHBOR);
+            } else {
+                x = p[0]; y = p[1]; z = p[2];
+                w = types[nj];
+                if (seg.offsets) pos = seg.offsets[(size_t)b * NF + nj] + seg.rank[pr];
+                if ((unsigned)w >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); w = 0; }
+            }
+        }
+        L.x[s * FLS + la] = x; L.y[s * FLS + la] = y; L.z[s * FLS + la] = z;
+        L.w[s * FLS + la] = w; L.p[s * FLS + la] = pos;
+    }
+}
+
+// Bit masks of a thread's staged entries: bit s set when entry s lies inside the angular cutoff,
+// bit 8+s inside the radial cutoff, bit 16+s when the entry is a pair of the list at all.
+template <typename T>
+__device__ __forceinline__ unsigned staged_classify(const StagedLds<T>& L, int tid, T rr, T ra)
+{
+    unsigned m = 0;
+#pragma unroll
+    for (int s = 0; s < FCH; s++) {
+        const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+        const T r = sqrt_t(x * x + y * y + z * z);
+        if (r <= ra) m |= 1u << s;
+        if (r <= rr) m |= 0x100u << s;
+        if (x < (T)1.0e17) m |= 0x10000u << s;
+    }
+    return m;
+}
+
+// Compact-list entries: [x y z species]
+__device__ __forceinline__ void ang_store(float* p, float x, float y, float z, int w)
+{
+    *reinterpret_cast<float4*>(p) = make_float4(x, y, z, __int_as_float(w));
+}
+__device__ __forceinline__ void ang_load(const float* p, float& x, float& y, float& z, int& w)
+{
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    x = v.x; y = v.y; z = v.z; w = __float_as_int(v.w);
+}
+__device__ __forceinline__ void ang_store(double* p, double x, double y, double z, int w)
+{
+    *reinterpret_cast<double2*>(p) = make_double2(x, y);
+    *reinterpret_cast<double2*>(p + 2) = make_double2(z, __longlong_as_double((long long)w));
+}
+__device__ __forceinline__ void ang_load(const double* p, double& x, double& y, double& z, int& w)
+{
+    const double2 v0 = *reinterpret_cast<const double2*>(p);
+    const double2 v1 = *reinterpret_cast<const double2*>(p + 2);
+    x = v0.x; y = v0.y; z = v1.x; w = (int)__double_as_longlong(v1.y);
+}
+
+template <typename T, int NTC>
+__global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
+nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T* __restrict__ ang_xyz,
+                  int* __restrict__ ang_pos)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int tid = threadIdx.x;
+    const int b = blockIdx.y;
+    const int ii = blockIdx.x * FB + tid;
+    const int H = a.H, nt = a.ntypes;
+    const int NF = a.P + a.nghost;
+    StagedLds<T> L;
+    staged_lds_layout<T>(nt, H, NTC, smem_raw, L);
+
+    for (int i = tid; i < nt * nt * NB * KC; i += FB) L.coef[i] = a.coeffs[i];
+#pragma unroll
+    for (int i = 0; i < NTC * KC; i++) L.acc[i * FB + tid] = (T)0;
+
+    const int inum = a.binum[b];
+    const bool active = ii < inum;
+    const size_t rowbase = (size_t)b * a.P + (size_t)blockIdx.x * FB;
+    const size_t row = rowbase + tid;
+    int center = 0, ti = 0, nn = 0;
+    if (active) {
+        center = a.bilist[row];
+        nn = a.bnumneigh[row];
+        if (nn > a.U) { atomicOr(a.status, ST_NEIGH_OVERFLOW); nn = a.U; }
+        if ((unsigned)center >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); center = 0; nn = 0; }
+        ti = a.btypes[(size_t)b * NF + center];
+        if ((unsigned)ti >= (unsigned)nt) { atomicOr(a.status, ST_BAD_TYPE); ti = 0; nn = 0; }
+    }
+    L.nn[tid] = nn;
+    {
+        int m = nn;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+        if ((tid & 63) == 0) L.red[tid >> 6] = m;
+    }
+    __syncthreads();
+    int maxnn = 0;
+#pragma unroll
+    for (int w = 0; w < FB / 64; w++) maxnn = max(maxnn, L.red[w]);
+
+    const T rr = a.rr, ra = a.ra;
+    const T rr_inv = (T)1 / rr, ra_inv = (T)1 / ra;
+    // compact lists of this thread: entry k at [k * FB]; radial-only entries occupy k = 0 ..
+    // n_rad-1, entries inside the angular cutoff k = U-1 .. U-n_ang (n_rad + n_ang <= nn <= U)
+    const size_t list0 = (size_t)(b * a.nblocks + blockIdx.x) * a.U * FB + tid;
+    T* const lxyz = ang_xyz + list0 * 4;
+    int* const lpos = ang_pos + list0;
+    const int back = a.U - 1;
+    const bool want_pairs = a.force != nullptr || a.want_virial;
+
+    T S[NAC][NLM];
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
+
+    // ---- pass 1 -------------------------------------------------------------------------------
+    int n_ang = 0, n_rad = 0;
+    for (int c0 = 0; c0 < maxnn; c0 += FCH) {
+        __syncthreads();
+        staged_load<T>(a, seg, L, tid, c0, rowbase, b, NF);
+        __syncthreads();
+        const unsigned cls = staged_classify<T>(L, tid, rr, ra);
+        unsigned bits = (cls >> 8) & 0xffu;
+        while (bits) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+            const int tj = L.w[s * FLS + tid];
+            const T r = sqrt_t(x * x + y * y + z * z);
+            T f[KC], df[KC];
+            radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+            for (int k = 0; k < KC; k++) L.acc[(tj * KC + k) * FB + tid] += f[k];
+            if (want_pairs && !((cls >> s) & 1u)) {
+                ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, tj);
+                lpos[(size_t)n_rad * FB] = L.p[s * FLS + tid];
+                n_rad++;
+            }
+        }
+        bits = cls & 0xffu;
+        while (bits) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            const int k = back - n_ang;
+            ang_store(lxyz + (size_t)k * FB * 4, L.x[s * FLS + tid], L.y[s * FLS + tid], L.z[s * FLS + tid],
+                      L.w[s * FLS + tid]);
+            lpos[(size_t)k * FB] = L.p[s * FLS + tid];
+            n_ang++;
+        }
+        // pairs of the list beyond both cutoffs still own a place in their segment
+        bits = (cls >> 16) & ~(cls >> 8) & ~cls & 0xffu;
+        while (bits && seg_g) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            T* dst = seg_g + (size_t)L.p[s * FLS + tid] * 3;
+            dst[0] = (T)0; dst[1] = (T)0; dst[2] = (T)0;
+        }
+    }
+    // the network tables take the place of the staging arrays
+    __syncthreads();
+    for (int i = tid; i < nt * H * FDP; i += FB) {
+        const int r = i / FDP, j = i - r * FDP;
+        L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
+    }
+    for (int i = tid; i < nt * H; i += FB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
+    if (tid < FDP) L.qs[tid] = tid < DC ? (T)1 / a.q_scaler[tid] : (T)0;
+
+    // angular moments over the back list (the next entry is in flight while one is processed)
+    T px = (T)0, py = (T)0, pz = (T)0;
+    int pw = 0;
+    if (n_ang > 0) ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw);
+    for (int e = 0; e < n_ang; e++) {
+        const T x = px, y = py, z = pz;
+        const int tj = pw;
+        if (e + 1 < n_ang) ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
+        const T r = sqrt_t(x * x + y * y + z * z);
+        const T rinv = (T)1 / r;
+        T f[KC], df[KC];
+        radial_basis<T, KC, false>(r, ra_inv, KC, f, df);
+        const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
+        T bl[NLM];
+        blm_values<T, LC>(x * rinv, y * rinv, z * rinv, bl);
+#pragma unroll
+        for (int n = 0; n < NAC; n++) {
+            T c0v[4], c1v[4];
+            lds_load4(c + n * KC, c0v);
+            lds_load4(c + n * KC + 4, c1v);
+            T g = (T)0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) g += c0v[k] * f[k];
+#pragma unroll
+            for (int k = 0; k < 4; k++) g += c1v[k] * f[4 + k];
+#pragma unroll
+            for (int m = 0; m < NLM; m++) S[n][m] += g * bl[m];
+        }
+    }
+    __syncthreads();
+
+    // ---- descriptors --------------------------------------------------------------------------
+    T q[DC];
+#pragma unroll
+    for (int j = 0; j < DC; j++) q[j] = (T)0;
+    for (int t = 0; t < nt; t++) {
+        const T* c = L.coef + (ti * nt + t) * NB * KC;
+        T fs[KC];
+#pragma unroll
+        for (int k = 0; k < KC; k++) fs[k] = L.acc[(t * KC + k) * FB + tid];
+#pragma unroll
+        for (int n = 0; n < NRC; n++) {
+            T c0v[4], c1v[4];
+            lds_load4(c + n * KC, c0v);
+            lds_load4(c + n * KC + 4, c1v);
+#pragma unroll
+            for (int k = 0; k < 4; k++) q[n] += c0v[k] * fs[k];
+#pragma unroll
+            for (int k = 0; k < 4; k++) q[n] += c1v[k] * fs[4 + k];
+        }
+    }
+    // q_{n,l} = sum_m w_m C_lm S^2  (nepBasis.h:174-190)
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int l = 1; l <= LC; l++) {
+            T acc = (T)0;
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                acc += (T)(mp == 0 ? 1.0 : 2.0) * (T)kC3B[m] * S[n][m] * S[n][m];
+            }
+            q[NRC + n * LC + (l - 1)] = acc;
+        }
+    if (active && a.desc) {
+        T* dst = a.desc + row * DC;
+#pragma unroll
+        for (int j = 0; j < DC; j++) dst[j] = q[j];
+    }
+
+    // ---- hidden layer (nep.h:415-447) ----------------------------------------------------------
+    T dEdq[DC];
+    T e_site = active ? a.bias[ti] : (T)0;
+    {
+        T qn[DC];
+#pragma unroll
+        for (int j = 0; j < DC; j++) { qn[j] = q[j] * L.qs[j]; dEdq[j] = (T)0; }
+        for (int p = 0; p < H; p++) {
+            const T* wrow = L.w0 + (size_t)(ti * H + p) * FDP;
+            T wv[FDP];
+#pragma unroll
+            for (int j = 0; j < FDP; j += 4) {
+                T v[4];
+                lds_load4(wrow + j, v);
+                wv[j] = v[0]; wv[j + 1] = v[1]; wv[j + 2] = v[2]; wv[j + 3] = v[3];
+            }
+            T h = L.b0[ti * H + p];
+#pragma unroll
+            for (int j = 0; j < DC; j++) h += wv[j] * qn[j];
+            const T t = tanh_t(h);
+            const T w1p = L.w1[ti * H + p];
+            e_site += w1p * t;
+            const T sde = w1p * ((T)1 - t * t);
+#pragma unroll
+            for (int j = 0; j < DC; j++) dEdq[j] += sde * wv[j];
+        }
+#pragma unroll
+        for (int j = 0; j < DC; j++) dEdq[j] *= L.qs[j];
+    }
+    // dE/dS (nep.h:450-466), overwriting S
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int l = 1; l <= LC; l++)
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                S[n][m] *= dEdq[NRC + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+            }
+
+    // ---- pass 2: pair derivatives ---------------------------------------------------------------
+    T fx = (T)0, fy = (T)0, fz = (T)0;
+    T vir[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vir[i] = (T)0;
+    if (want_pairs) {
+        // radial coefficients contracted with dE/dq, per neighbour species (thread-private cells)
+        for (int t = 0; t < nt; t++) {
+            const T* c = L.coef + (ti * nt + t) * NB * KC;
+            T cc[KC];
+#pragma unroll
+            for (int k = 0; k < KC; k++) cc[k] = (T)0;
+#pragma unroll
+            for (int n = 0; n < NRC; n++) {
+                T c0v[4], c1v[4];
+                lds_load4(c + n * KC, c0v);
+                lds_load4(c + n * KC + 4, c1v);
+#pragma unroll
+                for (int k = 0; k < 4; k++) { cc[k] += dEdq[n] * c0v[k]; cc[4 + k] += dEdq[n] * c1v[k]; }
+            }
+#pragma unroll
+            for (int k = 0; k < KC; k++) L.acc[(t * KC + k) * FB + tid] = cc[k];
+        }
+        auto emit = [&](int pos, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
+            if (seg_g) {
+                T* dst = seg_g + (size_t)pos * 3;
+                dst[0] = gx; dst[1] = gy; dst[2] = gz;
+            }
+            fx += gx; fy += gy; fz += gz;
+            vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
+            vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
+            vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
+        };
+        // radial-only pairs (front list)
+        int ppos = 0;
+        if (n_rad > 0) { ang_load(lxyz, px, py, pz, pw); ppos = lpos[0]; }
+        for (int e = 0; e < n_rad; e++) {
+            const T x = px, y = py, z = pz;
+            const int tj = pw, pos = ppos;
+            if (e + 1 < n_rad) {
+                ang_load(lxyz + (size_t)(e + 1) * FB * 4, px, py, pz, pw);
+                ppos = lpos[(size_t)(e + 1) * FB];
+            }
+            const T r = sqrt_t(x * x + y * y + z * z);
+            T f[KC], df[KC];
+            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+            T sr = (T)0;
+#pragma unroll
+            for (int k = 0; k < KC; k++) sr += L.acc[(tj * KC + k) * FB + tid] * df[k];
+            sr /= r;
+            emit(pos, x, y, z, sr * x, sr * y, sr * z);
+        }
+        // pairs inside the angular cutoff, radial and angular part together (back list)
+        if (n_ang > 0) { ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw); ppos = lpos[(size_t)back * FB]; }
+        for (int e = 0; e < n_ang; e++) {
+            const T x = px, y = py, z = pz;
+            const int tj = pw, pos = ppos;
+            if (e + 1 < n_ang) {
+                ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
+                ppos = lpos[(size_t)(back - e - 1) * FB];
+            }
+            const T r = sqrt_t(x * x + y * y + z * z);
+            const T rinv = (T)1 / r;
+            const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+            T f[KC], df[KC];
+            T srad = (T)0;
+            if (r <= rr) {
+                radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+#pragma unroll
+                for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * FB + tid] * df[k];
+            }
+            radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+            const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
+            T A[NLM], Ad[NLM];
+#pragma unroll
+            for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
+#pragma unroll
+            for (int n = 0; n < NAC; n++) {
+                T c0v[4], c1v[4];
+                lds_load4(c + n * KC, c0v);
+                lds_load4(c + n * KC + 4, c1v);
+                T g = (T)0, dg = (T)0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
+#pragma unroll
+                for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
+#pragma unroll
+                for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
+            }
+            T bl[NLM];
+            blm_values<T, LC>(ux, uy, uz, bl);
+#pragma unroll
+            for (int l = 1; l <= LC; l++)
+#pragma unroll
+                for (int mp = 0; mp < 2 * l + 1; mp++) {
+                    const int m = l * l - 1 + mp;
+                    srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+                }
+            T wx = (T)0, wy = (T)0, wz = (T)0;
+            blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
+            emit(pos, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
+        }
+        if (active && a.force) {
+            T* fo = a.force + ((size_t)b * NF + center) * 3;
+            fo[0] = fx; fo[1] = fy; fo[2] = fz;
+        }
+    }
+
+    // ---- workgroup partial sums of energy and virial (fp64) ---------------------------------
+    __syncthreads();
+    double* s_red = (double*)L.red;
+    double vals[10];
+    vals[0] = active ? (double)e_site : 0.0;
+#pragma unroll
+    for (int i = 0; i < 9; i++) vals[1 + i] = active ? (double)vir[i] : 0.0;
+#pragma unroll
+    for (int i = 0; i < 10; i++) {
+        double v = wave_sum(vals[i]);
+        if ((tid & 63) == 0) s_red[(tid >> 6) * 10 + i] = v;
+    }
+    __syncthreads();
+    if (tid < 10) {
+        double v = 0.0;
+        for (int w = 0; w < FB / 64; w++) v += s_red[w * 10 + tid];
+        a.partial[((size_t)b * a.nblocks + blockIdx.x) * 10 + tid] = v;
+    }
+}
+
+template <typename T, int NTC>
+int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
+{
+    // compact lists: [workgroup][entry < U][thread] of 4 T, then the same of int
+    const size_t nent = (size_t)a.B * a.nblocks * a.U * FB;
+    void* ws = nullptr;
+    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)), &ws);
+    if (rc) return rc;
+    T* ang_xyz = (T*)ws;
+    int* ang_pos = (int*)((char*)ws + nent * 4 * sizeof(T));
+    SegArgs seg{csr.offsets, csr.rank};
+    auto kern = nep_staged_kernel<T, NTC>;
+    if (lds > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)lds));
+    prof_begin("nep_staged_kernel", stream);
+    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, seg, (T*)csr.seg_g, ang_xyz,
+                       ang_pos);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+int ntc_of(int ntypes) { return ntypes <= 1 ? 1 : ntypes == 2 ? 2 : ntypes == 3 ? 3 : 4; }
+
+}  // namespace
+
+int nep_staged_nblocks(int P) { return ceil_div(P, FB); }
+
+template <typename T>
+bool nep_staged_supported(const NepArgs<T>& a, size_t* lds_bytes)
+{
+    if (!(a.K == KC && a.n_r == NRC && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
+    StagedLds<T> unused;
+    *lds_bytes = staged_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), nullptr, unused);
+    return *lds_bytes <= 150 * 1024;
+}
+
+template <typename T>
+int nep_staged_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
+{
+    PairCsr csr{};
+    int rc;
+    if (a.force) {
+        rc = fill_zero(a.force, (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), stream);
+        if (rc) return rc;
+        rc = pair_csr_begin<T>(&csr, true, a.B, a.P, a.U, a.nghost, a.binum, a.bnumneigh, a.bfirstneigh, stream);
+        if (rc) return rc;
+    }
+    switch (ntc_of(a.ntypes)) {
+    case 1: rc = launch_staged<T, 1>(a, lds_bytes, csr, stream); break;
+    case 2: rc = launch_staged<T, 2>(a, lds_bytes, csr, stream); break;
+    case 3: rc = launch_staged<T, 3>(a, lds_bytes, csr, stream); break;
+    default: rc = launch_staged<T, 4>(a, lds_bytes, csr, stream); break;
+    }
+    if (rc) return rc;
+    if (a.force) rc = pair_csr_finish<T>(a.force, csr, stream);
+    return rc;
+}
+
+template bool nep_staged_supported<float>(const NepArgs<float>&, size_t*);
+template bool nep_staged_supported<double>(const NepArgs<double>&, size_t*);
+template int nep_staged_run<float>(const NepArgs<float>&, size_t, hipStream_t);
+template int nep_staged_run<double>(const NepArgs<double>&, size_t, hipStream_t);
+
+}  // namespace a2p

@@ -24,11 +24,12 @@ constexpr int SCAN_BLOCK = 256;
 constexpr int SCAN_ITEMS = 8;   // items per thread
 constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;
 
-__global__ void count_kernel(int* __restrict__ counts, int B, int P, int U, int NF,
+__global__ void count_kernel(int* __restrict__ counts, int* __restrict__ rank, int B, int P, int U, int NF,
                              const int* __restrict__ binum, const int* __restrict__ bnumneigh,
                              const int* __restrict__ bfirstneigh, int* __restrict__ status)
 {
-    // one wave per row; lanes stride the valid slots (coalesced over the row)
+    // one wave per row; lanes stride the valid slots (coalesced over the row).  With `rank` the
+    // pair also learns its place inside its target's segment.
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int lane = threadIdx.x & 63;
     if (wave >= B * P) return;
@@ -44,9 +45,11 @@ __global__ void count_kernel(int* __restrict__ counts, int B, int P, int U, int 
         int j = row[s];
         if ((unsigned)j >= (unsigned)NF) {
             atomicOr(status, ST_BAD_NEIGHBOR);
+            if (rank) rank[(size_t)wave * U + s] = -1;
             continue;
         }
-        atomicAdd(&counts[(size_t)b * NF + j], 1);
+        if (rank) rank[(size_t)wave * U + s] = atomicAdd(&counts[(size_t)b * NF + j], 1);
+        else atomicAdd(&counts[(size_t)b * NF + j], 1);
     }
 }
 
@@ -220,7 +223,7 @@ int exclusive_scan_i32(const int* in, int* out, int n, int* tmp, hipStream_t str
 }
 
 template <typename T>
-int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* binum,
+int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost, const int* binum,
                    const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
 {
     const int NF = P + nghost;
@@ -230,12 +233,13 @@ int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* bin
                 "pair_reduce: batch too large for 32-bit pair indexing");
     const int n = (int)NT;
     const int ntiles = ceil_div(n, SCAN_TILE);
-    // workspace: counts[n] | offsets[n] | cursor[n] | tile[ntiles] | total[1] | seg_g[rows*U*3]
+    // workspace: counts[n] | offsets[n] | cursor[n] | tile[ntiles] | total[1] | seg_g[rows*U*3] | rank[rows*U]
     size_t ints = (size_t)n * 3 + ntiles + 8;
     size_t bytes = ((ints * sizeof(int) + 255) / 256) * 256;
-    size_t seg_bytes = (size_t)rows * U * 3 * sizeof(T);
+    size_t seg_bytes = (((size_t)rows * U * 3 * sizeof(T) + 255) / 256) * 256;
+    size_t rank_bytes = with_rank ? (size_t)rows * U * sizeof(int) : 0;
     void* ws = nullptr;
-    int rc = ws_get(WS_CSR, bytes + seg_bytes, &ws);
+    int rc = ws_get(WS_CSR, bytes + seg_bytes + rank_bytes, &ws);
     if (rc) return rc;
     void* flags = nullptr;
     rc = ws_get(WS_FLAGS, 64, &flags);
@@ -246,6 +250,7 @@ int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* bin
     csr->cursor = csr->offsets + n;
     int* tiles = csr->cursor + n;
     csr->seg_g = (void*)((char*)ws + bytes);
+    csr->rank = with_rank ? (int*)((char*)ws + bytes + seg_bytes) : nullptr;
 
     // counts and cursor are adjacent and start at zero (offsets is fully overwritten)
     rc = fill_zero(csr->counts, (size_t)n * sizeof(int), stream);
@@ -255,8 +260,8 @@ int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* bin
 
     const int wave_blocks = ceil_div(rows * 64, 256);
     prof_begin("reduce_count", stream);
-    hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, csr->counts, B, P, U, NF,
-                       binum, bnumneigh, bfirstneigh, (int*)flags);
+    hipLaunchKernelGGL(count_kernel, dim3(wave_blocks), dim3(256), 0, stream, csr->counts, csr->rank, B, P,
+                       U, NF, binum, bnumneigh, bfirstneigh, (int*)flags);
     prof_end(stream);
     return exclusive_scan_i32(csr->counts, csr->offsets, n, tiles, stream);
 }
@@ -264,10 +269,11 @@ int pair_csr_begin(PairCsr* csr, int B, int P, int U, int nghost, const int* bin
 template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream)
 {
-    // the cursor holds how many entries of each segment were filled
+    // with ranks every counted pair has its place in the segment; otherwise the cursor holds
+    // how many entries were filled
     prof_begin("reduce_sum", stream);
     hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)csr.n * 16, 256)), dim3(256), 0, stream,
-                       force, (const T*)csr.seg_g, csr.offsets, csr.cursor, csr.n);
+                       force, (const T*)csr.seg_g, csr.offsets, csr.rank ? csr.counts : csr.cursor, csr.n);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -278,7 +284,7 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
                 const int* bnumneigh, const int* bfirstneigh, hipStream_t stream)
 {
     PairCsr csr;
-    int rc = pair_csr_begin<T>(&csr, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+    int rc = pair_csr_begin<T>(&csr, false, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
     if (rc) return rc;
     const long long rows = (long long)B * P;
     const int wave_blocks = ceil_div(rows * 64, 256);
@@ -289,8 +295,8 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
     return pair_csr_finish<T>(force, csr, stream);
 }
 
-template int pair_csr_begin<float>(PairCsr*, int, int, int, int, const int*, const int*, const int*, hipStream_t);
-template int pair_csr_begin<double>(PairCsr*, int, int, int, int, const int*, const int*, const int*, hipStream_t);
+template int pair_csr_begin<float>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
+template int pair_csr_begin<double>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
 template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
 template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,
