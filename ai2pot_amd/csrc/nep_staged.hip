@@ -30,7 +30,7 @@ using namespace nepdev;
 namespace {
 
 constexpr int FB = 256;        // atoms (threads) per workgroup
-constexpr int FCH = 8;         // neighbour slots staged per round
+constexpr int FCH = 16;        // neighbour slots staged per round
 constexpr int FLS = FB + 8;    // padded row length of the staging arrays
 constexpr int FDP = 24;        // padded descriptor count (22)
 constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
@@ -49,31 +49,35 @@ __device__ __forceinline__ void lds_load4(const double* p, double (&o)[4])
 
 template <typename T>
 struct StagedLds {
-    T *coef, *acc;
+    T* coef;
     T *x, *y, *z;            // staging arrays [FCH][FLS] ...
-    int *w, *p;              // ... species of the neighbour, place in the reduction segment
-    T *w0, *b0, *w1, *qs;    // network tables; they share the staging arrays' memory
+    int* p;                  // ... place of the pair in its target's reduction segment
+    unsigned char* w;        // ... species of the neighbour
+    T *w0, *b0, *w1, *qs;    // network tables (between the passes) and
+    T* acc;                  // contracted radial coefficients (pass 2) share the staging memory
     int *nn, *red;
 };
 
 __host__ __device__ __forceinline__ size_t lds_round16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
 
-// LDS layout; returns the total size.  The network tables are only needed between the two
-// passes and overlay the staging arrays.
+// LDS layout; returns the total size.  The staging arrays are used in pass 1 only, the network
+// tables between the passes, the contracted coefficients in pass 2: the three share one region.
 template <typename T>
 __host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
                                                              StagedLds<T>& L)
 {
     size_t off = 0;
     L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * NB * KC * sizeof(T));
-    L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * KC * FB * sizeof(T));
     const size_t u0 = off;
     L.x = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
     L.y = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
     L.z = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
-    L.w = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
     L.p = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
-    const size_t u1 = off;
+    L.w = base + off;          off += lds_round16((size_t)FCH * FLS);
+    size_t u1 = off;
+    off = u0;
+    L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * KC * FB * sizeof(T));
+    u1 = off > u1 ? off : u1;
     off = u0;
     L.w0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * FDP * sizeof(T));
     L.b0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
@@ -86,9 +90,17 @@ __host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, 
 }
 
 struct SegArgs {
-    const int* offsets;   // [B * NF] start of each target's segment, or null (no forces wanted)
-    const int* rank;      // [B*P, U] place of each pair inside its target's segment
+    const int2* meta;     // [B * NF] per atom: .x start of its reduction segment (0 without forces), .y species
+    const int* rank;      // [B*P, U] place of each pair inside its target's segment, or null (no forces wanted)
 };
+
+// meta[t] = (offsets[t], types[t]): one 8-byte gather per pair instead of two 4-byte ones
+__global__ void pack_meta_kernel(int2* __restrict__ meta, const int* __restrict__ offsets,
+                                 const int* __restrict__ types, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) meta[i] = make_int2(offsets ? offsets[i] : 0, types[i]);
+}
 
 // Stage slots [c0, c0 + FCH) of the workgroup's rows: thread e handles row e / FCH, slot e % FCH,
 // so FCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
@@ -97,7 +109,7 @@ template <typename T>
 __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StagedLds<T>& L,
                                             int tid, int c0, size_t rowbase, int b, int NF)
 {
-    const int* types = a.btypes + (size_t)b * NF;
+    const int2* meta = seg.meta + (size_t)b * NF;
 #pragma unroll
     for (int it = 0; it < FCH; it++) {
         const int e = it * FB + tid;
@@ -113,31 +125,32 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
                 atomicOr(a.status, ST_BAD_NEIGHBOR);
             } else {
                 x = p[0]; y = p[1]; z = p[2];
-                w = types[nj];
-                if (seg.offsets) pos = seg.offsets[(size_t)b * NF + nj] + seg.rank[pr];
+                const int2 m = meta[nj];
+                w = m.y;
+                if (seg.rank) pos = m.x + seg.rank[pr];
                 if ((unsigned)w >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); w = 0; }
             }
         }
         L.x[s * FLS + la] = x; L.y[s * FLS + la] = y; L.z[s * FLS + la] = z;
-        L.w[s * FLS + la] = w; L.p[s * FLS + la] = pos;
+        L.w[s * FLS + la] = (unsigned char)w; L.p[s * FLS + la] = pos;
     }
 }
 
-// Bit masks of a thread's staged entries: bit s set when entry s lies inside the angular cutoff,
-// bit 8+s inside the radial cutoff, bit 16+s when the entry is a pair of the list at all.
+// Bit masks of a thread's staged entries: bit s of mA set when entry s lies inside the angular
+// cutoff, of mR inside the radial cutoff, of mV when the entry is a pair of the list at all.
 template <typename T>
-__device__ __forceinline__ unsigned staged_classify(const StagedLds<T>& L, int tid, T rr, T ra)
+__device__ __forceinline__ void staged_classify(const StagedLds<T>& L, int tid, T rr, T ra, unsigned& mA,
+                                                unsigned& mR, unsigned& mV)
 {
-    unsigned m = 0;
+    mA = 0; mR = 0; mV = 0;
 #pragma unroll
     for (int s = 0; s < FCH; s++) {
         const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
         const T r = sqrt_t(x * x + y * y + z * z);
-        if (r <= ra) m |= 1u << s;
-        if (r <= rr) m |= 0x100u << s;
-        if (x < (T)1.0e17) m |= 0x10000u << s;
+        if (r <= ra) mA |= 1u << s;
+        if (r <= rr) mR |= 1u << s;
+        if (x < (T)1.0e17) mV |= 1u << s;
     }
-    return m;
 }
 
 // Compact-list entries: [x y z species]
@@ -177,8 +190,6 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
     staged_lds_layout<T>(nt, H, NTC, smem_raw, L);
 
     for (int i = tid; i < nt * nt * NB * KC; i += FB) L.coef[i] = a.coeffs[i];
-#pragma unroll
-    for (int i = 0; i < NTC * KC; i++) L.acc[i * FB + tid] = (T)0;
 
     const int inum = a.binum[b];
     const bool active = ii < inum;
@@ -222,13 +233,19 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
         for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
 
     // ---- pass 1 -------------------------------------------------------------------------------
+    T F[NTC][KC];                 // radial functions summed per neighbour species
+#pragma unroll
+    for (int t = 0; t < NTC; t++)
+#pragma unroll
+        for (int k = 0; k < KC; k++) F[t][k] = (T)0;
     int n_ang = 0, n_rad = 0;
     for (int c0 = 0; c0 < maxnn; c0 += FCH) {
         __syncthreads();
         staged_load<T>(a, seg, L, tid, c0, rowbase, b, NF);
         __syncthreads();
-        const unsigned cls = staged_classify<T>(L, tid, rr, ra);
-        unsigned bits = (cls >> 8) & 0xffu;
+        unsigned mA, mR, mV;
+        staged_classify<T>(L, tid, rr, ra, mA, mR, mV);
+        unsigned bits = mR;
         while (bits) {
             const int s = __ffs(bits) - 1;
             bits &= bits - 1;
@@ -238,14 +255,16 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
             T f[KC], df[KC];
             radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
 #pragma unroll
-            for (int k = 0; k < KC; k++) L.acc[(tj * KC + k) * FB + tid] += f[k];
-            if (want_pairs && !((cls >> s) & 1u)) {
+            for (int t = 0; t < NTC; t++)
+#pragma unroll
+                for (int k = 0; k < KC; k++) F[t][k] += (tj == t) ? f[k] : (T)0;
+            if (want_pairs && !((mA >> s) & 1u)) {
                 ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, tj);
                 lpos[(size_t)n_rad * FB] = L.p[s * FLS + tid];
                 n_rad++;
             }
         }
-        bits = cls & 0xffu;
+        bits = mA;
         while (bits) {
             const int s = __ffs(bits) - 1;
             bits &= bits - 1;
@@ -256,7 +275,7 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
             n_ang++;
         }
         // pairs of the list beyond both cutoffs still own a place in their segment
-        bits = (cls >> 16) & ~(cls >> 8) & ~cls & 0xffu;
+        bits = mV & ~mR & ~mA;
         while (bits && seg_g) {
             const int s = __ffs(bits) - 1;
             bits &= bits - 1;
@@ -308,20 +327,20 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
     T q[DC];
 #pragma unroll
     for (int j = 0; j < DC; j++) q[j] = (T)0;
-    for (int t = 0; t < nt; t++) {
-        const T* c = L.coef + (ti * nt + t) * NB * KC;
-        T fs[KC];
 #pragma unroll
-        for (int k = 0; k < KC; k++) fs[k] = L.acc[(t * KC + k) * FB + tid];
+    for (int t = 0; t < NTC; t++) {
+        if (t < nt) {
+            const T* c = L.coef + (ti * nt + t) * NB * KC;
 #pragma unroll
-        for (int n = 0; n < NRC; n++) {
-            T c0v[4], c1v[4];
-            lds_load4(c + n * KC, c0v);
-            lds_load4(c + n * KC + 4, c1v);
+            for (int n = 0; n < NRC; n++) {
+                T c0v[4], c1v[4];
+                lds_load4(c + n * KC, c0v);
+                lds_load4(c + n * KC + 4, c1v);
 #pragma unroll
-            for (int k = 0; k < 4; k++) q[n] += c0v[k] * fs[k];
+                for (int k = 0; k < 4; k++) q[n] += c0v[k] * F[t][k];
 #pragma unroll
-            for (int k = 0; k < 4; k++) q[n] += c1v[k] * fs[4 + k];
+                for (int k = 0; k < 4; k++) q[n] += c1v[k] * F[t][4 + k];
+            }
         }
     }
     // q_{n,l} = sum_m w_m C_lm S^2  (nepBasis.h:174-190)
@@ -388,6 +407,7 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
     T vir[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) vir[i] = (T)0;
+    __syncthreads();   // every thread is done with the network tables: their memory becomes L.acc
     if (want_pairs) {
         // radial coefficients contracted with dE/dq, per neighbour species (thread-private cells)
         for (int t = 0; t < nt; t++) {
@@ -517,11 +537,15 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
     // compact lists: [workgroup][entry < U][thread] of 4 T, then the same of int
     const size_t nent = (size_t)a.B * a.nblocks * a.U * FB;
     void* ws = nullptr;
-    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)), &ws);
+    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)) + (size_t)a.B * (a.P + a.nghost) * sizeof(int2), &ws);
     if (rc) return rc;
     T* ang_xyz = (T*)ws;
     int* ang_pos = (int*)((char*)ws + nent * 4 * sizeof(T));
-    SegArgs seg{csr.offsets, csr.rank};
+    int2* meta = (int2*)((char*)ws + nent * (4 * sizeof(T) + sizeof(int)));
+    const int ntarget = a.B * (a.P + a.nghost);
+    hipLaunchKernelGGL(pack_meta_kernel, dim3(ceil_div(ntarget, 256)), dim3(256), 0, stream, meta,
+                       (const int*)csr.offsets, a.btypes, ntarget);
+    SegArgs seg{meta, csr.rank};
     auto kern = nep_staged_kernel<T, NTC>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
