@@ -222,9 +222,11 @@ __global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int*
 }
 
 // ---- 5. order inside a bin: descending supercell index (head insertion, binLinkedList.h:833) -
+// Afterwards only the atom behind a supercell entry matters (neighborList.h:561), so the sorted
+// indices are reduced modulo natoms here, once per entry instead of once per candidate pair.
 template <typename T>
 __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* __restrict__ s_idx,
-                               T* __restrict__ s_x)
+                               T* __restrict__ s_x, int natoms)
 {
     const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (b >= nbins) return;
@@ -245,6 +247,7 @@ __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* 
         s_x[(size_t)(j + 1) * 3 + 1] = ky;
         s_x[(size_t)(j + 1) * 3 + 2] = kz;
     }
+    for (int i = beg; i < end; i++) s_idx[i] %= natoms;
 }
 
 // squared distance as the reference forms it: differences in T, squares and sum in double,
@@ -256,8 +259,39 @@ __device__ __forceinline__ double dist2_double(T dx, T dy, T dz)
     return __dadd_rn(__dadd_rn(__dmul_rn(a, a), __dmul_rn(b, b)), __dmul_rn(c, c));
 }
 
+// row[beg .. end) = v by one wave: single elements up to the first 16-byte boundary, then
+// 16-byte stores, then the tail
+template <typename V>
+__device__ __forceinline__ void pad_fill(V* __restrict__ row, int beg, int end, V v, int lane)
+{
+    constexpr int PER = 16 / (int)sizeof(V);
+    const uintptr_t addr = (uintptr_t)(row + beg);
+    int head = (int)(((16 - (addr & 15)) & 15) / sizeof(V));
+    head = min(head, end - beg);
+    if (lane < head) row[beg + lane] = v;
+    const int b0 = beg + head;
+    const int nvec = (end - b0) / PER;
+    struct alignas(16) Vec { V e[PER]; };
+    Vec vv;
+#pragma unroll
+    for (int i = 0; i < PER; i++) vv.e[i] = v;
+    Vec* dst = reinterpret_cast<Vec*>(row + b0);
+    for (int i = lane; i < nvec; i += 64) dst[i] = vv;
+    const int t0 = b0 + nvec * PER;
+    if (t0 + lane < end) row[t0 + lane] = v;
+}
+
 // ---- 6. per-atom lists: one wavefront per centre atom ----------------------------------------
-template <typename T>
+// The reference walks the (2e+1)^3 bins around the centre's bin, dx outermost and dz innermost
+// (binLinkedList.h:925-927), and appends every atom closer than rcut.  Bins are stored so that
+// the dz run of a (dx, dy) column is contiguous: lane c owns column c.  A column, or the ends of
+// its dz run, that lies farther from the centre atom than rcut (with a margin for the rounding
+// of the binning) cannot contribute and is left out; the order of what remains is unchanged.
+// The runs are then laid out back to back in LDS as a flat candidate list, which the wave
+// scans 64 candidates at a time; accepted candidates are appended with a ballot prefix.
+constexpr int NBL_ENT_CAP = 512;   // flat candidate list per wave (entries); longer lists search the runs
+
+template <typename T, bool SORT>
 __global__ void __launch_bounds__(NBL_BLOCK)
 lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
@@ -267,6 +301,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
 {
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
+    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int p = blockIdx.x * (NBL_BLOCK / 64) + wv;
     if (p >= g.N) return;                         // whole wave leaves together
@@ -278,18 +313,42 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         cb[a] = bin_of(c[a], g.mn[a], g.bin_size);
     }
     const int e = g.ext_bins, side = 2 * e + 1, nruns = side * side;
-    // column `lane` = (dx, dy): binLinkedList.h:925-927 order, dz innermost
     int start = 0, len = 0;
     if (lane < nruns) {
-        const int bx = cb[0] + lane / side - e, by = cb[1] + lane % side - e;
+        const int lq = (int)(((float)lane + 0.5f) / (float)side);    // lane / side for small integers
+        const int bx = cb[0] + lq - e, by = cb[1] + (lane - lq * side) - e;
         int zlo = cb[2] - e, zhi = cb[2] + e;
         // bins outside the reference's grid are skipped (binLinkedList.h:952-968); inside it the
         // box kept here covers every bin within `e` of a centre atom
-        const bool ok = bx >= 0 && bx < g.nbin[0] && by >= 0 && by < g.nbin[1] &&
-                        bx >= g.rlo[0] && bx < g.rlo[0] + g.rdim[0] && by >= g.rlo[1] &&
-                        by < g.rlo[1] + g.rdim[1];
+        bool ok = bx >= 0 && bx < g.nbin[0] && by >= 0 && by < g.nbin[1] &&
+                  bx >= g.rlo[0] && bx < g.rlo[0] + g.rdim[0] && by >= g.rlo[1] &&
+                  by < g.rlo[1] + g.rdim[1];
         zlo = max(zlo, max(0, g.rlo[2]));
         zhi = min(zhi, min(g.nbin[2] - 1, g.rlo[2] + g.rdim[2] - 1));
+        // geometric pruning in double: distance from the atom to the column's rectangle in x, y
+        {
+            const double bs = (double)g.bin_size, eps = sizeof(T) == 4 ? 1.2e-7 : 2.3e-16;
+            double lat2 = 0.0, tolmax = 0.0;
+            const int bxy[2] = {bx, by};
+#pragma unroll
+            for (int a = 0; a < 2; a++) {
+                const double rel = (double)c[a] - (double)g.mn[a];
+                const double tol = 1.0e-3 * bs + 8.0 * eps * (fabs(rel) + fabs((double)c[a]) + bs);
+                const double lo = bxy[a] * bs, hi = lo + bs;
+                double d = fmax(fmax(lo - rel, rel - hi), 0.0) - tol;
+                d = fmax(d, 0.0);
+                lat2 += d * d;
+                tolmax = fmax(tolmax, tol);
+            }
+            if (lat2 > g.rcut2) ok = false;
+            else {
+                const double rel = (double)c[2] - (double)g.mn[2];
+                const double tol = 1.0e-3 * bs + 8.0 * eps * (fabs(rel) + fabs((double)c[2]) + bs);
+                const double reach = sqrt(g.rcut2 - lat2) + tol;
+                zlo = max(zlo, (int)floor((rel - reach) / bs));
+                zhi = min(zhi, (int)floor((rel + reach) / bs));
+            }
+        }
         if (ok && zlo <= zhi) {
             const int col = ((bx - g.rlo[0]) * g.rdim[1] + (by - g.rlo[1])) * g.rdim[2] - g.rlo[2];
             start = offsets[col + zlo];
@@ -298,8 +357,12 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     }
     const int incl = wave_inclusive_scan(len);
     const int total = __shfl(incl, 63, 64);
+    const int base = incl - len;
     sh_start[wv][lane] = start;
-    sh_base[wv][lane] = incl - len;
+    sh_base[wv][lane] = base;
+    const bool flat = total <= NBL_ENT_CAP;       // wave-uniform
+    if (flat)
+        for (int k = 0; k < len; k++) sh_ent[wv][base + k] = start + k;
     __builtin_amdgcn_wave_barrier();
 
     int cnt = 0;
@@ -311,13 +374,18 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         int sj = 0;
         double d2d = 0.0;
         if (ci < total) {
-            // last column whose base is <= ci
-            int lo = 0, hi = nruns - 1;
-            while (lo < hi) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+            int ent;
+            if (flat) {
+                ent = sh_ent[wv][ci];
+            } else {
+                // last column whose base is <= ci
+                int lo = 0, hi = nruns - 1;
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+                }
+                ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
             }
-            const int ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
             sj = s_idx[ent];
             dx = sub_rn(s_x[(size_t)ent * 3 + 0], c[0]);
             dy = sub_rn(s_x[(size_t)ent * 3 + 1], c[1]);
@@ -330,11 +398,11 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         const int rank = __popcll(mask & ((1ull << lane) - 1ull));
         const int slot = cnt + rank;
         if (in && slot < umax) {
-            firstneigh[rowi + slot] = sj % g.N;                     // neighborList.h:561
+            firstneigh[rowi + slot] = sj;                           // neighborList.h:561 (already mod natoms)
             rcs[(rowi + slot) * 3 + 0] = dx;
             rcs[(rowi + slot) * 3 + 1] = dy;
             rcs[(rowi + slot) * 3 + 2] = dz;
-            if (keys) keys[rowi + slot] = (T)__dsqrt_rn(d2d);            // neighborList.h:318-322
+            if (SORT) keys[rowi + slot] = (T)__dsqrt_rn(d2d);       // neighborList.h:318-322
         }
         cnt += __popcll(mask);
     }
@@ -346,8 +414,8 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     }
     // padding: -1 / 0 (neighborList.h:557, 563)
     const int first_pad = min(cnt, umax);
-    for (int s = first_pad + lane; s < umax; s += 64) firstneigh[rowi + s] = -1;
-    for (int s = first_pad * 3 + lane; s < umax * 3; s += 64) rcs[rowi * 3 + s] = (T)0;
+    pad_fill(firstneigh + rowi, first_pad, umax, -1, lane);
+    pad_fill(rcs + rowi * 3, first_pad * 3, umax * 3, (T)0, lane);
 }
 
 // ---- 7. distance sort, emulating libstdc++ std::sort(indices, cmp = d[a] < d[b]) --------------
@@ -695,13 +763,16 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
-                       (int)nregion, offsets, s_idx, s_x);
+                       (int)nregion, offsets, s_idx, s_x, g.N);
     prof_end(stream);
     const int list_blocks = ceil_div(N, NBL_BLOCK / 64);
     prof_begin("nbl_lists", stream);
-    hipLaunchKernelGGL(lists_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types, offsets,
-                       s_idx, s_x, umax, ilist, numneigh, sort ? tmp_first : firstneigh,
-                       sort ? tmp_rcs : rcs, types_out, keys, status);
+    if (sort)
+        hipLaunchKernelGGL((lists_kernel<T, true>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types,
+                           offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys, status);
+    else
+        hipLaunchKernelGGL((lists_kernel<T, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types,
+                           offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys, status);
     prof_end(stream);
     if (sort) {
         prof_begin("nbl_sort_rows", stream);
