@@ -101,15 +101,16 @@ __device__ __forceinline__ long long shfl_xor_ll(long long v, int off)
     return ((long long)hi << 32) | (unsigned int)lo;
 }
 
-// inclusive prefix sum across the 64 lanes of a wave
+// inclusive prefix sum across the 64 lanes of a wave: shifts by 1, 2, 4, 8 inside each row of
+// 16 lanes, then the last lane of row 0 / 2 is added to row 1 / 3 and lane 31 to rows 2 and 3
 __device__ __forceinline__ int wave_inclusive_scan(int v)
 {
-    int lane = lane_id();
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        int o = __shfl_up(v, off, 64);
-        if (lane >= off) v += o;
-    }
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);    // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);    // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);    // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);    // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 -> rows 1, 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 -> rows 2, 3
     return v;
 }
 

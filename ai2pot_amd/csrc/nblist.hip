@@ -325,28 +325,27 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
                   by < g.rlo[1] + g.rdim[1];
         zlo = max(zlo, max(0, g.rlo[2]));
         zhi = min(zhi, min(g.nbin[2] - 1, g.rlo[2] + g.rdim[2] - 1));
-        // geometric pruning in double: distance from the atom to the column's rectangle in x, y
+        // geometric pruning (float is enough: the margin dwarfs its rounding): distance from the
+        // atom to the column's rectangle in x and y, then the reach left for z
         {
-            const double bs = (double)g.bin_size, eps = sizeof(T) == 4 ? 1.2e-7 : 2.3e-16;
-            double lat2 = 0.0, tolmax = 0.0;
+            const float bs = (float)g.bin_size, inv_bs = 1.0f / bs, rc2 = (float)g.rcut2 * 1.00001f;
+            float lat2 = 0.0f;
             const int bxy[2] = {bx, by};
 #pragma unroll
             for (int a = 0; a < 2; a++) {
-                const double rel = (double)c[a] - (double)g.mn[a];
-                const double tol = 1.0e-3 * bs + 8.0 * eps * (fabs(rel) + fabs((double)c[a]) + bs);
-                const double lo = bxy[a] * bs, hi = lo + bs;
-                double d = fmax(fmax(lo - rel, rel - hi), 0.0) - tol;
-                d = fmax(d, 0.0);
+                const float rel = (float)c[a] - (float)g.mn[a];
+                const float tol = 1.0e-3f * bs + 1.0e-5f * (fabsf(rel) + fabsf((float)c[a]) + fabsf((float)g.mn[a]));
+                const float lo = (float)bxy[a] * bs;
+                const float d = fmaxf(fmaxf(lo - rel, rel - (lo + bs)) - tol, 0.0f);
                 lat2 += d * d;
-                tolmax = fmax(tolmax, tol);
             }
-            if (lat2 > g.rcut2) ok = false;
+            if (lat2 > rc2) ok = false;
             else {
-                const double rel = (double)c[2] - (double)g.mn[2];
-                const double tol = 1.0e-3 * bs + 8.0 * eps * (fabs(rel) + fabs((double)c[2]) + bs);
-                const double reach = sqrt(g.rcut2 - lat2) + tol;
-                zlo = max(zlo, (int)floor((rel - reach) / bs));
-                zhi = min(zhi, (int)floor((rel + reach) / bs));
+                const float rel = (float)c[2] - (float)g.mn[2];
+                const float tol = 1.0e-3f * bs + 1.0e-5f * (fabsf(rel) + fabsf((float)c[2]) + fabsf((float)g.mn[2]));
+                const float reach = sqrtf(rc2 - lat2) + tol;
+                zlo = max(zlo, (int)floorf((rel - reach) * inv_bs - 1.0e-3f));
+                zhi = min(zhi, (int)floorf((rel + reach) * inv_bs + 1.0e-3f));
             }
         }
         if (ok && zlo <= zhi) {
