@@ -133,6 +133,10 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 //                    for EVERY valid pair (zeros where the derivative vanishes), or, without
 //                    ranks, claims  pos = offsets[t] + atomicAdd(&cursor[t], 1)  and may skip pairs;
 //   pair_csr_finish  sums the filled part of every segment onto `force` as above.
+// pair_fixed_begin skips counting: every target owns a segment of fixed capacity seg_cap = U
+// (a cutoff-built list sends an atom no more pairs than its own row could hold); the producer
+// claims  rank = atomicAdd(&cursor[t], 1),  stores at  pos = t*seg_cap + rank  when rank < seg_cap
+// and otherwise raises ST_NEIGH_OVERFLOW and stores at the spare entry n*seg_cap.
 struct PairCsr {
     int* counts;
     int* offsets;
@@ -140,10 +144,13 @@ struct PairCsr {
     int* rank;      // [B*P, U] or null
     void* seg_g;
     int n;          // B * (P + nghost) targets
+    int seg_cap;    // > 0: fixed-capacity segments (offsets, counts and rank are null)
 };
 template <typename T>
 int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost, const int* binum,
                    const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
+template <typename T>
+int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream);
 template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);
 

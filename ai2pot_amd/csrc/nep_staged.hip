@@ -7,7 +7,7 @@
 //   * the neighbour rows are read ONCE: the workgroup stages FCH slots of its FB rows through
 //     LDS per round with row-contiguous loads (FCH consecutive lanes per row); the loading lane
 //     also gathers the neighbour's species and the pair's place in its target's reduction
-//     segment (a2p::PairCsr ranks);
+//     segment with an integer atomic (a2p::PairCsr, fixed-capacity segments);
 //   * every thread copies its staged entries into two compact per-thread lists in global
 //     scratch, laid out [entry][thread] so that the k-th entries of a wave are contiguous:
 //     radial-only neighbours from the front, neighbours inside the angular cutoff from the back.
@@ -90,17 +90,10 @@ __host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, 
 }
 
 struct SegArgs {
-    const int2* meta;     // [B * NF] per atom: .x start of its reduction segment (0 without forces), .y species
-    const int* rank;      // [B*P, U] place of each pair inside its target's segment, or null (no forces wanted)
+    int* cursor;   // [B * NF] entries claimed so far in each target's reduction segment, or null (no forces)
+    int cap;       // capacity of a segment
+    int spare;     // entry that takes what overflows a segment
 };
-
-// meta[t] = (offsets[t], types[t]): one 8-byte gather per pair instead of two 4-byte ones
-__global__ void pack_meta_kernel(int2* __restrict__ meta, const int* __restrict__ offsets,
-                                 const int* __restrict__ types, int n)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) meta[i] = make_int2(offsets ? offsets[i] : 0, types[i]);
-}
 
 // Stage slots [c0, c0 + FCH) of the workgroup's rows: thread e handles row e / FCH, slot e % FCH,
 // so FCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
@@ -109,7 +102,7 @@ template <typename T>
 __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StagedLds<T>& L,
                                             int tid, int c0, size_t rowbase, int b, int NF)
 {
-    const int2* meta = seg.meta + (size_t)b * NF;
+    const int* types = a.btypes + (size_t)b * NF;
 #pragma unroll
     for (int it = 0; it < FCH; it++) {
         const int e = it * FB + tid;
@@ -125,9 +118,13 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
                 atomicOr(a.status, ST_BAD_NEIGHBOR);
             } else {
                 x = p[0]; y = p[1]; z = p[2];
-                const int2 m = meta[nj];
-                w = m.y;
-                if (seg.rank) pos = m.x + seg.rank[pr];
+                w = types[nj];
+                if (seg.cursor) {
+                    const int t = b * NF + nj;
+                    const int rk = atomicAdd(&seg.cursor[t], 1);
+                    pos = rk < seg.cap ? t * seg.cap + rk : seg.spare;
+                    if (rk >= seg.cap) atomicOr(a.status, ST_NEIGH_OVERFLOW);
+                }
                 if ((unsigned)w >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); w = 0; }
             }
         }
@@ -537,15 +534,11 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
     // compact lists: [workgroup][entry < U][thread] of 4 T, then the same of int
     const size_t nent = (size_t)a.B * a.nblocks * a.U * FB;
     void* ws = nullptr;
-    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)) + (size_t)a.B * (a.P + a.nghost) * sizeof(int2), &ws);
+    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)), &ws);
     if (rc) return rc;
     T* ang_xyz = (T*)ws;
     int* ang_pos = (int*)((char*)ws + nent * 4 * sizeof(T));
-    int2* meta = (int2*)((char*)ws + nent * (4 * sizeof(T) + sizeof(int)));
-    const int ntarget = a.B * (a.P + a.nghost);
-    hipLaunchKernelGGL(pack_meta_kernel, dim3(ceil_div(ntarget, 256)), dim3(256), 0, stream, meta,
-                       (const int*)csr.offsets, a.btypes, ntarget);
-    SegArgs seg{meta, csr.rank};
+    SegArgs seg{csr.cursor, csr.seg_cap, csr.n * csr.seg_cap};
     auto kern = nep_staged_kernel<T, NTC>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -581,7 +574,7 @@ int nep_staged_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     if (a.force) {
         rc = fill_zero(a.force, (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), stream);
         if (rc) return rc;
-        rc = pair_csr_begin<T>(&csr, true, a.B, a.P, a.U, a.nghost, a.binum, a.bnumneigh, a.bfirstneigh, stream);
+        rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream);
         if (rc) return rc;
     }
     switch (ntc_of(a.ntypes)) {

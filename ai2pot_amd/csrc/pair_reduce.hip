@@ -152,14 +152,16 @@ __global__ void fill_kernel(T* __restrict__ seg_g, int* __restrict__ cursor,
 // 16 lanes per target atom.
 template <typename T>
 __global__ void reduce_kernel(T* __restrict__ force, const T* __restrict__ seg_g,
-                              const int* __restrict__ offsets, const int* __restrict__ counts, int NT)
+                              const int* __restrict__ offsets, const int* __restrict__ counts, int NT,
+                              int seg_cap)
 {
     const int gid = blockIdx.x * blockDim.x + threadIdx.x;
     const int t = gid >> 4;
     const int sub = gid & 15;
     const bool live = t < NT;
-    const int beg = live ? offsets[t] : 0;
-    const int cnt = live ? counts[t] : 0;
+    // seg_cap > 0: segments of fixed capacity, target t owns entries [t*seg_cap, (t+1)*seg_cap)
+    const int beg = !live ? 0 : seg_cap > 0 ? t * seg_cap : offsets[t];
+    const int cnt = !live ? 0 : seg_cap > 0 ? min(counts[t], seg_cap) : counts[t];
     // pass 1: largest magnitude of the segment
     double m = 0.0;
     for (int e = sub; e < cnt; e += 16) {
@@ -245,6 +247,7 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
     rc = ws_get(WS_FLAGS, 64, &flags);
     if (rc) return rc;
     csr->n = n;
+    csr->seg_cap = 0;
     csr->counts = (int*)ws;
     csr->offsets = csr->counts + n;
     csr->cursor = csr->offsets + n;
@@ -267,13 +270,37 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
 }
 
 template <typename T>
+int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream)
+{
+    const long long NT = (long long)B * (P + nghost);
+    A2P_REQUIRE(NT * U + 1 < (1ll << 31), A2P_ERR_INVALID,
+                "pair_reduce: (natoms_pad + nghost) * umax exceeds 32-bit pair indexing");
+    const int n = (int)NT;
+    // workspace: cursor[n] | seg_g[(n*U + 1) * 3]   (the last entry takes what overflows)
+    size_t bytes = (((size_t)n * sizeof(int) + 255) / 256) * 256;
+    size_t seg_bytes = ((size_t)n * U + 1) * 3 * sizeof(T);
+    void* ws = nullptr;
+    int rc = ws_get(WS_CSR, bytes + seg_bytes, &ws);
+    if (rc) return rc;
+    csr->n = n;
+    csr->seg_cap = U;
+    csr->counts = nullptr;
+    csr->offsets = nullptr;
+    csr->rank = nullptr;
+    csr->cursor = (int*)ws;
+    csr->seg_g = (void*)((char*)ws + bytes);
+    return fill_zero(csr->cursor, (size_t)n * sizeof(int), stream);
+}
+
+template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream)
 {
     // with ranks every counted pair has its place in the segment; otherwise the cursor holds
     // how many entries were filled
     prof_begin("reduce_sum", stream);
     hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)csr.n * 16, 256)), dim3(256), 0, stream,
-                       force, (const T*)csr.seg_g, csr.offsets, csr.rank ? csr.counts : csr.cursor, csr.n);
+                       force, (const T*)csr.seg_g, csr.offsets, csr.rank ? csr.counts : csr.cursor, csr.n,
+                       csr.seg_cap);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -297,6 +324,8 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 
 template int pair_csr_begin<float>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
 template int pair_csr_begin<double>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
+template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t);
+template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t);
 template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
 template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,
