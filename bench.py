@@ -79,6 +79,15 @@ def timed(step, steps, warmup, L):
     return t1 - t0, kernels
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
+# counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
+# summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
+MEASURED_TRAFFIC = {
+    ("nep_md_1048576", "nep_staged_kernel"): 6.584e6 * 1024,
+    ("nep_md_1048576", "nbl_lists"): 4.100e6 * 1024,
+}
+
+
 def roofline_of(kernels, work):
     """work: {label: (bound, amount per launch, unit, peak, scale, engine)}; picks the label with
     the largest total time."""
@@ -150,7 +159,10 @@ def run_nep_md(args, kind, size, rebuild=True):
               "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 7.0, "rcut_angular": 4.0,
               "umax": 200, "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
               "per_step": ("neighbor rebuild + " if rebuild else "") + "descriptors + ANN + force/virial"}
-    return n, elapsed, kernels, roofline_of(kernels, work), config, "f32"
+    roof = roofline_of(kernels, work)
+    if roof is not None:
+        roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, roof["kernel"]))
+    return n, elapsed, kernels, roof, config, "f32"
 
 
 def cpu_baseline_nep(sample_reps=32, repeats=2):
@@ -294,6 +306,26 @@ def cpu_baseline_mtp(cfg):
                 sample="the full workload (%d atoms), %s, OpenMP %d threads, one run" % (natoms, what, threads))
 
 
+def run_copy_probe(args):
+    """Plain device copy of a known size (1 GiB read, 1 GiB written per step).  It is the yardstick
+    for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters the roofline `traffic` figures are scaled by."""
+    import torch
+    n = 1 << 28
+    x = torch.full((n,), 1.0, dtype=torch.float32, device="cuda:0")
+    y = torch.empty_like(x)
+    for _ in range(args.warmup):
+        y.copy_(x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y.copy_(x)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    print(json.dumps({"metric": "device copy bandwidth (read + write)", "value": 2 * 4 * n / dt / 1e9, "unit": "GB/s",
+                      "bytes_read_per_step": 4 * n, "bytes_written_per_step": 4 * n, "ms_per_step": dt * 1e3,
+                      "steps": args.steps, "warmup": args.warmup, "n_gpus": 1}))
+
+
 WORKLOADS = {
     "nep_md_1048576": lambda a: run_nep_md(a, "fcc", 64),         # BASELINE.json configs[4] (headline)
     "nep_md_131072": lambda a: run_nep_md(a, "fcc", 32),
@@ -301,6 +333,7 @@ WORKLOADS = {
     "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]
     "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
     "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]
+    "hbm_copy_probe": None,                                       # counter calibration, not a workload of the path
 }
 
 
@@ -319,6 +352,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
+    if args.workload == "hbm_copy_probe":
+        return run_copy_probe(args)
 
     n, elapsed, kernels, roofline, config, dtype = WORKLOADS[args.workload](args)
     ms_per_step = elapsed * 1e3 / args.steps
