@@ -143,55 +143,116 @@ __device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, int lan
     }
 }
 
-// forward products: M[dst] = sum mult M[m0] M[m1]; with TANGENT also the product rule on Tg
-template <typename T, bool TANGENT>
-__device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, int lane)
+// forward products: M[dst] = sum mult M[m0] M[m1]; with TANGENT also the product rule on Tg.
+// `part` (and `part2` with TANGENT) hold one partial sum per slot of the current level.
+template <typename T, bool TANGENT, int NT>
+__device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, T* part, T* part2, int tid)
 {
     for (int l = 0; l < p.n_levels; l++) {
-        for (int s = p.f_level[l] + lane; s < p.f_level[l + 1]; s += 64) {
+        const int s0 = p.f_level[l], s1 = p.f_lend[l];
+        const bool multi = p.f_multi[l] != 0;
+        for (int s = s0 + tid; s < s1; s += NT) {
+            const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group
+            const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
             T acc = (T)0, tacc = (T)0;
-            for (int t = p.f_begin[s]; t < p.f_begin[s + 1]; t++) {
-                const int m0 = p.f_m0[t], m1 = p.f_m1[t];
-                const T mult = (T)p.f_mult[t];
+#pragma unroll 4
+            for (int k = 0; k < depth; k++) {
+                const int2 w = tp[k * 64];
+                const int m0 = w.x & 0xffff, m1 = (int)((unsigned)w.x >> 16);
+                const T mult = (T)w.y;
                 const T v0 = M[m0], v1 = M[m1];
                 acc += mult * v0 * v1;
                 if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
             }
-            const int dst = p.f_dst[s];
-            M[dst] = acc;
-            if (TANGENT) Tg[dst] = tacc;
+            if (multi) {
+                part[s - s0] = acc;
+                if (TANGENT) part2[s - s0] = tacc;
+            } else {
+                const int dst = p.f_dst[s];
+                M[dst] = acc;
+                if (TANGENT) Tg[dst] = tacc;
+            }
         }
         __syncthreads();
+        if (multi) {
+            for (int s = s0 + tid; s < s1; s += NT) {
+                const int np = p.f_lead[s];
+                if (np == 0) continue;
+                T acc = (T)0, tacc = (T)0;
+                for (int q = 0; q < np; q++) {
+                    acc += part[s - s0 + q];
+                    if (TANGENT) tacc += part2[s - s0 + q];
+                }
+                const int dst = p.f_dst[s];
+                M[dst] = acc;
+                if (TANGENT) Tg[dst] = tacc;
+            }
+            __syncthreads();
+        }
     }
 }
 
 // reverse gather: X[m] += sum mult (X[dst] M[other] (+ A[dst] Tg[other] when MIXED))
-template <typename T, bool MIXED>
+template <typename T, bool MIXED, int NT>
 __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M, T* X, const T* A,
-                                              const T* Tg, int lane)
+                                              const T* Tg, T* part, int tid)
 {
     for (int l = p.n_levels - 1; l >= 0; l--) {
-        for (int s = p.r_level[l] + lane; s < p.r_level[l + 1]; s += 64) {
-            const int m = p.r_src[s];
-            T acc = X[m];
-            for (int t = p.r_begin[s]; t < p.r_begin[s + 1]; t++) {
-                const int dst = p.r_dst[t], other = p.r_other[t];
-                const T mult = (T)p.r_mult[t];
+        const int s0 = p.r_level[l], s1 = p.r_lend[l];
+        const bool multi = p.r_multi[l] != 0;
+        for (int s = s0 + tid; s < s1; s += NT) {
+            const int depth = p.r_gdepth[s >> 6];
+            const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
+            T acc = (T)0;
+#pragma unroll 4
+            for (int k = 0; k < depth; k++) {
+                const int2 w = tp[k * 64];
+                const int dst = w.x & 0xffff, other = (int)((unsigned)w.x >> 16);
+                const T mult = (T)w.y;
                 acc += X[dst] * mult * M[other];
                 if (MIXED) acc += mult * A[dst] * Tg[other];
             }
-            X[m] = acc;
+            if (multi) part[s - s0] = acc;
+            else X[p.r_src[s]] += acc;
         }
         __syncthreads();
+        if (multi) {
+            for (int s = s0 + tid; s < s1; s += NT) {
+                const int np = p.r_lead[s];
+                if (np == 0) continue;
+                const int m = p.r_src[s];
+                T acc = X[m];
+                for (int q = 0; q < np; q++) acc += part[s - s0 + q];
+                X[m] = acc;
+            }
+            __syncthreads();
+        }
     }
 }
 
-template <typename T, bool LOSS>
-__global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
+// sum over the NT threads of a workgroup in a fixed order (wave sums, then wave 0 .. last)
+template <typename T, int NT>
+__device__ __forceinline__ T block_sum(T v, T* scratch, int tid)
 {
+    v = wave_sum(v);
+    if (NT == 64) return v;
+    __syncthreads();
+    if ((tid & 63) == 0) scratch[tid >> 6] = v;
+    __syncthreads();
+    T t = (T)0;
+#pragma unroll
+    for (int w = 0; w < NT / 64; w++) t += scratch[w];
+    return t;
+}
+
+// NT threads per centre atom: 64 for small tables, 256 when there is enough work per atom
+template <typename T, bool LOSS, int NT>
+__global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
+{
+    constexpr int NG = NT / 32;       // thread groups of the pair passes: group h, neighbour j
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const MtpPlanDevice& p = a.p;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x;     // thread in the workgroup
     const int ii = blockIdx.x, b = blockIdx.y;
     const int NF = a.P + a.nghost;
     const size_t row = (size_t)b * a.P + ii;
@@ -205,12 +266,13 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
     T* Tg = A + n_moms;                      // loss mode only
     T* Bm = Tg + (LOSS ? n_moms : 0);        // loss mode only
     T* tab = Bm + (LOSS ? n_moms : 0);
-    T* pq = tab + MTP_NC * E;                // loss mode: P[nc][nmus] | Q[nc][nmus]
+    T* gred = tab + MTP_NC * E;              // [256/32][32][4] partial sums of the thread groups
+    T* pq = tab + max(MTP_NC * E + (256 / 32) * 32 * 4, p.max_level_slots * (LOSS ? 2 : 1));              // loss mode: P[nc][nmus] | Q[nc][nmus]
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
         if (!LOSS && lane < 10) a.partial[row * 10 + lane] = 0.0;
         if (LOSS)
-            for (int q = lane; q < a.ngrad; q += 64) a.gpart[row * a.ngrad + q] = (T)0;
+            for (int q = lane; q < a.ngrad; q += NT) a.gpart[row * a.ngrad + q] = (T)0;
         return;
     }
     int center = a.bilist[row];
@@ -223,7 +285,7 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
     const int* first = a.bfirstneigh + row * a.U;
     const T* rcs = a.brcs + row * a.U * 3;
 
-    for (int i = lane; i < n_moms; i += 64) {
+    for (int i = lane; i < n_moms; i += NT) {
         M[i] = (T)0; A[i] = (T)0;
         if (LOSS) { Tg[i] = (T)0; Bm[i] = (T)0; }
     }
@@ -235,7 +297,7 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
         int nj; bool valid; T d[3];
         build_table<T, LOSS>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
         __syncthreads();
-        for (int i = lane; i < n_basic; i += 64) {
+        for (int i = lane; i < n_basic; i += NT) {
             const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
                       ec = p.basic[i * 4 + 3];
             const T kk = (T)(ea + eb + ec);
@@ -261,14 +323,14 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
     }
 
     // ---- products, energy, adjoint ------------------------------------------------------------
-    sweep_forward<T, LOSS>(p, M, Tg, lane);
+    sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
     T e_part = (T)0;
-    for (int s = lane; s < p.n_scalar; s += 64) {
+    for (int s = lane; s < p.n_scalar; s += NT) {
         e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
         A[p.mapping[s]] = a.lin[s] / a.q_scaler[s];
     }
     __syncthreads();
-    sweep_reverse<T, false>(p, M, A, nullptr, nullptr, lane);
+    sweep_reverse<T, false, NT>(p, M, A, nullptr, nullptr, tab, lane);
 
     if (!LOSS) {
         // ---- pair derivatives: lane = half * 32 + neighbour ------------------------------------
@@ -288,7 +350,7 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
             if (j < nc) {
                 const T* t = tab + j * E;
                 const T rinv = t[OU + 3];
-                for (int i = h; i < n_basic; i += 2) {
+                for (int i = h; i < n_basic; i += NG) {
                     const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
                               ec = p.basic[i * 4 + 3];
                     const T adj = A[i];
@@ -302,10 +364,19 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
                     wz += ag * (T)ec * xa * yb * t[OZ + max(ec - 1, 0)];
                 }
             }
-            gs += __shfl_xor(gs, 32, 64);
-            wx += __shfl_xor(wx, 32, 64);
-            wy += __shfl_xor(wy, 32, 64);
-            wz += __shfl_xor(wz, 32, 64);
+            // group sums in the order h = 0 .. NG-1
+            {
+                T* gr = gred + (h * 32 + j) * 4;
+                gr[0] = gs; gr[1] = wx; gr[2] = wy; gr[3] = wz;
+            }
+            __syncthreads();
+            if (h == 0) {
+#pragma unroll
+                for (int hh = 1; hh < NG; hh++) {
+                    const T* gr = gred + (hh * 32 + j) * 4;
+                    gs += gr[0]; wx += gr[1]; wy += gr[2]; wz += gr[3];
+                }
+            }
             if (h == 0 && j < nc) {
                 const T* t = tab + j * E;
                 const T rinv = t[OU + 3];
@@ -321,8 +392,9 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
                 vir[6] -= gz * d[0]; vir[7] -= gz * d[1]; vir[8] -= gz * d[2];
             }
         }
+        // only the threads of group 0 (inside wave 0) hold force and virial terms
         fx = wave_sum(fx); fy = wave_sum(fy); fz = wave_sum(fz);
-        double e_atom = (double)wave_sum(e_part);
+        double e_atom = (double)block_sum<T, NT>(e_part, gred, lane);
         double out[10];
         out[0] = e_atom + (double)a.bias[ti];
 #pragma unroll
@@ -339,15 +411,15 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
     // ---- loss gradient ------------------------------------------------------------------------
     if (LOSS) {
         const T cE = a.cE[b];
-        sweep_reverse<T, true>(p, M, Bm, A, Tg, lane);      // linearMtpLoss.h:417-434
+        sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);      // linearMtpLoss.h:417-434
         T* grow = a.gpart + row * a.ngrad;
-        for (int q = lane; q < a.ngrad; q += 64) grow[q] = (T)0;
+        for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
         const int j = lane & 31, h = lane >> 5;
         T* Pm = pq;
         T* Qm = pq + MTP_NC * nmus;
         int* tjs = (int*)(pq + 2 * MTP_NC * nmus);
         T* gacc = pq + 2 * MTP_NC * nmus + MTP_NC;          // [ntypes][nmus][K] for this centre type
-        for (int q = lane; q < a.ntypes * nmus * K; q += 64) gacc[q] = (T)0;
+        for (int q = lane; q < a.ntypes * nmus * K; q += NT) gacc[q] = (T)0;
         for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
             const int nc = min(MTP_NC, nn - c0);
             int nj; bool valid; T d[3];
@@ -360,7 +432,7 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
                 if (j < nc) {
                     const T* t = tab + j * E;
                     const T rinv = t[OU + 3], wu = t[OW + 3];
-                    for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += 2) {
+                    for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += NG) {
                         const int ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2], ec = p.basic[i * 4 + 3];
                         const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
                         const T m = xa * yb * zc;
@@ -372,15 +444,26 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
                         Qv += adj * m * wu;
                     }
                 }
-                Pv += __shfl_xor(Pv, 32, 64);
-                Qv += __shfl_xor(Qv, 32, 64);
-                if (h == 0 && j < nc) { Pm[j * nmus + mu] = Pv; Qm[j * nmus + mu] = Qv; }
+                {
+                    T* gr = gred + (h * 32 + j) * 4;
+                    gr[0] = Pv; gr[1] = Qv;
+                }
+                __syncthreads();
+                if (h == 0) {
+#pragma unroll
+                    for (int hh = 1; hh < NG; hh++) {
+                        const T* gr = gred + (hh * 32 + j) * 4;
+                        Pv += gr[0]; Qv += gr[1];
+                    }
+                    if (j < nc) { Pm[j * nmus + mu] = Pv; Qm[j * nmus + mu] = Qv; }
+                }
+                __syncthreads();
             }
             // tj of each neighbour of the chunk, for the accumulation below
             if (h == 0 && j < nc) tjs[j] = valid ? types[nj] : -1;
             __syncthreads();
             // lanes <- (mu, k): sequential over neighbours keeps the sum order fixed
-            for (int q = lane; q < nmus * K; q += 64) {
+            for (int q = lane; q < nmus * K; q += NT) {
                 const int mu = q / K, k = q - mu * K;
                 for (int jn = 0; jn < nc; jn++) {
                     const int tj = tjs[jn];
@@ -391,10 +474,10 @@ __global__ void __launch_bounds__(64) mtp_atom_kernel(const MtpArgs<T> a)
             }
         }
         __syncthreads();
-        for (int q = lane; q < a.ntypes * nmus * K; q += 64)
+        for (int q = lane; q < a.ntypes * nmus * K; q += NT)
             grow[(size_t)ti * a.ntypes * nmus * K + q] = gacc[q];
         // linear coefficients and bias: linearMtpLoss.h:539-554
-        for (int s = lane; s < p.n_scalar; s += 64)
+        for (int s = lane; s < p.n_scalar; s += NT)
             grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
         if (lane == 0) grow[ncoef + p.n_scalar + ti] = cE;
     }
@@ -527,53 +610,78 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
         A2P_REQUIRE(!seen[mapping[s]], A2P_ERR_INVALID, "mtp plan: alpha_moment_mapping repeats a moment");
         seen[mapping[s]] = 1;
     }
-    // forward gather lists
-    std::vector<std::vector<int>> terms_of(n_moms);          // product entries per dst, file order
-    for (int e = 0; e < n_times; e++) terms_of[times[e * 4 + 3]].push_back(e);
-    std::vector<int> f_level(n_levels + 1, 0), f_dst, f_begin(1, 0), f_m0, f_m1;
-    std::vector<double> f_mult;
-    for (int l = 1; l <= n_levels; l++) {
-        std::vector<int> dsts;
-        for (int m = n_basic; m < n_moms; m++)
-            if (level[m] == l && !terms_of[m].empty()) dsts.push_back(m);
-        std::stable_sort(dsts.begin(), dsts.end(),
-                         [&](int x, int y) { return terms_of[x].size() > terms_of[y].size(); });
-        for (int m : dsts) {
-            f_dst.push_back(m);
-            for (int e : terms_of[m]) {
-                f_m0.push_back(times[e * 4]);
-                f_m1.push_back(times[e * 4 + 1]);
-                f_mult.push_back((double)times[e * 4 + 2]);
+    A2P_REQUIRE(n_moms < 65536, A2P_ERR_INVALID, "mtp plan: more than 65535 moments");
+    // Interleaved gather lists (see mtp_plan.h).  `lists[m]` holds the packed terms of moment m.
+    struct Ell {
+        std::vector<int> level, lend, multi, slot, lead, gbase, gdepth;
+        std::vector<int2> terms;
+        int max_slots = 0;
+    };
+    auto build_ell = [&](const std::vector<std::vector<int2>>& lists, const std::vector<std::vector<int>>& by_level) {
+        Ell e;
+        for (const auto& members : by_level) {
+            const int first_slot = (int)e.slot.size();
+            e.level.push_back(first_slot);
+            std::vector<int> ms = members;
+            std::stable_sort(ms.begin(), ms.end(),
+                             [&](int x, int y) { return lists[x].size() > lists[y].size(); });
+            // slots of the level: (moment, first term, term count), pieces of a list adjacent
+            struct Piece { int m, t0, n, lead; };
+            std::vector<Piece> pieces;
+            int multi = 0;
+            for (int m : ms) {
+                const int n = (int)lists[m].size();
+                const int np = (n + MTP_SLOT_CAP - 1) / MTP_SLOT_CAP;
+                if (np > 1) multi = 1;
+                for (int q = 0; q < np; q++)
+                    pieces.push_back({m, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, n - q * MTP_SLOT_CAP), q == 0 ? np : 0});
             }
-            f_begin.push_back((int)f_m0.size());
+            e.multi.push_back(multi);
+            for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
+                const size_t g1 = std::min(pieces.size(), g0 + 64);
+                int depth = 0;
+                for (size_t q = g0; q < g1; q++) depth = std::max(depth, pieces[q].n);
+                e.gbase.push_back((int)e.terms.size());
+                e.gdepth.push_back(depth);
+                e.terms.resize(e.terms.size() + (size_t)depth * 64, make_int2(0, 0));
+                for (size_t q = g0; q < g1; q++) {
+                    const Piece& pc = pieces[q];
+                    for (int k = 0; k < pc.n; k++)
+                        e.terms[e.gbase.back() + (size_t)k * 64 + (q - g0)] = lists[pc.m][pc.t0 + k];
+                    e.slot.push_back(pc.m);
+                    e.lead.push_back(pc.lead);
+                }
+            }
+            e.lend.push_back((int)e.slot.size());
+            e.max_slots = std::max(e.max_slots, (int)e.slot.size() - first_slot);
+            while (e.slot.size() % 64) { e.slot.push_back(-1); e.lead.push_back(0); }
         }
-        f_level[l] = (int)f_dst.size();
+        e.level.push_back((int)e.slot.size());
+        e.lend.push_back((int)e.slot.size());
+        e.multi.push_back(0);
+        if (e.terms.empty()) e.terms.push_back(make_int2(0, 0));
+        if (e.gbase.empty()) { e.gbase.push_back(0); e.gdepth.push_back(0); }
+        if (e.slot.empty()) { e.slot.push_back(-1); e.lead.push_back(0); }
+        return e;
+    };
+    // forward: terms per destination in file order; level l >= 1 at index l - 1
+    std::vector<std::vector<int2>> fl(n_moms), rl(n_moms);
+    for (int e = 0; e < n_times; e++) {
+        const int* q = times + e * 4;
+        fl[q[3]].push_back(make_int2(q[0] | (q[1] << 16), q[2]));
     }
-    // reverse gather lists: terms per source in reverse file order
-    std::vector<std::vector<int>> uses(n_moms);              // encoded 2*e + which
+    std::vector<std::vector<int>> f_by(n_levels), r_by(n_levels);
+    for (int m = n_basic; m < n_moms; m++)
+        if (level[m] >= 1 && !fl[m].empty()) f_by[level[m] - 1].push_back(m);
+    // reverse: terms per source in reverse file order
     for (int e = n_times - 1; e >= 0; e--) {
-        uses[times[e * 4 + 1]].push_back(2 * e + 1);         // adj[m1] += adj[dst] mult M[m0]
-        uses[times[e * 4 + 0]].push_back(2 * e + 0);         // adj[m0] += adj[dst] mult M[m1]
+        const int* q = times + e * 4;
+        rl[q[1]].push_back(make_int2(q[3] | (q[0] << 16), q[2]));     // adj[m1] += adj[dst] mult M[m0]
+        rl[q[0]].push_back(make_int2(q[3] | (q[1] << 16), q[2]));     // adj[m0] += adj[dst] mult M[m1]
     }
-    std::vector<int> r_level(n_levels + 1, 0), r_src, r_begin(1, 0), r_dst, r_other;
-    std::vector<double> r_mult;
-    for (int l = 0; l < n_levels; l++) {
-        std::vector<int> srcs;
-        for (int m = 0; m < n_moms; m++)
-            if (level[m] == l && !uses[m].empty()) srcs.push_back(m);
-        std::stable_sort(srcs.begin(), srcs.end(), [&](int x, int y) { return uses[x].size() > uses[y].size(); });
-        for (int m : srcs) {
-            r_src.push_back(m);
-            for (int code : uses[m]) {
-                const int e = code >> 1, which = code & 1;
-                r_dst.push_back(times[e * 4 + 3]);
-                r_other.push_back(which ? times[e * 4 + 0] : times[e * 4 + 1]);
-                r_mult.push_back((double)times[e * 4 + 2]);
-            }
-            r_begin.push_back((int)r_dst.size());
-        }
-        r_level[l + 1] = (int)r_src.size();
-    }
+    for (int m = 0; m < n_moms; m++)
+        if (level[m] < n_levels && !rl[m].empty()) r_by[level[m]].push_back(m);
+    const Ell F = build_ell(fl, f_by), R = build_ell(rl, r_by);
     std::vector<int> mu_begin(nmus + 1, n_basic);
     for (int i = n_basic - 1; i >= 0; i--) mu_begin[basic[i * 4]] = i;
     for (int m = nmus - 1; m >= 0; m--) mu_begin[m] = std::min(mu_begin[m], mu_begin[m + 1]);
@@ -592,18 +700,22 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     const size_t o_basic = add(basic, sizeof(int) * 4 * n_basic);
     const size_t o_mu = add(mu_begin.data(), sizeof(int) * mu_begin.size());
     const size_t o_map = add(mapping, sizeof(int) * n_scalar);
-    const size_t o_fl = add(f_level.data(), sizeof(int) * f_level.size());
-    const size_t o_fd = add(f_dst.data(), sizeof(int) * f_dst.size());
-    const size_t o_fb = add(f_begin.data(), sizeof(int) * f_begin.size());
-    const size_t o_f0 = add(f_m0.data(), sizeof(int) * f_m0.size());
-    const size_t o_f1 = add(f_m1.data(), sizeof(int) * f_m1.size());
-    const size_t o_fm = add(f_mult.data(), sizeof(double) * f_mult.size());
-    const size_t o_rl = add(r_level.data(), sizeof(int) * r_level.size());
-    const size_t o_rs = add(r_src.data(), sizeof(int) * r_src.size());
-    const size_t o_rb = add(r_begin.data(), sizeof(int) * r_begin.size());
-    const size_t o_rd = add(r_dst.data(), sizeof(int) * r_dst.size());
-    const size_t o_ro = add(r_other.data(), sizeof(int) * r_other.size());
-    const size_t o_rm = add(r_mult.data(), sizeof(double) * r_mult.size());
+    const size_t o_fl = add(F.level.data(), sizeof(int) * F.level.size());
+    const size_t o_fe = add(F.lend.data(), sizeof(int) * F.lend.size());
+    const size_t o_fx = add(F.multi.data(), sizeof(int) * F.multi.size());
+    const size_t o_fd = add(F.slot.data(), sizeof(int) * F.slot.size());
+    const size_t o_fc = add(F.lead.data(), sizeof(int) * F.lead.size());
+    const size_t o_fg = add(F.gbase.data(), sizeof(int) * F.gbase.size());
+    const size_t o_fh = add(F.gdepth.data(), sizeof(int) * F.gdepth.size());
+    const size_t o_ft = add(F.terms.data(), sizeof(int2) * F.terms.size());
+    const size_t o_rl = add(R.level.data(), sizeof(int) * R.level.size());
+    const size_t o_re = add(R.lend.data(), sizeof(int) * R.lend.size());
+    const size_t o_rx = add(R.multi.data(), sizeof(int) * R.multi.size());
+    const size_t o_rs = add(R.slot.data(), sizeof(int) * R.slot.size());
+    const size_t o_rc = add(R.lead.data(), sizeof(int) * R.lead.size());
+    const size_t o_rg = add(R.gbase.data(), sizeof(int) * R.gbase.size());
+    const size_t o_rh = add(R.gdepth.data(), sizeof(int) * R.gdepth.size());
+    const size_t o_rt = add(R.terms.data(), sizeof(int2) * R.terms.size());
     std::vector<unsigned char> host(total + 16, 0);
     for (auto& s : segs)
         if (s.bytes) std::memcpy(host.data() + s.off, s.src, s.bytes);
@@ -617,12 +729,17 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.nmus = nmus; d.kmax = kmax; d.n_levels = n_levels;
     d.basic = (const int*)(base + o_basic); d.mu_begin = (const int*)(base + o_mu);
     d.mapping = (const int*)(base + o_map);
-    d.f_level = (const int*)(base + o_fl); d.f_dst = (const int*)(base + o_fd);
-    d.f_begin = (const int*)(base + o_fb); d.f_m0 = (const int*)(base + o_f0);
-    d.f_m1 = (const int*)(base + o_f1); d.f_mult = (const double*)(base + o_fm);
-    d.r_level = (const int*)(base + o_rl); d.r_src = (const int*)(base + o_rs);
-    d.r_begin = (const int*)(base + o_rb); d.r_dst = (const int*)(base + o_rd);
-    d.r_other = (const int*)(base + o_ro); d.r_mult = (const double*)(base + o_rm);
+    d.f_level = (const int*)(base + o_fl); d.f_lend = (const int*)(base + o_fe);
+    d.f_multi = (const int*)(base + o_fx);
+    d.f_dst = (const int*)(base + o_fd); d.f_lead = (const int*)(base + o_fc);
+    d.f_gbase = (const int*)(base + o_fg); d.f_gdepth = (const int*)(base + o_fh);
+    d.f_terms = (const int2*)(base + o_ft);
+    d.r_level = (const int*)(base + o_rl); d.r_lend = (const int*)(base + o_re);
+    d.r_multi = (const int*)(base + o_rx);
+    d.r_src = (const int*)(base + o_rs); d.r_lead = (const int*)(base + o_rc);
+    d.r_gbase = (const int*)(base + o_rg); d.r_gdepth = (const int*)(base + o_rh);
+    d.r_terms = (const int2*)(base + o_rt);
+    d.max_level_slots = std::max(F.max_slots, R.max_slots);
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         g_plans.insert(plan);
@@ -651,7 +768,9 @@ int table_entries(const MtpPlanDevice& p, int K, bool loss)
 template <typename T>
 size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K)
 {
-    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + (size_t)MTP_NC * E;
+    // the neighbour table and the group sums double as the sweeps' partial-sum arrays
+    const size_t tabs = std::max((size_t)MTP_NC * E + (size_t)(256 / 32) * 32 * 4, (size_t)p.max_level_slots * (loss ? 2 : 1));
+    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs;
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
     return n * sizeof(T) + 64;
@@ -692,12 +811,13 @@ int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
     const size_t lds = lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K);
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
                 "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
-    auto kern = mtp_atom_kernel<T, LOSS>;
+    const bool wide = a.p.n_moms >= 1000;      // enough moments to keep 256 threads busy
+    auto kern = wide ? mtp_atom_kernel<T, LOSS, 256> : mtp_atom_kernel<T, LOSS, 64>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
     prof_begin(LOSS ? "mtp_loss_bwd_kernel" : "mtp_efv_kernel", stream);
-    hipLaunchKernelGGL(kern, dim3(a.P, a.B), dim3(64), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.P, a.B), dim3(wide ? 256 : 64), lds, stream, a);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;

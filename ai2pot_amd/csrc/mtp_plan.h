@@ -13,9 +13,12 @@
 // The plan is valid only if no product is read before its last contribution in file order;
 // plan creation verifies this.
 #pragma once
+#include <hip/hip_runtime.h>
 #include <vector>
 
 namespace a2p {
+
+constexpr int MTP_SLOT_CAP = 16;
 
 struct MtpPlanDevice {
     // sizes
@@ -25,21 +28,33 @@ struct MtpPlanDevice {
     const int* basic;          // [n_basic*4]  (mu, a, b, c)
     const int* mu_begin;       // [nmus+1]     basics are grouped by mu: run of each mu
     const int* mapping;        // [n_scalar]
-    // forward gather: level l covers dst slots [f_level[l], f_level[l+1])
+    // forward gather.  A slot holds up to MTP_SLOT_CAP terms of one destination moment; a longer
+    // list is cut into consecutive slots (pieces) whose partial sums are added in slot order, so
+    // that no lane walks a long list alone.  Slots are grouped 64 at a time; level l covers slots
+    // [f_level[l], f_lend[l]) and starts at a multiple of 64.  The terms of a group are stored
+    // interleaved and padded with zero terms to the group's depth: term k of slot s is
+    // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
+    // a group read consecutive words and share the trip count.  A term packs x = m0 | m1 << 16,
+    // y = multiplicity.
     const int* f_level;        // [n_levels+1]
-    const int* f_dst;          // [n_fdst]
-    const int* f_begin;        // [n_fdst+1] -> terms
-    const int* f_m0;           // [n_times]
-    const int* f_m1;           // [n_times]
-    const double* f_mult;      // [n_times]
-    // reverse gather: sources by level, level l covers [r_level[l], r_level[l+1]),
-    // processed from the last level (deepest factors' consumers first) to level 0
-    const int* r_level;        // [n_levels+1]  index l = level of the SOURCE moment
-    const int* r_src;          // [n_rsrc]
-    const int* r_begin;        // [n_rsrc+1]
-    const int* r_dst;          // [2*n_times]
-    const int* r_other;        // [2*n_times]
-    const double* r_mult;      // [2*n_times]
+    const int* f_lend;         // [n_levels+1]
+    const int* f_multi;        // [n_levels]   1 when the level has a list cut into pieces
+    const int* f_dst;          // [n_fslots]   destination (-1 in padding slots)
+    const int* f_lead;         // [n_fslots]   number of pieces if the slot is the first of its list, else 0
+    const int* f_gbase;        // [n_fslots/64]
+    const int* f_gdepth;       // [n_fslots/64]
+    const int2* f_terms;
+    // reverse gather, same layout: sources by level (index l = level of the SOURCE moment),
+    // processed from the last level to level 0; a term packs x = dst | other << 16, y = mult
+    const int* r_level;        // [n_levels+1]
+    const int* r_lend;         // [n_levels+1]
+    const int* r_multi;        // [n_levels]
+    const int* r_src;          // [n_rslots]
+    const int* r_lead;         // [n_rslots]
+    const int* r_gbase;        // [n_rslots/64]
+    const int* r_gdepth;       // [n_rslots/64]
+    const int2* r_terms;
+    int max_level_slots;       // most slots of any level (forward or reverse)
 };
 
 struct MtpPlan {
