@@ -54,6 +54,7 @@ struct MtpArgs {
     const T* dVs;      // [B, 9]     2 v_w / (9N) (V - V_dft)
     T* gpart;          // [B, P, ngrad] per-atom gradient rows (ngrad = ncoef + n_scalar + ntypes)
     int ngrad;
+    int lds_basic_off;  // byte offset of the packed basic-moment table in LDS
 };
 
 __device__ __forceinline__ float sqrt_t(float x) { return sqrtf(x); }
@@ -285,6 +286,11 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     const int* first = a.bfirstneigh + row * a.U;
     const T* rcs = a.brcs + row * a.U * 3;
 
+    // (mu, a, b, c) of every basic moment, one byte each, behind everything else in LDS
+    unsigned* bas = (unsigned*)(smem_raw + a.lds_basic_off);
+    for (int i = lane; i < n_basic; i += NT)
+        bas[i] = (unsigned)p.basic[i * 4] | ((unsigned)p.basic[i * 4 + 1] << 8) |
+                 ((unsigned)p.basic[i * 4 + 2] << 16) | ((unsigned)p.basic[i * 4 + 3] << 24);
     for (int i = lane; i < n_moms; i += NT) {
         M[i] = (T)0; A[i] = (T)0;
         if (LOSS) { Tg[i] = (T)0; Bm[i] = (T)0; }
@@ -298,8 +304,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         build_table<T, LOSS>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
         __syncthreads();
         for (int i = lane; i < n_basic; i += NT) {
-            const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
-                      ec = p.basic[i * 4 + 3];
+            const unsigned bw = bas[i];
+            const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
             const T kk = (T)(ea + eb + ec);
             T acc = (T)0, tacc = (T)0;
             for (int j = 0; j < nc; j++) {
@@ -350,9 +356,10 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
             if (j < nc) {
                 const T* t = tab + j * E;
                 const T rinv = t[OU + 3];
+#pragma unroll 4
                 for (int i = h; i < n_basic; i += NG) {
-                    const int mu = p.basic[i * 4], ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2],
-                              ec = p.basic[i * 4 + 3];
+                    const unsigned bw = bas[i];
+                    const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
                     const T adj = A[i];
                     const T g = t[OG + mu], dg = t[ODG + mu];
                     const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
@@ -433,7 +440,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                     const T* t = tab + j * E;
                     const T rinv = t[OU + 3], wu = t[OW + 3];
                     for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += NG) {
-                        const int ea = p.basic[i * 4 + 1], eb = p.basic[i * 4 + 2], ec = p.basic[i * 4 + 3];
+                        const unsigned bw = bas[i];
+                        const int ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
                         const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
                         const T m = xa * yb * zc;
                         const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
@@ -773,7 +781,7 @@ size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K)
     size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs;
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
-    return n * sizeof(T) + 64;
+    return n * sizeof(T) + 64;      // the packed basic-moment table (4 n_basic bytes) follows
 }
 
 template <typename T>
@@ -808,10 +816,12 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
 template <typename T, bool LOSS>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
-    const size_t lds = lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K);
+    const size_t lds_main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K) + 15) / 16 * 16;
+    const size_t lds = lds_main + (size_t)a.p.n_basic * sizeof(unsigned);
+    const_cast<MtpArgs<T>&>(a).lds_basic_off = (int)lds_main;
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
                 "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
-    const bool wide = a.p.n_moms >= 1000;      // enough moments to keep 256 threads busy
+    const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
     auto kern = wide ? mtp_atom_kernel<T, LOSS, 256> : mtp_atom_kernel<T, LOSS, 64>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
