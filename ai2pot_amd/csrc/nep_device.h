@@ -151,6 +151,49 @@ __device__ __forceinline__ void blm_grad_dot(T x, T y, T z, const T (&a)[LC * LC
     }
 }
 
+// d[lm] = w . grad b_lm(u): the directional derivative of every homogeneous polynomial b_lm along
+// w, evaluated on the unit sphere (the same gradients as blm_grad_dot, taken apart per lm)
+template <typename T, int LC>
+__device__ __forceinline__ void blm_dir_derivs(T x, T y, T z, T wx, T wy, T wz, T (&d)[LC * LC + 2 * LC])
+{
+    const T x2 = x * x, y2 = y * y, z2 = z * z;
+    const T xy = x * y, xz = x * z, yz = y * z;
+    if (LC >= 1) { d[0] = wz; d[1] = wx; d[2] = wy; }
+    if (LC >= 2) {
+        d[3] = (T)-2 * x * wx + (T)-2 * y * wy + (T)4 * z * wz;
+        d[4] = z * wx + x * wz;
+        d[5] = z * wy + y * wz;
+        d[6] = (T)2 * x * wx - (T)2 * y * wy;
+        d[7] = (T)2 * y * wx + (T)2 * x * wy;
+    }
+    if (LC >= 3) {
+        const T c = (T)5 * z2 - (T)1;
+        d[8] = (T)-6 * xz * wx + (T)-6 * yz * wy + ((T)9 * z2 - (T)3) * wz;
+        d[9] = (c - (T)2 * x2) * wx + (T)-2 * xy * wy + (T)8 * xz * wz;
+        d[10] = (T)-2 * xy * wx + (c - (T)2 * y2) * wy + (T)8 * yz * wz;
+        d[11] = (T)2 * xz * wx + (T)-2 * yz * wy + (x2 - y2) * wz;
+        d[12] = (T)2 * yz * wx + (T)2 * xz * wy + (T)2 * xy * wz;
+        d[13] = (T)3 * (x2 - y2) * wx + (T)-6 * xy * wy;
+        d[14] = (T)6 * xy * wx + (T)3 * (x2 - y2) * wy;
+    }
+    if (LC >= 4) {
+        const T z3 = z2 * z, x3 = x2 * x, y3 = y2 * y;
+        const T c73 = (T)7 * z3 - (T)3 * z;
+        d[15] = ((T)-60 * x * z2 + (T)12 * x) * wx + ((T)-60 * y * z2 + (T)12 * y) * wy +
+                ((T)80 * z3 - (T)48 * z) * wz;
+        d[16] = ((T)-6 * x2 * z + c73) * wx + ((T)-6 * xy * z) * wy + ((T)15 * x * z2 - (T)3 * x) * wz;
+        d[17] = ((T)-6 * xy * z) * wx + ((T)-6 * y2 * z + c73) * wy + ((T)15 * y * z2 - (T)3 * y) * wz;
+        d[18] = ((T)-2 * x3 + (T)2 * x * y2 + (T)14 * x * z2 - (T)2 * x) * wx +
+                ((T)-2 * x2 * y + (T)2 * y3 - (T)14 * y * z2 + (T)2 * y) * wy + ((T)12 * z * (x2 - y2)) * wz;
+        d[19] = ((T)-4 * x2 * y + (T)14 * y * z2 - (T)2 * y) * wx +
+                ((T)-4 * x * y2 + (T)14 * x * z2 - (T)2 * x) * wy + ((T)24 * xy * z) * wz;
+        d[20] = ((T)3 * (x2 - y2) * z) * wx + ((T)-6 * xy * z) * wy + ((x2 - (T)3 * y2) * x) * wz;
+        d[21] = ((T)6 * xy * z) * wx + ((T)3 * (x2 - y2) * z) * wy + (((T)3 * x2 - y2) * y) * wz;
+        d[22] = ((T)4 * x3 - (T)12 * x * y2) * wx + ((T)4 * y3 - (T)12 * x2 * y) * wy;
+        d[23] = ((T)12 * x2 * y - (T)4 * y3) * wx + ((T)4 * x3 - (T)12 * x * y2) * wy;
+    }
+}
+
 }  // namespace nepdev
 
 // The staged kernel for the common model shape (nep_staged.hip).  staged_supported() tells

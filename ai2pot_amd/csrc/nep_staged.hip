@@ -144,7 +144,7 @@ __device__ __forceinline__ void staged_classify(const StagedLds<T>& L, int tid, 
     for (int s = 0; s < FCH; s++) {
         const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
         const T r = sqrt_t(x * x + y * y + z * z);
-        if (r <= ra) mA |= 1u << s;
+        if (r <= ra && r <= rr) mA |= 1u << s;     // nepBasis.h:106, 135: beyond the radial cutoff a neighbour is skipped
         if (r <= rr) mR |= 1u << s;
         if (x < (T)1.0e17) mV |= 1u << s;
     }

@@ -165,6 +165,121 @@ def nepToDescriptorsOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, c
     return [d]
 
 
+def nep_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size,
+                  n_radial_basis, n_angular_basis, l_max, coeffs, w0, b0, w1, type_bias, binum, bilist,
+                  bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax_radial, rmax_angular, q_scaler,
+                  want_grad=True, validate=True):
+    """Forward and (optionally) the per-structure parameter gradients of the NEP training loss in one
+    call.  Returns a dict with bloss[B], rmse[3], energy, force, virial and, with want_grad,
+    dcoeffs[B, .], dw0[B, .], db0[B, .], dw1[B, .], dbias[B, ntypes] (flattened parameter layouts)."""
+    _req(int(nghost) == 0, "the loss operator requires nghost == 0, as the reference does")
+    _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
+         "brcs must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = brcs.dtype, brcs.device
+    _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
+    _req(brcs.is_contiguous(), "brcs must be contiguous")
+    for name, t in (("coeffs", coeffs), ("w0", w0), ("b0", b0), ("w1", w1), ("type_bias", type_bias),
+                    ("q_scaler", q_scaler)):
+        _check_float(name, t, dtype, device)
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh), ("btypes", btypes)):
+        _check_int(name, t, device)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, 0)
+    ntypes = int(type_map.numel())
+    _req(ntypes > 0, "type_map is empty")
+    _req(0 <= l_max <= 4, "l_max must be in [0, 4]")
+    H = w1.numel() // ntypes
+    D = n_radial_basis + n_angular_basis * l_max if l_max > 0 else n_radial_basis
+    _req(w0.numel() == ntypes * H * D and b0.numel() == ntypes * H and type_bias.numel() == ntypes and
+         q_scaler.numel() == D, "w0 / b0 / type_bias / q_scaler size mismatch")
+    _req(coeffs.numel() == ntypes * ntypes * (n_radial_basis + n_angular_basis) * chebyshev_size,
+         "coeffs size mismatch")
+    for name, t, n_expected in (("betot_dft", betot_dft, B), ("bforce_dft", bforce_dft, B * P * 3),
+                                ("bvirial_dft", bvirial_dft, B * 9)):
+        _check_float(name, t, dtype, device)
+        _req(t.numel() == n_expected, "%s has %d elements, expected %d" % (name, t.numel(), n_expected))
+    if validate:
+        _validate_batch(binum, bnumneigh, U, P)
+    z = lambda *s_: torch.zeros(s_, dtype=dtype, device=device)
+    out = dict(bloss=z(B), rmse=z(3), energy=z(B), force=z(B, P, 3), virial=z(B, 9))
+    if want_grad:
+        out.update(dcoeffs=z(B, coeffs.numel()), dw0=z(B, w0.numel()), db0=z(B, b0.numel()),
+                   dw1=z(B, w1.numel()), dbias=z(B, ntypes))
+    L = _lib.lib()
+    fn = L.a2p_nep_loss_f32 if dtype == torch.float32 else L.a2p_nep_loss_f64
+    with torch.cuda.device(device):
+        rc = fn(_c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+                _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_int(n_radial_basis),
+                _c.c_int(n_angular_basis), _c.c_int(l_max), _c.c_int(H), _c.c_int(ntypes), _ptr(coeffs), _ptr(w0),
+                _ptr(b0), _ptr(w1), _ptr(type_bias), _ptr(q_scaler), _c.c_double(rmax_radial),
+                _c.c_double(rmax_angular), _c.c_int(B), _c.c_int(P), _c.c_int(U), _ptr(binum), _ptr(bilist),
+                _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(out["bloss"]), _ptr(out["rmse"]),
+                _ptr(out["energy"]), _ptr(out["force"]), _ptr(out["virial"]), _ptr(out.get("dcoeffs")),
+                _ptr(out.get("dw0")), _ptr(out.get("db0")), _ptr(out.get("dw1")), _ptr(out.get("dbias")),
+                _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return out
+
+
+class _NepToLoss(torch.autograd.Function):
+    """Autograd wrapper with the reference's contract (nepOp.cc:2359-2960): gradients flow to coeffs,
+    w0, b0, w1 and type_bias only, as grad_output[B] @ dloss/dtheta."""
+
+    @staticmethod
+    def forward(ctx, coeffs, w0, b0, w1, type_bias, args):
+        (e_w, f_w, v_w, e_dft, f_dft, v_dft, K, n_r, n_a, l_max, binum, bilist, bnumneigh, bfirstneigh, brcs,
+         btypes, type_map, nghost, rr, ra, q_scaler, validate) = args
+        params = (coeffs, w0, b0, w1, type_bias)
+        need = any(p.requires_grad for p in params)
+        r = nep_loss_step(e_w, f_w, v_w, e_dft, f_dft, v_dft, K, n_r, n_a, l_max, coeffs.detach(), w0.detach(),
+                          b0.detach(), w1.detach(), type_bias.detach(), binum, bilist, bnumneigh, bfirstneigh,
+                          brcs, btypes, type_map, nghost, rr, ra, q_scaler, want_grad=need, validate=validate)
+        if need:
+            # unlike the reference, which recomputes E/F/V in backward, the gradients are produced by
+            # the same call and kept
+            ctx.save_for_backward(r["dcoeffs"], r["dw0"], r["db0"], r["dw1"], r["dbias"])
+        ctx.shapes = tuple(p.shape for p in params)
+        ctx.have = need
+        rm = r["rmse"]
+        return r["bloss"], rm[0:1].clone(), rm[1:2].clone(), rm[2:3].clone()
+
+    @staticmethod
+    def backward(ctx, gl, ge, gf, gv):
+        if not ctx.have:
+            return None, None, None, None, None, None
+        return tuple(torch.matmul(gl, g).reshape(sh) for g, sh in zip(ctx.saved_tensors, ctx.shapes)) + (None,)
+
+
+def nepToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size,
+                n_radial_basis, n_angular_basis, l_max, coeffs, w0, b0, w1, type_bias, binum, bilist, bnumneigh,
+                bfirstneigh, brcs, btypes, type_map, nghost, rmax_radial, rmax_angular, q_scaler, zbl_rmax=0.0,
+                zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
+    """[bloss[B], e_rmse[1], f_rmse[1], v_rmse[1]], differentiable w.r.t. coeffs, w0, b0, w1 and
+    type_bias; nep_bind.cc:205-276, nepOp.cc:2359-2960."""
+    _no_zbl(zbl_rmax)
+    args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, n_radial_basis,
+            n_angular_basis, l_max, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+            rmax_radial, rmax_angular, q_scaler, validate)
+    return list(_NepToLoss.apply(coeffs, w0, b0, w1, type_bias, args))
+
+
+def nepToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, n_radial_basis, n_angular_basis,
+                  l_max, coeffs, w0, b0, w1, type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                  type_map, nghost, rmax_radial, rmax_angular, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None,
+                  zbl_dks=None, validate=True):
+    """[bloss[B], e_rmse[1], f_rmse[1]]: the loss without the virial term; nep_bind.cc:136-203,
+    nepOp.cc:2962-3484 (nepLoss.h:139-166 is nepLoss.h:170-209 with v_weight = 0)."""
+    _no_zbl(zbl_rmax)
+    B = int(binum.numel())
+    v0 = torch.zeros((B, 9), dtype=brcs.dtype, device=brcs.device)
+    args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v0, chebyshev_size, n_radial_basis, n_angular_basis,
+            l_max, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax_radial,
+            rmax_angular, q_scaler, validate)
+    return list(_NepToLoss.apply(coeffs, w0, b0, w1, type_bias, args))[:3]
+
+
 # --------------------------------------------------------------------------------------------
 # linear MTP  (source/descriptor/mtpr/bind/mtpr_bind.cc:30-457)
 # --------------------------------------------------------------------------------------------

@@ -167,6 +167,39 @@ int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weig
                      float* dbias, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * NEP training loss, forward and analytic backward -- replaces the compute of
+ * torch.ops.nep.nepToLossOp and torch.ops.nep.nepToEFLossOp
+ * (source/descriptor/nep/bind/nep_bind.cc:136-276; src/nepOp.cc:2359-3484;
+ *  include/nepLoss.h:139-209 loss, :213-745 and :752-1298 backward;
+ *  include/nepLoss_cpu_launcher.h:31-163, 167-330 launchers, :333-406 RMSEs).
+ * Per structure  loss = e_w/N (E-E0)^2 + f_w/(3N) sum |F-F0|^2 + v_w/(9N) sum (V-V0)^2;
+ * nepToEFLossOp is the same call with v_weight = 0 (v_dft still has to point at B*9 values).
+ * Outputs (device): bloss[B]; rmse[3] = (E per atom, F per component, V per component: the
+ * virial one is not divided by the atom count, unlike the MTP operator); the model's
+ * etot[B], force[B,P,3], virial[B,9]; and per-structure gradients dcoeffs[B, ntypes^2 (n_r+n_a) K],
+ * dw0[B, ntypes H D], db0[B, ntypes H], dw1[B, ntypes H], dbias[B, ntypes] (any may be NULL;
+ * all NULL skips the backward kernels).  The operator's backward multiplies them by
+ * grad_output[B] (nepOp.cc:2901-2960).  nghost is 0, as in the reference's loss launchers,
+ * which index forces with stride natoms_pad.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nep_loss_f64(double e_weight, double f_weight, double v_weight, const double* e_dft, const double* f_dft,
+                     const double* v_dft, int chebyshev_size, int n_radial_basis, int n_angular_basis, int l_max,
+                     int num_neurons, int ntypes, const double* coeffs, const double* w0, const double* b0,
+                     const double* w1, const double* type_bias, const double* q_scaler, double rmax_radial,
+                     double rmax_angular, int batch, int natoms_pad, int umax, const int* binum, const int* bilist,
+                     const int* bnumneigh, const int* bfirstneigh, const double* brcs, const int* btypes,
+                     double* bloss, double* rmse, double* etot, double* force, double* virial, double* dcoeffs,
+                     double* dw0, double* db0, double* dw1, double* dbias, void* stream);
+int a2p_nep_loss_f32(double e_weight, double f_weight, double v_weight, const float* e_dft, const float* f_dft,
+                     const float* v_dft, int chebyshev_size, int n_radial_basis, int n_angular_basis, int l_max,
+                     int num_neurons, int ntypes, const float* coeffs, const float* w0, const float* b0,
+                     const float* w1, const float* type_bias, const float* q_scaler, double rmax_radial,
+                     double rmax_angular, int batch, int natoms_pad, int umax, const int* binum, const int* bilist,
+                     const int* bnumneigh, const int* bfirstneigh, const float* brcs, const int* btypes,
+                     float* bloss, float* rmse, float* etot, float* force, float* virial, float* dcoeffs,
+                     float* dw0, float* db0, float* dw1, float* dbias, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Short-range force / virial from per-pair derivatives -- replaces the compute of
  * torch.ops.fvt.ForceSrOp and torch.ops.fvt.VirialSrOp, forward and backward
  * (source/fvt/bind/fvt_sr_op_bind.cc:9-46; src/force_sr_op.cc:11-179, src/virial_sr_op.cc:10-164

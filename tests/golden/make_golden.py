@@ -103,6 +103,39 @@ def mtp_cases():
     print("mtp.npz")
 
 
+def nep_loss_cases():
+    """Two small structures, two species: the reference's loss forward + backward (fp64)."""
+    out = {}
+    lists = []
+    for i, n in enumerate((40, 27)):
+        lat, pos = synth.random_packed(n, [9.0 + 0.2 * i, 9.5, 10.0], 2.0, 5 + 3 * i)
+        lists.append(oracle.ref_nblist(lat, synth.rng_randint(6 + 3 * i, n, 2), pos, 5.0, 80))
+    nb = synth.pack_batch(lists)
+    w = max(int(nb["bnumneigh"].max()), 1)
+    nb["bfirstneigh"] = np.ascontiguousarray(nb["bfirstneigh"][:, :, :w])
+    nb["brcs"] = np.ascontiguousarray(nb["brcs"][:, :, :w])
+    B, P = nb["bilist"].shape
+    m = synth.nep_model(ntypes=2, seed=905, rmax_radial=5.0, rmax_angular=3.5, num_neurons=7)
+    m["q_scaler"] = np.linspace(0.7, 1.4, m["q_scaler"].size)
+    labels = dict(energy=synth.rng_normal(55, B, -3.0, 1.0), force=synth.rng_normal(56, B * P * 3).reshape(B, P, 3),
+                  virial=synth.rng_normal(57, B * 9, 0.0, 0.5).reshape(B, 9))
+    for k in ("binum", "bilist", "bnumneigh", "bfirstneigh", "brcs", "btypes"):
+        out["in_" + k] = nb[k]
+    for k in ("coeffs", "w0", "b0", "w1", "type_bias", "q_scaler", "type_map"):
+        out["model_" + k] = np.asarray(m[k])
+    out["model_sizes"] = np.array([m["chebyshev_size"], m["n_radial_basis"], m["n_angular_basis"], m["l_max"]])
+    out["model_cutoffs"] = np.array([m["rmax_radial"], m["rmax_angular"]])
+    for k, v in labels.items():
+        out["label_" + k] = v
+    for tag, wts in (("efv", (1.0, 0.7, 0.3)), ("ef", (1.0, 0.7, 0.0))):
+        r = oracle.ref_nep_loss_step(m, nb, wts, labels)
+        out[tag + "/weights"] = np.array(wts)
+        for k, v in r.items():
+            out[tag + "/" + k] = v
+    np.savez_compressed(os.path.join(HERE, "nep_loss.npz"), **out)
+    print("nep_loss.npz")
+
+
 def fvt_cases():
     rng = np.random.default_rng(0)
     inum, U, ng = 10, 6, 3
@@ -124,4 +157,5 @@ if __name__ == "__main__":
     nblist_cases()
     nep_cases()
     mtp_cases()
+    nep_loss_cases()
     fvt_cases()
