@@ -1,8 +1,10 @@
 // libnep_bind.so -- registers torch.ops.nep.* with the reference's schemas
 // (source/descriptor/nep/bind/nep_bind.cc:23-312) on top of libai2pot_hip.so.
-// nepToEFOp / nepToEFVOp / nepToDescriptorsOp run on the GPU; like the reference's, they are
-// inference operators: no gradient flows to any input (src/nepOp.cc:1287-1312).
-// The NEP training-loss operators are registered with their reference signatures and raise.
+// nepToEFOp / nepToEFVOp / nepToDescriptorsOp are inference operators like the reference's: no
+// gradient flows to any input (src/nepOp.cc:1287-1312).  nepToLossOp / nepToEFLossOp return the
+// per-structure loss and the RMSEs and back-propagate grad_output @ dloss/dtheta to coeffs, w0,
+// b0, w1 and type_bias (src/nepOp.cc:2359-3484); the gradients are produced by the forward call
+// and kept, where the reference recomputes E/F/V in backward.
 #include "bind_common.h"
 
 using namespace a2p_bind;
@@ -85,6 +87,85 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
     return {e, f};
 }
 
+struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
+    static variable_list forward(torch::autograd::AutogradContext* ctx, bool with_virial, double e_w, double f_w,
+                                 double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
+                                 const at::Tensor& v_dft_in, int64_t K, int64_t n_r, int64_t n_a, int64_t l_max,
+                                 const at::Tensor& coeffs, const at::Tensor& w0, const at::Tensor& b0,
+                                 const at::Tensor& w1, const at::Tensor& bias, const at::Tensor& binum,
+                                 const at::Tensor& bilist, const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
+                                 const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map,
+                                 int64_t nghost, double rr, double ra, const at::Tensor& q_scaler)
+    {
+        TORCH_CHECK(nghost == 0, "the loss operator requires nghost == 0, as the reference does");
+        Batch s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+        NepModel m = check_model(K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, type_map, brcs);
+        check_device_float(brcs, q_scaler, "q_scaler");
+        TORCH_CHECK(q_scaler.numel() == m.D, "q_scaler must have ", m.D, " elements");
+        a2p_bind::DeviceGuard guard(brcs);
+        auto opt = brcs.options();
+        const int B = s.B, P = s.P;
+        at::Tensor v_dft = with_virial ? v_dft_in : at::zeros({B, 9}, opt);
+        check_device_float(brcs, e_dft, "betot_dft");
+        check_device_float(brcs, f_dft, "bforce_dft");
+        check_device_float(brcs, v_dft, "bvirial_dft");
+        TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
+                    "label tensors must have shapes [B], [B, P, 3], [B, 9]");
+        const bool need = coeffs.requires_grad() || w0.requires_grad() || b0.requires_grad() ||
+                          w1.requires_grad() || bias.requires_grad();
+        at::Tensor bloss = at::zeros({B}, opt), rmse = at::zeros({3}, opt), e = at::zeros({B}, opt),
+                   f = at::zeros({B, P, 3}, opt), v = at::zeros({B, 9}, opt), dc, dw0, db0, dw1, db;
+        if (need) {
+            dc = at::zeros({B, coeffs.numel()}, opt);
+            dw0 = at::zeros({B, w0.numel()}, opt);
+            db0 = at::zeros({B, b0.numel()}, opt);
+            dw1 = at::zeros({B, w1.numel()}, opt);
+            db = at::zeros({B, bias.numel()}, opt);
+        }
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_nep_loss_f64(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
+                                  m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
+                                  B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                  bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
+                                  p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_nep_loss_f32(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
+                                  m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
+                                  B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                  bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
+                                  p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
+        }
+        check_rc(rc);
+        check_device_status(brcs);
+        ctx->saved_data["need"] = need;
+        if (need) ctx->save_for_backward({dc, dw0, db0, dw1, db});
+        ctx->saved_data["shape_c"] = coeffs.sizes().vec();
+        ctx->saved_data["shape_w0"] = w0.sizes().vec();
+        ctx->saved_data["shape_b0"] = b0.sizes().vec();
+        ctx->saved_data["shape_w1"] = w1.sizes().vec();
+        ctx->saved_data["shape_b"] = bias.sizes().vec();
+        if (with_virial)
+            return {bloss, rmse.slice(0, 0, 1).clone(), rmse.slice(0, 1, 2).clone(), rmse.slice(0, 2, 3).clone()};
+        return {bloss, rmse.slice(0, 0, 1).clone(), rmse.slice(0, 1, 2).clone()};
+    }
+
+    static variable_list backward(torch::autograd::AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(27);                   // one slot per forward argument after ctx
+        if (!ctx->saved_data["need"].toBool()) return out;
+        auto saved = ctx->get_saved_variables();
+        at::Tensor gl = grads[0].contiguous();
+        const char* keys[5] = {"shape_c", "shape_w0", "shape_b0", "shape_w1", "shape_b"};
+        for (int i = 0; i < 5; i++)              // coeffs, w0, b0, w1, type_bias are arguments 11..15
+            out[11 + i] = torch::matmul(gl, saved[i]).reshape(ctx->saved_data[keys[i]].toIntVector());
+        return out;
+    }
+};
+
 }  // namespace
 
 TORCH_LIBRARY(nep, m)
@@ -120,8 +201,10 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& type_map, int64_t nghost, double rr, double ra, const at::Tensor& q_scaler,
              double zbl_rmax, double zbl_rmin, const at::Tensor& zbl_cks,
              const at::Tensor& zbl_dks) -> variable_list {
-              TORCH_CHECK(false, "nepToLossOp (NEP training loss) is not implemented in this build");
-              return {};
+              require_no_zbl(zbl_rmax);
+              return NepLossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, K, n_r, n_a, l_max, coeffs, w0,
+                                            b0, w1, bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                                            type_map, nghost, rr, ra, q_scaler);
           });
     m.def("nepToEFLossOp",
           [](double e_w, double f_w, const at::Tensor& e_dft, const at::Tensor& f_dft, int64_t K, int64_t n_r,
@@ -131,8 +214,10 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rr, double ra,
              const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin, const at::Tensor& zbl_cks,
              const at::Tensor& zbl_dks) -> variable_list {
-              TORCH_CHECK(false, "nepToEFLossOp (NEP training loss) is not implemented in this build");
-              return {};
+              require_no_zbl(zbl_rmax);
+              return NepLossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft, at::zeros({(int64_t)binum.numel(), 9}, brcs.options()),
+                                            K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist, bnumneigh,
+                                            bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
           });
     m.def("nepToDescriptorsOp",
           [](int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const at::Tensor& coeffs, const at::Tensor& binum,

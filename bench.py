@@ -281,6 +281,57 @@ def run_mtp(args, cfg):
     return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f64"
 
 
+def run_nep_train(args):
+    """NEP training step (the second model family's counterpart of configuration 4): the 64 x 128-atom
+    structures of that configuration, fp32 (the reference trains NEP in single precision), loss forward
+    + analytic gradient w.r.t. all parameters."""
+    import torch
+    from ai2pot_amd import _lib, nblist, ops, synth
+    dev = torch.device("cuda:0")
+    rho = synth.rng_uniform(1005, 64, 0.03, 0.05)
+    lists = []
+    for b in range(64):
+        Lb = (128.0 / rho[b]) ** (1.0 / 3.0)
+        lat, pos = synth.random_packed(128, [Lb, Lb, Lb], 2.0, 11005 + b)
+        ty = synth.rng_randint(21005 + b, 128, 3)
+        out = nblist.find_info4mlff_device(lat, torch.from_numpy(ty).to(dev), torch.from_numpy(pos).to(dev), 6.0, 200)
+        lists.append(tuple(o.cpu().numpy() if hasattr(o, "cpu") else o for o in out))
+    nb = synth.pack_batch(lists)
+    m = synth.nep_model(seed=3007, rmax_radial=6.0, rmax_angular=4.0)
+    f32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(dev)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(dev)
+    md = {k: f32(m[k]) for k in ("coeffs", "w0", "b0", "w1", "type_bias", "q_scaler")}
+    d = {k: i32(nb[k]) for k in ("binum", "bilist", "bnumneigh", "bfirstneigh", "btypes")}
+    d["brcs"] = f32(nb["brcs"])
+    B, P = nb["bilist"].shape
+    natoms = int(nb["binum"].sum())
+    nn = float(nb["bnumneigh"].sum()) / natoms
+    r = np.linalg.norm(nb["brcs"], axis=3)
+    nn_a = float(((r > 0) & (r <= m["rmax_angular"])).sum()) / natoms
+    lab = (f32(synth.rng_normal(4005, B * P, -4.0, 0.2).reshape(B, P).sum(1)),
+           f32(synth.rng_normal(4006, B * P * 3, 0.0, 1.0).reshape(B, P, 3)),
+           f32(synth.rng_normal(4007, B * 9, 0.0, 0.5).reshape(B, 9)))
+    tm = i32(m["type_map"])
+
+    def step(k):
+        ops.nep_loss_step(1.0, 1.0, 1.0, lab[0], lab[1], lab[2], m["chebyshev_size"], m["n_radial_basis"],
+                          m["n_angular_basis"], m["l_max"], md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"],
+                          d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"], tm, 0,
+                          m["rmax_radial"], m["rmax_angular"], md["q_scaler"], want_grad=True, validate=False)
+    L = _lib.lib()
+    elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
+    # the gradient pass repeats the descriptor work with tangents (x2) and adds the outer products of the
+    # hidden layer (4 D H) and the two coefficient-gradient contractions: counted as 2.5 x the E/F/V flops
+    work = {"nep_loss_bwd_kernel": ("mfma", 2.5 * nep_flops_per_atom(nn, nn_a) * natoms, "TFLOP/s", PEAK_FP32_TFLOPS,
+                                    1e12, "valu_fp32")}
+    config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P, "species": 3,
+              "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 6.0, "rcut_angular": 4.0,
+              "mean_neighbors_radial": nn, "mean_neighbors_angular": nn_a,
+              "per_step": "E/F/V + loss forward + analytic gradient w.r.t. coeffs/w0/b0/w1/bias"}
+    return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f32"
+
+
 def cpu_baseline_mtp(cfg):
     import oracle
     from ai2pot_amd import synth
@@ -333,6 +384,7 @@ WORKLOADS = {
     "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]
     "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
     "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]
+    "nep_train_64x128": run_nep_train,                            # NEP counterpart of configs[3] (not a BASELINE line)
     "hbm_copy_probe": None,                                       # counter calibration, not a workload of the path
 }
 
@@ -366,7 +418,9 @@ def main():
     }
     if not args.no_cpu_baseline:
         try:
-            if args.workload.startswith("nep"):
+            if args.workload == "nep_train_64x128":
+                out["cpu_baseline"] = {"note": "no CPU baseline leg for this extra workload"}
+            elif args.workload.startswith("nep"):
                 out["cpu_baseline"] = cpu_baseline_nep()
             else:
                 out["cpu_baseline"] = cpu_baseline_mtp({"mtp10_efv_216": 1, "mtp20_efv_8192": 3,

@@ -185,3 +185,29 @@ def test_fvt_ops(oracle, dropin):
     assert torch.autograd.gradgradcheck(force, (d,), eps=1e-6, atol=1e-7)
     assert torch.autograd.gradcheck(virial, (r, d), eps=1e-6, atol=1e-7)
     assert torch.autograd.gradgradcheck(virial, (r, d), eps=1e-6, atol=1e-7)
+
+
+def test_nep_loss_ops(dropin):
+    """torch.ops.nep.nepToLossOp / nepToEFLossOp against the reference's own output."""
+    import torch
+    from test_gpu_nep_loss import GRADS, PARAMS, close, golden_case
+    g, m, nb, labels = golden_case()
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64)).to("cuda:0")
+    d = to_device(nb, torch.float64)
+    params = [t(m[k]).requires_grad_(True) for k in PARAMS]
+    z = torch.zeros(16, dtype=torch.float64, device="cuda:0")
+    tail = (d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"],
+            torch.from_numpy(np.asarray(m["type_map"], np.int32)).to("cuda:0"), 0, m["rmax_radial"], m["rmax_angular"],
+            t(m["q_scaler"]), 0.0, 0.0, z, z)
+    sizes = (m["chebyshev_size"], m["n_radial_basis"], m["n_angular_basis"], m["l_max"])
+    out = torch.ops.nep.nepToLossOp(1.0, 0.7, 0.3, t(labels["energy"]), t(labels["force"]), t(labels["virial"]),
+                                    *sizes, *params, *tail)
+    assert len(out) == 4 and close(out[0].detach().cpu().numpy(), g["efv/bloss"])
+    assert close(torch.cat(out[1:]).detach().cpu().numpy(), g["efv/rmse"])
+    gl = torch.tensor([1.5, -0.5], dtype=torch.float64, device="cuda:0")
+    (out[0] * gl).sum().backward()
+    for p, k in zip(params, GRADS):
+        assert close(p.grad.cpu().numpy().ravel(), gl.cpu().numpy() @ g["efv/" + k]), k
+    out2 = torch.ops.nep.nepToEFLossOp(1.0, 0.7, t(labels["energy"]), t(labels["force"]), *sizes,
+                                       *[p.detach() for p in params], *tail)
+    assert len(out2) == 3 and close(out2[0].cpu().numpy(), g["ef/bloss"])
