@@ -1,10 +1,10 @@
 // libmtpr_bind.so -- registers torch.ops.mtpr.* with the reference's schemas
 // (source/descriptor/mtpr/bind/mtpr_bind.cc:30-569) on top of libai2pot_hip.so:
-// set_ai2pot_path, mtpParamOp, linearMtpToEFVOp, linearMtpToEFOp, linearMtpToLossOp and
-// linearMtpToEFLossOp (autograd to coeffs, linear_coeffs, type_bias only, as
-// src/linearMtpOp.cc:1732-1765).  The legacy and solver operators of the reference
-// (mtpBasisOp, LinMatrixLinVectorOp, CoeffsSchmidtOrthOp, linearMtpToEsitesOp,
-// linearMtpToDescriptorsOp) are not part of this build.
+// set_ai2pot_path, mtpParamOp, linearMtpToEFVOp, linearMtpToEFOp, linearMtpToLossOp,
+// linearMtpToEFLossOp, linearMtpToEsitesOp (autograd to coeffs, linear_coeffs, type_bias only, as
+// src/linearMtpOp.cc:1732-1765, 4002-4027) and linearMtpToDescriptorsOp.  The legacy and solver
+// operators of the reference (mtpBasisOp, LinMatrixLinVectorOp, CoeffsSchmidtOrthOp) are not part
+// of this build.
 #include "bind_common.h"
 
 #include <cstdlib>
@@ -288,6 +288,121 @@ struct LossFunction : public torch::autograd::Function<LossFunction> {
     }
 };
 
+// e_sites[B, P] and / or descriptors[B, P, S] of one batch
+void run_esites(const MtpCtx& c, int64_t K, double scaling, const at::Tensor& coeffs, const at::Tensor& lin,
+                const at::Tensor& bias, int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist,
+                const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                const at::Tensor& btypes, double rmax, double rmin, const at::Tensor& q_scaler, at::Tensor es,
+                at::Tensor desc)
+{
+    a2p_bind::DeviceGuard guard(brcs);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble) {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+        rc = a2p_mtp_esites_f64(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
+                                p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
+                                bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
+    } else {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+        rc = a2p_mtp_esites_f32(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
+                                p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
+                                bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
+    }
+    check_rc(rc);
+    check_device_status(brcs);
+}
+
+// forward: [e_sites[B, P]]; backward: sum over structures and rows of grad * d e_sites / d theta
+struct EsitesFunction : public torch::autograd::Function<EsitesFunction> {
+    static variable_list forward(AutogradContext* ctx, int64_t K, double scaling, const at::Tensor& coeffs,
+                                 const at::Tensor& lin, const at::Tensor& bias, int64_t n_moms,
+                                 const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping,
+                                 int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist,
+                                 const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                                 const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax,
+                                 double rmin, const at::Tensor& q_scaler)
+    {
+        MtpCtx c = check_mtp(K, coeffs, lin, bias, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                             bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
+        a2p_bind::DeviceGuard guard(brcs);
+        at::Tensor es = at::zeros({c.s.B, c.s.P}, brcs.options());
+        run_esites(c, K, scaling, coeffs, lin, bias, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, rmax,
+                   rmin, q_scaler, es, at::Tensor());
+        ctx->save_for_backward({coeffs, lin, bias, basic, times, mapping, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                                btypes, type_map, q_scaler});
+        ctx->saved_data["K"] = K;
+        ctx->saved_data["scaling"] = scaling;
+        ctx->saved_data["n_moms"] = n_moms;
+        ctx->saved_data["nmus"] = nmus;
+        ctx->saved_data["nghost"] = nghost;
+        ctx->saved_data["rmax"] = rmax;
+        ctx->saved_data["rmin"] = rmin;
+        return {es};
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(21);                   // one slot per forward argument after ctx
+        auto sv = ctx->get_saved_variables();
+        const at::Tensor &coeffs = sv[0], &lin = sv[1], &bias = sv[2], &brcs = sv[10], &q_scaler = sv[13];
+        const int64_t K = ctx->saved_data["K"].toInt(), nmus = ctx->saved_data["nmus"].toInt();
+        MtpCtx c = check_mtp(K, coeffs, lin, bias, ctx->saved_data["n_moms"].toInt(), sv[3], sv[4], sv[5], nmus,
+                             sv[6], sv[7], sv[8], sv[9], brcs, sv[11], sv[12], ctx->saved_data["nghost"].toInt(),
+                             q_scaler);
+        a2p_bind::DeviceGuard guard(brcs);
+        auto opt = brcs.options();
+        at::Tensor g = grads[0].contiguous();
+        TORCH_CHECK(g.dim() == 2 && g.size(0) == c.s.B && g.size(1) == c.s.P, "grad of e_sites must be [B, P]");
+        at::Tensor dc = at::zeros({c.s.B, coeffs.numel()}, opt), dl = at::zeros({c.s.B, lin.numel()}, opt),
+                   db = at::zeros({c.s.B, bias.numel()}, opt);
+        const double scaling = ctx->saved_data["scaling"].toDouble(), rmax = ctx->saved_data["rmax"].toDouble(),
+                     rmin = ctx->saved_data["rmin"].toDouble();
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+            rc = a2p_mtp_esites_bwd_f64(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus,
+                                        c.ntypes, p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost,
+                                        sv[6].data_ptr<int>(), sv[7].data_ptr<int>(), sv[8].data_ptr<int>(),
+                                        sv[9].data_ptr<int>(), p(brcs), sv[11].data_ptr<int>(), p(g), p(dc), p(dl),
+                                        p(db), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+            rc = a2p_mtp_esites_bwd_f32(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus,
+                                        c.ntypes, p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost,
+                                        sv[6].data_ptr<int>(), sv[7].data_ptr<int>(), sv[8].data_ptr<int>(),
+                                        sv[9].data_ptr<int>(), p(brcs), sv[11].data_ptr<int>(), p(g), p(dc), p(dl),
+                                        p(db), st);
+        }
+        check_rc(rc);
+        out[2] = dc.sum(0).reshape(coeffs.sizes());
+        out[3] = dl.sum(0).reshape(lin.sizes());
+        out[4] = db.sum(0).reshape(bias.sizes());
+        return out;
+    }
+};
+
+variable_list mtp_descriptors(int64_t K, double scaling, const at::Tensor& coeffs, int64_t n_moms,
+                              const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping,
+                              int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist,
+                              const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                              const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax,
+                              double rmin)
+{
+    // the descriptors do not depend on the read-out: unit weights and scalers, zero bias
+    at::Tensor one = at::ones({mapping.numel()}, brcs.options()), zero = at::zeros({type_map.numel()}, brcs.options());
+    MtpCtx c = check_mtp(K, coeffs, one, zero, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                         bfirstneigh, brcs, btypes, type_map, nghost, one);
+    a2p_bind::DeviceGuard guard(brcs);
+    at::Tensor desc = at::zeros({c.s.B, c.s.P, c.plan.n_scalar}, brcs.options());
+    run_esites(c, K, scaling, coeffs.detach(), one, zero, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+               rmax, rmin, one, at::Tensor(), desc);
+    return {desc};
+}
+
 }  // namespace
 
 #define MTP_EFV_ARGS int64_t K, double scaling, const at::Tensor& coeffs, const at::Tensor& lin, \
@@ -319,5 +434,18 @@ TORCH_LIBRARY(mtpr, m)
               // no virial labels in this variant: zero weight, zero labels
               return LossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
                                          at::zeros({e_dft.numel(), 9}, e_dft.options()), MTP_EFV_PASS);
+          });
+    m.def("linearMtpToEsitesOp", [](MTP_EFV_ARGS) -> variable_list {
+        require_no_zbl(zbl_rmax);
+        return EsitesFunction::apply(MTP_EFV_PASS);
+    });
+    m.def("linearMtpToDescriptorsOp",
+          [](int64_t K, double scaling, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic,
+             const at::Tensor& times, const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum,
+             const at::Tensor& bilist, const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
+             const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost,
+             double rmax, double rmin) -> variable_list {
+              return mtp_descriptors(K, scaling, coeffs, n_moms, basic, times, mapping, nmus, binum, bilist,
+                                     bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin);
           });
 }

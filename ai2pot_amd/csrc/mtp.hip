@@ -56,6 +56,11 @@ struct MtpArgs {
     T* gpart;          // [B, P, ngrad] per-atom gradient rows (ngrad = ncoef + n_scalar + ntypes)
     int ngrad;
     int lds_basic_off;  // byte offset of the packed basic-moment table in LDS
+    // site-energy / descriptor mode (linearMtp.h:514-611, 821-890)
+    T* e_sites;        // [B, P] per-row energies, or null
+    T* desc;           // [B, P, n_scalar] scalar moments, or null
+    int energy_only;   // stop after the energy: no adjoint, no pair derivatives
+    int cE_per_atom;   // loss-gradient mode: cE is indexed per row (weights of the site energies)
 };
 
 __device__ __forceinline__ float sqrt_t(float x) { return sqrtf(x); }
@@ -272,7 +277,10 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     T* pq = tab + max(MTP_NC * E + (256 / 32) * 32 * 4, p.max_level_slots * (LOSS ? 2 : 1));              // loss mode: P[nc][nmus] | Q[nc][nmus]
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
-        if (!LOSS && lane < 10) a.partial[row * 10 + lane] = 0.0;
+        if (!LOSS && a.partial && lane < 10) a.partial[row * 10 + lane] = 0.0;
+        if (!LOSS && a.e_sites && lane == 0) a.e_sites[row] = (T)0;
+        if (!LOSS && a.desc)
+            for (int s = lane; s < p.n_scalar; s += NT) a.desc[row * p.n_scalar + s] = (T)0;
         if (LOSS)
             for (int q = lane; q < a.ngrad; q += NT) a.gpart[row * a.ngrad + q] = (T)0;
         return;
@@ -335,6 +343,13 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     for (int s = lane; s < p.n_scalar; s += NT) {
         e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
         A[p.mapping[s]] = a.lin[s] / a.q_scaler[s];
+    }
+    if (!LOSS && (a.e_sites || a.desc)) {
+        if (a.desc)                                          // linearMtp.h:884-885: unscaled scalar moments
+            for (int s = lane; s < p.n_scalar; s += NT) a.desc[row * p.n_scalar + s] = M[p.mapping[s]];
+        const T e_row = block_sum<T, NT>(e_part, gred, lane) + a.bias[ti];
+        if (a.e_sites && lane == 0) a.e_sites[row] = e_row;  // linearMtp.h:594-599
+        if (a.energy_only) return;
     }
     __syncthreads();
     sweep_reverse<T, false, NT>(p, M, A, nullptr, nullptr, tab, lane);
@@ -418,7 +433,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
 
     // ---- loss gradient ------------------------------------------------------------------------
     if (LOSS) {
-        const T cE = a.cE[b];
+        const T cE = a.cE_per_atom ? a.cE[row] : a.cE[b];
         sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);      // linearMtpLoss.h:417-434
         T* grow = a.gpart + row * a.ngrad;
         for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
@@ -745,6 +760,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.brcs = brcs; a.btypes = btypes;
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
     a.force = nullptr; a.pair_g = nullptr; a.partial = nullptr;
+    a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
     if (rc) return rc;
@@ -874,6 +890,69 @@ int mtp_loss(void* handle, double e_w, double f_w, double v_w, const T* e_dft, c
     return A2P_OK;
 }
 
+// Site energies e_sites[B, P] (row order) and / or the scalar moments desc[B, P, n_scalar].
+template <typename T>
+int mtp_esites(void* handle, int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus,
+               int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
+               const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
+               const int* btypes, T* e_sites, T* desc, hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    A2P_REQUIRE(e_sites || desc, A2P_ERR_INVALID, "mtp e_sites: no output requested");
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
+                   binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    a.E = table_entries<T>(a.p, K, false);
+    a.e_sites = e_sites; a.desc = desc; a.energy_only = 1;
+    return launch_atoms<T, false>(a, stream);
+}
+
+// sum over rows of gout[b, ii] * d e_sites[b, ii] / d(coeffs, linear_coeffs, type_bias), per structure:
+// the loss-gradient kernel with the per-row weight in place of cE and no force / virial residuals.
+template <typename T>
+int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus,
+                   int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
+                   const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
+                   const T* brcs, const int* btypes, const T* gout, T* dcoeffs, T* dlin, T* dbias,
+                   hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    A2P_REQUIRE(gout && (dcoeffs || dlin || dbias), A2P_ERR_INVALID, "mtp e_sites backward: null pointer");
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
+                   binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    const int ncoef = ntypes * ntypes * nmus * K;
+    const int ngrad = ncoef + a.p.n_scalar + ntypes;
+    // workspace: dVs[B*9] | dFs[(B*P + nghost)*3] (both zero) | gpart[B*P*ngrad]
+    const size_t nzero = (size_t)B * 9 + ((size_t)B * P + nghost) * 3;
+    void* ws = nullptr;
+    rc = ws_get(WS_MTP, (nzero + (size_t)B * P * ngrad) * sizeof(T), &ws);
+    if (rc) return rc;
+    T* dVs = (T*)ws;
+    T* dFs = dVs + (size_t)B * 9;
+    T* gpart = (T*)ws + nzero;
+    rc = fill_zero(ws, ((nzero * sizeof(T) + 3) / 4) * 4, stream);
+    if (rc) return rc;
+    a.E = table_entries<T>(a.p, K, true);
+    a.cE = gout; a.cE_per_atom = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = ngrad;
+    rc = launch_atoms<T, true>(a, stream);
+    if (rc) return rc;
+    prof_begin("mtp_grad_reduce", stream);
+    hipLaunchKernelGGL(mtp_grad_reduce_kernel<T>, dim3(ceil_div(ngrad, 256), B), dim3(256), 0, stream, P, ncoef,
+                       a.p.n_scalar, ntypes, binum, gpart, dcoeffs, dlin, dbias);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 }  // namespace
 }  // namespace a2p
 
@@ -909,6 +988,7 @@ int a2p_mtp_plan_destroy(void* handle)
 #define MTP_MODEL_PASS K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin
 #define MTP_BATCH(T) const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, \
     const T* brcs, const int* btypes
+#define MTP_BATCH_PASS binum, bilist, bnumneigh, bfirstneigh, brcs, btypes
 
 int a2p_mtp_efv_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
                     double* etot, double* force, double* virial, void* stream)
@@ -942,5 +1022,30 @@ int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weig
     return a2p::mtp_loss<float>(plan, e_weight, f_weight, v_weight, e_dft, f_dft, v_dft, MTP_MODEL_PASS, B, P,
                                 U, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, bloss, rmse, etot, force,
                                 virial, dcoeffs, dlinear, dbias, (hipStream_t)stream);
+}
+
+int a2p_mtp_esites_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
+                       double* e_sites, double* descriptors, void* stream)
+{
+    return a2p::mtp_esites<double>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, e_sites, descriptors,
+                                   (hipStream_t)stream);
+}
+int a2p_mtp_esites_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int nghost, MTP_BATCH(float),
+                       float* e_sites, float* descriptors, void* stream)
+{
+    return a2p::mtp_esites<float>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, e_sites, descriptors,
+                                  (hipStream_t)stream);
+}
+int a2p_mtp_esites_bwd_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
+                           const double* grad_e_sites, double* dcoeffs, double* dlinear, double* dbias, void* stream)
+{
+    return a2p::mtp_esites_bwd<double>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, grad_e_sites, dcoeffs,
+                                       dlinear, dbias, (hipStream_t)stream);
+}
+int a2p_mtp_esites_bwd_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int nghost, MTP_BATCH(float),
+                           const float* grad_e_sites, float* dcoeffs, float* dlinear, float* dbias, void* stream)
+{
+    return a2p::mtp_esites_bwd<float>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, grad_e_sites, dcoeffs,
+                                      dlinear, dbias, (hipStream_t)stream);
 }
 }

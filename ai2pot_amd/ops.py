@@ -502,6 +502,128 @@ def linearMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bviri
     return list(_LinearMtpToLoss.apply(coeffs, linear_coeffs, type_bias, args))
 
 
+def linearMtpToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, scaling, coeffs,
+                        linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+                        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                        type_map, nghost, rmax, rmin, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None,
+                        zbl_dks=None, validate=True):
+    """[bloss[B], e_rmse[1], f_rmse[1]]: the loss without virial labels (zero weight, zero labels);
+    mtpr_bind.cc:263-331, linearMtpOp.cc:1768-2831."""
+    _no_zbl(zbl_rmax)
+    v_dft = torch.zeros((betot_dft.numel(), 9), dtype=betot_dft.dtype, device=betot_dft.device)
+    args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v_dft, chebyshev_size, scaling,
+            alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
+            bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, validate)
+    return list(_LinearMtpToLoss.apply(coeffs, linear_coeffs, type_bias, args))[:3]
+
+
+def _mtp_esites_raw(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                    alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh,
+                    bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, want_esites, want_desc,
+                    validate):
+    dtype, device, B, P, U, nghost, ntypes, plan, n_scalar = _mtp_common(
+        coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+        q_scaler, chebyshev_size, validate)
+    e_sites = torch.zeros((B, P), dtype=dtype, device=device) if want_esites else None
+    desc = torch.zeros((B, P, n_scalar), dtype=dtype, device=device) if want_desc else None
+    L = _lib.lib()
+    fn = L.a2p_mtp_esites_f32 if dtype == torch.float32 else L.a2p_mtp_esites_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
+                _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax),
+                _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
+                _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(e_sites),
+                _ptr(desc), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return e_sites, desc
+
+
+def mtp_esites_backward(grad_esites, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias,
+                        alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
+                        binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin,
+                        q_scaler, validate=False):
+    """Per-structure gradients of sum_i grad_esites[b, i] * e_sites[b, i]:
+    (dcoeffs[B, ncoef], dlinear[B, S], dbias[B, ntypes])."""
+    dtype, device, B, P, U, nghost, ntypes, plan, n_scalar = _mtp_common(
+        coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+        q_scaler, chebyshev_size, validate)
+    _check_float("grad_esites", grad_esites, dtype, device)
+    _req(tuple(grad_esites.shape) == (B, P), "grad_esites must have shape [B, P]")
+    z = lambda *s: torch.zeros(s, dtype=dtype, device=device)
+    dc, dl, db = z(B, coeffs.numel()), z(B, n_scalar), z(B, ntypes)
+    L = _lib.lib()
+    fn = L.a2p_mtp_esites_bwd_f32 if dtype == torch.float32 else L.a2p_mtp_esites_bwd_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs),
+                _ptr(linear_coeffs), _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_scaler),
+                _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost),
+                _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes),
+                _ptr(grad_esites), _ptr(dc), _ptr(dl), _ptr(db), _stream(device))
+        _lib.check(rc)
+    return dc, dl, db
+
+
+class _LinearMtpToEsites(torch.autograd.Function):
+    """Site energies with the reference's autograd contract (linearMtpOp.cc:3589-3825, 3829-4027):
+    gradients flow to coeffs, linear_coeffs and type_bias only, summed over structures and atoms."""
+
+    @staticmethod
+    def forward(ctx, coeffs, linear_coeffs, type_bias, args):
+        (K, scaling, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+         type_map, nghost, rmax, rmin, q_scaler, validate) = args
+        es, _ = _mtp_esites_raw(K, scaling, coeffs.detach(), linear_coeffs.detach(), type_bias.detach(), n_moms,
+                                basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                                type_map, nghost, rmax, rmin, q_scaler, True, False, validate)
+        ctx.save_for_backward(coeffs, linear_coeffs, type_bias)
+        ctx.args = args
+        return es
+
+    @staticmethod
+    def backward(ctx, ges):
+        coeffs, linear_coeffs, type_bias = ctx.saved_tensors
+        (K, scaling, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+         type_map, nghost, rmax, rmin, q_scaler, _) = ctx.args
+        dc, dl, db = mtp_esites_backward(ges.contiguous(), K, scaling, coeffs.detach(), linear_coeffs.detach(),
+                                         type_bias.detach(), n_moms, basic, times, mapping, nmus, binum, bilist,
+                                         bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin,
+                                         q_scaler)
+        return (dc.sum(0).reshape(coeffs.shape), dl.sum(0).reshape(linear_coeffs.shape),
+                db.sum(0).reshape(type_bias.shape), None)
+
+
+def linearMtpToEsitesOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
+                        alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                        bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
+                        zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
+    """[e_sites[B, P]] in row order (zero beyond binum), differentiable w.r.t. coeffs, linear_coeffs
+    and type_bias; mtpr_bind.cc:458-518."""
+    _no_zbl(zbl_rmax)
+    args = (chebyshev_size, scaling, alpha_moments_count, alpha_index_basic, alpha_index_times,
+            alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+            rmax, rmin, q_scaler, validate)
+    return [_LinearMtpToEsites.apply(coeffs, linear_coeffs, type_bias, args)]
+
+
+def linearMtpToDescriptorsOp(chebyshev_size, scaling, coeffs, alpha_moments_count, alpha_index_basic,
+                             alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh,
+                             bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, validate=True):
+    """[descriptors[B, P, alpha_scalar_moments]]: the unscaled scalar moments of every row; no
+    gradient, as in the reference (mtpr_bind.cc:521-570, linearMtpOp.cc:4030-4240)."""
+    n_scalar = int(alpha_moment_mapping.numel())
+    ntypes = int(type_map.numel())
+    one = torch.ones((n_scalar,), dtype=brcs.dtype, device=brcs.device)
+    zero_b = torch.zeros((ntypes,), dtype=brcs.dtype, device=brcs.device)
+    _, desc = _mtp_esites_raw(chebyshev_size, scaling, coeffs.detach(), one, zero_b, alpha_moments_count,
+                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                              bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, one, False, True,
+                              validate)
+    return [desc]
+
+
 # --------------------------------------------------------------------------------------------
 # fvt  (source/fvt/bind/fvt_sr_op_bind.cc:9-46)
 # --------------------------------------------------------------------------------------------

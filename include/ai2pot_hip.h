@@ -167,6 +167,45 @@ int a2p_mtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weig
                      float* dbias, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Linear-MTP site energies and scalar moments -- replaces the compute of
+ * torch.ops.mtpr.linearMtpToEsitesOp (forward and backward) and linearMtpToDescriptorsOp
+ * (source/descriptor/mtpr/bind/mtpr_bind.cc:459-569; src/linearMtpOp.cc:3589-4240;
+ *  include/linearMtp.h:514-611 find_e_sites, :616-818 find_e_sites_backward, :821-890
+ *  find_descriptors).
+ * a2p_mtp_esites_*: e_sites[B, P] (row order, bias + sum_s lin[s] M[map[s]] / q_scaler[s]; may be
+ * NULL) and descriptors[B, P, n_scalar] = M[map[s]] (unscaled; may be NULL); padded rows are zero.
+ * a2p_mtp_esites_bwd_*: per-structure  sum_ii grad_e_sites[b, ii] * d e_sites[b, ii] / d theta  into
+ * dcoeffs[B, ncoef], dlinear[B, n_scalar], dbias[B, ntypes] (any may be NULL); the operator's
+ * backward sums them over the batch (linearMtpOp.cc:4002-4005).
+ * ------------------------------------------------------------------------------------------ */
+int a2p_mtp_esites_f64(void* plan, int chebyshev_size, double scaling, const double* coeffs,
+                       const double* linear_coeffs, const double* type_bias, int nmus, int ntypes,
+                       const double* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                       int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                       const int* bfirstneigh, const double* brcs, const int* btypes, double* e_sites,
+                       double* descriptors, void* stream);
+int a2p_mtp_esites_f32(void* plan, int chebyshev_size, double scaling, const float* coeffs,
+                       const float* linear_coeffs, const float* type_bias, int nmus, int ntypes,
+                       const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                       int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                       const int* bfirstneigh, const float* brcs, const int* btypes, float* e_sites,
+                       float* descriptors, void* stream);
+int a2p_mtp_esites_bwd_f64(void* plan, int chebyshev_size, double scaling, const double* coeffs,
+                           const double* linear_coeffs, const double* type_bias, int nmus, int ntypes,
+                           const double* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                           int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                           const int* bfirstneigh, const double* brcs, const int* btypes,
+                           const double* grad_e_sites, double* dcoeffs, double* dlinear, double* dbias,
+                           void* stream);
+int a2p_mtp_esites_bwd_f32(void* plan, int chebyshev_size, double scaling, const float* coeffs,
+                           const float* linear_coeffs, const float* type_bias, int nmus, int ntypes,
+                           const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                           int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                           const int* bfirstneigh, const float* brcs, const int* btypes,
+                           const float* grad_e_sites, float* dcoeffs, float* dlinear, float* dbias,
+                           void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * NEP training loss, forward and analytic backward -- replaces the compute of
  * torch.ops.nep.nepToLossOp and torch.ops.nep.nepToEFLossOp
  * (source/descriptor/nep/bind/nep_bind.cc:136-276; src/nepOp.cc:2359-3484;

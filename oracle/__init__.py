@@ -353,6 +353,50 @@ def mtp_loss_step(model, nb, weights, labels):
     return _mtp_loss_step(oracle_lib(), "orc_mtp", model, nb, weights, labels)
 
 
+def _mtp_esites(lib, prefix, model, nb):
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    S = np.asarray(model["alpha_moment_mapping"]).size
+    e_sites = np.zeros((B, P))
+    desc = np.zeros((B, P, S))
+    fn = getattr(lib, prefix + "_esites_f64")
+    fn.restype = None
+    fn(_p(e_sites), _p(desc), *margs, *largs)
+    return e_sites, desc
+
+
+def _mtp_esites_bwd(lib, prefix, model, nb, gout):
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    S = np.asarray(model["alpha_moment_mapping"]).size
+    ncoef = ntypes * ntypes * model["nmus"] * model["chebyshev_size"]
+    gout = _c(gout, np.float64)
+    assert gout.shape == (B, P)
+    dc, dl, db = np.zeros((B, ncoef)), np.zeros((B, S)), np.zeros((B, ntypes))
+    fn = getattr(lib, prefix + "_esites_bwd_f64")
+    fn.restype = None
+    fn(_p(dc), _p(dl), _p(db), _p(gout), *margs, *largs)
+    return dc, dl, db
+
+
+def ref_mtp_esites(model, nb):
+    """(e_sites[B, P], descriptors[B, P, S]) by the reference (row order, zero beyond inum)."""
+    return _mtp_esites(_load("_ref/libref_mtpr.so"), "ref_mtp", model, nb)
+
+
+def mtp_esites(model, nb):
+    return _mtp_esites(oracle_lib(), "orc_mtp", model, nb)
+
+
+def ref_mtp_esites_bwd(model, nb, gout):
+    """Per-structure gradients of sum(gout * e_sites) w.r.t. coeffs, linear_coeffs, type_bias."""
+    return _mtp_esites_bwd(_load("_ref/libref_mtpr.so"), "ref_mtp", model, nb, gout)
+
+
+def mtp_esites_bwd(model, nb, gout):
+    return _mtp_esites_bwd(oracle_lib(), "orc_mtp", model, nb, gout)
+
+
 # ----------------------------------------------------------------------------------------
 # fvt (single structure, fp64)
 # ----------------------------------------------------------------------------------------

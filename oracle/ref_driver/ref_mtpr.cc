@@ -6,6 +6,8 @@
 // (src/linearMtpOp.cc:621-1181, 1184-1765): E/F/V, per-structure loss, RMSEs, then the
 // per-structure parameter gradients [B, n] before the grad_output matmul.
 #include <cstring>
+#include <vector>
+#include <algorithm>
 #include <string>
 #include "descriptor/mtpr/include/mtpParam.h"
 #include "descriptor/mtpr/include/linearMtp_cpu_launcher.h"
@@ -81,4 +83,66 @@ void ref_mtp_loss_step_f64(double* bloss, double* rmse, double* betot, double* b
                                             const_cast<double*>(v_dft), MTP_MODEL_PASS, MTP_LIST_PASS);
 }
 
+
+// site energies and scalar moments by the reference (linearMtp.h:514-611, 821-890), per structure as
+// the operator's CPU branch calls them (linearMtpOp.cc:3680-3760, 4110-4190)
+void ref_mtp_esites_f64(double* e_sites, double* desc, MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    for (int b = 0; b < B; b++) {
+        int* il = const_cast<int*>(&bilist[(size_t)b * P]);
+        int* nn = const_cast<int*>(&bnumneigh[(size_t)b * P]);
+        int* fn = const_cast<int*>(&bfirstneigh[(size_t)b * P * U]);
+        double(*rc)[3] = (double(*)[3])const_cast<double*>(&brcs[(size_t)b * P * U * 3]);
+        int* ty = const_cast<int*>(&btypes[(size_t)b * (P + nghost)]);
+        if (e_sites)
+            LinearMtp<double>::find_e_sites(&e_sites[(size_t)b * P], K, scaling, const_cast<double*>(coeffs),
+                                            const_cast<double*>(lin), const_cast<double*>(bias), n_moms, n_basic,
+                                            (const int(*)[4])basic, n_times, (const int(*)[4])times, n_scalar, mapping,
+                                            nmus, binum[b], il, nn, fn, rc, ty, ntypes, const_cast<int*>(type_map), U,
+                                            nghost, rmax, rmin, const_cast<double*>(q_scaler));
+        if (desc)
+            LinearMtp<double>::find_descriptors(&desc[(size_t)b * P * n_scalar], K, scaling,
+                                                const_cast<double*>(coeffs), n_moms, n_basic, (const int(*)[4])basic,
+                                                n_times, (const int(*)[4])times, n_scalar, mapping, nmus, binum[b], il,
+                                                nn, fn, rc, ty, ntypes, const_cast<int*>(type_map), U, nghost, rmax,
+                                                rmin);
+    }
+}
+
+// per-row derivatives of the site energies (linearMtp.h:616-818), contracted with gout[B, P] per
+// structure as the operator's backward does (linearMtpOp.cc:4002-4005, before its sum over the batch)
+void ref_mtp_esites_bwd_f64(double* dcoeffs, double* dlin, double* dbias, const double* gout, MTP_MODEL_ARGS,
+                            MTP_LIST_ARGS)
+{
+    const int ncoef = ntypes * ntypes * nmus * K;
+    std::vector<double> dc((size_t)P * ncoef), dl((size_t)P * n_scalar), db((size_t)P * ntypes);
+    for (int b = 0; b < B; b++) {
+        std::fill(dc.begin(), dc.end(), 0.0);
+        std::fill(dl.begin(), dl.end(), 0.0);
+        std::fill(db.begin(), db.end(), 0.0);
+        LinearMtp<double>::find_e_sites_backward(
+            dc.data(), dl.data(), db.data(), K, scaling, const_cast<double*>(coeffs), const_cast<double*>(lin),
+            const_cast<double*>(bias), n_moms, n_basic, (const int(*)[4])basic, n_times, (const int(*)[4])times,
+            n_scalar, mapping, nmus, binum[b], const_cast<int*>(&bilist[(size_t)b * P]),
+            const_cast<int*>(&bnumneigh[(size_t)b * P]), const_cast<int*>(&bfirstneigh[(size_t)b * P * U]),
+            (double(*)[3])const_cast<double*>(&brcs[(size_t)b * P * U * 3]),
+            const_cast<int*>(&btypes[(size_t)b * (P + nghost)]), ntypes, const_cast<int*>(type_map), U, nghost, rmax,
+            rmin, const_cast<double*>(q_scaler));
+        for (int q = 0; q < ncoef; q++) {
+            double a = 0;
+            for (int ii = 0; ii < binum[b]; ii++) a += gout[(size_t)b * P + ii] * dc[(size_t)ii * ncoef + q];
+            dcoeffs[(size_t)b * ncoef + q] = a;
+        }
+        for (int q = 0; q < n_scalar; q++) {
+            double a = 0;
+            for (int ii = 0; ii < binum[b]; ii++) a += gout[(size_t)b * P + ii] * dl[(size_t)ii * n_scalar + q];
+            dlin[(size_t)b * n_scalar + q] = a;
+        }
+        for (int q = 0; q < ntypes; q++) {
+            double a = 0;
+            for (int ii = 0; ii < binum[b]; ii++) a += gout[(size_t)b * P + ii] * db[(size_t)ii * ntypes + q];
+            dbias[(size_t)b * ntypes + q] = a;
+        }
+    }
+}
 }

@@ -67,7 +67,8 @@ template <typename S>
 void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeffs, const S* lin,
              const S* bias, const Tables& t, int inum, const int* ilist, const int* numneigh,
              const int* firstneigh, const double* rcs, const int* types, int ntypes, int U,
-             int nforce, double rmax, double rmin, const double* q_scaler)
+             int nforce, double rmax, double rmin, const double* q_scaler, S* e_sites = nullptr,
+             S* desc = nullptr)
 {
     etot = S(0);
     for (int i = 0; i < nforce * 3; i++) force[i] = S(0);   // linearMtp.h:228-230
@@ -114,6 +115,9 @@ void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeff
         S e = bias[ti];                                        // linearMtp.h:281-285
         for (int s = 0; s < t.n_scalar; s++) e += lin[s] * M[t.mapping[s]] / S(q_scaler[s]);
         etot += e;
+        if (e_sites) e_sites[ii] = e;                          // linearMtp.h:594-599 (row order)
+        if (desc)                                              // linearMtp.h:884-885 (unscaled moments)
+            for (int s = 0; s < t.n_scalar; s++) desc[(size_t)ii * t.n_scalar + s] = M[t.mapping[s]];
         std::fill(adj.begin(), adj.end(), S(0));               // linearMtp.h:292-306
         for (int s = 0; s < t.n_scalar; s++) adj[t.mapping[s]] = lin[s] / S(q_scaler[s]);
         for (int i = t.n_times - 1; i >= 0; i--) {
@@ -278,4 +282,50 @@ void orc_mtp_loss_step_f64(double* bloss, double* rmse, double* betot, double* b
     }
 }
 
+
+// site energies e_sites[B, P] and scalar moments desc[B, P, n_scalar] (either may be null)
+void orc_mtp_esites_f64(double* e_sites, double* desc, MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    for (int b = 0; b < B; b++) {
+        double e;
+        std::vector<double> force((size_t)(P + nghost) * 3), virial(9);
+        efv_one<double>(e, force.data(), virial.data(), K, scaling, coeffs, lin, bias, t, binum[b],
+                        &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                        &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost,
+                        rmax, rmin, q_scaler, e_sites ? &e_sites[(size_t)b * P] : nullptr,
+                        desc ? &desc[(size_t)b * P * n_scalar] : nullptr);
+    }
+}
+
+// d/dtheta of sum_ii gout[b, ii] e_sites[b, ii] per structure, by forward-mode AD
+void orc_mtp_esites_bwd_f64(double* dcoeffs, double* dlin, double* dbias, const double* gout, MTP_MODEL_ARGS,
+                            MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int ncoef = ntypes * ntypes * nmus * K;
+    const int npar = ncoef + n_scalar + ntypes;
+#pragma omp parallel
+    {
+        std::vector<Dual> c(ncoef), l(n_scalar), bi(ntypes), force((size_t)(P + nghost) * 3), virial(9), es(P);
+#pragma omp for schedule(dynamic) collapse(2)
+        for (int b = 0; b < B; b++)
+            for (int p = 0; p < npar; p++) {
+                for (int i = 0; i < ncoef; i++) c[i] = Dual(coeffs[i], i == p);
+                for (int i = 0; i < n_scalar; i++) l[i] = Dual(lin[i], ncoef + i == p);
+                for (int i = 0; i < ntypes; i++) bi[i] = Dual(bias[i], ncoef + n_scalar + i == p);
+                Dual e;
+                efv_one<Dual>(e, force.data(), virial.data(), K, scaling, c.data(), l.data(), bi.data(), t,
+                              binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P],
+                              &bfirstneigh[(size_t)b * P * U], &brcs[(size_t)b * P * U * 3],
+                              &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost, rmax, rmin, q_scaler,
+                              es.data());
+                double acc = 0;
+                for (int ii = 0; ii < binum[b]; ii++) acc += gout[(size_t)b * P + ii] * es[ii].d;
+                if (p < ncoef) dcoeffs[(size_t)b * ncoef + p] = acc;
+                else if (p < ncoef + n_scalar) dlin[(size_t)b * n_scalar + p - ncoef] = acc;
+                else dbias[(size_t)b * ntypes + p - ncoef - n_scalar] = acc;
+            }
+    }
+}
 }

@@ -96,6 +96,10 @@ def mtp_cases():
         out.update({tag + "/E": e, tag + "/F": f, tag + "/V": v})
         for k, val in r.items():
             out[tag + "/loss_" + k] = val
+        es, desc = oracle.ref_mtp_esites(m, nb)
+        dc, dl, db = oracle.ref_mtp_esites_bwd(m, nb, synth.rng_normal(4, B * P).reshape(B, P))
+        out.update({tag + "/esites": es, tag + "/desc": desc, tag + "/es_dcoeffs": dc,
+                    tag + "/es_dlinear": dl, tag + "/es_dbias": db})
         out[tag + "/table_sizes"] = np.array([t["alpha_moments_count"], t["alpha_index_basic"].shape[0],
                                               t["alpha_index_times"].shape[0],
                                               t["alpha_moment_mapping"].size, t["nmus"]])

@@ -163,6 +163,18 @@ def test_mtpr_ops(oracle, dropin, tmp_path):
     out2[0].sum().backward()
     r2 = oracle.mtp_loss_step(m, nb, (1.0, 0.7, 0.0), lab)
     assert close(out2[0].detach().cpu().numpy(), r2["bloss"]) and close(params2[0].grad.cpu().numpy(), r2["dcoeffs"].sum(0))
+    # site energies (autograd) and descriptors
+    params3 = [md[k].clone().requires_grad_(True) for k in ("coeffs", "linear_coeffs", "type_bias")]
+    es = torch.ops.mtpr.linearMtpToEsitesOp(8, 1.0, params3[0], params3[1], params3[2], *efv_args[5:])
+    desc = torch.ops.mtpr.linearMtpToDescriptorsOp(8, 1.0, md["coeffs"], *efv_args[5:20])
+    es_ref, desc_ref = oracle.mtp_esites(m, nb)
+    assert len(es) == 1 and len(desc) == 1
+    assert close(es[0].detach().cpu().numpy(), es_ref) and close(desc[0].cpu().numpy(), desc_ref)
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    (es[0] * t(gout)).sum().backward()
+    rc, rl, rb = oracle.mtp_esites_bwd(m, nb, gout)
+    assert close(params3[0].grad.cpu().numpy(), rc.sum(0)) and close(params3[1].grad.cpu().numpy(), rl.sum(0))
+    assert close(params3[2].grad.cpu().numpy(), rb.sum(0))
 
 
 def test_fvt_ops(oracle, dropin):

@@ -203,6 +203,98 @@ def test_loss_autograd_contract(oracle):
     assert close(md["type_bias"].grad.cpu().numpy(), ref["dbias"].mean(0))
 
 
+def esites_args(m, md, d):
+    return (m["chebyshev_size"], m["scaling"], md["coeffs"], md["linear_coeffs"], md["type_bias"],
+            m["alpha_moments_count"], md["alpha_index_basic"], md["alpha_index_times"],
+            md["alpha_moment_mapping"], m["nmus"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"],
+            d["brcs"], d["btypes"], md["type_map"], d["nghost"], m["rmax"], m["rmin"], md["q_scaler"])
+
+
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3), (20, 2)])
+def test_site_energies_and_descriptors(oracle, level, nt):
+    """linearMtpToEsitesOp / linearMtpToDescriptorsOp against the oracle (itself pinned to the
+    reference's committed outputs), with a padded structure and, at level 20, the wide kernel."""
+    import torch
+    from ai2pot_amd import ops
+    m, nb, _ = loss_inputs(oracle, level, nt, sizes=(48, 30), P=52)
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    args = esites_args(m, md, d)
+    es = ops.linearMtpToEsitesOp(*args, 0.0, 0.0, None, None)[0]
+    desc = ops.linearMtpToDescriptorsOp(*(args[:3] + args[5:20]))[0]
+    es_ref, desc_ref = oracle.mtp_esites(m, nb)
+    assert es.shape == es_ref.shape and desc.shape == desc_ref.shape
+    assert close(es.cpu().numpy(), es_ref) and close(desc.cpu().numpy(), desc_ref)
+    assert np.all(es.cpu().numpy()[1, 30:] == 0) and np.all(desc.cpu().numpy()[1, 30:] == 0)
+    e = ops.linearMtpToEFVOp(*args, 0.0, 0.0, None, None)[0]
+    assert close(es.sum(1).cpu().numpy(), e.cpu().numpy())
+    if level > 10:
+        return
+    B, P = nb["bilist"].shape
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    dc, dl, db = ops.mtp_esites_backward(torch.from_numpy(gout).to("cuda:0"), *args)
+    rc, rl, rb = oracle.mtp_esites_bwd(m, nb, gout)
+    assert close(dc.cpu().numpy(), rc) and close(dl.cpu().numpy(), rl) and close(db.cpu().numpy(), rb)
+
+
+def test_site_energies_against_golden_and_autograd(oracle):
+    """Level 16 against the committed outputs of the reference's find_e_sites, find_descriptors and
+    find_e_sites_backward; then the operator's autograd contract: gradients reach coeffs,
+    linear_coeffs and type_bias, summed over structures and rows (linearMtpOp.cc:4002-4005)."""
+    import os
+    import torch
+    from ai2pot_amd import ops
+    with np.load(os.path.join(os.path.dirname(__file__), "golden", "mtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L16/")}
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    ty = synth.rng_randint(22, 48, 3)
+    m = synth.mtp_model(mtp_param.mtp_param(16), 3, 8, 5.0, 1.8, 3016)
+    o = oracle.nblist(lat, ty, pos, 5.0, 100)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.01
+    B, P = nb["bilist"].shape
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    for k in ("coeffs", "linear_coeffs", "type_bias"):
+        md[k].requires_grad_(True)
+    args = esites_args(m, md, d)
+    es = ops.linearMtpToEsitesOp(*args, 0.0, 0.0, None, None)[0]
+    desc = ops.linearMtpToDescriptorsOp(*(args[:3] + args[5:20]))[0]
+    assert close(es.detach().cpu().numpy(), g["esites"]) and close(desc.cpu().numpy(), g["desc"])
+    assert not desc.requires_grad
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    (es * torch.from_numpy(gout).to("cuda:0")).sum().backward()
+    assert close(md["coeffs"].grad.cpu().numpy(), g["es_dcoeffs"].sum(0))
+    assert close(md["linear_coeffs"].grad.cpu().numpy(), g["es_dlinear"].sum(0))
+    assert close(md["type_bias"].grad.cpu().numpy(), g["es_dbias"].sum(0))
+
+
+def test_site_energies_with_ghosts(oracle):
+    """Rows are the local atoms; neighbours may be ghosts (index >= natoms_pad)."""
+    import torch
+    from ai2pot_amd import ops
+    o = structure(oracle, 64, (9.0, 9.5, 10.0), 2, 1004, 5.0, umax=150)
+    m = synth.mtp_model(mtp_param.mtp_param(10), 2, 8, 5.0, 1.5, 3004)
+    inum, ilist, numneigh, first, rcs, types, _ = o
+    nl = 40
+    first = first.copy()
+    first[first < 0] = 0
+    nbg = dict(binum=np.array([nl], np.int32), bilist=ilist[None, :nl].copy(), bnumneigh=numneigh[None, :nl].copy(),
+               bfirstneigh=first[None, :nl].copy(), brcs=rcs[None, :nl].copy(), btypes=types[None, :].copy(),
+               nghost=inum - nl)
+    md = model_to_device(m, torch.float64)
+    d = to_device(nbg, torch.float64)
+    args = esites_args(m, md, d)
+    es = ops.linearMtpToEsitesOp(*args, 0.0, 0.0, None, None)[0]
+    es_ref, _ = oracle.mtp_esites(m, nbg)
+    assert close(es.cpu().numpy(), es_ref)
+    gout = synth.rng_normal(5, nl).reshape(1, nl)
+    got = ops.mtp_esites_backward(torch.from_numpy(gout).to("cuda:0"), *args)
+    ref = oracle.mtp_esites_bwd(m, nbg, gout)
+    for a, b in zip(got, ref):
+        assert close(a.cpu().numpy(), b)
+
+
 def test_errors(oracle):
     import torch
     from ai2pot_amd import _lib, ops

@@ -59,6 +59,41 @@ def test_against_golden(oracle, level, nt):
         assert np.abs(val - ref).max() <= 1e-11 * max(np.abs(ref).max(), 1e-300), k
 
 
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3)])
+def test_site_energies_and_descriptors(oracle, level, nt):
+    """Site energies, scalar moments and the site-energy gradient: the reference's committed
+    outputs, then what fixes them without it (sum rule, the linear read-out, dE_i/dbias = 1)."""
+    with np.load(os.path.join(HERE, "golden", "mtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+    m, nb, _ = small_batch(oracle, level, nt)
+    B, P = nb["bilist"].shape
+    es, desc = oracle.mtp_esites(m, nb)
+    assert np.abs(es - g["esites"]).max() <= 1e-12 * np.abs(g["esites"]).max()
+    assert np.abs(desc - g["desc"]).max() <= 1e-12 * np.abs(g["desc"]).max()
+    e, _, _ = oracle.mtp_efv(m, nb)
+    assert np.abs(es.sum(1) - e).max() < 1e-12 * np.abs(e).max()
+    # e_i = bias[t_i] + sum_s lin_s * desc_is / q_scaler_s   (linearMtp.h:594-599)
+    ti = np.take_along_axis(nb["btypes"], nb["bilist"], 1)
+    want = m["type_bias"][ti] + (desc * (m["linear_coeffs"] / m["q_scaler"])).sum(-1)
+    assert np.abs(es - want).max() < 1e-12 * np.abs(es).max()
+    if level == 16:
+        return
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    dc, dl, db = oracle.mtp_esites_bwd(m, nb, gout)
+    for got, key in ((dc, "es_dcoeffs"), (dl, "es_dlinear"), (db, "es_dbias")):
+        assert np.abs(got - g[key]).max() <= 1e-11 * max(np.abs(g[key]).max(), 1e-300), key
+    assert np.abs(dl - np.einsum("bi,bis->bs", gout, desc) / m["q_scaler"]).max() < 1e-11 * np.abs(dl).max()
+    for t in range(nt):
+        assert np.abs(db[:, t] - (gout * (ti == t)).sum(1)).max() < 1e-12
+    h = 1e-6
+    for i in (0, 9, m["coeffs"].size - 1):
+        mp, mm = dict(m), dict(m)
+        mp["coeffs"] = m["coeffs"].copy(); mp["coeffs"][i] += h
+        mm["coeffs"] = m["coeffs"].copy(); mm["coeffs"][i] -= h
+        fd = ((oracle.mtp_esites(mp, nb)[0] - oracle.mtp_esites(mm, nb)[0]) * gout).sum(1) / (2 * h)
+        assert np.abs(fd - dc[:, i]).max() < 1e-6 * max(1.0, np.abs(fd).max())
+
+
 def test_energy_force_finite_difference_and_linearity(oracle):
     lat, pos = synth.random_packed(30, [8.0, 8.5, 9.0], 2.0, 31)
     ty = synth.rng_randint(32, 30, 2)
