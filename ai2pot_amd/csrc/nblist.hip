@@ -289,9 +289,16 @@ __device__ __forceinline__ void pad_fill(V* __restrict__ row, int beg, int end, 
 // of the binning) cannot contribute and is left out; the order of what remains is unchanged.
 // The runs are then laid out back to back in LDS as a flat candidate list, which the wave
 // scans 64 candidates at a time; accepted candidates are appended with a ballot prefix.
-constexpr int NBL_ENT_CAP = 512;   // flat candidate list per wave (entries); longer lists search the runs
+// With ROWBUF the wave assembles its whole output row (accepted entries, then the -1 / 0 padding)
+// in LDS and writes it with 16-byte stores, one full row of firstneigh and one of rcs; this needs
+// umax % 4 == 0 and 16-byte aligned outputs.
+constexpr int NBL_UNROLL = 4;
+constexpr int NBL_ENT_CAP = 256;   // flat candidate list per wave (entries); longer lists search the runs
 
-template <typename T, bool SORT>
+template <typename T>
+inline size_t rowbuf_bytes(int umax) { return (size_t)umax * (4 + 3 * sizeof(T)); }
+
+template <typename T, bool SORT, bool ROWBUF>
 __global__ void __launch_bounds__(NBL_BLOCK)
 lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
@@ -302,9 +309,19 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
     __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
+    extern __shared__ __align__(16) unsigned char sh_rows[];
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int p = blockIdx.x * (NBL_BLOCK / 64) + wv;
     if (p >= g.N) return;                         // whole wave leaves together
+    T* rb_rcs = nullptr;
+    int* rb_first = nullptr;
+    if (ROWBUF) {
+        unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T));
+        rb_rcs = (T*)mine;
+        rb_first = (int*)(mine + (size_t)umax * 3 * sizeof(T));
+        for (int i = lane; i < umax; i += 64) rb_first[i] = -1;            // neighborList.h:557, 563
+        for (int i = lane; i < umax * 3; i += 64) rb_rcs[i] = (T)0;
+    }
     T c[3];
     int cb[3];
 #pragma unroll
@@ -366,50 +383,78 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
 
     int cnt = 0;
     const size_t rowi = (size_t)p * umax;
-    for (int c0 = 0; c0 < total; c0 += 64) {
-        const int ci = c0 + lane;
-        bool in = false;
-        T dx = 0, dy = 0, dz = 0;
-        int sj = 0;
-        double d2d = 0.0;
-        if (ci < total) {
-            int ent;
-            if (flat) {
-                ent = sh_ent[wv][ci];
-            } else {
-                // last column whose base is <= ci
-                int lo = 0, hi = nruns - 1;
-                while (lo < hi) {
-                    const int mid = (lo + hi + 1) >> 1;
-                    if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+    // NBL_UNROLL chunks of 64 candidates per trip: all their loads are issued before the first is
+    // used, so a typical row (100 - 250 candidates) costs one memory round trip
+    for (int c0 = 0; c0 < total; c0 += 64 * NBL_UNROLL) {
+        int sj[NBL_UNROLL];
+        T px[NBL_UNROLL], py[NBL_UNROLL], pz[NBL_UNROLL];
+#pragma unroll
+        for (int u = 0; u < NBL_UNROLL; u++) {
+            const int ci = c0 + u * 64 + lane;
+            sj[u] = 0; px[u] = c[0]; py[u] = c[1]; pz[u] = c[2];
+            if (ci < total) {
+                int ent;
+                if (flat) {
+                    ent = sh_ent[wv][ci];
+                } else {
+                    // last column whose base is <= ci
+                    int lo = 0, hi = nruns - 1;
+                    while (lo < hi) {
+                        const int mid = (lo + hi + 1) >> 1;
+                        if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+                    }
+                    ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
                 }
-                ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
+                sj[u] = s_idx[ent];
+                px[u] = s_x[(size_t)ent * 3 + 0];
+                py[u] = s_x[(size_t)ent * 3 + 1];
+                pz[u] = s_x[(size_t)ent * 3 + 2];
             }
-            sj = s_idx[ent];
-            dx = sub_rn(s_x[(size_t)ent * 3 + 0], c[0]);
-            dy = sub_rn(s_x[(size_t)ent * 3 + 1], c[1]);
-            dz = sub_rn(s_x[(size_t)ent * 3 + 2], c[2]);
-            d2d = dist2_double(dx, dy, dz);
-            const T d2 = (T)d2d;                                   // `CoordType relative_distance2`
-            in = ((double)d2 < g.rcut2) && ((double)d2 > kEpsilon);   // binLinkedList.h:1014-1017
         }
-        const unsigned long long mask = __ballot(in);
-        const int rank = __popcll(mask & ((1ull << lane) - 1ull));
-        const int slot = cnt + rank;
-        if (in && slot < umax) {
-            firstneigh[rowi + slot] = sj;                           // neighborList.h:561 (already mod natoms)
-            rcs[(rowi + slot) * 3 + 0] = dx;
-            rcs[(rowi + slot) * 3 + 1] = dy;
-            rcs[(rowi + slot) * 3 + 2] = dz;
-            if (SORT) keys[rowi + slot] = (T)__dsqrt_rn(d2d);       // neighborList.h:318-322
+#pragma unroll
+        for (int u = 0; u < NBL_UNROLL; u++) {
+            if (c0 + u * 64 >= total) break;                           // wave-uniform
+            const bool have = c0 + u * 64 + lane < total;
+            const T dx = sub_rn(px[u], c[0]), dy = sub_rn(py[u], c[1]), dz = sub_rn(pz[u], c[2]);
+            const double d2d = dist2_double(dx, dy, dz);
+            const T d2 = (T)d2d;                                       // `CoordType relative_distance2`
+            const bool in = have && ((double)d2 < g.rcut2) && ((double)d2 > kEpsilon);   // binLinkedList.h:1014-1017
+            const unsigned long long mask = __ballot(in);
+            const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+            const int slot = cnt + rank;
+            if (in && slot < umax) {
+                if (ROWBUF) {
+                    rb_first[slot] = sj[u];
+                    rb_rcs[slot * 3 + 0] = dx;
+                    rb_rcs[slot * 3 + 1] = dy;
+                    rb_rcs[slot * 3 + 2] = dz;
+                } else {
+                    firstneigh[rowi + slot] = sj[u];                   // neighborList.h:561 (already mod natoms)
+                    rcs[(rowi + slot) * 3 + 0] = dx;
+                    rcs[(rowi + slot) * 3 + 1] = dy;
+                    rcs[(rowi + slot) * 3 + 2] = dz;
+                }
+                if (SORT) keys[rowi + slot] = (T)__dsqrt_rn(d2d);      // neighborList.h:318-322
+            }
+            cnt += __popcll(mask);
         }
-        cnt += __popcll(mask);
     }
     if (lane == 0) {
         ilist[p] = p;
         numneigh[p] = cnt;
         types_out[p] = types[p];
         if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
+    }
+    if (ROWBUF) {
+        __builtin_amdgcn_wave_barrier();
+        const uint4* s1 = reinterpret_cast<const uint4*>(rb_first);
+        uint4* d1 = reinterpret_cast<uint4*>(firstneigh + rowi);
+        for (int i = lane; i < umax / 4; i += 64) d1[i] = s1[i];
+        const uint4* s2 = reinterpret_cast<const uint4*>(rb_rcs);
+        uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
+        const int nv = (int)((size_t)umax * 3 * sizeof(T) / 16);
+        for (int i = lane; i < nv; i += 64) d2[i] = s2[i];
+        return;
     }
     // padding: -1 / 0 (neighborList.h:557, 563)
     const int first_pad = min(cnt, umax);
@@ -766,12 +811,21 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     const int list_blocks = ceil_div(N, NBL_BLOCK / 64);
     prof_begin("nbl_lists", stream);
+    const size_t rows_lds = rowbuf_bytes<T>(umax) * (NBL_BLOCK / 64);
+    const bool rowbuf = !sort && umax % 4 == 0 && rows_lds <= 32 * 1024 && (uintptr_t)firstneigh % 16 == 0 &&
+                        (uintptr_t)rcs % 16 == 0;
     if (sort)
-        hipLaunchKernelGGL((lists_kernel<T, true>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types,
-                           offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys, status);
+        hipLaunchKernelGGL((lists_kernel<T, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
+                           types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
+                           status);
+    else if (rowbuf)
+        hipLaunchKernelGGL((lists_kernel<T, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream, g,
+                           x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           status);
     else
-        hipLaunchKernelGGL((lists_kernel<T, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x, types,
-                           offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys, status);
+        hipLaunchKernelGGL((lists_kernel<T, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
+                           types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           status);
     prof_end(stream);
     if (sort) {
         prof_begin("nbl_sort_rows", stream);

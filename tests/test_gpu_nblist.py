@@ -64,6 +64,18 @@ def test_unwrapped_coordinates_small_cell(oracle, dt):
     assert a[5].dtype == np.int32
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("umax", [56, 54, 2000])
+def test_row_capacities(oracle, dt, umax):
+    """Capacities that take the LDS row buffer (multiple of 4, small), the direct stores (not a
+    multiple of 4) and a row too large for the buffer."""
+    lat, pos = synth.random_packed(200, [14.0, 15.0, 16.0], 2.2, 91)
+    types = synth.rng_randint(92, 200, 2)
+    a = gpu_list(lat.astype(dt), types, pos.astype(dt), 5.0, umax)
+    b = oracle.nblist(lat.astype(dt), types, pos.astype(dt), 5.0, umax)
+    assert_same(a, b)
+
+
 @pytest.mark.parametrize("sort", [False, True])
 def test_config2_size(oracle, sort):
     lat, pos = synth.random_packed(4096, [49.8848] * 3, 2.2, 1003)
