@@ -1,0 +1,154 @@
+// libnnmtp_bind.so -- registers torch.ops.nnmtp.* with the reference's schemas
+// (source/descriptor/nnmtp/bind/nnmtp_bind.cc:27-430) on top of libai2pot_hip.so:
+// set_ai2pot_path, mtpParamOp, nnMtpToEFVOp, nnMtpToEFOp, nnMtpToEsitesOp (forward) and
+// nnMtpToDescriptorsOp.  The training operators of the reference (nnMtpToLossOp, nnMtpToEFLossOp)
+// and the backward of nnMtpToEsitesOp are not part of this build: they are registered and raise.
+#include "mtp_bind_common.h"
+
+namespace {
+
+#define NNMTP_ARGS int64_t K, const at::Tensor& coeffs, const at::Tensor& w0, const at::Tensor& w1, \
+    const at::Tensor& bias, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times, \
+    const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist, \
+    const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs, \
+    const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax, double rmin, \
+    const at::Tensor& q_shifter, const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin, \
+    const at::Tensor& zbl_cks, const at::Tensor& zbl_dks
+#define NNMTP_PASS K, coeffs, w0, w1, bias, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh, \
+    bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler
+
+// want_e: E and F (and V with want_v); want_es: the site energies
+variable_list nnmtp_run(bool want_e, bool want_v, bool want_es, int64_t K, const at::Tensor& coeffs,
+                        const at::Tensor& w0, const at::Tensor& w1, const at::Tensor& bias, int64_t n_moms,
+                        const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping, int64_t nmus,
+                        const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                        const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                        const at::Tensor& type_map, int64_t nghost, double rmax, double rmin,
+                        const at::Tensor& q_shifter, const at::Tensor& q_scaler)
+{
+    Batch s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+    const int ntypes = (int)type_map.numel();
+    TORCH_CHECK(ntypes > 0, "type_map is empty");
+    for (auto& pr : {std::make_pair(&coeffs, "coeffs"), std::make_pair(&w0, "w0"), std::make_pair(&w1, "w1"),
+                     std::make_pair(&bias, "type_bias"), std::make_pair(&q_shifter, "q_shifter"),
+                     std::make_pair(&q_scaler, "q_scaler")})
+        check_device_float(brcs, *pr.first, pr.second);
+    a2p_bind::DeviceGuard guard(brcs);
+    PlanEntry plan = get_plan(brcs.device().index(), n_moms, basic, times, mapping);
+    TORCH_CHECK(coeffs.numel() == (int64_t)ntypes * ntypes * nmus * K, "coeffs size mismatch");
+    TORCH_CHECK(w1.numel() > 0 && w1.numel() % ntypes == 0, "w1 must have ntypes * num_neurons elements");
+    const int H = (int)(w1.numel() / ntypes);
+    TORCH_CHECK(w0.numel() == (int64_t)ntypes * H * plan.n_scalar,
+                "w0 must have ntypes * num_neurons * alpha_scalar_moments elements");
+    TORCH_CHECK(q_shifter.numel() == plan.n_scalar && q_scaler.numel() == plan.n_scalar,
+                "q_shifter and q_scaler must have alpha_scalar_moments elements");
+    TORCH_CHECK(bias.numel() == ntypes, "type_bias size mismatch");
+    auto opt = brcs.options();
+    at::Tensor e, f, v, es;
+    if (want_e) {
+        e = at::zeros({s.B}, opt);
+        f = at::zeros({s.B, s.P + s.nghost, 3}, opt);
+        if (want_v) v = at::zeros({s.B, 9}, opt);
+    }
+    if (want_es) es = at::zeros({s.B, s.P}, opt);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble) {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+        rc = a2p_nnmtp_efv_f64(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                               p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                               binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                               bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
+                               st);
+    } else {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+        rc = a2p_nnmtp_efv_f32(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                               p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                               binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                               bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
+                               st);
+    }
+    check_rc(rc);
+    check_device_status(brcs);
+    if (want_es) return {es};
+    if (want_v) return {e, f, v};
+    return {e, f};
+}
+
+variable_list nnmtp_descriptors(int64_t K, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic,
+                                const at::Tensor& times, const at::Tensor& mapping, int64_t nmus,
+                                const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                                const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                                const at::Tensor& type_map, int64_t nghost, double rmax, double rmin)
+{
+    // the scalar moments themselves (nnMtp.h:570-645): the linear-MTP kernel at scaling 1
+    Batch s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+    const int ntypes = (int)type_map.numel();
+    TORCH_CHECK(ntypes > 0, "type_map is empty");
+    check_device_float(brcs, coeffs, "coeffs");
+    a2p_bind::DeviceGuard guard(brcs);
+    PlanEntry plan = get_plan(brcs.device().index(), n_moms, basic, times, mapping);
+    TORCH_CHECK(coeffs.numel() == (int64_t)ntypes * ntypes * nmus * K, "coeffs size mismatch");
+    auto opt = brcs.options();
+    at::Tensor one = at::ones({plan.n_scalar}, opt), zero = at::zeros({ntypes}, opt);
+    at::Tensor desc = at::zeros({s.B, s.P, plan.n_scalar}, opt);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble) {
+        auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+        rc = a2p_mtp_esites_f64(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
+                                rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                btypes.data_ptr<int>(), nullptr, p(desc), st);
+    } else {
+        auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+        rc = a2p_mtp_esites_f32(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
+                                rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                btypes.data_ptr<int>(), nullptr, p(desc), st);
+    }
+    check_rc(rc);
+    check_device_status(brcs);
+    return {desc};
+}
+
+}  // namespace
+
+TORCH_LIBRARY(nnmtp, m)
+{
+    m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
+    m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
+    m.def("nnMtpToEFVOp", [](NNMTP_ARGS) -> variable_list {
+        require_no_zbl(zbl_rmax);
+        return nnmtp_run(true, true, false, NNMTP_PASS);
+    });
+    m.def("nnMtpToEFOp", [](NNMTP_ARGS) -> variable_list {
+        require_no_zbl(zbl_rmax);
+        return nnmtp_run(true, false, false, NNMTP_PASS);
+    });
+    m.def("nnMtpToEsitesOp", [](NNMTP_ARGS) -> variable_list {
+        require_no_zbl(zbl_rmax);
+        for (auto* t : {&coeffs, &w0, &w1, &bias})
+            TORCH_CHECK(!(at::GradMode::is_enabled() && t->requires_grad()),
+                        "nnMtpToEsitesOp: the backward to coeffs, w0, w1, type_bias is not implemented in this build");
+        return nnmtp_run(false, false, true, NNMTP_PASS);
+    });
+    m.def("nnMtpToDescriptorsOp",
+          [](int64_t K, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times,
+             const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist,
+             const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+             const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax,
+             double rmin) -> variable_list {
+              return nnmtp_descriptors(K, coeffs, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                                       bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin);
+          });
+    m.def("nnMtpToLossOp",
+          [](double, double, double, const at::Tensor&, const at::Tensor&, const at::Tensor&,
+             NNMTP_ARGS) -> variable_list {
+              TORCH_CHECK(false, "nnMtpToLossOp is not implemented in this build");
+          });
+    m.def("nnMtpToEFLossOp",
+          [](double, double, const at::Tensor&, const at::Tensor&, NNMTP_ARGS) -> variable_list {
+              TORCH_CHECK(false, "nnMtpToEFLossOp is not implemented in this build");
+          });
+}

@@ -61,7 +61,14 @@ struct MtpArgs {
     T* desc;           // [B, P, n_scalar] scalar moments, or null
     int energy_only;   // stop after the energy: no adjoint, no pair derivatives
     int cE_per_atom;   // loss-gradient mode: cE is indexed per row (weights of the site energies)
+    // neural-network read-out (source/descriptor/nnmtp/include/nnMtp.h:470-507) when H > 0:
+    // e_i = bias + sum_p w1[t,p] tanh(sum_k w0[t,p,k] (M_k - q_shift[k]) / q_scaler[k]); `lin` is unused
+    int H;
+    const T *w0, *w1, *q_shift;
 };
+
+__device__ __forceinline__ float tanh_t(float x) { return tanhf(x); }
+__device__ __forceinline__ double tanh_t(double x) { return tanh(x); }
 
 __device__ __forceinline__ float sqrt_t(float x) { return sqrtf(x); }
 __device__ __forceinline__ double sqrt_t(double x) { return sqrt(x); }
@@ -340,9 +347,39 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     // ---- products, energy, adjoint ------------------------------------------------------------
     sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
     T e_part = (T)0;
-    for (int s = lane; s < p.n_scalar; s += NT) {
-        e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
-        A[p.mapping[s]] = a.lin[s] / a.q_scaler[s];
+    if (!LOSS && a.H > 0) {
+        // one tanh layer of the centre's species on the shifted, scaled scalar moments; the
+        // adjoint is seeded with dE_i/dM_k = sum_p w1_p tanh'(h_p) w0_pk / q_scaler_k
+        const int S = p.n_scalar, H = a.H;
+        T* qv = pq;                           // [S] network inputs
+        T* hv = pq + S;                       // [H] pre-activations, then w1 * tanh'
+        const T* w0 = a.w0 + (size_t)ti * H * S;
+        const T* w1 = a.w1 + (size_t)ti * H;
+        for (int s = lane; s < S; s += NT) qv[s] = (M[p.mapping[s]] - a.q_shift[s]) / a.q_scaler[s];
+        __syncthreads();
+        for (int n = lane >> 6; n < H; n += NT / 64) {          // one wave per neuron
+            T acc = (T)0;
+            for (int k = lane & 63; k < S; k += 64) acc += w0[(size_t)n * S + k] * qv[k];
+            acc = wave_sum(acc);
+            if ((lane & 63) == 0) hv[n] = acc;
+        }
+        __syncthreads();
+        for (int n = lane; n < H; n += NT) {
+            const T th = tanh_t(hv[n]);
+            e_part += w1[n] * th;
+            hv[n] = w1[n] * ((T)1 - th * th);
+        }
+        __syncthreads();
+        for (int k = lane; k < S; k += NT) {
+            T acc = (T)0;
+            for (int n = 0; n < H; n++) acc += hv[n] * w0[(size_t)n * S + k];
+            A[p.mapping[k]] = acc / a.q_scaler[k];
+        }
+    } else {
+        for (int s = lane; s < p.n_scalar; s += NT) {
+            e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
+            A[p.mapping[s]] = a.lin[s] / a.q_scaler[s];
+        }
     }
     if (!LOSS && (a.e_sites || a.desc)) {
         if (a.desc)                                          // linearMtp.h:884-885: unscaled scalar moments
@@ -728,13 +765,14 @@ int table_entries(const MtpPlanDevice& p, int K, bool loss)
 }
 
 template <typename T>
-size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K)
+size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H)
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
     const size_t tabs = std::max((size_t)MTP_NC * E + (size_t)(256 / 32) * 32 * 4, (size_t)p.max_level_slots * (loss ? 2 : 1));
     size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs;
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
+    else if (H > 0) n += (size_t)p.n_scalar + H;     // network inputs and pre-activations
     return n * sizeof(T) + 64;      // the packed basic-moment table (4 n_basic bytes) follows
 }
 
@@ -749,7 +787,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
                 plan->d.nmus);
     A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0 && U >= 1 && nghost >= 0, A2P_ERR_INVALID, "mtp: bad shape");
     A2P_REQUIRE(rmax > rmin && rmin >= 0, A2P_ERR_INVALID, "mtp: need 0 <= rmin < rmax");
-    A2P_REQUIRE(coeffs && lin && bias && q_scaler && binum && bilist && bnumneigh && bfirstneigh && brcs &&
+    A2P_REQUIRE(coeffs && bias && q_scaler && binum && bilist && bnumneigh && bfirstneigh && brcs &&
                     btypes, A2P_ERR_INVALID, "mtp: null input pointer");
     A2P_REQUIRE((long long)B * P * U < (1ll << 31), A2P_ERR_INVALID, "mtp: batch too large");
     a.p = plan->d;
@@ -761,6 +799,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
     a.force = nullptr; a.pair_g = nullptr; a.partial = nullptr;
     a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
+    a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
     if (rc) return rc;
@@ -771,7 +810,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
 template <typename T, bool LOSS>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
-    const size_t lds_main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K) + 15) / 16 * 16;
+    const size_t lds_main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H) + 15) / 16 * 16;
     const size_t lds = lds_main + (size_t)a.p.n_basic * sizeof(unsigned);
     const_cast<MtpArgs<T>&>(a).lds_basic_off = (int)lds_main;
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
@@ -788,11 +827,32 @@ int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
     return A2P_OK;
 }
 
+// network of the neural-network MTP: w0[ntypes, H, n_scalar], w1[ntypes, H], q_shift[n_scalar]
+template <typename T>
+struct MtpNet {
+    int H;
+    const T *w0, *w1, *q_shift;
+};
+
+template <typename T>
+int set_net(MtpArgs<T>& a, const MtpNet<T>* net)
+{
+    if (!net) {
+        A2P_REQUIRE(a.lin, A2P_ERR_INVALID, "mtp: null linear_coeffs");
+        return A2P_OK;
+    }
+    A2P_REQUIRE(net->H >= 1 && net->w0 && net->w1 && net->q_shift, A2P_ERR_INVALID,
+                "nnmtp: need num_neurons >= 1 and non-null w0, w1, q_shifter");
+    a.H = net->H; a.w0 = net->w0; a.w1 = net->w1; a.q_shift = net->q_shift;
+    return A2P_OK;
+}
+
 template <typename T>
 int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus,
             int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
             const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
-            const int* btypes, T* etot, T* force, T* virial, hipStream_t stream)
+            const int* btypes, T* etot, T* force, T* virial, hipStream_t stream,
+            const MtpNet<T>* net = nullptr, T* e_sites = nullptr)
 {
     MtpPlan* plan = nullptr;
     int rc = plan_check(handle, &plan);
@@ -801,7 +861,10 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
     rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
                    binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
     if (rc) return rc;
+    rc = set_net(a, net);
+    if (rc) return rc;
     if (B == 0 || P == 0) return A2P_OK;
+    a.e_sites = e_sites;
     a.E = table_entries<T>(a.p, K, false);
     void* ws = nullptr;
     rc = ws_get(WS_PARTIAL, (size_t)B * P * 10 * sizeof(double), &ws);
@@ -844,8 +907,8 @@ int mtp_loss(void* handle, double e_w, double f_w, double v_w, const T* e_dft, c
              T* bloss, T* rmse, T* etot, T* force, T* virial, T* dcoeffs, T* dlin, T* dbias,
              hipStream_t stream)
 {
-    A2P_REQUIRE(e_dft && f_dft && v_dft && bloss && etot && force && virial, A2P_ERR_INVALID,
-                "mtp loss: null label or output pointer");
+    A2P_REQUIRE(e_dft && f_dft && v_dft && bloss && etot && force && virial && lin, A2P_ERR_INVALID,
+                "mtp loss: null label, parameter or output pointer");
     int rc = mtp_efv<T>(handle, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, 0,
                         binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, stream);
     if (rc) return rc;
@@ -895,7 +958,7 @@ template <typename T>
 int mtp_esites(void* handle, int K, double scaling, const T* coeffs, const T* lin, const T* bias, int nmus,
                int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
                const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
-               const int* btypes, T* e_sites, T* desc, hipStream_t stream)
+               const int* btypes, T* e_sites, T* desc, hipStream_t stream, const MtpNet<T>* net = nullptr)
 {
     MtpPlan* plan = nullptr;
     int rc = plan_check(handle, &plan);
@@ -904,6 +967,8 @@ int mtp_esites(void* handle, int K, double scaling, const T* coeffs, const T* li
     MtpArgs<T> a;
     rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
                    binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    rc = set_net(a, net);
     if (rc) return rc;
     if (B == 0 || P == 0) return A2P_OK;
     a.E = table_entries<T>(a.p, K, false);
@@ -923,7 +988,7 @@ int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T
     MtpPlan* plan = nullptr;
     int rc = plan_check(handle, &plan);
     if (rc) return rc;
-    A2P_REQUIRE(gout && (dcoeffs || dlin || dbias), A2P_ERR_INVALID, "mtp e_sites backward: null pointer");
+    A2P_REQUIRE(gout && lin && (dcoeffs || dlin || dbias), A2P_ERR_INVALID, "mtp e_sites backward: null pointer");
     MtpArgs<T> a;
     rc = fill_args(a, plan, K, scaling, coeffs, lin, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, nghost,
                    binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
@@ -1036,6 +1101,22 @@ int a2p_mtp_esites_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int ng
     return a2p::mtp_esites<float>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, e_sites, descriptors,
                                   (hipStream_t)stream);
 }
+#define NNMTP_ENTRY(T, SUFFIX)                                                                                  \
+    int a2p_nnmtp_efv_##SUFFIX(void* plan, int K, int H, const T* coeffs, const T* w0, const T* w1, const T* bias, \
+                               int nmus, int ntypes, const T* q_shifter, const T* q_scaler, double rmax,          \
+                               double rmin, int B, int P, int U, int nghost, MTP_BATCH(T), T* etot, T* force,      \
+                               T* virial, T* e_sites, void* stream)                                               \
+    {                                                                                                           \
+        a2p::MtpNet<T> net{H, w0, w1, q_shifter};                                                                 \
+        if (!etot && !force && !virial)                                                                           \
+            return a2p::mtp_esites<T>(plan, K, 1.0, coeffs, nullptr, bias, nmus, ntypes, q_scaler, rmax, rmin, B, \
+                                      P, U, nghost, MTP_BATCH_PASS, e_sites, nullptr, (hipStream_t)stream, &net); \
+        return a2p::mtp_efv<T>(plan, K, 1.0, coeffs, nullptr, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U,   \
+                               nghost, MTP_BATCH_PASS, etot, force, virial, (hipStream_t)stream, &net, e_sites);  \
+    }
+NNMTP_ENTRY(double, f64)
+NNMTP_ENTRY(float, f32)
+
 int a2p_mtp_esites_bwd_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
                            const double* grad_e_sites, double* dcoeffs, double* dlinear, double* dbias, void* stream)
 {

@@ -625,6 +625,113 @@ def linearMtpToDescriptorsOp(chebyshev_size, scaling, coeffs, alpha_moments_coun
 
 
 # --------------------------------------------------------------------------------------------
+# neural-network MTP  (source/descriptor/nnmtp/bind/nnmtp_bind.cc:193-430)
+# --------------------------------------------------------------------------------------------
+def _nnmtp_call(want, chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, alpha_index_basic,
+                alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, validate):
+    """want: subset of {"e", "f", "v", "es"}.  Returns (etot, force, virial, e_sites), None where not asked."""
+    _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
+         "brcs must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = brcs.dtype, brcs.device
+    _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
+    _req(brcs.is_contiguous(), "brcs must be contiguous")
+    for name, t in (("coeffs", coeffs), ("w0", w0), ("w1", w1), ("type_bias", type_bias),
+                    ("q_shifter", q_shifter), ("q_scaler", q_scaler)):
+        _check_float(name, t, dtype, device)
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh), ("btypes", btypes)):
+        _check_int(name, t, device)
+    nghost = int(nghost)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost)
+    ntypes = int(type_map.numel())
+    _req(ntypes > 0, "type_map is empty")
+    plan, n_scalar = _mtp_plan(alpha_moments_count, alpha_index_basic, alpha_index_times,
+                               alpha_moment_mapping, device)
+    _req(coeffs.numel() == ntypes * ntypes * int(nmus) * int(chebyshev_size), "coeffs size mismatch")
+    _req(w1.numel() % ntypes == 0 and w1.numel() > 0, "w1 must have ntypes * num_neurons elements")
+    H = w1.numel() // ntypes                                    # nnMtpOp.cc: num_neurons = w1.size(1)
+    _req(w0.numel() == ntypes * H * n_scalar, "w0 has %d elements, expected ntypes*H*alpha_scalar_moments = %d"
+         % (w0.numel(), ntypes * H * n_scalar))
+    _req(q_shifter.numel() == n_scalar and q_scaler.numel() == n_scalar,
+         "q_shifter and q_scaler must have alpha_scalar_moments = %d elements" % n_scalar)
+    _req(type_bias.numel() == ntypes, "type_bias size mismatch")
+    if validate:
+        _validate_batch(binum, bnumneigh, U, P)
+    z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
+    etot = z(B) if "e" in want else None
+    force = z(B, P + nghost, 3) if "f" in want else None
+    virial = z(B, 9) if "v" in want else None
+    e_sites = z(B, P) if "es" in want else None
+    L = _lib.lib()
+    fn = L.a2p_nnmtp_efv_f32 if dtype == torch.float32 else L.a2p_nnmtp_efv_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0), _ptr(w1), _ptr(type_bias),
+                _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_shifter), _ptr(q_scaler), _c.c_double(rmax),
+                _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
+                _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(etot),
+                _ptr(force), _ptr(virial), _ptr(e_sites), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return etot, force, virial, e_sites
+
+
+def nnMtpToEFVOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, alpha_index_basic,
+                 alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                 btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
+                 zbl_cks=None, zbl_dks=None, validate=True):
+    """[E[B], F[B, P+nghost, 3], V[B, 9]]; nnmtp_bind.cc:258-322, nnMtpOp.cc:2785-3010."""
+    _no_zbl(zbl_rmax)
+    e, f, v, _ = _nnmtp_call("efv", chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
+                             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                             bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
+                             q_scaler, validate)
+    return [e, f, v]
+
+
+def nnMtpToEFOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, alpha_index_basic,
+                alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
+                zbl_cks=None, zbl_dks=None, validate=True):
+    """[E[B], F[B, P+nghost, 3]]; nnmtp_bind.cc:193-256."""
+    _no_zbl(zbl_rmax)
+    e, f, _, _ = _nnmtp_call("ef", chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
+                             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                             bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
+                             q_scaler, validate)
+    return [e, f]
+
+
+def nnMtpToEsitesOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, alpha_index_basic,
+                    alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                    btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
+                    zbl_cks=None, zbl_dks=None, validate=True):
+    """[e_sites[B, P]] in row order; nnmtp_bind.cc:370-430.  Forward only: the reference's backward
+    to coeffs, w0, w1, type_bias (nnMtp.h:756-990) is not part of this build, so parameters that
+    require grad are refused instead of returning a result that silently carries no gradient."""
+    _no_zbl(zbl_rmax)
+    for name, t in (("coeffs", coeffs), ("w0", w0), ("w1", w1), ("type_bias", type_bias)):
+        _req(not (torch.is_grad_enabled() and t.requires_grad),
+             "nnMtpToEsitesOp: the backward w.r.t. %s is not implemented in this build" % name)
+    _, _, _, es = _nnmtp_call(("es",), chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
+                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                              bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
+                              q_scaler, validate)
+    return [es]
+
+
+def nnMtpToDescriptorsOp(chebyshev_size, coeffs, alpha_moments_count, alpha_index_basic, alpha_index_times,
+                         alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                         type_map, nghost, rmax, rmin, validate=True):
+    """[descriptors[B, P, alpha_scalar_moments]]: the scalar moments, i.e. the linear-MTP descriptors
+    at scaling 1 (nnmtp_bind.cc:323-368, nnMtp.h:570-645)."""
+    return linearMtpToDescriptorsOp(chebyshev_size, 1.0, coeffs, alpha_moments_count, alpha_index_basic,
+                                    alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh,
+                                    bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, validate)
+
+
+# --------------------------------------------------------------------------------------------
 # fvt  (source/fvt/bind/fvt_sr_op_bind.cc:9-46)
 # --------------------------------------------------------------------------------------------
 def _fvt_fn(name, dtype):

@@ -185,6 +185,21 @@ def mtp_model(tables, ntypes, chebyshev_size, rmax, rmin, seed, lo=-0.1, hi=0.1,
     return m
 
 
+def nnmtp_model(tables, ntypes, chebyshev_size, num_neurons, rmax, rmin, seed, lo=-0.1, hi=0.1,
+                type_map=None):
+    """Neural-network MTP parameters: the radial coefficients of mtp_model, one tanh layer per
+    species (w0[ntypes, H, S], w1[ntypes, H], no hidden bias), a shift and a scale per scalar moment."""
+    S = len(tables["alpha_moment_mapping"])
+    m = mtp_model(tables, ntypes, chebyshev_size, rmax, rmin, seed, lo, hi, type_map)
+    del m["linear_coeffs"], m["scaling"]
+    m.update(num_neurons=num_neurons,
+             w0=rng_normal(seed + 3, ntypes * num_neurons * S, 0, 0.3),
+             w1=rng_normal(seed + 4, ntypes * num_neurons, 0, 0.3),
+             q_shifter=rng_uniform(seed + 5, S, -0.05, 0.05),
+             q_scaler=rng_uniform(seed + 6, S, 0.7, 1.4))
+    return m
+
+
 def mtp_model_closed_form(tables):
     """Parameter fill of the reference's linear-MTP unit test
     (source/descriptor/mtpr/tests/test_linearMtp.cc:142-156, 272-279, 317-324; level 16,

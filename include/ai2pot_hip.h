@@ -206,6 +206,31 @@ int a2p_mtp_esites_bwd_f32(void* plan, int chebyshev_size, double scaling, const
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Neural-network MTP: energy, force, virial and site energies -- replaces the compute of
+ * torch.ops.nnmtp.nnMtpToEFVOp / nnMtpToEFOp / nnMtpToEsitesOp (forward)
+ * (source/descriptor/nnmtp/bind/nnmtp_bind.cc:193-322, 370-430; src/nnMtpOp.cc:2785-3190;
+ *  include/nnMtp.h:378-567 find_efv, :648-753 find_e_sites).  The moments are those of the linear
+ * MTP at scaling 1 (nnmtp/include/mtpBasis.h), so `plan` comes from a2p_mtp_plan_create; the
+ * read-out is one tanh layer per centre species without hidden bias:
+ *   e_i = type_bias[t] + sum_p w1[t,p] tanh( sum_k w0[t,p,k] (M_k - q_shifter[k]) / q_scaler[k] ).
+ * w0[ntypes, num_neurons, n_scalar], w1[ntypes, num_neurons].  Outputs as a2p_mtp_efv_*; e_sites[B, P]
+ * in row order (may be NULL); with etot, force and virial all NULL only the site energies are
+ * computed.  nnMtpToDescriptorsOp is a2p_mtp_esites_* with scaling 1 (nnMtp.h:570-645).
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nnmtp_efv_f64(void* plan, int chebyshev_size, int num_neurons, const double* coeffs, const double* w0,
+                      const double* w1, const double* type_bias, int nmus, int ntypes, const double* q_shifter,
+                      const double* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                      int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                      const int* bfirstneigh, const double* brcs, const int* btypes, double* etot, double* force,
+                      double* virial, double* e_sites, void* stream);
+int a2p_nnmtp_efv_f32(void* plan, int chebyshev_size, int num_neurons, const float* coeffs, const float* w0,
+                      const float* w1, const float* type_bias, int nmus, int ntypes, const float* q_shifter,
+                      const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                      int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                      const int* bfirstneigh, const float* brcs, const int* btypes, float* etot, float* force,
+                      float* virial, float* e_sites, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * NEP training loss, forward and analytic backward -- replaces the compute of
  * torch.ops.nep.nepToLossOp and torch.ops.nep.nepToEFLossOp
  * (source/descriptor/nep/bind/nep_bind.cc:136-276; src/nepOp.cc:2359-3484;

@@ -5,7 +5,8 @@ may import this package; the product (``ai2pot_amd``) never does.
 
 Two families of functions with identical NumPy signatures:
 
-* ``nblist``, ``nep_efv``, ``nep_loss``, ``mtp_efv``, ``mtp_loss_step``, ``fvt_force``, ``fvt_virial`` --
+* ``nblist``, ``nep_efv``, ``nep_loss``, ``mtp_efv``, ``mtp_loss_step``, ``mtp_esites``, ``mtp_esites_bwd``,
+  ``nnmtp_efv``, ``fvt_force``, ``fvt_virial`` --
   this repository's own C++ restatement of the reference algorithm (``oracle/src``,
   ``liboracle.so``), each function citing the reference file:line it follows;
 * ``ref_*`` -- the reference's own headers compiled where they lie (``oracle/_ref/*.so``,
@@ -395,6 +396,40 @@ def ref_mtp_esites_bwd(model, nb, gout):
 
 def mtp_esites_bwd(model, nb, gout):
     return _mtp_esites_bwd(oracle_lib(), "orc_mtp", model, nb, gout)
+
+
+# ----------------------------------------------------------------------------------------
+# neural-network MTP (fp64)
+# ----------------------------------------------------------------------------------------
+def _nnmtp_efv(lib, prefix, model, nb, want_esites=True):
+    coeffs = _c(model["coeffs"], np.float64)
+    w0, w1 = _c(model["w0"], np.float64), _c(model["w1"], np.float64)
+    bias = _c(model["type_bias"], np.float64)
+    basic = _c(model["alpha_index_basic"], np.int32)
+    times = _c(model["alpha_index_times"], np.int32)
+    mapping = _c(model["alpha_moment_mapping"], np.int32)
+    shift, scale = _c(model["q_shifter"], np.float64), _c(model["q_scaler"], np.float64)
+    type_map = _c(model["type_map"], np.int32)
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    e, f, v = np.zeros(B), np.zeros((B, P + nghost, 3)), np.zeros((B, 9))
+    es = np.zeros((B, P)) if want_esites else None
+    fn = getattr(lib, prefix + "_efv_f64")
+    fn.restype = None
+    fn(_p(e), _p(f), _p(v), _p(es), _I(model["chebyshev_size"]), _I(model["num_neurons"]), _p(coeffs), _p(w0),
+       _p(w1), _p(bias), _I(model["alpha_moments_count"]), _I(basic.shape[0]), _p(basic), _I(times.shape[0]),
+       _p(times), _I(mapping.size), _p(mapping), _I(model["nmus"]), _I(B), _I(P), _p(binum), _p(bilist),
+       _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes), _I(type_map.size), _p(type_map), _I(U), _I(nghost),
+       _D(model["rmax"]), _D(model["rmin"]), _p(shift), _p(scale))
+    return e, f, v, es
+
+
+def ref_nnmtp_efv(model, nb):
+    """(E[B], F[B, P+nghost, 3], V[B, 9], e_sites[B, P]) by the reference's NNMtp."""
+    return _nnmtp_efv(_load("_ref/libref_nnmtp.so"), "ref_nnmtp", model, nb)
+
+
+def nnmtp_efv(model, nb):
+    return _nnmtp_efv(oracle_lib(), "orc_nnmtp", model, nb)
 
 
 # ----------------------------------------------------------------------------------------

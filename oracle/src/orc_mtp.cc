@@ -15,6 +15,7 @@
 // function end values (tests/test_basis.cc:106-111); linearity of E in linear_coeffs.
 #include <cmath>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 namespace {
@@ -36,6 +37,13 @@ inline double val(Dual x) { return x.v; }
 struct Tables {
     int n_moms, n_basic, n_times, n_scalar, nmus;
     const int *basic, *times, *mapping;
+};
+
+// Read-out of the neural-network MTP (source/descriptor/nnmtp/include/nnMtp.h:470-507): one tanh
+// layer per centre species on the shifted and scaled scalar moments, no hidden bias.
+struct NNReadout {
+    int H;
+    const double *w0, *w1, *shift;     // w0[ntypes, H, n_scalar], w1[ntypes, H], shift[n_scalar]
 };
 
 // f_k(r) = scaling * s(u) * T_k(x) and its r-derivative (basis.h:154-196, 351-381, 620-637)
@@ -68,7 +76,7 @@ void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeff
              const S* bias, const Tables& t, int inum, const int* ilist, const int* numneigh,
              const int* firstneigh, const double* rcs, const int* types, int ntypes, int U,
              int nforce, double rmax, double rmin, const double* q_scaler, S* e_sites = nullptr,
-             S* desc = nullptr)
+             S* desc = nullptr, const NNReadout* net = nullptr)
 {
     etot = S(0);
     for (int i = 0; i < nforce * 3; i++) force[i] = S(0);   // linearMtp.h:228-230
@@ -113,13 +121,31 @@ void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeff
             M[q[3]] += S((double)q[2]) * M[q[0]] * M[q[1]];
         }
         S e = bias[ti];                                        // linearMtp.h:281-285
-        for (int s = 0; s < t.n_scalar; s++) e += lin[s] * M[t.mapping[s]] / S(q_scaler[s]);
+        std::fill(adj.begin(), adj.end(), S(0));               // linearMtp.h:292-306
+        if constexpr (std::is_same<S, double>::value) {
+            if (net) {                                         // nnMtp.h:470-507
+                const double* w0 = net->w0 + (size_t)ti * net->H * t.n_scalar;
+                const double* w1 = net->w1 + (size_t)ti * net->H;
+                for (int p = 0; p < net->H; p++) {
+                    double h = 0;
+                    for (int s = 0; s < t.n_scalar; s++)
+                        h += w0[p * t.n_scalar + s] * (M[t.mapping[s]] - net->shift[s]) / q_scaler[s];
+                    // nnMtpUtils.h:54-71: tanh and its derivative from exponentials
+                    const double th = (std::exp(h) - std::exp(-h)) / (std::exp(h) + std::exp(-h));
+                    e += w1[p] * th;
+                    for (int s = 0; s < t.n_scalar; s++)
+                        adj[t.mapping[s]] += w1[p] * (1 - th * th) * w0[p * t.n_scalar + s] / q_scaler[s];
+                }
+            }
+        }
+        if (!net) {
+            for (int s = 0; s < t.n_scalar; s++) e += lin[s] * M[t.mapping[s]] / S(q_scaler[s]);
+            for (int s = 0; s < t.n_scalar; s++) adj[t.mapping[s]] = lin[s] / S(q_scaler[s]);
+        }
         etot += e;
         if (e_sites) e_sites[ii] = e;                          // linearMtp.h:594-599 (row order)
         if (desc)                                              // linearMtp.h:884-885 (unscaled moments)
             for (int s = 0; s < t.n_scalar; s++) desc[(size_t)ii * t.n_scalar + s] = M[t.mapping[s]];
-        std::fill(adj.begin(), adj.end(), S(0));               // linearMtp.h:292-306
-        for (int s = 0; s < t.n_scalar; s++) adj[t.mapping[s]] = lin[s] / S(q_scaler[s]);
         for (int i = t.n_times - 1; i >= 0; i--) {
             const int* q = &t.times[i * 4];
             S w = adj[q[3]] * S((double)q[2]);
@@ -327,5 +353,26 @@ void orc_mtp_esites_bwd_f64(double* dcoeffs, double* dlin, double* dbias, const 
                 else dbias[(size_t)b * ntypes + p - ncoef - n_scalar] = acc;
             }
     }
+}
+
+// Neural-network MTP (source/descriptor/nnmtp): E/F/V, site energies e_sites[B, P] (may be null)
+// with the moments of the linear MTP at scaling 1 (nnmtp/include/mtpBasis.h differs from
+// mtpr/include/mtpBasis.h only by that factor) and the tanh read-out of nnMtp.h:378-567, 648-753.
+void orc_nnmtp_efv_f64(double* betot, double* bforce, double* bvirial, double* e_sites, int K, int H,
+                       const double* coeffs, const double* w0, const double* w1, const double* bias, int n_moms,
+                       int n_basic, const int* basic, int n_times, const int* times, int n_scalar,
+                       const int* mapping, int nmus, int B, int P, const int* binum, const int* bilist,
+                       const int* bnumneigh, const int* bfirstneigh, const double* brcs, const int* btypes,
+                       int ntypes, const int* type_map, int U, int nghost, double rmax, double rmin,
+                       const double* q_shifter, const double* q_scaler)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    NNReadout nn{H, w0, w1, q_shifter};
+    for (int b = 0; b < B; b++)
+        efv_one<double>(betot[b], &bforce[(size_t)b * (P + nghost) * 3], &bvirial[b * 9], K, 1.0, coeffs, nullptr,
+                        bias, t, binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P],
+                        &bfirstneigh[(size_t)b * P * U], &brcs[(size_t)b * P * U * 3],
+                        &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost, rmax, rmin, q_scaler,
+                        e_sites ? &e_sites[(size_t)b * P] : nullptr, nullptr, &nn);
 }
 }

@@ -107,6 +107,23 @@ def mtp_cases():
     print("mtp.npz")
 
 
+def nnmtp_cases():
+    """Neural-network MTP: E/F/V and site energies of the reference's NNMtp (fp64)."""
+    out = {}
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    for level, nt, H in ((8, 2, 7), (16, 3, 20)):
+        ty = synth.rng_randint(22, 48, nt)
+        m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.8, 3200 + level)
+        o = oracle.ref_nblist(lat, ty, pos, 5.0, 100)
+        nb = synth.pack_batch([o, o])
+        nb["brcs"][1] *= 1.01
+        e, f, v, es = oracle.ref_nnmtp_efv(m, nb)
+        tag = "L%02d" % level
+        out.update({tag + "/E": e, tag + "/F": f, tag + "/V": v, tag + "/esites": es})
+    np.savez_compressed(os.path.join(HERE, "nnmtp.npz"), **out)
+    print("nnmtp.npz")
+
+
 def nep_loss_cases():
     """Two small structures, two species: the reference's loss forward + backward (fp64)."""
     out = {}
@@ -157,9 +174,11 @@ def fvt_cases():
 
 
 if __name__ == "__main__":
+    # usage: make_golden.py [nblist nep mtp nnmtp nep_loss fvt]; default all.  The reference sums
+    # energies and forces with OpenMP atomics, so a regenerated floating-point fixture can differ
+    # from the committed one in the last bits: regenerate only what changed.
     assert oracle.ref_available("nblist"), "build oracle/_ref first: make -C oracle ref"
-    nblist_cases()
-    nep_cases()
-    mtp_cases()
-    nep_loss_cases()
-    fvt_cases()
+    cases = dict(nblist=nblist_cases, nep=nep_cases, mtp=mtp_cases, nnmtp=nnmtp_cases, nep_loss=nep_loss_cases,
+                 fvt=fvt_cases)
+    for name in (sys.argv[1:] or list(cases)):
+        cases[name]()

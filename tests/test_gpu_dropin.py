@@ -20,7 +20,7 @@ LIBDIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))
 @pytest.fixture(scope="module")
 def dropin():
     import torch
-    for name in ("libnep_bind.so", "libmtpr_bind.so", "libfvt_sr_op_bind.so"):
+    for name in ("libnep_bind.so", "libmtpr_bind.so", "libnnmtp_bind.so", "libfvt_sr_op_bind.so"):
         path = os.path.join(LIBDIR, name)
         assert os.path.exists(path), "%s missing: run python -m ai2pot_amd.build --bind" % path
         torch.ops.load_library(path)
@@ -175,6 +175,38 @@ def test_mtpr_ops(oracle, dropin, tmp_path):
     rc, rl, rb = oracle.mtp_esites_bwd(m, nb, gout)
     assert close(params3[0].grad.cpu().numpy(), rc.sum(0)) and close(params3[1].grad.cpu().numpy(), rl.sum(0))
     assert close(params3[2].grad.cpu().numpy(), rb.sum(0))
+
+
+def test_nnmtp_ops(oracle, dropin, tmp_path):
+    import torch
+    from test_gpu_nnmtp import model_to_device, op_args
+    d = tmp_path / "_data" / "MTP_templates"
+    d.mkdir(parents=True)
+    mtp_param.write_almtp(str(d / "10.almtp"), mtp_param.mtp_param(10))
+    os.environ.pop("AI2POT_PATH", None)
+    torch.ops.nnmtp.set_ai2pot_path(str(tmp_path))
+    p = torch.ops.nnmtp.mtpParamOp(10)
+    assert len(p) == 7 and int(p[0]) == mtp_param.mtp_param(10)["alpha_moments_count"]
+    lat, pos, ty, o = small(oracle, n=60, nt=2, rcut=5.0, dtype=np.float64)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.02
+    m = synth.nnmtp_model(mtp_param.mtp_param(10), 2, 8, 12, 5.0, 1.0, 77)
+    md = model_to_device(m, torch.float64)
+    z = torch.zeros(16, dtype=torch.float64, device="cuda:0")
+    args = op_args(m, md, to_device(nb, torch.float64)) + (0.0, 0.0, z, z)
+    close = lambda a, b: np.abs(a.cpu().numpy() - b).max() <= 1e-10 * np.abs(b).max()
+    er, fr, vr, esr = oracle.nnmtp_efv(m, nb)
+    e, f, v = torch.ops.nnmtp.nnMtpToEFVOp(*args)
+    assert close(e, er) and close(f, fr) and close(v, vr)
+    assert len(torch.ops.nnmtp.nnMtpToEFOp(*args)) == 2
+    assert close(torch.ops.nnmtp.nnMtpToEsitesOp(*args)[0], esr)
+    desc = torch.ops.nnmtp.nnMtpToDescriptorsOp(*(args[:2] + args[5:20]))[0]
+    lin = dict(m); lin["scaling"] = 1.0; lin["linear_coeffs"] = np.zeros(m["q_scaler"].size)
+    assert close(desc, oracle.mtp_esites(lin, nb)[1])
+    with pytest.raises(RuntimeError):                      # training operators are declared and refuse
+        torch.ops.nnmtp.nnMtpToEFLossOp(1.0, 1.0, e, f, *args)
+    with pytest.raises(RuntimeError):
+        torch.ops.nnmtp.nnMtpToEsitesOp(*(args[:2] + (md["w0"].clone().requires_grad_(True),) + args[3:]))
 
 
 def test_fvt_ops(oracle, dropin):

@@ -1,0 +1,98 @@
+"""Pins the CPU oracle's neural-network MTP (E/F/V and site energies): the reference's committed
+outputs, finite differences of the energy, the linear-MTP limit of a small network and the
+exponential form of tanh the reference uses.  The reference's own unit tests for this model
+(source/descriptor/nnmtp/tests/test_nnMtp.cc) print values and assert nothing, so there is no
+known answer to take from them."""
+import os
+
+import numpy as np
+import pytest
+
+from ai2pot_amd import mtp_param, synth
+
+HERE = os.path.dirname(__file__)
+
+
+def small_batch(oracle, level, nt, H):
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    ty = synth.rng_randint(22, 48, nt)
+    m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.8, 3200 + level)
+    o = oracle.nblist(lat, ty, pos, 5.0, 100)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.01
+    return m, nb
+
+
+@pytest.mark.parametrize("level,nt,H", [(8, 2, 7), (16, 3, 20)])
+def test_against_golden(oracle, level, nt, H):
+    with np.load(os.path.join(HERE, "golden", "nnmtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+    m, nb = small_batch(oracle, level, nt, H)
+    e, f, v, es = oracle.nnmtp_efv(m, nb)
+    for got, key in ((e, "E"), (f, "F"), (v, "V"), (es, "esites")):
+        assert np.abs(got - g[key]).max() <= 1e-12 * np.abs(g[key]).max(), key
+    assert np.abs(es.sum(1) - e).max() < 1e-12 * np.abs(e).max()
+
+
+def test_energy_force_virial_finite_differences(oracle):
+    lat, pos = synth.random_packed(30, [8.0, 8.5, 9.0], 2.0, 31)
+    ty = synth.rng_randint(32, 30, 2)
+    m = synth.nnmtp_model(mtp_param.mtp_param(10), 2, 8, 9, 4.0, 1.5, 77)
+
+    def efv(p, L=lat):
+        return oracle.nnmtp_efv(m, synth.pack_batch([oracle.nblist(L, ty, p, 4.0, 120)]))
+
+    e0, f0, v0, _ = efv(pos)
+    h = 1e-5
+    for i, a in ((0, 0), (11, 1), (29, 2)):
+        p = pos.copy(); p[i, a] += h
+        ep = efv(p)[0][0]
+        p[i, a] -= 2 * h
+        em = efv(p)[0][0]
+        assert abs(-(ep - em) / (2 * h) - f0[0, i, a]) < 1e-6 * max(1.0, abs(f0[0, i, a]))
+    assert np.abs(f0.sum(1)).max() < 1e-10 * np.abs(f0).max()
+    # virial = -dE/d(strain): scale the cell and the positions along x by (1 +- h)
+    for a in range(3):
+        sp, sm = np.eye(3), np.eye(3)
+        sp[a, a] += h; sm[a, a] -= h
+        ep = efv(pos @ sp, lat @ sp)[0][0]
+        em = efv(pos @ sm, lat @ sm)[0][0]
+        assert abs(-(ep - em) / (2 * h) - v0[0, 4 * a]) < 1e-6 * max(1.0, abs(v0[0, 4 * a]))
+
+
+def test_small_network_is_the_linear_model(oracle):
+    """tanh(x) = x - x^3/3 + ...: with weights scaled by eps the site energy minus the bias tends
+    to eps * sum_k (sum_p w1_p w0_pk) (M_k - shift_k) / scale_k, the linear MTP with those
+    coefficients; the cubic remainder is checked through its eps^3 scaling."""
+    m, nb = small_batch(oracle, 8, 2, 7)
+    one = dict(m); one["type_bias"] = np.zeros(2)
+    S = m["q_scaler"].size
+    rem = []
+    for eps in (1e-2, 5e-3):
+        net = dict(one); net["w0"] = eps * m["w0"]
+        _, _, _, es = oracle.nnmtp_efv(net, nb)
+        # the linear model has one coefficient vector for all species: evaluate per centre species
+        lin_es = np.zeros_like(es)
+        for t in range(2):
+            lin = (m["w1"].reshape(2, 7)[t][:, None] * net["w0"].reshape(2, 7, S)[t]).sum(0)
+            lm = dict(m); lm["scaling"] = 1.0; lm["linear_coeffs"] = lin
+            lm["type_bias"] = np.full(2, -(lin * m["q_shifter"] / m["q_scaler"]).sum())
+            est, _ = oracle.mtp_esites(lm, nb)
+            ti = np.take_along_axis(nb["btypes"], nb["bilist"], 1)
+            lin_es[ti == t] = est[ti == t]
+        rem.append(np.abs(es - lin_es).max())
+        assert rem[-1] < 50 * eps ** 3
+    assert 6.0 < rem[0] / rem[1] < 10.0          # halving eps divides the remainder by 8
+
+
+def test_reference_tanh_form(oracle):
+    """nnMtpUtils.h:54-71 builds tanh from exponentials; one neuron, one neighbour-free atom:
+    E = bias + w1 * tanh(-sum_k w0_k shift_k / scale_k)."""
+    t = mtp_param.mtp_param(6)
+    m = synth.nnmtp_model(t, 1, 8, 1, 5.0, 2.0, 5)
+    nb = dict(binum=np.array([1], np.int32), bilist=np.zeros((1, 1), np.int32),
+              bnumneigh=np.array([[0]], np.int32), bfirstneigh=np.zeros((1, 1, 1), np.int32),
+              brcs=np.zeros((1, 1, 1, 3)), btypes=np.zeros((1, 1), np.int32), nghost=0)
+    e, f, v, es = oracle.nnmtp_efv(m, nb)
+    want = m["type_bias"][0] + m["w1"][0] * np.tanh(-(m["w0"] * m["q_shifter"] / m["q_scaler"]).sum())
+    assert abs(e[0] - want) < 1e-15 and np.all(f == 0) and np.all(v == 0)
