@@ -31,6 +31,7 @@ namespace a2p {
 namespace {
 
 constexpr int MTP_NC = 32;        // neighbours per chunk
+constexpr int MTP_NGMAX = 16;     // most thread groups that share the basic moments of a chunk
 constexpr int MTP_KMAX = 16;      // radial basis size limit
 constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
 
@@ -73,86 +74,95 @@ __device__ __forceinline__ double tanh_t(double x) { return tanh(x); }
 __device__ __forceinline__ float sqrt_t(float x) { return sqrtf(x); }
 __device__ __forceinline__ double sqrt_t(double x) { return sqrt(x); }
 
-// Per-neighbour table for neighbours [c0, c0+nc) of the row, built by lanes j < nc.
+// Per-neighbour table for neighbours [c0, c0+nc) of the row.
 // Layout per neighbour (E entries of T): ux^0..kmax | uy^.. | uz^.. | g[nmus] | dg[nmus] |
 // ux uy uz 1/r | (loss mode) wx wy wz w.u | f[K] | df[K]
-template <typename T, bool LOSS>
-__device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, int lane, int nc, int c0,
-                                            const T* rcs, const int* first, const int* types, int ti,
-                                            int center, int b, int NF, int* nj_out, bool* valid_out,
-                                            T* d_out)
+// The work is spread over nc * (nmus + 3) tasks: task (role, j) computes for neighbour j either
+// one radial function g_role(r) with its derivative (role < nmus; coefficients from the LDS copy
+// `cf` of the centre species' block) or the powers of one unit-vector component (role - nmus),
+// so the table costs one Chebyshev recurrence of latency instead of nmus of them on nc lanes.
+// Lanes j < nc also return the neighbour's index, validity and displacement.
+template <typename T, bool LOSS, int NT>
+__device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, const T* cf, int lane, int nc, int c0,
+                                            const T* rcs, const int* first, const int* types, int center,
+                                            int b, int NF, int* nj_out, bool* valid_out, T* d_out)
 {
     const int kmax = a.p.kmax, nmus = a.p.nmus, K = a.K;
-    const int OX = 0, OY = kmax + 1, OZ = 2 * (kmax + 1), OG = 3 * (kmax + 1), ODG = OG + nmus,
-              OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
+    const int OG = 3 * (kmax + 1), ODG = OG + nmus, OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
     *valid_out = false;
     *nj_out = center;
     if (lane < nc) {
         const int jj = c0 + lane;
         const T x = rcs[jj * 3 + 0], y = rcs[jj * 3 + 1], z = rcs[jj * 3 + 2];
         d_out[0] = x; d_out[1] = y; d_out[2] = z;
-        const T r = sqrt_t(x * x + y * y + z * z);
         int nj = first[jj];
         if ((unsigned)nj >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); nj = center; }
-        int tj = types[nj];
-        if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
+        if ((unsigned)types[nj] >= (unsigned)a.ntypes) atomicOr(a.status, ST_BAD_TYPE);
         *nj_out = nj;
-        const bool valid = !(r > a.rmax);                // mtpBasis.h:457, linearMtp.h:316
-        *valid_out = valid;
-        T* t = tab + lane * a.E;
-        const T rinv = (T)1 / r;
-        const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
-        T px = (T)1, py = (T)1, pz = (T)1;
-        for (int k = 0; k <= kmax; k++) {
-            t[OX + k] = px; t[OY + k] = py; t[OZ + k] = pz;
-            px *= ux; py *= uy; pz *= uz;
-        }
-        t[OU + 0] = ux; t[OU + 1] = uy; t[OU + 2] = uz; t[OU + 3] = rinv;
+        *valid_out = !(sqrt_t(x * x + y * y + z * z) > a.rmax);      // mtpBasis.h:457, linearMtp.h:316
+    }
+    const int ntask = nc * (nmus + 3);
+    for (int task = lane; task < ntask; task += NT) {
+        const int role = task / nc, j = task - role * nc;
+        const int jj = c0 + j;
+        const T x = rcs[jj * 3 + 0], y = rcs[jj * 3 + 1], z = rcs[jj * 3 + 2];
+        const T r = sqrt_t(x * x + y * y + z * z);
+        T* t = tab + j * a.E;
         // radial functions, basis.h:154-196, 351-381, 620-637
         const T span = a.rmax - a.rmin;
         const T xx = ((T)2 * r - (a.rmax + a.rmin)) / span;
         const T dxx = (T)2 / span;
         const T u = (r - a.rmin) / span;
         T s = (T)0, ds = (T)0;
-        if (valid && r >= a.rmin && r < a.rmax) {
+        if (!(r > a.rmax) && r >= a.rmin && r < a.rmax) {
             s = u * u * u * ((T)-6 * u * u + (T)15 * u - (T)10) + (T)1;
             ds = (T)1 / span * ((T)-30 * u * u * u * u + (T)60 * u * u * u - (T)30 * u * u);
         }
-        T g[MTP_NMUS_MAX], dg[MTP_NMUS_MAX];
-#pragma unroll
-        for (int m = 0; m < MTP_NMUS_MAX; m++) { g[m] = (T)0; dg[m] = (T)0; }
-        const T* c = a.coeffs + (size_t)(ti * a.ntypes + tj) * nmus * K;
-        T t0 = (T)1, t1 = xx, d0 = (T)0, d1 = (T)1;
-        for (int k = 0; k < K; k++) {
-            T tv, dv;
-            if (k == 0) { tv = t0; dv = d0; }
-            else if (k == 1) { tv = t1; dv = d1; }
-            else {
-                tv = (T)2 * xx * t1 - t0;
-                dv = (T)2 * t1 + (T)2 * xx * d1 - d0;
-                t0 = t1; t1 = tv; d0 = d1; d1 = dv;
+        int nj = first[jj];
+        if ((unsigned)nj >= (unsigned)NF) nj = center;
+        if (role < nmus || (LOSS && role == nmus + 1)) {
+            int tj = types[nj];
+            if ((unsigned)tj >= (unsigned)a.ntypes) tj = 0;
+            const T* c = cf + (tj * nmus + (role < nmus ? role : 0)) * K;
+            T g = (T)0, dg = (T)0;
+            T t0 = (T)1, t1 = xx, d0 = (T)0, d1 = (T)1;
+            for (int k = 0; k < K; k++) {
+                T tv, dv;
+                if (k == 0) { tv = t0; dv = d0; }
+                else if (k == 1) { tv = t1; dv = d1; }
+                else {
+                    tv = (T)2 * xx * t1 - t0;
+                    dv = (T)2 * t1 + (T)2 * xx * d1 - d0;
+                    t0 = t1; t1 = tv; d0 = d1; d1 = dv;
+                }
+                const T f = a.scaling * s * tv;
+                const T df = a.scaling * (ds * tv + s * dv * dxx);
+                if (role < nmus) { g += c[k] * f; dg += c[k] * df; }
+                else { t[OF + k] = f; t[ODF + k] = df; }
             }
-            const T f = a.scaling * s * tv;
-            const T df = a.scaling * (ds * tv + s * dv * dxx);
-            if (LOSS) { t[OF + k] = f; t[ODF + k] = df; }
-#pragma unroll
-            for (int m = 0; m < MTP_NMUS_MAX; m++)
-                if (m < nmus) { g[m] += c[m * K + k] * f; dg[m] += c[m * K + k] * df; }
+            if (role < nmus) { t[OG + role] = g; t[ODG + role] = dg; }
         }
+        if (role >= nmus) {
+            const int ax = role - nmus;
+            const T rinv = (T)1 / r;
+            const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+            const T uc = ax == 0 ? ux : (ax == 1 ? uy : uz);
+            T pw = (T)1;
+            T* tp = t + ax * (kmax + 1);
+            for (int k = 0; k <= kmax; k++) { tp[k] = pw; pw *= uc; }
+            if (ax == 0) { t[OU + 0] = ux; t[OU + 1] = uy; t[OU + 2] = uz; t[OU + 3] = rinv; }
+            if (LOSS && ax == 2) {
+                // w_a = dFs[centre]_a - dFs[neighbour]_a - sum_b dVs[a,b] r_b   (linearMtpLoss.h:371-386)
+                const T* fc = a.dFs + ((size_t)b * a.P + center) * 3;
+                const T* fn = a.dFs + ((size_t)b * a.P + nj) * 3;
+                const T* dv = a.dVs + (size_t)b * 9;
+                T w[3];
 #pragma unroll
-        for (int m = 0; m < MTP_NMUS_MAX; m++)
-            if (m < nmus) { t[OG + m] = g[m]; t[ODG + m] = dg[m]; }
-        if (LOSS) {
-            // w_a = dFs[centre]_a - dFs[neighbour]_a - sum_b dVs[a,b] r_b   (linearMtpLoss.h:371-386)
-            const T* fc = a.dFs + ((size_t)b * a.P + center) * 3;
-            const T* fn = a.dFs + ((size_t)b * a.P + nj) * 3;
-            const T* dv = a.dVs + (size_t)b * 9;
-            T w[3];
-#pragma unroll
-            for (int q = 0; q < 3; q++)
-                w[q] = fc[q] - fn[q] - (dv[q * 3 + 0] * x + dv[q * 3 + 1] * y + dv[q * 3 + 2] * z);
-            t[OW + 0] = w[0]; t[OW + 1] = w[1]; t[OW + 2] = w[2];
-            t[OW + 3] = w[0] * ux + w[1] * uy + w[2] * uz;
+                for (int q = 0; q < 3; q++)
+                    w[q] = fc[q] - fn[q] - (dv[q * 3 + 0] * x + dv[q * 3 + 1] * y + dv[q * 3 + 2] * z);
+                t[OW + 0] = w[0]; t[OW + 1] = w[1]; t[OW + 2] = w[2];
+                t[OW + 3] = w[0] * ux + w[1] * uy + w[2] * uz;
+            }
         }
     }
 }
@@ -279,7 +289,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     T* A = M + n_moms;
     T* Tg = A + n_moms;                      // loss mode only
     T* Bm = Tg + (LOSS ? n_moms : 0);        // loss mode only
-    T* tab = Bm + (LOSS ? n_moms : 0);
+    T* cf = Bm + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
+    T* tab = cf + a.ntypes * nmus * K;
     T* gred = tab + MTP_NC * E;              // [256/32][32][4] partial sums of the thread groups
     T* pq = tab + max(MTP_NC * E + (256 / 32) * 32 * 4, p.max_level_slots * (LOSS ? 2 : 1));              // loss mode: P[nc][nmus] | Q[nc][nmus]
 
@@ -307,6 +318,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     for (int i = lane; i < n_basic; i += NT)
         bas[i] = (unsigned)p.basic[i * 4] | ((unsigned)p.basic[i * 4 + 1] << 8) |
                  ((unsigned)p.basic[i * 4 + 2] << 16) | ((unsigned)p.basic[i * 4 + 3] << 24);
+    for (int q = lane; q < a.ntypes * nmus * K; q += NT) cf[q] = a.coeffs[(size_t)ti * a.ntypes * nmus * K + q];
     for (int i = lane; i < n_moms; i += NT) {
         M[i] = (T)0; A[i] = (T)0;
         if (LOSS) { Tg[i] = (T)0; Bm[i] = (T)0; }
@@ -317,7 +329,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
         const int nc = min(MTP_NC, nn - c0);
         int nj; bool valid; T d[3];
-        build_table<T, LOSS>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+        build_table<T, LOSS, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
         __syncthreads();
         for (int i = lane; i < n_basic; i += NT) {
             const unsigned bw = bas[i];
@@ -392,25 +404,31 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     sweep_reverse<T, false, NT>(p, M, A, nullptr, nullptr, tab, lane);
 
     if (!LOSS) {
-        // ---- pair derivatives: lane = half * 32 + neighbour ------------------------------------
-        const int j = lane & 31, h = lane >> 5;
+        // ---- pair derivatives ------------------------------------------------------------------
+        // The row is cut into equal chunks of at most MTP_NC neighbours; within a chunk of nc
+        // neighbours thread = group h * nc + neighbour j, and the groups (as many as fit, at most
+        // MTP_NGMAX) share the basic moments, so a short chunk still keeps the workgroup busy.
         T fx = (T)0, fy = (T)0, fz = (T)0;
         T vir[9];
 #pragma unroll
         for (int q = 0; q < 9; q++) vir[q] = (T)0;
         T* grow = a.pair_g + row * a.U * 3;
-        for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
-            const int nc = min(MTP_NC, nn - c0);
+        const int nchunks = (nn + MTP_NC - 1) / MTP_NC;
+        const int csize = nchunks > 0 ? (nn + nchunks - 1) / nchunks : 1;
+        for (int c0 = 0; c0 < nn; c0 += csize) {
+            const int nc = min(csize, nn - c0);
+            const int ng = min(NT / nc, MTP_NGMAX);
+            const int h = lane / nc, j = lane - h * nc;
             int nj; bool valid; T d[3] = {(T)0, (T)0, (T)0};
             __syncthreads();
-            build_table<T, false>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+            build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
             __syncthreads();
             T gs = (T)0, wx = (T)0, wy = (T)0, wz = (T)0;
-            if (j < nc) {
+            if (h < ng) {
                 const T* t = tab + j * E;
                 const T rinv = t[OU + 3];
 #pragma unroll 4
-                for (int i = h; i < n_basic; i += NG) {
+                for (int i = h; i < n_basic; i += ng) {
                     const unsigned bw = bas[i];
                     const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
                     const T adj = A[i];
@@ -424,20 +442,19 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                     wz += ag * (T)ec * xa * yb * t[OZ + max(ec - 1, 0)];
                 }
             }
-            // group sums in the order h = 0 .. NG-1
+            // group sums in the order h = 0 .. ng-1
             {
-                T* gr = gred + (h * 32 + j) * 4;
+                T* gr = gred + lane * 4;
                 gr[0] = gs; gr[1] = wx; gr[2] = wy; gr[3] = wz;
             }
             __syncthreads();
             if (h == 0) {
-#pragma unroll
-                for (int hh = 1; hh < NG; hh++) {
-                    const T* gr = gred + (hh * 32 + j) * 4;
+                for (int hh = 1; hh < ng; hh++) {
+                    const T* gr = gred + (hh * nc + j) * 4;
                     gs += gr[0]; wx += gr[1]; wy += gr[2]; wz += gr[3];
                 }
             }
-            if (h == 0 && j < nc) {
+            if (h == 0) {
                 const T* t = tab + j * E;
                 const T rinv = t[OU + 3];
                 T gx = gs * t[OU + 0] + wx * rinv;
@@ -484,7 +501,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
             const int nc = min(MTP_NC, nn - c0);
             int nj; bool valid; T d[3];
             __syncthreads();
-            build_table<T, true>(a, tab, lane, nc, c0, rcs, first, types, ti, center, b, NF, &nj, &valid, d);
+            build_table<T, true, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
             __syncthreads();
             // P_mu(j), Q_mu(j): linearMtpLoss.h:438-536 with the k-sum factored out
             for (int mu = 0; mu < nmus; mu++) {
@@ -769,7 +786,7 @@ size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, in
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
     const size_t tabs = std::max((size_t)MTP_NC * E + (size_t)(256 / 32) * 32 * 4, (size_t)p.max_level_slots * (loss ? 2 : 1));
-    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs;
+    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
     else if (H > 0) n += (size_t)p.n_scalar + H;     // network inputs and pre-activations
