@@ -273,7 +273,6 @@ __device__ __forceinline__ T block_sum(T v, T* scratch, int tid)
 template <typename T, bool LOSS, int NT>
 __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
 {
-    constexpr int NG = NT / 32;       // thread groups of the pair passes: group h, neighbour j
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const MtpPlanDevice& p = a.p;
     const int lane = threadIdx.x;     // thread in the workgroup
@@ -326,8 +325,9 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     __syncthreads();
 
     // ---- basic moments (and their tangents) --------------------------------------------------
-    for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
-        const int nc = min(MTP_NC, nn - c0);
+    const int chunk = nn > 0 ? (nn + (nn + MTP_NC - 1) / MTP_NC - 1) / ((nn + MTP_NC - 1) / MTP_NC) : 1;
+    for (int c0 = 0; c0 < nn; c0 += chunk) {
+        const int nc = min(chunk, nn - c0);
         int nj; bool valid; T d[3];
         build_table<T, LOSS, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
         __syncthreads();
@@ -491,14 +491,18 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);      // linearMtpLoss.h:417-434
         T* grow = a.gpart + row * a.ngrad;
         for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
-        const int j = lane & 31, h = lane >> 5;
         T* Pm = pq;
         T* Qm = pq + MTP_NC * nmus;
         int* tjs = (int*)(pq + 2 * MTP_NC * nmus);
         T* gacc = pq + 2 * MTP_NC * nmus + MTP_NC;          // [ntypes][nmus][K] for this centre type
         for (int q = lane; q < a.ntypes * nmus * K; q += NT) gacc[q] = (T)0;
-        for (int c0 = 0; c0 < nn; c0 += MTP_NC) {
-            const int nc = min(MTP_NC, nn - c0);
+        const int nchunks = (nn + MTP_NC - 1) / MTP_NC;
+        const int csize = nchunks > 0 ? (nn + nchunks - 1) / nchunks : 1;
+        for (int c0 = 0; c0 < nn; c0 += csize) {
+            // equal chunks and as many thread groups per chunk as fit, as in the pair-derivative pass
+            const int nc = min(csize, nn - c0);
+            const int ng = min(NT / nc, MTP_NGMAX);
+            const int h = lane / nc, j = lane - h * nc;
             int nj; bool valid; T d[3];
             __syncthreads();
             build_table<T, true, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
@@ -506,10 +510,10 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
             // P_mu(j), Q_mu(j): linearMtpLoss.h:438-536 with the k-sum factored out
             for (int mu = 0; mu < nmus; mu++) {
                 T Pv = (T)0, Qv = (T)0;
-                if (j < nc) {
+                if (h < ng) {
                     const T* t = tab + j * E;
                     const T rinv = t[OU + 3], wu = t[OW + 3];
-                    for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += NG) {
+                    for (int i = p.mu_begin[mu] + h; i < p.mu_begin[mu + 1]; i += ng) {
                         const unsigned bw = bas[i];
                         const int ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
                         const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
@@ -523,22 +527,21 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                     }
                 }
                 {
-                    T* gr = gred + (h * 32 + j) * 4;
+                    T* gr = gred + lane * 2;
                     gr[0] = Pv; gr[1] = Qv;
                 }
                 __syncthreads();
                 if (h == 0) {
-#pragma unroll
-                    for (int hh = 1; hh < NG; hh++) {
-                        const T* gr = gred + (hh * 32 + j) * 4;
+                    for (int hh = 1; hh < ng; hh++) {
+                        const T* gr = gred + (hh * nc + j) * 2;
                         Pv += gr[0]; Qv += gr[1];
                     }
-                    if (j < nc) { Pm[j * nmus + mu] = Pv; Qm[j * nmus + mu] = Qv; }
+                    Pm[j * nmus + mu] = Pv; Qm[j * nmus + mu] = Qv;
                 }
                 __syncthreads();
             }
             // tj of each neighbour of the chunk, for the accumulation below
-            if (h == 0 && j < nc) tjs[j] = valid ? types[nj] : -1;
+            if (h == 0) tjs[j] = valid ? types[nj] : -1;
             __syncthreads();
             // lanes <- (mu, k): sequential over neighbours keeps the sum order fixed
             for (int q = lane; q < nmus * K; q += NT) {

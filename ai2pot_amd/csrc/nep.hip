@@ -431,6 +431,10 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     size_t lds_staged = 0;
     const bool staged = nep_staged_supported<T>(a, &lds_staged);
     if (staged) a.nblocks = nep_staged_nblocks(P);
+    size_t lds_group = 0;
+    // fewer staged workgroups than half the compute units: the system is small, spread it wider
+    const bool group = staged && (long long)B * nep_staged_nblocks(P) < 128 && nep_group_supported<T>(a, &lds_group);
+    if (group) a.nblocks = nep_group_nblocks(P);
 
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
@@ -443,7 +447,10 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     a.force = force;
     const size_t force_bytes = (size_t)B * (P + nghost) * 3 * sizeof(T);
 
-    if (staged) {
+    if (group) {
+        rc = nep_group_run<T>(a, lds_group, stream);
+        if (rc) return rc;
+    } else if (staged) {
         rc = nep_staged_run<T>(a, lds_staged, stream);
         if (rc) return rc;
     } else {

@@ -152,6 +152,7 @@ def run_nep_md(args, kind, size, rebuild=True):
     work = {
         "nep_efv_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
         "nep_staged_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
+        "nep_group_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
         "nbl_lists": ("hbm", ((3 * s + 4) + 12 + U * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
         "reduce_fill": ("hbm", (nn_r * (3 * s + 4) + nn_r * 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
     }

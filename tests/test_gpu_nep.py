@@ -99,6 +99,20 @@ def test_batch_padding_permuted_ilist(oracle):
     check(run_gpu(m, nb, np.float32), oracle.nep_efv(m, nb, np.float32), np.float32)
 
 
+@pytest.mark.parametrize("reps", [4, 21])
+def test_angular_cutoff_beyond_radial(oracle, reps):
+    """A neighbour beyond the radial cutoff is skipped altogether, also when it lies inside a larger
+    angular cutoff (nepBasis.h:106, 135).  256 atoms take the kernel with 8 lanes per atom, 37044
+    atoms the one with a thread per atom."""
+    lat, pos = synth.fcc_cell(reps, 4.6, 0.15, 61)
+    ty = synth.rng_randint(62, pos.shape[0], 3)
+    nb = synth.pack_batch([oracle.nblist(lat, ty, pos, 6.0, 100)])
+    m = synth.nep_model(rmax_radial=4.5, rmax_angular=5.5)
+    for dt in (np.float64, np.float32):
+        nbt = dict(nb, brcs=nb["brcs"].astype(dt))
+        check(run_gpu(m, nbt, dt), oracle.nep_efv(m, nbt, dt), dt)
+
+
 def test_ghost_atoms(oracle):
     """The LAMMPS contract: neighbour indices point into [0, P + nghost); ghosts have a type
     and receive forces but own no row (interface/lammps/AI2POT/pair_ai2pot.cpp:175-249)."""
