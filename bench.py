@@ -79,6 +79,19 @@ def timed(step, steps, warmup, L):
     return t1 - t0, kernels
 
 
+def timed_replay(replay, steps, warmup):
+    """Wall time of `steps` replays of a captured step (no per-kernel events: a replay is one launch)."""
+    import torch
+    for _ in range(warmup):
+        replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        replay()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
@@ -142,6 +155,13 @@ def run_nep_md(args, kind, size, rebuild=True):
 
     L = _lib.lib()
     elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    if args.graph:
+        if rebuild:
+            sys.exit("bench.py: --graph needs a workload without list rebuild (the build synchronises with the host)")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            calc.evaluate(ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        elapsed = timed_replay(graph.replay, args.steps, args.warmup)
     calc.check()
     if not np.isfinite(float(calc.etot.item())):
         sys.exit("bench.py: non-finite energy")
@@ -159,7 +179,8 @@ def run_nep_md(args, kind, size, rebuild=True):
     config = {"workload": args.workload, "natoms": n, "species": 3,
               "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 7.0, "rcut_angular": 4.0,
               "umax": 200, "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
-              "per_step": ("neighbor rebuild + " if rebuild else "") + "descriptors + ANN + force/virial"}
+              "per_step": ("neighbor rebuild + " if rebuild else "") + "descriptors + ANN + force/virial",
+              "launch": "hip graph replay" if args.graph else "eager"}
     roof = roofline_of(kernels, work)
     if roof is not None:
         roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, roof["kernel"]))
@@ -269,6 +290,12 @@ def run_mtp(args, cfg):
         label = "mtp_efv_kernel"
     L = _lib.lib()
     elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    if args.graph:
+        if cfg == 4:
+            sys.exit("bench.py: --graph is wired for the energy / force / virial workloads")
+        from ai2pot_amd.graph import GraphedCall
+        g = GraphedCall(ops.linearMtpToEFVOp, *common, 0.0, 0.0, None, None)
+        elapsed = timed_replay(g.replay, args.steps, args.warmup)
     _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
     work = {label: ("mfma", flops if cfg != 4 else flops - mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s",
                     PEAK_FP64_TFLOPS, 1e12, "valu_fp64"),
@@ -278,7 +305,8 @@ def run_mtp(args, cfg):
               "model": "linear MTP level %d K=%d" % ({1: 10, 3: 20, 4: 16}[cfg], m["chebyshev_size"]),
               "species": int(m["type_map"].size), "rmax": m["rmax"], "rmin": m["rmin"], "mean_neighbors": nn,
               "per_step": "loss forward + analytic gradient w.r.t. coeffs/linear/bias" if cfg == 4 else
-                          "energy + force + virial (list built once, outside the timed region)"}
+                          "energy + force + virial (list built once, outside the timed region)",
+              "launch": "hip graph replay" if args.graph else "eager"}
     return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f64"
 
 
@@ -397,6 +425,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="nep_md_1048576", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of the step captured as a HIP graph (workloads without list rebuild)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
