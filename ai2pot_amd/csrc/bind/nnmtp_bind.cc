@@ -1,9 +1,15 @@
 // libnnmtp_bind.so -- registers torch.ops.nnmtp.* with the reference's schemas
 // (source/descriptor/nnmtp/bind/nnmtp_bind.cc:27-430) on top of libai2pot_hip.so:
-// set_ai2pot_path, mtpParamOp, nnMtpToEFVOp, nnMtpToEFOp, nnMtpToEsitesOp (forward) and
-// nnMtpToDescriptorsOp.  The training operators of the reference (nnMtpToLossOp, nnMtpToEFLossOp)
-// and the backward of nnMtpToEsitesOp are not part of this build: they are registered and raise.
+// set_ai2pot_path, mtpParamOp, nnMtpToEFVOp, nnMtpToEFOp, nnMtpToEsitesOp (forward),
+// nnMtpToDescriptorsOp, nnMtpToLossOp and nnMtpToEFLossOp (autograd to coeffs, w0, w1, type_bias as
+// src/nnMtpOp.cc:2748-2780).  The backward of nnMtpToEsitesOp is not part of this build: parameters
+// that require grad are refused.
+// The loss operators evaluate the reference's backward formulas, which are not the complete
+// derivative of the loss (see include/ai2pot_hip.h, a2p_nnmtp_loss_*); with the environment variable
+// A2P_NNMTP_EXACT_GRADIENT=1 they return the complete derivative instead.
 #include "mtp_bind_common.h"
+
+#include <cstdlib>
 
 namespace {
 
@@ -112,6 +118,98 @@ variable_list nnmtp_descriptors(int64_t K, const at::Tensor& coeffs, int64_t n_m
     return {desc};
 }
 
+// forward: [bloss]; backward: grad_output @ per-structure gradients
+struct NNLossFunction : public torch::autograd::Function<NNLossFunction> {
+    static variable_list forward(AutogradContext* ctx, bool with_virial, double e_w, double f_w, double v_w,
+                                 const at::Tensor& e_dft, const at::Tensor& f_dft, const at::Tensor& v_dft_in,
+                                 int64_t K, const at::Tensor& coeffs, const at::Tensor& w0, const at::Tensor& w1,
+                                 const at::Tensor& bias, int64_t n_moms, const at::Tensor& basic,
+                                 const at::Tensor& times, const at::Tensor& mapping, int64_t nmus,
+                                 const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                                 const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                                 const at::Tensor& type_map, int64_t nghost, double rmax, double rmin,
+                                 const at::Tensor& q_shifter, const at::Tensor& q_scaler)
+    {
+        TORCH_CHECK(nghost == 0, "the loss operator requires nghost == 0, as the reference does");
+        Batch s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+        const int ntypes = (int)type_map.numel();
+        TORCH_CHECK(ntypes > 0, "type_map is empty");
+        for (auto& pr : {std::make_pair(&coeffs, "coeffs"), std::make_pair(&w0, "w0"), std::make_pair(&w1, "w1"),
+                         std::make_pair(&bias, "type_bias"), std::make_pair(&q_shifter, "q_shifter"),
+                         std::make_pair(&q_scaler, "q_scaler"), std::make_pair(&e_dft, "betot_dft"),
+                         std::make_pair(&f_dft, "bforce_dft")})
+            check_device_float(brcs, *pr.first, pr.second);
+        a2p_bind::DeviceGuard guard(brcs);
+        PlanEntry plan = get_plan(brcs.device().index(), n_moms, basic, times, mapping);
+        TORCH_CHECK(coeffs.numel() == (int64_t)ntypes * ntypes * nmus * K, "coeffs size mismatch");
+        TORCH_CHECK(w1.numel() > 0 && w1.numel() % ntypes == 0, "w1 must have ntypes * num_neurons elements");
+        const int H = (int)(w1.numel() / ntypes);
+        TORCH_CHECK(w0.numel() == (int64_t)ntypes * H * plan.n_scalar,
+                    "w0 must have ntypes * num_neurons * alpha_scalar_moments elements");
+        TORCH_CHECK(q_shifter.numel() == plan.n_scalar && q_scaler.numel() == plan.n_scalar,
+                    "q_shifter and q_scaler must have alpha_scalar_moments elements");
+        TORCH_CHECK(bias.numel() == ntypes, "type_bias size mismatch");
+        auto opt = brcs.options();
+        const int B = s.B, P = s.P;
+        at::Tensor v_dft = with_virial ? v_dft_in : at::zeros({B, 9}, opt);
+        check_device_float(brcs, v_dft, "bvirial_dft");
+        TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
+                    "label tensors must have shapes [B], [B, P, 3], [B, 9]");
+        const bool need = coeffs.requires_grad() || w0.requires_grad() || w1.requires_grad() || bias.requires_grad();
+        at::Tensor bloss = at::zeros({B}, opt), e = at::zeros({B}, opt), f = at::zeros({B, P, 3}, opt),
+                   v = at::zeros({B, 9}, opt), dc, d0, d1, db;
+        if (need) {
+            dc = at::zeros({B, coeffs.numel()}, opt);
+            d0 = at::zeros({B, w0.numel()}, opt);
+            d1 = at::zeros({B, w1.numel()}, opt);
+            db = at::zeros({B, bias.numel()}, opt);
+        }
+        const char* env = std::getenv("A2P_NNMTP_EXACT_GRADIENT");
+        const int exact = env && env[0] == '1';
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_nnmtp_loss_f64(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
+                                    H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
+                                    rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                    btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
+                                    exact, st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_nnmtp_loss_f32(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
+                                    H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
+                                    rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                    btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
+                                    exact, st);
+        }
+        check_rc(rc);
+        check_device_status(brcs);
+        ctx->saved_data["need"] = need;
+        if (need) ctx->save_for_backward({dc, d0, d1, db});
+        ctx->saved_data["shape_c"] = coeffs.sizes().vec();
+        ctx->saved_data["shape_0"] = w0.sizes().vec();
+        ctx->saved_data["shape_1"] = w1.sizes().vec();
+        ctx->saved_data["shape_b"] = bias.sizes().vec();
+        return {bloss};
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(29);                   // one slot per forward argument after ctx
+        if (!ctx->saved_data["need"].toBool()) return out;
+        auto saved = ctx->get_saved_variables();
+        at::Tensor gl = grads[0].contiguous();
+        out[8] = torch::matmul(gl, saved[0]).reshape(ctx->saved_data["shape_c"].toIntVector());
+        out[9] = torch::matmul(gl, saved[1]).reshape(ctx->saved_data["shape_0"].toIntVector());
+        out[10] = torch::matmul(gl, saved[2]).reshape(ctx->saved_data["shape_1"].toIntVector());
+        out[11] = torch::matmul(gl, saved[3]).reshape(ctx->saved_data["shape_b"].toIntVector());
+        return out;
+    }
+};
+
 }  // namespace
 
 TORCH_LIBRARY(nnmtp, m)
@@ -143,12 +241,15 @@ TORCH_LIBRARY(nnmtp, m)
                                        bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin);
           });
     m.def("nnMtpToLossOp",
-          [](double, double, double, const at::Tensor&, const at::Tensor&, const at::Tensor&,
-             NNMTP_ARGS) -> variable_list {
-              TORCH_CHECK(false, "nnMtpToLossOp is not implemented in this build");
+          [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
+             const at::Tensor& v_dft, NNMTP_ARGS) -> variable_list {
+              require_no_zbl(zbl_rmax);
+              return NNLossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, NNMTP_PASS);
           });
     m.def("nnMtpToEFLossOp",
-          [](double, double, const at::Tensor&, const at::Tensor&, NNMTP_ARGS) -> variable_list {
-              TORCH_CHECK(false, "nnMtpToEFLossOp is not implemented in this build");
+          [](double e_w, double f_w, const at::Tensor& e_dft, const at::Tensor& f_dft, NNMTP_ARGS) -> variable_list {
+              require_no_zbl(zbl_rmax);
+              return NNLossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
+                                           at::zeros({e_dft.numel(), 9}, e_dft.options()), NNMTP_PASS);
           });
 }

@@ -66,6 +66,7 @@ struct MtpArgs {
     // e_i = bias + sum_p w1[t,p] tanh(sum_k w0[t,p,k] (M_k - q_shift[k]) / q_scaler[k]); `lin` is unused
     int H;
     const T *w0, *w1, *q_shift;
+    int nn_exact;      // loss mode: 1 = complete derivative, 0 = the reference's formulas (see nnmtp_loss)
 };
 
 __device__ __forceinline__ float tanh_t(float x) { return tanhf(x); }
@@ -359,33 +360,57 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     // ---- products, energy, adjoint ------------------------------------------------------------
     sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
     T e_part = (T)0;
-    if (!LOSS && a.H > 0) {
+    // network buffers (H > 0): inputs q[S]; per neuron w1 tanh', and in loss mode tanh, tanh', tanh'', tau
+    T* nnb = LOSS ? pq + 2 * MTP_NC * nmus + MTP_NC + a.ntypes * nmus * K : pq;
+    if (a.H > 0) {
         // one tanh layer of the centre's species on the shifted, scaled scalar moments; the
         // adjoint is seeded with dE_i/dM_k = sum_p w1_p tanh'(h_p) w0_pk / q_scaler_k
+        // (nnMtp.h:470-507).  Loss mode also needs the derivative of that seed along the tangent:
+        // tau_p = sum_k w0_pk Tg_k / q_scaler_k is the tangent of h_p, and the adjoint of
+        // D_w E = sum_p w1_p tanh'(h_p) tau_p  w.r.t. M_k is  sum_p w1_p tanh''(h_p) tau_p w0_pk / q_scaler_k,
+        // the seed of the mixed sweep (nnMtpLoss.h:216-610 computes the same quantities atom by atom).
         const int S = p.n_scalar, H = a.H;
-        T* qv = pq;                           // [S] network inputs
-        T* hv = pq + S;                       // [H] pre-activations, then w1 * tanh'
+        T* qv = nnb;                          // [S] network inputs
+        T* hv = nnb + S;                      // [H] pre-activations, then w1 * tanh'
+        T* n_th = hv + H;                     // loss mode: tanh, tanh', tanh'', tau   [H] each
+        T* n_d1 = n_th + H;
+        T* n_d2 = n_d1 + H;
+        T* n_tau = n_d2 + H;
         const T* w0 = a.w0 + (size_t)ti * H * S;
         const T* w1 = a.w1 + (size_t)ti * H;
         for (int s = lane; s < S; s += NT) qv[s] = (M[p.mapping[s]] - a.q_shift[s]) / a.q_scaler[s];
         __syncthreads();
         for (int n = lane >> 6; n < H; n += NT / 64) {          // one wave per neuron
-            T acc = (T)0;
-            for (int k = lane & 63; k < S; k += 64) acc += w0[(size_t)n * S + k] * qv[k];
+            T acc = (T)0, tac = (T)0;
+            for (int k = lane & 63; k < S; k += 64) {
+                acc += w0[(size_t)n * S + k] * qv[k];
+                if (LOSS) tac += w0[(size_t)n * S + k] * Tg[p.mapping[k]] / a.q_scaler[k];
+            }
             acc = wave_sum(acc);
-            if ((lane & 63) == 0) hv[n] = acc;
+            if (LOSS) tac = wave_sum(tac);
+            if ((lane & 63) == 0) {
+                hv[n] = acc;
+                if (LOSS) n_tau[n] = tac;
+            }
         }
         __syncthreads();
         for (int n = lane; n < H; n += NT) {
             const T th = tanh_t(hv[n]);
+            const T d1 = (T)1 - th * th;
             e_part += w1[n] * th;
-            hv[n] = w1[n] * ((T)1 - th * th);
+            hv[n] = w1[n] * d1;
+            if (LOSS) { n_th[n] = th; n_d1[n] = d1; n_d2[n] = (T)-2 * th * d1; }
         }
         __syncthreads();
         for (int k = lane; k < S; k += NT) {
-            T acc = (T)0;
-            for (int n = 0; n < H; n++) acc += hv[n] * w0[(size_t)n * S + k];
+            T acc = (T)0, bac = (T)0;
+            for (int n = 0; n < H; n++) {
+                const T w = w0[(size_t)n * S + k];
+                acc += hv[n] * w;
+                if (LOSS) bac += w1[n] * n_d2[n] * n_tau[n] * w;
+            }
             A[p.mapping[k]] = acc / a.q_scaler[k];
+            if (LOSS && a.nn_exact) Bm[p.mapping[k]] = bac / a.q_scaler[k];
         }
     } else {
         for (int s = lane; s < p.n_scalar; s += NT) {
@@ -488,7 +513,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     // ---- loss gradient ------------------------------------------------------------------------
     if (LOSS) {
         const T cE = a.cE_per_atom ? a.cE[row] : a.cE[b];
-        sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);      // linearMtpLoss.h:417-434
+        // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
+        if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
         T* grow = a.gpart + row * a.ngrad;
         for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
         T* Pm = pq;
@@ -555,6 +581,29 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
             }
         }
         __syncthreads();
+        if (a.H > 0) {
+            // compact row of the centre species: coefficient block | w0[H, S] | w1[H] | bias
+            const int S = p.n_scalar, H = a.H, nblk = a.ntypes * nmus * K;
+            const T* qv = nnb;
+            const T* n_th = nnb + S + H;
+            const T* n_d1 = n_th + H;
+            const T* n_d2 = n_d1 + H;
+            const T* n_tau = n_d2 + H;
+            const T* w1 = a.w1 + (size_t)ti * H;
+            for (int q = lane; q < nblk; q += NT) grow[q] = gacc[q];
+            const T* w0 = a.w0 + (size_t)ti * H * S;
+            for (int q = lane; q < H * S; q += NT) {
+                const int n = q / S, k = q - n * S;
+                const T tk = Tg[p.mapping[k]] / a.q_scaler[k];
+                if (a.nn_exact)
+                    grow[nblk + q] = w1[n] * ((cE * n_d1[n] + n_d2[n] * n_tau[n]) * qv[k] + n_d1[n] * tk);
+                else        // nnMtpLoss.h:560-585: only the k' = k term of tau
+                    grow[nblk + q] = w1[n] * (cE * n_d1[n] * qv[k] + tk * (n_d1[n] + n_d2[n] * w0[q] * qv[k]));
+            }
+            for (int n = lane; n < H; n += NT) grow[nblk + H * S + n] = cE * n_th[n] + n_d1[n] * n_tau[n];
+            if (lane == 0) grow[nblk + H * S + H] = cE;
+            return;
+        }
         for (int q = lane; q < a.ntypes * nmus * K; q += NT)
             grow[(size_t)ti * a.ntypes * nmus * K + q] = gacc[q];
         // linear coefficients and bias: linearMtpLoss.h:539-554
@@ -581,6 +630,33 @@ mtp_grad_reduce_kernel(int P, int ncoef, int nlin, int nbias, const int* __restr
     if (q < ncoef) { if (dcoeffs) dcoeffs[(size_t)b * ncoef + q] = acc; }
     else if (q < ncoef + nlin) { if (dlin) dlin[(size_t)b * nlin + q - ncoef] = acc; }
     else if (dbias) dbias[(size_t)b * nbias + q - ncoef - nlin] = acc;
+}
+
+// The same for the compact rows of the neural-network MTP: row = [coefficient block of the centre
+// species | w0[H, S] | w1[H] | bias]; out[b] is laid out coeffs[ntypes^2 nmus K] | w0[ntypes H S] |
+// w1[ntypes H] | bias[ntypes].  Thread q of block (x, t, b) sums entry q of the rows of species t.
+template <typename T>
+__global__ void __launch_bounds__(256)
+nnmtp_grad_reduce_kernel(int P, int NF, int nblk, int HS, int H, int ntypes, const int* __restrict__ binum,
+                         const int* __restrict__ bilist, const int* __restrict__ btypes,
+                         const T* __restrict__ gpart, T* __restrict__ dcoeffs, T* __restrict__ dw0,
+                         T* __restrict__ dw1, T* __restrict__ dbias)
+{
+    const int b = blockIdx.z, t = blockIdx.y;
+    const int nrow = nblk + HS + H + 1;
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= nrow) return;
+    const int inum = binum[b];
+    T acc = (T)0;
+    for (int ii = 0; ii < inum; ii++) {
+        const int c = bilist[(size_t)b * P + ii];
+        if ((unsigned)c >= (unsigned)NF || btypes[(size_t)b * NF + c] != t) continue;
+        acc += gpart[((size_t)b * P + ii) * nrow + q];
+    }
+    if (q < nblk) { if (dcoeffs) dcoeffs[((size_t)b * ntypes + t) * nblk + q] = acc; }
+    else if (q < nblk + HS) { if (dw0) dw0[((size_t)b * ntypes + t) * HS + q - nblk] = acc; }
+    else if (q < nblk + HS + H) { if (dw1) dw1[((size_t)b * ntypes + t) * H + q - nblk - HS] = acc; }
+    else if (dbias) dbias[(size_t)b * ntypes + t] = acc;
 }
 
 // ---- plan construction ---------------------------------------------------------------------------
@@ -792,7 +868,7 @@ size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, in
     size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
-    else if (H > 0) n += (size_t)p.n_scalar + H;     // network inputs and pre-activations
+    if (H > 0) n += (size_t)p.n_scalar + (loss ? 5 : 1) * (size_t)H;     // network inputs and per-neuron values
     return n * sizeof(T) + 64;      // the packed basic-moment table (4 n_basic bytes) follows
 }
 
@@ -819,6 +895,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
     a.force = nullptr; a.pair_g = nullptr; a.partial = nullptr;
     a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
+    a.nn_exact = 1;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
@@ -968,6 +1045,70 @@ int mtp_loss(void* handle, double e_w, double f_w, double v_w, const T* e_dft, c
     prof_begin("mtp_grad_reduce", stream);
     hipLaunchKernelGGL(mtp_grad_reduce_kernel<T>, dim3(ceil_div(ngrad, 256), B), dim3(256), 0, stream, P, ncoef,
                        a.p.n_scalar, ntypes, binum, gpart, dcoeffs, dlin, dbias);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+// Training loss of the neural-network MTP: E/F/V, per-structure loss and the per-structure gradients
+// w.r.t. coeffs, w0, w1, type_bias (nnMtpLoss.h:141-181, 216-610; nnMtpOp.cc:1641-2780).
+// exact = 0 evaluates the reference's backward formulas, which leave out two contributions of the
+// force and virial terms: in d/dcoeffs the dependence of the adjoint on the moments (the mixed
+// sweep of the linear MTP, linearMtpLoss.h:417-434, and the tanh'' term), and in d/dw0[p,k] the
+// k' != k part of the tangent of the pre-activation (nnMtpLoss.h:497-529, 560-585).  exact = 1 is the
+// complete derivative of the loss (it agrees with finite differences; the reference's does not).
+template <typename T>
+int nnmtp_loss(void* handle, double e_w, double f_w, double v_w, const T* e_dft, const T* f_dft, const T* v_dft,
+               int K, const MtpNet<T>& net, const T* coeffs, const T* bias, int nmus, int ntypes,
+               const T* q_scaler, double rmax, double rmin, int B, int P, int U, const int* binum,
+               const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs, const int* btypes,
+               T* bloss, T* etot, T* force, T* virial, T* dcoeffs, T* dw0, T* dw1, T* dbias, int exact,
+               hipStream_t stream)
+{
+    A2P_REQUIRE(e_dft && f_dft && v_dft && bloss && etot && force && virial, A2P_ERR_INVALID,
+                "nnmtp loss: null label or output pointer");
+    int rc = mtp_efv<T>(handle, K, 1.0, coeffs, nullptr, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, 0, binum,
+                        bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, stream, &net);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    MtpPlan* plan = nullptr;
+    rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, 1.0, coeffs, (const T*)nullptr, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U, 0,
+                   binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    rc = set_net(a, &net);
+    if (rc) return rc;
+    const int S = a.p.n_scalar, H = net.H;
+    const int nblk = ntypes * nmus * K;
+    const int nrow = nblk + H * S + H + 1;
+    const bool want_grad = dcoeffs || dw0 || dw1 || dbias;
+    // workspace: cE[B] | dVs[B*9] | dFs[B*P*3] | gpart[B*P*nrow] | sq[B*3] (double)
+    size_t nT = (size_t)B + (size_t)B * 9 + (size_t)B * P * 3 + (want_grad ? (size_t)B * P * nrow : 0);
+    size_t bytesT = (nT * sizeof(T) + 15) / 16 * 16;
+    void* ws = nullptr;
+    rc = ws_get(WS_MTP, bytesT + (size_t)B * 3 * sizeof(double), &ws);
+    if (rc) return rc;
+    T* cE = (T*)ws;
+    T* dVs = cE + B;
+    T* dFs = dVs + (size_t)B * 9;
+    T* gpart = dFs + (size_t)B * P * 3;
+    double* sq = (double*)((char*)ws + bytesT);
+    prof_begin("mtp_loss_forward", stream);
+    hipLaunchKernelGGL(losskern::loss_forward_kernel<T>, dim3(B), dim3(256), 0, stream, P, binum, bilist, (T)e_w,
+                       (T)f_w, (T)v_w, etot, e_dft, force, f_dft, virial, v_dft, bloss, cE, dFs, dVs, sq, 1);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    if (!want_grad) return A2P_OK;
+    a.E = table_entries<T>(a.p, K, true);
+    a.cE = cE; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = nrow;
+    a.nn_exact = exact ? 1 : 0;
+    rc = launch_atoms<T, true>(a, stream);
+    if (rc) return rc;
+    prof_begin("mtp_grad_reduce", stream);
+    hipLaunchKernelGGL(nnmtp_grad_reduce_kernel<T>, dim3(ceil_div(nrow, 256), ntypes, B), dim3(256), 0, stream, P, P,
+                       nblk, H * S, H, ntypes, binum, bilist, btypes, gpart, dcoeffs, dw0, dw1, dbias);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -1136,6 +1277,22 @@ int a2p_mtp_esites_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int ng
     }
 NNMTP_ENTRY(double, f64)
 NNMTP_ENTRY(float, f32)
+
+#define NNMTP_LOSS_ENTRY(T, SUFFIX)                                                                              \
+    int a2p_nnmtp_loss_##SUFFIX(void* plan, double e_w, double f_w, double v_w, const T* e_dft, const T* f_dft,    \
+                                const T* v_dft, int K, int H, const T* coeffs, const T* w0, const T* w1,           \
+                                const T* bias, int nmus, int ntypes, const T* q_shifter, const T* q_scaler,        \
+                                double rmax, double rmin, int B, int P, int U, MTP_BATCH(T), T* bloss, T* etot,    \
+                                T* force, T* virial, T* dcoeffs, T* dw0, T* dw1, T* dbias, int exact_gradient,     \
+                                void* stream)                                                                      \
+    {                                                                                                            \
+        a2p::MtpNet<T> net{H, w0, w1, q_shifter};                                                                  \
+        return a2p::nnmtp_loss<T>(plan, e_w, f_w, v_w, e_dft, f_dft, v_dft, K, net, coeffs, bias, nmus, ntypes,    \
+                                  q_scaler, rmax, rmin, B, P, U, MTP_BATCH_PASS, bloss, etot, force, virial,       \
+                                  dcoeffs, dw0, dw1, dbias, exact_gradient, (hipStream_t)stream);                  \
+    }
+NNMTP_LOSS_ENTRY(double, f64)
+NNMTP_LOSS_ENTRY(float, f32)
 
 int a2p_mtp_esites_bwd_f64(void* plan, MTP_MODEL(double), int B, int P, int U, int nghost, MTP_BATCH(double),
                            const double* grad_e_sites, double* dcoeffs, double* dlinear, double* dbias, void* stream)

@@ -731,6 +731,118 @@ def nnMtpToDescriptorsOp(chebyshev_size, coeffs, alpha_moments_count, alpha_inde
                                     bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, validate)
 
 
+def nnmtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, coeffs, w0,
+                    w1, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+                    alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+                    nghost, rmax, rmin, q_shifter, q_scaler, want_grad=True, exact_gradient=False, validate=True):
+    """Forward and (optionally) the per-structure parameter gradients of the NN-MTP training loss.
+    Returns a dict with bloss[B], energy, force, virial and, with want_grad, dcoeffs[B, ncoef],
+    dw0[B, ntypes*H*S], dw1[B, ntypes*H], dbias[B, ntypes].  exact_gradient=False evaluates the
+    reference's backward formulas (nnMtpLoss.h:216-610), which are not the full derivative of the
+    loss for the force and virial terms; exact_gradient=True returns the full derivative."""
+    _req(int(nghost) == 0, "the loss operator requires nghost == 0, as the reference does")
+    _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
+         "brcs must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = brcs.dtype, brcs.device
+    _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
+    _req(brcs.is_contiguous(), "brcs must be contiguous")
+    for name, t in (("coeffs", coeffs), ("w0", w0), ("w1", w1), ("type_bias", type_bias),
+                    ("q_shifter", q_shifter), ("q_scaler", q_scaler)):
+        _check_float(name, t, dtype, device)
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh), ("btypes", btypes)):
+        _check_int(name, t, device)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, 0)
+    ntypes = int(type_map.numel())
+    _req(ntypes > 0, "type_map is empty")
+    plan, n_scalar = _mtp_plan(alpha_moments_count, alpha_index_basic, alpha_index_times,
+                               alpha_moment_mapping, device)
+    _req(coeffs.numel() == ntypes * ntypes * int(nmus) * int(chebyshev_size), "coeffs size mismatch")
+    _req(w1.numel() % ntypes == 0 and w1.numel() > 0, "w1 must have ntypes * num_neurons elements")
+    H = w1.numel() // ntypes
+    _req(w0.numel() == ntypes * H * n_scalar, "w0 must have ntypes*H*alpha_scalar_moments elements")
+    _req(q_shifter.numel() == n_scalar and q_scaler.numel() == n_scalar,
+         "q_shifter and q_scaler must have alpha_scalar_moments = %d elements" % n_scalar)
+    _req(type_bias.numel() == ntypes, "type_bias size mismatch")
+    for name, t, n_expected in (("betot_dft", betot_dft, B), ("bforce_dft", bforce_dft, B * P * 3),
+                                ("bvirial_dft", bvirial_dft, B * 9)):
+        _check_float(name, t, dtype, device)
+        _req(t.numel() == n_expected, "%s has %d elements, expected %d" % (name, t.numel(), n_expected))
+    if validate:
+        _validate_batch(binum, bnumneigh, U, P)
+    z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
+    out = dict(bloss=z(B), energy=z(B), force=z(B, P, 3), virial=z(B, 9))
+    if want_grad:
+        out.update(dcoeffs=z(B, coeffs.numel()), dw0=z(B, w0.numel()), dw1=z(B, w1.numel()), dbias=z(B, ntypes))
+    L = _lib.lib()
+    fn = L.a2p_nnmtp_loss_f32 if dtype == torch.float32 else L.a2p_nnmtp_loss_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+                _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0),
+                _ptr(w1), _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_shifter), _ptr(q_scaler),
+                _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _ptr(binum),
+                _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(out["bloss"]),
+                _ptr(out["energy"]), _ptr(out["force"]), _ptr(out["virial"]), _ptr(out.get("dcoeffs")),
+                _ptr(out.get("dw0")), _ptr(out.get("dw1")), _ptr(out.get("dbias")),
+                _c.c_int(1 if exact_gradient else 0), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return out
+
+
+class _NNMtpToLoss(torch.autograd.Function):
+    """Autograd wrapper with the reference's contract (nnMtpOp.cc:1641-2780): one output, bloss[B];
+    gradients flow to coeffs, w0, w1 and type_bias as grad_output[B] @ dloss/dtheta."""
+
+    @staticmethod
+    def forward(ctx, coeffs, w0, w1, type_bias, args):
+        (e_w, f_w, v_w, e_dft, f_dft, v_dft, K, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+         bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, exact, validate) = args
+        need = any(t.requires_grad for t in (coeffs, w0, w1, type_bias))
+        r = nnmtp_loss_step(e_w, f_w, v_w, e_dft, f_dft, v_dft, K, coeffs.detach(), w0.detach(), w1.detach(),
+                            type_bias.detach(), n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                            bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler,
+                            want_grad=need, exact_gradient=exact, validate=validate)
+        if need:
+            ctx.save_for_backward(r["dcoeffs"], r["dw0"], r["dw1"], r["dbias"])
+        ctx.shapes = (coeffs.shape, w0.shape, w1.shape, type_bias.shape)
+        ctx.have = need
+        return r["bloss"]
+
+    @staticmethod
+    def backward(ctx, gl):
+        if not ctx.have:
+            return None, None, None, None, None
+        return tuple(torch.matmul(gl, g).reshape(sh) for g, sh in zip(ctx.saved_tensors, ctx.shapes)) + (None,)
+
+
+def nnMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, coeffs, w0, w1,
+                  type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
+                  binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
+                  q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, exact_gradient=False,
+                  validate=True):
+    """[bloss[B]], differentiable w.r.t. coeffs, w0, w1, type_bias; nnmtp_bind.cc:116-191."""
+    _no_zbl(zbl_rmax)
+    args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, alpha_moments_count,
+            alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh,
+            brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, exact_gradient, validate)
+    return [_NNMtpToLoss.apply(coeffs, w0, w1, type_bias, args)]
+
+
+def nnMtpToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, coeffs, w0, w1, type_bias,
+                    alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
+                    bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler,
+                    zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, exact_gradient=False, validate=True):
+    """[bloss[B]] without virial labels (zero weight, zero labels); nnmtp_bind.cc:43-114."""
+    _no_zbl(zbl_rmax)
+    v_dft = torch.zeros((betot_dft.numel(), 9), dtype=betot_dft.dtype, device=betot_dft.device)
+    args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v_dft, chebyshev_size, alpha_moments_count,
+            alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh,
+            brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, exact_gradient, validate)
+    return [_NNMtpToLoss.apply(coeffs, w0, w1, type_bias, args)]
+
+
 # --------------------------------------------------------------------------------------------
 # fvt  (source/fvt/bind/fvt_sr_op_bind.cc:9-46)
 # --------------------------------------------------------------------------------------------

@@ -231,6 +231,39 @@ int a2p_nnmtp_efv_f32(void* plan, int chebyshev_size, int num_neurons, const flo
                       float* virial, float* e_sites, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Neural-network MTP training loss, forward and analytic backward -- replaces the compute of
+ * torch.ops.nnmtp.nnMtpToLossOp and nnMtpToEFLossOp
+ * (source/descriptor/nnmtp/bind/nnmtp_bind.cc:43-191; src/nnMtpOp.cc:569-2780;
+ *  include/nnMtpLoss.h:141-181 loss, :216-610 and :612-994 backward).
+ * Per structure  loss = e_w/N (E-E0)^2 + f_w/(3N) sum |F-F0|^2 + v_w/(9N) sum (V-V0)^2;
+ * nnMtpToEFLossOp is the same call with v_weight = 0 (v_dft still has to point at B*9 values).
+ * Outputs (device): bloss[B]; the model's etot[B], force[B,P,3], virial[B,9]; per-structure
+ * gradients dcoeffs[B, ntypes^2 nmus K], dw0[B, ntypes H S], dw1[B, ntypes H], dbias[B, ntypes] (any
+ * may be NULL; all NULL skips the backward kernels).  The operator's backward multiplies them by
+ * grad_output[B] (nnMtpOp.cc:2748-2780).  nghost is 0, as in the reference's loss launchers.
+ * exact_gradient = 0 evaluates the reference's backward formulas; these omit, for the force and
+ * virial terms, the dependence of dE/dM on the moments in d/dcoeffs (nnMtpLoss.h:497-529) and the
+ * off-diagonal part of the pre-activation tangent in d/dw0 (:560-585), so they are not the
+ * derivative of the loss.  exact_gradient = 1 returns the complete derivative.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nnmtp_loss_f64(void* plan, double e_weight, double f_weight, double v_weight, const double* e_dft,
+                       const double* f_dft, const double* v_dft, int chebyshev_size, int num_neurons,
+                       const double* coeffs, const double* w0, const double* w1, const double* type_bias, int nmus,
+                       int ntypes, const double* q_shifter, const double* q_scaler, double rmax, double rmin,
+                       int batch, int natoms_pad, int umax, const int* binum, const int* bilist,
+                       const int* bnumneigh, const int* bfirstneigh, const double* brcs, const int* btypes,
+                       double* bloss, double* etot, double* force, double* virial, double* dcoeffs, double* dw0,
+                       double* dw1, double* dbias, int exact_gradient, void* stream);
+int a2p_nnmtp_loss_f32(void* plan, double e_weight, double f_weight, double v_weight, const float* e_dft,
+                       const float* f_dft, const float* v_dft, int chebyshev_size, int num_neurons,
+                       const float* coeffs, const float* w0, const float* w1, const float* type_bias, int nmus,
+                       int ntypes, const float* q_shifter, const float* q_scaler, double rmax, double rmin,
+                       int batch, int natoms_pad, int umax, const int* binum, const int* bilist,
+                       const int* bnumneigh, const int* bfirstneigh, const float* brcs, const int* btypes,
+                       float* bloss, float* etot, float* force, float* virial, float* dcoeffs, float* dw0,
+                       float* dw1, float* dbias, int exact_gradient, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * NEP training loss, forward and analytic backward -- replaces the compute of
  * torch.ops.nep.nepToLossOp and torch.ops.nep.nepToEFLossOp
  * (source/descriptor/nep/bind/nep_bind.cc:136-276; src/nepOp.cc:2359-3484;

@@ -432,6 +432,45 @@ def nnmtp_efv(model, nb):
     return _nnmtp_efv(oracle_lib(), "orc_nnmtp", model, nb)
 
 
+def _nnmtp_loss_step(lib, prefix, model, nb, weights, labels):
+    coeffs = _c(model["coeffs"], np.float64)
+    w0, w1 = _c(model["w0"], np.float64), _c(model["w1"], np.float64)
+    bias = _c(model["type_bias"], np.float64)
+    basic = _c(model["alpha_index_basic"], np.int32)
+    times = _c(model["alpha_index_times"], np.int32)
+    mapping = _c(model["alpha_moment_mapping"], np.int32)
+    shift, scale = _c(model["q_shifter"], np.float64), _c(model["q_scaler"], np.float64)
+    type_map = _c(model["type_map"], np.int32)
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    assert nghost == 0
+    e_dft = _c(labels["energy"], np.float64)
+    f_dft = _c(labels["force"], np.float64)
+    v_dft = _c(labels["virial"], np.float64)
+    assert e_dft.shape == (B,) and f_dft.shape == (B, P, 3) and v_dft.shape == (B, 9)
+    out = dict(bloss=np.zeros(B), energy=np.zeros(B), force=np.zeros((B, P, 3)), virial=np.zeros((B, 9)),
+               dcoeffs=np.zeros((B, coeffs.size)), dw0=np.zeros((B, w0.size)), dw1=np.zeros((B, w1.size)),
+               dbias=np.zeros((B, bias.size)))
+    fn = getattr(lib, prefix + "_loss_step_f64")
+    fn.restype = None
+    fn(_p(out["bloss"]), _p(out["energy"]), _p(out["force"]), _p(out["virial"]), _p(out["dcoeffs"]), _p(out["dw0"]),
+       _p(out["dw1"]), _p(out["dbias"]), _D(weights[0]), _D(weights[1]), _D(weights[2]), _p(e_dft), _p(f_dft),
+       _p(v_dft), _I(model["chebyshev_size"]), _I(model["num_neurons"]), _p(coeffs), _p(w0), _p(w1), _p(bias),
+       _I(model["alpha_moments_count"]), _I(basic.shape[0]), _p(basic), _I(times.shape[0]), _p(times),
+       _I(mapping.size), _p(mapping), _I(model["nmus"]), _I(B), _I(P), _p(binum), _p(bilist), _p(bnumneigh),
+       _p(bfirst), _p(brcs), _p(btypes), _I(type_map.size), _p(type_map), _I(U), _I(nghost), _D(model["rmax"]),
+       _D(model["rmin"]), _p(shift), _p(scale))
+    return out
+
+
+def ref_nnmtp_loss_step(model, nb, weights, labels):
+    """Loss forward + the reference's find_loss_backward: per-structure gradients [B, n]."""
+    return _nnmtp_loss_step(_load("_ref/libref_nnmtp.so"), "ref_nnmtp", model, nb, weights, labels)
+
+
+def nnmtp_loss_step(model, nb, weights, labels):
+    return _nnmtp_loss_step(oracle_lib(), "orc_nnmtp", model, nb, weights, labels)
+
+
 # ----------------------------------------------------------------------------------------
 # fvt (single structure, fp64)
 # ----------------------------------------------------------------------------------------

@@ -41,10 +41,19 @@ struct Tables {
 
 // Read-out of the neural-network MTP (source/descriptor/nnmtp/include/nnMtp.h:470-507): one tanh
 // layer per centre species on the shifted and scaled scalar moments, no hidden bias.
+template <typename S>
 struct NNReadout {
     int H;
-    const double *w0, *w1, *shift;     // w0[ntypes, H, n_scalar], w1[ntypes, H], shift[n_scalar]
+    const S *w0, *w1;                  // w0[ntypes, H, n_scalar], w1[ntypes, H]
+    const double* shift;               // [n_scalar]
 };
+// nnMtpUtils.h:54-71: tanh from exponentials
+inline double tanh_exp(double h) { return (std::exp(h) - std::exp(-h)) / (std::exp(h) + std::exp(-h)); }
+inline Dual tanh_exp(Dual h)
+{
+    const double th = tanh_exp(h.v);
+    return {th, (1 - th * th) * h.d};
+}
 
 // f_k(r) = scaling * s(u) * T_k(x) and its r-derivative (basis.h:154-196, 351-381, 620-637)
 void radial_basis(int K, double rmax, double rmin, double scaling, double r, double* f, double* df)
@@ -76,7 +85,7 @@ void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeff
              const S* bias, const Tables& t, int inum, const int* ilist, const int* numneigh,
              const int* firstneigh, const double* rcs, const int* types, int ntypes, int U,
              int nforce, double rmax, double rmin, const double* q_scaler, S* e_sites = nullptr,
-             S* desc = nullptr, const NNReadout* net = nullptr)
+             S* desc = nullptr, const NNReadout<S>* net = nullptr)
 {
     etot = S(0);
     for (int i = 0; i < nforce * 3; i++) force[i] = S(0);   // linearMtp.h:228-230
@@ -122,23 +131,19 @@ void efv_one(S& etot, S* force, S* virial, int K, double scaling, const S* coeff
         }
         S e = bias[ti];                                        // linearMtp.h:281-285
         std::fill(adj.begin(), adj.end(), S(0));               // linearMtp.h:292-306
-        if constexpr (std::is_same<S, double>::value) {
-            if (net) {                                         // nnMtp.h:470-507
-                const double* w0 = net->w0 + (size_t)ti * net->H * t.n_scalar;
-                const double* w1 = net->w1 + (size_t)ti * net->H;
-                for (int p = 0; p < net->H; p++) {
-                    double h = 0;
-                    for (int s = 0; s < t.n_scalar; s++)
-                        h += w0[p * t.n_scalar + s] * (M[t.mapping[s]] - net->shift[s]) / q_scaler[s];
-                    // nnMtpUtils.h:54-71: tanh and its derivative from exponentials
-                    const double th = (std::exp(h) - std::exp(-h)) / (std::exp(h) + std::exp(-h));
-                    e += w1[p] * th;
-                    for (int s = 0; s < t.n_scalar; s++)
-                        adj[t.mapping[s]] += w1[p] * (1 - th * th) * w0[p * t.n_scalar + s] / q_scaler[s];
-                }
+        if (net) {                                             // nnMtp.h:470-507
+            const S* w0 = net->w0 + (size_t)ti * net->H * t.n_scalar;
+            const S* w1 = net->w1 + (size_t)ti * net->H;
+            for (int p = 0; p < net->H; p++) {
+                S h(0);
+                for (int s = 0; s < t.n_scalar; s++)
+                    h += w0[p * t.n_scalar + s] * (M[t.mapping[s]] - S(net->shift[s])) / S(q_scaler[s]);
+                const S th = tanh_exp(h);
+                e += w1[p] * th;
+                for (int s = 0; s < t.n_scalar; s++)
+                    adj[t.mapping[s]] += w1[p] * (S(1) - th * th) * w0[p * t.n_scalar + s] / S(q_scaler[s]);
             }
-        }
-        if (!net) {
+        } else {
             for (int s = 0; s < t.n_scalar; s++) e += lin[s] * M[t.mapping[s]] / S(q_scaler[s]);
             for (int s = 0; s < t.n_scalar; s++) adj[t.mapping[s]] = lin[s] / S(q_scaler[s]);
         }
@@ -367,12 +372,63 @@ void orc_nnmtp_efv_f64(double* betot, double* bforce, double* bvirial, double* e
                        const double* q_shifter, const double* q_scaler)
 {
     Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
-    NNReadout nn{H, w0, w1, q_shifter};
+    NNReadout<double> nn{H, w0, w1, q_shifter};
     for (int b = 0; b < B; b++)
         efv_one<double>(betot[b], &bforce[(size_t)b * (P + nghost) * 3], &bvirial[b * 9], K, 1.0, coeffs, nullptr,
                         bias, t, binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P],
                         &bfirstneigh[(size_t)b * P * U], &brcs[(size_t)b * P * U * 3],
                         &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost, rmax, rmin, q_scaler,
                         e_sites ? &e_sites[(size_t)b * P] : nullptr, nullptr, &nn);
+}
+
+// one training step of the neural-network MTP: E/F/V, per-structure loss (nnMtpLoss.h:141-181, the
+// linear MTP's formula) and its gradients w.r.t. coeffs, w0, w1, type_bias by forward-mode AD
+void orc_nnmtp_loss_step_f64(double* bloss, double* betot, double* bforce, double* bvirial, double* dcoeffs,
+                             double* dw0, double* dw1, double* dbias, double e_w, double f_w, double v_w,
+                             const double* e_dft, const double* f_dft, const double* v_dft, int K, int H,
+                             const double* coeffs, const double* w0, const double* w1, const double* bias,
+                             int n_moms, int n_basic, const int* basic, int n_times, const int* times,
+                             int n_scalar, const int* mapping, int nmus, int B, int P, const int* binum,
+                             const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                             const int* btypes, int ntypes, const int* type_map, int U, int nghost, double rmax,
+                             double rmin, const double* q_shifter, const double* q_scaler)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int ncoef = ntypes * ntypes * nmus * K, nw0 = ntypes * H * n_scalar, nw1 = ntypes * H;
+    const int npar = ncoef + nw0 + nw1 + ntypes;
+    NNReadout<double> nn{H, w0, w1, q_shifter};
+    for (int b = 0; b < B; b++) {
+        efv_one<double>(betot[b], &bforce[(size_t)b * P * 3], &bvirial[b * 9], K, 1.0, coeffs, nullptr, bias, t,
+                        binum[b], &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                        &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * P], ntypes, U, P, rmax, rmin, q_scaler,
+                        nullptr, nullptr, &nn);
+        bloss[b] = loss_one<double>(binum[b], &bilist[(size_t)b * P], e_w, f_w, v_w, betot[b], e_dft[b],
+                                    &bforce[(size_t)b * P * 3], &f_dft[(size_t)b * P * 3], &bvirial[b * 9],
+                                    &v_dft[b * 9]);
+    }
+#pragma omp parallel
+    {
+        std::vector<Dual> c(ncoef), a0(nw0), a1(nw1), bi(ntypes), force((size_t)P * 3), virial(9);
+#pragma omp for schedule(dynamic) collapse(2)
+        for (int b = 0; b < B; b++)
+            for (int p = 0; p < npar; p++) {
+                for (int i = 0; i < ncoef; i++) c[i] = Dual(coeffs[i], i == p);
+                for (int i = 0; i < nw0; i++) a0[i] = Dual(w0[i], ncoef + i == p);
+                for (int i = 0; i < nw1; i++) a1[i] = Dual(w1[i], ncoef + nw0 + i == p);
+                for (int i = 0; i < ntypes; i++) bi[i] = Dual(bias[i], ncoef + nw0 + nw1 + i == p);
+                NNReadout<Dual> nd{H, a0.data(), a1.data(), q_shifter};
+                Dual e;
+                efv_one<Dual>(e, force.data(), virial.data(), K, 1.0, c.data(), nullptr, bi.data(), t, binum[b],
+                              &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                              &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * P], ntypes, U, P, rmax, rmin,
+                              q_scaler, nullptr, nullptr, &nd);
+                Dual L = loss_one<Dual>(binum[b], &bilist[(size_t)b * P], e_w, f_w, v_w, e, e_dft[b], force.data(),
+                                        &f_dft[(size_t)b * P * 3], virial.data(), &v_dft[b * 9]);
+                if (p < ncoef) dcoeffs[(size_t)b * ncoef + p] = L.d;
+                else if (p < ncoef + nw0) dw0[(size_t)b * nw0 + p - ncoef] = L.d;
+                else if (p < ncoef + nw0 + nw1) dw1[(size_t)b * nw1 + p - ncoef - nw0] = L.d;
+                else dbias[(size_t)b * ntypes + p - ncoef - nw0 - nw1] = L.d;
+            }
+    }
 }
 }

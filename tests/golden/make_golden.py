@@ -120,6 +120,13 @@ def nnmtp_cases():
         e, f, v, es = oracle.ref_nnmtp_efv(m, nb)
         tag = "L%02d" % level
         out.update({tag + "/E": e, tag + "/F": f, tag + "/V": v, tag + "/esites": es})
+        B, P = nb["bilist"].shape
+        labels = dict(energy=synth.rng_normal(1, B, -4 * 48, 3),
+                      force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                      virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+        r = oracle.ref_nnmtp_loss_step(m, nb, (1.0, 0.7, 0.3), labels)
+        for k, val in r.items():
+            out[tag + "/loss_" + k] = val
     np.savez_compressed(os.path.join(HERE, "nnmtp.npz"), **out)
     print("nnmtp.npz")
 

@@ -179,6 +179,7 @@ def test_mtpr_ops(oracle, dropin, tmp_path):
 
 def test_nnmtp_ops(oracle, dropin, tmp_path):
     import torch
+    from ai2pot_amd import ops
     from test_gpu_nnmtp import model_to_device, op_args
     d = tmp_path / "_data" / "MTP_templates"
     d.mkdir(parents=True)
@@ -203,8 +204,25 @@ def test_nnmtp_ops(oracle, dropin, tmp_path):
     desc = torch.ops.nnmtp.nnMtpToDescriptorsOp(*(args[:2] + args[5:20]))[0]
     lin = dict(m); lin["scaling"] = 1.0; lin["linear_coeffs"] = np.zeros(m["q_scaler"].size)
     assert close(desc, oracle.mtp_esites(lin, nb)[1])
-    with pytest.raises(RuntimeError):                      # training operators are declared and refuse
-        torch.ops.nnmtp.nnMtpToEFLossOp(1.0, 1.0, e, f, *args)
+    # training operators: the reference's formulas by default, as committed from its own backward
+    B, P = nb["bilist"].shape
+    lab = dict(energy=synth.rng_normal(1, B, -200, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+               virial=synth.rng_normal(3, B * 9).reshape(B, 9))
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    params = [md[k].clone().requires_grad_(True) for k in ("coeffs", "w0", "w1", "type_bias")]
+    pargs = args[:1] + tuple(params) + args[5:]
+    out = torch.ops.nnmtp.nnMtpToLossOp(1.0, 0.7, 0.3, t(lab["energy"]), t(lab["force"]), t(lab["virial"]), *pargs)
+    assert len(out) == 1 and out[0].shape == (B,)
+    out[0].sum().backward()
+    r = ops.nnmtp_loss_step(1.0, 0.7, 0.3, t(lab["energy"]), t(lab["force"]), t(lab["virial"]), *args[:22],
+                            exact_gradient=False)
+    assert torch.equal(out[0].detach(), r["bloss"])
+    for prm, key in zip(params, ("dcoeffs", "dw0", "dw1", "dbias")):
+        assert close(prm.grad, r[key].sum(0).cpu().numpy()), key
+    rr = oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.3), lab)
+    assert close(out[0].detach(), rr["bloss"]) and close(params[2].grad, rr["dw1"].sum(0))
+    out2 = torch.ops.nnmtp.nnMtpToEFLossOp(1.0, 0.7, t(lab["energy"]), t(lab["force"]), *args)
+    assert len(out2) == 1 and close(out2[0], oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.0), lab)["bloss"])
     with pytest.raises(RuntimeError):
         torch.ops.nnmtp.nnMtpToEsitesOp(*(args[:2] + (md["w0"].clone().requires_grad_(True),) + args[3:]))
 

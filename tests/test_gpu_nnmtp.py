@@ -111,3 +111,94 @@ def test_errors(oracle):
     w0g = md["w0"].clone().requires_grad_(True)
     with pytest.raises(RuntimeError):                       # no silent gradient-free result
         ops.nnMtpToEsitesOp(*(args[:2] + [w0g] + args[3:]))
+
+
+def loss_inputs(oracle, level, nt, H, sizes=(48, 30, 37)):
+    lists = [structure(oracle, n, (8.5 + 0.1 * i, 9.0, 9.5), nt, 21 + 5 * i, 5.0) for i, n in enumerate(sizes)]
+    nb = synth.pack_batch(lists)
+    B, P = nb["bilist"].shape
+    m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.5, 3300 + level)
+    labels = dict(energy=synth.rng_normal(1, B, -4 * 40, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                  virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+    return m, nb, labels
+
+
+def gpu_loss(m, nb, labels, w, exact, want_grad=True):
+    import torch
+    from ai2pot_amd import ops
+    md = model_to_device(m, torch.float64)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    args = op_args(m, md, to_device(nb, torch.float64))
+    r = ops.nnmtp_loss_step(w[0], w[1], w[2], t(labels["energy"]), t(labels["force"]), t(labels["virial"]), *args,
+                            want_grad=want_grad, exact_gradient=exact)
+    torch.cuda.synchronize()
+    return {k: v.cpu().numpy() for k, v in r.items()}
+
+
+@pytest.mark.parametrize("level,nt,H", [(8, 2, 7), (10, 1, 12), (12, 3, 5)])
+def test_loss_step_complete_derivative(oracle, level, nt, H):
+    """exact_gradient=True against the oracle's forward-mode derivative of the loss (which agrees
+    with finite differences)."""
+    m, nb, labels = loss_inputs(oracle, level, nt, H)
+    w = (1.0, 0.7, 0.3)
+    got = gpu_loss(m, nb, labels, w, True)
+    ref = oracle.nnmtp_loss_step(m, nb, w, labels)
+    for k in ("bloss", "energy", "force", "virial", "dcoeffs", "dw0", "dw1", "dbias"):
+        assert close(got[k], ref[k]), k
+    fwd = gpu_loss(m, nb, labels, w, True, want_grad=False)
+    assert np.array_equal(fwd["bloss"], got["bloss"]) and "dcoeffs" not in fwd
+
+
+@pytest.mark.parametrize("level,nt,H", [(8, 2, 7), (16, 3, 20)])
+def test_loss_step_reference_formulas(oracle, level, nt, H):
+    """exact_gradient=False (the operators' default) against the committed output of the reference's
+    NNMtpLoss::find_loss_backward; and the two modes agree where the reference's formulas are
+    complete: on w1 and type_bias always, on everything for an energy-only loss."""
+    with np.load(os.path.join(os.path.dirname(__file__), "golden", "nnmtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    ty = synth.rng_randint(22, 48, nt)
+    m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.8, 3200 + level)
+    o = oracle.nblist(lat, ty, pos, 5.0, 100)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.01
+    B, P = nb["bilist"].shape
+    labels = dict(energy=synth.rng_normal(1, B, -4 * 48, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                  virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+    got = gpu_loss(m, nb, labels, (1.0, 0.7, 0.3), False)
+    for k in ("bloss", "energy", "force", "virial", "dcoeffs", "dw0", "dw1", "dbias"):
+        assert close(got[k], g["loss_" + k]), k
+    full = gpu_loss(m, nb, labels, (1.0, 0.7, 0.3), True)
+    assert close(full["dw1"], got["dw1"]) and close(full["dbias"], got["dbias"])
+    assert not close(full["dcoeffs"], got["dcoeffs"], 1e-4)          # the omitted terms are not small
+    e_only_ref, e_only_full = (gpu_loss(m, nb, labels, (1.0, 0.0, 0.0), x) for x in (False, True))
+    for k in ("dcoeffs", "dw0", "dw1", "dbias"):
+        assert close(e_only_ref[k], e_only_full[k]), k
+
+
+def test_loss_autograd_contract(oracle):
+    """One output, bloss[B]; backward = grad_output @ per-structure gradients to coeffs, w0, w1, type_bias."""
+    import torch
+    from ai2pot_amd import ops
+    m, nb, labels = loss_inputs(oracle, 8, 2, 7)
+    md = model_to_device(m, torch.float64)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    for k in ("coeffs", "w0", "w1", "type_bias"):
+        md[k].requires_grad_(True)
+    args = op_args(m, md, to_device(nb, torch.float64))
+    out = ops.nnMtpToLossOp(1.0, 0.7, 0.3, t(labels["energy"]), t(labels["force"]), t(labels["virial"]), *args,
+                            0.0, 0.0, None, None, exact_gradient=True)
+    assert len(out) == 1 and out[0].shape == (3,)
+    out[0].mean().backward()
+    ref = oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.3), labels)
+    for k, g in (("coeffs", "dcoeffs"), ("w0", "dw0"), ("w1", "dw1"), ("type_bias", "dbias")):
+        assert close(md[k].grad.cpu().numpy(), ref[g].mean(0)), k
+    # energy + force variant = zero virial weight
+    for k in ("coeffs", "w0", "w1", "type_bias"):
+        md[k].grad = None
+    out2 = ops.nnMtpToEFLossOp(1.0, 0.7, t(labels["energy"]), t(labels["force"]), *args, 0.0, 0.0, None, None,
+                               exact_gradient=True)
+    out2[0].sum().backward()
+    ref2 = oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.0), labels)
+    assert close(out2[0].detach().cpu().numpy(), ref2["bloss"])
+    assert close(md["w0"].grad.cpu().numpy(), ref2["dw0"].sum(0))

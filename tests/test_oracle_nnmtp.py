@@ -96,3 +96,53 @@ def test_reference_tanh_form(oracle):
     e, f, v, es = oracle.nnmtp_efv(m, nb)
     want = m["type_bias"][0] + m["w1"][0] * np.tanh(-(m["w0"] * m["q_shifter"] / m["q_scaler"]).sum())
     assert abs(e[0] - want) < 1e-15 and np.all(f == 0) and np.all(v == 0)
+
+
+def labels_for(nb):
+    B, P = nb["bilist"].shape
+    return dict(energy=synth.rng_normal(1, B, -4 * 48, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+
+
+def test_loss_step_against_golden(oracle):
+    """The restated loss step against the committed output of the reference (level 8): loss, E/F/V and
+    the gradients w.r.t. w1 and type_bias agree.  The gradients w.r.t. coeffs and w0 do NOT: the
+    reference's NNMtpLoss::find_loss_backward leaves out, for the force and virial terms, the
+    dependence of dE/dM on the moments (nnMtpLoss.h:497-529 has no counterpart of
+    linearMtpLoss.h:417-434) and the off-diagonal part of the pre-activation tangent (:560-585).
+    The oracle's forward-mode derivative is the complete one: it agrees with finite differences
+    (next test), the reference's does not."""
+    with np.load(os.path.join(HERE, "golden", "nnmtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L08/")}
+    m, nb = small_batch(oracle, 8, 2, 7)
+    r = oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.3), labels_for(nb))
+    for k in ("bloss", "energy", "force", "virial", "dw1", "dbias"):
+        ref = g["loss_" + k]
+        assert np.abs(r[k] - ref).max() <= 1e-10 * max(np.abs(ref).max(), 1e-300), k
+    for k in ("dcoeffs", "dw0"):
+        ref = g["loss_" + k]
+        assert np.abs(r[k] - ref).max() > 1e-4 * np.abs(ref).max(), k
+    if oracle.ref_available("nnmtp"):
+        # with an energy-only loss the reference's formulas are complete
+        r1 = oracle.nnmtp_loss_step(m, nb, (1.0, 0.0, 0.0), labels_for(nb))
+        g1 = oracle.ref_nnmtp_loss_step(m, nb, (1.0, 0.0, 0.0), labels_for(nb))
+        for k in ("dcoeffs", "dw0", "dw1", "dbias"):
+            assert np.abs(r1[k] - g1[k]).max() <= 1e-10 * np.abs(g1[k]).max(), k
+
+
+def test_loss_gradient_by_finite_differences(oracle):
+    m, nb = small_batch(oracle, 8, 2, 7)
+    lab = labels_for(nb)
+    w = (1.0, 0.7, 0.3)
+    r0 = oracle.nnmtp_loss_step(m, nb, w, lab)
+    h = 1e-6
+    for key, gkey, idxs in (("coeffs", "dcoeffs", (0, 17, 40)), ("w0", "dw0", (0, 33, 100)), ("w1", "dw1", (2, 9)),
+                            ("type_bias", "dbias", (1,))):
+        for i in idxs:
+            mp, mm = dict(m), dict(m)
+            mp[key] = m[key].copy(); mp[key][i] += h
+            mm[key] = m[key].copy(); mm[key][i] -= h
+            lp = oracle.nnmtp_loss_step(mp, nb, w, lab)["bloss"]
+            lm = oracle.nnmtp_loss_step(mm, nb, w, lab)["bloss"]
+            fd = (lp - lm) / (2 * h)
+            assert np.abs(fd - r0[gkey][:, i]).max() < 1e-5 * max(1.0, np.abs(fd).max()), (key, i)
