@@ -1,9 +1,8 @@
 // libnnmtp_bind.so -- registers torch.ops.nnmtp.* with the reference's schemas
 // (source/descriptor/nnmtp/bind/nnmtp_bind.cc:27-430) on top of libai2pot_hip.so:
-// set_ai2pot_path, mtpParamOp, nnMtpToEFVOp, nnMtpToEFOp, nnMtpToEsitesOp (forward),
-// nnMtpToDescriptorsOp, nnMtpToLossOp and nnMtpToEFLossOp (autograd to coeffs, w0, w1, type_bias as
-// src/nnMtpOp.cc:2748-2780).  The backward of nnMtpToEsitesOp is not part of this build: parameters
-// that require grad are refused.
+// set_ai2pot_path, mtpParamOp, nnMtpToEFVOp, nnMtpToEFOp, nnMtpToEsitesOp, nnMtpToDescriptorsOp,
+// nnMtpToLossOp and nnMtpToEFLossOp (autograd to coeffs, w0, w1, type_bias as
+// src/nnMtpOp.cc:2748-2780, 4170-4330).
 // The loss operators evaluate the reference's backward formulas, which are not the complete
 // derivative of the loss (see include/ai2pot_hip.h, a2p_nnmtp_loss_*); with the environment variable
 // A2P_NNMTP_EXACT_GRADIENT=1 they return the complete derivative instead.
@@ -118,6 +117,75 @@ variable_list nnmtp_descriptors(int64_t K, const at::Tensor& coeffs, int64_t n_m
     return {desc};
 }
 
+// forward: [e_sites[B, P]]; backward: sum over structures and rows of grad * d e_sites / d theta.
+// The reference writes its per-row w0 / w1 derivatives without the species offset
+// (nnMtp.h:965-971 against the allocation at nnMtpOp.cc:4236-4239), which mis-assigns them for more
+// than one species; this returns the derivative itself (identical for a single species).
+struct NNEsitesFunction : public torch::autograd::Function<NNEsitesFunction> {
+    static variable_list forward(AutogradContext* ctx, int64_t K, const at::Tensor& coeffs, const at::Tensor& w0,
+                                 const at::Tensor& w1, const at::Tensor& bias, int64_t n_moms,
+                                 const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping,
+                                 int64_t nmus, const at::Tensor& binum, const at::Tensor& bilist,
+                                 const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                                 const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rmax,
+                                 double rmin, const at::Tensor& q_shifter, const at::Tensor& q_scaler)
+    {
+        variable_list out = nnmtp_run(false, false, true, NNMTP_PASS);
+        ctx->save_for_backward({coeffs, w0, w1, bias, basic, times, mapping, binum, bilist, bnumneigh, bfirstneigh,
+                                brcs, btypes, type_map, q_shifter, q_scaler});
+        ctx->saved_data["K"] = K;
+        ctx->saved_data["n_moms"] = n_moms;
+        ctx->saved_data["nmus"] = nmus;
+        ctx->saved_data["nghost"] = nghost;
+        ctx->saved_data["rmax"] = rmax;
+        ctx->saved_data["rmin"] = rmin;
+        return out;
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(22);                   // one slot per forward argument after ctx
+        auto sv = ctx->get_saved_variables();
+        const at::Tensor &coeffs = sv[0], &w0 = sv[1], &w1 = sv[2], &bias = sv[3], &brcs = sv[11];
+        const int64_t K = ctx->saved_data["K"].toInt(), nmus = ctx->saved_data["nmus"].toInt(),
+                      nghost = ctx->saved_data["nghost"].toInt();
+        Batch s = check_batch(sv[7], sv[8], sv[9], sv[10], brcs, sv[12], nghost);
+        const int ntypes = (int)sv[13].numel();
+        a2p_bind::DeviceGuard guard(brcs);
+        PlanEntry plan = get_plan(brcs.device().index(), ctx->saved_data["n_moms"].toInt(), sv[4], sv[5], sv[6]);
+        const int H = (int)(w1.numel() / ntypes);
+        auto opt = brcs.options();
+        at::Tensor g = grads[0].contiguous();
+        TORCH_CHECK(g.dim() == 2 && g.size(0) == s.B && g.size(1) == s.P, "grad of e_sites must be [B, P]");
+        at::Tensor dc = at::zeros({s.B, coeffs.numel()}, opt), d0 = at::zeros({s.B, w0.numel()}, opt),
+                   d1 = at::zeros({s.B, w1.numel()}, opt), db = at::zeros({s.B, bias.numel()}, opt);
+        const double rmax = ctx->saved_data["rmax"].toDouble(), rmin = ctx->saved_data["rmin"].toDouble();
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+            rc = a2p_nnmtp_esites_bwd_f64(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                                          p(sv[14]), p(sv[15]), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                                          sv[7].data_ptr<int>(), sv[8].data_ptr<int>(), sv[9].data_ptr<int>(),
+                                          sv[10].data_ptr<int>(), p(brcs), sv[12].data_ptr<int>(), p(g), p(dc), p(d0),
+                                          p(d1), p(db), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+            rc = a2p_nnmtp_esites_bwd_f32(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                                          p(sv[14]), p(sv[15]), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                                          sv[7].data_ptr<int>(), sv[8].data_ptr<int>(), sv[9].data_ptr<int>(),
+                                          sv[10].data_ptr<int>(), p(brcs), sv[12].data_ptr<int>(), p(g), p(dc), p(d0),
+                                          p(d1), p(db), st);
+        }
+        check_rc(rc);
+        out[1] = dc.sum(0).reshape(coeffs.sizes());
+        out[2] = d0.sum(0).reshape(w0.sizes());
+        out[3] = d1.sum(0).reshape(w1.sizes());
+        out[4] = db.sum(0).reshape(bias.sizes());
+        return out;
+    }
+};
+
 // forward: [bloss]; backward: grad_output @ per-structure gradients
 struct NNLossFunction : public torch::autograd::Function<NNLossFunction> {
     static variable_list forward(AutogradContext* ctx, bool with_virial, double e_w, double f_w, double v_w,
@@ -226,10 +294,7 @@ TORCH_LIBRARY(nnmtp, m)
     });
     m.def("nnMtpToEsitesOp", [](NNMTP_ARGS) -> variable_list {
         require_no_zbl(zbl_rmax);
-        for (auto* t : {&coeffs, &w0, &w1, &bias})
-            TORCH_CHECK(!(at::GradMode::is_enabled() && t->requires_grad()),
-                        "nnMtpToEsitesOp: the backward to coeffs, w0, w1, type_bias is not implemented in this build");
-        return nnmtp_run(false, false, true, NNMTP_PASS);
+        return NNEsitesFunction::apply(NNMTP_PASS);
     });
     m.def("nnMtpToDescriptorsOp",
           [](int64_t K, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times,

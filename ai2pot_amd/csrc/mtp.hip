@@ -1179,6 +1179,51 @@ int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T
     return A2P_OK;
 }
 
+// The same for the neural-network MTP: gradients w.r.t. coeffs, w0, w1, type_bias
+// (nnMtp.h:756-990, contracted with gout as nnMtpOp.cc does after find_e_sites_backward).
+template <typename T>
+int nnmtp_esites_bwd(void* handle, int K, const MtpNet<T>& net, const T* coeffs, const T* bias, int nmus,
+                     int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P, int U, int nghost,
+                     const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
+                     const T* brcs, const int* btypes, const T* gout, T* dcoeffs, T* dw0, T* dw1, T* dbias,
+                     hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    A2P_REQUIRE(gout && (dcoeffs || dw0 || dw1 || dbias), A2P_ERR_INVALID, "nnmtp e_sites backward: null pointer");
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, 1.0, coeffs, (const T*)nullptr, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U,
+                   nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes);
+    if (rc) return rc;
+    rc = set_net(a, &net);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    const int S = a.p.n_scalar, H = net.H;
+    const int nblk = ntypes * nmus * K;
+    const int nrow = nblk + H * S + H + 1;
+    // workspace: dVs[B*9] | dFs[(B*P + nghost)*3] (both zero) | gpart[B*P*nrow]
+    const size_t nzero = (size_t)B * 9 + ((size_t)B * P + nghost) * 3;
+    void* ws = nullptr;
+    rc = ws_get(WS_MTP, (nzero + (size_t)B * P * nrow) * sizeof(T), &ws);
+    if (rc) return rc;
+    T* dVs = (T*)ws;
+    T* dFs = dVs + (size_t)B * 9;
+    T* gpart = (T*)ws + nzero;
+    rc = fill_zero(ws, ((nzero * sizeof(T) + 3) / 4) * 4, stream);
+    if (rc) return rc;
+    a.E = table_entries<T>(a.p, K, true);
+    a.cE = gout; a.cE_per_atom = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = nrow;
+    rc = launch_atoms<T, true>(a, stream);
+    if (rc) return rc;
+    prof_begin("mtp_grad_reduce", stream);
+    hipLaunchKernelGGL(nnmtp_grad_reduce_kernel<T>, dim3(ceil_div(nrow, 256), ntypes, B), dim3(256), 0, stream, P,
+                       P + nghost, nblk, H * S, H, ntypes, binum, bilist, btypes, gpart, dcoeffs, dw0, dw1, dbias);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 }  // namespace
 }  // namespace a2p
 
@@ -1277,6 +1322,20 @@ int a2p_mtp_esites_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int ng
     }
 NNMTP_ENTRY(double, f64)
 NNMTP_ENTRY(float, f32)
+
+#define NNMTP_ESITES_BWD_ENTRY(T, SUFFIX)                                                                         \
+    int a2p_nnmtp_esites_bwd_##SUFFIX(void* plan, int K, int H, const T* coeffs, const T* w0, const T* w1,          \
+                                      const T* bias, int nmus, int ntypes, const T* q_shifter, const T* q_scaler,   \
+                                      double rmax, double rmin, int B, int P, int U, int nghost, MTP_BATCH(T),      \
+                                      const T* grad_e_sites, T* dcoeffs, T* dw0, T* dw1, T* dbias, void* stream)    \
+    {                                                                                                             \
+        a2p::MtpNet<T> net{H, w0, w1, q_shifter};                                                                   \
+        return a2p::nnmtp_esites_bwd<T>(plan, K, net, coeffs, bias, nmus, ntypes, q_scaler, rmax, rmin, B, P, U,    \
+                                        nghost, MTP_BATCH_PASS, grad_e_sites, dcoeffs, dw0, dw1, dbias,            \
+                                        (hipStream_t)stream);                                                       \
+    }
+NNMTP_ESITES_BWD_ENTRY(double, f64)
+NNMTP_ESITES_BWD_ENTRY(float, f32)
 
 #define NNMTP_LOSS_ENTRY(T, SUFFIX)                                                                              \
     int a2p_nnmtp_loss_##SUFFIX(void* plan, double e_w, double f_w, double v_w, const T* e_dft, const T* f_dft,    \

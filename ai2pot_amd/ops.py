@@ -703,22 +703,75 @@ def nnMtpToEFOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, 
     return [e, f]
 
 
+def nnmtp_esites_backward(grad_esites, chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
+                          alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
+                          bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler):
+    """Per-structure gradients of sum_i grad_esites[b, i] * e_sites[b, i]:
+    (dcoeffs[B, ncoef], dw0[B, ntypes*H*S], dw1[B, ntypes*H], dbias[B, ntypes])."""
+    dtype, device = brcs.dtype, brcs.device
+    nghost = int(nghost)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost)
+    ntypes = int(type_map.numel())
+    plan, n_scalar = _mtp_plan(alpha_moments_count, alpha_index_basic, alpha_index_times,
+                               alpha_moment_mapping, device)
+    H = w1.numel() // ntypes
+    _check_float("grad_esites", grad_esites, dtype, device)
+    _req(tuple(grad_esites.shape) == (B, P), "grad_esites must have shape [B, P]")
+    z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
+    out = (z(B, coeffs.numel()), z(B, w0.numel()), z(B, w1.numel()), z(B, ntypes))
+    L = _lib.lib()
+    fn = L.a2p_nnmtp_esites_bwd_f32 if dtype == torch.float32 else L.a2p_nnmtp_esites_bwd_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0), _ptr(w1), _ptr(type_bias),
+                _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_shifter), _ptr(q_scaler), _c.c_double(rmax),
+                _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
+                _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(grad_esites),
+                _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _ptr(out[3]), _stream(device))
+        _lib.check(rc)
+    return out
+
+
+class _NNMtpToEsites(torch.autograd.Function):
+    """Site energies of the neural-network MTP; gradients flow to coeffs, w0, w1, type_bias, summed
+    over structures and rows (nnMtpOp.cc:4170-4330).  The reference fills its per-row derivative
+    tensors for w0 and w1 without the species offset (nnMtp.h:965-971 index rows of num_neurons
+    entries inside tensors allocated with ntypes * num_neurons, nnMtpOp.cc:4236-4239), so for more
+    than one species its result is mis-assigned; this build returns the derivative itself, which
+    coincides with the reference for a single species."""
+
+    @staticmethod
+    def forward(ctx, coeffs, w0, w1, type_bias, args):
+        (K, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+         nghost, rmax, rmin, q_shifter, q_scaler, validate) = args
+        _, _, _, es = _nnmtp_call(("es",), K, coeffs.detach(), w0.detach(), w1.detach(), type_bias.detach(), n_moms,
+                                  basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                                  type_map, nghost, rmax, rmin, q_shifter, q_scaler, validate)
+        ctx.save_for_backward(coeffs, w0, w1, type_bias)
+        ctx.args = args
+        return es
+
+    @staticmethod
+    def backward(ctx, ges):
+        coeffs, w0, w1, type_bias = ctx.saved_tensors
+        (K, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+         nghost, rmax, rmin, q_shifter, q_scaler, _) = ctx.args
+        g = nnmtp_esites_backward(ges.contiguous(), K, coeffs.detach(), w0.detach(), w1.detach(),
+                                  type_bias.detach(), n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                                  bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler)
+        return tuple(x.sum(0).reshape(p.shape) for x, p in zip(g, (coeffs, w0, w1, type_bias))) + (None,)
+
+
 def nnMtpToEsitesOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, alpha_index_basic,
                     alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
                     btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
                     zbl_cks=None, zbl_dks=None, validate=True):
-    """[e_sites[B, P]] in row order; nnmtp_bind.cc:370-430.  Forward only: the reference's backward
-    to coeffs, w0, w1, type_bias (nnMtp.h:756-990) is not part of this build, so parameters that
-    require grad are refused instead of returning a result that silently carries no gradient."""
+    """[e_sites[B, P]] in row order, differentiable w.r.t. coeffs, w0, w1, type_bias;
+    nnmtp_bind.cc:370-430."""
     _no_zbl(zbl_rmax)
-    for name, t in (("coeffs", coeffs), ("w0", w0), ("w1", w1), ("type_bias", type_bias)):
-        _req(not (torch.is_grad_enabled() and t.requires_grad),
-             "nnMtpToEsitesOp: the backward w.r.t. %s is not implemented in this build" % name)
-    _, _, _, es = _nnmtp_call(("es",), chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
-                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
-                              bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
-                              q_scaler, validate)
-    return [es]
+    args = (chebyshev_size, alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
+            binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler,
+            validate)
+    return [_NNMtpToEsites.apply(coeffs, w0, w1, type_bias, args)]
 
 
 def nnMtpToDescriptorsOp(chebyshev_size, coeffs, alpha_moments_count, alpha_index_basic, alpha_index_times,

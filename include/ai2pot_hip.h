@@ -230,6 +230,24 @@ int a2p_nnmtp_efv_f32(void* plan, int chebyshev_size, int num_neurons, const flo
                       const int* bfirstneigh, const float* brcs, const int* btypes, float* etot, float* force,
                       float* virial, float* e_sites, void* stream);
 
+/* Backward of nnMtpToEsitesOp (src/nnMtpOp.cc:4170-4330; include/nnMtp.h:756-990 find_e_sites_backward):
+ * per structure  sum_ii grad_e_sites[b, ii] * d e_sites[b, ii] / d theta  into dcoeffs[B, ntypes^2 nmus K],
+ * dw0[B, ntypes H S], dw1[B, ntypes H], dbias[B, ntypes] (any may be NULL); the operator sums them over the batch. */
+int a2p_nnmtp_esites_bwd_f64(void* plan, int chebyshev_size, int num_neurons, const double* coeffs,
+                             const double* w0, const double* w1, const double* type_bias, int nmus, int ntypes,
+                             const double* q_shifter, const double* q_scaler, double rmax, double rmin, int batch,
+                             int natoms_pad, int umax, int nghost, const int* binum, const int* bilist,
+                             const int* bnumneigh, const int* bfirstneigh, const double* brcs, const int* btypes,
+                             const double* grad_e_sites, double* dcoeffs, double* dw0, double* dw1, double* dbias,
+                             void* stream);
+int a2p_nnmtp_esites_bwd_f32(void* plan, int chebyshev_size, int num_neurons, const float* coeffs, const float* w0,
+                             const float* w1, const float* type_bias, int nmus, int ntypes, const float* q_shifter,
+                             const float* q_scaler, double rmax, double rmin, int batch, int natoms_pad, int umax,
+                             int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                             const int* bfirstneigh, const float* brcs, const int* btypes,
+                             const float* grad_e_sites, float* dcoeffs, float* dw0, float* dw1, float* dbias,
+                             void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Neural-network MTP training loss, forward and analytic backward -- replaces the compute of
  * torch.ops.nnmtp.nnMtpToLossOp and nnMtpToEFLossOp

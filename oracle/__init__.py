@@ -471,6 +471,38 @@ def nnmtp_loss_step(model, nb, weights, labels):
     return _nnmtp_loss_step(oracle_lib(), "orc_nnmtp", model, nb, weights, labels)
 
 
+def _nnmtp_esites_bwd(lib, prefix, model, nb, gout):
+    coeffs = _c(model["coeffs"], np.float64)
+    w0, w1 = _c(model["w0"], np.float64), _c(model["w1"], np.float64)
+    bias = _c(model["type_bias"], np.float64)
+    basic = _c(model["alpha_index_basic"], np.int32)
+    times = _c(model["alpha_index_times"], np.int32)
+    mapping = _c(model["alpha_moment_mapping"], np.int32)
+    shift, scale = _c(model["q_shifter"], np.float64), _c(model["q_scaler"], np.float64)
+    type_map = _c(model["type_map"], np.int32)
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    gout = _c(gout, np.float64)
+    assert gout.shape == (B, P)
+    out = (np.zeros((B, coeffs.size)), np.zeros((B, w0.size)), np.zeros((B, w1.size)), np.zeros((B, bias.size)))
+    fn = getattr(lib, prefix + "_esites_bwd_f64")
+    fn.restype = None
+    fn(_p(out[0]), _p(out[1]), _p(out[2]), _p(out[3]), _p(gout), _I(model["chebyshev_size"]),
+       _I(model["num_neurons"]), _p(coeffs), _p(w0), _p(w1), _p(bias), _I(model["alpha_moments_count"]),
+       _I(basic.shape[0]), _p(basic), _I(times.shape[0]), _p(times), _I(mapping.size), _p(mapping),
+       _I(model["nmus"]), _I(B), _I(P), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes),
+       _I(type_map.size), _p(type_map), _I(U), _I(nghost), _D(model["rmax"]), _D(model["rmin"]), _p(shift), _p(scale))
+    return out
+
+
+def ref_nnmtp_esites_bwd(model, nb, gout):
+    """Per-structure gradients of sum(gout * e_sites) w.r.t. coeffs, w0, w1, type_bias (reference)."""
+    return _nnmtp_esites_bwd(_load("_ref/libref_nnmtp.so"), "ref_nnmtp", model, nb, gout)
+
+
+def nnmtp_esites_bwd(model, nb, gout):
+    return _nnmtp_esites_bwd(oracle_lib(), "orc_nnmtp", model, nb, gout)
+
+
 # ----------------------------------------------------------------------------------------
 # fvt (single structure, fp64)
 # ----------------------------------------------------------------------------------------

@@ -6,6 +6,7 @@
 // NNMtpLoss::find_loss (include/nnMtpLoss.h:141-181), then find_loss_backward (:216-610) per
 // structure, i.e. the per-structure gradients before the grad_output matmul.
 #include <cstring>
+#include <vector>
 #include "descriptor/nnmtp/include/nnMtp.h"
 
 using namespace ai2pot::nnmtp;
@@ -80,6 +81,45 @@ void ref_nnmtp_loss_step_f64(double* bloss, double* betot, double* bforce, doubl
             (double(*)[3])const_cast<double*>(&brcs[(size_t)b * P * U * 3]),
             const_cast<int*>(&btypes[(size_t)b * (P + nghost)]), ntypes, const_cast<int*>(type_map), U, nghost, rmax,
             rmin, const_cast<double*>(q_shifter), const_cast<double*>(q_scaler));
+    }
+}
+
+// per-row derivatives of the site energies (nnMtp.h:756-990), contracted with gout[B, P] per structure
+// as the operator's backward does before its sum over the batch
+void ref_nnmtp_esites_bwd_f64(double* dcoeffs, double* dw0, double* dw1, double* dbias, const double* gout, int K,
+                              int H, const double* coeffs, const double* w0, const double* w1, const double* bias,
+                              int n_moms, int n_basic, const int* basic, int n_times, const int* times,
+                              int n_scalar, const int* mapping, int nmus, int B, int P, const int* binum,
+                              const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                              const int* btypes, int ntypes, const int* type_map, int U, int nghost, double rmax,
+                              double rmin, const double* q_shifter, const double* q_scaler)
+{
+    const int ncoef = ntypes * ntypes * nmus * K, nw0 = ntypes * H * n_scalar, nw1 = ntypes * H;
+    std::vector<double> pc((size_t)P * ncoef), p0((size_t)P * nw0), p1((size_t)P * nw1), pb((size_t)P * ntypes);
+    for (int b = 0; b < B; b++) {
+        std::fill(pc.begin(), pc.end(), 0.0);
+        std::fill(p0.begin(), p0.end(), 0.0);
+        std::fill(p1.begin(), p1.end(), 0.0);
+        std::fill(pb.begin(), pb.end(), 0.0);
+        NNMtp<double>::find_e_sites_backward(
+            pc.data(), p0.data(), p1.data(), pb.data(), K, H, const_cast<double*>(coeffs), const_cast<double*>(w0),
+            const_cast<double*>(w1), const_cast<double*>(bias), n_moms, n_basic, (const int(*)[4])basic, n_times,
+            (const int(*)[4])times, n_scalar, mapping, nmus, binum[b], const_cast<int*>(&bilist[(size_t)b * P]),
+            const_cast<int*>(&bnumneigh[(size_t)b * P]), const_cast<int*>(&bfirstneigh[(size_t)b * P * U]),
+            (double(*)[3])const_cast<double*>(&brcs[(size_t)b * P * U * 3]),
+            const_cast<int*>(&btypes[(size_t)b * (P + nghost)]), ntypes, const_cast<int*>(type_map), U, nghost, rmax,
+            rmin, const_cast<double*>(q_shifter), const_cast<double*>(q_scaler));
+        auto contract = [&](const std::vector<double>& per, int n, double* out) {
+            for (int q = 0; q < n; q++) {
+                double a = 0;
+                for (int ii = 0; ii < binum[b]; ii++) a += gout[(size_t)b * P + ii] * per[(size_t)ii * n + q];
+                out[(size_t)b * n + q] = a;
+            }
+        };
+        contract(pc, ncoef, dcoeffs);
+        contract(p0, nw0, dw0);
+        contract(p1, nw1, dw1);
+        contract(pb, ntypes, dbias);
     }
 }
 }

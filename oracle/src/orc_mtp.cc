@@ -431,4 +431,42 @@ void orc_nnmtp_loss_step_f64(double* bloss, double* betot, double* bforce, doubl
             }
     }
 }
+
+// d/dtheta of sum_ii gout[b, ii] e_sites[b, ii] per structure for the neural-network MTP, forward-mode AD
+void orc_nnmtp_esites_bwd_f64(double* dcoeffs, double* dw0, double* dw1, double* dbias, const double* gout, int K,
+                              int H, const double* coeffs, const double* w0, const double* w1, const double* bias,
+                              int n_moms, int n_basic, const int* basic, int n_times, const int* times,
+                              int n_scalar, const int* mapping, int nmus, int B, int P, const int* binum,
+                              const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                              const int* btypes, int ntypes, const int* type_map, int U, int nghost, double rmax,
+                              double rmin, const double* q_shifter, const double* q_scaler)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int ncoef = ntypes * ntypes * nmus * K, nw0 = ntypes * H * n_scalar, nw1 = ntypes * H;
+    const int npar = ncoef + nw0 + nw1 + ntypes;
+#pragma omp parallel
+    {
+        std::vector<Dual> c(ncoef), a0(nw0), a1(nw1), bi(ntypes), force((size_t)(P + nghost) * 3), virial(9), es(P);
+#pragma omp for schedule(dynamic) collapse(2)
+        for (int b = 0; b < B; b++)
+            for (int p = 0; p < npar; p++) {
+                for (int i = 0; i < ncoef; i++) c[i] = Dual(coeffs[i], i == p);
+                for (int i = 0; i < nw0; i++) a0[i] = Dual(w0[i], ncoef + i == p);
+                for (int i = 0; i < nw1; i++) a1[i] = Dual(w1[i], ncoef + nw0 + i == p);
+                for (int i = 0; i < ntypes; i++) bi[i] = Dual(bias[i], ncoef + nw0 + nw1 + i == p);
+                NNReadout<Dual> nd{H, a0.data(), a1.data(), q_shifter};
+                Dual e;
+                efv_one<Dual>(e, force.data(), virial.data(), K, 1.0, c.data(), nullptr, bi.data(), t, binum[b],
+                              &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                              &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost,
+                              rmax, rmin, q_scaler, es.data(), nullptr, &nd);
+                double acc = 0;
+                for (int ii = 0; ii < binum[b]; ii++) acc += gout[(size_t)b * P + ii] * es[ii].d;
+                if (p < ncoef) dcoeffs[(size_t)b * ncoef + p] = acc;
+                else if (p < ncoef + nw0) dw0[(size_t)b * nw0 + p - ncoef] = acc;
+                else if (p < ncoef + nw0 + nw1) dw1[(size_t)b * nw1 + p - ncoef - nw0] = acc;
+                else dbias[(size_t)b * ntypes + p - ncoef - nw0 - nw1] = acc;
+            }
+    }
+}
 }

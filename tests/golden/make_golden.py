@@ -111,7 +111,7 @@ def nnmtp_cases():
     """Neural-network MTP: E/F/V and site energies of the reference's NNMtp (fp64)."""
     out = {}
     lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
-    for level, nt, H in ((8, 2, 7), (16, 3, 20)):
+    for level, nt, H in ((8, 2, 7), (16, 3, 20), (10, 1, 6)):
         ty = synth.rng_randint(22, 48, nt)
         m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.8, 3200 + level)
         o = oracle.ref_nblist(lat, ty, pos, 5.0, 100)
@@ -127,6 +127,10 @@ def nnmtp_cases():
         r = oracle.ref_nnmtp_loss_step(m, nb, (1.0, 0.7, 0.3), labels)
         for k, val in r.items():
             out[tag + "/loss_" + k] = val
+        if nt == 1:     # the reference's site-energy backward assigns w0 / w1 rows correctly only for one species
+            g = oracle.ref_nnmtp_esites_bwd(m, nb, synth.rng_normal(4, B * P).reshape(B, P))
+            for k, val in zip(("dcoeffs", "dw0", "dw1", "dbias"), g):
+                out[tag + "/es_" + k] = val
     np.savez_compressed(os.path.join(HERE, "nnmtp.npz"), **out)
     print("nnmtp.npz")
 

@@ -223,8 +223,11 @@ def test_nnmtp_ops(oracle, dropin, tmp_path):
     assert close(out[0].detach(), rr["bloss"]) and close(params[2].grad, rr["dw1"].sum(0))
     out2 = torch.ops.nnmtp.nnMtpToEFLossOp(1.0, 0.7, t(lab["energy"]), t(lab["force"]), *args)
     assert len(out2) == 1 and close(out2[0], oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.0), lab)["bloss"])
-    with pytest.raises(RuntimeError):
-        torch.ops.nnmtp.nnMtpToEsitesOp(*(args[:2] + (md["w0"].clone().requires_grad_(True),) + args[3:]))
+    w0g = md["w0"].clone().requires_grad_(True)
+    es_g = torch.ops.nnmtp.nnMtpToEsitesOp(*(args[:2] + (w0g,) + args[3:]))[0]
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    (es_g * t(gout)).sum().backward()
+    assert close(w0g.grad, oracle.nnmtp_esites_bwd(m, nb, gout)[1].sum(0))
 
 
 def test_fvt_ops(oracle, dropin):

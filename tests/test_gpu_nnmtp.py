@@ -108,9 +108,6 @@ def test_errors(oracle):
         ops.nnMtpToEFVOp(*(args[:2] + [md["w0"][:-1].contiguous()] + args[3:]))
     with pytest.raises(RuntimeError):                       # ZBL is not part of this build
         ops.nnMtpToEFVOp(*args, 2.0, 1.0, None, None)
-    w0g = md["w0"].clone().requires_grad_(True)
-    with pytest.raises(RuntimeError):                       # no silent gradient-free result
-        ops.nnMtpToEsitesOp(*(args[:2] + [w0g] + args[3:]))
 
 
 def loss_inputs(oracle, level, nt, H, sizes=(48, 30, 37)):
@@ -202,3 +199,34 @@ def test_loss_autograd_contract(oracle):
     ref2 = oracle.nnmtp_loss_step(m, nb, (1.0, 0.7, 0.0), labels)
     assert close(out2[0].detach().cpu().numpy(), ref2["bloss"])
     assert close(md["w0"].grad.cpu().numpy(), ref2["dw0"].sum(0))
+
+
+@pytest.mark.parametrize("level,nt,H", [(8, 2, 7), (10, 1, 6)])
+def test_site_energy_backward(oracle, level, nt, H):
+    """Autograd of nnMtpToEsitesOp against the oracle's forward-mode derivative (two species, a padded
+    structure) and, for one species, against the committed output of the reference's
+    find_e_sites_backward (for several species the reference mis-assigns its w0 / w1 rows)."""
+    import torch
+    from ai2pot_amd import ops
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    ty = synth.rng_randint(22, 48, nt)
+    m = synth.nnmtp_model(mtp_param.mtp_param(level), nt, 8, H, 5.0, 1.8, 3200 + level)
+    o = oracle.nblist(lat, ty, pos, 5.0, 100)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.01
+    B, P = nb["bilist"].shape
+    gout = synth.rng_normal(4, B * P).reshape(B, P)
+    md = model_to_device(m, torch.float64)
+    for k in ("coeffs", "w0", "w1", "type_bias"):
+        md[k].requires_grad_(True)
+    args = op_args(m, md, to_device(nb, torch.float64))
+    es = ops.nnMtpToEsitesOp(*args, 0.0, 0.0, None, None)[0]
+    (es * torch.from_numpy(gout).to("cuda:0")).sum().backward()
+    ref = oracle.nnmtp_esites_bwd(m, nb, gout)
+    for k, r in zip(("coeffs", "w0", "w1", "type_bias"), ref):
+        assert close(md[k].grad.cpu().numpy(), r.sum(0)), k
+    if nt == 1:
+        with np.load(os.path.join(os.path.dirname(__file__), "golden", "nnmtp.npz")) as z:
+            g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+        for k, gk in (("coeffs", "es_dcoeffs"), ("w0", "es_dw0"), ("w1", "es_dw1"), ("type_bias", "es_dbias")):
+            assert close(md[k].grad.cpu().numpy(), g[gk].sum(0)), k
