@@ -2,9 +2,9 @@
 // (source/descriptor/mtpr/bind/mtpr_bind.cc:30-569) on top of libai2pot_hip.so:
 // set_ai2pot_path, mtpParamOp, linearMtpToEFVOp, linearMtpToEFOp, linearMtpToLossOp,
 // linearMtpToEFLossOp, linearMtpToEsitesOp (autograd to coeffs, linear_coeffs, type_bias only, as
-// src/linearMtpOp.cc:1732-1765, 4002-4027) and linearMtpToDescriptorsOp.  The legacy and solver
-// operators of the reference (mtpBasisOp, LinMatrixLinVectorOp, CoeffsSchmidtOrthOp) are not part
-// of this build.
+// src/linearMtpOp.cc:1732-1765, 4002-4027), linearMtpToDescriptorsOp, and the linear-solver
+// operators LinMatrixLinVectorOp and CoeffsSchmidtOrthOp.  The legacy mtpBasisOp is not part of
+// this build.
 #include "mtp_bind_common.h"
 
 namespace {
@@ -264,6 +264,73 @@ variable_list mtp_descriptors(int64_t K, double scaling, const at::Tensor& coeff
     return {desc};
 }
 
+// normal equations of the linear parameters (linear_mtp_gram_and_cross.h:446-575): components by the
+// library, Gram products by torch's BLAS
+variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at::Tensor& e_dft,
+                                    const at::Tensor& f_dft, const at::Tensor& v_dft, int64_t K, double scaling,
+                                    const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic,
+                                    const at::Tensor& times, const at::Tensor& mapping, int64_t nmus,
+                                    const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+                                    const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+                                    const at::Tensor& type_map, int64_t nghost, double rmax, double rmin,
+                                    const at::Tensor& q_scaler)
+{
+    TORCH_CHECK(nghost == 0, "LinMatrixLinVectorOp requires nghost == 0: the reference's force components have "
+                             "natoms_pad rows");
+    auto opt = brcs.options();
+    at::Tensor lin0 = at::zeros({mapping.numel()}, opt), bias0 = at::zeros({type_map.numel()}, opt);
+    MtpCtx c = check_mtp(K, coeffs, lin0, bias0, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
+                         bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
+    check_device_float(brcs, e_dft, "betot_dft");
+    check_device_float(brcs, f_dft, "bforce_dft");
+    check_device_float(brcs, v_dft, "bvirial_dft");
+    const int B = c.s.B, P = c.s.P;
+    const int64_t n = c.plan.n_scalar + c.ntypes;
+    TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
+                "label tensors must have shapes [B], [B, P, 3], [B, 9]");
+    a2p_bind::DeviceGuard guard(brcs);
+    at::Tensor ec = at::zeros({B, n}, opt), fc = at::zeros({(int64_t)B * P * 3, n}, opt), vc = at::zeros({B * 9, n}, opt);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble) {
+        auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+        rc = a2p_mtp_lin_components_f64(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
+                                        rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                        btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
+    } else {
+        auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+        rc = a2p_mtp_lin_components_f32(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
+                                        rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                        btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
+    }
+    check_rc(rc);
+    check_device_status(brcs);
+    at::Tensor A = e_w * at::matmul(ec.t(), ec) + f_w * at::matmul(fc.t(), fc) + v_w * at::matmul(vc.t(), vc);
+    at::Tensor b = e_w * at::matmul(ec.t(), e_dft.reshape({B})) + f_w * at::matmul(fc.t(), f_dft.reshape({-1})) +
+                   v_w * at::matmul(vc.t(), v_dft.reshape({-1}));
+    return {A, b};
+}
+
+variable_list schmidt_orth(int64_t ntypes, int64_t nmus, int64_t K, const at::Tensor& coeffs)
+{
+    TORCH_CHECK(coeffs.is_cuda(), "coeffs must be on a HIP device: this build has no CPU path");
+    TORCH_CHECK((coeffs.scalar_type() == at::kFloat || coeffs.scalar_type() == at::kDouble) && coeffs.is_contiguous(),
+                "coeffs must be a contiguous float32 or float64 tensor");
+    TORCH_CHECK(coeffs.numel() == ntypes * ntypes * nmus * K, "coeffs size mismatch");
+    a2p_bind::DeviceGuard guard(coeffs);
+    at::Tensor src = coeffs.detach(), out = at::empty_like(src);
+    void* st = current_stream(coeffs);
+    const int rc = coeffs.scalar_type() == at::kDouble
+                       ? a2p_mtp_schmidt_orth_f64((int)ntypes, (int)nmus, (int)K, src.data_ptr<double>(),
+                                                  out.data_ptr<double>(), st)
+                       : a2p_mtp_schmidt_orth_f32((int)ntypes, (int)nmus, (int)K, src.data_ptr<float>(),
+                                                  out.data_ptr<float>(), st);
+    check_rc(rc);
+    return {out};
+}
+
 }  // namespace
 
 #define MTP_EFV_ARGS int64_t K, double scaling, const at::Tensor& coeffs, const at::Tensor& lin, \
@@ -296,6 +363,17 @@ TORCH_LIBRARY(mtpr, m)
               return LossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
                                          at::zeros({e_dft.numel(), 9}, e_dft.options()), MTP_EFV_PASS);
           });
+    m.def("LinMatrixLinVectorOp",
+          [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
+             const at::Tensor& v_dft, MTP_EFV_ARGS) -> variable_list {
+              require_no_zbl(zbl_rmax);
+              return lin_matrix_lin_vector(e_w, f_w, v_w, e_dft, f_dft, v_dft, K, scaling, coeffs, n_moms, basic, times,
+                                           mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+                                           nghost, rmax, rmin, q_scaler);
+          });
+    m.def("CoeffsSchmidtOrthOp", [](int64_t ntypes, int64_t nmus, int64_t K, const at::Tensor& coeffs) -> variable_list {
+        return schmidt_orth(ntypes, nmus, K, coeffs);
+    });
     m.def("linearMtpToEsitesOp", [](MTP_EFV_ARGS) -> variable_list {
         require_no_zbl(zbl_rmax);
         return EsitesFunction::apply(MTP_EFV_PASS);

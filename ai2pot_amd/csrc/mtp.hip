@@ -659,6 +659,68 @@ nnmtp_grad_reduce_kernel(int P, int NF, int nblk, int HS, int H, int ntypes, con
     else if (dbias) dbias[(size_t)b * ntypes + t] = acc;
 }
 
+// dst[(i * ncols) + col] = src[i] for i < n: one column of a row-major matrix
+template <typename T>
+__global__ void __launch_bounds__(256)
+column_store_kernel(T* __restrict__ dst, const T* __restrict__ src, long long n, int ncols, int col)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i * ncols + col] = src[i];
+}
+
+// eye[s * S + s] = 1 (the matrix is zero-filled before); counts[b, S + t] = atoms of species t
+template <typename T>
+__global__ void __launch_bounds__(256)
+lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, int B, int P, int NF, int ntypes,
+                           const int* __restrict__ binum, const int* __restrict__ bilist,
+                           const int* __restrict__ btypes)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < S) eye[(size_t)i * S + i] = (T)1;
+    if (i < B * ntypes) {
+        const int b = i / ntypes, t = i - b * ntypes;
+        int cnt = 0;
+        for (int ii = 0; ii < binum[b]; ii++) {
+            const int c = bilist[(size_t)b * P + ii];
+            if ((unsigned)c < (unsigned)NF && btypes[(size_t)b * NF + c] == t) cnt++;
+        }
+        ecomp[(size_t)b * (S + ntypes) + S + t] = (T)cnt;
+    }
+}
+
+// Gram-Schmidt over the nmus radial functions, each the vector of its ntypes^2 * K coefficients
+// (schmidt_orth.h:38-116), in the reference's summation order by one thread (the problem is tiny).
+template <typename T>
+__global__ void schmidt_orth_kernel(T* __restrict__ out, const T* __restrict__ in, int npairs, int nmus, int K)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int n = npairs * nmus * K;
+    for (int i = 0; i < n; i++) out[i] = in[i];
+    for (int k1 = 0; k1 < nmus; k1++) {
+        for (int k2 = 0; k2 < k1; k2++) {
+            T norm2 = (T)0, scal = (T)0;
+            for (int pr = 0; pr < npairs; pr++)
+                for (int xi = 0; xi < K; xi++) {
+                    const T v1 = out[(pr * nmus + k1) * K + xi], v2 = out[(pr * nmus + k2) * K + xi];
+                    norm2 += v2 * v2;
+                    scal += v1 * v2;
+                }
+            for (int pr = 0; pr < npairs; pr++)
+                for (int xi = 0; xi < K; xi++)
+                    out[(pr * nmus + k1) * K + xi] -= out[(pr * nmus + k2) * K + xi] * scal / norm2;
+        }
+        T norm2 = (T)1e-10;
+        for (int pr = 0; pr < npairs; pr++)
+            for (int xi = 0; xi < K; xi++) {
+                const T v = out[(pr * nmus + k1) * K + xi];
+                norm2 += v * v;
+            }
+        const T norm = sqrt_t(norm2);
+        for (int pr = 0; pr < npairs; pr++)
+            for (int xi = 0; xi < K; xi++) out[(pr * nmus + k1) * K + xi] /= norm;
+    }
+}
+
 // ---- plan construction ---------------------------------------------------------------------------
 std::mutex g_plan_mutex;
 std::set<MtpPlan*> g_plans;
@@ -1179,6 +1241,72 @@ int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T
     return A2P_OK;
 }
 
+// Energy, force and virial of every linear parameter taken alone (linear_mtp_gram_and_cross.h:125-374):
+// ecomp[B, n], fcomp[B, P, 3, n], vcomp[B, 9, n] with n = n_scalar + ntypes.  Column s < n_scalar is the
+// E/F/V of the model with linear_coeffs = e_s and no bias (the reference obtains the same numbers by
+// differentiating each scalar moment along every pair displacement); column n_scalar + t counts the
+// atoms of species t in the energy and is zero in force and virial.  One E/F/V pass per scalar
+// moment: simple and exact, at the price of recomputing the moments n_scalar times.
+template <typename T>
+int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int nmus, int ntypes,
+                       const T* q_scaler, double rmax, double rmin, int B, int P, int U, const int* binum,
+                       const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
+                       const int* btypes, T* ecomp, T* fcomp, T* vcomp, hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    A2P_REQUIRE(ecomp && fcomp && vcomp, A2P_ERR_INVALID, "mtp components: null output pointer");
+    A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0, A2P_ERR_INVALID, "mtp components: bad shape");
+    const int S = plan->d.n_scalar, n = S + ntypes;
+    if (B == 0 || P == 0) return A2P_OK;
+    // workspace: eye[S*S] | zero bias[ntypes] | etot[B] | force[B*P*3] | virial[B*9]
+    const size_t nT = (size_t)S * S + ntypes + B + (size_t)B * P * 3 + (size_t)B * 9;
+    void* ws = nullptr;
+    rc = ws_get(WS_MISC, nT * sizeof(T), &ws);
+    if (rc) return rc;
+    T* eye = (T*)ws;
+    T* zero_bias = eye + (size_t)S * S;
+    T* etot = zero_bias + ntypes;
+    T* force = etot + B;
+    T* virial = force + (size_t)B * P * 3;
+    rc = fill_zero(ws, (((size_t)S * S + ntypes) * sizeof(T) + 3) / 4 * 4, stream);
+    if (rc) return rc;
+    rc = fill_zero(ecomp, (size_t)B * n * sizeof(T), stream);
+    if (rc) return rc;
+    rc = fill_zero(fcomp, (size_t)B * P * 3 * n * sizeof(T), stream);
+    if (rc) return rc;
+    rc = fill_zero(vcomp, (size_t)B * 9 * n * sizeof(T), stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(std::max(S, B * ntypes), 256)), dim3(256), 0,
+                       stream, eye, S, ecomp, B, P, P, ntypes, binum, bilist, btypes);
+    A2P_HIP_CHECK(hipGetLastError());
+    for (int s = 0; s < S; s++) {
+        // force / virial go to WS_MISC, which mtp_efv does not touch when a force pointer is given
+        rc = mtp_efv<T>(handle, K, scaling, coeffs, eye + (size_t)s * S, zero_bias, nmus, ntypes, q_scaler, rmax, rmin,
+                        B, P, U, 0, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, stream);
+        if (rc) return rc;
+        hipLaunchKernelGGL(column_store_kernel<T>, dim3(ceil_div(B, 256)), dim3(256), 0, stream, ecomp, etot,
+                           (long long)B, n, s);
+        hipLaunchKernelGGL(column_store_kernel<T>, dim3(ceil_div((long long)B * P * 3, 256)), dim3(256), 0, stream,
+                           fcomp, force, (long long)B * P * 3, n, s);
+        hipLaunchKernelGGL(column_store_kernel<T>, dim3(ceil_div(B * 9, 256)), dim3(256), 0, stream, vcomp, virial,
+                           (long long)B * 9, n, s);
+        A2P_HIP_CHECK(hipGetLastError());
+    }
+    return A2P_OK;
+}
+
+template <typename T>
+int mtp_schmidt_orth(int ntypes, int nmus, int K, const T* coeffs, T* out, hipStream_t stream)
+{
+    A2P_REQUIRE(ntypes >= 1 && nmus >= 1 && K >= 1 && coeffs && out && coeffs != out, A2P_ERR_INVALID,
+                "schmidt orth: bad argument");
+    hipLaunchKernelGGL(schmidt_orth_kernel<T>, dim3(1), dim3(64), 0, stream, out, coeffs, ntypes * ntypes, nmus, K);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 // The same for the neural-network MTP: gradients w.r.t. coeffs, w0, w1, type_bias
 // (nnMtp.h:756-990, contracted with gout as nnMtpOp.cc does after find_e_sites_backward).
 template <typename T>
@@ -1322,6 +1450,21 @@ int a2p_mtp_esites_f32(void* plan, MTP_MODEL(float), int B, int P, int U, int ng
     }
 NNMTP_ENTRY(double, f64)
 NNMTP_ENTRY(float, f32)
+
+#define MTP_SOLVER_ENTRIES(T, SUFFIX)                                                                            \
+    int a2p_mtp_lin_components_##SUFFIX(void* plan, int K, double scaling, const T* coeffs, int nmus, int ntypes,   \
+                                        const T* q_scaler, double rmax, double rmin, int B, int P, int U,           \
+                                        MTP_BATCH(T), T* ecomp, T* fcomp, T* vcomp, void* stream)                   \
+    {                                                                                                             \
+        return a2p::mtp_lin_components<T>(plan, K, scaling, coeffs, nmus, ntypes, q_scaler, rmax, rmin, B, P, U,    \
+                                          MTP_BATCH_PASS, ecomp, fcomp, vcomp, (hipStream_t)stream);                \
+    }                                                                                                             \
+    int a2p_mtp_schmidt_orth_##SUFFIX(int ntypes, int nmus, int K, const T* coeffs, T* orth_coeffs, void* stream)   \
+    {                                                                                                             \
+        return a2p::mtp_schmidt_orth<T>(ntypes, nmus, K, coeffs, orth_coeffs, (hipStream_t)stream);                 \
+    }
+MTP_SOLVER_ENTRIES(double, f64)
+MTP_SOLVER_ENTRIES(float, f32)
 
 #define NNMTP_ESITES_BWD_ENTRY(T, SUFFIX)                                                                         \
     int a2p_nnmtp_esites_bwd_##SUFFIX(void* plan, int K, int H, const T* coeffs, const T* w0, const T* w1,          \

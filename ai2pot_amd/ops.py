@@ -624,6 +624,83 @@ def linearMtpToDescriptorsOp(chebyshev_size, scaling, coeffs, alpha_moments_coun
     return [desc]
 
 
+def mtp_lin_components(chebyshev_size, scaling, coeffs, alpha_moments_count, alpha_index_basic, alpha_index_times,
+                       alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
+                       rmax, rmin, q_scaler, validate=True):
+    """Energy [B, n], force [B, P, 3, n] and virial [B, 9, n] of every linear parameter taken alone,
+    n = alpha_scalar_moments + ntypes (linear_mtp_gram_and_cross.h:125-374)."""
+    ntypes = int(type_map.numel())
+    S = int(alpha_moment_mapping.numel())
+    dtype, device = brcs.dtype, brcs.device
+    dummy_lin = torch.zeros((S,), dtype=dtype, device=device)
+    dummy_bias = torch.zeros((ntypes,), dtype=dtype, device=device)
+    dtype, device, B, P, U, nghost, ntypes, plan, n_scalar = _mtp_common(
+        coeffs, dummy_lin, dummy_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
+        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, 0, q_scaler,
+        chebyshev_size, validate)
+    n = n_scalar + ntypes
+    z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
+    ecomp, fcomp, vcomp = z(B, n), z(B, P, 3, n), z(B, 9, n)
+    L = _lib.lib()
+    fn = L.a2p_mtp_lin_components_f32 if dtype == torch.float32 else L.a2p_mtp_lin_components_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _c.c_int(int(nmus)),
+                _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P),
+                _c.c_int(U), _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes),
+                _ptr(ecomp), _ptr(fcomp), _ptr(vcomp), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return ecomp, fcomp, vcomp
+
+
+def LinMatrixLinVectorOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, scaling,
+                         coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic,
+                         alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                         btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None,
+                         zbl_dks=None, validate=True):
+    """[lin_matrix[n, n], lin_vector[n]]: the normal equations of the linear parameters
+    (linear_coeffs / q_scaler, then type_bias) for fixed radial coefficients; mtpr_bind.cc:57-131,
+    linear_mtp_gram_and_cross.h:446-575.  linear_coeffs and type_bias do not enter, as in the
+    reference; no gradient."""
+    _no_zbl(zbl_rmax)
+    _req(int(nghost) == 0, "LinMatrixLinVectorOp requires nghost == 0: the reference's force components "
+                           "have natoms_pad rows")
+    ecomp, fcomp, vcomp = mtp_lin_components(chebyshev_size, scaling, coeffs.detach(), alpha_moments_count,
+                                             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
+                                             binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, rmax,
+                                             rmin, q_scaler, validate)
+    B, P = bilist.shape
+    n = ecomp.shape[1]
+    for name, t, numel in (("betot_dft", betot_dft, B), ("bforce_dft", bforce_dft, B * P * 3),
+                           ("bvirial_dft", bvirial_dft, B * 9)):
+        _check_float(name, t, brcs.dtype, brcs.device)
+        _req(t.numel() == numel, "%s has %d elements, expected %d" % (name, t.numel(), numel))
+    F = fcomp.reshape(B * P * 3, n)          # rows of padded atoms are zero
+    V = vcomp.reshape(B * 9, n)
+    lin_matrix = e_weight * (ecomp.t() @ ecomp) + f_weight * (F.t() @ F) + v_weight * (V.t() @ V)
+    lin_vector = (e_weight * (ecomp.t() @ betot_dft.reshape(B)) + f_weight * (F.t() @ bforce_dft.reshape(-1)) +
+                  v_weight * (V.t() @ bvirial_dft.reshape(-1)))
+    return [lin_matrix, lin_vector]
+
+
+def CoeffsSchmidtOrthOp(ntypes, nmus, chebyshev_size, coeffs):
+    """[orth_coeffs]: Gram-Schmidt over the nmus radial functions (mtpr_bind.cc:38-55,
+    schmidt_orth.h:38-116); same shape as coeffs, no gradient."""
+    _req(isinstance(coeffs, torch.Tensor) and coeffs.is_cuda, "coeffs must be a tensor on a HIP device")
+    _req(coeffs.dtype in (torch.float32, torch.float64) and coeffs.is_contiguous(),
+         "coeffs must be a contiguous float32 or float64 tensor")
+    _req(coeffs.numel() == int(ntypes) * int(ntypes) * int(nmus) * int(chebyshev_size), "coeffs size mismatch")
+    src = coeffs.detach()
+    out = torch.empty_like(src)
+    L = _lib.lib()
+    fn = L.a2p_mtp_schmidt_orth_f32 if src.dtype == torch.float32 else L.a2p_mtp_schmidt_orth_f64
+    with torch.cuda.device(src.device):
+        _lib.check(fn(_c.c_int(int(ntypes)), _c.c_int(int(nmus)), _c.c_int(int(chebyshev_size)), _ptr(src),
+                      _ptr(out), _stream(src.device)))
+    return [out]
+
+
 # --------------------------------------------------------------------------------------------
 # neural-network MTP  (source/descriptor/nnmtp/bind/nnmtp_bind.cc:193-430)
 # --------------------------------------------------------------------------------------------

@@ -206,6 +206,36 @@ int a2p_mtp_esites_bwd_f32(void* plan, int chebyshev_size, double scaling, const
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Linear solver support of the linear MTP -- replaces the compute of torch.ops.mtpr.LinMatrixLinVectorOp
+ * and torch.ops.mtpr.CoeffsSchmidtOrthOp (source/descriptor/mtpr/bind/mtpr_bind.cc:38-131;
+ *  include/linear_mtp_gram_and_cross.h:125-374 components, :377-443 accumulation, :446-575 launcher;
+ *  include/schmidt_orth.h:38-116).
+ * a2p_mtp_lin_components_*: with n = n_scalar + ntypes, per structure the energy ecomp[B, n], force
+ * fcomp[B, P, 3, n] and virial vcomp[B, 9, n] of every linear parameter taken alone (column s: scalar
+ * moment s over q_scaler[s]; column n_scalar + t: the species count in the energy, zero elsewhere).
+ * The normal equations of the reference,
+ *   lin_matrix = sum_b e_w E_b^T E_b + f_w F_b^T F_b + v_w V_b^T V_b,   lin_vector = the same against the residuals,
+ * are plain GEMMs over these arrays and are left to the caller's BLAS (the bind library uses torch's).
+ * nghost is 0, as the reference's force_components has natoms_pad rows.
+ * a2p_mtp_schmidt_orth_*: Gram-Schmidt over the nmus radial functions, each the vector of its
+ * ntypes^2 * chebyshev_size coefficients; orth_coeffs must not alias coeffs.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_mtp_lin_components_f64(void* plan, int chebyshev_size, double scaling, const double* coeffs, int nmus,
+                               int ntypes, const double* q_scaler, double rmax, double rmin, int batch,
+                               int natoms_pad, int umax, const int* binum, const int* bilist, const int* bnumneigh,
+                               const int* bfirstneigh, const double* brcs, const int* btypes, double* ecomp,
+                               double* fcomp, double* vcomp, void* stream);
+int a2p_mtp_lin_components_f32(void* plan, int chebyshev_size, double scaling, const float* coeffs, int nmus,
+                               int ntypes, const float* q_scaler, double rmax, double rmin, int batch,
+                               int natoms_pad, int umax, const int* binum, const int* bilist, const int* bnumneigh,
+                               const int* bfirstneigh, const float* brcs, const int* btypes, float* ecomp,
+                               float* fcomp, float* vcomp, void* stream);
+int a2p_mtp_schmidt_orth_f64(int ntypes, int nmus, int chebyshev_size, const double* coeffs, double* orth_coeffs,
+                             void* stream);
+int a2p_mtp_schmidt_orth_f32(int ntypes, int nmus, int chebyshev_size, const float* coeffs, float* orth_coeffs,
+                             void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Neural-network MTP: energy, force, virial and site energies -- replaces the compute of
  * torch.ops.nnmtp.nnMtpToEFVOp / nnMtpToEFOp / nnMtpToEsitesOp (forward)
  * (source/descriptor/nnmtp/bind/nnmtp_bind.cc:193-322, 370-430; src/nnMtpOp.cc:2785-3190;

@@ -398,6 +398,49 @@ def mtp_esites_bwd(model, nb, gout):
     return _mtp_esites_bwd(oracle_lib(), "orc_mtp", model, nb, gout)
 
 
+def _mtp_lin_system(lib, prefix, model, nb, weights, labels):
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    assert nghost == 0
+    n = np.asarray(model["alpha_moment_mapping"]).size + ntypes
+    e_res = _c(labels["energy"], np.float64)
+    f_res = _c(labels["force"], np.float64)
+    v_res = _c(labels["virial"], np.float64)
+    assert e_res.shape == (B,) and f_res.shape == (B, P, 3) and v_res.shape == (B, 9)
+    A, b = np.zeros((n, n)), np.zeros(n)
+    fn = getattr(lib, prefix + "_lin_system_f64")
+    fn.restype = None
+    fn(_p(A), _p(b), _D(weights[0]), _D(weights[1]), _D(weights[2]), _p(e_res), _p(f_res), _p(v_res), *margs, *largs)
+    return A, b
+
+
+def ref_mtp_lin_system(model, nb, weights, labels):
+    """(lin_matrix[n, n], lin_vector[n]) of the reference's LinMatrixLinVector CPU launcher."""
+    return _mtp_lin_system(_load("_ref/libref_mtpr.so"), "ref_mtp", model, nb, weights, labels)
+
+
+def mtp_lin_system(model, nb, weights, labels):
+    return _mtp_lin_system(oracle_lib(), "orc_mtp", model, nb, weights, labels)
+
+
+def _schmidt(lib, prefix, coeffs, ntypes, nmus, K):
+    c = _c(coeffs, np.float64)
+    assert c.size == ntypes * ntypes * nmus * K
+    out = np.zeros_like(c)
+    fn = getattr(lib, prefix + "_schmidt_orth_f64")
+    fn.restype = None
+    fn(_p(out), _I(ntypes), _I(nmus), _I(K), _p(c))
+    return out
+
+
+def ref_mtp_schmidt_orth(coeffs, ntypes, nmus, K):
+    return _schmidt(_load("_ref/libref_mtpr.so"), "ref_mtp", coeffs, ntypes, nmus, K)
+
+
+def mtp_schmidt_orth(coeffs, ntypes, nmus, K):
+    return _schmidt(oracle_lib(), "orc_mtp", coeffs, ntypes, nmus, K)
+
+
 # ----------------------------------------------------------------------------------------
 # neural-network MTP (fp64)
 # ----------------------------------------------------------------------------------------

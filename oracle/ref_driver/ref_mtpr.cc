@@ -12,6 +12,8 @@
 #include "descriptor/mtpr/include/mtpParam.h"
 #include "descriptor/mtpr/include/linearMtp_cpu_launcher.h"
 #include "descriptor/mtpr/include/linearMtpLoss_cpu_launcher.h"
+#include "descriptor/mtpr/include/linear_mtp_gram_and_cross.h"
+#include "descriptor/mtpr/include/schmidt_orth.h"
 
 using namespace ai2pot::mtpr;
 
@@ -144,5 +146,25 @@ void ref_mtp_esites_bwd_f64(double* dcoeffs, double* dlin, double* dbias, const 
             dbias[(size_t)b * ntypes + q] = a;
         }
     }
+}
+
+// normal equations of the linear parameters by the reference's CPU launcher
+// (linear_mtp_gram_and_cross.h:446-575), residuals = labels (the operator subtracts only a ZBL part)
+void ref_mtp_lin_system_f64(double* lin_matrix, double* lin_vector, double e_w, double f_w, double v_w,
+                            const double* e_res, const double* f_res, const double* v_res, MTP_MODEL_ARGS,
+                            MTP_LIST_ARGS)
+{
+    LinearMtpGramAndCross<double>::find_lin_matrix_lin_vector_launcher(
+        lin_matrix, lin_vector, e_w, f_w, v_w, const_cast<double*>(e_res), (double(*)[3])const_cast<double*>(f_res),
+        const_cast<double*>(v_res), K, scaling, const_cast<double*>(coeffs), const_cast<double*>(lin),
+        const_cast<double*>(bias), n_moms, n_basic, (const int(*)[4])basic, n_times, (const int(*)[4])times, n_scalar,
+        mapping, nmus, B, P, const_cast<int*>(binum), const_cast<int*>(bilist), const_cast<int*>(bnumneigh),
+        const_cast<int*>(bfirstneigh), (double(*)[3])const_cast<double*>(brcs), const_cast<int*>(btypes), ntypes,
+        const_cast<int*>(type_map), U, nghost, rmax, rmin, const_cast<double*>(q_scaler));
+}
+
+void ref_mtp_schmidt_orth_f64(double* out, int ntypes, int nmus, int K, const double* in)
+{
+    CoeffsSchmidtOrth<double>::find_orthogonal_basis_set(out, ntypes, nmus, K, const_cast<double*>(in));
 }
 }

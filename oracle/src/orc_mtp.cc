@@ -13,6 +13,7 @@
 // test fixtures; the reference unit test's known answer E = -0.938157350795572
 // (tests/test_linearMtp.cc, efv_force_accuracy set-up); finite differences of E; switch
 // function end values (tests/test_basis.cc:106-111); linearity of E in linear_coeffs.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <type_traits>
@@ -467,6 +468,150 @@ void orc_nnmtp_esites_bwd_f64(double* dcoeffs, double* dw0, double* dw1, double*
                 else if (p < ncoef + nw0 + nw1) dw1[(size_t)b * nw1 + p - ncoef - nw0] = acc;
                 else dbias[(size_t)b * ntypes + p - ncoef - nw0 - nw1] = acc;
             }
+    }
+}
+
+// Normal equations of the linear parameters (linear_mtp_gram_and_cross.h:446-575): per structure the
+// energy / force / virial of every parameter taken alone (:125-374, by forward differentiation of the
+// scalar moments along each pair displacement), accumulated into lin_matrix[n, n] and lin_vector[n]
+// (:377-443), n = n_scalar + ntypes; the residuals are the labels themselves (no ZBL part).
+void orc_mtp_lin_system_f64(double* lin_matrix, double* lin_vector, double e_w, double f_w, double v_w,
+                            const double* e_res, const double* f_res, const double* v_res, MTP_MODEL_ARGS,
+                            MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int n = n_scalar + ntypes;
+    std::fill(lin_matrix, lin_matrix + (size_t)n * n, 0.0);
+    std::fill(lin_vector, lin_vector + n, 0.0);
+    int kmax = 0;
+    for (int i = 0; i < n_basic; i++) kmax = std::max(kmax, basic[i * 4 + 1] + basic[i * 4 + 2] + basic[i * 4 + 3]);
+    std::vector<double> ec(n), fc((size_t)P * 3 * n), vc((size_t)9 * n), M(n_moms), dM(n_moms), f(K), df(K),
+        pw((kmax + 1) * 3), rp(kmax + 1);
+    for (int b = 0; b < B; b++) {
+        std::fill(ec.begin(), ec.end(), 0.0);
+        std::fill(fc.begin(), fc.end(), 0.0);
+        std::fill(vc.begin(), vc.end(), 0.0);
+        const int* ilist = &bilist[(size_t)b * P];
+        const int* types = &btypes[(size_t)b * P];
+        for (int ii = 0; ii < binum[b]; ii++) {
+            const int ci = ilist[ii], ti = types[ci], nn = bnumneigh[(size_t)b * P + ii];
+            const int* first = &bfirstneigh[((size_t)b * P + ii) * U];
+            const double* rcs = &brcs[((size_t)b * P + ii) * U * 3];
+            // moments, as efv_one
+            std::fill(M.begin(), M.end(), 0.0);
+            auto pair_terms = [&](int jj, double& r) {
+                const double* v = &rcs[jj * 3];
+                r = std::sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
+                radial_basis(K, rmax, rmin, scaling, r, f.data(), df.data());
+                rp[0] = 1; pw[0] = pw[1] = pw[2] = 1;
+                for (int k = 1; k <= kmax; k++) {
+                    rp[k] = rp[k - 1] * r;
+                    for (int a = 0; a < 3; a++) pw[k * 3 + a] = pw[(k - 1) * 3 + a] * v[a];
+                }
+            };
+            for (int jj = 0; jj < nn; jj++) {
+                double r;
+                pair_terms(jj, r);
+                if (r > rmax) continue;
+                const double* c = &coeffs[(size_t)(ti * ntypes + types[first[jj]]) * nmus * K];
+                for (int i = 0; i < n_basic; i++) {
+                    const int* q = &basic[i * 4];
+                    double g = 0;
+                    for (int k = 0; k < K; k++) g += c[q[0] * K + k] * f[k];
+                    M[i] += g * pw[q[1] * 3] * pw[q[2] * 3 + 1] * pw[q[3] * 3 + 2] / rp[q[1] + q[2] + q[3]];
+                }
+            }
+            for (int i = 0; i < n_times; i++) {
+                const int* q = &times[i * 4];
+                M[q[3]] += q[2] * M[q[0]] * M[q[1]];
+            }
+            ec[n_scalar + ti] += 1.0;                                          // :248-255
+            for (int s = 0; s < n_scalar; s++) ec[s] += M[mapping[s]] / q_scaler[s];
+            // derivative of every moment along each component of each pair displacement, :258-352
+            for (int jj = 0; jj < nn; jj++) {
+                double r;
+                pair_terms(jj, r);
+                if (r > rmax) continue;
+                const int nj = first[jj];
+                const double* v = &rcs[jj * 3];
+                const double* c = &coeffs[(size_t)(ti * ntypes + types[nj]) * nmus * K];
+                for (int a = 0; a < 3; a++) {
+                    std::fill(dM.begin(), dM.end(), 0.0);
+                    for (int i = 0; i < n_basic; i++) {
+                        const int* q = &basic[i * 4];
+                        const int kk = q[1] + q[2] + q[3];
+                        double g = 0, dg = 0;
+                        for (int k = 0; k < K; k++) { g += c[q[0] * K + k] * f[k]; dg += c[q[0] * K + k] * df[k]; }
+                        const double mono = pw[q[1] * 3] * pw[q[2] * 3 + 1] * pw[q[3] * 3 + 2];
+                        double dmono = 0;
+                        if (q[1 + a] > 0) {
+                            int e[3] = {q[1], q[2], q[3]};
+                            e[a]--;
+                            dmono = q[1 + a] * pw[e[0] * 3] * pw[e[1] * 3 + 1] * pw[e[2] * 3 + 2];
+                        }
+                        dM[i] = dg * v[a] / r * mono / rp[kk] + g * dmono / rp[kk] -
+                                g * mono * kk / (rp[kk] * r * r) * v[a];
+                    }
+                    for (int i = 0; i < n_times; i++) {
+                        const int* q = &times[i * 4];
+                        dM[q[3]] += q[2] * (dM[q[0]] * M[q[1]] + M[q[0]] * dM[q[1]]);
+                    }
+                    for (int s = 0; s < n_scalar; s++) {
+                        const double d = dM[mapping[s]] / q_scaler[s];
+                        fc[((size_t)ci * 3 + a) * n + s] += d;
+                        fc[((size_t)nj * 3 + a) * n + s] -= d;
+                        for (int bb = 0; bb < 3; bb++) vc[(size_t)(a * 3 + bb) * n + s] -= d * v[bb];
+                    }
+                }
+            }
+        }
+        // accumulation, :377-443 (upper triangle, mirrored at the end)
+        for (int k1 = 0; k1 < n; k1++) {
+            for (int k2 = k1; k2 < n; k2++) lin_matrix[(size_t)k1 * n + k2] += e_w * ec[k1] * ec[k2];
+            lin_vector[k1] += e_w * e_res[b] * ec[k1];
+        }
+        for (int ii = 0; ii < binum[b]; ii++) {
+            const int ci = ilist[ii];
+            for (int a = 0; a < 3; a++) {
+                const double* row = &fc[((size_t)ci * 3 + a) * n];
+                for (int k1 = 0; k1 < n; k1++) {
+                    for (int k2 = k1; k2 < n; k2++) lin_matrix[(size_t)k1 * n + k2] += f_w * row[k1] * row[k2];
+                    lin_vector[k1] += f_w * f_res[((size_t)b * P + ci) * 3 + a] * row[k1];
+                }
+            }
+        }
+        for (int ab = 0; ab < 9; ab++) {
+            const double* row = &vc[(size_t)ab * n];
+            for (int k1 = 0; k1 < n; k1++) {
+                for (int k2 = k1; k2 < n; k2++) lin_matrix[(size_t)k1 * n + k2] += v_w * row[k1] * row[k2];
+                lin_vector[k1] += v_w * v_res[b * 9 + ab] * row[k1];
+            }
+        }
+    }
+    for (int k1 = 0; k1 < n; k1++)
+        for (int k2 = k1 + 1; k2 < n; k2++) lin_matrix[(size_t)k2 * n + k1] = lin_matrix[(size_t)k1 * n + k2];
+}
+
+// schmidt_orth.h:38-116
+void orc_mtp_schmidt_orth_f64(double* out, int ntypes, int nmus, int K, const double* in)
+{
+    const int np = ntypes * ntypes;
+    for (int i = 0; i < np * nmus * K; i++) out[i] = in[i];
+    auto at = [&](int pr, int mu, int xi) -> double& { return out[(pr * nmus + mu) * K + xi]; };
+    for (int k1 = 0; k1 < nmus; k1++) {
+        for (int k2 = 0; k2 < k1; k2++) {
+            double norm2 = 0, scal = 0;
+            for (int pr = 0; pr < np; pr++)
+                for (int xi = 0; xi < K; xi++) { norm2 += at(pr, k2, xi) * at(pr, k2, xi); scal += at(pr, k1, xi) * at(pr, k2, xi); }
+            for (int pr = 0; pr < np; pr++)
+                for (int xi = 0; xi < K; xi++) at(pr, k1, xi) -= at(pr, k2, xi) * scal / norm2;
+        }
+        double norm2 = 1e-10;
+        for (int pr = 0; pr < np; pr++)
+            for (int xi = 0; xi < K; xi++) norm2 += at(pr, k1, xi) * at(pr, k1, xi);
+        const double norm = std::sqrt(norm2);
+        for (int pr = 0; pr < np; pr++)
+            for (int xi = 0; xi < K; xi++) at(pr, k1, xi) /= norm;
     }
 }
 }

@@ -100,6 +100,11 @@ def mtp_cases():
         dc, dl, db = oracle.ref_mtp_esites_bwd(m, nb, synth.rng_normal(4, B * P).reshape(B, P))
         out.update({tag + "/esites": es, tag + "/desc": desc, tag + "/es_dcoeffs": dc,
                     tag + "/es_dlinear": dl, tag + "/es_dbias": db})
+        m2 = dict(m)
+        m2["q_scaler"] = np.linspace(0.7, 1.4, m["q_scaler"].size)
+        A, bv = oracle.ref_mtp_lin_system(m2, nb, (1.0, 0.7, 0.3), labels)
+        out.update({tag + "/lin_matrix": A, tag + "/lin_vector": bv,
+                    tag + "/orth_coeffs": oracle.ref_mtp_schmidt_orth(m["coeffs"], nt, t["nmus"], 8)})
         out[tag + "/table_sizes"] = np.array([t["alpha_moments_count"], t["alpha_index_basic"].shape[0],
                                               t["alpha_index_times"].shape[0],
                                               t["alpha_moment_mapping"].size, t["nmus"]])

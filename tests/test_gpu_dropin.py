@@ -163,6 +163,13 @@ def test_mtpr_ops(oracle, dropin, tmp_path):
     out2[0].sum().backward()
     r2 = oracle.mtp_loss_step(m, nb, (1.0, 0.7, 0.0), lab)
     assert close(out2[0].detach().cpu().numpy(), r2["bloss"]) and close(params2[0].grad.cpu().numpy(), r2["dcoeffs"].sum(0))
+    # linear-solver operators
+    A, bvec = torch.ops.mtpr.LinMatrixLinVectorOp(1.0, 0.7, 0.3, t(lab["energy"]), t(lab["force"]), t(lab["virial"]),
+                                                  *efv_args)
+    Ar, br = oracle.mtp_lin_system(m, nb, (1.0, 0.7, 0.3), lab)
+    assert close(A.cpu().numpy(), Ar) and close(bvec.cpu().numpy(), br)
+    oc = torch.ops.mtpr.CoeffsSchmidtOrthOp(2, int(p[6]), 8, md["coeffs"])
+    assert len(oc) == 1 and close(oc[0].cpu().numpy(), oracle.mtp_schmidt_orth(m["coeffs"], 2, int(p[6]), 8))
     # site energies (autograd) and descriptors
     params3 = [md[k].clone().requires_grad_(True) for k in ("coeffs", "linear_coeffs", "type_bias")]
     es = torch.ops.mtpr.linearMtpToEsitesOp(8, 1.0, params3[0], params3[1], params3[2], *efv_args[5:])

@@ -295,6 +295,50 @@ def test_site_energies_with_ghosts(oracle):
         assert close(a.cpu().numpy(), b)
 
 
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (12, 3)])
+def test_linear_system(oracle, level, nt):
+    """LinMatrixLinVectorOp against the oracle (a padded batch), fp64 1e-10."""
+    import torch
+    from ai2pot_amd import ops
+    m, nb, labels = loss_inputs(oracle, level, nt)
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    A, b = ops.LinMatrixLinVectorOp(1.0, 0.7, 0.3, t(labels["energy"]), t(labels["force"]), t(labels["virial"]),
+                                    *esites_args(m, md, d), 0.0, 0.0, None, None)
+    Ar, br = oracle.mtp_lin_system(m, nb, (1.0, 0.7, 0.3), labels)
+    assert close(A.cpu().numpy(), Ar) and close(b.cpu().numpy(), br)
+
+
+def test_linear_system_and_schmidt_against_golden(oracle):
+    """Level 16 against the committed outputs of the reference's CPU launcher and of its Gram-Schmidt."""
+    import os
+    import torch
+    from ai2pot_amd import ops
+    with np.load(os.path.join(os.path.dirname(__file__), "golden", "mtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L16/")}
+    lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+    ty = synth.rng_randint(22, 48, 3)
+    m = synth.mtp_model(mtp_param.mtp_param(16), 3, 8, 5.0, 1.8, 3016)
+    m["q_scaler"] = np.linspace(0.7, 1.4, m["q_scaler"].size)
+    o = oracle.nblist(lat, ty, pos, 5.0, 100)
+    nb = synth.pack_batch([o, o])
+    nb["brcs"][1] *= 1.01
+    B, P = nb["bilist"].shape
+    labels = dict(energy=synth.rng_normal(1, B, -4 * 48, 3), force=synth.rng_normal(2, B * P * 3).reshape(B, P, 3),
+                  virial=synth.rng_normal(3, B * 9, 0, 0.5).reshape(B, 9))
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    A, b = ops.LinMatrixLinVectorOp(1.0, 0.7, 0.3, t(labels["energy"]), t(labels["force"]), t(labels["virial"]),
+                                    *esites_args(m, md, d), 0.0, 0.0, None, None)
+    assert close(A.cpu().numpy(), g["lin_matrix"]) and close(b.cpu().numpy(), g["lin_vector"])
+    oc = ops.CoeffsSchmidtOrthOp(3, m["nmus"], 8, md["coeffs"])[0]
+    assert oc.shape == md["coeffs"].shape and close(oc.cpu().numpy(), g["orth_coeffs"], 1e-13)
+    oc32 = ops.CoeffsSchmidtOrthOp(3, m["nmus"], 8, md["coeffs"].float())[0]
+    assert oc32.dtype == torch.float32 and close(oc32.cpu().numpy(), g["orth_coeffs"], 1e-5)
+
+
 def test_errors(oracle):
     import torch
     from ai2pot_amd import _lib, ops

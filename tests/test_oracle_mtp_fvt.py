@@ -94,6 +94,52 @@ def test_site_energies_and_descriptors(oracle, level, nt):
         assert np.abs(fd - dc[:, i]).max() < 1e-6 * max(1.0, np.abs(fd).max())
 
 
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3)])
+def test_linear_system_and_schmidt(oracle, level, nt):
+    """Normal equations of the linear parameters and the Gram-Schmidt of the radial functions: the
+    reference's committed outputs; then what fixes them without it: column s of the components is
+    the E/F/V of the model with linear_coeffs = e_s (so the system is rebuilt from E/F/V calls),
+    the solution of the system reproduces labels generated by a linear model, and the
+    orthogonalised functions are orthonormal."""
+    with np.load(os.path.join(HERE, "golden", "mtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+    m, nb, _ = small_batch(oracle, level, nt)
+    m["q_scaler"] = np.linspace(0.7, 1.4, m["q_scaler"].size)
+    lab = labels_for(nb)
+    w = (1.0, 0.7, 0.3)
+    A, b = oracle.mtp_lin_system(m, nb, w, lab)
+    assert np.abs(A - g["lin_matrix"]).max() <= 1e-12 * np.abs(g["lin_matrix"]).max()
+    assert np.abs(b - g["lin_vector"]).max() <= 1e-12 * np.abs(g["lin_vector"]).max()
+    assert np.array_equal(A, A.T)
+    K, nmus = m["chebyshev_size"], m["nmus"]
+    oc = oracle.mtp_schmidt_orth(m["coeffs"], nt, nmus, K)
+    assert np.array_equal(oc, g["orth_coeffs"])
+    vecs = oc.reshape(nt * nt, nmus, K).transpose(1, 0, 2).reshape(nmus, -1)
+    gram = vecs @ vecs.T
+    assert np.abs(gram - np.diag(np.diag(gram))).max() < 1e-12
+    assert np.abs(np.diag(gram) - 1).max() < 1e-6           # the reference adds 1e-10 to every squared norm
+    if level == 16:
+        return
+    S = m["q_scaler"].size
+    n = S + nt
+    B, P = nb["bilist"].shape
+    Ec, Fc, Vc = np.zeros((B, n)), np.zeros((B, P, 3, n)), np.zeros((B, 9, n))
+    for s_ in range(S):
+        one = dict(m, linear_coeffs=np.eye(S)[s_], type_bias=np.zeros(nt))
+        Ec[:, s_], Fc[..., s_], Vc[..., s_] = oracle.mtp_efv(one, nb)
+    ti = np.take_along_axis(nb["btypes"], nb["bilist"], 1)
+    for t_ in range(nt):
+        Ec[:, S + t_] = (ti == t_).sum(1)
+    F2, V2 = Fc.reshape(-1, n), Vc.reshape(-1, n)
+    A2 = w[0] * Ec.T @ Ec + w[1] * F2.T @ F2 + w[2] * V2.T @ V2
+    assert np.abs(A2 - A).max() < 1e-12 * np.abs(A).max()
+    # labels of a linear model are reproduced by the solution of its own normal equations
+    e, f, v = oracle.mtp_efv(m, nb)
+    A3, b3 = oracle.mtp_lin_system(m, nb, w, dict(energy=e, force=f, virial=v))
+    x_true = np.concatenate([m["linear_coeffs"], m["type_bias"]])
+    assert np.abs(A3 @ x_true - b3).max() < 1e-10 * np.abs(b3).max()
+
+
 def test_energy_force_finite_difference_and_linearity(oracle):
     lat, pos = synth.random_packed(30, [8.0, 8.5, 9.0], 2.0, 31)
     ty = synth.rng_randint(32, 30, 2)
