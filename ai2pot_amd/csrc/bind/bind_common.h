@@ -93,7 +93,41 @@ inline void check_device_status(const at::Tensor& t)
 
 inline void require_no_zbl(double zbl_rmax)
 {
-    TORCH_CHECK(zbl_rmax == 0.0, "the ZBL correction (zbl_rmax > 0) is not implemented in this build");
+    TORCH_CHECK(zbl_rmax == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
+                                 "operators only; this operator needs zbl_rmax == 0");
+}
+
+// Adds the ZBL pair repulsion onto a model's E/F/V when zbl_rmax > 0, as the reference's operators
+// do on the device (correction/gpu/include/zbl.cuh:422-620); v may be undefined.
+inline void apply_zbl(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, const at::Tensor& dks,
+                      const at::Tensor& type_map, const at::Tensor& binum, const at::Tensor& bilist,
+                      const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                      const at::Tensor& btypes, int64_t nghost, at::Tensor e, at::Tensor f, at::Tensor v)
+{
+    if (zbl_rmax == 0.0) return;
+    const int ntypes = (int)type_map.numel();
+    check_device_float(brcs, cks, "zbl_cks");
+    check_device_float(brcs, dks, "zbl_dks");
+    TORCH_CHECK(cks.numel() == (int64_t)ntypes * ntypes * 4 && dks.numel() == (int64_t)ntypes * ntypes * 4,
+                "zbl_cks and zbl_dks must have ntypes * ntypes * 4 elements");
+    at::Tensor tm = type_map.to(brcs.device(), at::kInt).contiguous();
+    DeviceGuard guard(brcs);
+    const int B = (int)brcs.size(0), P = (int)brcs.size(1), U = (int)brcs.size(2);
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble) {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+        rc = a2p_zbl_correct_f64(zbl_rmax, zbl_rmin, p(cks), p(dks), ntypes, tm.data_ptr<int>(), B, P, U, (int)nghost,
+                                 binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                 bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), st);
+    } else {
+        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+        rc = a2p_zbl_correct_f32(zbl_rmax, zbl_rmin, p(cks), p(dks), ntypes, tm.data_ptr<int>(), B, P, U, (int)nghost,
+                                 binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                 bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), st);
+    }
+    check_rc(rc);
+    check_device_status(brcs);
 }
 
 }  // namespace a2p_bind

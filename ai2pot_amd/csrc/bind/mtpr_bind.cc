@@ -43,9 +43,9 @@ variable_list mtp_efv(bool want_virial, int64_t K, double scaling, const at::Ten
                       const at::Tensor& times, const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum,
                       const at::Tensor& bilist, const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
                       const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost,
-                      double rmax, double rmin, const at::Tensor& q_scaler, double zbl_rmax)
+                      double rmax, double rmin, const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin,
+                      const at::Tensor& zbl_cks, const at::Tensor& zbl_dks)
 {
-    require_no_zbl(zbl_rmax);
     MtpCtx c = check_mtp(K, coeffs, lin, bias, n_moms, basic, times, mapping, nmus, binum, bilist, bnumneigh,
                          bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
     a2p_bind::DeviceGuard guard(brcs);
@@ -70,6 +70,8 @@ variable_list mtp_efv(bool want_virial, int64_t K, double scaling, const at::Ten
                              v.defined() ? v.data_ptr<float>() : nullptr, st);
     check_rc(rc);
     check_device_status(brcs);
+    apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+              e, f, v);
     if (want_virial) return {e, f, v};
     return {e, f};
 }
@@ -347,8 +349,8 @@ TORCH_LIBRARY(mtpr, m)
 {
     m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
     m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
-    m.def("linearMtpToEFVOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(true, MTP_EFV_PASS, zbl_rmax); });
-    m.def("linearMtpToEFOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(false, MTP_EFV_PASS, zbl_rmax); });
+    m.def("linearMtpToEFVOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(true, MTP_EFV_PASS, zbl_rmax, zbl_rmin, zbl_cks, zbl_dks); });
+    m.def("linearMtpToEFOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(false, MTP_EFV_PASS, zbl_rmax, zbl_rmin, zbl_cks, zbl_dks); });
     m.def("linearMtpToLossOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
              const at::Tensor& v_dft, MTP_EFV_ARGS) -> variable_list {

@@ -177,9 +177,11 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost,
              double rr, double ra, const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin,
              const at::Tensor& zbl_cks, const at::Tensor& zbl_dks) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return nep_run(false, false, K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist, bnumneigh,
-                             bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
+              variable_list out = nep_run(false, false, K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist,
+                                          bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
+              apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                        btypes, nghost, out[0], out[1], at::Tensor());
+              return out;
           });
     m.def("nepToEFVOp",
           [](int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const at::Tensor& coeffs, const at::Tensor& w0,
@@ -188,9 +190,11 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& brcs, const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost,
              double rr, double ra, const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin,
              const at::Tensor& zbl_cks, const at::Tensor& zbl_dks) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return nep_run(true, false, K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist, bnumneigh,
-                             bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
+              variable_list out = nep_run(true, false, K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist,
+                                          bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
+              apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                        btypes, nghost, out[0], out[1], out[2]);
+              return out;
           });
     m.def("nepToLossOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,

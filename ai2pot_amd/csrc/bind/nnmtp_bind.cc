@@ -285,12 +285,16 @@ TORCH_LIBRARY(nnmtp, m)
     m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
     m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
     m.def("nnMtpToEFVOp", [](NNMTP_ARGS) -> variable_list {
-        require_no_zbl(zbl_rmax);
-        return nnmtp_run(true, true, false, NNMTP_PASS);
+        variable_list out = nnmtp_run(true, true, false, NNMTP_PASS);
+        apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                  nghost, out[0], out[1], out[2]);
+        return out;
     });
     m.def("nnMtpToEFOp", [](NNMTP_ARGS) -> variable_list {
-        require_no_zbl(zbl_rmax);
-        return nnmtp_run(true, false, false, NNMTP_PASS);
+        variable_list out = nnmtp_run(true, false, false, NNMTP_PASS);
+        apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                  nghost, out[0], out[1], at::Tensor());
+        return out;
     });
     m.def("nnMtpToEsitesOp", [](NNMTP_ARGS) -> variable_list {
         require_no_zbl(zbl_rmax);

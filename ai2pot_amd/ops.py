@@ -122,7 +122,33 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
 
 
 def _no_zbl(zbl_rmax):
-    _req(float(zbl_rmax) == 0.0, "the ZBL correction (zbl_rmax > 0) is not implemented in this build")
+    _req(float(zbl_rmax) == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
+                                 "operators only; this operator needs zbl_rmax == 0")
+
+
+def _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             nghost, etot, force, virial, validate):
+    """Adds the ZBL pair repulsion onto a model's E/F/V when zbl_rmax > 0, as the reference's
+    operators do on the device (correction/gpu/include/zbl.cuh:422-620; e.g. nepOp.cc:1086-1110)."""
+    if float(zbl_rmax) == 0.0:
+        return
+    dtype, device = brcs.dtype, brcs.device
+    ntypes = int(type_map.numel())
+    for name, t in (("zbl_cks", zbl_cks), ("zbl_dks", zbl_dks)):
+        _check_float(name, t, dtype, device)
+        _req(t.numel() == ntypes * ntypes * 4, "%s must have ntypes*ntypes*4 = %d elements" % (name, ntypes * ntypes * 4))
+    tm = type_map.to(device=device, dtype=torch.int32).contiguous()
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, int(nghost))
+    L = _lib.lib()
+    fn = L.a2p_zbl_correct_f32 if dtype == torch.float32 else L.a2p_zbl_correct_f64
+    with torch.cuda.device(device):
+        rc = fn(_c.c_double(zbl_rmax), _c.c_double(zbl_rmin), _ptr(zbl_cks), _ptr(zbl_dks), _c.c_int(ntypes), _ptr(tm),
+                _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(int(nghost)), _ptr(binum), _ptr(bilist),
+                _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(etot), _ptr(force), _ptr(virial),
+                _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
 
 
 def nepToEFVOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w0, b0, w1, type_bias,
@@ -130,10 +156,11 @@ def nepToEFVOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w
                rmax_angular, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None,
                validate=True):
     """[E[B], F[B, P+nghost, 3], V[B, 9]]; nep_bind.cc:81-135, nepOp.cc:947-1284."""
-    _no_zbl(zbl_rmax)
     e, f, v, _ = _nep_call(True, False, chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs,
                            w0, b0, w1, type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
                            type_map, nghost, rmax_radial, rmax_angular, q_scaler, validate)
+    _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             nghost, e, f, v, validate)
     return [e, f, v]
 
 
@@ -142,10 +169,11 @@ def nepToEFOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w0
               rmax_angular, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None,
               validate=True):
     """[E[B], F[B, P+nghost, 3]]; nep_bind.cc:26-79."""
-    _no_zbl(zbl_rmax)
     e, f, _, _ = _nep_call(False, False, chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs,
                            w0, b0, w1, type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
                            type_map, nghost, rmax_radial, rmax_angular, q_scaler, validate)
+    _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             nghost, e, f, None, validate)
     return [e, f]
 
 
@@ -368,8 +396,7 @@ def _mtp_common(coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_ind
 
 def _mtp_efv(want_virial, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh,
-             bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax, validate):
-    _no_zbl(zbl_rmax)
+             bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl, validate):
     dtype, device, B, P, U, nghost, ntypes, plan, _ = _mtp_common(
         coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
         alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
@@ -388,6 +415,8 @@ def _mtp_efv(want_virial, chebyshev_size, scaling, coeffs, linear_coeffs, type_b
         _lib.check(rc)
         if validate:
             _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    _zbl_add(zbl[0], zbl[1], zbl[2], zbl[3], type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+             etot, force, virial, validate)
     return etot, force, virial
 
 
@@ -398,8 +427,8 @@ def linearMtpToEFVOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, 
     """[E[B], F[B, P+nghost, 3], V[B, 9]]; mtpr_bind.cc:333-394, linearMtpOp.cc:2834-3180."""
     e, f, v = _mtp_efv(True, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
                        alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
-                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax,
-                       validate)
+                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
+                       (zbl_rmax, zbl_rmin, zbl_cks, zbl_dks), validate)
     return [e, f, v]
 
 
@@ -410,8 +439,8 @@ def linearMtpToEFOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, a
     """[E[B], F[B, P+nghost, 3]]; mtpr_bind.cc:396-457."""
     e, f, _ = _mtp_efv(False, chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, alpha_moments_count,
                        alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
-                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, zbl_rmax,
-                       validate)
+                       bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
+                       (zbl_rmax, zbl_rmin, zbl_cks, zbl_dks), validate)
     return [e, f]
 
 
@@ -759,11 +788,12 @@ def nnMtpToEFVOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
                  btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
                  zbl_cks=None, zbl_dks=None, validate=True):
     """[E[B], F[B, P+nghost, 3], V[B, 9]]; nnmtp_bind.cc:258-322, nnMtpOp.cc:2785-3010."""
-    _no_zbl(zbl_rmax)
     e, f, v, _ = _nnmtp_call("efv", chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
                              bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
                              q_scaler, validate)
+    _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             nghost, e, f, v, validate)
     return [e, f, v]
 
 
@@ -772,11 +802,12 @@ def nnMtpToEFOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count, 
                 btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
                 zbl_cks=None, zbl_dks=None, validate=True):
     """[E[B], F[B, P+nghost, 3]]; nnmtp_bind.cc:193-256."""
-    _no_zbl(zbl_rmax)
     e, f, _, _ = _nnmtp_call("ef", chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_count,
                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist,
                              bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter,
                              q_scaler, validate)
+    _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             nghost, e, f, None, validate)
     return [e, f]
 
 

@@ -206,6 +206,26 @@ int a2p_mtp_esites_bwd_f32(void* plan, int chebyshev_size, double scaling, const
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * ZBL short-range correction -- the part of every E/F/V operator that its zbl_rmax > 0 argument
+ * switches on (source/descriptor/correction/include/zbl.h:262-395 pair formulas;
+ *  correction/gpu/include/zbl.cuh:422-620 composition per centre atom;
+ *  e.g. src/nepOp.cc:1086-1110, src/linearMtpOp.cc:2975-3000 call sites).
+ * ADDS onto etot[B], force[B, P+nghost, 3] and virial[B, 9] (any may be NULL), which normally hold the
+ * model's result: 0.5 E_pair per ordered pair to the energy, dE_pair/dr * r_vec / r to the force of
+ * the centre atom only (a full list supplies the other half; ghosts receive nothing), and
+ * -0.5 r_a dE_pair/dr r_b / r to the virial.  zbl_cks / zbl_dks: [ntypes, ntypes, 4] (device);
+ * type_map: atomic numbers [ntypes] (device int32).
+ * ------------------------------------------------------------------------------------------ */
+int a2p_zbl_correct_f64(double zbl_rmax, double zbl_rmin, const double* zbl_cks, const double* zbl_dks, int ntypes,
+                        const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                        const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                        const int* btypes, double* etot, double* force, double* virial, void* stream);
+int a2p_zbl_correct_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, const float* zbl_dks, int ntypes,
+                        const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                        const int* bilist, const int* bnumneigh, const int* bfirstneigh, const float* brcs,
+                        const int* btypes, float* etot, float* force, float* virial, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Linear solver support of the linear MTP -- replaces the compute of torch.ops.mtpr.LinMatrixLinVectorOp
  * and torch.ops.mtpr.CoeffsSchmidtOrthOp (source/descriptor/mtpr/bind/mtpr_bind.cc:38-131;
  *  include/linear_mtp_gram_and_cross.h:125-374 components, :377-443 accumulation, :446-575 launcher;

@@ -547,6 +547,35 @@ def nnmtp_esites_bwd(model, nb, gout):
 
 
 # ----------------------------------------------------------------------------------------
+# ZBL correction (fp64): adds onto copies of the given E/F/V
+# ----------------------------------------------------------------------------------------
+def _zbl(lib, name, zbl, nb, type_map, efv=None):
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    type_map = _c(type_map, np.int32)
+    cks, dks = _c(zbl["cks"], np.float64), _c(zbl["dks"], np.float64)
+    nt = type_map.size
+    assert cks.size == nt * nt * 4 and dks.size == nt * nt * 4
+    if efv is None:
+        e, f, v = np.zeros(B), np.zeros((B, P + nghost, 3)), np.zeros((B, 9))
+    else:
+        e, f, v = (np.array(x, np.float64, copy=True) for x in efv)
+    fn = getattr(lib, name)
+    fn.restype = None
+    fn(_p(e), _p(f), _p(v), _D(zbl["rmax"]), _D(zbl["rmin"]), _p(cks), _p(dks), _I(nt), _p(type_map), _I(B), _I(P),
+       _I(U), _I(nghost), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes))
+    return e, f, v
+
+
+def ref_zbl_correct(zbl, nb, type_map, efv=None):
+    """E/F/V plus the ZBL terms, pair by pair through the reference's PairZBL member functions."""
+    return _zbl(_load("_ref/libref_zbl.so"), "ref_zbl_correct_f64", zbl, nb, type_map, efv)
+
+
+def zbl_correct(zbl, nb, type_map, efv=None):
+    return _zbl(oracle_lib(), "orc_zbl_correct_f64", zbl, nb, type_map, efv)
+
+
+# ----------------------------------------------------------------------------------------
 # fvt (single structure, fp64)
 # ----------------------------------------------------------------------------------------
 def _fvt_force(lib, prefix, ilist, numneigh, firstneigh, nghost, dei_drij, grad_in=None):

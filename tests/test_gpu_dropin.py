@@ -77,6 +77,12 @@ def test_nep_ops_and_torchscript(oracle, dropin):
         assert torch.equal(a, b)
     ef = torch.ops.nep.nepToEFOp(*args)
     assert len(ef) == 2 and torch.equal(ef[0], want[0]) and torch.equal(ef[1], want[1])
+    # with the ZBL correction switched on the registered operator and the Python mirror agree
+    ck = torch.tensor([0.18175, 0.50986, 0.28022, 0.02817], device="cuda:0").repeat(9)
+    dk = torch.tensor([3.1998, 0.94229, 0.4029, 0.20162], device="cuda:0").repeat(9)
+    zgot = torch.ops.nep.nepToEFVOp(*(args[:20] + (2.4, 1.2, ck, dk)))
+    zwant = ops.nepToEFVOp(*(args[:20] + (2.4, 1.2, ck, dk)))
+    assert all(torch.equal(a, b) for a, b in zip(zgot, zwant)) and not torch.equal(zgot[0], want[0])
     d = torch.ops.nep.nepToDescriptorsOp(*(args[:5] + args[9:19]))
     assert d[0].shape == (1, 120, 22)
     assert torch.equal(d[0], ops.nepToDescriptorsOp(*(args[:5] + args[9:19]))[0])

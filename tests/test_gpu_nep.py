@@ -218,7 +218,7 @@ def test_errors(oracle):
         call(bfirstneigh=bad)
     with pytest.raises(_lib.A2PError):                      # type index out of range
         call(btypes=d["btypes"] + 7)
-    with pytest.raises(RuntimeError):                       # ZBL not built
+    with pytest.raises(RuntimeError):                       # ZBL switched on without its parameter tensors
         ops.nepToEFVOp(8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"],
                        d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"],
                        md["type_map"], 0, 7.0, 4.0, md["q_scaler"], 1.0, 0.5, None, None)

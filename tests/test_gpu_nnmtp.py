@@ -106,7 +106,7 @@ def test_errors(oracle):
     args = list(op_args(m, md, to_device(nb, torch.float64)))
     with pytest.raises(RuntimeError):                       # w0 of the wrong size
         ops.nnMtpToEFVOp(*(args[:2] + [md["w0"][:-1].contiguous()] + args[3:]))
-    with pytest.raises(RuntimeError):                       # ZBL is not part of this build
+    with pytest.raises(RuntimeError):                       # ZBL switched on without its parameter tensors
         ops.nnMtpToEFVOp(*args, 2.0, 1.0, None, None)
 
 
