@@ -6,6 +6,9 @@
 // Pinned by: the reference's own PairZBL member functions compiled from zbl.h
 // (oracle/_ref/libref_zbl.so) pair by pair; finite differences of the energy for the force and the
 // virial; switching-function end values (tests/test_pair_zbl.cc:75-77).
+// Parity unpinned for the composition per centre atom (which atom receives the force, the halves):
+// it is read off the device source, which cannot be compiled or run here, and no output of it
+// ships with the reference; energy consistency (force = -dE/dx for a full list) is what checks it.
 #include <cmath>
 #include <cstddef>
 
