@@ -13,6 +13,18 @@
 // test fixtures; the reference unit test's known answer E = -0.938157350795572
 // (tests/test_linearMtp.cc, efv_force_accuracy set-up); finite differences of E; switch
 // function end values (tests/test_basis.cc:106-111); linearity of E in linear_coeffs.
+//
+// Also here, each with its own citations below: site energies / scalar moments and their
+// gradient (pinned by the reference's committed outputs, the sum rule and the linear read-out);
+// the normal equations of the linear parameters and the Gram-Schmidt of the radial functions
+// (reference outputs; rebuilt independently from one-hot E/F/V calls); the neural-network MTP
+// (source/descriptor/nnmtp): E/F/V and site energies (reference outputs, finite differences, the
+// linear limit of a small network), its training-loss gradient and site-energy gradient by
+// forward-mode AD.  For the last two the reference's hand-derived backward is NOT reproduced
+// by this file: it omits terms (loss: d/dcoeffs, d/dw0 of the force and virial parts) or
+// mis-assigns rows (site energies: w0 / w1 for several species); the AD results are pinned by
+// finite differences and by the reference where its formulas are complete (w1, type_bias,
+// energy-only loss, one species).
 #include <algorithm>
 #include <cmath>
 #include <cstring>
