@@ -56,15 +56,21 @@ class NepCalculator:
         self.virial = torch.empty(9, dtype=dtype, device=dev)
         L = _lib.lib()
         f32 = dtype == torch.float32
-        self._nbl = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
+        self._nbl_build = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
+        self._nbl_update = L.a2p_nblist_update_f32 if f32 else L.a2p_nblist_update_f64
+        self._have_list = False
         self._efv = L.a2p_nep_efv_f32 if f32 else L.a2p_nep_efv_f64
 
     def rebuild(self, coords, stream):
-        rc = self._nbl(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
-                       _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
-                       self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self.sort else 0),
-                       _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
-                       _vp(self.types_out), None, stream)
+        # after the first build the list buffers hold a valid list: later builds write each row
+        # only as far as its old or new length reaches
+        fn = self._nbl_update if self._have_list else self._nbl_build
+        rc = fn(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
+                _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
+                self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self.sort else 0),
+                _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
+                _vp(self.types_out), None, stream)
+        self._have_list = rc == 0
         _lib.check(rc)
 
     def evaluate(self, stream):

@@ -304,7 +304,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
              int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
              T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
-             int* __restrict__ status)
+             int* __restrict__ status, int update)
 {
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
@@ -383,6 +383,9 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
 
     int cnt = 0;
     const size_t rowi = (size_t)p * umax;
+    // update of an earlier result held in the same buffers: beyond the row's old length the
+    // padding is already in place
+    const int old_len = update ? min(max(numneigh[p], 0), umax) : umax;
     // NBL_UNROLL chunks of 64 candidates per trip: all their loads are issued before the first is
     // used, so a typical row (100 - 250 candidates) costs one memory round trip
     for (int c0 = 0; c0 < total; c0 += 64 * NBL_UNROLL) {
@@ -449,17 +452,19 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         __builtin_amdgcn_wave_barrier();
         const uint4* s1 = reinterpret_cast<const uint4*>(rb_first);
         uint4* d1 = reinterpret_cast<uint4*>(firstneigh + rowi);
-        for (int i = lane; i < umax / 4; i += 64) d1[i] = s1[i];
+        const int live = (max(min(cnt, umax), old_len) + 3) & ~3;     // umax is a multiple of 4
+        for (int i = lane; i < live / 4; i += 64) d1[i] = s1[i];
         const uint4* s2 = reinterpret_cast<const uint4*>(rb_rcs);
         uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
-        const int nv = (int)((size_t)umax * 3 * sizeof(T) / 16);
+        const int nv = (int)((size_t)live * 3 * sizeof(T) / 16);
         for (int i = lane; i < nv; i += 64) d2[i] = s2[i];
         return;
     }
     // padding: -1 / 0 (neighborList.h:557, 563)
     const int first_pad = min(cnt, umax);
-    pad_fill(firstneigh + rowi, first_pad, umax, -1, lane);
-    pad_fill(rcs + rowi * 3, first_pad * 3, umax * 3, (T)0, lane);
+    const int last_pad = max(first_pad, old_len);
+    pad_fill(firstneigh + rowi, first_pad, last_pad, -1, lane);
+    pad_fill(rcs + rowi * 3, first_pad * 3, last_pad * 3, (T)0, lane);
 }
 
 // ---- 7. distance sort, emulating libstdc++ std::sort(indices, cmp = d[a] < d[b]) --------------
@@ -666,7 +671,7 @@ T host_plane_distance(const T* v, const T* n)        // structure.h:818-842, vec
 template <typename T>
 int nblist_build(const T* lattice, const int* types, const T* coords, int N, double rcut_in, int umax,
                  int is_cart, const int* pbc, int sort, int* ilist, int* numneigh, int* firstneigh,
-                 T* rcs, int* types_out, int* max_nn_host, hipStream_t stream)
+                 T* rcs, int* types_out, int* max_nn_host, hipStream_t stream, int update = 0)
 {
     A2P_REQUIRE(lattice && pbc, A2P_ERR_INVALID, "nblist: lattice and pbc must be host pointers");
     A2P_REQUIRE(N > 0, A2P_ERR_INVALID, "nblist: the structure has no atoms");   // binLinkedList.h:659
@@ -817,15 +822,15 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (sort)
         hipLaunchKernelGGL((lists_kernel<T, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
-                           status);
+                           status, 0);
     else if (rowbuf)
         hipLaunchKernelGGL((lists_kernel<T, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream, g,
                            x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status);
+                           status, update);
     else
         hipLaunchKernelGGL((lists_kernel<T, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status);
+                           status, update);
     prof_end(stream);
     if (sort) {
         prof_begin("nbl_sort_rows", stream);
@@ -883,5 +888,25 @@ int a2p_nblist_build_f64(const double* lattice, const int* types, const double* 
     return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
                                      numneigh, firstneigh, rcs, types_out, max_numneigh,
                                      (hipStream_t)stream);
+}
+
+int a2p_nblist_update_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                          double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                          int* numneigh, int* firstneigh, float* rcs, int* types_out, int* max_numneigh,
+                          void* stream)
+{
+    return a2p::nblist_build<float>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
+                                    numneigh, firstneigh, rcs, types_out, max_numneigh, (hipStream_t)stream,
+                                    1);
+}
+
+int a2p_nblist_update_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                          double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                          int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
+                          void* stream)
+{
+    return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
+                                     numneigh, firstneigh, rcs, types_out, max_numneigh,
+                                     (hipStream_t)stream, 1);
 }
 }

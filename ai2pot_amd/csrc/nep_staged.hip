@@ -17,9 +17,12 @@
 //     coefficients once per atom (pass 1), and the coefficients are contracted with dE/dq once
 //     per atom before the radial derivative loop (pass 2);
 //   * pair derivatives are stored straight into the reduction segments.
-// Pass 1: rounds (radial sums, lists), angular moments over the back list; then descriptors,
-// hidden layer, dE/dq, dE/dS.  Pass 2: pair derivatives of the radial-only pairs (front list)
-// and of the pairs inside the angular cutoff, both parts together (back list); own force, virial.
+// Two kernels.  nep_stage_kernel does the rounds (radial sums, lists, places in the reduction
+// segments): it needs few registers, so many waves per SIMD hide the latency of its gathers and
+// atomics.  nep_staged_kernel holds the angular moments in registers (two waves per SIMD) and only
+// streams the dense lists: angular moments over the back list; descriptors, hidden layer, dE/dq,
+// dE/dS; then the pair derivatives of the radial-only pairs (front list) and of the pairs inside
+// the angular cutoff, both parts together (back list); own force, virial.
 //
 // Formulas: source/descriptor/nep/include/{nepBasis.h:57-196; nep.h:320-529}.
 #include "a2p_common.h"
@@ -29,9 +32,10 @@ namespace a2p {
 using namespace nepdev;
 namespace {
 
-constexpr int FB = 256;        // atoms (threads) per workgroup
-constexpr int FCH = 16;        // neighbour slots staged per round
-constexpr int FLS = FB + 8;    // padded row length of the staging arrays
+constexpr int FB = 256;        // atoms (threads) per workgroup of the model kernel; geometry of the lists
+constexpr int SB = 256;        // atoms (threads) per workgroup of the staging kernel (divides FB)
+constexpr int SCH = 8;         // neighbour slots staged per round
+constexpr int SLS = SB + 8;    // padded row length of the staging arrays
 constexpr int FDP = 24;        // padded descriptor count (22)
 constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
 
@@ -47,21 +51,41 @@ __device__ __forceinline__ void lds_load4(const double* p, double (&o)[4])
     o[0] = v0.x; o[1] = v0.y; o[2] = v1.x; o[3] = v1.y;
 }
 
+// LDS of the staging kernel: staging arrays [SCH][SLS] and the rows' lengths
 template <typename T>
-struct StagedLds {
-    T* coef;
-    T *x, *y, *z;            // staging arrays [FCH][FLS] ...
-    int* p;                  // ... place of the pair in its target's reduction segment
-    unsigned char* w;        // ... species of the neighbour
-    T *w0, *b0, *w1, *qs;    // network tables (between the passes) and
-    T* acc;                  // contracted radial coefficients (pass 2) share the staging memory
+struct StageLds {
+    T *x, *y, *z;
+    int* p;                  // place of the pair in its target's reduction segment
+    unsigned char* w;        // species of the neighbour
     int *nn, *red;
 };
 
 __host__ __device__ __forceinline__ size_t lds_round16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
 
-// LDS layout; returns the total size.  The staging arrays are used in pass 1 only, the network
-// tables between the passes, the contracted coefficients in pass 2: the three share one region.
+template <typename T>
+__host__ __device__ __forceinline__ size_t stage_lds_layout(unsigned char* base, StageLds<T>& L)
+{
+    size_t off = 0;
+    L.x = (T*)(base + off);    off += lds_round16((size_t)SCH * SLS * sizeof(T));
+    L.y = (T*)(base + off);    off += lds_round16((size_t)SCH * SLS * sizeof(T));
+    L.z = (T*)(base + off);    off += lds_round16((size_t)SCH * SLS * sizeof(T));
+    L.p = (int*)(base + off);  off += lds_round16((size_t)SCH * SLS * sizeof(int));
+    L.w = base + off;          off += lds_round16((size_t)SCH * SLS);
+    L.nn = (int*)(base + off); off += lds_round16((size_t)SB * sizeof(int));
+    L.red = (int*)(base + off); off += lds_round16((size_t)(SB / 64) * sizeof(int));
+    return off;
+}
+
+// LDS of the model kernel: coefficients; network tables (before pass 2) and the contracted radial
+// coefficients (pass 2) share one region; partial sums
+template <typename T>
+struct StagedLds {
+    T* coef;
+    T *w0, *b0, *w1, *qs;
+    T* acc;
+    double* red;
+};
+
 template <typename T>
 __host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
                                                              StagedLds<T>& L)
@@ -69,23 +93,15 @@ __host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, 
     size_t off = 0;
     L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * NB * KC * sizeof(T));
     const size_t u0 = off;
-    L.x = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
-    L.y = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
-    L.z = (T*)(base + off);    off += lds_round16((size_t)FCH * FLS * sizeof(T));
-    L.p = (int*)(base + off);  off += lds_round16((size_t)FCH * FLS * sizeof(int));
-    L.w = base + off;          off += lds_round16((size_t)FCH * FLS);
-    size_t u1 = off;
-    off = u0;
     L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * KC * FB * sizeof(T));
-    u1 = off > u1 ? off : u1;
+    const size_t u1 = off;
     off = u0;
     L.w0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * FDP * sizeof(T));
     L.b0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
     L.w1 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
     L.qs = (T*)(base + off);   off += lds_round16((size_t)FDP * sizeof(T));
     off = off > u1 ? off : u1;
-    L.nn = (int*)(base + off); off += lds_round16((size_t)FB * sizeof(int));
-    L.red = (int*)(base + off); off += lds_round16((size_t)(FB / 64) * 10 * sizeof(double));
+    L.red = (double*)(base + off); off += lds_round16((size_t)(FB / 64) * 10 * sizeof(double));
     return off;
 }
 
@@ -95,18 +111,18 @@ struct SegArgs {
     int spare;     // entry that takes what overflows a segment
 };
 
-// Stage slots [c0, c0 + FCH) of the workgroup's rows: thread e handles row e / FCH, slot e % FCH,
-// so FCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
+// Stage slots [c0, c0 + SCH) of the workgroup's rows: thread e handles row e / SCH, slot e % SCH,
+// so SCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
 // row's end (or with an index out of range) are stored far outside every cutoff.
 template <typename T>
-__device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StagedLds<T>& L,
+__device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StageLds<T>& L,
                                             int tid, int c0, size_t rowbase, int b, int NF)
 {
     const int* types = a.btypes + (size_t)b * NF;
 #pragma unroll
-    for (int it = 0; it < FCH; it++) {
-        const int e = it * FB + tid;
-        const int la = e / FCH, s = e % FCH;
+    for (int it = 0; it < SCH; it++) {
+        const int e = it * SB + tid;
+        const int la = e / SCH, s = e % SCH;
         const int slot = c0 + s;
         T x = (T)1.0e18, y = (T)0, z = (T)0;
         int w = 0, pos = 0;
@@ -128,21 +144,21 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
                 if ((unsigned)w >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); w = 0; }
             }
         }
-        L.x[s * FLS + la] = x; L.y[s * FLS + la] = y; L.z[s * FLS + la] = z;
-        L.w[s * FLS + la] = (unsigned char)w; L.p[s * FLS + la] = pos;
+        L.x[s * SLS + la] = x; L.y[s * SLS + la] = y; L.z[s * SLS + la] = z;
+        L.w[s * SLS + la] = (unsigned char)w; L.p[s * SLS + la] = pos;
     }
 }
 
 // Bit masks of a thread's staged entries: bit s of mA set when entry s lies inside the angular
 // cutoff, of mR inside the radial cutoff, of mV when the entry is a pair of the list at all.
 template <typename T>
-__device__ __forceinline__ void staged_classify(const StagedLds<T>& L, int tid, T rr, T ra, unsigned& mA,
+__device__ __forceinline__ void staged_classify(const StageLds<T>& L, int tid, T rr, T ra, unsigned& mA,
                                                 unsigned& mR, unsigned& mV)
 {
     mA = 0; mR = 0; mV = 0;
 #pragma unroll
-    for (int s = 0; s < FCH; s++) {
-        const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
+    for (int s = 0; s < SCH; s++) {
+        const T x = L.x[s * SLS + tid], y = L.y[s * SLS + tid], z = L.z[s * SLS + tid];
         const T r = sqrt_t(x * x + y * y + z * z);
         if (r <= ra && r <= rr) mA |= 1u << s;     // nepBasis.h:106, 135: beyond the radial cutoff a neighbour is skipped
         if (r <= rr) mR |= 1u << s;
@@ -172,10 +188,130 @@ __device__ __forceinline__ void ang_load(const double* p, double& x, double& y, 
     x = v0.x; y = v0.y; z = v1.x; w = (int)__double_as_longlong(v1.y);
 }
 
+// Rows' header shared by both kernels: centre, its species and the row length, with the checks
+template <typename T>
+__device__ __forceinline__ void row_header(const NepArgs<T>& a, bool active, size_t row, int b, int NF,
+                                           int& center, int& ti, int& nn)
+{
+    center = 0; ti = 0; nn = 0;
+    if (active) {
+        center = a.bilist[row];
+        nn = a.bnumneigh[row];
+        if (nn > a.U) { atomicOr(a.status, ST_NEIGH_OVERFLOW); nn = a.U; }
+        if ((unsigned)center >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); center = 0; nn = 0; }
+        ti = a.btypes[(size_t)b * NF + center];
+        if ((unsigned)ti >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); ti = 0; nn = 0; }
+    }
+}
+
+// Staging kernel.  Per row: radial functions summed per neighbour species (radial[k][row], k <
+// NTC*KC), list lengths (counts[0][row] radial-only, counts[1][row] inside the angular cutoff),
+// the two compact lists, and zeros in the reduction segments for pairs beyond both cutoffs.
+template <typename T, int NTC>
+__global__ void __launch_bounds__(SB, (sizeof(T) == 4 ? 4 : 2))
+nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T* __restrict__ ang_xyz,
+                 int* __restrict__ ang_pos, T* __restrict__ radial, int* __restrict__ counts)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int tid = threadIdx.x;
+    const int b = blockIdx.y;
+    const int r0 = blockIdx.x * SB;             // first row of the workgroup within the batch
+    const int ii = r0 + tid;
+    const int NF = a.P + a.nghost;
+    StageLds<T> L;
+    stage_lds_layout<T>(smem_raw, L);
+
+    const bool active = ii < a.binum[b];
+    const size_t rowbase = (size_t)b * a.P + r0;
+    int center, ti, nn;
+    row_header<T>(a, active, rowbase + tid, b, NF, center, ti, nn);
+    L.nn[tid] = nn;
+    {
+        const int m = wave_max(nn);
+        if ((tid & 63) == 0) L.red[tid >> 6] = m;
+    }
+    __syncthreads();
+    int maxnn = 0;
+#pragma unroll
+    for (int w = 0; w < SB / 64; w++) maxnn = max(maxnn, L.red[w]);
+
+    const T rr = a.rr, ra = a.ra;
+    const T rr_inv = (T)1 / rr;
+    // compact lists of this row: entry k at [k * FB]; radial-only entries occupy k = 0 ..
+    // n_rad-1, entries inside the angular cutoff k = U-1 .. U-n_ang (n_rad + n_ang <= nn <= U)
+    const int mblk = ii / FB, mtid = ii - mblk * FB;
+    const size_t list0 = (size_t)(b * a.nblocks + mblk) * a.U * FB + mtid;
+    T* const lxyz = ang_xyz + list0 * 4;
+    int* const lpos = ang_pos + list0;
+    const int back = a.U - 1;
+    const bool want_pairs = a.force != nullptr || a.want_virial;
+
+    T F[NTC][KC];                 // radial functions summed per neighbour species
+#pragma unroll
+    for (int t = 0; t < NTC; t++)
+#pragma unroll
+        for (int k = 0; k < KC; k++) F[t][k] = (T)0;
+    int n_ang = 0, n_rad = 0;
+    for (int c0 = 0; c0 < maxnn; c0 += SCH) {
+        __syncthreads();
+        staged_load<T>(a, seg, L, tid, c0, rowbase, b, NF);
+        __syncthreads();
+        unsigned mA, mR, mV;
+        staged_classify<T>(L, tid, rr, ra, mA, mR, mV);
+        unsigned bits = mR;
+        while (bits) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            const T x = L.x[s * SLS + tid], y = L.y[s * SLS + tid], z = L.z[s * SLS + tid];
+            const int tj = L.w[s * SLS + tid];
+            const T r = sqrt_t(x * x + y * y + z * z);
+            T f[KC], df[KC];
+            radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+            for (int t = 0; t < NTC; t++)
+#pragma unroll
+                for (int k = 0; k < KC; k++) F[t][k] += (tj == t) ? f[k] : (T)0;
+            if (want_pairs && !((mA >> s) & 1u)) {
+                ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, tj);
+                lpos[(size_t)n_rad * FB] = L.p[s * SLS + tid];
+                n_rad++;
+            }
+        }
+        bits = mA;
+        while (bits) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            const int k = back - n_ang;
+            ang_store(lxyz + (size_t)k * FB * 4, L.x[s * SLS + tid], L.y[s * SLS + tid], L.z[s * SLS + tid],
+                      L.w[s * SLS + tid]);
+            lpos[(size_t)k * FB] = L.p[s * SLS + tid];
+            n_ang++;
+        }
+        // pairs of the list beyond both cutoffs still own a place in their segment
+        bits = mV & ~mR & ~mA;
+        while (bits && seg_g) {
+            const int s = __ffs(bits) - 1;
+            bits &= bits - 1;
+            T* dst = seg_g + (size_t)L.p[s * SLS + tid] * 3;
+            dst[0] = (T)0; dst[1] = (T)0; dst[2] = (T)0;
+        }
+    }
+    if (ii < a.P) {
+        const size_t o = (size_t)(b * a.nblocks + mblk) * FB + mtid;
+        const size_t plane = (size_t)a.B * a.nblocks * FB;
+#pragma unroll
+        for (int t = 0; t < NTC; t++)
+#pragma unroll
+            for (int k = 0; k < KC; k++) radial[(size_t)(t * KC + k) * plane + o] = F[t][k];
+        counts[o] = n_rad;
+        counts[plane + o] = n_ang;
+    }
+}
+
 template <typename T, int NTC>
 __global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
-nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T* __restrict__ ang_xyz,
-                  int* __restrict__ ang_pos)
+nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict__ ang_xyz,
+                  const int* __restrict__ ang_pos, const T* __restrict__ radial, const int* __restrict__ counts)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tid = threadIdx.x;
@@ -187,107 +323,43 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
     staged_lds_layout<T>(nt, H, NTC, smem_raw, L);
 
     for (int i = tid; i < nt * nt * NB * KC; i += FB) L.coef[i] = a.coeffs[i];
-
-    const int inum = a.binum[b];
-    const bool active = ii < inum;
-    const size_t rowbase = (size_t)b * a.P + (size_t)blockIdx.x * FB;
-    const size_t row = rowbase + tid;
-    int center = 0, ti = 0, nn = 0;
-    if (active) {
-        center = a.bilist[row];
-        nn = a.bnumneigh[row];
-        if (nn > a.U) { atomicOr(a.status, ST_NEIGH_OVERFLOW); nn = a.U; }
-        if ((unsigned)center >= (unsigned)NF) { atomicOr(a.status, ST_BAD_NEIGHBOR); center = 0; nn = 0; }
-        ti = a.btypes[(size_t)b * NF + center];
-        if ((unsigned)ti >= (unsigned)nt) { atomicOr(a.status, ST_BAD_TYPE); ti = 0; nn = 0; }
-    }
-    L.nn[tid] = nn;
-    {
-        int m = nn;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
-        if ((tid & 63) == 0) L.red[tid >> 6] = m;
-    }
-    __syncthreads();
-    int maxnn = 0;
-#pragma unroll
-    for (int w = 0; w < FB / 64; w++) maxnn = max(maxnn, L.red[w]);
-
-    const T rr = a.rr, ra = a.ra;
-    const T rr_inv = (T)1 / rr, ra_inv = (T)1 / ra;
-    // compact lists of this thread: entry k at [k * FB]; radial-only entries occupy k = 0 ..
-    // n_rad-1, entries inside the angular cutoff k = U-1 .. U-n_ang (n_rad + n_ang <= nn <= U)
-    const size_t list0 = (size_t)(b * a.nblocks + blockIdx.x) * a.U * FB + tid;
-    T* const lxyz = ang_xyz + list0 * 4;
-    int* const lpos = ang_pos + list0;
-    const int back = a.U - 1;
-    const bool want_pairs = a.force != nullptr || a.want_virial;
-
-    T S[NAC][NLM];
-#pragma unroll
-    for (int n = 0; n < NAC; n++)
-#pragma unroll
-        for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
-
-    // ---- pass 1 -------------------------------------------------------------------------------
-    T F[NTC][KC];                 // radial functions summed per neighbour species
-#pragma unroll
-    for (int t = 0; t < NTC; t++)
-#pragma unroll
-        for (int k = 0; k < KC; k++) F[t][k] = (T)0;
-    int n_ang = 0, n_rad = 0;
-    for (int c0 = 0; c0 < maxnn; c0 += FCH) {
-        __syncthreads();
-        staged_load<T>(a, seg, L, tid, c0, rowbase, b, NF);
-        __syncthreads();
-        unsigned mA, mR, mV;
-        staged_classify<T>(L, tid, rr, ra, mA, mR, mV);
-        unsigned bits = mR;
-        while (bits) {
-            const int s = __ffs(bits) - 1;
-            bits &= bits - 1;
-            const T x = L.x[s * FLS + tid], y = L.y[s * FLS + tid], z = L.z[s * FLS + tid];
-            const int tj = L.w[s * FLS + tid];
-            const T r = sqrt_t(x * x + y * y + z * z);
-            T f[KC], df[KC];
-            radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
-#pragma unroll
-            for (int t = 0; t < NTC; t++)
-#pragma unroll
-                for (int k = 0; k < KC; k++) F[t][k] += (tj == t) ? f[k] : (T)0;
-            if (want_pairs && !((mA >> s) & 1u)) {
-                ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, tj);
-                lpos[(size_t)n_rad * FB] = L.p[s * FLS + tid];
-                n_rad++;
-            }
-        }
-        bits = mA;
-        while (bits) {
-            const int s = __ffs(bits) - 1;
-            bits &= bits - 1;
-            const int k = back - n_ang;
-            ang_store(lxyz + (size_t)k * FB * 4, L.x[s * FLS + tid], L.y[s * FLS + tid], L.z[s * FLS + tid],
-                      L.w[s * FLS + tid]);
-            lpos[(size_t)k * FB] = L.p[s * FLS + tid];
-            n_ang++;
-        }
-        // pairs of the list beyond both cutoffs still own a place in their segment
-        bits = mV & ~mR & ~mA;
-        while (bits && seg_g) {
-            const int s = __ffs(bits) - 1;
-            bits &= bits - 1;
-            T* dst = seg_g + (size_t)L.p[s * FLS + tid] * 3;
-            dst[0] = (T)0; dst[1] = (T)0; dst[2] = (T)0;
-        }
-    }
-    // the network tables take the place of the staging arrays
-    __syncthreads();
     for (int i = tid; i < nt * H * FDP; i += FB) {
         const int r = i / FDP, j = i - r * FDP;
         L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
     }
     for (int i = tid; i < nt * H; i += FB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
     if (tid < FDP) L.qs[tid] = tid < DC ? (T)1 / a.q_scaler[tid] : (T)0;
+
+    const bool active = ii < a.binum[b];
+    const size_t row = (size_t)b * a.P + (size_t)blockIdx.x * FB + tid;
+    int center, ti, nn;
+    row_header<T>(a, active, row, b, NF, center, ti, nn);
+
+    const T rr = a.rr, ra = a.ra;
+    const T rr_inv = (T)1 / rr, ra_inv = (T)1 / ra;
+    const size_t o = (size_t)(b * a.nblocks + blockIdx.x) * FB + tid;
+    const size_t plane = (size_t)a.B * a.nblocks * FB;
+    const size_t list0 = (size_t)(b * a.nblocks + blockIdx.x) * a.U * FB + tid;
+    const T* const lxyz = ang_xyz + list0 * 4;
+    const int* const lpos = ang_pos + list0;
+    const int back = a.U - 1;
+    const bool want_pairs = a.force != nullptr || a.want_virial;
+    // rows past P were not staged
+    const bool staged_row = ii < a.P;
+    const int n_rad = staged_row ? counts[o] : 0;
+    const int n_ang = staged_row ? counts[plane + o] : 0;
+    T F[NTC][KC];
+#pragma unroll
+    for (int t = 0; t < NTC; t++)
+#pragma unroll
+        for (int k = 0; k < KC; k++) F[t][k] = staged_row ? radial[(size_t)(t * KC + k) * plane + o] : (T)0;
+
+    T S[NAC][NLM];
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
+    __syncthreads();
 
     // angular moments over the back list (the next entry is in flight while one is processed)
     T px = (T)0, py = (T)0, pz = (T)0;
@@ -318,7 +390,6 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
             for (int m = 0; m < NLM; m++) S[n][m] += g * bl[m];
         }
     }
-    __syncthreads();
 
     // ---- descriptors --------------------------------------------------------------------------
     T q[DC];
@@ -510,7 +581,7 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
 
     // ---- workgroup partial sums of energy and virial (fp64) ---------------------------------
     __syncthreads();
-    double* s_red = (double*)L.red;
+    double* s_red = L.red;
     double vals[10];
     vals[0] = active ? (double)e_site : 0.0;
 #pragma unroll
@@ -531,21 +602,36 @@ nep_staged_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, 
 template <typename T, int NTC>
 int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
 {
-    // compact lists: [workgroup][entry < U][thread] of 4 T, then the same of int
-    const size_t nent = (size_t)a.B * a.nblocks * a.U * FB;
+    // workspace: compact lists [workgroup][entry < U][thread] of 4 T, the same of int, then per
+    // row the summed radial functions [NTC*KC] and the two list lengths
+    const size_t plane = (size_t)a.B * a.nblocks * FB;
+    const size_t nent = plane * a.U;
     void* ws = nullptr;
-    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)), &ws);
+    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)) + plane * (NTC * KC * sizeof(T) + 2 * sizeof(int)),
+                    &ws);
     if (rc) return rc;
     T* ang_xyz = (T*)ws;
     int* ang_pos = (int*)((char*)ws + nent * 4 * sizeof(T));
+    T* radial = (T*)((char*)ws + nent * (4 * sizeof(T) + sizeof(int)));
+    int* counts = (int*)(radial + plane * NTC * KC);
     SegArgs seg{csr.cursor, csr.seg_cap, csr.n * csr.seg_cap};
+    StageLds<T> unused;
+    const size_t lds_stage = stage_lds_layout<T>(nullptr, unused);
+    auto stage = nep_stage_kernel<T, NTC>;
+    if (lds_stage > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)stage, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)lds_stage));
+    prof_begin("nep_stage_kernel", stream);
+    hipLaunchKernelGGL(stage, dim3(ceil_div(a.P, SB), a.B), dim3(SB), lds_stage, stream, a, seg, (T*)csr.seg_g,
+                       ang_xyz, ang_pos, radial, counts);
+    prof_end(stream);
     auto kern = nep_staged_kernel<T, NTC>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
     prof_begin("nep_staged_kernel", stream);
-    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, seg, (T*)csr.seg_g, ang_xyz,
-                       ang_pos);
+    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, (T*)csr.seg_g, (const T*)ang_xyz,
+                       (const int*)ang_pos, (const T*)radial, (const int*)counts);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -563,6 +649,7 @@ bool nep_staged_supported(const NepArgs<T>& a, size_t* lds_bytes)
     if (!(a.K == KC && a.n_r == NRC && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
     StagedLds<T> unused;
     *lds_bytes = staged_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), nullptr, unused);
+    static_assert(FB % SB == 0, "a staging workgroup must not straddle two model workgroups");
     return *lds_bytes <= 150 * 1024;
 }
 

@@ -38,6 +38,19 @@ def nep_flops_per_atom(nr_mean, na_mean, K=8, n_r=6, n_a=4, D=22, H=50):
             na_mean * (cK + 4 * K * n_a + 210 + 48 * n_a + 432 * n_a) + 144 * n_a + 4 * D * H + 15 * H)
 
 
+def nep_stage_flops_per_atom(nr_mean, K=8):
+    """Staging kernel's share of nep_flops_per_atom: per radial neighbour the distance (14), the
+    basis values (half of c(K)) and their accumulation per species (K)."""
+    return nr_mean * (14 + (14 * K + 24) // 2 + K)
+
+
+def nep_stage_bytes_per_atom(nr_mean, s, ntc=3, K=8):
+    """Staging kernel, algorithmic bytes: per pair the relative vector, the neighbour index, its
+    species, the segment counter (read and written by the atomic), and the compact-list entry with
+    its place; per atom the row header and the summed radial functions with the two list lengths."""
+    return nr_mean * ((3 * s + 4 + 4 + 8) + (4 * s + 4)) + 12 + ntc * K * s + 8
+
+
 def mtp_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar):
     """Linear-MTP E/F/V: per neighbour 8 + 8K + 30 + 4K nmus + 4 kmax + 29 n_basic, per atom
     9 n_times + 4 n_scalar."""
@@ -96,8 +109,9 @@ def timed_replay(replay, steps, warmup):
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
 MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nep_staged_kernel"): 6.584e6 * 1024,
-    ("nep_md_1048576", "nbl_lists"): 4.100e6 * 1024,
+    ("nep_md_1048576", "nep_stage_kernel"): 4.402e6 * 1024,
+    ("nep_md_1048576", "nep_staged_kernel"): 3.218e6 * 1024,
+    ("nep_md_1048576", "nbl_lists"): 1.216e6 * 1024,
 }
 
 
@@ -168,12 +182,16 @@ def run_nep_md(args, kind, size, rebuild=True):
     nn_r = float(calc.numneigh.float().mean().item())
     r = calc.rcs.norm(dim=2)
     nn_a = float(((r > 0) & (r <= model["rmax_angular"])).sum().item()) / n
-    s, U = 4, 200
+    s = 4
     work = {
         "nep_efv_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
-        "nep_staged_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
+        "nep_stage_kernel": ("hbm", nep_stage_bytes_per_atom(nn_r, s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
+        "nep_staged_kernel": ("mfma", (nep_flops_per_atom(nn_r, nn_a) - nep_stage_flops_per_atom(nn_r)) * n, "TFLOP/s",
+                              PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
         "nep_group_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
-        "nbl_lists": ("hbm", ((3 * s + 4) + 12 + U * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
+        # the calculator updates its list in place: a row is written as far as its old or new
+        # length reaches, rounded up to four slots (about two more than its length on average)
+        "nbl_lists": ("hbm", ((3 * s + 4) + 12 + (nn_r + 2) * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
         "reduce_fill": ("hbm", (nn_r * (3 * s + 4) + nn_r * 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
     }
     config = {"workload": args.workload, "natoms": n, "species": 3,

@@ -102,6 +102,24 @@ int a2p_nblist_build_f64(const double* lattice, const int* types, const double* 
                          int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
                          void* stream);
 
+/* Rebuild into buffers that already hold a list.  Same arguments and results as
+ * a2p_nblist_build_*, for a caller that keeps its list buffers between steps (molecular
+ * dynamics; the reference allocates fresh arrays per call, nblist_bind.cc:95-134, so it has no
+ * counterpart of the distinction).  Contract: numneigh, firstneigh and rcs hold the unmodified
+ * result of an earlier a2p_nblist_build_* or a2p_nblist_update_* call with the same natoms and
+ * umax.  With sort = 0 a row is then written only up to the longer of its old and new lengths:
+ * the -1 / 0 padding beyond is already in place, which saves three quarters of the writes at
+ * umax = 200 and 48 neighbours.  With sort = 1 the call is the same as a2p_nblist_build_*. */
+int a2p_nblist_update_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                          double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                          int* numneigh, int* firstneigh, float* rcs, int* types_out, int* max_numneigh,
+                          void* stream);
+
+int a2p_nblist_update_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                          double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,
+                          int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
+                          void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Linear Moment Tensor Potential.
  *

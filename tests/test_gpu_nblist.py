@@ -76,6 +76,55 @@ def test_row_capacities(oracle, dt, umax):
     assert_same(a, b)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("umax", [56, 54, 2000])
+def test_update_in_place(oracle, dt, umax):
+    """a2p_nblist_update_* into buffers that hold an earlier list: after every step the whole
+    arrays, padding included, are those of a fresh build.  The atoms move far enough between the
+    steps for rows to grow and to shrink; the three capacities take the LDS row buffer, the
+    direct stores and the rows too large for the buffer."""
+    import ctypes as c
+    import torch
+    from ai2pot_amd import _lib
+    L = _lib.lib()
+    f32 = dt == np.float32
+    build = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
+    update = L.a2p_nblist_update_f32 if f32 else L.a2p_nblist_update_f64
+    n = 200
+    lat, pos = synth.random_packed(n, [14.0, 15.0, 16.0], 2.2, 91)
+    types = synth.rng_randint(92, n, 2)
+    dev = "cuda:0"
+    tdt = torch.float32 if f32 else torch.float64
+    i32 = dict(dtype=torch.int32, device=dev)
+    t_types = torch.from_numpy(types.astype(np.int32)).to(dev)
+    ilist, numneigh, types_out = torch.empty(n, **i32), torch.empty(n, **i32), torch.empty(n, **i32)
+    first = torch.empty((n, umax), **i32)
+    rcs = torch.empty((n, umax, 3), dtype=tdt, device=dev)
+    lat_h = np.ascontiguousarray(lat, dt).reshape(9)
+    pbc = np.ones(3, np.int32)
+    vp = lambda t: c.c_void_p(t.data_ptr())
+    lengths = []
+    for step in range(4):
+        p = (pos + synth.rng_normal(300 + step, pos.size, 0.0, 0.35 * step).reshape(-1, 3)).astype(dt)
+        coords = torch.from_numpy(p).to(dev)
+        fn = build if step == 0 else update
+        rc = fn(lat_h.ctypes.data_as(c.c_void_p), vp(t_types), vp(coords), c.c_int(n), c.c_double(5.0),
+                c.c_int(umax), c.c_int(1), pbc.ctypes.data_as(c.c_void_p), c.c_int(0), vp(ilist),
+                vp(numneigh), vp(first), vp(rcs), vp(types_out), None,
+                c.c_void_p(torch.cuda.current_stream().cuda_stream))
+        _lib.check(rc)
+        torch.cuda.synchronize()
+        _lib.check_status(torch.cuda.current_stream().cuda_stream)
+        b = oracle.nblist(lat.astype(dt), types, p, 5.0, umax)
+        a = (n, ilist.cpu().numpy(), numneigh.cpu().numpy(), first.cpu().numpy(), rcs.cpu().numpy(),
+             types_out.cpu().numpy(), 0)
+        assert_same(a, b)
+        lengths.append(a[2].copy())
+    grew = sum(int((lengths[k + 1] > lengths[k]).sum()) for k in range(3))
+    shrank = sum(int((lengths[k + 1] < lengths[k]).sum()) for k in range(3))
+    assert grew > 20 and shrank > 20        # the sequence exercises both directions
+
+
 @pytest.mark.parametrize("sort", [False, True])
 def test_config2_size(oracle, sort):
     lat, pos = synth.random_packed(4096, [49.8848] * 3, 2.2, 1003)
