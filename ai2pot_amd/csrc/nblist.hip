@@ -61,6 +61,8 @@ struct Grid {
     int N;
     int ext_bins;     // ceil(rcut / bin_size) = 2
     int is_cart;
+    float inv_side;   // 1 / (2 ext_bins + 1), 1 / bin_size: for the pruning arithmetic of the
+    float inv_bin;    // list kernel, which is approximate by design
 };
 
 // image coordinate x + b0*ii + b1*jj + b2*kk, left to right (structure.h:659-676)
@@ -319,8 +321,6 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T));
         rb_rcs = (T*)mine;
         rb_first = (int*)(mine + (size_t)umax * 3 * sizeof(T));
-        for (int i = lane; i < umax; i += 64) rb_first[i] = -1;            // neighborList.h:557, 563
-        for (int i = lane; i < umax * 3; i += 64) rb_rcs[i] = (T)0;
     }
     T c[3];
     int cb[3];
@@ -332,7 +332,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     const int e = g.ext_bins, side = 2 * e + 1, nruns = side * side;
     int start = 0, len = 0;
     if (lane < nruns) {
-        const int lq = (int)(((float)lane + 0.5f) / (float)side);    // lane / side for small integers
+        const int lq = (int)(((float)lane + 0.5f) * g.inv_side);     // lane / side for small integers
         const int bx = cb[0] + lq - e, by = cb[1] + (lane - lq * side) - e;
         int zlo = cb[2] - e, zhi = cb[2] + e;
         // bins outside the reference's grid are skipped (binLinkedList.h:952-968); inside it the
@@ -345,7 +345,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         // geometric pruning (float is enough: the margin dwarfs its rounding): distance from the
         // atom to the column's rectangle in x and y, then the reach left for z
         {
-            const float bs = (float)g.bin_size, inv_bs = 1.0f / bs, rc2 = (float)g.rcut2 * 1.00001f;
+            const float bs = (float)g.bin_size, inv_bs = g.inv_bin, rc2 = (float)g.rcut2 * 1.00001f;
             float lat2 = 0.0f;
             const int bxy[2] = {bx, by};
 #pragma unroll
@@ -360,7 +360,8 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
             else {
                 const float rel = (float)c[2] - (float)g.mn[2];
                 const float tol = 1.0e-3f * bs + 1.0e-5f * (fabsf(rel) + fabsf((float)c[2]) + fabsf((float)g.mn[2]));
-                const float reach = sqrtf(rc2 - lat2) + tol;
+                // the hardware square root is within an ulp; the tolerance is five orders above that
+                const float reach = __builtin_amdgcn_sqrtf(rc2 - lat2) + tol;
                 zlo = max(zlo, (int)floorf((rel - reach) * inv_bs - 1.0e-3f));
                 zhi = min(zhi, (int)floorf((rel + reach) * inv_bs + 1.0e-3f));
             }
@@ -452,7 +453,13 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         __builtin_amdgcn_wave_barrier();
         const uint4* s1 = reinterpret_cast<const uint4*>(rb_first);
         uint4* d1 = reinterpret_cast<uint4*>(firstneigh + rowi);
-        const int live = (max(min(cnt, umax), old_len) + 3) & ~3;     // umax is a multiple of 4
+        const int used = min(cnt, umax);
+        const int live = (max(used, old_len) + 3) & ~3;               // umax is a multiple of 4
+        for (int i = used + lane; i < live; i += 64) {                 // padding, neighborList.h:557, 563
+            rb_first[i] = -1;
+            rb_rcs[i * 3 + 0] = (T)0; rb_rcs[i * 3 + 1] = (T)0; rb_rcs[i * 3 + 2] = (T)0;
+        }
+        __builtin_amdgcn_wave_barrier();
         for (int i = lane; i < live / 4; i += 64) d1[i] = s1[i];
         const uint4* s2 = reinterpret_cast<const uint4*>(rb_rcs);
         uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
@@ -709,6 +716,8 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     g.nimg = (int)nimg;
     g.ext_bins = (int)std::ceil(g.rcut / g.bin_size);          // binLinkedList.h:914-915
     A2P_REQUIRE(g.ext_bins >= 1 && g.ext_bins <= 3, A2P_ERR_INVALID, "nblist: unsupported bin stencil");
+    g.inv_side = 1.0f / (float)(2 * g.ext_bins + 1);
+    g.inv_bin = 1.0f / (float)g.bin_size;
 
     // workspace A: x[N*3] | partial[nblocks*12] | ext[12]
     const int nblocks = ceil_div(N, NBL_BLOCK);
