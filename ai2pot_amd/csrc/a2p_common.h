@@ -50,6 +50,8 @@ enum WsSlot {
 // Returns a device pointer valid until the next ws_get on the same slot with a larger size.
 // Growth synchronises the device (hipFree); steady-state calls do not allocate.
 int ws_get(int slot, size_t bytes, void** out);
+size_t ws_bytes();     // held on the current device
+int ws_release();      // synchronises the device, frees the current device's buffers
 
 // Device status word bits written by kernels when inputs violate the contract.
 enum StatusBits {

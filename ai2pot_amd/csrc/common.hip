@@ -52,6 +52,32 @@ int ws_get(int slot, size_t bytes, void** out)
     return A2P_OK;
 }
 
+size_t ws_bytes()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if ((int)g_ws.size() <= dev) return 0;
+    size_t total = 0;
+    for (const Buf& b : g_ws[dev].slot) total += b.bytes;
+    return total;
+}
+
+int ws_release()
+{
+    int dev = 0;
+    A2P_HIP_CHECK(hipGetDevice(&dev));
+    A2P_HIP_CHECK(hipDeviceSynchronize());          // no kernel of any stream still uses the buffers
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if ((int)g_ws.size() <= dev) return A2P_OK;
+    for (Buf& b : g_ws[dev].slot) {
+        if (b.ptr) A2P_HIP_CHECK(hipFree(b.ptr));
+        b.ptr = nullptr;
+        b.bytes = 0;
+    }
+    return A2P_OK;
+}
+
 // ---- per-kernel timing ---------------------------------------------------------------------
 namespace {
 struct ProfRec {
@@ -143,6 +169,10 @@ extern "C" {
 const char* a2p_last_error(void) { return a2p::last_error(); }
 
 int a2p_abi_version(void) { return 1; }
+
+size_t a2p_workspace_bytes(void) { return a2p::ws_bytes(); }
+
+int a2p_workspace_release(void) { return a2p::ws_release(); }
 
 void a2p_profile_enable(int on)
 {

@@ -30,6 +30,15 @@ const char* a2p_last_error(void);
 /* Version of this ABI (bumped on incompatible change). */
 int a2p_abi_version(void);
 
+/* The per-device workspace (no counterpart in the reference, whose operators allocate their
+ * scratch per call, e.g. source/descriptor/nep/include/nep.h:391-392).  It grows to what the
+ * largest call so far needed and is then reused, so calls on ONE device must not overlap in
+ * time: issue them on one stream, or order the streams with events.  Different devices are
+ * independent.  a2p_workspace_bytes returns what the library holds on the current device;
+ * a2p_workspace_release synchronises the device and frees it (the next call allocates again). */
+size_t a2p_workspace_bytes(void);
+int a2p_workspace_release(void);
+
 /* Reads and clears the device status word that kernels set when an input violates the
  * contract (neighbour index outside [0, natoms_pad+nghost), type index outside
  * [0, ntypes), numneigh > umax).  Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT or

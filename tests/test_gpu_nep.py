@@ -223,3 +223,23 @@ def test_errors(oracle):
                        d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"],
                        md["type_map"], 0, 7.0, 4.0, md["q_scaler"], 1.0, 0.5, None, None)
     call()                                                  # the library is still usable
+
+
+def test_workspace_release(oracle):
+    """a2p_workspace_bytes / a2p_workspace_release: the library holds scratch after a call, frees
+    it on request, and the next call (which allocates again) returns the same bits."""
+    import ctypes
+    from ai2pot_amd import _lib
+    L = _lib.lib()
+    L.a2p_workspace_bytes.restype = ctypes.c_size_t
+    m = synth.nep_model(seed=71)
+    nb = synth.pack_batch([small_structure(oracle, dtype=np.float32)])
+    first = run_gpu(m, nb, np.float32)
+    held = L.a2p_workspace_bytes()
+    assert held > 0
+    _lib.check(L.a2p_workspace_release())
+    assert L.a2p_workspace_bytes() == 0
+    again = run_gpu(m, nb, np.float32)
+    assert L.a2p_workspace_bytes() > 0
+    for a, b in zip(first, again):
+        assert np.array_equal(a, b)
