@@ -30,7 +30,8 @@
 namespace a2p {
 namespace {
 
-constexpr int MTP_NC = 32;        // neighbours per chunk
+constexpr int MTP_NC = 32;        // neighbours per chunk (rows of the LDS table); the energy / force / virial
+constexpr int MTP_NC_MAX = 48;    // launch raises it up to MTP_NC_MAX while that costs no workgroup per CU
 constexpr int MTP_NGMAX = 16;     // most thread groups that share the basic moments of a chunk
 constexpr int MTP_KMAX = 16;      // radial basis size limit
 constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
@@ -57,6 +58,7 @@ struct MtpArgs {
     T* gpart;          // [B, P, ngrad] per-atom gradient rows (ngrad = ncoef + n_scalar + ntypes)
     int ngrad;
     int lds_basic_off;  // byte offset of the packed basic-moment table in LDS
+    int nc_cap;         // rows of the LDS neighbour table: a row is processed in chunks of at most nc_cap
     // site-energy / descriptor mode (linearMtp.h:514-611, 821-890)
     T* e_sites;        // [B, P] per-row energies, or null
     T* desc;           // [B, P, n_scalar] scalar moments, or null
@@ -285,6 +287,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
               OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
     const int ncoef = a.ntypes * a.ntypes * nmus * K;
 
+    const int MTP_NC = a.nc_cap;
     T* M = (T*)smem_raw;
     T* A = M + n_moms;
     T* Tg = A + n_moms;                      // loss mode only
@@ -923,7 +926,7 @@ int table_entries(const MtpPlanDevice& p, int K, bool loss)
 }
 
 template <typename T>
-size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H)
+size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC)
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
     const size_t tabs = std::max((size_t)MTP_NC * E + (size_t)(256 / 32) * 32 * 4, (size_t)p.max_level_slots * (loss ? 2 : 1));
@@ -969,9 +972,25 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
 template <typename T, bool LOSS>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
-    const size_t lds_main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H) + 15) / 16 * 16;
-    const size_t lds = lds_main + (size_t)a.p.n_basic * sizeof(unsigned);
+    auto lds_for = [&](int nc, size_t* main) {
+        *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc) + 15) / 16 * 16;
+        return *main + (size_t)a.p.n_basic * sizeof(unsigned);
+    };
+    size_t lds_main = 0;
+    int nc_cap = MTP_NC;
+    size_t lds = lds_for(nc_cap, &lds_main);
+    // A longer table halves the chunks (table builds, barriers) of rows just above MTP_NC neighbours;
+    // taken only while as many workgroups still fit a CU.  The loss kernels keep MTP_NC.
+    if (!LOSS && lds <= 160 * 1024) {
+        const size_t per_cu = 160 * 1024, fit = per_cu / lds;
+        for (int nc = MTP_NC_MAX; nc > MTP_NC; nc -= 8) {
+            size_t m = 0;
+            const size_t l = lds_for(nc, &m);
+            if (per_cu / l == fit) { nc_cap = nc; lds = l; lds_main = m; break; }
+        }
+    }
     const_cast<MtpArgs<T>&>(a).lds_basic_off = (int)lds_main;
+    const_cast<MtpArgs<T>&>(a).nc_cap = nc_cap;
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
                 "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
     const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
