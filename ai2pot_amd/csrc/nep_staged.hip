@@ -166,7 +166,8 @@ __device__ __forceinline__ void staged_classify(const StageLds<T>& L, int tid, T
     }
 }
 
-// Compact-list entries: [x y z species]
+// Compact-list entries: [x y z place-in-segment]; the species (two bits) of 16 consecutive entries
+// of a thread's list share one word of a separate array
 __device__ __forceinline__ void ang_store(float* p, float x, float y, float z, int w)
 {
     *reinterpret_cast<float4*>(p) = make_float4(x, y, z, __int_as_float(w));
@@ -210,7 +211,7 @@ __device__ __forceinline__ void row_header(const NepArgs<T>& a, bool active, siz
 template <typename T, int NTC>
 __global__ void __launch_bounds__(SB, (sizeof(T) == 4 ? 4 : 2))
 nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T* __restrict__ ang_xyz,
-                 int* __restrict__ ang_pos, T* __restrict__ radial, int* __restrict__ counts)
+                 unsigned* __restrict__ typew, T* __restrict__ radial, int* __restrict__ counts)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tid = threadIdx.x;
@@ -242,9 +243,15 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
     const int mblk = ii / FB, mtid = ii - mblk * FB;
     const size_t list0 = (size_t)(b * a.nblocks + mblk) * a.U * FB + mtid;
     T* const lxyz = ang_xyz + list0 * 4;
-    int* const lpos = ang_pos + list0;
     const int back = a.U - 1;
     const bool want_pairs = a.force != nullptr || a.want_virial;
+    // species words of the two lists: word w of the front list at typew[w * plane + o], of the
+    // back list (counted from its own first entry) behind the front list's NW words
+    const size_t o = (size_t)(b * a.nblocks + mblk) * FB + mtid;
+    const size_t plane = (size_t)a.B * a.nblocks * FB;
+    unsigned* const tw_front = typew + o;
+    unsigned* const tw_back = typew + (size_t)((a.U + 15) / 16) * plane + o;
+    unsigned tw_rad = 0u, tw_ang = 0u;
 
     T F[NTC][KC];                 // radial functions summed per neighbour species
 #pragma unroll
@@ -272,9 +279,10 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
 #pragma unroll
                 for (int k = 0; k < KC; k++) F[t][k] += (tj == t) ? f[k] : (T)0;
             if (want_pairs && !((mA >> s) & 1u)) {
-                ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, tj);
-                lpos[(size_t)n_rad * FB] = L.p[s * SLS + tid];
+                ang_store(lxyz + (size_t)n_rad * FB * 4, x, y, z, L.p[s * SLS + tid]);
+                tw_rad |= (unsigned)tj << (2 * (n_rad & 15));
                 n_rad++;
+                if ((n_rad & 15) == 0) { tw_front[(size_t)((n_rad >> 4) - 1) * plane] = tw_rad; tw_rad = 0u; }
             }
         }
         bits = mA;
@@ -283,9 +291,10 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
             bits &= bits - 1;
             const int k = back - n_ang;
             ang_store(lxyz + (size_t)k * FB * 4, L.x[s * SLS + tid], L.y[s * SLS + tid], L.z[s * SLS + tid],
-                      L.w[s * SLS + tid]);
-            lpos[(size_t)k * FB] = L.p[s * SLS + tid];
+                      L.p[s * SLS + tid]);
+            tw_ang |= (unsigned)L.w[s * SLS + tid] << (2 * (n_ang & 15));
             n_ang++;
+            if ((n_ang & 15) == 0) { tw_back[(size_t)((n_ang >> 4) - 1) * plane] = tw_ang; tw_ang = 0u; }
         }
         // pairs of the list beyond both cutoffs still own a place in their segment
         bits = mV & ~mR & ~mA;
@@ -296,9 +305,9 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
             dst[0] = (T)0; dst[1] = (T)0; dst[2] = (T)0;
         }
     }
+    if (n_rad & 15) tw_front[(size_t)(n_rad >> 4) * plane] = tw_rad;
+    if (n_ang & 15) tw_back[(size_t)(n_ang >> 4) * plane] = tw_ang;
     if (ii < a.P) {
-        const size_t o = (size_t)(b * a.nblocks + mblk) * FB + mtid;
-        const size_t plane = (size_t)a.B * a.nblocks * FB;
 #pragma unroll
         for (int t = 0; t < NTC; t++)
 #pragma unroll
@@ -311,7 +320,7 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
 template <typename T, int NTC>
 __global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
 nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict__ ang_xyz,
-                  const int* __restrict__ ang_pos, const T* __restrict__ radial, const int* __restrict__ counts)
+                  const unsigned* __restrict__ typew, const T* __restrict__ radial, const int* __restrict__ counts)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tid = threadIdx.x;
@@ -341,7 +350,8 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
     const size_t plane = (size_t)a.B * a.nblocks * FB;
     const size_t list0 = (size_t)(b * a.nblocks + blockIdx.x) * a.U * FB + tid;
     const T* const lxyz = ang_xyz + list0 * 4;
-    const int* const lpos = ang_pos + list0;
+    const unsigned* const tw_front = typew + o;
+    const unsigned* const tw_back = typew + (size_t)((a.U + 15) / 16) * plane + o;
     const int back = a.U - 1;
     const bool want_pairs = a.force != nullptr || a.want_virial;
     // rows past P were not staged
@@ -365,9 +375,11 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
     T px = (T)0, py = (T)0, pz = (T)0;
     int pw = 0;
     if (n_ang > 0) ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw);
+    unsigned tw = 0u;
     for (int e = 0; e < n_ang; e++) {
         const T x = px, y = py, z = pz;
-        const int tj = pw;
+        if ((e & 15) == 0) tw = tw_back[(size_t)(e >> 4) * plane];
+        const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
         if (e + 1 < n_ang) ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
         const T r = sqrt_t(x * x + y * y + z * z);
         const T rinv = (T)1 / r;
@@ -505,15 +517,13 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
             vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
         };
         // radial-only pairs (front list)
-        int ppos = 0;
-        if (n_rad > 0) { ang_load(lxyz, px, py, pz, pw); ppos = lpos[0]; }
+        if (n_rad > 0) ang_load(lxyz, px, py, pz, pw);
         for (int e = 0; e < n_rad; e++) {
             const T x = px, y = py, z = pz;
-            const int tj = pw, pos = ppos;
-            if (e + 1 < n_rad) {
-                ang_load(lxyz + (size_t)(e + 1) * FB * 4, px, py, pz, pw);
-                ppos = lpos[(size_t)(e + 1) * FB];
-            }
+            const int pos = pw;
+            if ((e & 15) == 0) tw = tw_front[(size_t)(e >> 4) * plane];
+            const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
+            if (e + 1 < n_rad) ang_load(lxyz + (size_t)(e + 1) * FB * 4, px, py, pz, pw);
             const T r = sqrt_t(x * x + y * y + z * z);
             T f[KC], df[KC];
             radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
@@ -524,14 +534,13 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
             emit(pos, x, y, z, sr * x, sr * y, sr * z);
         }
         // pairs inside the angular cutoff, radial and angular part together (back list)
-        if (n_ang > 0) { ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw); ppos = lpos[(size_t)back * FB]; }
+        if (n_ang > 0) ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw);
         for (int e = 0; e < n_ang; e++) {
             const T x = px, y = py, z = pz;
-            const int tj = pw, pos = ppos;
-            if (e + 1 < n_ang) {
-                ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
-                ppos = lpos[(size_t)(back - e - 1) * FB];
-            }
+            const int pos = pw;
+            if ((e & 15) == 0) tw = tw_back[(size_t)(e >> 4) * plane];
+            const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
+            if (e + 1 < n_ang) ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
             const T r = sqrt_t(x * x + y * y + z * z);
             const T rinv = (T)1 / r;
             const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
@@ -602,17 +611,19 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
 template <typename T, int NTC>
 int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
 {
-    // workspace: compact lists [workgroup][entry < U][thread] of 4 T, the same of int, then per
-    // row the summed radial functions [NTC*KC] and the two list lengths
+    // workspace: compact lists [workgroup][entry < U][thread] of 4 T; species words of the front and
+    // of the back list, [2][ceil(U / 16)][row]; per row the summed radial functions [NTC*KC] and the
+    // two list lengths
     const size_t plane = (size_t)a.B * a.nblocks * FB;
     const size_t nent = plane * a.U;
+    const size_t nwords = 2 * (size_t)((a.U + 15) / 16) * plane;
     void* ws = nullptr;
-    int rc = ws_get(WS_PAIR_G, nent * (4 * sizeof(T) + sizeof(int)) + plane * (NTC * KC * sizeof(T) + 2 * sizeof(int)),
-                    &ws);
+    int rc = ws_get(WS_PAIR_G, nent * 4 * sizeof(T) + nwords * sizeof(unsigned) +
+                                   plane * (NTC * KC * sizeof(T) + 2 * sizeof(int)), &ws);
     if (rc) return rc;
     T* ang_xyz = (T*)ws;
-    int* ang_pos = (int*)((char*)ws + nent * 4 * sizeof(T));
-    T* radial = (T*)((char*)ws + nent * (4 * sizeof(T) + sizeof(int)));
+    unsigned* typew = (unsigned*)((char*)ws + nent * 4 * sizeof(T));
+    T* radial = (T*)((char*)ws + nent * 4 * sizeof(T) + nwords * sizeof(unsigned));
     int* counts = (int*)(radial + plane * NTC * KC);
     SegArgs seg{csr.cursor, csr.seg_cap, csr.n * csr.seg_cap};
     StageLds<T> unused;
@@ -623,7 +634,7 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
                                           (int)lds_stage));
     prof_begin("nep_stage_kernel", stream);
     hipLaunchKernelGGL(stage, dim3(ceil_div(a.P, SB), a.B), dim3(SB), lds_stage, stream, a, seg, (T*)csr.seg_g,
-                       ang_xyz, ang_pos, radial, counts);
+                       ang_xyz, typew, radial, counts);
     prof_end(stream);
     auto kern = nep_staged_kernel<T, NTC>;
     if (lds > 48 * 1024)
@@ -631,7 +642,7 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
                                           (int)lds));
     prof_begin("nep_staged_kernel", stream);
     hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, (T*)csr.seg_g, (const T*)ang_xyz,
-                       (const int*)ang_pos, (const T*)radial, (const int*)counts);
+                       (const unsigned*)typew, (const T*)radial, (const int*)counts);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
