@@ -46,9 +46,10 @@ def nep_stage_flops_per_atom(nr_mean, K=8):
 
 def nep_stage_bytes_per_atom(nr_mean, s, ntc=3, K=8):
     """Staging kernel, algorithmic bytes: per pair the relative vector, the neighbour index, its
-    species, the segment counter (read and written by the atomic), and the compact-list entry with
-    its place; per atom the row header and the summed radial functions with the two list lengths."""
-    return nr_mean * ((3 * s + 4 + 4 + 8) + (4 * s + 4)) + 12 + ntc * K * s + 8
+    species, the segment counter (read and written by the atomic), and the compact-list entry (vector
+    and place, plus two bits of species); per atom the row header and the summed radial functions
+    with the two list lengths."""
+    return nr_mean * ((3 * s + 4 + 4 + 8) + (4 * s + 0.25)) + 12 + ntc * K * s + 8
 
 
 def mtp_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar):
@@ -109,9 +110,9 @@ def timed_replay(replay, steps, warmup):
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
 MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nep_stage_kernel"): 4.402e6 * 1024,
-    ("nep_md_1048576", "nep_staged_kernel"): 3.218e6 * 1024,
-    ("nep_md_1048576", "nbl_lists"): 1.216e6 * 1024,
+    ("nep_md_1048576", "nep_stage_kernel"): 4.075e6 * 1024,
+    ("nep_md_1048576", "nep_staged_kernel"): 3.023e6 * 1024,
+    ("nep_md_1048576", "nbl_lists"): 1.214e6 * 1024,
 }
 
 
