@@ -120,8 +120,9 @@ __device__ __forceinline__ int wave_inclusive_scan(int v)
 // Deterministic reduction of per-pair derivatives g[row, slot, 3] onto atoms:
 //   force[b, j] = own[b, j] - sum over pairs (row, slot) of structure b whose neighbour is j.
 // `force` must already hold the `own` part (zero for atoms without a row).  Integer atomics
-// build the incoming lists; the floating-point sums are order-independent (exact fixed-point
-// accumulation against the per-target maximum), so results are reproducible run to run.
+// build the incoming lists; the floating-point sums are order-independent (terms rounded to a
+// common quantum chosen from the per-target maximum, then added exactly), so results are
+// reproducible run to run.
 template <typename T>
 int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, const int* binum,
                 const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);

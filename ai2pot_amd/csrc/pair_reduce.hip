@@ -162,6 +162,76 @@ __global__ void reduce_kernel(T* __restrict__ force, const T* __restrict__ seg_g
     // seg_cap > 0: segments of fixed capacity, target t owns entries [t*seg_cap, (t+1)*seg_cap)
     const int beg = !live ? 0 : seg_cap > 0 ? t * seg_cap : offsets[t];
     const int cnt = !live ? 0 : seg_cap > 0 ? min(counts[t], seg_cap) : counts[t];
+    if constexpr (sizeof(T) == 4) {
+        // fp32 segments: every value is rounded to a multiple of 2^q, q chosen from the segment's
+        // largest magnitude and its length so that any partial sum of the rounded values fits the
+        // 53 bits of a double: the additions are then exact in whatever order they happen.  The
+        // first four entries of every lane stay in registers between the two passes.
+        float gx[4], gy[4], gz[4];
+        float mf = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int e = sub + 16 * k;
+            gx[k] = 0.0f; gy[k] = 0.0f; gz[k] = 0.0f;
+            if (e < cnt) {
+                const float* g = seg_g + (size_t)(beg + e) * 3;
+                gx[k] = g[0]; gy[k] = g[1]; gz[k] = g[2];
+            }
+            mf = fmaxf(mf, fmaxf(fabsf(gx[k]), fmaxf(fabsf(gy[k]), fabsf(gz[k]))));
+            // fmaxf drops a NaN operand: keep it
+            if (gx[k] != gx[k] || gy[k] != gy[k] || gz[k] != gz[k]) mf = NAN;
+        }
+        for (int e = sub + 64; e < cnt; e += 16) {
+            const float* g = seg_g + (size_t)(beg + e) * 3;
+            const float a0 = g[0], a1 = g[1], a2 = g[2];
+            if (!(mf != mf)) mf = fmaxf(mf, fmaxf(fabsf(a0), fmaxf(fabsf(a1), fabsf(a2))));
+            if (a0 != a0 || a1 != a1 || a2 != a2) mf = NAN;
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+            const float o = __shfl_xor(mf, off, 64);
+            mf = (mf != mf || o != o) ? NAN : fmaxf(mf, o);
+        }
+        if (cnt == 0) return;               // uniform over the 16 lanes of a target
+        const bool finite = mf < 3.0e38f && mf == mf;
+        double s0 = 0.0, s1 = 0.0, s2 = 0.0;
+        const bool any = finite && mf > 0.0f;
+        if (any) {
+            // |v| < 2^(ex+1), fewer than 2^hb of them: sums stay below 2^(ex+1+hb), so q = ex + hb - 52;
+            // (v + C) - C with C = 1.5 * 2^(52+q) rounds v to a multiple of 2^q (needs hb >= 2)
+            const int hb = max(32 - __clz(cnt), 2);
+            const double C = ldexp(1.5, ilogbf(mf) + hb);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                s0 += ((double)gx[k] + C) - C;
+                s1 += ((double)gy[k] + C) - C;
+                s2 += ((double)gz[k] + C) - C;
+            }
+            for (int e = sub + 64; e < cnt; e += 16) {
+                const float* g = seg_g + (size_t)(beg + e) * 3;
+                s0 += ((double)g[0] + C) - C;
+                s1 += ((double)g[1] + C) - C;
+                s2 += ((double)g[2] + C) - C;
+            }
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+            s0 += __shfl_xor(s0, off, 64);
+            s1 += __shfl_xor(s1, off, 64);
+            s2 += __shfl_xor(s2, off, 64);
+        }
+        if (sub == 0) {
+            T* f = force + (size_t)t * 3;
+            if (!finite) {
+                f[0] = f[1] = f[2] = (T)NAN;
+            } else if (any) {
+                f[0] = (T)((double)f[0] - s0);
+                f[1] = (T)((double)f[1] - s1);
+                f[2] = (T)((double)f[2] - s2);
+            }
+        }
+        return;
+    }
     // pass 1: largest magnitude of the segment
     double m = 0.0;
     for (int e = sub; e < cnt; e += 16) {
