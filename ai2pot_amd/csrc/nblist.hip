@@ -63,6 +63,8 @@ struct Grid {
     int is_cart;
     float inv_side;   // 1 / (2 ext_bins + 1), 1 / bin_size: for the pruning arithmetic of the
     float inv_bin;    // list kernel, which is approximate by design
+    T keep_lo[3];     // coordinates outside [keep_lo, keep_hi] lie outside the kept bin box for sure
+    T keep_hi[3];     // (the box widened by far more than the rounding of the binning)
 };
 
 // image coordinate x + b0*ii + b1*jj + b2*kk, left to right (structure.h:659-676)
@@ -146,81 +148,85 @@ __global__ void coords_minmax_kernel(const Grid<T> g, const T* __restrict__ coor
     }
 }
 
+// 12 wavefronts, one per extent (minima of the image coordinates, their maxima, minima and maxima
+// of the centre atoms, three axes each)
 template <typename T>
 __global__ void minmax_finish_kernel(const T* __restrict__ partial, int nblocks, T* __restrict__ out)
 {
-    __shared__ T sh[256];
-    for (int q = 0; q < 12; q++) {
-        const bool is_min = (q % 6) < 3;
-        T r = is_min ? (T)INT_MAX : (T)INT_MIN;
-        for (int k = threadIdx.x; k < nblocks; k += 256) {
-            T o = partial[(size_t)k * 12 + q];
-            r = is_min ? (o < r ? o : r) : (o > r ? o : r);
-        }
-        sh[threadIdx.x] = r;
-        __syncthreads();
-        for (int s = 128; s > 0; s >>= 1) {
-            if ((int)threadIdx.x < s) {
-                T o = sh[threadIdx.x + s];
-                T m = sh[threadIdx.x];
-                sh[threadIdx.x] = is_min ? (o < m ? o : m) : (o > m ? o : m);
-            }
-            __syncthreads();
-        }
-        if (threadIdx.x == 0) out[q] = sh[0];
-        __syncthreads();
+    const int q = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool is_min = (q % 6) < 3;
+    T r = is_min ? (T)INT_MAX : (T)INT_MIN;
+    for (int k = lane; k < nblocks; k += 64) {
+        const T o = partial[(size_t)k * 12 + q];
+        r = is_min ? (o < r ? o : r) : (o > r ? o : r);
     }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const T o = __shfl_xor(r, off, 64);
+        r = is_min ? (o < r ? o : r) : (o > r ? o : r);
+    }
+    if (lane == 0) out[q] = r;
 }
 
 // ---- 2 / 4. binning of (atom, image) pairs ---------------------------------------------------
-// Returns the storage index of the pair's bin inside the box, or -1 when it lies outside.
+// Image (i, j, k) of an atom at xp: storage index of its bin inside the box, or -1 when outside.
 template <typename T>
-__device__ __forceinline__ int locate(const Grid<T>& g, const T* __restrict__ x, long long pair, T* c,
-                                      int* sidx)
+__device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i, int j, int k, T* c)
 {
-    const int m = (int)(pair / g.N);
-    const int p = (int)(pair - (long long)m * g.N);
-    const int k = m % g.img_dim[2];
-    const int j = (m / g.img_dim[2]) % g.img_dim[1];
-    const int i = m / (g.img_dim[2] * g.img_dim[1]);
     int bin[3];
+    // most images of most atoms lie far outside the box: two comparisons per axis settle them
+    // before the exactly rounded divisions of the binning
 #pragma unroll
     for (int a = 0; a < 3; a++) {
-        c[a] = image_coord(x[(size_t)p * 3 + a], g.b[0][a], g.b[1][a], g.b[2][a], g.img_lo[0] + i,
-                           g.img_lo[1] + j, g.img_lo[2] + k);
+        c[a] = image_coord(xp[a], g.b[0][a], g.b[1][a], g.b[2][a], g.img_lo[0] + i, g.img_lo[1] + j,
+                           g.img_lo[2] + k);
+        if (c[a] < g.keep_lo[a] || c[a] > g.keep_hi[a]) return -1;
+    }
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
         bin[a] = bin_of(c[a], g.mn[a], g.bin_size) - g.rlo[a];
         if (bin[a] < 0 || bin[a] >= g.rdim[a]) return -1;
     }
-    *sidx = m * g.N + p;      // supercell index: image-major, x outer / z inner (structure.h:654-681)
     return (bin[0] * g.rdim[1] + bin[1]) * g.rdim[2] + bin[2];
 }
 
+// One thread per atom walks its images (x outer, z inner: image m = (i * dim_y + j) * dim_z + k,
+// supercell index m * N + p, structure.h:654-681).
 template <typename T>
 __global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __restrict__ counts)
 {
-    const long long pair = (long long)blockIdx.x * NBL_BLOCK + threadIdx.x;
-    if (pair >= (long long)g.N * g.nimg) return;
-    T c[3];
-    int sidx;
-    const int bin = locate(g, x, pair, c, &sidx);
-    if (bin >= 0) atomicAdd(&counts[bin], 1);
+    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (p >= g.N) return;
+    const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
+    for (int i = 0; i < g.img_dim[0]; i++)
+        for (int j = 0; j < g.img_dim[1]; j++)
+            for (int k = 0; k < g.img_dim[2]; k++) {
+                T c[3];
+                const int bin = locate(g, xp, i, j, k, c);
+                if (bin >= 0) atomicAdd(&counts[bin], 1);
+            }
 }
 
 template <typename T>
 __global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ offsets,
                             int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x)
 {
-    const long long pair = (long long)blockIdx.x * NBL_BLOCK + threadIdx.x;
-    if (pair >= (long long)g.N * g.nimg) return;
-    T c[3];
-    int sidx;
-    const int bin = locate(g, x, pair, c, &sidx);
-    if (bin < 0) return;
-    const int pos = offsets[bin] + atomicAdd(&cursor[bin], 1);
-    s_idx[pos] = sidx;
-    s_x[(size_t)pos * 3 + 0] = c[0];
-    s_x[(size_t)pos * 3 + 1] = c[1];
-    s_x[(size_t)pos * 3 + 2] = c[2];
+    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (p >= g.N) return;
+    const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
+    int m = 0;
+    for (int i = 0; i < g.img_dim[0]; i++)
+        for (int j = 0; j < g.img_dim[1]; j++)
+            for (int k = 0; k < g.img_dim[2]; k++, m++) {
+                T c[3];
+                const int bin = locate(g, xp, i, j, k, c);
+                if (bin < 0) continue;
+                const int pos = offsets[bin] + atomicAdd(&cursor[bin], 1);
+                s_idx[pos] = m * g.N + p;
+                s_x[(size_t)pos * 3 + 0] = c[0];
+                s_x[(size_t)pos * 3 + 1] = c[1];
+                s_x[(size_t)pos * 3 + 2] = c[2];
+            }
 }
 
 // ---- 5. order inside a bin: descending supercell index (head insertion, binLinkedList.h:833) -
@@ -739,7 +745,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                        partial);
     prof_end(stream);
     prof_begin("nbl_coords_minmax", stream);
-    hipLaunchKernelGGL(minmax_finish_kernel<T>, dim3(1), dim3(256), 0, stream, partial, nblocks, ext_dev);
+    hipLaunchKernelGGL(minmax_finish_kernel<T>, dim3(1), dim3(12 * 64), 0, stream, partial, nblocks, ext_dev);
     prof_end(stream);
     T ext[12];
     A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
@@ -761,6 +767,14 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         const int rhi = std::min(cb_hi + g.ext_bins, g.nbin[a] - 1);
         g.rdim[a] = rhi - g.rlo[a] + 1;
         A2P_REQUIRE(g.rdim[a] > 0, A2P_ERR_INVALID, "nblist: empty bin box");
+        {
+            // a coordinate c is binned as floor((c - mn) / bin_size) in T: the slack covers the
+            // rounding of that expression and of the two bounds by orders of magnitude
+            const double big = std::max(std::fabs((double)mn), std::fabs((double)mx));
+            const double slack = 1.0e-3 * (double)g.bin_size + 1.0e-5 * (big + (double)pl);
+            g.keep_lo[a] = (T)((double)mn + (double)g.rlo[a] * (double)g.bin_size - slack);
+            g.keep_hi[a] = (T)((double)mn + (double)(g.rlo[a] + g.rdim[a]) * (double)g.bin_size + slack);
+        }
         nregion *= g.rdim[a];
     }
     A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID,
@@ -783,10 +797,9 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (rc) return rc;
     rc = fill_zero(cursor, (size_t)nb1 * sizeof(int), stream);
     if (rc) return rc;
-    const long long npairs = (long long)N * g.nimg;
-    const int pair_blocks = ceil_div(npairs, NBL_BLOCK);
+    const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
     prof_begin("nbl_count", stream);
-    hipLaunchKernelGGL(count_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, counts);
+    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts);
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
@@ -815,7 +828,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
 
     prof_begin("nbl_fill", stream);
 
-    hipLaunchKernelGGL(fill_kernel<T>, dim3(pair_blocks), dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
+    hipLaunchKernelGGL(fill_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
                        s_idx, s_x);
 
     prof_end(stream);
