@@ -306,37 +306,17 @@ constexpr int NBL_ENT_CAP = 256;   // flat candidate list per wave (entries); lo
 template <typename T>
 inline size_t rowbuf_bytes(int umax) { return (size_t)umax * (4 + 3 * sizeof(T)); }
 
-template <typename T, bool SORT, bool ROWBUF>
-__global__ void __launch_bounds__(NBL_BLOCK)
-lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
-             const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
-             int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
-             T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
-             int* __restrict__ status, int update)
+// Run of supercell entries that column `lane` of the (2e+1)^2 columns around the bin of the atom at
+// c can contribute: start index and length (0 for lanes without a column or with nothing in reach).
+template <typename T>
+__device__ __forceinline__ void column_setup(const Grid<T>& g, const T (&c)[3], int lane,
+                                             const int* __restrict__ offsets, int& start, int& len)
 {
-    __shared__ int sh_start[NBL_BLOCK / 64][64];
-    __shared__ int sh_base[NBL_BLOCK / 64][64];
-    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
-    extern __shared__ __align__(16) unsigned char sh_rows[];
-    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int p = blockIdx.x * (NBL_BLOCK / 64) + wv;
-    if (p >= g.N) return;                         // whole wave leaves together
-    T* rb_rcs = nullptr;
-    int* rb_first = nullptr;
-    if (ROWBUF) {
-        unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T));
-        rb_rcs = (T*)mine;
-        rb_first = (int*)(mine + (size_t)umax * 3 * sizeof(T));
-    }
-    T c[3];
     int cb[3];
 #pragma unroll
-    for (int a = 0; a < 3; a++) {
-        c[a] = x[(size_t)p * 3 + a];
-        cb[a] = bin_of(c[a], g.mn[a], g.bin_size);
-    }
+    for (int a = 0; a < 3; a++) cb[a] = bin_of(c[a], g.mn[a], g.bin_size);
     const int e = g.ext_bins, side = 2 * e + 1, nruns = side * side;
-    int start = 0, len = 0;
+    start = 0; len = 0;
     if (lane < nruns) {
         const int lq = (int)(((float)lane + 0.5f) * g.inv_side);     // lane / side for small integers
         const int bx = cb[0] + lq - e, by = cb[1] + (lane - lq * side) - e;
@@ -378,6 +358,51 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
             len = offsets[col + zhi + 1] - start;
         }
     }
+}
+
+constexpr int NBL_APW = 2;         // consecutive centre atoms per wavefront
+
+template <typename T, bool SORT, bool ROWBUF>
+__global__ void __launch_bounds__(NBL_BLOCK)
+lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
+             const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
+             int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
+             T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
+             int* __restrict__ status, int update)
+{
+    __shared__ int sh_start[NBL_BLOCK / 64][64];
+    __shared__ int sh_base[NBL_BLOCK / 64][64];
+    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
+    extern __shared__ __align__(16) unsigned char sh_rows[];
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * NBL_APW;
+    if (p0 >= g.N) return;                        // whole wave leaves together
+    const int np = min(NBL_APW, g.N - p0);
+    T* rb_rcs = nullptr;
+    int* rb_first = nullptr;
+    if (ROWBUF) {
+        unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T));
+        rb_rcs = (T*)mine;
+        rb_first = (int*)(mine + (size_t)umax * 3 * sizeof(T));
+    }
+    // A row costs three dependent trips to memory (coordinates, column runs, candidates).  The
+    // wavefront takes NBL_APW atoms: all their coordinates are loaded first, and the column runs of
+    // the next atom are requested before the candidates of the current one are scanned.
+    T cs[NBL_APW][3];
+#pragma unroll
+    for (int a = 0; a < NBL_APW; a++)
+#pragma unroll
+        for (int d = 0; d < 3; d++) cs[a][d] = x[(size_t)min(p0 + a, g.N - 1) * 3 + d];
+    const int nruns = (2 * g.ext_bins + 1) * (2 * g.ext_bins + 1);
+    int start, len;
+    column_setup<T>(g, cs[0], lane, offsets, start, len);
+#pragma unroll
+    for (int ia = 0; ia < NBL_APW; ia++) {
+    if (ia >= np) break;                          // wave-uniform
+    const int p = p0 + ia;
+    const T (&c)[3] = cs[ia];
+    int nstart = 0, nlen = 0;
+    if (ia + 1 < NBL_APW && ia + 1 < np) column_setup<T>(g, cs[ia + 1 < NBL_APW ? ia + 1 : ia], lane, offsets, nstart, nlen);
     const int incl = wave_inclusive_scan(len);
     const int total = __shfl(incl, 63, 64);
     const int base = incl - len;
@@ -471,13 +496,17 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
         const int nv = (int)((size_t)live * 3 * sizeof(T) / 16);
         for (int i = lane; i < nv; i += 64) d2[i] = s2[i];
-        return;
+    } else {
+        // padding: -1 / 0 (neighborList.h:557, 563)
+        const int first_pad = min(cnt, umax);
+        const int last_pad = max(first_pad, old_len);
+        pad_fill(firstneigh + rowi, first_pad, last_pad, -1, lane);
+        pad_fill(rcs + rowi * 3, first_pad * 3, last_pad * 3, (T)0, lane);
     }
-    // padding: -1 / 0 (neighborList.h:557, 563)
-    const int first_pad = min(cnt, umax);
-    const int last_pad = max(first_pad, old_len);
-    pad_fill(firstneigh + rowi, first_pad, last_pad, -1, lane);
-    pad_fill(rcs + rowi * 3, first_pad * 3, last_pad * 3, (T)0, lane);
+    start = nstart;
+    len = nlen;
+    __builtin_amdgcn_wave_barrier();              // the LDS arrays are reused by the next atom
+    }
 }
 
 // ---- 7. distance sort, emulating libstdc++ std::sort(indices, cmp = d[a] < d[b]) --------------
@@ -836,7 +865,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
                        (int)nregion, offsets, s_idx, s_x, g.N);
     prof_end(stream);
-    const int list_blocks = ceil_div(N, NBL_BLOCK / 64);
+    const int list_blocks = ceil_div(N, (NBL_BLOCK / 64) * NBL_APW);
     prof_begin("nbl_lists", stream);
     const size_t rows_lds = rowbuf_bytes<T>(umax) * (NBL_BLOCK / 64);
     const bool rowbuf = !sort && umax % 4 == 0 && rows_lds <= 32 * 1024 && (uintptr_t)firstneigh % 16 == 0 &&
@@ -860,7 +889,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                            keys, order);
         prof_end(stream);
         prof_begin("nbl_gather_rows", stream);
-        hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, N, umax,
+        hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(ceil_div(N, NBL_BLOCK / 64)), dim3(NBL_BLOCK), 0, stream, N, umax,
                            numneigh, order, tmp_first, tmp_rcs, firstneigh, rcs);
         prof_end(stream);
     }
