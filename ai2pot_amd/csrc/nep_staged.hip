@@ -28,6 +28,8 @@
 #include "a2p_common.h"
 #include "nep_device.h"
 
+#include <type_traits>
+
 namespace a2p {
 using namespace nepdev;
 namespace {
@@ -319,7 +321,7 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
 
 template <typename T, int NTC>
 __global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
-nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict__ ang_xyz,
+nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, int spare, const T* __restrict__ ang_xyz,
                   const unsigned* __restrict__ typew, const T* __restrict__ radial, const int* __restrict__ counts)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -371,16 +373,43 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
         for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
     __syncthreads();
 
-    // angular moments over the back list (the next entry is in flight while one is processed)
-    T px = (T)0, py = (T)0, pz = (T)0;
-    int pw = 0;
-    if (n_ang > 0) ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw);
-    unsigned tw = 0u;
-    for (int e = 0; e < n_ang; e++) {
-        const T x = px, y = py, z = pz;
-        if ((e & 15) == 0) tw = tw_back[(size_t)(e >> 4) * plane];
-        const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
-        if (e + 1 < n_ang) ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
+    // Walks one of the thread's lists and calls body(valid, x, y, z, place, species) per entry.
+    // Every lane makes the same number of trips (the longest list of the wavefront, in steps of
+    // PD); a lane past the end of its own list computes on a unit vector with valid = false.  The loop body is straight-line code with one load, and in the derivative passes one
+    // store, per entry, none of them conditional: the compiler can then count the memory
+    // operations in flight and wait for the entry loaded PD entries ago without waiting for the
+    // scattered stores issued since (with conditional loads or stores it falls back to waiting
+    // for everything, and every trip would wait for the previous trip's store to be acknowledged).
+    const int last_word = (a.U + 15) / 16 - 1;
+    auto walk = [&](auto depth, int n, bool front, const unsigned* __restrict__ words, auto&& body) __attribute__((always_inline)) {
+        constexpr int PD = decltype(depth)::value;
+        const int trips = __builtin_amdgcn_readfirstlane(wave_max(n));
+        if (trips == 0) return;
+        T qx[PD], qy[PD], qz[PD];
+        int qw[PD];
+#pragma unroll
+        for (int d = 0; d < PD; d++)
+            ang_load(lxyz + (size_t)(front ? d : back - d) * FB * 4, qx[d], qy[d], qz[d], qw[d]);
+        unsigned tw = words[0], twn = 0u;
+        for (int e0 = 0; e0 < trips; e0 += PD) {
+            if ((e0 & 15) == 0 && e0 > 0) tw = twn;
+            twn = words[(size_t)min((e0 >> 4) + 1, last_word) * plane];
+#pragma unroll
+            for (int d = 0; d < PD; d++) {
+                const int e = e0 + d;
+                // past the end of the list: a harmless unit vector instead of whatever the slot holds
+                const bool valid = e < n;
+                const T x = valid ? qx[d] : (T)1, y = valid ? qy[d] : (T)0, z = valid ? qz[d] : (T)0;
+                const int place = qw[d];
+                const int nxt = min(e + PD, back);
+                ang_load(lxyz + (size_t)(front ? nxt : back - nxt) * FB * 4, qx[d], qy[d], qz[d], qw[d]);
+                body(valid, x, y, z, place, min((int)((tw >> (2 * (e & 15))) & 3u), nt - 1));
+            }
+        }
+    };
+
+    // angular moments over the back list
+    walk(std::integral_constant<int, (sizeof(T) == 4 ? 2 : 1)>{}, n_ang, false, tw_back, [&](bool valid, T x, T y, T z, int, int tj) __attribute__((always_inline)) {
         const T r = sqrt_t(x * x + y * y + z * z);
         const T rinv = (T)1 / r;
         T f[KC], df[KC];
@@ -398,10 +427,11 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
             for (int k = 0; k < 4; k++) g += c0v[k] * f[k];
 #pragma unroll
             for (int k = 0; k < 4; k++) g += c1v[k] * f[4 + k];
+            g = valid ? g : (T)0;
 #pragma unroll
             for (int m = 0; m < NLM; m++) S[n][m] += g * bl[m];
         }
-    }
+    });
 
     // ---- descriptors --------------------------------------------------------------------------
     T q[DC];
@@ -506,82 +536,77 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, const T* __restrict
 #pragma unroll
             for (int k = 0; k < KC; k++) L.acc[(t * KC + k) * FB + tid] = cc[k];
         }
-        auto emit = [&](int pos, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
-            if (seg_g) {
-                T* dst = seg_g + (size_t)pos * 3;
+        // one pair: its derivative goes into the target's segment (STORE) and into the thread's sums;
+        // an entry past the end of the list stores into the spare entry and adds zeros
+        auto emit = [&](auto store, bool valid, int place, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
+            if (decltype(store)::value) {
+                T* dst = seg_g + (size_t)(valid ? place : spare) * 3;
                 dst[0] = gx; dst[1] = gy; dst[2] = gz;
             }
+            gx = valid ? gx : (T)0; gy = valid ? gy : (T)0; gz = valid ? gz : (T)0;
             fx += gx; fy += gy; fz += gz;
             vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
             vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
             vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
         };
-        // radial-only pairs (front list)
-        if (n_rad > 0) ang_load(lxyz, px, py, pz, pw);
-        for (int e = 0; e < n_rad; e++) {
-            const T x = px, y = py, z = pz;
-            const int pos = pw;
-            if ((e & 15) == 0) tw = tw_front[(size_t)(e >> 4) * plane];
-            const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
-            if (e + 1 < n_rad) ang_load(lxyz + (size_t)(e + 1) * FB * 4, px, py, pz, pw);
-            const T r = sqrt_t(x * x + y * y + z * z);
-            T f[KC], df[KC];
-            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
-            T sr = (T)0;
-#pragma unroll
-            for (int k = 0; k < KC; k++) sr += L.acc[(tj * KC + k) * FB + tid] * df[k];
-            sr /= r;
-            emit(pos, x, y, z, sr * x, sr * y, sr * z);
-        }
-        // pairs inside the angular cutoff, radial and angular part together (back list)
-        if (n_ang > 0) ang_load(lxyz + (size_t)back * FB * 4, px, py, pz, pw);
-        for (int e = 0; e < n_ang; e++) {
-            const T x = px, y = py, z = pz;
-            const int pos = pw;
-            if ((e & 15) == 0) tw = tw_back[(size_t)(e >> 4) * plane];
-            const int tj = (int)((tw >> (2 * (e & 15))) & 3u);
-            if (e + 1 < n_ang) ang_load(lxyz + (size_t)(back - e - 1) * FB * 4, px, py, pz, pw);
-            const T r = sqrt_t(x * x + y * y + z * z);
-            const T rinv = (T)1 / r;
-            const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
-            T f[KC], df[KC];
-            T srad = (T)0;
-            if (r <= rr) {
+        auto pass2 = [&](auto store) __attribute__((always_inline)) {
+            // radial-only pairs (front list)
+            walk(std::integral_constant<int, (sizeof(T) == 4 ? 4 : 2)>{}, n_rad, true, tw_front, [&](bool valid, T x, T y, T z, int place, int tj) __attribute__((always_inline)) {
+                const T r = sqrt_t(x * x + y * y + z * z);
+                T f[KC], df[KC];
                 radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+                T sr = (T)0;
 #pragma unroll
-                for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * FB + tid] * df[k];
-            }
-            radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
-            const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
-            T A[NLM], Ad[NLM];
+                for (int k = 0; k < KC; k++) sr += L.acc[(tj * KC + k) * FB + tid] * df[k];
+                sr /= r;
+                emit(store, valid, place, x, y, z, sr * x, sr * y, sr * z);
+            });
+            // pairs inside the angular cutoff, radial and angular part together (back list)
+            walk(std::integral_constant<int, (sizeof(T) == 4 ? 2 : 1)>{}, n_ang, false, tw_back, [&](bool valid, T x, T y, T z, int place, int tj) __attribute__((always_inline)) {
+                const T r = sqrt_t(x * x + y * y + z * z);
+                const T rinv = (T)1 / r;
+                const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+                T f[KC], df[KC];
+                T srad = (T)0;
+                if (r <= rr) {
+                    radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
 #pragma unroll
-            for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
-#pragma unroll
-            for (int n = 0; n < NAC; n++) {
-                T c0v[4], c1v[4];
-                lds_load4(c + n * KC, c0v);
-                lds_load4(c + n * KC + 4, c1v);
-                T g = (T)0, dg = (T)0;
-#pragma unroll
-                for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
-#pragma unroll
-                for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
-#pragma unroll
-                for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
-            }
-            T bl[NLM];
-            blm_values<T, LC>(ux, uy, uz, bl);
-#pragma unroll
-            for (int l = 1; l <= LC; l++)
-#pragma unroll
-                for (int mp = 0; mp < 2 * l + 1; mp++) {
-                    const int m = l * l - 1 + mp;
-                    srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+                    for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * FB + tid] * df[k];
                 }
-            T wx = (T)0, wy = (T)0, wz = (T)0;
-            blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
-            emit(pos, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
-        }
+                radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+                const T* c = L.coef + ((ti * nt + tj) * NB + NRC) * KC;
+                T A[NLM], Ad[NLM];
+#pragma unroll
+                for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
+#pragma unroll
+                for (int n = 0; n < NAC; n++) {
+                    T c0v[4], c1v[4];
+                    lds_load4(c + n * KC, c0v);
+                    lds_load4(c + n * KC + 4, c1v);
+                    T g = (T)0, dg = (T)0;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
+#pragma unroll
+                    for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
+                }
+                T bl[NLM];
+                blm_values<T, LC>(ux, uy, uz, bl);
+#pragma unroll
+                for (int l = 1; l <= LC; l++)
+#pragma unroll
+                    for (int mp = 0; mp < 2 * l + 1; mp++) {
+                        const int m = l * l - 1 + mp;
+                        srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+                    }
+                T wx = (T)0, wy = (T)0, wz = (T)0;
+                blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
+                emit(store, valid, place, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
+            });
+        };
+        if (seg_g) pass2(std::true_type{});
+        else pass2(std::false_type{});
         if (active && a.force) {
             T* fo = a.force + ((size_t)b * NF + center) * 3;
             fo[0] = fx; fo[1] = fy; fo[2] = fz;
@@ -641,7 +666,7 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
     prof_begin("nep_staged_kernel", stream);
-    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, (T*)csr.seg_g, (const T*)ang_xyz,
+    hipLaunchKernelGGL(kern, dim3(a.nblocks, a.B), dim3(FB), lds, stream, a, (T*)csr.seg_g, seg.spare, (const T*)ang_xyz,
                        (const unsigned*)typew, (const T*)radial, (const int*)counts);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
