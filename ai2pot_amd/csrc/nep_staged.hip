@@ -116,39 +116,55 @@ struct SegArgs {
 // Stage slots [c0, c0 + SCH) of the workgroup's rows: thread e handles row e / SCH, slot e % SCH,
 // so SCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
 // row's end (or with an index out of range) are stored far outside every cutoff.
+// Three phases, each over all SCH entries of the thread, so that the loads of the entries overlap:
+// neighbour indices and vectors; species gathers and segment atomics; LDS stores.  (Letting the
+// atomics of the entries overlap as well needs more registers than it gains: their rate, not
+// their latency, is what the kernel waits for.)
 template <typename T>
 __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& seg, const StageLds<T>& L,
                                             int tid, int c0, size_t rowbase, int b, int NF)
 {
     const int* types = a.btypes + (size_t)b * NF;
+    int nj[SCH], w[SCH], pos[SCH];
+    T x[SCH], y[SCH], z[SCH];
+    bool have[SCH];
+#pragma unroll
+    for (int it = 0; it < SCH; it++) {
+        const int e = it * SB + tid;
+        const int la = e / SCH, slot = c0 + e % SCH;
+        have[it] = slot < L.nn[la];
+        // a slot past the row's end reads the row's first slot instead (always inside the arrays)
+        const size_t pr = (rowbase + la) * a.U + (have[it] ? slot : 0);
+        const T* p = a.brcs + pr * 3;
+        nj[it] = a.bfirstneigh[pr];
+        x[it] = p[0]; y[it] = p[1]; z[it] = p[2];
+    }
+    int err = 0;
+#pragma unroll
+    for (int it = 0; it < SCH; it++) {
+        w[it] = 0; pos[it] = 0;
+        if (have[it] && (unsigned)nj[it] >= (unsigned)NF) { err |= ST_BAD_NEIGHBOR; have[it] = false; }
+        const int njc = have[it] ? nj[it] : 0;
+        w[it] = types[njc];
+        if (have[it] && seg.cursor) {
+            const int t = b * NF + njc;
+            const int rk = atomicAdd(&seg.cursor[t], 1);
+            pos[it] = rk < seg.cap ? t * seg.cap + rk : seg.spare;
+            if (rk >= seg.cap) err |= ST_NEIGH_OVERFLOW;
+        }
+    }
 #pragma unroll
     for (int it = 0; it < SCH; it++) {
         const int e = it * SB + tid;
         const int la = e / SCH, s = e % SCH;
-        const int slot = c0 + s;
-        T x = (T)1.0e18, y = (T)0, z = (T)0;
-        int w = 0, pos = 0;
-        if (slot < L.nn[la]) {
-            const size_t pr = (rowbase + la) * a.U + slot;
-            const T* p = a.brcs + pr * 3;
-            const int nj = a.bfirstneigh[pr];
-            if ((unsigned)nj >= (unsigned)NF) {
-                atomicOr(a.status, ST_BAD_NEIGHBOR);
-            } else {
-                x = p[0]; y = p[1]; z = p[2];
-                w = types[nj];
-                if (seg.cursor) {
-                    const int t = b * NF + nj;
-                    const int rk = atomicAdd(&seg.cursor[t], 1);
-                    pos = rk < seg.cap ? t * seg.cap + rk : seg.spare;
-                    if (rk >= seg.cap) atomicOr(a.status, ST_NEIGH_OVERFLOW);
-                }
-                if ((unsigned)w >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); w = 0; }
-            }
-        }
-        L.x[s * SLS + la] = x; L.y[s * SLS + la] = y; L.z[s * SLS + la] = z;
-        L.w[s * SLS + la] = (unsigned char)w; L.p[s * SLS + la] = pos;
+        if (have[it] && (unsigned)w[it] >= (unsigned)a.ntypes) { err |= ST_BAD_TYPE; w[it] = 0; }
+        L.x[s * SLS + la] = have[it] ? x[it] : (T)1.0e18;
+        L.y[s * SLS + la] = have[it] ? y[it] : (T)0;
+        L.z[s * SLS + la] = have[it] ? z[it] : (T)0;
+        L.w[s * SLS + la] = (unsigned char)(have[it] ? w[it] : 0);
+        L.p[s * SLS + la] = pos[it];
     }
+    if (err) atomicOr(a.status, err);
 }
 
 // Bit masks of a thread's staged entries: bit s of mA set when entry s lies inside the angular
@@ -211,7 +227,7 @@ __device__ __forceinline__ void row_header(const NepArgs<T>& a, bool active, siz
 // NTC*KC), list lengths (counts[0][row] radial-only, counts[1][row] inside the angular cutoff),
 // the two compact lists, and zeros in the reduction segments for pairs beyond both cutoffs.
 template <typename T, int NTC>
-__global__ void __launch_bounds__(SB, (sizeof(T) == 4 ? 4 : 2))
+__global__ void __launch_bounds__(SB, (sizeof(T) == 4 ? 3 : 2))
 nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T* __restrict__ ang_xyz,
                  unsigned* __restrict__ typew, T* __restrict__ radial, int* __restrict__ counts)
 {
