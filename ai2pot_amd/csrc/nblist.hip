@@ -156,9 +156,12 @@ __global__ void minmax_finish_kernel(const T* __restrict__ partial, int nblocks,
     const int q = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool is_min = (q % 6) < 3;
     T r = is_min ? (T)INT_MAX : (T)INT_MIN;
-    for (int k = lane; k < nblocks; k += 64) {
-        const T o = partial[(size_t)k * 12 + q];
-        r = is_min ? (o < r ? o : r) : (o > r ? o : r);
+    for (int k0 = lane; k0 < nblocks; k0 += 64 * 8) {
+        T o[8];                                    // eight loads in flight
+#pragma unroll
+        for (int u = 0; u < 8; u++) o[u] = partial[(size_t)min(k0 + 64 * u, nblocks - 1) * 12 + q];
+#pragma unroll
+        for (int u = 0; u < 8; u++) r = is_min ? (o[u] < r ? o[u] : r) : (o[u] > r ? o[u] : r);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
