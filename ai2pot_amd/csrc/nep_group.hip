@@ -10,8 +10,8 @@
 //   * GL = 8 lanes work on one atom, a wave on 8 atoms, a workgroup of 256 threads on 32;
 //   * a wave reads the rows of its atoms one after the other with lane = slot, i.e. whole rows
 //     as contiguous, fully used cache lines, exactly once; the same lanes gather the
-//     neighbour's species and the pair's place in its target's reduction segment
-//     (a2p::PairCsr ranks), classify the pair against the two cutoffs and compact the row with
+//     neighbour's species and claim the pair's place in its target's reduction segment with an
+//     integer atomic (a2p::PairCsr, fixed-capacity segments), classify the pair against the two cutoffs and compact the row with
 //     wave ballots into LDS: pairs inside the angular cutoff from the front of the atom's
 //     tile, radial-only pairs from the back;
 //   * the tile stays in LDS for both passes (rows longer than the tile are processed in
@@ -134,8 +134,9 @@ __host__ __device__ __forceinline__ size_t group_lds_layout(int ntypes, int H, i
 }
 
 struct SegArgs {
-    const int* offsets;   // [B * NF] start of each target's segment, or null (no forces wanted)
-    const int* rank;      // [B*P, U] place of each pair inside its target's segment
+    int* cursor;   // [B * NF] entries claimed so far in each target's reduction segment, or null (no forces)
+    int cap;       // capacity of a segment
+    int spare;     // entry that takes what overflows a segment
 };
 
 // Load slots [t*CAP, (t+1)*CAP) of the rows of the wave's 8 atoms (lane = slot) and compact them
@@ -145,7 +146,7 @@ struct SegArgs {
 template <typename T>
 __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& seg, T* __restrict__ seg_g,
                                           const GroupLds<T>& L, int t, int lane, int wave, size_t wave_row0, int b,
-                                          int NF, int nn, T rr, T ra, int& nA, int& nR)
+                                          int NF, int nn, T rr, T ra, int& nA, int& nR, bool claim)
 {
     constexpr int CAP = Tile<T>::CAP, CAPP = Tile<T>::CAPP;
     const int* types = a.btypes + (size_t)b * NF;
@@ -168,7 +169,13 @@ __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& se
                 const T* p = a.brcs + pr * 3;
                 x = p[0]; y = p[1]; z = p[2];
                 tj = types[nj];
-                if (seg.offsets) pos = seg.offsets[(size_t)b * NF + nj] + seg.rank[pr];
+                if (seg.cursor && claim) {
+                    // fixed-capacity segments: the pair claims its entry here (a2p::PairCsr)
+                    const int tg = b * NF + nj;
+                    const int rk = atomicAdd(&seg.cursor[tg], 1);
+                    pos = rk < seg.cap ? tg * seg.cap + rk : seg.spare;
+                    if (rk >= seg.cap) atomicOr(a.status, ST_NEIGH_OVERFLOW);
+                }
                 if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
             }
         }
@@ -182,7 +189,7 @@ __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& se
             const int k = inA ? __popcll(mA & lt) : CAP - 1 - __popcll(mR & lt);
             ent_store(ent + k * 4, x, y, z, tj);
             epos[k] = pos;
-        } else if (valid && seg_g) {
+        } else if (valid && seg_g && claim) {
             // a pair of the list beyond both cutoffs still owns a place in its segment
             T* dst = seg_g + (size_t)pos * 3;
             dst[0] = (T)0; dst[1] = (T)0; dst[2] = (T)0;
@@ -253,7 +260,9 @@ nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
     int nA = 0, nR = 0;
     for (int t = 0; t < ntiles; t++) {
         if (t > 0) __builtin_amdgcn_wave_barrier();
-        load_tile<T>(a, seg, seg_g, L, t, lane, wave, wave_row0, b, NF, nn, rr, ra, nA, nR);
+        // a tile is loaded once when the rows fit one tile and again in pass 2 otherwise: the pairs
+        // claim their segment entries in the last load
+        load_tile<T>(a, seg, seg_g, L, t, lane, wave, wave_row0, b, NF, nn, rr, ra, nA, nR, ntiles == 1);
         for (int k = sub; k < nA; k += GL) {
             T x, y, z;
             int tj;
@@ -423,7 +432,7 @@ nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
         for (int t = 0; t < ntiles; t++) {
             if (ntiles > 1) {      // the tiles of pass 1 are gone: read the rows again
                 __builtin_amdgcn_wave_barrier();
-                load_tile<T>(a, seg, nullptr, L, t, lane, wave, wave_row0, b, NF, nn, rr, ra, nA, nR);
+                load_tile<T>(a, seg, seg_g, L, t, lane, wave, wave_row0, b, NF, nn, rr, ra, nA, nR, true);
             }
             // pairs inside the angular cutoff, radial and angular part together
             for (int k = sub; k < nA; k += GL) {
@@ -526,7 +535,7 @@ nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
 template <typename T, int NTC>
 int launch_group(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
 {
-    SegArgs seg{csr.offsets, csr.rank};
+    SegArgs seg{csr.cursor, csr.seg_cap, csr.n * csr.seg_cap};
     auto kern = nep_group_kernel<T, NTC>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -561,7 +570,7 @@ int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     if (a.force) {
         rc = fill_zero(a.force, (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), stream);
         if (rc) return rc;
-        rc = pair_csr_begin<T>(&csr, true, a.B, a.P, a.U, a.nghost, a.binum, a.bnumneigh, a.bfirstneigh, stream);
+        rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream);
         if (rc) return rc;
     }
     switch (ntc_of(a.ntypes)) {
