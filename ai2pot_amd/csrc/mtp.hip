@@ -14,7 +14,7 @@
 //   adjoint       : seed + reverse gather                                  (linearMtp.h:292-306)
 //   pair forces   : lane <- (neighbour, half of the basic moments):
 //                   dE_i/dr_ij = u sum_i adj_i m_i (g' - k g / r) + (1/r) sum_i adj_i g grad_u m_i
-//                   -> pair buffer, folded onto neighbours by a2p::pair_reduce (no float atomics)
+//                   -> reduction segments of the neighbours (a2p::PairCsr), summed without float atomics
 // The loss gradient adds the tangent sweep (include/linearMtpLoss.h:371-398), the mixed
 // adjoint (:417-434) and the coefficient-gradient pass (:438-536) in the same structure;
 // per-structure gradients are accumulated per workgroup and summed by a second kernel.
@@ -47,7 +47,9 @@ struct MtpArgs {
     const T* brcs;
     const int* btypes;
     T* force;          // [B, P+nghost, 3]
-    T* pair_g;         // [B*P, U, 3]
+    int* seg_cursor;   // reduction segments of fixed capacity U (a2p::PairCsr): entries claimed per target,
+    T* seg_g;          // the entries, and the entry that takes what overflows a segment;
+    int seg_spare;     // seg_cursor is null when no forces are wanted
     double* partial;   // [B, P, 10]  energy + virial per atom
     int* status;
     int E;             // table entries per neighbour
@@ -440,7 +442,6 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         T vir[9];
 #pragma unroll
         for (int q = 0; q < 9; q++) vir[q] = (T)0;
-        T* grow = a.pair_g + row * a.U * 3;
         const int nchunks = (nn + MTP_NC - 1) / MTP_NC;
         const int csize = nchunks > 0 ? (nn + nchunks - 1) / nchunks : 1;
         for (int c0 = 0; c0 < nn; c0 += csize) {
@@ -489,8 +490,15 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                 T gy = gs * t[OU + 1] + wy * rinv;
                 T gz = gs * t[OU + 2] + wz * rinv;
                 if (!valid) { gx = (T)0; gy = (T)0; gz = (T)0; }
-                const int jj = c0 + j;
-                grow[jj * 3 + 0] = gx; grow[jj * 3 + 1] = gy; grow[jj * 3 + 2] = gz;
+                if (a.seg_cursor && j < nc) {
+                    // the pair claims an entry of its target's segment (zeros too: the count of a segment
+                    // is the number of pairs naming the target)
+                    const int tg = b * NF + nj;
+                    const int rk = atomicAdd(&a.seg_cursor[tg], 1);
+                    T* dst = a.seg_g + (size_t)(rk < a.U ? tg * a.U + rk : a.seg_spare) * 3;
+                    if (rk >= a.U) atomicOr(a.status, ST_NEIGH_OVERFLOW);
+                    dst[0] = gx; dst[1] = gy; dst[2] = gz;
+                }
                 fx += gx; fy += gy; fz += gz;
                 vir[0] -= gx * d[0]; vir[1] -= gx * d[1]; vir[2] -= gx * d[2];
                 vir[3] -= gy * d[0]; vir[4] -= gy * d[1]; vir[5] -= gy * d[2];
@@ -958,7 +966,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.binum = binum; a.bilist = bilist; a.bnumneigh = bnumneigh; a.bfirstneigh = bfirstneigh;
     a.brcs = brcs; a.btypes = btypes;
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
-    a.force = nullptr; a.pair_g = nullptr; a.partial = nullptr;
+    a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.partial = nullptr;
     a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
     a.nn_exact = 1;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
@@ -1055,15 +1063,20 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
         if (rc) return rc;
         a.force = (T*)ws;
     }
-    rc = ws_get(WS_PAIR_G, (size_t)B * P * U * 3 * sizeof(T), &ws);
-    if (rc) return rc;
-    a.pair_g = (T*)ws;
     rc = fill_zero(a.force, force_bytes, stream);      // the reference zeroes on entry, linearMtp.h:228-230
     if (rc) return rc;
+    PairCsr csr{};
+    if (force) {
+        rc = pair_fixed_begin<T>(&csr, B, P, U, nghost, stream);
+        if (rc) return rc;
+        a.seg_cursor = csr.cursor;
+        a.seg_g = (T*)csr.seg_g;
+        a.seg_spare = csr.n * csr.seg_cap;
+    }
     rc = launch_atoms<T, false>(a, stream);
     if (rc) return rc;
     if (force) {
-        rc = pair_reduce<T>(force, a.pair_g, B, P, U, nghost, binum, bnumneigh, bfirstneigh, stream);
+        rc = pair_csr_finish<T>(force, csr, stream);
         if (rc) return rc;
     }
     if (etot) {
