@@ -152,8 +152,11 @@ struct PairCsr {
 template <typename T>
 int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost, const int* binum,
                    const int* bnumneigh, const int* bfirstneigh, hipStream_t stream);
+// also_zero / also_bytes: a second range cleared by the same launch that clears the cursors
+// (the force array of the caller, as a rule)
 template <typename T>
-int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream);
+int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero = nullptr,
+                     size_t also_bytes = 0);
 template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);
 
@@ -163,7 +166,13 @@ template <typename T>
 int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
                     int out_stride, hipStream_t stream);
 
+// etot[b] and virial[b*9 + c] from partial[(b*nblocks + block)*10 + (0 | 1 + c)], one launch; either
+// output may be null.
+template <typename T>
+int finish_energy_virial(T* etot, T* virial, const double* partial, int B, int nblocks, hipStream_t stream);
+
 int fill_zero(void* ptr, size_t bytes, hipStream_t stream);
+int fill_zero2(void* ptr, size_t bytes, void* ptr2, size_t bytes2, hipStream_t stream);   // two ranges, one launch
 
 // out[i] = in[0] + ... + in[i-1] for i < n (out must not alias in); tmp holds
 // scan_tmp_ints(n) ints, and tmp[ceil(n/2048)] receives the total.

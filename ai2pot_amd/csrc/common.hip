@@ -115,6 +115,29 @@ __global__ void fill_zero_kernel(uint32_t* p, size_t nwords)
     for (; i < nwords; i += stride) p[i] = 0u;
 }
 
+__global__ void fill_zero2_kernel(uint32_t* p, size_t nwords, uint32_t* q, size_t mwords)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t k = i; k < nwords; k += stride) p[k] = 0u;
+    for (size_t k = i; k < mwords; k += stride) q[k] = 0u;
+}
+
+int fill_zero2(void* ptr, size_t bytes, void* ptr2, size_t bytes2, hipStream_t stream)
+{
+    if (bytes == 0) return fill_zero(ptr2, bytes2, stream);
+    if (bytes2 == 0) return fill_zero(ptr, bytes, stream);
+    A2P_REQUIRE(bytes % 4 == 0 && bytes2 % 4 == 0, A2P_ERR_INVALID, "fill_zero: size not a multiple of 4");
+    const size_t nwords = bytes / 4, mwords = bytes2 / 4;
+    const int blocks = (int)std::min<size_t>((std::max(nwords, mwords) + 255) / 256, 256 * 32);
+    prof_begin("fill_zero", stream);
+    hipLaunchKernelGGL(fill_zero2_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t*)ptr, nwords,
+                       (uint32_t*)ptr2, mwords);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
 int fill_zero(void* ptr, size_t bytes, hipStream_t stream)
 {
     if (bytes == 0) return A2P_OK;
@@ -159,6 +182,41 @@ int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
+// Energy (component 0) and virial (components 1-9) of partial[.., 10] in one launch; either output
+// may be null.  Same summation per component as finish_partials.
+template <typename T>
+__global__ void finish_ev_kernel(T* etot, T* virial, const double* partial, int nblocks)
+{
+    __shared__ double sh[256];
+    const int b = blockIdx.y, c = blockIdx.x;
+    if (c == 0 ? etot == nullptr : virial == nullptr) return;      // uniform over the workgroup
+    const double* src = partial + ((size_t)b * nblocks) * 10 + c;
+    double acc = 0.0;
+    for (int k = threadIdx.x; k < nblocks; k += 256) acc += src[(size_t)k * 10];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (c == 0) etot[b] = (T)sh[0];
+        else virial[(size_t)b * 9 + c - 1] = (T)sh[0];
+    }
+}
+
+template <typename T>
+int finish_energy_virial(T* etot, T* virial, const double* partial, int B, int nblocks, hipStream_t stream)
+{
+    if (!etot && !virial) return A2P_OK;
+    prof_begin("finish_partials", stream);
+    hipLaunchKernelGGL(finish_ev_kernel<T>, dim3(10, B), dim3(256), 0, stream, etot, virial, partial, nblocks);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+template int finish_energy_virial<float>(float*, float*, const double*, int, int, hipStream_t);
+template int finish_energy_virial<double>(double*, double*, const double*, int, int, hipStream_t);
 template int finish_partials<float>(float*, const double*, int, int, int, int, int, hipStream_t);
 template int finish_partials<double>(double*, const double*, int, int, int, int, int, hipStream_t);
 

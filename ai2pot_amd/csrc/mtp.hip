@@ -1063,15 +1063,16 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
         if (rc) return rc;
         a.force = (T*)ws;
     }
-    rc = fill_zero(a.force, force_bytes, stream);      // the reference zeroes on entry, linearMtp.h:228-230
-    if (rc) return rc;
     PairCsr csr{};
-    if (force) {
-        rc = pair_fixed_begin<T>(&csr, B, P, U, nghost, stream);
+    if (force) {       // the force array is zeroed with the cursors (the reference zeroes on entry, linearMtp.h:228-230)
+        rc = pair_fixed_begin<T>(&csr, B, P, U, nghost, stream, a.force, force_bytes);
         if (rc) return rc;
         a.seg_cursor = csr.cursor;
         a.seg_g = (T*)csr.seg_g;
         a.seg_spare = csr.n * csr.seg_cap;
+    } else {
+        rc = fill_zero(a.force, force_bytes, stream);
+        if (rc) return rc;
     }
     rc = launch_atoms<T, false>(a, stream);
     if (rc) return rc;
@@ -1079,15 +1080,7 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
         rc = pair_csr_finish<T>(force, csr, stream);
         if (rc) return rc;
     }
-    if (etot) {
-        rc = finish_partials<T>(etot, a.partial, B, P, 1, 10, 1, stream);
-        if (rc) return rc;
-    }
-    if (virial) {
-        rc = finish_partials<T>(virial, a.partial + 1, B, P, 9, 10, 9, stream);
-        if (rc) return rc;
-    }
-    return A2P_OK;
+    return finish_energy_virial<T>(etot, virial, a.partial, B, P, stream);
 }
 
 template <typename T>

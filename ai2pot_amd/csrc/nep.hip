@@ -480,15 +480,7 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
             if (rc) return rc;
         }
     }
-    if (etot) {
-        rc = finish_partials<T>(etot, a.partial, B, a.nblocks, 1, 10, 1, stream);
-        if (rc) return rc;
-    }
-    if (virial) {
-        rc = finish_partials<T>(virial, a.partial + 1, B, a.nblocks, 9, 10, 9, stream);
-        if (rc) return rc;
-    }
-    return A2P_OK;
+    return finish_energy_virial<T>(etot, virial, a.partial, B, a.nblocks, stream);
 }
 
 }  // namespace

@@ -568,9 +568,8 @@ int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     PairCsr csr{};
     int rc;
     if (a.force) {
-        rc = fill_zero(a.force, (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), stream);
-        if (rc) return rc;
-        rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream);
+        rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream, a.force,
+                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T));
         if (rc) return rc;
     }
     switch (ntc_of(a.ntypes)) {
