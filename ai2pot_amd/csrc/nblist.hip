@@ -825,9 +825,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     int* offsets = counts + nb1;
     int* cursor = offsets + nb1;
     int* tmp = cursor + nb1;
-    rc = fill_zero(counts, (size_t)nb1 * sizeof(int), stream);
-    if (rc) return rc;
-    rc = fill_zero(cursor, (size_t)nb1 * sizeof(int), stream);
+    rc = fill_zero2(counts, (size_t)nb1 * sizeof(int), cursor, (size_t)nb1 * sizeof(int), stream);
     if (rc) return rc;
     const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
     prof_begin("nbl_count", stream);
