@@ -110,6 +110,18 @@ def test_config3_reduced_and_ghosts(oracle):
     assert close(eg, er) and close(fg, fr) and close(vg, vr)
 
 
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_reproducible(oracle, np_dtype):
+    """Two runs give bit-identical results: the pairs claim their segment entries in an order that
+    changes from run to run, the sums over a segment do not depend on it."""
+    nb = synth.pack_batch([structure(oracle, 400, (20.0, 21.0, 19.0), 2, 31, 5.0)])
+    m = synth.mtp_model(mtp_param.mtp_param(10), 2, 8, 5.0, 0.5, 3032, lo=-0.05, hi=0.05)
+    a = gpu_efv(m, nb, np_dtype)
+    b = gpu_efv(m, nb, np_dtype)
+    for x, y in zip(a, b):
+        assert np.array_equal(x.view(np.uint8), y.view(np.uint8))
+
+
 def test_fp32_runs_close_to_fp64(oracle):
     o = structure(oracle, 40, (8.5, 9.0, 9.5), 2, 21, 5.0)
     nb = synth.pack_batch([o])

@@ -77,12 +77,12 @@ def test_row_capacities(oracle, dt, umax):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-@pytest.mark.parametrize("umax", [56, 54, 2000])
-def test_update_in_place(oracle, dt, umax):
+@pytest.mark.parametrize("umax,sort", [(56, False), (54, False), (2000, False), (56, True)])
+def test_update_in_place(oracle, dt, umax, sort):
     """a2p_nblist_update_* into buffers that hold an earlier list: after every step the whole
     arrays, padding included, are those of a fresh build.  The atoms move far enough between the
     steps for rows to grow and to shrink; the three capacities take the LDS row buffer, the
-    direct stores and the rows too large for the buffer."""
+    direct stores and the rows too large for the buffer; the sorted list is rebuilt in full."""
     import ctypes as c
     import torch
     from ai2pot_amd import _lib
@@ -109,13 +109,13 @@ def test_update_in_place(oracle, dt, umax):
         coords = torch.from_numpy(p).to(dev)
         fn = build if step == 0 else update
         rc = fn(lat_h.ctypes.data_as(c.c_void_p), vp(t_types), vp(coords), c.c_int(n), c.c_double(5.0),
-                c.c_int(umax), c.c_int(1), pbc.ctypes.data_as(c.c_void_p), c.c_int(0), vp(ilist),
+                c.c_int(umax), c.c_int(1), pbc.ctypes.data_as(c.c_void_p), c.c_int(1 if sort else 0), vp(ilist),
                 vp(numneigh), vp(first), vp(rcs), vp(types_out), None,
                 c.c_void_p(torch.cuda.current_stream().cuda_stream))
         _lib.check(rc)
         torch.cuda.synchronize()
         _lib.check_status(torch.cuda.current_stream().cuda_stream)
-        b = oracle.nblist(lat.astype(dt), types, p, 5.0, umax)
+        b = oracle.nblist(lat.astype(dt), types, p, 5.0, umax, sort=sort)
         a = (n, ilist.cpu().numpy(), numneigh.cpu().numpy(), first.cpu().numpy(), rcs.cpu().numpy(),
              types_out.cpu().numpy(), 0)
         assert_same(a, b)

@@ -188,6 +188,18 @@ def test_reproducible(oracle):
         assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
 
 
+def test_reproducible_staged_pair(oracle):
+    """The same for a system large enough for the staging + model kernel pair (40,000 atoms)."""
+    lat, pos = synth.fcc_cell(22, 4.6, 0.15, 67)
+    ty = synth.rng_randint(68, pos.shape[0], 3)
+    nb = synth.pack_batch([oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 6.0, 100)])
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    a = run_gpu(m, nb, np.float32)
+    b = run_gpu(m, nb, np.float32)
+    for x, y in zip(a, b):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+
+
 def test_errors(oracle):
     import torch
     from ai2pot_amd import ops, _lib
