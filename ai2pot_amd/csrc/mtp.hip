@@ -181,23 +181,27 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
         const int s0 = p.f_level[l], s1 = p.f_lend[l];
         const bool multi = p.f_multi[l] != 0;
         for (int s = s0 + tid; s < s1; s += NT) {
-            const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group
+            const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group, a multiple of 4
             const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
+            const int dst = p.f_dst[s];                      // requested with the two words above
             T acc = (T)0, tacc = (T)0;
-#pragma unroll 4
-            for (int k = 0; k < depth; k++) {
-                const int2 w = tp[k * 64];
-                const int m0 = w.x & 0xffff, m1 = (int)((unsigned)w.x >> 16);
-                const T mult = (T)w.y;
-                const T v0 = M[m0], v1 = M[m1];
-                acc += mult * v0 * v1;
-                if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+            for (int k = 0; k < depth; k += 4) {
+                int2 w[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) w[u] = tp[(k + u) * 64];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int m0 = w[u].x & 0xffff, m1 = (int)((unsigned)w[u].x >> 16);
+                    const T mult = (T)w[u].y;
+                    const T v0 = M[m0], v1 = M[m1];
+                    acc += mult * v0 * v1;
+                    if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+                }
             }
             if (multi) {
                 part[s - s0] = acc;
                 if (TANGENT) part2[s - s0] = tacc;
             } else {
-                const int dst = p.f_dst[s];
                 M[dst] = acc;
                 if (TANGENT) Tg[dst] = tacc;
             }
@@ -232,17 +236,22 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
         for (int s = s0 + tid; s < s1; s += NT) {
             const int depth = p.r_gdepth[s >> 6];
             const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
+            const int src = p.r_src[s];
             T acc = (T)0;
-#pragma unroll 4
-            for (int k = 0; k < depth; k++) {
-                const int2 w = tp[k * 64];
-                const int dst = w.x & 0xffff, other = (int)((unsigned)w.x >> 16);
-                const T mult = (T)w.y;
-                acc += X[dst] * mult * M[other];
-                if (MIXED) acc += mult * A[dst] * Tg[other];
+            for (int k = 0; k < depth; k += 4) {
+                int2 w[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) w[u] = tp[(k + u) * 64];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int dst = w[u].x & 0xffff, other = (int)((unsigned)w[u].x >> 16);
+                    const T mult = (T)w[u].y;
+                    acc += X[dst] * mult * M[other];
+                    if (MIXED) acc += mult * A[dst] * Tg[other];
+                }
             }
             if (multi) part[s - s0] = acc;
-            else X[p.r_src[s]] += acc;
+            else X[src] += acc;
         }
         __syncthreads();
         if (multi) {
@@ -809,6 +818,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
                 const size_t g1 = std::min(pieces.size(), g0 + 64);
                 int depth = 0;
                 for (size_t q = g0; q < g1; q++) depth = std::max(depth, pieces[q].n);
+                depth = (depth + 3) / 4 * 4;        // the kernels fetch four terms at a time
                 e.gbase.push_back((int)e.terms.size());
                 e.gdepth.push_back(depth);
                 e.terms.resize(e.terms.size() + (size_t)depth * 64, make_int2(0, 0));

@@ -32,7 +32,7 @@ struct MtpPlanDevice {
     // list is cut into consecutive slots (pieces) whose partial sums are added in slot order, so
     // that no lane walks a long list alone.  Slots are grouped 64 at a time; level l covers slots
     // [f_level[l], f_lend[l]) and starts at a multiple of 64.  The terms of a group are stored
-    // interleaved and padded with zero terms to the group's depth: term k of slot s is
+    // interleaved and padded with zero terms to the group's depth (a multiple of four): term k of slot s is
     // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
     // a group read consecutive words and share the trip count.  A term packs x = m0 | m1 << 16,
     // y = multiplicity.
