@@ -32,6 +32,17 @@ namespace {
 
 constexpr int MTP_NC = 32;        // neighbours per chunk (rows of the LDS table); the energy / force / virial
 constexpr int MTP_NC_MAX = 48;    // launch raises it up to MTP_NC_MAX while that costs no workgroup per CU
+
+// The group sums of the pair-derivative pass live in the moment vector when it is long enough
+// (energy / force / virial kernel only), else behind the neighbour table.
+__host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms) { return !loss && n_moms >= 1024; }
+// entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums
+__host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots)
+{
+    const int a = nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4);
+    const int b = max_level_slots * (loss ? 2 : 1);
+    return a > b ? a : b;
+}
 constexpr int MTP_NGMAX = 16;     // most thread groups that share the basic moments of a chunk
 constexpr int MTP_KMAX = 16;      // radial basis size limit
 constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
@@ -305,8 +316,11 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     T* Bm = Tg + (LOSS ? n_moms : 0);        // loss mode only
     T* cf = Bm + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
     T* tab = cf + a.ntypes * nmus * K;
-    T* gred = tab + MTP_NC * E;              // [256/32][32][4] partial sums of the thread groups
-    T* pq = tab + max(MTP_NC * E + (256 / 32) * 32 * 4, p.max_level_slots * (LOSS ? 2 : 1));              // loss mode: P[nc][nmus] | Q[nc][nmus]
+    // [256/32][32][4] partial sums of the thread groups.  The energy / force / virial kernel needs them
+    // only after the reverse sweep, when the moments are dead: a long moment vector lends them its place
+    const bool share = mtp_gred_in_moments(LOSS, n_moms);
+    T* gred = share ? M : tab + MTP_NC * E;
+    T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots);   // loss mode: P[nc][nmus] | Q[nc][nmus]
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
         if (!LOSS && a.partial && lane < 10) a.partial[row * 10 + lane] = 0.0;
@@ -435,7 +449,7 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     if (!LOSS && (a.e_sites || a.desc)) {
         if (a.desc)                                          // linearMtp.h:884-885: unscaled scalar moments
             for (int s = lane; s < p.n_scalar; s += NT) a.desc[row * p.n_scalar + s] = M[p.mapping[s]];
-        const T e_row = block_sum<T, NT>(e_part, gred, lane) + a.bias[ti];
+        const T e_row = block_sum<T, NT>(e_part, tab, lane) + a.bias[ti];      // the table is idle between the sweeps
         if (a.e_sites && lane == 0) a.e_sites[row] = e_row;  // linearMtp.h:594-599
         if (a.energy_only) return;
     }
@@ -947,7 +961,7 @@ template <typename T>
 size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC)
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
-    const size_t tabs = std::max((size_t)MTP_NC * E + (size_t)(256 / 32) * 32 * 4, (size_t)p.max_level_slots * (loss ? 2 : 1));
+    const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots);
     size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
