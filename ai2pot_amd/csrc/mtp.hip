@@ -33,9 +33,13 @@ namespace {
 constexpr int MTP_NC = 32;        // neighbours per chunk (rows of the LDS table); the energy / force / virial
 constexpr int MTP_NC_MAX = 48;    // launch raises it up to MTP_NC_MAX while that costs no workgroup per CU
 
-// The group sums of the pair-derivative pass live in the moment vector when it is long enough
-// (energy / force / virial kernel only), else behind the neighbour table.
-__host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms) { return !loss && n_moms >= 1024; }
+// The group sums of the last pass over the neighbours (four per thread for the pair derivatives, two
+// for the loss gradient) live in the moment vector (loss mode: moments and tangents) when it is long
+// enough, else behind the neighbour table.
+__host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms)
+{
+    return loss ? 2 * n_moms >= 512 : n_moms >= 1024;
+}
 // entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums
 __host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots)
 {
@@ -310,14 +314,16 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     const int ncoef = a.ntypes * a.ntypes * nmus * K;
 
     const int MTP_NC = a.nc_cap;
+    // moments | (loss mode: their tangents) | adjoints | (loss mode: mixed adjoints)
     T* M = (T*)smem_raw;
-    T* A = M + n_moms;
-    T* Tg = A + n_moms;                      // loss mode only
-    T* Bm = Tg + (LOSS ? n_moms : 0);        // loss mode only
+    T* Tg = M + n_moms;
+    T* A = Tg + (LOSS ? n_moms : 0);
+    T* Bm = A + n_moms;
     T* cf = Bm + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
     T* tab = cf + a.ntypes * nmus * K;
-    // [256/32][32][4] partial sums of the thread groups.  The energy / force / virial kernel needs them
-    // only after the reverse sweep, when the moments are dead: a long moment vector lends them its place
+    // [256/32][32][4] partial sums of the thread groups.  They are needed only in the last pass over the
+    // neighbours, when the moments (and, in loss mode, their tangents) are dead: a long enough moment
+    // vector lends them its place
     const bool share = mtp_gred_in_moments(LOSS, n_moms);
     T* gred = share ? M : tab + MTP_NC * E;
     T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots);   // loss mode: P[nc][nmus] | Q[nc][nmus]
@@ -551,6 +557,35 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
         T* grow = a.gpart + row * a.ngrad;
         for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
+        __syncthreads();         // other threads overwrite some of these entries below
+        // everything but the coefficient block is written now: the pass over the neighbours below does
+        // not read the moments or their tangents, and the group sums may take their place
+        if (a.H > 0) {
+            // compact row of the centre species: coefficient block | w0[H, S] | w1[H] | bias
+            const int S = p.n_scalar, H = a.H, nblk = a.ntypes * nmus * K;
+            const T* qv = nnb;
+            const T* n_th = nnb + S + H;
+            const T* n_d1 = n_th + H;
+            const T* n_d2 = n_d1 + H;
+            const T* n_tau = n_d2 + H;
+            const T* w1 = a.w1 + (size_t)ti * H;
+            const T* w0 = a.w0 + (size_t)ti * H * S;
+            for (int q = lane; q < H * S; q += NT) {
+                const int n = q / S, k = q - n * S;
+                const T tk = Tg[p.mapping[k]] / a.q_scaler[k];
+                if (a.nn_exact)
+                    grow[nblk + q] = w1[n] * ((cE * n_d1[n] + n_d2[n] * n_tau[n]) * qv[k] + n_d1[n] * tk);
+                else        // nnMtpLoss.h:560-585: only the k' = k term of tau
+                    grow[nblk + q] = w1[n] * (cE * n_d1[n] * qv[k] + tk * (n_d1[n] + n_d2[n] * w0[q] * qv[k]));
+            }
+            for (int n = lane; n < H; n += NT) grow[nblk + H * S + n] = cE * n_th[n] + n_d1[n] * n_tau[n];
+            if (lane == 0) grow[nblk + H * S + H] = cE;
+        } else {
+            // linear coefficients and bias: linearMtpLoss.h:539-554
+            for (int s = lane; s < p.n_scalar; s += NT)
+                grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
+            if (lane == 0) grow[ncoef + p.n_scalar + ti] = cE;
+        }
         T* Pm = pq;
         T* Qm = pq + MTP_NC * nmus;
         int* tjs = (int*)(pq + 2 * MTP_NC * nmus);
@@ -616,34 +651,11 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         }
         __syncthreads();
         if (a.H > 0) {
-            // compact row of the centre species: coefficient block | w0[H, S] | w1[H] | bias
-            const int S = p.n_scalar, H = a.H, nblk = a.ntypes * nmus * K;
-            const T* qv = nnb;
-            const T* n_th = nnb + S + H;
-            const T* n_d1 = n_th + H;
-            const T* n_d2 = n_d1 + H;
-            const T* n_tau = n_d2 + H;
-            const T* w1 = a.w1 + (size_t)ti * H;
-            for (int q = lane; q < nblk; q += NT) grow[q] = gacc[q];
-            const T* w0 = a.w0 + (size_t)ti * H * S;
-            for (int q = lane; q < H * S; q += NT) {
-                const int n = q / S, k = q - n * S;
-                const T tk = Tg[p.mapping[k]] / a.q_scaler[k];
-                if (a.nn_exact)
-                    grow[nblk + q] = w1[n] * ((cE * n_d1[n] + n_d2[n] * n_tau[n]) * qv[k] + n_d1[n] * tk);
-                else        // nnMtpLoss.h:560-585: only the k' = k term of tau
-                    grow[nblk + q] = w1[n] * (cE * n_d1[n] * qv[k] + tk * (n_d1[n] + n_d2[n] * w0[q] * qv[k]));
-            }
-            for (int n = lane; n < H; n += NT) grow[nblk + H * S + n] = cE * n_th[n] + n_d1[n] * n_tau[n];
-            if (lane == 0) grow[nblk + H * S + H] = cE;
+            for (int q = lane; q < a.ntypes * nmus * K; q += NT) grow[q] = gacc[q];
             return;
         }
         for (int q = lane; q < a.ntypes * nmus * K; q += NT)
             grow[(size_t)ti * a.ntypes * nmus * K + q] = gacc[q];
-        // linear coefficients and bias: linearMtpLoss.h:539-554
-        for (int s = lane; s < p.n_scalar; s += NT)
-            grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
-        if (lane == 0) grow[ncoef + p.n_scalar + ti] = cE;
     }
 }
 
