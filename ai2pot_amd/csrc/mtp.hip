@@ -1,9 +1,9 @@
 // Linear Moment Tensor Potential for gfx950: energy / force / virial, and the analytic
 // gradient of the training loss w.r.t. coeffs, linear_coeffs and type_bias.
 //
-// One wavefront (a 64-thread workgroup) per centre atom; the moment vector M, its adjoint
-// and (for the loss gradient) the tangent and mixed vectors live in LDS.  Neighbours are
-// processed in chunks of 32: a per-neighbour table (powers of the unit vector, contracted
+// One workgroup (64 threads, or 256 for the larger levels) per centre atom; the moment vector M,
+// its adjoint and (for the loss gradient) the tangent and mixed vectors live in LDS.  Neighbours
+// are processed in equal chunks of at most 32 to 48: a per-neighbour table (powers of the unit vector, contracted
 // radial functions g_mu(r) = sum_k c[ti,tj,mu,k] f_k(r) and their r-derivatives) is staged
 // in LDS, then
 //   basic moments : lane <- basic moment i,  M_i += sum_j g_mu(r_j) ux^a uy^b uz^c
@@ -12,7 +12,7 @@
 //   products      : level-ordered gather over the host-built plan (mtp_plan.h)
 //   energy        : E_i = bias[t] + sum_s lin[s] M[map[s]] / q_scaler[s]  (linearMtp.h:281-285)
 //   adjoint       : seed + reverse gather                                  (linearMtp.h:292-306)
-//   pair forces   : lane <- (neighbour, half of the basic moments):
+//   pair forces   : lane <- (neighbour, a share of the basic moments):
 //                   dE_i/dr_ij = u sum_i adj_i m_i (g' - k g / r) + (1/r) sum_i adj_i g grad_u m_i
 //                   -> reduction segments of the neighbours (a2p::PairCsr), summed without float atomics
 // The loss gradient adds the tangent sweep (include/linearMtpLoss.h:371-398), the mixed

@@ -4,15 +4,15 @@
 // The generic kernel (nep.hip) lets every thread walk its own neighbour row four times, so each
 // wave-wide load touches 64 different cache lines, and it holds the pair derivatives in a
 // [row, slot, 3] buffer that a separate pass copies into the reduction segments.  Here
-//   * the neighbour rows are read ONCE: the workgroup stages FCH slots of its FB rows through
-//     LDS per round with row-contiguous loads (FCH consecutive lanes per row); the loading lane
+//   * the neighbour rows are read ONCE: the workgroup stages SCH slots of its SB rows through
+//     LDS per round with row-contiguous loads (SCH consecutive lanes per row); the loading lane
 //     also gathers the neighbour's species and the pair's place in its target's reduction
 //     segment with an integer atomic (a2p::PairCsr, fixed-capacity segments);
 //   * every thread copies its staged entries into two compact per-thread lists in global
 //     scratch, laid out [entry][thread] so that the k-th entries of a wave are contiguous:
 //     radial-only neighbours from the front, neighbours inside the angular cutoff from the back.
-//     All later loops run over these dense lists with coalesced 16-byte loads, equal trip counts
-//     across a wave, no barriers and the next entry prefetched;
+//     All later loops run over these dense lists with coalesced 16-byte loads, the trip count of
+//     the longest list of the wave, no barriers and several entries in flight;
 //   * the radial functions are summed per neighbour species and contracted with the
 //     coefficients once per atom (pass 1), and the coefficients are contracted with dE/dq once
 //     per atom before the radial derivative loop (pass 2);
