@@ -352,11 +352,22 @@ nep_grad_reduce_kernel(NepLossArgs<T> a, T* __restrict__ dcoeffs, T* __restrict_
     if (!out) return;
     const int inum = a.binum[b];
     T acc = (T)0;
-    for (int ii = 0; ii < inum; ii++) {
-        const int c = a.bilist[(size_t)b * a.P + ii];
-        if ((unsigned)c >= (unsigned)a.P) continue;
-        if (a.btypes[(size_t)b * a.P + c] != t) continue;
-        acc += a.gpart[((size_t)b * a.P + ii) * a.nrow + q];
+    // eight rows in flight; the rows of other species add zero, the order of the sum is the atom order
+    for (int i0 = 0; i0 < inum; i0 += 8) {
+        int c[8], ty[8];
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) c[u] = a.bilist[(size_t)b * a.P + min(i0 + u, inum - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const bool ok = i0 + u < inum && (unsigned)c[u] < (unsigned)a.P;
+            ty[u] = a.btypes[(size_t)b * a.P + (ok ? c[u] : 0)];
+            if (!ok) ty[u] = -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = a.gpart[((size_t)b * a.P + min(i0 + u, inum - 1)) * a.nrow + q];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc += ty[u] == t ? v[u] : (T)0;
     }
     *out = acc;
 }
