@@ -833,9 +833,16 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
-    int total = 0;
-    A2P_HIP_CHECK(hipMemcpyAsync(&total, offsets + nregion, sizeof(int), hipMemcpyDeviceToHost, stream));
-    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    // Entries of the sorted image arrays.  Every (atom, image) pair can own at most one: while that
+    // bound stays below 2 GiB the arrays are simply sized for it and the host never learns the count
+    // (one synchronisation less per build); beyond, the count is read back.
+    long long total = (long long)N * g.nimg;
+    if (total * (long long)(sizeof(int) + 3 * sizeof(T)) > (2ll << 30)) {
+        int counted = 0;
+        A2P_HIP_CHECK(hipMemcpyAsync(&counted, offsets + nregion, sizeof(int), hipMemcpyDeviceToHost, stream));
+        A2P_HIP_CHECK(hipStreamSynchronize(stream));
+        total = counted;
+    }
 
     size_t sorted_bytes = (size_t)total * (sizeof(int) + 3 * sizeof(T)) + 256;
     size_t sort_bytes = sort ? (size_t)N * umax * (2 * sizeof(int) + 4 * sizeof(T)) + 256 : 0;

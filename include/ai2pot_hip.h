@@ -95,8 +95,9 @@ int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, 
  * outputs are device pointers: ilist[natoms], numneigh[natoms], firstneigh[natoms][umax]
  * (-1 padded, indices modulo natoms), rcs[natoms][umax][3] (r_j - r_i, 0 padded),
  * types_out[natoms].  Results are bit-identical to the reference's, in both sort modes.
- * The call synchronises `stream` twice (extents and image count are read back to size the
- * bin grid).  max_numneigh (HOST int, may be NULL): when given, the call synchronises once
+ * The call synchronises `stream` once (the extents are read back to size the bin grid), and a
+ * second time only when natoms times the number of periodic images exceeds 2 GiB of scratch
+ * (the count of kept images is then read back instead of bounded).  max_numneigh (HOST int, may be NULL): when given, the call synchronises once
  * more, stores the largest neighbour count and returns A2P_ERR_OVERFLOW if it exceeds umax
  * (rows are then truncated, never overrun; the reference overruns, neighborList.h:550).
  * When NULL the check is left to a2p_check_status.
