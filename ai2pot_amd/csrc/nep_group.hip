@@ -1,5 +1,5 @@
-// NEP energy / force / virial, lane-group kernel for the common model shape
-// (chebyshev_size 8, n_radial 6, n_angular 4, l_max 4, up to 4 species), used for small systems:
+// NEP energy / force / virial, lane-group kernel for the common model shapes
+// (chebyshev_size 8, n_radial 4 or 6, n_angular 4, l_max 4, up to 4 species), used for small systems:
 // it spreads an atom over 8 lanes and a workgroup over 32 atoms, so a few thousand atoms already
 // occupy the device, at the price of more instructions per atom than the staged kernel.
 //
@@ -28,6 +28,8 @@
 #include "a2p_common.h"
 #include "nep_device.h"
 
+#include <type_traits>
+
 namespace a2p {
 using namespace nepdev;
 namespace {
@@ -36,8 +38,8 @@ constexpr int GL = 8;                    // lanes per atom
 constexpr int GTHREADS = 256;            // threads per workgroup
 constexpr int GATOMS = GTHREADS / GL;    // atoms per workgroup
 constexpr int GWAVES = GTHREADS / 64;
-constexpr int FDP = 24;                  // padded descriptor count (22)
-constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
+constexpr int FDP = 24;                  // padded descriptor count (at most 24: n_radial <= 8)
+constexpr int KC = 8, NAC = 4, LC = 4, NLM = 24;     // n_radial: template parameter NR of the kernel (4 and 6)
 
 // Tile capacity (pairs per atom held in LDS) and padded tile length.  With CAPP = 8 (mod 16)
 // the 16-byte entry reads of 16 consecutive lanes (2 atoms x 8 lanes) fall into distinct banks.
@@ -116,13 +118,13 @@ struct GroupLds {
 __host__ __device__ __forceinline__ size_t lds_round16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
 
 template <typename T>
-__host__ __device__ __forceinline__ size_t group_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
+__host__ __device__ __forceinline__ size_t group_lds_layout(int ntypes, int H, int ntc, int nb, unsigned char* base,
                                                             GroupLds<T>& L)
 {
     constexpr int CAPP = Tile<T>::CAPP;
     size_t off = 0;
     L.w0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * FDP * sizeof(T));
-    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * NB * KC * sizeof(T));
+    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * nb * KC * sizeof(T));
     L.b0 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
     L.w1 = (T*)(base + off);   off += lds_round16((size_t)ntypes * H * sizeof(T));
     L.qs = (T*)(base + off);   off += lds_round16((size_t)FDP * sizeof(T));
@@ -199,7 +201,7 @@ __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& se
     __builtin_amdgcn_wave_barrier();
 }
 
-template <typename T, int NTC>
+template <typename T, int NTC, int NR>
 __global__ void __launch_bounds__(GTHREADS, (sizeof(T) == 4 ? 2 : 1))
 nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
 {
@@ -213,8 +215,10 @@ nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
     const int ii = blockIdx.x * GATOMS + al;
     const int H = a.H, nt = a.ntypes;
     const int NF = a.P + a.nghost;
+    constexpr int NRC = NR, NB = NR + NAC, DC = NR + NAC * LC;
+    static_assert(DC <= FDP, "descriptor count exceeds the padded row");
     GroupLds<T> L;
-    group_lds_layout<T>(nt, H, NTC, smem_raw, L);
+    group_lds_layout<T>(nt, H, NTC, NB, smem_raw, L);
 
     for (int i = tid; i < nt * H * FDP; i += GTHREADS) {
         const int r = i / FDP, j = i - r * FDP;
@@ -532,11 +536,11 @@ nep_group_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g)
     }
 }
 
-template <typename T, int NTC>
+template <typename T, int NTC, int NR>
 int launch_group(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
 {
     SegArgs seg{csr.cursor, csr.seg_cap, csr.n * csr.seg_cap};
-    auto kern = nep_group_kernel<T, NTC>;
+    auto kern = nep_group_kernel<T, NTC, NR>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
@@ -556,9 +560,9 @@ int nep_group_nblocks(int P) { return ceil_div(P, GATOMS); }
 template <typename T>
 bool nep_group_supported(const NepArgs<T>& a, size_t* lds_bytes)
 {
-    if (!(a.K == KC && a.n_r == NRC && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
+    if (!(a.K == KC && (a.n_r == 4 || a.n_r == 6) && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
     GroupLds<T> unused;
-    *lds_bytes = group_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), nullptr, unused);
+    *lds_bytes = group_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), a.n_r + NAC, nullptr, unused);
     return *lds_bytes <= 150 * 1024;
 }
 
@@ -572,12 +576,16 @@ int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
                                  (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T));
         if (rc) return rc;
     }
-    switch (ntc_of(a.ntypes)) {
-    case 1: rc = launch_group<T, 1>(a, lds_bytes, csr, stream); break;
-    case 2: rc = launch_group<T, 2>(a, lds_bytes, csr, stream); break;
-    case 3: rc = launch_group<T, 3>(a, lds_bytes, csr, stream); break;
-    default: rc = launch_group<T, 4>(a, lds_bytes, csr, stream); break;
-    }
+    auto launch = [&](auto nr) {
+        constexpr int NR = decltype(nr)::value;
+        switch (ntc_of(a.ntypes)) {
+        case 1: return launch_group<T, 1, NR>(a, lds_bytes, csr, stream);
+        case 2: return launch_group<T, 2, NR>(a, lds_bytes, csr, stream);
+        case 3: return launch_group<T, 3, NR>(a, lds_bytes, csr, stream);
+        default: return launch_group<T, 4, NR>(a, lds_bytes, csr, stream);
+        }
+    };
+    rc = a.n_r == 4 ? launch(std::integral_constant<int, 4>{}) : launch(std::integral_constant<int, 6>{});
     if (rc) return rc;
     if (a.force) rc = pair_csr_finish<T>(a.force, csr, stream);
     return rc;

@@ -1,5 +1,5 @@
-// NEP energy / force / virial, staged kernel for the common model shape
-// (chebyshev_size 8, n_radial 6, n_angular 4, l_max 4, up to 4 species).
+// NEP energy / force / virial, staged kernels for the common model shapes
+// (chebyshev_size 8, n_radial 4 or 6, n_angular 4, l_max 4, up to 4 species).
 //
 // The generic kernel (nep.hip) lets every thread walk its own neighbour row four times, so each
 // wave-wide load touches 64 different cache lines, and it holds the pair derivatives in a
@@ -38,8 +38,10 @@ constexpr int FB = 256;        // atoms (threads) per workgroup of the model ker
 constexpr int SB = 256;        // atoms (threads) per workgroup of the staging kernel (divides FB)
 constexpr int SCH = 8;         // neighbour slots staged per round
 constexpr int SLS = SB + 8;    // padded row length of the staging arrays
-constexpr int FDP = 24;        // padded descriptor count (22)
-constexpr int KC = 8, NRC = 6, NAC = 4, LC = 4, NLM = 24, DC = 22, NB = NRC + NAC;
+constexpr int FDP = 24;        // padded descriptor count (at most 24: n_radial <= 8)
+constexpr int KC = 8, NAC = 4, LC = 4, NLM = 24;
+// n_radial is a template parameter NR of the model kernel: 4 (the reference's default model,
+// ai2pot/models/nep/nep.py:36) and 6 are instantiated
 
 __device__ __forceinline__ void lds_load4(const float* p, float (&o)[4])
 {
@@ -89,11 +91,11 @@ struct StagedLds {
 };
 
 template <typename T>
-__host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, unsigned char* base,
+__host__ __device__ __forceinline__ size_t staged_lds_layout(int ntypes, int H, int ntc, int nb, unsigned char* base,
                                                              StagedLds<T>& L)
 {
     size_t off = 0;
-    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * NB * KC * sizeof(T));
+    L.coef = (T*)(base + off); off += lds_round16((size_t)ntypes * ntypes * nb * KC * sizeof(T));
     const size_t u0 = off;
     L.acc = (T*)(base + off);  off += lds_round16((size_t)ntc * KC * FB * sizeof(T));
     const size_t u1 = off;
@@ -335,7 +337,7 @@ nep_stage_kernel(const NepArgs<T> a, const SegArgs seg, T* __restrict__ seg_g, T
     }
 }
 
-template <typename T, int NTC>
+template <typename T, int NTC, int NR>
 __global__ void __launch_bounds__(FB, (sizeof(T) == 4 ? 2 : 1))
 nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, int spare, const T* __restrict__ ang_xyz,
                   const unsigned* __restrict__ typew, const T* __restrict__ radial, const int* __restrict__ counts)
@@ -346,8 +348,10 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, int spare, const T*
     const int ii = blockIdx.x * FB + tid;
     const int H = a.H, nt = a.ntypes;
     const int NF = a.P + a.nghost;
+    constexpr int NRC = NR, NB = NR + NAC, DC = NR + NAC * LC;
+    static_assert(DC <= FDP, "descriptor count exceeds the padded row");
     StagedLds<T> L;
-    staged_lds_layout<T>(nt, H, NTC, smem_raw, L);
+    staged_lds_layout<T>(nt, H, NTC, NB, smem_raw, L);
 
     for (int i = tid; i < nt * nt * NB * KC; i += FB) L.coef[i] = a.coeffs[i];
     for (int i = tid; i < nt * H * FDP; i += FB) {
@@ -649,7 +653,7 @@ nep_staged_kernel(const NepArgs<T> a, T* __restrict__ seg_g, int spare, const T*
     }
 }
 
-template <typename T, int NTC>
+template <typename T, int NTC, int NR>
 int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream_t stream)
 {
     // workspace: compact lists [workgroup][entry < U][thread] of 4 T; species words of the front and
@@ -677,7 +681,7 @@ int launch_staged(const NepArgs<T>& a, size_t lds, const PairCsr& csr, hipStream
     hipLaunchKernelGGL(stage, dim3(ceil_div(a.P, SB), a.B), dim3(SB), lds_stage, stream, a, seg, (T*)csr.seg_g,
                        ang_xyz, typew, radial, counts);
     prof_end(stream);
-    auto kern = nep_staged_kernel<T, NTC>;
+    auto kern = nep_staged_kernel<T, NTC, NR>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
@@ -698,9 +702,9 @@ int nep_staged_nblocks(int P) { return ceil_div(P, FB); }
 template <typename T>
 bool nep_staged_supported(const NepArgs<T>& a, size_t* lds_bytes)
 {
-    if (!(a.K == KC && a.n_r == NRC && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
+    if (!(a.K == KC && (a.n_r == 4 || a.n_r == 6) && a.n_a == NAC && a.l_max == LC && a.ntypes <= 4)) return false;
     StagedLds<T> unused;
-    *lds_bytes = staged_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), nullptr, unused);
+    *lds_bytes = staged_lds_layout<T>(a.ntypes, a.H, ntc_of(a.ntypes), a.n_r + NAC, nullptr, unused);
     static_assert(FB % SB == 0, "a staging workgroup must not straddle two model workgroups");
     return *lds_bytes <= 150 * 1024;
 }
@@ -715,12 +719,16 @@ int nep_staged_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
                                  (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T));
         if (rc) return rc;
     }
-    switch (ntc_of(a.ntypes)) {
-    case 1: rc = launch_staged<T, 1>(a, lds_bytes, csr, stream); break;
-    case 2: rc = launch_staged<T, 2>(a, lds_bytes, csr, stream); break;
-    case 3: rc = launch_staged<T, 3>(a, lds_bytes, csr, stream); break;
-    default: rc = launch_staged<T, 4>(a, lds_bytes, csr, stream); break;
-    }
+    auto launch = [&](auto nr) {
+        constexpr int NR = decltype(nr)::value;
+        switch (ntc_of(a.ntypes)) {
+        case 1: return launch_staged<T, 1, NR>(a, lds_bytes, csr, stream);
+        case 2: return launch_staged<T, 2, NR>(a, lds_bytes, csr, stream);
+        case 3: return launch_staged<T, 3, NR>(a, lds_bytes, csr, stream);
+        default: return launch_staged<T, 4, NR>(a, lds_bytes, csr, stream);
+        }
+    };
+    rc = a.n_r == 4 ? launch(std::integral_constant<int, 4>{}) : launch(std::integral_constant<int, 6>{});
     if (rc) return rc;
     if (a.force) rc = pair_csr_finish<T>(a.force, csr, stream);
     return rc;

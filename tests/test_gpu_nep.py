@@ -113,6 +113,21 @@ def test_angular_cutoff_beyond_radial(oracle, reps):
         check(run_gpu(m, nbt, dt), oracle.nep_efv(m, nbt, dt), dt)
 
 
+@pytest.mark.parametrize("reps", [4, 21])
+def test_reference_default_model(oracle, reps):
+    """The hyperparameters ai2pot/models/nep/nep.py:32-46 defaults to (n_radial_basis 4, 30 neurons)
+    take the same fast kernels as the benchmark model (n_radial_basis 6): 256 atoms the one with
+    8 lanes per atom, 37044 atoms the staging + model pair."""
+    lat, pos = synth.fcc_cell(reps, 4.6, 0.15, 63)
+    ty = synth.rng_randint(64, pos.shape[0], 2)
+    nb = synth.pack_batch([oracle.nblist(lat, ty, pos, 6.0, 100)])
+    m = synth.nep_model(ntypes=2, n_radial_basis=4, num_neurons=30, rmax_radial=6.0, rmax_angular=4.0,
+                        seed=3063, type_map=(14, 8))
+    for dt in (np.float64, np.float32):
+        nbt = dict(nb, brcs=nb["brcs"].astype(dt))
+        check(run_gpu(m, nbt, dt), oracle.nep_efv(m, nbt, dt), dt)
+
+
 def test_ghost_atoms(oracle):
     """The LAMMPS contract: neighbour indices point into [0, P + nghost); ghosts have a type
     and receive forces but own no row (interface/lammps/AI2POT/pair_ai2pot.cpp:175-249)."""
