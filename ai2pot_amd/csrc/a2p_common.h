@@ -156,7 +156,14 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
 // (the force array of the caller, as a rule)
 template <typename T>
 int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero = nullptr,
-                     size_t also_bytes = 0);
+                     size_t also_bytes = 0, const int* incoming = nullptr);
+// incoming (optional): final counts per target from pair_ranks; the producer then stores at
+// pos = t*seg_cap + rank without claiming, and the cursors are neither zeroed nor written.
+
+// rank[B, P, U] = index of pair (row, slot) among the pairs naming the same neighbour (-1 for an
+// index out of range), incoming[B, P+nghost] = number of pairs naming each atom.
+int pair_ranks(int B, int P, int U, int nghost, const int* binum, const int* bnumneigh, const int* bfirstneigh,
+               int* rank, int* incoming, hipStream_t stream);
 template <typename T>
 int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);
 

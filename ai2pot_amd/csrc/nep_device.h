@@ -34,6 +34,10 @@ struct NepArgs {
     int* status;
     int want_virial;
     int w_in_lds;    // network weights staged in LDS (else read from global memory)
+    // optional: places of the pairs in their targets' reduction segments, known in advance
+    // (a2p_pair_ranks): brank[B, P, U], and bincoming[B, P+nghost] pairs naming each atom
+    const int* brank;
+    const int* bincoming;
 };
 
 __device__ __forceinline__ void sincospi_t(float x, float* s, float* c) { sincospif(x, s, c); }

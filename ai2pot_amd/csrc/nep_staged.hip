@@ -140,19 +140,22 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
         const T* p = a.brcs + pr * 3;
         nj[it] = a.bfirstneigh[pr];
         x[it] = p[0]; y[it] = p[1]; z[it] = p[2];
+        pos[it] = a.brank ? a.brank[pr] : 0;           // the pair's rank when the caller knows it
     }
     int err = 0;
 #pragma unroll
     for (int it = 0; it < SCH; it++) {
-        w[it] = 0; pos[it] = 0;
+        w[it] = 0;
         if (have[it] && (unsigned)nj[it] >= (unsigned)NF) { err |= ST_BAD_NEIGHBOR; have[it] = false; }
         const int njc = have[it] ? nj[it] : 0;
         w[it] = types[njc];
         if (have[it] && seg.cursor) {
             const int t = b * NF + njc;
-            const int rk = atomicAdd(&seg.cursor[t], 1);
+            const int rk = a.brank ? pos[it] : atomicAdd(&seg.cursor[t], 1);
             pos[it] = rk < seg.cap ? t * seg.cap + rk : seg.spare;
-            if (rk >= seg.cap) err |= ST_NEIGH_OVERFLOW;
+            if ((unsigned)rk >= (unsigned)seg.cap) { err |= ST_NEIGH_OVERFLOW; pos[it] = seg.spare; }
+        } else {
+            pos[it] = 0;
         }
     }
 #pragma unroll
@@ -716,7 +719,7 @@ int nep_staged_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     int rc;
     if (a.force) {
         rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream, a.force,
-                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T));
+                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), a.bincoming);
         if (rc) return rc;
     }
     auto launch = [&](auto nr) {

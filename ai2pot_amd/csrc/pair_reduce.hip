@@ -341,7 +341,7 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
 
 template <typename T>
 int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero,
-                     size_t also_bytes)
+                     size_t also_bytes, const int* incoming)
 {
     const long long NT = (long long)B * (P + nghost);
     A2P_REQUIRE(NT * U + 1 < (1ll << 31), A2P_ERR_INVALID,
@@ -360,7 +360,31 @@ int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t 
     csr->rank = nullptr;
     csr->cursor = (int*)ws;
     csr->seg_g = (void*)((char*)ws + bytes);
+    if (incoming) {      // the producer knows every pair's place: the counts are final already
+        csr->cursor = const_cast<int*>(incoming);
+        return fill_zero(also_zero, also_bytes, stream);
+    }
     return fill_zero2(csr->cursor, (size_t)n * sizeof(int), also_zero, also_bytes, stream);
+}
+
+int pair_ranks(int B, int P, int U, int nghost, const int* binum, const int* bnumneigh, const int* bfirstneigh,
+               int* rank, int* incoming, hipStream_t stream)
+{
+    A2P_REQUIRE(B >= 0 && P >= 0 && U >= 1 && nghost >= 0, A2P_ERR_INVALID, "pair_ranks: bad shape");
+    A2P_REQUIRE(binum && bnumneigh && bfirstneigh && rank && incoming, A2P_ERR_INVALID, "pair_ranks: null pointer");
+    if (B == 0 || P == 0) return A2P_OK;
+    const int NF = P + nghost;
+    void* flags = nullptr;
+    int rc = ws_get(WS_FLAGS, 64, &flags);
+    if (rc) return rc;
+    rc = fill_zero(incoming, (size_t)B * NF * sizeof(int), stream);
+    if (rc) return rc;
+    prof_begin("pair_ranks", stream);
+    hipLaunchKernelGGL(count_kernel, dim3(ceil_div((long long)B * P * 64, 256)), dim3(256), 0, stream, incoming, rank,
+                       B, P, U, NF, binum, bnumneigh, bfirstneigh, (int*)flags);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
 }
 
 template <typename T>
@@ -395,8 +419,8 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 
 template int pair_csr_begin<float>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
 template int pair_csr_begin<double>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
-template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t);
-template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t);
+template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, const int*);
+template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, const int*);
 template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
 template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,
@@ -405,3 +429,10 @@ template int pair_reduce<double>(double*, const double*, int, int, int, int, con
                                  const int*, hipStream_t);
 
 }  // namespace a2p
+
+extern "C" int a2p_pair_ranks(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
+                              const int* bfirstneigh, int* rank, int* incoming, void* stream)
+{
+    return a2p::pair_ranks(batch, natoms_pad, umax, nghost, binum, bnumneigh, bfirstneigh, rank, incoming,
+                           (hipStream_t)stream);
+}

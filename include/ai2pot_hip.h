@@ -85,6 +85,38 @@ int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, 
                     const int* bfirstneigh, const double* brcs, const int* btypes, double* etot,
                     double* force, double* virial, double* descriptors, void* stream);
 
+/* Places of the pairs of a list in their targets' reduction segments, computed once per list (no
+ * counterpart in the reference, which adds forces with atomics, nep.h:498-513).  The fast NEP
+ * kernels give every pair (row, slot) an entry in the segment of the neighbour it names; without
+ * help they claim it with one integer atomic per pair and call.  A caller that keeps a list for
+ * several steps (molecular dynamics with a skin) computes
+ *   rank[batch][natoms_pad][umax]      index of the pair among the pairs naming the same neighbour
+ *                                      (-1 for a neighbour index out of range), and
+ *   incoming[batch][natoms_pad+nghost] number of pairs naming each atom
+ * once with a2p_pair_ranks and passes both to a2p_nep_efv_ranked_*, which otherwise equals
+ * a2p_nep_efv_*.  Results do not depend on the ranks (the sums over a segment are exact): they are
+ * bit-identical to those of a2p_nep_efv_*.  Kernels that have no use for ranks ignore them. */
+int a2p_pair_ranks(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
+                   const int* bfirstneigh, int* rank, int* incoming, void* stream);
+
+int a2p_nep_efv_ranked_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
+                           int ntypes, const float* coeffs, const float* w0, const float* b0,
+                           const float* w1, const float* type_bias, const float* q_scaler,
+                           double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
+                           int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                           const int* bfirstneigh, const float* brcs, const int* btypes, const int* rank,
+                           const int* incoming, float* etot, float* force, float* virial,
+                           float* descriptors, void* stream);
+
+int a2p_nep_efv_ranked_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
+                           int ntypes, const double* coeffs, const double* w0, const double* b0,
+                           const double* w1, const double* type_bias, const double* q_scaler,
+                           double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
+                           int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                           const int* bfirstneigh, const double* brcs, const int* btypes, const int* rank,
+                           const int* incoming, double* etot, double* force, double* virial,
+                           double* descriptors, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Neighbour list -- replaces the compute of the CPython module function
  * nblist.find_info4mlff(lattice, types, coords, rcut, umax, is_cart, pbc_xyz, sort)

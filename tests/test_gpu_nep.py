@@ -215,6 +215,50 @@ def test_reproducible_staged_pair(oracle):
         assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
 
 
+def test_ranked_call_equals_plain_call(oracle):
+    """a2p_pair_ranks + a2p_nep_efv_ranked_f32: the places of the pairs in the reduction segments are
+    computed once for the list instead of claimed per call; E, F and V are bit-identical to the
+    plain call (40,000 atoms: the staging + model kernel pair, which is the path that uses ranks)."""
+    import ctypes as c
+    import torch
+    from ai2pot_amd import _lib
+    L = _lib.lib()
+    lat, pos = synth.fcc_cell(22, 4.6, 0.15, 67)
+    ty = synth.rng_randint(68, pos.shape[0], 3)
+    nb = synth.pack_batch([oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 6.0, 100)])
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    plain = run_gpu(m, nb, np.float32)
+    md = _model_to_device(m, torch.float32)
+    d = to_device(nb, torch.float32)
+    B, P, U = d["bfirstneigh"].shape
+    dev = d["brcs"].device
+    rank = torch.empty((B, P, U), dtype=torch.int32, device=dev)
+    incoming = torch.empty((B, P), dtype=torch.int32, device=dev)
+    vp = lambda t: c.c_void_p(t.data_ptr())
+    stream = c.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(L.a2p_pair_ranks(c.c_int(B), c.c_int(P), c.c_int(U), c.c_int(0), vp(d["binum"]),
+                                vp(d["bnumneigh"]), vp(d["bfirstneigh"]), vp(rank), vp(incoming), stream))
+    e = torch.empty(B, dtype=torch.float32, device=dev)
+    f = torch.empty((B, P, 3), dtype=torch.float32, device=dev)
+    v = torch.empty((B, 9), dtype=torch.float32, device=dev)
+    H = md["w1"].numel() // 3
+    for _ in range(2):          # the ranks serve any number of calls
+        _lib.check(L.a2p_nep_efv_ranked_f32(
+            c.c_int(m["chebyshev_size"]), c.c_int(m["n_radial_basis"]), c.c_int(m["n_angular_basis"]),
+            c.c_int(m["l_max"]), c.c_int(H), c.c_int(3), vp(md["coeffs"]), vp(md["w0"]), vp(md["b0"]),
+            vp(md["w1"]), vp(md["type_bias"]), vp(md["q_scaler"]), c.c_double(m["rmax_radial"]),
+            c.c_double(m["rmax_angular"]), c.c_int(B), c.c_int(P), c.c_int(U), c.c_int(0), vp(d["binum"]),
+            vp(d["bilist"]), vp(d["bnumneigh"]), vp(d["bfirstneigh"]), vp(d["brcs"]), vp(d["btypes"]),
+            vp(rank), vp(incoming), vp(e), vp(f), vp(v), None, stream))
+        torch.cuda.synchronize()
+        _lib.check_status(torch.cuda.current_stream().cuda_stream)
+        assert np.array_equal(e.cpu().numpy().view(np.uint32), plain[0].view(np.uint32))
+        assert np.array_equal(f.cpu().numpy().view(np.uint32), plain[1].view(np.uint32))
+        assert np.array_equal(v.cpu().numpy().view(np.uint32), plain[2].reshape(B, 9).view(np.uint32))
+    # every atom is named by as many pairs as it has neighbours (a full list is symmetric)
+    assert np.array_equal(incoming.cpu().numpy(), nb["bnumneigh"])
+
+
 def test_errors(oracle):
     import torch
     from ai2pot_amd import ops, _lib
