@@ -59,7 +59,14 @@ class NepCalculator:
         self._nbl_build = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
         self._nbl_update = L.a2p_nblist_update_f32 if f32 else L.a2p_nblist_update_f64
         self._have_list = False
-        self._efv = L.a2p_nep_efv_f32 if f32 else L.a2p_nep_efv_f64
+        self._efv = L.a2p_nep_efv_ranked_f32 if f32 else L.a2p_nep_efv_ranked_f64
+        # Places of the pairs in their targets' reduction segments.  A list that is evaluated a second
+        # time is probably kept for a while (a skin): that evaluation records the places (which costs
+        # about a sixth more than a plain call), the following ones use them (a seventh less).  A list
+        # rebuilt every step never pays for the record.
+        self.rank = None
+        self.incoming = None
+        self._evals = 0          # evaluations of the current list
 
     def rebuild(self, coords, stream):
         # after the first build the list buffers hold a valid list: later builds write each row
@@ -72,18 +79,26 @@ class NepCalculator:
                 _vp(self.types_out), None, stream)
         self._have_list = rc == 0
         _lib.check(rc)
+        self._evals = 0
 
     def evaluate(self, stream):
         m = self.m
+        if self._evals >= 1 and self.rank is None:
+            i32 = dict(dtype=torch.int32, device=self.device)
+            self.rank = torch.empty((self.n, self.umax), **i32)
+            self.incoming = torch.empty(self.n, **i32)
+        ranked = self._evals >= 1
         rc = self._efv(_c.c_int(m["chebyshev_size"]), _c.c_int(m["n_radial_basis"]),
                        _c.c_int(m["n_angular_basis"]), _c.c_int(m["l_max"]), _c.c_int(self.H),
                        _c.c_int(self.ntypes), _vp(self.coeffs), _vp(self.w0), _vp(self.b0), _vp(self.w1),
                        _vp(self.bias), _vp(self.q_scaler), _c.c_double(m["rmax_radial"]),
                        _c.c_double(m["rmax_angular"]), _c.c_int(1), _c.c_int(self.n), _c.c_int(self.umax),
                        _c.c_int(0), _vp(self.binum), _vp(self.ilist), _vp(self.numneigh),
-                       _vp(self.firstneigh), _vp(self.rcs), _vp(self.types_out), _vp(self.etot),
-                       _vp(self.force), _vp(self.virial), None, stream)
+                       _vp(self.firstneigh), _vp(self.rcs), _vp(self.types_out), _vp(self.rank) if ranked else None,
+                       _vp(self.incoming) if ranked else None, _c.c_int(1 if self._evals >= 2 else 0),
+                       _vp(self.etot), _vp(self.force), _vp(self.virial), None, stream)
         _lib.check(rc)
+        self._evals += 1
 
     def step(self, coords):
         """coords: [N, 3] Cartesian tensor on the device.  Returns (E[1], F[N,3], V[9]) views of

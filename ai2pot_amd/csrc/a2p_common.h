@@ -156,9 +156,10 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
 // (the force array of the caller, as a rule)
 template <typename T>
 int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero = nullptr,
-                     size_t also_bytes = 0, const int* incoming = nullptr);
-// incoming (optional): final counts per target from pair_ranks; the producer then stores at
-// pos = t*seg_cap + rank without claiming, and the cursors are neither zeroed nor written.
+                     size_t also_bytes = 0, int* cursor_ext = nullptr, bool cursor_final = false);
+// cursor_ext (optional): the caller's array takes the place of the cursors, so that the counts
+// survive the call; cursor_final: it already holds the final counts (every pair's place is known
+// from an earlier call), so it is neither zeroed nor written.
 
 // rank[B, P, U] = index of pair (row, slot) among the pairs naming the same neighbour (-1 for an
 // index out of range), incoming[B, P+nghost] = number of pairs naming each atom.

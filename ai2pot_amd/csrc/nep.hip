@@ -392,7 +392,7 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
             const T* b0, const T* w1, const T* bias, const T* q_scaler, double rr, double ra, int B,
             int P, int U, int nghost, const int* binum, const int* bilist, const int* bnumneigh,
             const int* bfirstneigh, const T* brcs, const int* btypes, T* etot, T* force, T* virial,
-            T* desc, hipStream_t stream, const int* brank = nullptr, const int* bincoming = nullptr)
+            T* desc, hipStream_t stream, int* brank = nullptr, int* bincoming = nullptr, int ranks_valid = 0)
 {
     A2P_REQUIRE((brank == nullptr) == (bincoming == nullptr), A2P_ERR_INVALID,
                 "nep: pair ranks and incoming counts come together");
@@ -418,7 +418,7 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     a.B = B; a.P = P; a.U = U; a.nghost = nghost; a.nblocks = ceil_div(P, NEP_BLOCK);
     a.binum = binum; a.bilist = bilist; a.bnumneigh = bnumneigh; a.bfirstneigh = bfirstneigh;
     a.brcs = brcs; a.btypes = btypes; a.desc = desc; a.want_virial = virial != nullptr;
-    a.brank = brank; a.bincoming = bincoming;
+    a.brank = brank; a.bincoming = bincoming; a.ranks_valid = ranks_valid;
     a.w_in_lds = 1;
     size_t lds = nep_lds_bytes(a);
     if (lds > 64 * 1024) {          // keep only the coefficient table in LDS
@@ -519,23 +519,23 @@ int a2p_nep_efv_ranked_f32(int K, int n_r, int n_a, int l_max, int H, int ntypes
                            const float* w0, const float* b0, const float* w1, const float* bias,
                            const float* q_scaler, double rr, double ra, int B, int P, int U, int nghost,
                            const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
-                           const float* brcs, const int* btypes, const int* brank, const int* bincoming,
-                           float* etot, float* force, float* virial, float* desc, void* stream)
+                           const float* brcs, const int* btypes, int* brank, int* bincoming,
+                           int ranks_valid, float* etot, float* force, float* virial, float* desc, void* stream)
 {
     return a2p::nep_efv<float>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra,
                                B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot,
-                               force, virial, desc, (hipStream_t)stream, brank, bincoming);
+                               force, virial, desc, (hipStream_t)stream, brank, bincoming, ranks_valid);
 }
 
 int a2p_nep_efv_ranked_f64(int K, int n_r, int n_a, int l_max, int H, int ntypes, const double* coeffs,
                            const double* w0, const double* b0, const double* w1, const double* bias,
                            const double* q_scaler, double rr, double ra, int B, int P, int U, int nghost,
                            const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
-                           const double* brcs, const int* btypes, const int* brank, const int* bincoming,
-                           double* etot, double* force, double* virial, double* desc, void* stream)
+                           const double* brcs, const int* btypes, int* brank, int* bincoming,
+                           int ranks_valid, double* etot, double* force, double* virial, double* desc, void* stream)
 {
     return a2p::nep_efv<double>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra,
                                 B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot,
-                                force, virial, desc, (hipStream_t)stream, brank, bincoming);
+                                force, virial, desc, (hipStream_t)stream, brank, bincoming, ranks_valid);
 }
 }

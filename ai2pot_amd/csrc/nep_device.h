@@ -34,10 +34,13 @@ struct NepArgs {
     int* status;
     int want_virial;
     int w_in_lds;    // network weights staged in LDS (else read from global memory)
-    // optional: places of the pairs in their targets' reduction segments, known in advance
-    // (a2p_pair_ranks): brank[B, P, U], and bincoming[B, P+nghost] pairs naming each atom
-    const int* brank;
-    const int* bincoming;
+    // optional: places of the pairs in their targets' reduction segments, kept by the caller from
+    // call to call while the list stays the same: brank[B, P, U], and bincoming[B, P+nghost] pairs
+    // naming each atom.  ranks_valid = 0: this call claims the places and records them there;
+    // 1: it uses what an earlier call recorded.
+    int* brank;
+    int* bincoming;
+    int ranks_valid;
 };
 
 __device__ __forceinline__ void sincospi_t(float x, float* s, float* c) { sincospif(x, s, c); }

@@ -140,7 +140,7 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
         const T* p = a.brcs + pr * 3;
         nj[it] = a.bfirstneigh[pr];
         x[it] = p[0]; y[it] = p[1]; z[it] = p[2];
-        pos[it] = a.brank ? a.brank[pr] : 0;           // the pair's rank when the caller knows it
+        pos[it] = a.brank && a.ranks_valid ? a.brank[pr] : 0;     // the pair's rank when an earlier call recorded it
     }
     int err = 0;
 #pragma unroll
@@ -151,7 +151,16 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
         w[it] = types[njc];
         if (have[it] && seg.cursor) {
             const int t = b * NF + njc;
-            const int rk = a.brank ? pos[it] : atomicAdd(&seg.cursor[t], 1);
+            int rk;
+            if (a.brank && a.ranks_valid) {
+                rk = pos[it];
+            } else {
+                rk = atomicAdd(&seg.cursor[t], 1);
+                if (a.brank) {                         // recorded for the later calls on the same list
+                    const int e = it * SB + tid;
+                    a.brank[(rowbase + e / SCH) * a.U + c0 + e % SCH] = rk;
+                }
+            }
             pos[it] = rk < seg.cap ? t * seg.cap + rk : seg.spare;
             if ((unsigned)rk >= (unsigned)seg.cap) { err |= ST_NEIGH_OVERFLOW; pos[it] = seg.spare; }
         } else {
@@ -719,7 +728,8 @@ int nep_staged_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     int rc;
     if (a.force) {
         rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream, a.force,
-                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), a.bincoming);
+                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), a.bincoming,
+                                 a.bincoming != nullptr && a.ranks_valid != 0);
         if (rc) return rc;
     }
     auto launch = [&](auto nr) {

@@ -341,7 +341,7 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
 
 template <typename T>
 int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero,
-                     size_t also_bytes, const int* incoming)
+                     size_t also_bytes, int* cursor_ext, bool cursor_final)
 {
     const long long NT = (long long)B * (P + nghost);
     A2P_REQUIRE(NT * U + 1 < (1ll << 31), A2P_ERR_INVALID,
@@ -360,10 +360,9 @@ int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t 
     csr->rank = nullptr;
     csr->cursor = (int*)ws;
     csr->seg_g = (void*)((char*)ws + bytes);
-    if (incoming) {      // the producer knows every pair's place: the counts are final already
-        csr->cursor = const_cast<int*>(incoming);
+    if (cursor_ext) csr->cursor = cursor_ext;            // the caller keeps the counts
+    if (cursor_ext && cursor_final)                      // ... and they are final: every pair's place is known
         return fill_zero(also_zero, also_bytes, stream);
-    }
     return fill_zero2(csr->cursor, (size_t)n * sizeof(int), also_zero, also_bytes, stream);
 }
 
@@ -419,8 +418,8 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 
 template int pair_csr_begin<float>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
 template int pair_csr_begin<double>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
-template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, const int*);
-template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, const int*);
+template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, int*, bool);
+template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, int*, bool);
 template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
 template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,

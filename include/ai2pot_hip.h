@@ -85,17 +85,18 @@ int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, 
                     const int* bfirstneigh, const double* brcs, const int* btypes, double* etot,
                     double* force, double* virial, double* descriptors, void* stream);
 
-/* Places of the pairs of a list in their targets' reduction segments, computed once per list (no
- * counterpart in the reference, which adds forces with atomics, nep.h:498-513).  The fast NEP
- * kernels give every pair (row, slot) an entry in the segment of the neighbour it names; without
- * help they claim it with one integer atomic per pair and call.  A caller that keeps a list for
- * several steps (molecular dynamics with a skin) computes
+/* E/F/V calls that keep the places of the pairs in their targets' reduction segments from call to
+ * call (no counterpart in the reference, which adds forces with atomics, nep.h:498-513).  The fast
+ * NEP kernels give every pair (row, slot) an entry in the segment of the neighbour it names and
+ * claim it with one integer atomic per pair and call.  A caller that uses a list for several
+ * steps (molecular dynamics with a skin) owns two buffers for that list,
  *   rank[batch][natoms_pad][umax]      index of the pair among the pairs naming the same neighbour
- *                                      (-1 for a neighbour index out of range), and
- *   incoming[batch][natoms_pad+nghost] number of pairs naming each atom
- * once with a2p_pair_ranks and passes both to a2p_nep_efv_ranked_*, which otherwise equals
- * a2p_nep_efv_*.  Results do not depend on the ranks (the sums over a segment are exact): they are
- * bit-identical to those of a2p_nep_efv_*.  Kernels that have no use for ranks ignore them. */
+ *   incoming[batch][natoms_pad+nghost] number of pairs naming each atom,
+ * and passes ranks_valid = 0 on the first call for a list (the call records the places it claims)
+ * and 1 on the following calls (they claim nothing: a third of the staging kernel's time).
+ * Otherwise the calls equal a2p_nep_efv_*: the results do not depend on the ranks (the sums over a
+ * segment are exact) and are bit-identical.  Kernels that have no use for ranks leave the buffers
+ * alone.  a2p_pair_ranks fills the two buffers from the list alone. */
 int a2p_pair_ranks(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
                    const int* bfirstneigh, int* rank, int* incoming, void* stream);
 
@@ -104,8 +105,8 @@ int a2p_nep_efv_ranked_f32(int chebyshev_size, int n_radial, int n_angular, int 
                            const float* w1, const float* type_bias, const float* q_scaler,
                            double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
                            int nghost, const int* binum, const int* bilist, const int* bnumneigh,
-                           const int* bfirstneigh, const float* brcs, const int* btypes, const int* rank,
-                           const int* incoming, float* etot, float* force, float* virial,
+                           const int* bfirstneigh, const float* brcs, const int* btypes, int* rank,
+                           int* incoming, int ranks_valid, float* etot, float* force, float* virial,
                            float* descriptors, void* stream);
 
 int a2p_nep_efv_ranked_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
@@ -113,8 +114,8 @@ int a2p_nep_efv_ranked_f64(int chebyshev_size, int n_radial, int n_angular, int 
                            const double* w1, const double* type_bias, const double* q_scaler,
                            double rmax_radial, double rmax_angular, int batch, int natoms_pad, int umax,
                            int nghost, const int* binum, const int* bilist, const int* bnumneigh,
-                           const int* bfirstneigh, const double* brcs, const int* btypes, const int* rank,
-                           const int* incoming, double* etot, double* force, double* virial,
+                           const int* bfirstneigh, const double* brcs, const int* btypes, int* rank,
+                           int* incoming, int ranks_valid, double* etot, double* force, double* virial,
                            double* descriptors, void* stream);
 
 /* ------------------------------------------------------------------------------------------

@@ -216,9 +216,10 @@ def test_reproducible_staged_pair(oracle):
 
 
 def test_ranked_call_equals_plain_call(oracle):
-    """a2p_pair_ranks + a2p_nep_efv_ranked_f32: the places of the pairs in the reduction segments are
-    computed once for the list instead of claimed per call; E, F and V are bit-identical to the
-    plain call (40,000 atoms: the staging + model kernel pair, which is the path that uses ranks)."""
+    """a2p_nep_efv_ranked_f32: the places of the pairs in the reduction segments are recorded by the
+    first call on a list (or computed by a2p_pair_ranks) and used by the following calls instead of
+    being claimed again; E, F and V are bit-identical to the plain call (40,000 atoms: the staging +
+    model kernel pair, which is the path that uses ranks)."""
     import ctypes as c
     import torch
     from ai2pot_amd import _lib
@@ -242,21 +243,60 @@ def test_ranked_call_equals_plain_call(oracle):
     f = torch.empty((B, P, 3), dtype=torch.float32, device=dev)
     v = torch.empty((B, 9), dtype=torch.float32, device=dev)
     H = md["w1"].numel() // 3
-    for _ in range(2):          # the ranks serve any number of calls
+
+    def ranked(valid):
         _lib.check(L.a2p_nep_efv_ranked_f32(
             c.c_int(m["chebyshev_size"]), c.c_int(m["n_radial_basis"]), c.c_int(m["n_angular_basis"]),
             c.c_int(m["l_max"]), c.c_int(H), c.c_int(3), vp(md["coeffs"]), vp(md["w0"]), vp(md["b0"]),
             vp(md["w1"]), vp(md["type_bias"]), vp(md["q_scaler"]), c.c_double(m["rmax_radial"]),
             c.c_double(m["rmax_angular"]), c.c_int(B), c.c_int(P), c.c_int(U), c.c_int(0), vp(d["binum"]),
             vp(d["bilist"]), vp(d["bnumneigh"]), vp(d["bfirstneigh"]), vp(d["brcs"]), vp(d["btypes"]),
-            vp(rank), vp(incoming), vp(e), vp(f), vp(v), None, stream))
+            vp(rank), vp(incoming), c.c_int(valid), vp(e), vp(f), vp(v), None, stream))
         torch.cuda.synchronize()
         _lib.check_status(torch.cuda.current_stream().cuda_stream)
         assert np.array_equal(e.cpu().numpy().view(np.uint32), plain[0].view(np.uint32))
         assert np.array_equal(f.cpu().numpy().view(np.uint32), plain[1].view(np.uint32))
         assert np.array_equal(v.cpu().numpy().view(np.uint32), plain[2].reshape(B, 9).view(np.uint32))
+
+    ranked(1)                   # ranks from a2p_pair_ranks
+    ranked(1)                   # ... serve any number of calls
+    rank.fill_(-7)
+    incoming.fill_(-7)
+    ranked(0)                   # this call claims the places and records them
+    live = np.arange(U)[None, None, :] < nb["bnumneigh"][:, :, None]
+    assert rank.cpu().numpy()[live].min() >= 0 and np.array_equal(incoming.cpu().numpy(), nb["bnumneigh"])
+    ranked(1)                   # ... for the following ones
     # every atom is named by as many pairs as it has neighbours (a full list is symmetric)
     assert np.array_equal(incoming.cpu().numpy(), nb["bnumneigh"])
+
+
+def test_calculator_kept_list(oracle):
+    """NepCalculator: evaluations on a kept list (plain, recording the pairs' places, using them) give
+    the same bits, and a rebuild starts over."""
+    import ctypes as c
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos = synth.fcc_cell(22, 4.6, 0.15, 69)
+    ty = synth.rng_randint(70, pos.shape[0], 3)
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    calc = NepCalculator(m, pos.shape[0], lat, ty, umax=100, dtype=torch.float32, device="cuda:0")
+    coords = torch.from_numpy(pos.astype(np.float32)).to("cuda:0")
+    stream = c.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for cycle in range(2):
+        calc.rebuild(coords, stream)
+        for _ in range(4):
+            calc.evaluate(stream)
+            torch.cuda.synchronize()
+            outs.append((calc.etot.cpu().numpy().copy(), calc.force.cpu().numpy().copy(),
+                         calc.virial.cpu().numpy().copy()))
+    calc.check()
+    for o in outs[1:]:
+        for x, y in zip(outs[0], o):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    ref = oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 6.0, 100)
+    er, fr, vr = oracle.nep_efv(m, synth.pack_batch([ref]), np.float32)
+    check((outs[0][0], outs[0][1][None], outs[0][2][None]), (er, fr, vr.reshape(1, 9)), np.float32)
 
 
 def test_errors(oracle):
