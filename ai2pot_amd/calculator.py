@@ -25,7 +25,7 @@ class NepCalculator:
     """Holds one NEP model and the neighbour buffers of one structure size."""
 
     def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
-                 sort=False, dtype=torch.float32, device="cuda:0"):
+                 sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None):
         self.device = torch.device(device)
         self.dtype = dtype
         self.n = int(natoms)
@@ -59,35 +59,58 @@ class NepCalculator:
         self._nbl_build = L.a2p_nblist_build_f32 if f32 else L.a2p_nblist_build_f64
         self._nbl_update = L.a2p_nblist_update_f32 if f32 else L.a2p_nblist_update_f64
         self._have_list = False
+        self._nbl_ranked = L.a2p_nblist_build_ranked_f32 if f32 else L.a2p_nblist_build_ranked_f64
         self._efv = L.a2p_nep_efv_ranked_f32 if f32 else L.a2p_nep_efv_ranked_f64
-        # Places of the pairs in their targets' reduction segments.  A list that is evaluated a second
-        # time is probably kept for a while (a skin): that evaluation records the places (which costs
-        # about a sixth more than a plain call), the following ones use them (a seventh less).  A list
-        # rebuilt every step never pays for the record.
+        # Places of the pairs in their targets' reduction segments: an evaluation that is given them
+        # needs no atomics.  With places_from_list the list build claims them (unsorted rows only).
+        # Otherwise a list that is evaluated a second time is probably kept for a while (a skin):
+        # that evaluation records the places (which costs about a sixth more than a plain call), the
+        # following ones use them (a seventh less).
+        # (the claims cost the list build what they save the first evaluation: worth it only for a
+        # list that is evaluated several times, hence off by default)
+        self.places_from_list = bool(places_from_list)
+        if self.places_from_list and self.sort:
+            raise ValueError("places_from_list needs sort=False")
         self.rank = None
         self.incoming = None
         self._evals = 0          # evaluations of the current list
+        self._places = False     # rank / incoming describe the current list
+        if self.places_from_list:
+            self._alloc_places()
+
+    def _alloc_places(self):
+        if self.rank is None:
+            i32 = dict(dtype=torch.int32, device=self.device)
+            self.rank = torch.empty((self.n, self.umax), **i32)
+            self.incoming = torch.empty(self.n, **i32)
 
     def rebuild(self, coords, stream):
         # after the first build the list buffers hold a valid list: later builds write each row
         # only as far as its old or new length reaches
-        fn = self._nbl_update if self._have_list else self._nbl_build
-        rc = fn(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
-                _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
-                self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self.sort else 0),
-                _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
-                _vp(self.types_out), None, stream)
+        if self.places_from_list:
+            rc = self._nbl_ranked(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
+                                  _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
+                                  self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self._have_list else 0),
+                                  _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
+                                  _vp(self.types_out), _vp(self.rank), _vp(self.incoming), None, stream)
+        else:
+            fn = self._nbl_update if self._have_list else self._nbl_build
+            rc = fn(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
+                    _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
+                    self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self.sort else 0),
+                    _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
+                    _vp(self.types_out), None, stream)
         self._have_list = rc == 0
+        self._places = False
         _lib.check(rc)
+        self._places = self.places_from_list
         self._evals = 0
 
     def evaluate(self, stream):
         m = self.m
-        if self._evals >= 1 and self.rank is None:
-            i32 = dict(dtype=torch.int32, device=self.device)
-            self.rank = torch.empty((self.n, self.umax), **i32)
-            self.incoming = torch.empty(self.n, **i32)
-        ranked = self._evals >= 1
+        ranked = self._places or self._evals >= 1
+        if ranked:
+            self._alloc_places()
         rc = self._efv(_c.c_int(m["chebyshev_size"]), _c.c_int(m["n_radial_basis"]),
                        _c.c_int(m["n_angular_basis"]), _c.c_int(m["l_max"]), _c.c_int(self.H),
                        _c.c_int(self.ntypes), _vp(self.coeffs), _vp(self.w0), _vp(self.b0), _vp(self.w1),
@@ -95,9 +118,10 @@ class NepCalculator:
                        _c.c_double(m["rmax_angular"]), _c.c_int(1), _c.c_int(self.n), _c.c_int(self.umax),
                        _c.c_int(0), _vp(self.binum), _vp(self.ilist), _vp(self.numneigh),
                        _vp(self.firstneigh), _vp(self.rcs), _vp(self.types_out), _vp(self.rank) if ranked else None,
-                       _vp(self.incoming) if ranked else None, _c.c_int(1 if self._evals >= 2 else 0),
+                       _vp(self.incoming) if ranked else None, _c.c_int(1 if self._places else 0),
                        _vp(self.etot), _vp(self.force), _vp(self.virial), None, stream)
         _lib.check(rc)
+        self._places = ranked
         self._evals += 1
 
     def step(self, coords):

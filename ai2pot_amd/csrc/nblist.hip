@@ -196,10 +196,12 @@ __device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i,
 // One thread per atom walks its images (x outer, z inner: image m = (i * dim_y + j) * dim_z + k,
 // supercell index m * N + p, structure.h:654-681).
 template <typename T>
-__global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __restrict__ counts)
+__global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __restrict__ counts,
+                             int* __restrict__ incoming)
 {
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= g.N) return;
+    if (incoming) incoming[p] = 0;                // counted up by the list kernel
     const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
     for (int i = 0; i < g.img_dim[0]; i++)
         for (int j = 0; j < g.img_dim[1]; j++)
@@ -307,7 +309,7 @@ constexpr int NBL_UNROLL = 4;
 constexpr int NBL_ENT_CAP = 256;   // flat candidate list per wave (entries); longer lists search the runs
 
 template <typename T>
-inline size_t rowbuf_bytes(int umax) { return (size_t)umax * (4 + 3 * sizeof(T)); }
+inline size_t rowbuf_bytes(int umax, bool rank) { return (size_t)umax * (4 + 3 * sizeof(T) + (rank ? 4 : 0)); }
 
 // Run of supercell entries that column `lane` of the (2e+1)^2 columns around the bin of the atom at
 // c can contribute: start index and length (0 for lanes without a column or with nothing in reach).
@@ -365,13 +367,13 @@ __device__ __forceinline__ void column_setup(const Grid<T>& g, const T (&c)[3], 
 
 constexpr int NBL_APW = 2;         // consecutive centre atoms per wavefront
 
-template <typename T, bool SORT, bool ROWBUF>
+template <typename T, bool SORT, bool ROWBUF, bool RANK>
 __global__ void __launch_bounds__(NBL_BLOCK)
 lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
              int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
              T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
-             int* __restrict__ status, int update)
+             int* __restrict__ status, int update, int* __restrict__ rank_out, int* __restrict__ incoming)
 {
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
@@ -383,10 +385,12 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     const int np = min(NBL_APW, g.N - p0);
     T* rb_rcs = nullptr;
     int* rb_first = nullptr;
+    int* rb_rank = nullptr;
     if (ROWBUF) {
-        unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T));
+        unsigned char* mine = sh_rows + (size_t)wv * umax * (4 + 3 * sizeof(T) + (RANK ? 4 : 0));
         rb_rcs = (T*)mine;
         rb_first = (int*)(mine + (size_t)umax * 3 * sizeof(T));
+        rb_rank = rb_first + umax;
     }
     // A row costs three dependent trips to memory (coordinates, column runs, candidates).  The
     // wavefront takes NBL_APW atoms: all their coordinates are loaded first, and the column runs of
@@ -449,6 +453,11 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
                 pz[u] = s_x[(size_t)ent * 3 + 2];
             }
         }
+        // RANK: the pair's place among the pairs that name the same neighbour, claimed here so that
+        // the force kernels need no atomics; the answers are collected after the chunk's last claim
+        int rk[NBL_UNROLL], rs[NBL_UNROLL];
+#pragma unroll
+        for (int u = 0; u < NBL_UNROLL; u++) rs[u] = -1;
 #pragma unroll
         for (int u = 0; u < NBL_UNROLL; u++) {
             if (c0 + u * 64 >= total) break;                           // wave-uniform
@@ -473,8 +482,20 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
                     rcs[(rowi + slot) * 3 + 2] = dz;
                 }
                 if (SORT) keys[rowi + slot] = (T)__dsqrt_rn(d2d);      // neighborList.h:318-322
+                if (RANK) {
+                    rk[u] = atomicAdd(&incoming[sj[u]], 1);
+                    rs[u] = slot;
+                }
             }
             cnt += __popcll(mask);
+        }
+        if (RANK) {
+#pragma unroll
+            for (int u = 0; u < NBL_UNROLL; u++)
+                if (rs[u] >= 0) {
+                    if (ROWBUF) rb_rank[rs[u]] = rk[u];
+                    else rank_out[rowi + rs[u]] = rk[u];
+                }
         }
     }
     if (lane == 0) {
@@ -499,6 +520,11 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
         const int nv = (int)((size_t)live * 3 * sizeof(T) / 16);
         for (int i = lane; i < nv; i += 64) d2[i] = s2[i];
+        if (RANK) {                                                    // slots past the row's end are not defined
+            const uint4* s3 = reinterpret_cast<const uint4*>(rb_rank);
+            uint4* d3 = reinterpret_cast<uint4*>(rank_out + rowi);
+            for (int i = lane; i < (used + 3) / 4; i += 64) d3[i] = s3[i];
+        }
     } else {
         // padding: -1 / 0 (neighborList.h:557, 563)
         const int first_pad = min(cnt, umax);
@@ -716,8 +742,12 @@ T host_plane_distance(const T* v, const T* n)        // structure.h:818-842, vec
 template <typename T>
 int nblist_build(const T* lattice, const int* types, const T* coords, int N, double rcut_in, int umax,
                  int is_cart, const int* pbc, int sort, int* ilist, int* numneigh, int* firstneigh,
-                 T* rcs, int* types_out, int* max_nn_host, hipStream_t stream, int update = 0)
+                 T* rcs, int* types_out, int* max_nn_host, hipStream_t stream, int update = 0,
+                 int* rank = nullptr, int* incoming = nullptr)
 {
+    A2P_REQUIRE((rank == nullptr) == (incoming == nullptr), A2P_ERR_INVALID,
+                "nblist: rank and incoming come together");
+    A2P_REQUIRE(!(rank && sort), A2P_ERR_INVALID, "nblist: places of the pairs are produced for unsorted rows only");
     A2P_REQUIRE(lattice && pbc, A2P_ERR_INVALID, "nblist: lattice and pbc must be host pointers");
     A2P_REQUIRE(N > 0, A2P_ERR_INVALID, "nblist: the structure has no atoms");   // binLinkedList.h:659
     A2P_REQUIRE(umax > 0 && rcut_in > 0, A2P_ERR_INVALID, "nblist: rcut and umax must be positive");
@@ -829,7 +859,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (rc) return rc;
     const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
     prof_begin("nbl_count", stream);
-    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts);
+    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming);
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
@@ -875,21 +905,29 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     const int list_blocks = ceil_div(N, (NBL_BLOCK / 64) * NBL_APW);
     prof_begin("nbl_lists", stream);
-    const size_t rows_lds = rowbuf_bytes<T>(umax) * (NBL_BLOCK / 64);
+    const size_t rows_lds = rowbuf_bytes<T>(umax, rank != nullptr) * (NBL_BLOCK / 64);
     const bool rowbuf = !sort && umax % 4 == 0 && rows_lds <= 32 * 1024 && (uintptr_t)firstneigh % 16 == 0 &&
-                        (uintptr_t)rcs % 16 == 0;
+                        (uintptr_t)rcs % 16 == 0 && (uintptr_t)rank % 16 == 0;
     if (sort)
-        hipLaunchKernelGGL((lists_kernel<T, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
+        hipLaunchKernelGGL((lists_kernel<T, true, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
-                           status, 0);
+                           status, 0, nullptr, nullptr);
+    else if (rowbuf && rank)
+        hipLaunchKernelGGL((lists_kernel<T, false, true, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
+                           g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           status, update, rank, incoming);
     else if (rowbuf)
-        hipLaunchKernelGGL((lists_kernel<T, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream, g,
-                           x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update);
-    else
-        hipLaunchKernelGGL((lists_kernel<T, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
+        hipLaunchKernelGGL((lists_kernel<T, false, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
+                           g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           status, update, nullptr, nullptr);
+    else if (rank)
+        hipLaunchKernelGGL((lists_kernel<T, false, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update);
+                           status, update, rank, incoming);
+    else
+        hipLaunchKernelGGL((lists_kernel<T, false, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
+                           types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           status, update, nullptr, nullptr);
     prof_end(stream);
     if (sort) {
         prof_begin("nbl_sort_rows", stream);
@@ -967,5 +1005,33 @@ int a2p_nblist_update_f64(const double* lattice, const int* types, const double*
     return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, sort, ilist,
                                      numneigh, firstneigh, rcs, types_out, max_numneigh,
                                      (hipStream_t)stream, 1);
+}
+
+int a2p_nblist_build_ranked_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                                double rcut, int umax, int is_cart, const int* pbc, int update, int* ilist,
+                                int* numneigh, int* firstneigh, float* rcs, int* types_out, int* rank,
+                                int* incoming, int* max_numneigh, void* stream)
+{
+    if (!rank || !incoming) {
+        a2p::set_error("nblist: rank and incoming must be device pointers");
+        return A2P_ERR_INVALID;
+    }
+    return a2p::nblist_build<float>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
+                                    firstneigh, rcs, types_out, max_numneigh, (hipStream_t)stream, update ? 1 : 0,
+                                    rank, incoming);
+}
+
+int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                                double rcut, int umax, int is_cart, const int* pbc, int update, int* ilist,
+                                int* numneigh, int* firstneigh, double* rcs, int* types_out, int* rank,
+                                int* incoming, int* max_numneigh, void* stream)
+{
+    if (!rank || !incoming) {
+        a2p::set_error("nblist: rank and incoming must be device pointers");
+        return A2P_ERR_INVALID;
+    }
+    return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
+                                     firstneigh, rcs, types_out, max_numneigh, (hipStream_t)stream, update ? 1 : 0,
+                                     rank, incoming);
 }
 }

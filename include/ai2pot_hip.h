@@ -163,6 +163,23 @@ int a2p_nblist_update_f64(const double* lattice, const int* types, const double*
                           int* numneigh, int* firstneigh, double* rcs, int* types_out, int* max_numneigh,
                           void* stream);
 
+/* The list together with the places of its pairs (no counterpart in the reference; for callers
+ * that go on to a2p_nep_efv_ranked_* with ranks_valid = 1, which then needs no atomics).  Rows are
+ * unsorted (the sort = 0 result of a2p_nblist_build_*, bit for bit).  update = 0 / 1 chooses
+ * between the contracts of a2p_nblist_build_* and a2p_nblist_update_*.  rank[natoms, umax] and
+ * incoming[natoms] (DEVICE int32) are filled as a2p_pair_ranks fills them: rank[i, k] is the
+ * place of pair (i, k) among the pairs that name the same neighbour, incoming[j] their number;
+ * slots past a row's end are undefined. */
+int a2p_nblist_build_ranked_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                                double rcut, int umax, int is_cart, const int* pbc, int update, int* ilist,
+                                int* numneigh, int* firstneigh, float* rcs, int* types_out, int* rank,
+                                int* incoming, int* max_numneigh, void* stream);
+
+int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                                double rcut, int umax, int is_cart, const int* pbc, int update, int* ilist,
+                                int* numneigh, int* firstneigh, double* rcs, int* types_out, int* rank,
+                                int* incoming, int* max_numneigh, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Linear Moment Tensor Potential.
  *

@@ -270,16 +270,18 @@ def test_ranked_call_equals_plain_call(oracle):
     assert np.array_equal(incoming.cpu().numpy(), nb["bnumneigh"])
 
 
-def test_calculator_kept_list(oracle):
-    """NepCalculator: evaluations on a kept list (plain, recording the pairs' places, using them) give
-    the same bits, and a rebuild starts over."""
+@pytest.mark.parametrize("from_list", [False, True])
+def test_calculator_kept_list(oracle, from_list):
+    """NepCalculator: evaluations on a kept list (plain, recording the pairs' places, using them; or
+    with the places the list build made) give the same bits, and a rebuild starts over."""
     import ctypes as c
     import torch
     from ai2pot_amd.calculator import NepCalculator
     lat, pos = synth.fcc_cell(22, 4.6, 0.15, 69)
     ty = synth.rng_randint(70, pos.shape[0], 3)
     m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
-    calc = NepCalculator(m, pos.shape[0], lat, ty, umax=100, dtype=torch.float32, device="cuda:0")
+    calc = NepCalculator(m, pos.shape[0], lat, ty, umax=100, dtype=torch.float32, device="cuda:0",
+                         places_from_list=from_list)
     coords = torch.from_numpy(pos.astype(np.float32)).to("cuda:0")
     stream = c.c_void_p(torch.cuda.current_stream().cuda_stream)
     outs = []
