@@ -110,6 +110,53 @@ def test_config3_reduced_and_ghosts(oracle):
     assert close(eg, er) and close(fg, fr) and close(vg, vr)
 
 
+def test_config3_full_size(oracle):
+    """Benchmark configuration 3 at full size: 8192 atoms in one cell, level 20, 4 species, K = 10,
+    rmax 5.5, rmin 1.8, against the oracle; the net force vanishes."""
+    lat, pos = synth.random_packed(8192, [64.0, 51.2, 50.0], 2.0, 1004)
+    ty = synth.rng_randint(2004, 8192, 4)
+    nb = synth.pack_batch([oracle.nblist(lat, ty, pos, 5.5, 200)])
+    m = synth.mtp_model(mtp_param.mtp_param(20), 4, 10, 5.5, 1.8, 3004, lo=-0.05, hi=0.05,
+                        type_map=[75, 41, 16, 34])
+    e, f, v = gpu_efv(m, nb)
+    er, fr, vr = oracle.mtp_efv(m, nb)
+    assert close(e, er) and close(f, fr) and close(v, vr)
+    assert np.abs(f.sum(1)).max() < 1e-9 * np.abs(f).max()
+
+
+def test_config4_full_size(oracle):
+    """Benchmark configuration 4 at full size: one training step over 64 structures of 128 atoms,
+    level 16, 3 species.  Every per-structure result of the batch (loss, energy, forces, virial,
+    gradient rows) equals the one-structure call's bit for bit; six of the structures are checked
+    against the oracle (the whole batch takes it 20 s)."""
+    rho = synth.rng_uniform(1005, 64, 0.03, 0.05)
+    lists = []
+    for b in range(64):
+        Lb = (128.0 / rho[b]) ** (1.0 / 3.0)
+        lat, pos = synth.random_packed(128, [Lb, Lb, Lb], 2.0, 11005 + b)
+        lists.append(oracle.nblist(lat, synth.rng_randint(21005 + b, 128, 3), pos, 5.0, 200))
+    nb = synth.pack_batch(lists)
+    m = synth.mtp_model(mtp_param.mtp_param(16), 3, 8, 5.0, 0.0, 3005)
+    B, P = nb["bilist"].shape
+    labels = dict(energy=synth.rng_normal(4005, B * P, -4.0, 0.2).reshape(B, P).sum(1),
+                  force=synth.rng_normal(4006, B * P * 3, 0.0, 1.0).reshape(B, P, 3),
+                  virial=synth.rng_normal(4007, B * 9, 0.0, 0.5).reshape(B, 9))
+    w = (1.0, 1.0, 1.0)
+    got = gpu_loss(m, nb, labels, w)
+    keys = ("bloss", "energy", "force", "virial", "dcoeffs", "dlinear", "dbias")
+    pick = [0, 7, 21, 38, 50, 63]
+    sub = {k: (v[pick].copy() if hasattr(v, "shape") else v) for k, v in nb.items()}
+    sub_labels = {k: v[pick] for k, v in labels.items()}
+    ref = oracle.mtp_loss_step(m, sub, w, sub_labels)
+    for k in keys:
+        assert close(got[k][pick], ref[k]), k
+    for b in (0, 38, 63):
+        one = {k: (v[b:b + 1].copy() if hasattr(v, "shape") else v) for k, v in nb.items()}
+        r1 = gpu_loss(m, one, {k: v[b:b + 1] for k, v in labels.items()}, w)
+        for k in keys:
+            assert np.array_equal(r1[k][0], got[k][b]), k
+
+
 @pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
 def test_reproducible(oracle, np_dtype):
     """Two runs give bit-identical results: the pairs claim their segment entries in an order that

@@ -193,6 +193,65 @@ def test_config2_full_size(oracle):
     assert np.abs(v - v.T).max() <= 2e-5 * np.abs(v).max()
 
 
+def test_config5_full_size(oracle):
+    """Benchmark configuration 5 at full size (1,048,576 atoms, list rebuilt and E/F/V on the device)
+    through a size-independent property: the cell is a 16^3 block of 16,384 atoms repeated 4 x 4 x 4,
+    so the energy and the virial are 64 times the block's and every replica carries the block's
+    forces; the block itself is checked against the oracle.  Also: the list is symmetric (every atom
+    is named as a neighbour as often as it has neighbours) and the net force vanishes."""
+    import ctypes as c
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    # coordinates on a 2^-14 A grid: block and replicas are then exactly representable in fp32, every
+    # relative vector of a replica equals the block's bit for bit, and so do the lists
+    q = 2.0 ** -14
+    a = np.round(316.7 / 64.0 / q) * q
+    lat16, pos16 = synth.fcc_cell(16, a, 0.15, 1006)
+    pos16 = np.mod(np.round(pos16 / q) * q, 16 * a)
+    n16 = pos16.shape[0]
+    ty16 = synth.rng_randint(2006, n16, 3)
+    m = synth.nep_model(seed=3006)
+    r = np.arange(4, dtype=np.float64)
+    sx, sy, sz = np.meshgrid(r, r, r, indexing="ij")
+    shifts = np.stack([sx.ravel(), sy.ravel(), sz.ravel()], axis=1) * (16 * a)
+    pos = (shifts[:, None, :] + pos16[None, :, :]).reshape(-1, 3)
+    types = np.tile(ty16, 64)
+    n = pos.shape[0]
+    assert n == 1048576
+    calc = NepCalculator(m, n, lat16 * 4, types, umax=200, dtype=torch.float32, device="cuda:0")
+    e, f, v = calc.step(torch.from_numpy(pos.astype(np.float32)).to("cuda:0"))
+    torch.cuda.synchronize()
+    calc.check()
+    e, f, v = e.cpu().numpy().astype(np.float64), f.cpu().numpy(), v.cpu().numpy().astype(np.float64)
+    ref = oracle.nblist(lat16.astype(np.float32), ty16, pos16.astype(np.float32), 7.0, 200)
+    er, fr, vr = oracle.nep_efv(m, synth.pack_batch([ref]), np.float32)
+    er, fr, vr = float(np.asarray(er).ravel()[0]), np.asarray(fr)[0], np.asarray(vr).reshape(9)
+    assert abs(e[0] - 64 * er) <= 1e-5 * abs(64 * er)
+    assert np.abs(v - 64 * vr).max() <= 1e-5 * np.abs(64 * vr).max()
+    fb = f.reshape(64, n16, 3)
+    assert np.all(np.abs(fb - fr[None]) <= 1e-4 + 1e-5 * np.abs(fr[None]))
+    assert np.abs(f.astype(np.float64).sum(0)).max() < 0.05
+    nn = calc.numneigh.cpu().numpy()
+    assert np.array_equal(nn.reshape(64, n16), np.broadcast_to(np.asarray(ref[2])[None, :], (64, n16)))
+    live = torch.arange(200, device="cuda:0", dtype=torch.int32)[None, :] < calc.numneigh[:, None]
+    incoming = torch.bincount(calc.firstneigh[live].long(), minlength=n)
+    assert torch.equal(incoming.int(), calc.numneigh)
+    # first and last replica: the rows name the block's neighbours with the block's relative vectors
+    # (as sets: the order within a row follows the bins, which differ between the two cells)
+    ref_rows = np.asarray(ref[3]).reshape(n16, 200)
+    ref_rcs = np.asarray(ref[4]).reshape(n16, 200, 3)
+    want_order = np.lexsort((ref_rcs[..., 2], ref_rcs[..., 1], ref_rcs[..., 0], np.where(ref_rows >= 0, ref_rows, n16)), axis=1)
+    for rep in (0, 63):
+        rows = calc.firstneigh[rep * n16:(rep + 1) * n16].cpu().numpy()
+        rcs = calc.rcs[rep * n16:(rep + 1) * n16].cpu().numpy()
+        key = np.where(rows >= 0, rows % n16, n16)
+        order = np.lexsort((rcs[..., 2], rcs[..., 1], rcs[..., 0], key), axis=1)
+        assert np.array_equal(np.take_along_axis(key, order, 1),
+                              np.take_along_axis(np.where(ref_rows >= 0, ref_rows, n16), want_order, 1))
+        assert np.array_equal(np.take_along_axis(rcs, order[..., None], 1).view(np.uint32),
+                              np.take_along_axis(ref_rcs, want_order[..., None], 1).view(np.uint32))
+
+
 def test_reproducible(oracle):
     """Two runs give bit-identical forces (no floating-point atomics anywhere)."""
     nb = synth.pack_batch([small_structure(oracle, 300, dtype=np.float32)])
