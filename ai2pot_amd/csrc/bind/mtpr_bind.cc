@@ -50,8 +50,12 @@ variable_list mtp_efv(bool want_virial, int64_t K, double scaling, const at::Ten
                          bfirstneigh, brcs, btypes, type_map, nghost, q_scaler);
     a2p_bind::DeviceGuard guard(brcs);
     auto opt = brcs.options();
-    at::Tensor e = at::zeros({c.s.B}, opt), f = at::zeros({c.s.B, c.s.P + c.s.nghost, 3}, opt), v;
-    if (want_virial) v = at::zeros({c.s.B, 9}, opt);
+    // the library writes every element of the three outputs (forces are zeroed on entry)
+    const bool fresh = c.s.B > 0 && c.s.P > 0;
+    at::Tensor e = fresh ? at::empty({c.s.B}, opt) : at::zeros({c.s.B}, opt);
+    at::Tensor f = fresh ? at::empty({c.s.B, c.s.P + c.s.nghost, 3}, opt) : at::zeros({c.s.B, c.s.P + c.s.nghost, 3}, opt);
+    at::Tensor v;
+    if (want_virial) v = fresh ? at::empty({c.s.B, 9}, opt) : at::zeros({c.s.B, 9}, opt);
     void* st = current_stream(brcs);
     int rc;
     if (brcs.scalar_type() == at::kDouble)

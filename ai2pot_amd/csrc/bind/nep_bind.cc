@@ -54,9 +54,11 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
     at::Tensor e, f, v, d;
     if (want_desc) d = at::zeros({s.B, s.P, m.D}, opt);
     else {
-        e = at::zeros({s.B}, opt);
-        f = at::zeros({s.B, s.P + s.nghost, 3}, opt);
-        if (want_virial) v = at::zeros({s.B, 9}, opt);
+        // the library writes every element of the three outputs (forces are zeroed on entry)
+        const bool fresh = s.B > 0 && s.P > 0;
+        e = fresh ? at::empty({s.B}, opt) : at::zeros({s.B}, opt);
+        f = fresh ? at::empty({s.B, s.P + s.nghost, 3}, opt) : at::zeros({s.B, s.P + s.nghost, 3}, opt);
+        if (want_virial) v = fresh ? at::empty({s.B, 9}, opt) : at::zeros({s.B, 9}, opt);
     }
     void* st = current_stream(brcs);
     int rc;

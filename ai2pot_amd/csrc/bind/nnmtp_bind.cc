@@ -51,9 +51,11 @@ variable_list nnmtp_run(bool want_e, bool want_v, bool want_es, int64_t K, const
     auto opt = brcs.options();
     at::Tensor e, f, v, es;
     if (want_e) {
-        e = at::zeros({s.B}, opt);
-        f = at::zeros({s.B, s.P + s.nghost, 3}, opt);
-        if (want_v) v = at::zeros({s.B, 9}, opt);
+        // the library writes every element of the three outputs (forces are zeroed on entry)
+        const bool fresh = s.B > 0 && s.P > 0;
+        e = fresh ? at::empty({s.B}, opt) : at::zeros({s.B}, opt);
+        f = fresh ? at::empty({s.B, s.P + s.nghost, 3}, opt) : at::zeros({s.B, s.P + s.nghost, 3}, opt);
+        if (want_v) v = fresh ? at::empty({s.B, 9}, opt) : at::zeros({s.B, 9}, opt);
     }
     if (want_es) es = at::zeros({s.B, s.P}, opt);
     void* st = current_stream(brcs);

@@ -102,10 +102,12 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
     if want_desc:
         desc = torch.zeros((B, P, D), dtype=dtype, device=device)
     else:
-        etot = torch.zeros((B,), dtype=dtype, device=device)
-        force = torch.zeros((B, P + nghost, 3), dtype=dtype, device=device)
+        # the library writes every element of the three outputs (forces are zeroed on entry)
+        new = torch.empty if B * P > 0 else torch.zeros
+        etot = new((B,), dtype=dtype, device=device)
+        force = new((B, P + nghost, 3), dtype=dtype, device=device)
         if want_virial:
-            virial = torch.zeros((B, 9), dtype=dtype, device=device)
+            virial = new((B, 9), dtype=dtype, device=device)
     L = _lib.lib()
     fn = L.a2p_nep_efv_f32 if dtype == torch.float32 else L.a2p_nep_efv_f64
     with torch.cuda.device(device):
@@ -401,9 +403,10 @@ def _mtp_efv(want_virial, chebyshev_size, scaling, coeffs, linear_coeffs, type_b
         coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic, alpha_index_times,
         alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
         q_scaler, chebyshev_size, validate)
-    etot = torch.zeros((B,), dtype=dtype, device=device)
-    force = torch.zeros((B, P + nghost, 3), dtype=dtype, device=device)
-    virial = torch.zeros((B, 9), dtype=dtype, device=device) if want_virial else None
+    new = torch.empty if B * P > 0 else torch.zeros      # the library writes every element of the outputs
+    etot = new((B,), dtype=dtype, device=device)
+    force = new((B, P + nghost, 3), dtype=dtype, device=device)
+    virial = new((B, 9), dtype=dtype, device=device) if want_virial else None
     L = _lib.lib()
     fn = L.a2p_mtp_efv_f32 if dtype == torch.float32 else L.a2p_mtp_efv_f64
     with torch.cuda.device(device):
@@ -765,9 +768,10 @@ def _nnmtp_call(want, chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_c
     if validate:
         _validate_batch(binum, bnumneigh, U, P)
     z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
-    etot = z(B) if "e" in want else None
-    force = z(B, P + nghost, 3) if "f" in want else None
-    virial = z(B, 9) if "v" in want else None
+    new = (lambda *sh: torch.empty(sh, dtype=dtype, device=device)) if B * P > 0 else z   # written in full by the library
+    etot = new(B) if "e" in want else None
+    force = new(B, P + nghost, 3) if "f" in want else None
+    virial = new(B, 9) if "v" in want else None
     e_sites = z(B, P) if "es" in want else None
     L = _lib.lib()
     fn = L.a2p_nnmtp_efv_f32 if dtype == torch.float32 else L.a2p_nnmtp_efv_f64
