@@ -165,14 +165,39 @@ int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t 
 // index out of range), incoming[B, P+nghost] = number of pairs naming each atom.
 int pair_ranks(int B, int P, int U, int nghost, const int* binum, const int* bnumneigh, const int* bfirstneigh,
                int* rank, int* incoming, hipStream_t stream);
+// With etot or virial given, the same launch also sums the energy / virial partials
+// (finish_energy_virial's work, in workgroups of its own behind those of the segments).
 template <typename T>
-int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream);
+int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream, T* etot = nullptr, T* virial = nullptr,
+                    const double* partial = nullptr, int B = 0, int nblocks = 0);
 
 // out[b*out_stride + c] = sum over blocks of partial[(b*nblocks + block)*src_stride + c], c < ncomp,
 // with a fixed summation tree (fp64).
 template <typename T>
 int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
                     int out_stride, hipStream_t stream);
+
+// One workgroup of 256 threads: component c (0 energy, 1..9 virial) of structure b from
+// partial[(b*nblocks + block)*10 + c], summed over the blocks by a fixed tree (fp64).
+template <typename T>
+__device__ __forceinline__ void finish_ev_body(T* etot, T* virial, const double* partial, int nblocks, int b, int c,
+                                               double* sh)
+{
+    if (c == 0 ? etot == nullptr : virial == nullptr) return;      // uniform over the workgroup
+    const double* src = partial + ((size_t)b * nblocks) * 10 + c;
+    double acc = 0.0;
+    for (int k = threadIdx.x; k < nblocks; k += 256) acc += src[(size_t)k * 10];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (c == 0) etot[b] = (T)sh[0];
+        else virial[(size_t)b * 9 + c - 1] = (T)sh[0];
+    }
+}
 
 // etot[b] and virial[b*9 + c] from partial[(b*nblocks + block)*10 + (0 | 1 + c)], one launch; either
 // output may be null.

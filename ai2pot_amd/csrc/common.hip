@@ -188,21 +188,7 @@ template <typename T>
 __global__ void finish_ev_kernel(T* etot, T* virial, const double* partial, int nblocks)
 {
     __shared__ double sh[256];
-    const int b = blockIdx.y, c = blockIdx.x;
-    if (c == 0 ? etot == nullptr : virial == nullptr) return;      // uniform over the workgroup
-    const double* src = partial + ((size_t)b * nblocks) * 10 + c;
-    double acc = 0.0;
-    for (int k = threadIdx.x; k < nblocks; k += 256) acc += src[(size_t)k * 10];
-    sh[threadIdx.x] = acc;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        if (c == 0) etot[b] = (T)sh[0];
-        else virial[(size_t)b * 9 + c - 1] = (T)sh[0];
-    }
+    finish_ev_body<T>(etot, virial, partial, nblocks, blockIdx.y, blockIdx.x, sh);
 }
 
 template <typename T>

@@ -1133,10 +1133,8 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
     }
     rc = launch_atoms<T, false>(a, stream);
     if (rc) return rc;
-    if (force) {
-        rc = pair_csr_finish<T>(force, csr, stream);
-        if (rc) return rc;
-    }
+    if (force)       // the segment sums and the energy / virial sums share a launch
+        return pair_csr_finish<T>(force, csr, stream, etot, virial, a.partial, B, P);
     return finish_energy_virial<T>(etot, virial, a.partial, B, P, stream);
 }
 

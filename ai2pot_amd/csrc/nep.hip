@@ -451,11 +451,9 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     const size_t force_bytes = (size_t)B * (P + nghost) * 3 * sizeof(T);
 
     if (group) {
-        rc = nep_group_run<T>(a, lds_group, stream);
-        if (rc) return rc;
+        return nep_group_run<T>(a, lds_group, etot, virial, stream);     // includes the energy / virial sums
     } else if (staged) {
-        rc = nep_staged_run<T>(a, lds_staged, stream);
-        if (rc) return rc;
+        return nep_staged_run<T>(a, lds_staged, etot, virial, stream);
     } else {
         if (!force && virial) {     // the virial needs the pair derivatives: use a scratch force
             rc = ws_get(WS_MISC, force_bytes, &ws);

@@ -205,8 +205,8 @@ __device__ __forceinline__ void blm_dir_derivs(T x, T y, T z, T wx, T wy, T wz, 
 
 // The staged kernel for the common model shape (nep_staged.hip).  staged_supported() tells
 // whether it applies; nep_staged_run() performs forces' zero-fill, pair counting, the kernel and
-// the pair reduction, leaving the workgroup partial sums in a.partial (a.nblocks is set by
-// staged_nblocks()).
+// the pair reduction, whose launch also sums the workgroup partial sums of a.partial (a.nblocks
+// is set by staged_nblocks()) into etot and virial.
 // The same model shape with 8 lanes per atom (nep_group.hip): an atom's latency is an eighth of
 // the staged kernel's and a workgroup holds 32 atoms, which is what a small system needs to
 // occupy the device; per atom it executes more instructions, so large systems stay with the
@@ -215,12 +215,12 @@ template <typename T>
 bool nep_group_supported(const nepdev::NepArgs<T>& a, size_t* lds_bytes);
 int nep_group_nblocks(int P);
 template <typename T>
-int nep_group_run(const nepdev::NepArgs<T>& a, size_t lds_bytes, hipStream_t stream);
+int nep_group_run(const nepdev::NepArgs<T>& a, size_t lds_bytes, T* etot, T* virial, hipStream_t stream);
 
 template <typename T>
 bool nep_staged_supported(const nepdev::NepArgs<T>& a, size_t* lds_bytes);
 int nep_staged_nblocks(int P);
 template <typename T>
-int nep_staged_run(const nepdev::NepArgs<T>& a, size_t lds_bytes, hipStream_t stream);
+int nep_staged_run(const nepdev::NepArgs<T>& a, size_t lds_bytes, T* etot, T* virial, hipStream_t stream);
 
 }  // namespace a2p

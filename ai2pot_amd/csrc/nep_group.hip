@@ -567,7 +567,7 @@ bool nep_group_supported(const NepArgs<T>& a, size_t* lds_bytes)
 }
 
 template <typename T>
-int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
+int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, T* etot, T* virial, hipStream_t stream)
 {
     PairCsr csr{};
     int rc;
@@ -587,13 +587,13 @@ int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, hipStream_t stream)
     };
     rc = a.n_r == 4 ? launch(std::integral_constant<int, 4>{}) : launch(std::integral_constant<int, 6>{});
     if (rc) return rc;
-    if (a.force) rc = pair_csr_finish<T>(a.force, csr, stream);
-    return rc;
+    if (a.force) return pair_csr_finish<T>(a.force, csr, stream, etot, virial, a.partial, a.B, a.nblocks);
+    return finish_energy_virial<T>(etot, virial, a.partial, a.B, a.nblocks, stream);
 }
 
 template bool nep_group_supported<float>(const NepArgs<float>&, size_t*);
 template bool nep_group_supported<double>(const NepArgs<double>&, size_t*);
-template int nep_group_run<float>(const NepArgs<float>&, size_t, hipStream_t);
-template int nep_group_run<double>(const NepArgs<double>&, size_t, hipStream_t);
+template int nep_group_run<float>(const NepArgs<float>&, size_t, float*, float*, hipStream_t);
+template int nep_group_run<double>(const NepArgs<double>&, size_t, double*, double*, hipStream_t);
 
 }  // namespace a2p

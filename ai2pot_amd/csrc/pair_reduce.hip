@@ -149,12 +149,20 @@ __global__ void fill_kernel(T* __restrict__ seg_g, int* __restrict__ cursor,
     }
 }
 
-// 16 lanes per target atom.
+// 16 lanes per target atom.  Workgroups from `reduce_blocks` on sum the energy / virial partials
+// instead (one component of one structure each), which saves small systems a launch.
 template <typename T>
 __global__ void reduce_kernel(T* __restrict__ force, const T* __restrict__ seg_g,
                               const int* __restrict__ offsets, const int* __restrict__ counts, int NT,
-                              int seg_cap)
+                              int seg_cap, int reduce_blocks, T* __restrict__ etot, T* __restrict__ virial,
+                              const double* __restrict__ partial, int nblocks)
 {
+    if ((int)blockIdx.x >= reduce_blocks) {
+        __shared__ double sh[256];
+        const int id = (int)blockIdx.x - reduce_blocks;
+        finish_ev_body<T>(etot, virial, partial, nblocks, id / 10, id % 10, sh);
+        return;
+    }
     const int gid = blockIdx.x * blockDim.x + threadIdx.x;
     const int t = gid >> 4;
     const int sub = gid & 15;
@@ -387,14 +395,17 @@ int pair_ranks(int B, int P, int U, int nghost, const int* binum, const int* bnu
 }
 
 template <typename T>
-int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream)
+int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream, T* etot, T* virial, const double* partial,
+                    int B, int nblocks)
 {
     // with ranks every counted pair has its place in the segment; otherwise the cursor holds
     // how many entries were filled
+    const int reduce_blocks = ceil_div((long long)csr.n * 16, 256);
+    const int ev_blocks = (etot || virial) ? 10 * B : 0;
     prof_begin("reduce_sum", stream);
-    hipLaunchKernelGGL(reduce_kernel<T>, dim3(ceil_div((long long)csr.n * 16, 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(reduce_kernel<T>, dim3(reduce_blocks + ev_blocks), dim3(256), 0, stream,
                        force, (const T*)csr.seg_g, csr.offsets, csr.rank ? csr.counts : csr.cursor, csr.n,
-                       csr.seg_cap);
+                       csr.seg_cap, reduce_blocks, etot, virial, partial, nblocks);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -420,8 +431,8 @@ template int pair_csr_begin<float>(PairCsr*, bool, int, int, int, int, const int
 template int pair_csr_begin<double>(PairCsr*, bool, int, int, int, int, const int*, const int*, const int*, hipStream_t);
 template int pair_fixed_begin<float>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, int*, bool);
 template int pair_fixed_begin<double>(PairCsr*, int, int, int, int, hipStream_t, void*, size_t, int*, bool);
-template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t);
-template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t);
+template int pair_csr_finish<float>(float*, const PairCsr&, hipStream_t, float*, float*, const double*, int, int);
+template int pair_csr_finish<double>(double*, const PairCsr&, hipStream_t, double*, double*, const double*, int, int);
 template int pair_reduce<float>(float*, const float*, int, int, int, int, const int*, const int*,
                                 const int*, hipStream_t);
 template int pair_reduce<double>(double*, const double*, int, int, int, int, const int*, const int*,
