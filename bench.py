@@ -110,8 +110,8 @@ def timed_replay(replay, steps, warmup):
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
 MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nep_stage_kernel"): 4.418e6 * 1024,
-    ("nep_md_1048576", "nep_staged_kernel"): 3.189e6 * 1024,
+    ("nep_md_1048576", "nep_stage_kernel"): 4.473e6 * 1024,
+    ("nep_md_1048576", "nep_staged_kernel"): 3.190e6 * 1024,
     ("nep_md_1048576", "nbl_lists"): 1.039e6 * 1024,
 }
 
