@@ -66,7 +66,9 @@ int a2p_profile_report(char* buf, size_t buflen);
  * Batch (the 7-tensor contract): binum[B], bilist[B][P], bnumneigh[B][P],
  * bfirstneigh[B][P][U], brcs[B][P][U][3] (r_j - r_i), btypes[B][P+nghost] (type indices).
  * Outputs (each may be NULL to skip): etot[B], force[B][P+nghost][3], virial[B][9]
- * (row-major a*3+b, V = -sum g_a r_b), descriptors[B][P][D].  Outputs are overwritten.
+ * (row-major a*3+b, V = -sum g_a r_b), descriptors[B][P][D].  Outputs are overwritten: etot,
+ * force (rows of padded atoms and ghosts included) and virial need no initialisation, every
+ * element is written; of descriptors only the rows below binum[b] are.
  * Sign convention as the reference: force[i] += dE_i/dr_ij, force[j] -= dE_i/dr_ij.
  * ------------------------------------------------------------------------------------------ */
 int a2p_nep_efv_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
