@@ -94,7 +94,7 @@ inline void check_device_status(const at::Tensor& t)
 inline void require_no_zbl(double zbl_rmax)
 {
     TORCH_CHECK(zbl_rmax == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
-                                 "operators only; this operator needs zbl_rmax == 0");
+                                 "and the loss operators only; this operator needs zbl_rmax == 0");
 }
 
 // Adds the ZBL pair repulsion onto a model's E/F/V when zbl_rmax > 0, as the reference's operators
@@ -128,6 +128,40 @@ inline void apply_zbl(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, c
     }
     check_rc(rc);
     check_device_status(brcs);
+}
+
+// Labels of a loss operator with the ZBL pair repulsion taken out.  The correction does not depend
+// on the model parameters, so model + ZBL - label = model - (label - ZBL): the loss, its RMSEs and
+// its gradients are those of the operator without ZBL on the shifted labels.  The reference adds
+// the correction to E/F/V before the loss and before its gradient (e.g. nepOp.cc:2552-2575,
+// 3127-3150).  v_dft may be undefined (operators without virial labels).
+struct ShiftedLabels {
+    at::Tensor e, f, v;
+};
+inline ShiftedLabels zbl_shift_labels(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, const at::Tensor& dks,
+                                      const at::Tensor& type_map, const at::Tensor& binum, const at::Tensor& bilist,
+                                      const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
+                                      const at::Tensor& brcs, const at::Tensor& btypes, int64_t nghost,
+                                      const at::Tensor& e_dft, const at::Tensor& f_dft, const at::Tensor& v_dft)
+{
+    ShiftedLabels out{e_dft, f_dft, v_dft};
+    if (zbl_rmax == 0.0) return out;
+    TORCH_CHECK(nghost == 0, "the loss operator requires nghost == 0, as the reference does");
+    TORCH_CHECK(brcs.dim() == 4, "brcs must have shape [B, P, U, 3]");
+    check_device_float(brcs, e_dft, "betot_dft");
+    check_device_float(brcs, f_dft, "bforce_dft");
+    if (v_dft.defined()) check_device_float(brcs, v_dft, "bvirial_dft");
+    const int64_t B = brcs.size(0), P = brcs.size(1);
+    TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == B * P * 3 && (!v_dft.defined() || v_dft.numel() == B * 9),
+                "label shapes do not match the batch");
+    auto opt = brcs.options();
+    at::Tensor e0 = at::zeros({B}, opt), f0 = at::zeros({B, P, 3}, opt), v0;
+    if (v_dft.defined()) v0 = at::zeros({B, 9}, opt);
+    apply_zbl(zbl_rmax, zbl_rmin, cks, dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, 0, e0, f0, v0);
+    out.e = e_dft.detach().reshape({B}) - e0;
+    out.f = f_dft.detach().reshape({B, P, 3}) - f0;
+    if (v_dft.defined()) out.v = v_dft.detach().reshape({B, 9}) - v0;
+    return out;
 }
 
 }  // namespace a2p_bind

@@ -358,15 +358,18 @@ TORCH_LIBRARY(mtpr, m)
     m.def("linearMtpToLossOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
              const at::Tensor& v_dft, MTP_EFV_ARGS) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return LossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, MTP_EFV_PASS);
+              // the reference's forward passes the model's cutoffs to the ZBL launcher
+              // (linearMtpOp.cc:819-820) where its backward passes the ZBL ones (:1400-1401); here both
+              // use the ZBL cutoffs
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, v_dft);
+              return LossFunction::apply(true, e_w, f_w, v_w, lab.e, lab.f, lab.v, MTP_EFV_PASS);
           });
     m.def("linearMtpToEFLossOp",
           [](double e_w, double f_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
              MTP_EFV_ARGS) -> variable_list {
-              require_no_zbl(zbl_rmax);
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, at::Tensor());
               // no virial labels in this variant: zero weight, zero labels
-              return LossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
+              return LossFunction::apply(false, e_w, f_w, 0.0, lab.e, lab.f,
                                          at::zeros({e_dft.numel(), 9}, e_dft.options()), MTP_EFV_PASS);
           });
     m.def("LinMatrixLinVectorOp",

@@ -207,8 +207,8 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& type_map, int64_t nghost, double rr, double ra, const at::Tensor& q_scaler,
              double zbl_rmax, double zbl_rmin, const at::Tensor& zbl_cks,
              const at::Tensor& zbl_dks) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return NepLossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, K, n_r, n_a, l_max, coeffs, w0,
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, v_dft);
+              return NepLossFunction::apply(true, e_w, f_w, v_w, lab.e, lab.f, lab.v, K, n_r, n_a, l_max, coeffs, w0,
                                             b0, w1, bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
                                             type_map, nghost, rr, ra, q_scaler);
           });
@@ -220,8 +220,8 @@ TORCH_LIBRARY(nep, m)
              const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rr, double ra,
              const at::Tensor& q_scaler, double zbl_rmax, double zbl_rmin, const at::Tensor& zbl_cks,
              const at::Tensor& zbl_dks) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return NepLossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft, at::zeros({(int64_t)binum.numel(), 9}, brcs.options()),
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, at::Tensor());
+              return NepLossFunction::apply(false, e_w, f_w, 0.0, lab.e, lab.f, at::zeros({(int64_t)binum.numel(), 9}, brcs.options()),
                                             K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist, bnumneigh,
                                             bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler);
           });

@@ -314,13 +314,13 @@ TORCH_LIBRARY(nnmtp, m)
     m.def("nnMtpToLossOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
              const at::Tensor& v_dft, NNMTP_ARGS) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return NNLossFunction::apply(true, e_w, f_w, v_w, e_dft, f_dft, v_dft, NNMTP_PASS);
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, v_dft);
+              return NNLossFunction::apply(true, e_w, f_w, v_w, lab.e, lab.f, lab.v, NNMTP_PASS);
           });
     m.def("nnMtpToEFLossOp",
           [](double e_w, double f_w, const at::Tensor& e_dft, const at::Tensor& f_dft, NNMTP_ARGS) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return NNLossFunction::apply(false, e_w, f_w, 0.0, e_dft, f_dft,
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, at::Tensor());
+              return NNLossFunction::apply(false, e_w, f_w, 0.0, lab.e, lab.f,
                                            at::zeros({e_dft.numel(), 9}, e_dft.options()), NNMTP_PASS);
           });
 }

@@ -125,7 +125,7 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
 
 def _no_zbl(zbl_rmax):
     _req(float(zbl_rmax) == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
-                                 "operators only; this operator needs zbl_rmax == 0")
+                                 "and the loss operators only; this operator needs zbl_rmax == 0")
 
 
 def _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
@@ -151,6 +151,31 @@ def _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnum
         _lib.check(rc)
         if validate:
             _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                      btypes, nghost, betot_dft, bforce_dft, bvirial_dft, validate):
+    """Labels of a loss operator with the ZBL pair repulsion taken out.  The correction does not
+    depend on the model parameters, so model + ZBL - label = model - (label - ZBL): the loss, its
+    RMSEs and its gradients are those of the operator without ZBL on the shifted labels.  The
+    reference adds the correction to E/F/V before the loss and before its gradient (e.g.
+    nepOp.cc:2552-2575, 3127-3150).  bvirial_dft may be None (operators without virial labels)."""
+    if float(zbl_rmax) == 0.0:
+        return betot_dft, bforce_dft, bvirial_dft
+    _req(int(nghost) == 0, "the loss operator requires nghost == 0, as the reference does")
+    dtype, device = brcs.dtype, brcs.device
+    for name, t in (("betot_dft", betot_dft), ("bforce_dft", bforce_dft), ("bvirial_dft", bvirial_dft)):
+        if t is not None:
+            _check_float(name, t, dtype, device)
+    B, P = int(brcs.shape[0]), int(brcs.shape[1])
+    e0 = torch.zeros((B,), dtype=dtype, device=device)
+    f0 = torch.zeros((B, P, 3), dtype=dtype, device=device)
+    v0 = torch.zeros((B, 9), dtype=dtype, device=device) if bvirial_dft is not None else None
+    _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+             0, e0, f0, v0, validate)
+    _req(betot_dft.numel() == B and bforce_dft.numel() == B * P * 3, "label shapes do not match the batch")
+    return (betot_dft.detach().reshape(B) - e0, bforce_dft.detach().reshape(B, P, 3) - f0,
+            None if bvirial_dft is None else bvirial_dft.detach().reshape(B, 9) - v0)
 
 
 def nepToEFVOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w0, b0, w1, type_bias,
@@ -288,7 +313,9 @@ def nepToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft
                 zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
     """[bloss[B], e_rmse[1], f_rmse[1], v_rmse[1]], differentiable w.r.t. coeffs, w0, b0, w1 and
     type_bias; nep_bind.cc:205-276, nepOp.cc:2359-2960."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, bvirial_dft = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, bvirial_dft, validate)
     args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, n_radial_basis,
             n_angular_basis, l_max, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
             rmax_radial, rmax_angular, q_scaler, validate)
@@ -301,7 +328,9 @@ def nepToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, n_r
                   zbl_dks=None, validate=True):
     """[bloss[B], e_rmse[1], f_rmse[1]]: the loss without the virial term; nep_bind.cc:136-203,
     nepOp.cc:2962-3484 (nepLoss.h:139-166 is nepLoss.h:170-209 with v_weight = 0)."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, _ = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, None, validate)
     B = int(binum.numel())
     v0 = torch.zeros((B, 9), dtype=brcs.dtype, device=brcs.device)
     args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v0, chebyshev_size, n_radial_basis, n_angular_basis,
@@ -527,7 +556,9 @@ def linearMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bviri
                       zbl_cks=None, zbl_dks=None, validate=True):
     """[bloss[B], e_rmse[1], f_rmse[1], v_rmse[1]], differentiable w.r.t. coeffs, linear_coeffs and
     type_bias; mtpr_bind.cc:189-261."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, bvirial_dft = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, bvirial_dft, validate)
     args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, scaling,
             alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
             bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler, validate)
@@ -541,7 +572,9 @@ def linearMtpToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_siz
                         zbl_dks=None, validate=True):
     """[bloss[B], e_rmse[1], f_rmse[1]]: the loss without virial labels (zero weight, zero labels);
     mtpr_bind.cc:263-331, linearMtpOp.cc:1768-2831."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, _ = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, None, validate)
     v_dft = torch.zeros((betot_dft.numel(), 9), dtype=betot_dft.dtype, device=betot_dft.device)
     args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v_dft, chebyshev_size, scaling,
             alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum,
@@ -988,7 +1021,9 @@ def nnMtpToLossOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
                   q_scaler, zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, exact_gradient=False,
                   validate=True):
     """[bloss[B]], differentiable w.r.t. coeffs, w0, w1, type_bias; nnmtp_bind.cc:116-191."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, bvirial_dft = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, bvirial_dft, validate)
     args = (e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, alpha_moments_count,
             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh,
             brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, exact_gradient, validate)
@@ -1000,7 +1035,9 @@ def nnMtpToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, c
                     bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler,
                     zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, exact_gradient=False, validate=True):
     """[bloss[B]] without virial labels (zero weight, zero labels); nnmtp_bind.cc:43-114."""
-    _no_zbl(zbl_rmax)
+    betot_dft, bforce_dft, _ = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, None, validate)
     v_dft = torch.zeros((betot_dft.numel(), 9), dtype=betot_dft.dtype, device=betot_dft.device)
     args = (e_weight, f_weight, 0.0, betot_dft, bforce_dft, v_dft, chebyshev_size, alpha_moments_count,
             alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh,
