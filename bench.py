@@ -426,13 +426,13 @@ def run_copy_probe(args):
 
 
 WORKLOADS = {
-    "nep_md_1048576": lambda a: run_nep_md(a, "fcc", 64),         # BASELINE.json configs[4] (headline)
+    "nep_md_1048576": lambda a: run_nep_md(a, "fcc", 64),         # the headline configuration (configs[4] of the benchmark definition)
     "nep_md_131072": lambda a: run_nep_md(a, "fcc", 32),
     "nep_efv_4096": lambda a: run_nep_md(a, "random", 4096, rebuild=False),   # configs[1]
     "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]
     "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
     "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]
-    "nep_train_64x128": run_nep_train,                            # NEP counterpart of configs[3] (not a BASELINE line)
+    "nep_train_64x128": run_nep_train,                            # NEP counterpart of configs[3] (not one of the benchmark configurations)
     "hbm_copy_probe": None,                                       # counter calibration, not a workload of the path
 }
 
