@@ -2,6 +2,7 @@
 #include "a2p_common.h"
 
 #include <mutex>
+#include <string>
 #include <vector>
 
 namespace a2p {
@@ -88,23 +89,44 @@ bool g_prof_on = false;
 std::mutex g_prof_mutex;
 std::vector<ProfRec> g_prof_recs;
 thread_local hipEvent_t g_prof_pending_stop = nullptr;
+std::string g_prof_select;                 // ",label,label,": only these are timed; empty: all
+std::vector<hipEvent_t> g_prof_pool;       // events of reported records, reused (one device's)
+int g_prof_pool_dev = -1;
+
+bool prof_event(hipEvent_t* e)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    if (dev != g_prof_pool_dev) {
+        for (hipEvent_t old : g_prof_pool) (void)hipEventDestroy(old);
+        g_prof_pool.clear();
+        g_prof_pool_dev = dev;
+    }
+    if (!g_prof_pool.empty()) {
+        *e = g_prof_pool.back();
+        g_prof_pool.pop_back();
+        return true;
+    }
+    return hipEventCreate(e) == hipSuccess;
+}
 }  // namespace
 
 void prof_begin(const char* label, hipStream_t stream)
 {
     if (!g_prof_on) return;
-    ProfRec r{label, nullptr, nullptr};
-    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
-    hipEventRecord(r.start, stream);
-    g_prof_pending_stop = r.stop;
     std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (!g_prof_select.empty() && g_prof_select.find("," + std::string(label) + ",") == std::string::npos) return;
+    ProfRec r{label, nullptr, nullptr};
+    if (!prof_event(&r.start) || !prof_event(&r.stop)) return;
+    (void)hipEventRecord(r.start, stream);
+    g_prof_pending_stop = r.stop;
     g_prof_recs.push_back(r);
 }
 
 void prof_end(hipStream_t stream)
 {
     if (!g_prof_on || !g_prof_pending_stop) return;
-    hipEventRecord(g_prof_pending_stop, stream);
+    (void)hipEventRecord(g_prof_pending_stop, stream);
     g_prof_pending_stop = nullptr;
 }
 
@@ -224,6 +246,13 @@ void a2p_profile_enable(int on)
     a2p::g_prof_on = on != 0;
 }
 
+void a2p_profile_select(const char* labels)
+{
+    std::lock_guard<std::mutex> lock(a2p::g_prof_mutex);
+    a2p::g_prof_select.clear();
+    if (labels && labels[0]) a2p::g_prof_select = "," + std::string(labels) + ",";
+}
+
 int a2p_profile_report(char* buf, size_t buflen)
 {
     A2P_HIP_CHECK(hipDeviceSynchronize());
@@ -238,8 +267,14 @@ int a2p_profile_report(char* buf, size_t buflen)
                 if (std::string(a.label) == r.label) { a.ms += ms; a.count++; found = true; break; }
             if (!found) acc.push_back({r.label, (double)ms, 1});
         }
-        hipEventDestroy(r.start);
-        hipEventDestroy(r.stop);
+        int dev = -1;
+        if (hipGetDevice(&dev) == hipSuccess && dev == a2p::g_prof_pool_dev && a2p::g_prof_pool.size() < 4096) {
+            a2p::g_prof_pool.push_back(r.start);
+            a2p::g_prof_pool.push_back(r.stop);
+        } else {
+            (void)hipEventDestroy(r.start);
+            (void)hipEventDestroy(r.stop);
+        }
     }
     a2p::g_prof_recs.clear();
     size_t used = 0;

@@ -54,6 +54,10 @@ int a2p_check_status(void* stream);
  * clears the records. */
 void a2p_profile_enable(int on);
 int a2p_profile_report(char* buf, size_t buflen);
+/* Restricts the timing to the kernel labels of a comma-separated list ("nep_stage_kernel,nbl_lists");
+ * NULL or "" times every kernel again.  Two events per launch cost a few microseconds each, which a
+ * step of fifteen launches feels: a benchmark times only the kernels it reports on. */
+void a2p_profile_select(const char* labels);
 
 /* ------------------------------------------------------------------------------------------
  * NEP energy / force / virial -- replaces the compute of torch.ops.nep.nepToEFVOp /
