@@ -115,6 +115,15 @@ struct SegArgs {
     int spare;     // entry that takes what overflows a segment
 };
 
+// Row of the padded arrays that local row `la` of the workgroup starting at `rowbase` (= b * P + first
+// row) loads from: its own, or the structure's last row for the tail of the last workgroup
+__host__ __device__ __forceinline__ size_t staged_row_index(size_t rowbase, int la, int b, int P)
+{
+    const size_t last = (size_t)b * P + (size_t)(P - 1);
+    const size_t r = rowbase + (size_t)la;
+    return r < last ? r : last;
+}
+
 // Stage slots [c0, c0 + SCH) of the workgroup's rows: thread e handles row e / SCH, slot e % SCH,
 // so SCH consecutive lanes read one row's contiguous coordinates and indices.  Entries past a
 // row's end (or with an index out of range) are stored far outside every cutoff.
@@ -135,8 +144,10 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
         const int e = it * SB + tid;
         const int la = e / SCH, slot = c0 + e % SCH;
         have[it] = slot < L.nn[la];
-        // a slot past the row's end reads the row's first slot instead (always inside the arrays)
-        const size_t pr = (rowbase + la) * a.U + (have[it] ? slot : 0);
+        // a slot past the row's end reads the row's first slot instead, and a row past the
+        // structure's last one (the tail of the last workgroup) the structure's last row: the
+        // address stays inside the caller's arrays whatever their allocation
+        const size_t pr = staged_row_index(rowbase, la, b, a.P) * a.U + (have[it] ? slot : 0);
         const T* p = a.brcs + pr * 3;
         nj[it] = a.bfirstneigh[pr];
         x[it] = p[0]; y[it] = p[1]; z[it] = p[2];

@@ -118,3 +118,23 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), "%s is declared in include/ai2pot_hip.h but not exported" % n
     lib.a2p_abi_version.restype = ctypes.c_int
     assert lib.a2p_abi_version() >= 1
+
+
+def test_staged_rows_never_load_past_the_arrays():
+    """Index arithmetic of the staging kernel's row loads (csrc/nep_staged.hip: staged_row_index and
+    the slot choice of staged_load), emulated on the host: whatever natoms_pad is, every address the
+    256 threads of the last workgroup form lies inside the caller's [B, P, U] arrays."""
+    SB, SCH = 256, 8
+    for B, P, U in ((1, 1, 8), (1, 96, 200), (2, 257, 16), (3, 42592 % 1024 + 3, 200), (2, 512, 8)):
+        for b in range(B):
+            for blk in range((P + SB - 1) // SB):
+                rowbase = b * P + blk * SB
+                for tid in range(0, SB, 7):
+                    for it in range(SCH):
+                        e = it * SB + tid
+                        la, slot = e // SCH, e % SCH + 192
+                        have = blk * SB + la < P and slot < U          # rows past P hold no neighbours
+                        row = min(rowbase + la, b * P + P - 1)
+                        pr = row * U + (slot if have else 0)
+                        assert 0 <= pr < B * P * U
+                        assert row // P == b                            # never another structure's row
