@@ -172,10 +172,11 @@ int pair_csr_finish(T* force, const PairCsr& csr, hipStream_t stream, T* etot = 
                     const double* partial = nullptr, int B = 0, int nblocks = 0);
 
 // out[b*out_stride + c] = sum over blocks of partial[(b*nblocks + block)*src_stride + c], c < ncomp,
-// with a fixed summation tree (fp64).
+// with a fixed summation tree (fp64).  timed = false: the launch is never bracketed by timing events
+// (which are created on first use), for the callers that must not allocate.
 template <typename T>
 int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
-                    int out_stride, hipStream_t stream);
+                    int out_stride, hipStream_t stream, bool timed = true);
 
 // One workgroup of 256 threads: component c (0 energy, 1..9 virial) of structure b from
 // partial[(b*nblocks + block)*10 + c], summed over the blocks by a fixed tree (fp64).

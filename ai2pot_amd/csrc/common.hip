@@ -195,12 +195,12 @@ __global__ void finish_partials_kernel(T* out, const double* partial, int nblock
 
 template <typename T>
 int finish_partials(T* out, const double* partial, int B, int nblocks, int ncomp, int src_stride,
-                    int out_stride, hipStream_t stream)
+                    int out_stride, hipStream_t stream, bool timed)
 {
-    prof_begin("finish_partials", stream);
+    if (timed) prof_begin("finish_partials", stream);
     hipLaunchKernelGGL(finish_partials_kernel<T>, dim3(ncomp, B), dim3(256), 0, stream, out, partial,
                        nblocks, src_stride, out_stride);
-    prof_end(stream);
+    if (timed) prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
 }
@@ -225,8 +225,8 @@ int finish_energy_virial(T* etot, T* virial, const double* partial, int B, int n
 }
 template int finish_energy_virial<float>(float*, float*, const double*, int, int, hipStream_t);
 template int finish_energy_virial<double>(double*, double*, const double*, int, int, hipStream_t);
-template int finish_partials<float>(float*, const double*, int, int, int, int, int, hipStream_t);
-template int finish_partials<double>(double*, const double*, int, int, int, int, int, hipStream_t);
+template int finish_partials<float>(float*, const double*, int, int, int, int, int, hipStream_t, bool);
+template int finish_partials<double>(double*, const double*, int, int, int, int, int, hipStream_t, bool);
 
 }  // namespace a2p
 

@@ -12,6 +12,8 @@
 //   dL/dg[ii,s,a]  = - sum_b gV[a,b] r[ii,s,b],   dL/dr[ii,s,b] = - sum_a gV[a,b] g[ii,s,a]
 #include "a2p_common.h"
 
+#include <mutex>
+
 namespace a2p {
 namespace {
 
@@ -208,6 +210,58 @@ int virial_bwd(int B, int P, int U, const int* bnumneigh, const T* rcs, const T*
     return A2P_OK;
 }
 
+// ---- virial without any allocation ------------------------------------------------------------
+// The row partial sums of virial_fwd live in a per-device workspace that is allocated on demand.
+// Callers that must not allocate (HIP graph capture, serving loops, harnesses that forbid it) get
+// the same two kernels on a buffer that is part of the library's image: each GPU the library runs
+// on holds its own copy of `scratch` from the first use until the process ends.
+constexpr int kNoAllocMaxRows = 65536;                           // batch * nlocal, 4.5 MiB of partial sums
+static __device__ __align__(256) double scratch[(size_t)kNoAllocMaxRows * 9];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+double* g_scratch_ptr[kMaxDevices];                              // device address of `scratch`, per device
+
+// Device address of `scratch` on the current device (its name is only a host-side stand-in).
+int scratch_address(double** out)
+{
+    int dev = -1;
+    A2P_HIP_CHECK(hipGetDevice(&dev));
+    A2P_REQUIRE(dev >= 0 && dev < kMaxDevices, A2P_ERR_INVALID, "fvt virial (no allocation): device %d not supported", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        A2P_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        A2P_REQUIRE(p != nullptr, A2P_ERR_HIP, "fvt virial (no allocation): scratch has no device address");
+        g_scratch_ptr[dev] = (double*)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return A2P_OK;
+}
+
+int virial_fwd_noalloc(int B, int P, int U, const int* bnumneigh, const float* rcs, const float* dei, float* virial,
+                       hipStream_t stream)
+{
+    int rc = check_shape(B, P, U, 0);
+    if (rc) return rc;
+    A2P_REQUIRE(bnumneigh && rcs && dei && virial, A2P_ERR_INVALID, "fvt virial: null pointer");
+    A2P_REQUIRE((long long)B * P <= kNoAllocMaxRows, A2P_ERR_INVALID,
+                "fvt virial (no allocation): batch * nlocal = %lld exceeds the %d rows of the built-in scratch; "
+                "use a2p_fvt_virial_fwd_f32", (long long)B * P, kNoAllocMaxRows);
+    if (B == 0) return A2P_OK;
+    double* partial = nullptr;
+    rc = scratch_address(&partial);
+    if (rc) return rc;
+    // every row below batch * nlocal is written by the first kernel before the second reads it, so
+    // what an earlier call left in the buffer never shows; nlocal == 0 leaves nothing to sum (zeros)
+    if (P > 0) {
+        hipLaunchKernelGGL(virial_rows_kernel<float>, dim3(ceil_div((long long)B * P * 64, 256)), dim3(256), 0, stream,
+                           partial, dei, rcs, B, P, U, bnumneigh);
+        A2P_HIP_CHECK(hipGetLastError());
+    }
+    return finish_partials<float>(virial, (const double*)partial, B, P, 9, 9, 9, stream, false);
+}
+
 }  // namespace
 }  // namespace a2p
 
@@ -228,6 +282,9 @@ int a2p_fvt_virial_fwd_f32(int B, int P, int U, const int* bnumneigh, const floa
 int a2p_fvt_virial_fwd_f64(int B, int P, int U, const int* bnumneigh, const double* rcs, const double* dei,
                            double* virial, void* s)
 { return a2p::virial_fwd<double>(B, P, U, bnumneigh, rcs, dei, virial, (hipStream_t)s); }
+int a2p_fvt_virial_fwd_noalloc_f32(int B, int P, int U, const int* bnumneigh, const float* rcs, const float* dei,
+                                   float* virial, void* s)
+{ return a2p::virial_fwd_noalloc(B, P, U, bnumneigh, rcs, dei, virial, (hipStream_t)s); }
 int a2p_fvt_virial_bwd_f32(int B, int P, int U, const int* bnumneigh, const float* rcs, const float* dei,
                            const float* gV, float* gdei, float* grcs, void* s)
 { return a2p::virial_bwd<float>(B, P, U, bnumneigh, rcs, dei, gV, gdei, grcs, (hipStream_t)s); }

@@ -478,6 +478,16 @@ int a2p_fvt_virial_fwd_f32(int batch, int nlocal, int umax, const int* bnumneigh
                            const float* dei_drij, float* virial, void* stream);
 int a2p_fvt_virial_fwd_f64(int batch, int nlocal, int umax, const int* bnumneigh, const double* rcs,
                            const double* dei_drij, double* virial, void* stream);
+/* a2p_fvt_virial_fwd_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, same kernels and bit-identical results, but the row partial sums go to a buffer that is
+ * part of the library's image (4.5 MiB per GPU the library runs on, held until the process ends)
+ * instead of the growable workspace, and the call never allocates or frees anything: no hipMalloc,
+ * no hipFree, no event creation.  Limit: batch * nlocal <= 65536 rows; more returns A2P_ERR_INVALID.
+ * All calls on one GPU share the buffer, so calls that overlap in time on one GPU (two streams, two
+ * host threads) race; order them on one stream or with events. */
+int a2p_fvt_virial_fwd_noalloc_f32(int batch, int nlocal, int umax, const int* bnumneigh, const float* rcs,
+                                   const float* dei_drij, float* virial, void* stream);
 int a2p_fvt_virial_bwd_f32(int batch, int nlocal, int umax, const int* bnumneigh, const float* rcs,
                            const float* dei_drij, const float* grad_virial, float* grad_dei, float* grad_rcs,
                            void* stream);
