@@ -25,7 +25,13 @@ class NepCalculator:
     """Holds one NEP model and the neighbour buffers of one structure size."""
 
     def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
-                 sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None):
+                 sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None, path="auto",
+                 padded=True):
+        """path: "gather" evaluates forces as a gather over compact lists cut by the list build (common
+        model shapes, unsorted rows, umax % 8 == 0); "segments" scatters pair derivatives into reduction
+        segments from the padded arrays (any model shape); "auto" takes the gather when it applies.
+        padded=False (gather only) skips the padded firstneigh / rcs arrays: the step then produces
+        energy, forces and virial alone."""
         self.device = torch.device(device)
         self.dtype = dtype
         self.n = int(natoms)
@@ -71,6 +77,27 @@ class NepCalculator:
         self.places_from_list = bool(places_from_list)
         if self.places_from_list and self.sort:
             raise ValueError("places_from_list needs sort=False")
+        L.a2p_nblist_compact_bytes.restype = _c.c_size_t
+        elem = _c.c_int(4 if f32 else 8)
+        can_gather = (not self.sort and not self.places_from_list and
+                      self.umax * (16 if f32 else 28) * 4 <= 32 * 1024 and      # a row per wavefront in LDS
+                      L.a2p_nblist_compact_bytes(_c.c_int(n), _c.c_int(U), elem) > 0 and
+                      L.a2p_nep_efv_compact_supported(_c.c_int(model["chebyshev_size"]), _c.c_int(model["n_radial_basis"]),
+                                                      _c.c_int(model["n_angular_basis"]), _c.c_int(model["l_max"]),
+                                                      _c.c_int(self.H), _c.c_int(self.ntypes), elem) == 1)
+        if path not in ("auto", "gather", "segments"):
+            raise ValueError("path must be auto, gather or segments")
+        if path == "gather" and not can_gather:
+            raise ValueError("the gather path does not cover this model shape / list options")
+        self.path = "gather" if (path != "segments" and can_gather) else "segments"
+        self.padded = bool(padded) or self.path != "gather"
+        if self.path == "gather":
+            nbytes = L.a2p_nblist_compact_bytes(_c.c_int(n), _c.c_int(U), elem)
+            self.compact = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            self._nbl_compact = L.a2p_nblist_build_compact_f32 if f32 else L.a2p_nblist_build_compact_f64
+            self._efv_compact = L.a2p_nep_efv_compact_f32 if f32 else L.a2p_nep_efv_compact_f64
+            if not self.padded:
+                self.ilist = self.numneigh = self.firstneigh = self.rcs = self.types_out = None
         self.rank = None
         self.incoming = None
         self._evals = 0          # evaluations of the current list
@@ -87,7 +114,16 @@ class NepCalculator:
     def rebuild(self, coords, stream):
         # after the first build the list buffers hold a valid list: later builds write each row
         # only as far as its old or new length reaches
-        if self.places_from_list:
+        if self.path == "gather":
+            m = self.m
+            rc = self._nbl_compact(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
+                                   _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
+                                   self.pbc.ctypes.data_as(_c.c_void_p),
+                                   _c.c_int(1 if (self._have_list and self.padded) else 0),
+                                   _c.c_double(m["rmax_radial"]), _c.c_double(m["rmax_angular"]),
+                                   _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
+                                   _vp(self.types_out), _vp(self.compact), stream)
+        elif self.places_from_list:
             rc = self._nbl_ranked(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
                                   _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
                                   self.pbc.ctypes.data_as(_c.c_void_p), _c.c_int(1 if self._have_list else 0),
@@ -108,6 +144,17 @@ class NepCalculator:
 
     def evaluate(self, stream):
         m = self.m
+        if self.path == "gather":
+            rc = self._efv_compact(_c.c_int(m["chebyshev_size"]), _c.c_int(m["n_radial_basis"]),
+                                   _c.c_int(m["n_angular_basis"]), _c.c_int(m["l_max"]), _c.c_int(self.H),
+                                   _c.c_int(self.ntypes), _vp(self.coeffs), _vp(self.w0), _vp(self.b0), _vp(self.w1),
+                                   _vp(self.bias), _vp(self.q_scaler), _c.c_double(m["rmax_radial"]),
+                                   _c.c_double(m["rmax_angular"]), _c.c_int(self.n), _c.c_int(self.umax),
+                                   _vp(self.types), _vp(self.compact), _vp(self.etot), _vp(self.force),
+                                   _vp(self.virial), stream)
+            _lib.check(rc)
+            self._evals += 1
+            return
         ranked = self._places or self._evals >= 1
         if ranked:
             self._alloc_places()

@@ -24,6 +24,9 @@
 // This translation unit is compiled with -ffp-contract=off and spells the critical
 // operations with the *_rn intrinsics: no fused multiply-add may change a rounding.
 #include "a2p_common.h"
+#include "compact_list.h"
+
+#include <hipcub/hipcub.hpp>
 
 #include <climits>
 #include <cmath>
@@ -237,9 +240,11 @@ __global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int*
 // ---- 5. order inside a bin: descending supercell index (head insertion, binLinkedList.h:833) -
 // Afterwards only the atom behind a supercell entry matters (neighborList.h:561), so the sorted
 // indices are reduced modulo natoms here, once per entry instead of once per candidate pair.
+// With `types` the species of the atom rides in the bits above CL_TYPE_SHIFT (compact lists: the list
+// kernel then never gathers a neighbour's species).
 template <typename T>
 __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* __restrict__ s_idx,
-                               T* __restrict__ s_x, int natoms)
+                               T* __restrict__ s_x, int natoms, const int* __restrict__ types)
 {
     const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (b >= nbins) return;
@@ -260,7 +265,37 @@ __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* 
         s_x[(size_t)(j + 1) * 3 + 1] = ky;
         s_x[(size_t)(j + 1) * 3 + 2] = kz;
     }
-    for (int i = beg; i < end; i++) s_idx[i] %= natoms;
+    for (int i = beg; i < end; i++) {
+        const int at = s_idx[i] % natoms;
+        s_idx[i] = types ? at | ((types[at] & 15) << CL_TYPE_SHIFT) : at;
+    }
+}
+
+// ---- processing order of the compact lists: atoms along a Morton curve through the bins ----------
+__device__ __forceinline__ unsigned spread3(unsigned v)      // 10 bits -> every third bit
+{
+    v &= 0x3ffu;
+    v = (v | (v << 16)) & 0x030000ffu;
+    v = (v | (v << 8)) & 0x0300f00fu;
+    v = (v | (v << 4)) & 0x030c30c3u;
+    v = (v | (v << 2)) & 0x09249249u;
+    return v;
+}
+
+template <typename T>
+__global__ void order_keys_kernel(const Grid<T> g, const T* __restrict__ x, int shift, unsigned* __restrict__ keys,
+                                  int* __restrict__ vals)
+{
+    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (p >= g.N) return;
+    unsigned b[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        const int bin = bin_of(x[(size_t)p * 3 + a], g.mn[a], g.bin_size) - g.rlo[a];
+        b[a] = (unsigned)min(max(bin, 0), g.rdim[a] - 1) >> shift;
+    }
+    keys[p] = spread3(b[0]) | (spread3(b[1]) << 1) | (spread3(b[2]) << 2);
+    vals[p] = p;
 }
 
 // squared distance as the reference forms it: differences in T, squares and sum in double,
@@ -367,14 +402,44 @@ __device__ __forceinline__ void column_setup(const Grid<T>& g, const T (&c)[3], 
 
 constexpr int NBL_APW = 2;         // consecutive centre atoms per wavefront
 
-template <typename T, bool SORT, bool ROWBUF, bool RANK>
+// Compact lists (compact_list.h) written next to, or instead of, the padded rows.  The wavefront
+// that holds a finished row in LDS sorts its entries into the two ends of the position's slots:
+// beyond `split` (and within `outer`) from slot 0 upwards, within `split` from slot umax-1 downwards.
+template <typename T>
+struct CompactEmit {
+    const int* order;   // position -> atom
+    T* entries;
+    int* n_outer;
+    int* n_inner;
+    int nch;
+    T split, outer;
+    int write_rows;     // the padded outputs are wanted as well
+};
+
+template <typename T>
+__device__ __forceinline__ void entry_store(T* p, T x, T y, T z, int bits);
+template <>
+__device__ __forceinline__ void entry_store<float>(float* p, float x, float y, float z, int bits)
+{
+    *reinterpret_cast<float4*>(p) = make_float4(x, y, z, __int_as_float(bits));
+}
+template <>
+__device__ __forceinline__ void entry_store<double>(double* p, double x, double y, double z, int bits)
+{
+    *reinterpret_cast<double2*>(p) = make_double2(x, y);
+    *reinterpret_cast<double2*>(p + 2) = make_double2(z, __longlong_as_double((long long)bits));
+}
+
+template <typename T, bool SORT, bool ROWBUF, bool RANK, bool COMPACT = false>
 __global__ void __launch_bounds__(NBL_BLOCK)
 lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
              int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
              T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
-             int* __restrict__ status, int update, int* __restrict__ rank_out, int* __restrict__ incoming)
+             int* __restrict__ status, int update, int* __restrict__ rank_out, int* __restrict__ incoming,
+             const CompactEmit<T> ce = CompactEmit<T>{})
 {
+    static_assert(!COMPACT || (ROWBUF && !SORT && !RANK), "compact lists are cut from the row held in LDS");
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
     __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
@@ -396,17 +461,25 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     // wavefront takes NBL_APW atoms: all their coordinates are loaded first, and the column runs of
     // the next atom are requested before the candidates of the current one are scanned.
     T cs[NBL_APW][3];
+    int atom[NBL_APW];                            // the atom behind each of the wave's positions
+#pragma unroll
+    for (int a = 0; a < NBL_APW; a++) {
+        const int q = min(p0 + a, g.N - 1);
+        atom[a] = COMPACT ? ce.order[q] : q;
+    }
 #pragma unroll
     for (int a = 0; a < NBL_APW; a++)
 #pragma unroll
-        for (int d = 0; d < 3; d++) cs[a][d] = x[(size_t)min(p0 + a, g.N - 1) * 3 + d];
+        for (int d = 0; d < 3; d++) cs[a][d] = x[(size_t)atom[a] * 3 + d];
     const int nruns = (2 * g.ext_bins + 1) * (2 * g.ext_bins + 1);
     int start, len;
     column_setup<T>(g, cs[0], lane, offsets, start, len);
 #pragma unroll
     for (int ia = 0; ia < NBL_APW; ia++) {
     if (ia >= np) break;                          // wave-uniform
-    const int p = p0 + ia;
+    const int pos = p0 + ia;                      // position in processing order
+    const int p = atom[ia];                       // atom, row of the padded outputs
+    const bool rows = !COMPACT || ce.write_rows;  // wave-uniform
     const T (&c)[3] = cs[ia];
     int nstart = 0, nlen = 0;
     if (ia + 1 < NBL_APW && ia + 1 < np) column_setup<T>(g, cs[ia + 1 < NBL_APW ? ia + 1 : ia], lane, offsets, nstart, nlen);
@@ -424,7 +497,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
     const size_t rowi = (size_t)p * umax;
     // update of an earlier result held in the same buffers: beyond the row's old length the
     // padding is already in place
-    const int old_len = update ? min(max(numneigh[p], 0), umax) : umax;
+    const int old_len = (update && rows) ? min(max(numneigh[p], 0), umax) : umax;
     // NBL_UNROLL chunks of 64 candidates per trip: all their loads are issued before the first is
     // used, so a typical row (100 - 250 candidates) costs one memory round trip
     for (int c0 = 0; c0 < total; c0 += 64 * NBL_UNROLL) {
@@ -499,12 +572,47 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         }
     }
     if (lane == 0) {
-        ilist[p] = p;
-        numneigh[p] = cnt;
-        types_out[p] = types[p];
+        if (rows) {
+            ilist[p] = p;
+            numneigh[p] = cnt;
+            types_out[p] = types[p];
+        }
         if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
     }
-    if (ROWBUF) {
+    if (COMPACT) {
+        // the row's entries, 64 at a time: class by distance, place by ballot prefix, one 16-byte
+        // (fp32) store per entry; 8 consecutive slots of a position are contiguous in memory
+        __builtin_amdgcn_wave_barrier();
+        const int used = min(cnt, umax);
+        int n_outer = 0, n_inner = 0;
+        for (int e0 = 0; e0 < used; e0 += 64) {
+            const int e = e0 + lane;
+            const bool have = e < used;
+            const int ee = have ? e : 0;
+            const T dx = rb_rcs[ee * 3 + 0], dy = rb_rcs[ee * 3 + 1], dz = rb_rcs[ee * 3 + 2];
+            const int bits = rb_first[ee];
+            const T r = sizeof(T) == 4 ? (T)sqrtf((float)(dx * dx + dy * dy + dz * dz)) : (T)sqrt((double)(dx * dx + dy * dy + dz * dz));
+            const bool in_outer = have && r <= ce.outer;
+            const bool is_inner = in_outer && r <= ce.split;
+            const bool is_outer = in_outer && !is_inner;
+            const unsigned long long mi = __ballot(is_inner), mo = __ballot(is_outer);
+            const unsigned long long below = (1ull << lane) - 1ull;
+            int slot = -1;
+            if (is_inner) slot = umax - 1 - (n_inner + __popcll(mi & below));
+            if (is_outer) slot = n_outer + __popcll(mo & below);
+            if (slot >= 0) entry_store<T>(ce.entries + compact_slot_offset(ce.nch, pos, slot), dx, dy, dz, bits);
+            n_inner += __popcll(mi);
+            n_outer += __popcll(mo);
+        }
+        if (lane == 0) {
+            ce.n_outer[pos] = n_outer;
+            ce.n_inner[pos] = n_inner;
+        }
+        // the padded row lists plain indices
+        if (rows)
+            for (int e = lane; e < used; e += 64) rb_first[e] &= CL_INDEX_MASK;
+    }
+    if (ROWBUF && rows) {
         __builtin_amdgcn_wave_barrier();
         const uint4* s1 = reinterpret_cast<const uint4*>(rb_first);
         uint4* d1 = reinterpret_cast<uint4*>(firstneigh + rowi);
@@ -525,7 +633,7 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
             uint4* d3 = reinterpret_cast<uint4*>(rank_out + rowi);
             for (int i = lane; i < (used + 3) / 4; i += 64) d3[i] = s3[i];
         }
-    } else {
+    } else if (!ROWBUF) {
         // padding: -1 / 0 (neighborList.h:557, 563)
         const int first_pad = min(cnt, umax);
         const int last_pad = max(first_pad, old_len);
@@ -739,20 +847,40 @@ T host_plane_distance(const T* v, const T* n)        // structure.h:818-842, vec
     return std::abs(d);
 }
 
+// compact lists wanted from a build: the caller's buffer (compact_list.h) and the two cutoffs
+struct CompactOut {
+    void* buffer;
+    double split, outer;
+};
+
 template <typename T>
 int nblist_build(const T* lattice, const int* types, const T* coords, int N, double rcut_in, int umax,
                  int is_cart, const int* pbc, int sort, int* ilist, int* numneigh, int* firstneigh,
                  T* rcs, int* types_out, int* max_nn_host, hipStream_t stream, int update = 0,
-                 int* rank = nullptr, int* incoming = nullptr)
+                 int* rank = nullptr, int* incoming = nullptr, const CompactOut* co = nullptr)
 {
+    const bool want_rows = !co || (ilist || numneigh || firstneigh || rcs || types_out);
+    if (co) {
+        A2P_REQUIRE(co->buffer, A2P_ERR_INVALID, "nblist: null compact-list buffer");
+        A2P_REQUIRE(!sort && !rank, A2P_ERR_INVALID, "nblist: compact lists come with unsorted rows and without places");
+        A2P_REQUIRE(compact_supported(N, umax), A2P_ERR_INVALID,
+                    "nblist: compact lists need umax %% 8 == 0 and fewer than 2^28 atoms (natoms %d, umax %d)", N, umax);
+        A2P_REQUIRE(co->split > 0 && co->outer >= co->split, A2P_ERR_INVALID, "nblist: bad cutoffs for the compact lists");
+        A2P_REQUIRE(rowbuf_bytes<T>(umax, false) * (NBL_BLOCK / 64) <= 32 * 1024, A2P_ERR_INVALID,
+                    "nblist: umax %d too large for compact lists", umax);
+        A2P_REQUIRE(!want_rows || ((uintptr_t)firstneigh % 16 == 0 && (uintptr_t)rcs % 16 == 0), A2P_ERR_INVALID,
+                    "nblist: firstneigh and rcs must be 16-byte aligned");
+    }
     A2P_REQUIRE((rank == nullptr) == (incoming == nullptr), A2P_ERR_INVALID,
                 "nblist: rank and incoming come together");
     A2P_REQUIRE(!(rank && sort), A2P_ERR_INVALID, "nblist: places of the pairs are produced for unsorted rows only");
     A2P_REQUIRE(lattice && pbc, A2P_ERR_INVALID, "nblist: lattice and pbc must be host pointers");
     A2P_REQUIRE(N > 0, A2P_ERR_INVALID, "nblist: the structure has no atoms");   // binLinkedList.h:659
     A2P_REQUIRE(umax > 0 && rcut_in > 0, A2P_ERR_INVALID, "nblist: rcut and umax must be positive");
-    A2P_REQUIRE(types && coords && ilist && numneigh && firstneigh && rcs && types_out, A2P_ERR_INVALID,
-                "nblist: null device pointer");
+    A2P_REQUIRE(types && coords, A2P_ERR_INVALID, "nblist: null device pointer");
+    A2P_REQUIRE(!want_rows || (ilist && numneigh && firstneigh && rcs && types_out), A2P_ERR_INVALID,
+                "nblist: null device pointer (the padded outputs come all or none)");
+    A2P_REQUIRE(want_rows || !max_nn_host, A2P_ERR_INVALID, "nblist: the largest neighbour count needs the padded outputs");
     A2P_REQUIRE((long long)N * umax < (1ll << 31), A2P_ERR_INVALID, "nblist: natoms*umax exceeds 2^31");
 
     Grid<T> g;
@@ -901,14 +1029,54 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
-                       (int)nregion, offsets, s_idx, s_x, g.N);
+                       (int)nregion, offsets, s_idx, s_x, g.N, co ? types : (const int*)nullptr);
     prof_end(stream);
+    CompactEmit<T> ce{};
+    if (co) {
+        // processing order: atoms sorted by the Morton code of their bin (ties by index: the sort is stable)
+        const CompactView<T> cv = compact_view<T>(co->buffer, N, umax);
+        int maxdim = std::max(g.rdim[0], std::max(g.rdim[1], g.rdim[2]));
+        int shift = 0;
+        while ((maxdim >> shift) > 1024) shift++;
+        int bits = 1;
+        while ((1 << bits) < ((maxdim >> shift) + 1)) bits++;
+        size_t tmp_bytes = 0;
+        A2P_HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, (const unsigned*)nullptr, (unsigned*)nullptr,
+                                                         (const int*)nullptr, (int*)nullptr, N, 0, 3 * bits, stream));
+        const size_t key_bytes = (((size_t)N * sizeof(unsigned) + 255) / 256) * 256;
+        void* wsD = nullptr;
+        rc = ws_get(WS_CSR, 3 * key_bytes + tmp_bytes, &wsD);
+        if (rc) return rc;
+        unsigned* keys_in = (unsigned*)wsD;
+        unsigned* keys_out = (unsigned*)((char*)wsD + key_bytes);
+        int* vals_in = (int*)((char*)wsD + 2 * key_bytes);
+        void* tmp_sort = (char*)wsD + 3 * key_bytes;
+        prof_begin("nbl_order", stream);
+        hipLaunchKernelGGL(order_keys_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, shift, keys_in, vals_in);
+        prof_end(stream);
+        prof_begin("nbl_order", stream);
+        A2P_HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(tmp_sort, tmp_bytes, (const unsigned*)keys_in, keys_out,
+                                                         (const int*)vals_in, cv.order, N, 0, 3 * bits, stream));
+        prof_end(stream);
+        ce.order = cv.order;
+        ce.entries = cv.entries;
+        ce.n_outer = cv.n_outer;
+        ce.n_inner = cv.n_inner;
+        ce.nch = cv.nch;
+        ce.split = (T)co->split;
+        ce.outer = (T)co->outer;
+        ce.write_rows = want_rows ? 1 : 0;
+    }
     const int list_blocks = ceil_div(N, (NBL_BLOCK / 64) * NBL_APW);
     prof_begin("nbl_lists", stream);
     const size_t rows_lds = rowbuf_bytes<T>(umax, rank != nullptr) * (NBL_BLOCK / 64);
     const bool rowbuf = !sort && umax % 4 == 0 && rows_lds <= 32 * 1024 && (uintptr_t)firstneigh % 16 == 0 &&
                         (uintptr_t)rcs % 16 == 0 && (uintptr_t)rank % 16 == 0;
-    if (sort)
+    if (co)
+        hipLaunchKernelGGL((lists_kernel<T, false, true, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds,
+                           stream, g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out,
+                           keys, status, update, nullptr, nullptr, ce);
+    else if (sort)
         hipLaunchKernelGGL((lists_kernel<T, true, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
                            status, 0, nullptr, nullptr);
@@ -1033,5 +1201,33 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
     return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
                                      firstneigh, rcs, types_out, max_numneigh, (hipStream_t)stream, update ? 1 : 0,
                                      rank, incoming);
+}
+
+size_t a2p_nblist_compact_bytes(int natoms, int umax, int elem_size)
+{
+    if (!a2p::compact_supported(natoms, umax) || (elem_size != 4 && elem_size != 8)) return 0;
+    return a2p::compact_layout(natoms, umax, (size_t)elem_size).bytes;
+}
+
+int a2p_nblist_build_compact_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                                 double rcut, int umax, int is_cart, const int* pbc, int update, double rcut_outer,
+                                 double rcut_inner, int* ilist, int* numneigh, int* firstneigh, float* rcs,
+                                 int* types_out, void* compact, void* stream)
+{
+    const a2p::CompactOut co{compact, rcut_inner, rcut_outer};
+    return a2p::nblist_build<float>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
+                                    firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, update ? 1 : 0, nullptr,
+                                    nullptr, &co);
+}
+
+int a2p_nblist_build_compact_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                                 double rcut, int umax, int is_cart, const int* pbc, int update, double rcut_outer,
+                                 double rcut_inner, int* ilist, int* numneigh, int* firstneigh, double* rcs,
+                                 int* types_out, void* compact, void* stream)
+{
+    const a2p::CompactOut co{compact, rcut_inner, rcut_outer};
+    return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
+                                     firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, update ? 1 : 0, nullptr,
+                                     nullptr, &co);
 }
 }

@@ -1,0 +1,690 @@
+// NEP energy / force / virial by gather, for neighbour lists this library built itself
+// (a2p_nblist_build_compact_*: one periodic structure, no ghosts, every pair listed from both ends).
+//
+// The reference scatters: atom i computes g_ij = dE_i/dr_ij for each neighbour and does
+// F_i += g_ij, F_j -= g_ij (source/descriptor/nep/include/nep.h:468-515).  With a list that holds
+// every pair from both ends the same forces are a gather,
+//     F_i = sum_j (g_ij - g_ji),        V = -1/2 sum_i sum_j (g_ij - g_ji) r_ij^T,
+// and g_ji is a function of the SAME distance vector and of atom j's adjoints: its dE/dq
+// contracted with the radial coefficients, cc_j[t][k] = sum_n dE_j/dq_n c[t_j][t][n][k], and its
+// dE/dS_{n,lm}.  The harmonics have parity (-1)^l, so both directions share the basis functions,
+// the harmonics and their gradients; the second direction only adds the contraction of atom j's
+// adjoints with its own radial functions:
+//     A_lm = sum_n dE_i/dS_{n,lm} g_n^{ij}(r) + (-1)^l sum_n dE_j/dS_{n,lm} g_n^{ji}(r).
+// No per-pair store, no atomics, no reduction pass: two kernels over the atoms.
+//   nep_adjoint_kernel : radial sums and angular moments over the compact lists, descriptors,
+//                        hidden layer, dE/dq, dE/dS; stores a 128-value record per atom
+//                        (96 dE/dS + 4 x 8 contracted radial coefficients) and the energy partials
+//   nep_gather_kernel  : walks the lists again, gathers the neighbours' records, forms
+//                        g_ij - g_ji, sums force and virial
+// One thread per atom, 256 per workgroup.  Atoms are processed in the Morton order of the list
+// build and workgroups are dealt to the XCDs in contiguous runs, so the records a workgroup
+// gathers were written for, and are being gathered by, its neighbours in space and time.  The
+// lists are read in 8 KiB chunks (8 slots of 64 positions), staged through LDS by each wavefront
+// for itself: global loads are contiguous, LDS reads are one 16-byte entry per lane.
+//
+// Formulas: source/descriptor/nep/include/{nepBasis.h:57-196; nep.h:320-529}.
+#include "a2p_common.h"
+#include "compact_list.h"
+#include "nep_device.h"
+
+#include <type_traits>
+
+namespace a2p {
+using namespace nepdev;
+namespace {
+
+constexpr int CB = 256;                 // positions (threads) per workgroup
+constexpr int KC = 8, NAC = 4, LC = 4, NLM = 24, FDP = 24;
+constexpr int REC = 128;                // values per adjoint record
+constexpr int REC_CC = NAC * NLM;       // the contracted radial coefficients follow the 96 dE/dS
+constexpr int STP = CL_CHUNK + 1;       // staged slots per position, padded: 16-byte reads of 8 lanes hit 8 banks
+
+template <typename T>
+struct GatherArgs {
+    int H, ntypes;
+    const T *coeffs, *w0, *b0, *w1, *bias, *q_scaler;
+    T rr, ra;
+    CompactView<T> cv;
+    const int* types;     // [natoms]
+    T* rec;               // [natoms][REC]
+    T* force;             // [natoms][3] or null
+    double* partial;      // [nblocks][10]: energy (adjoint kernel), virial (gather kernel)
+    int* status;
+    int want_virial;
+};
+
+__device__ __forceinline__ void ld4(const float* p, float (&o)[4])
+{
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void ld4(const double* p, double (&o)[4])
+{
+    const double2 v0 = *reinterpret_cast<const double2*>(p);
+    const double2 v1 = *reinterpret_cast<const double2*>(p + 2);
+    o[0] = v0.x; o[1] = v0.y; o[2] = v1.x; o[3] = v1.y;
+}
+__device__ __forceinline__ void st4(float* p, const float (&v)[4])
+{
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void st4(double* p, const double (&v)[4])
+{
+    *reinterpret_cast<double2*>(p) = make_double2(v[0], v[1]);
+    *reinterpret_cast<double2*>(p + 2) = make_double2(v[2], v[3]);
+}
+__device__ __forceinline__ int entry_bits(float w) { return __float_as_int(w); }
+__device__ __forceinline__ int entry_bits(double w) { return (int)__double_as_longlong(w); }
+
+__host__ __device__ __forceinline__ size_t lds16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
+
+// Workgroups are handed to the 8 XCDs round robin; giving XCD k the k-th contiguous run of blocks
+// keeps neighbours in space on one L2.
+__device__ __forceinline__ int xcd_block(int w, int nb)
+{
+    const int per = nb >> 3, rem = nb & 7, k = w & 7;
+    return k * per + min(k, rem) + (w >> 3);
+}
+
+// One chunk (8 slots of the tile's 64 positions, contiguous in memory) into the wavefront's
+// staging buffer, position-major with STP slots per position.
+template <typename T>
+__device__ __forceinline__ void stage_chunk(const T* __restrict__ g, T* __restrict__ st, int lane)
+{
+    T v[CL_CHUNK][4];
+#pragma unroll
+    for (int it = 0; it < CL_CHUNK; it++) ld4(g + (size_t)(it * 64 + lane) * 4, v[it]);
+#pragma unroll
+    for (int it = 0; it < CL_CHUNK; it++) {
+        const int idx = it * 64 + lane;
+        st4(st + ((idx >> 3) * STP + (idx & 7)) * 4, v[it]);
+    }
+}
+
+// Walks one of the two lists of the wavefront's 64 positions: chunk after chunk through the staging
+// buffer, every lane making the trips of the longest list; body(valid, x, y, z, bits).  A lane past
+// the end of its own list gets a unit vector and valid = false.
+template <typename T, typename Body>
+__device__ __forceinline__ void walk_list(const CompactView<T>& cv, int tile, int lane, T* st, int n, bool inner,
+                                          Body&& body)
+{
+    const int trips = __builtin_amdgcn_readfirstlane(wave_max(n));
+    for (int c = 0; c * CL_CHUNK < trips; c++) {
+        const int chunk = inner ? cv.nch - 1 - c : c;
+        __builtin_amdgcn_wave_barrier();
+        stage_chunk<T>(cv.entries + compact_chunk_offset<T>(cv.nch, tile, chunk), st, lane);
+        __builtin_amdgcn_wave_barrier();
+        for (int s = 0; s < CL_CHUNK; s++) {
+            const int e = c * CL_CHUNK + s;
+            if (e >= trips) break;                               // wave-uniform
+            T v[4];
+            ld4(st + (lane * STP + (inner ? CL_CHUNK - 1 - s : s)) * 4, v);
+            const bool valid = e < n;
+            body(valid, valid ? v[0] : (T)1, valid ? v[1] : (T)0, valid ? v[2] : (T)0, entry_bits(v[3]));
+        }
+    }
+}
+
+// position -> atom, species, list lengths; with the checks
+template <typename T>
+__device__ __forceinline__ bool position_header(const GatherArgs<T>& a, int p, int& atom, int& ti, int& n_outer,
+                                                int& n_inner)
+{
+    atom = 0; ti = 0; n_outer = 0; n_inner = 0;
+    if (p >= a.cv.natoms) return false;
+    atom = a.cv.order[p];
+    if ((unsigned)atom >= (unsigned)a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); atom = 0; return false; }
+    ti = a.types[atom];
+    if ((unsigned)ti >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); ti = 0; return false; }
+    n_outer = a.cv.n_outer[p];
+    n_inner = a.cv.n_inner[p];
+    if (n_outer < 0 || n_inner < 0 || n_outer + n_inner > a.cv.umax) {
+        atomicOr(a.status, ST_NEIGH_OVERFLOW);
+        n_outer = 0; n_inner = 0;
+    }
+    return true;
+}
+
+template <typename T>
+struct AdjointLds {
+    T *coef, *w0, *b0, *w1, *qs, *stage;
+    double* red;
+};
+template <typename T>
+__host__ __device__ __forceinline__ size_t adjoint_lds(int nt, int H, int nb, unsigned char* base, AdjointLds<T>& L)
+{
+    size_t off = 0;
+    L.coef = (T*)(base + off);  off += lds16((size_t)nt * nt * nb * KC * sizeof(T));
+    L.w0 = (T*)(base + off);    off += lds16((size_t)nt * H * FDP * sizeof(T));
+    L.b0 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
+    L.w1 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
+    L.qs = (T*)(base + off);    off += lds16((size_t)FDP * sizeof(T));
+    L.stage = (T*)(base + off); off += lds16((size_t)(CB / 64) * 64 * STP * 4 * sizeof(T));
+    L.red = (double*)(base + off); off += lds16((size_t)(CB / 64) * sizeof(double));
+    return off;
+}
+
+template <typename T>
+struct GatherLds {
+    T *coef, *acc, *stage;
+    double* red;
+};
+template <typename T>
+__host__ __device__ __forceinline__ size_t gather_lds(int nt, int ntc, int nb, unsigned char* base, GatherLds<T>& L)
+{
+    size_t off = 0;
+    L.coef = (T*)(base + off);  off += lds16((size_t)nt * nt * nb * KC * sizeof(T));
+    L.acc = (T*)(base + off);   off += lds16((size_t)ntc * KC * CB * sizeof(T));
+    L.stage = (T*)(base + off); off += lds16((size_t)(CB / 64) * 64 * STP * 4 * sizeof(T));
+    L.red = (double*)(base + off); off += lds16((size_t)(CB / 64) * 9 * sizeof(double));
+    return off;
+}
+
+// ---- kernel 1: descriptors, hidden layer, adjoints -------------------------------------------------
+template <typename T, int NTC, int NR>
+__global__ void __launch_bounds__(CB, (sizeof(T) == 4 ? 2 : 1))
+nep_adjoint_kernel(const GatherArgs<T> a)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int NB = NR + NAC, DC = NR + NAC * LC;
+    static_assert(DC <= FDP, "descriptor count exceeds the padded row");
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int blk = xcd_block(blockIdx.x, gridDim.x);
+    const int p = blk * CB + tid;
+    const int tile = p >> 6;
+    const int nt = a.ntypes, H = a.H;
+    AdjointLds<T> L;
+    adjoint_lds<T>(nt, H, NB, smem_raw, L);
+    T* const st = L.stage + (size_t)wv * 64 * STP * 4;
+
+    for (int i = tid; i < nt * nt * NB * KC; i += CB) L.coef[i] = a.coeffs[i];
+    for (int i = tid; i < nt * H * FDP; i += CB) {
+        const int r = i / FDP, j = i - r * FDP;
+        L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
+    }
+    for (int i = tid; i < nt * H; i += CB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
+    if (tid < FDP) L.qs[tid] = tid < DC ? (T)1 / a.q_scaler[tid] : (T)0;
+
+    int atom, ti, n_outer, n_inner;
+    const bool active = position_header<T>(a, p, atom, ti, n_outer, n_inner);
+    const T rr_inv = (T)1 / a.rr, ra_inv = (T)1 / a.ra;
+
+    T F[NTC][KC];                 // radial functions summed per neighbour species
+#pragma unroll
+    for (int t = 0; t < NTC; t++)
+#pragma unroll
+        for (int k = 0; k < KC; k++) F[t][k] = (T)0;
+    T S[NAC][NLM];
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int m = 0; m < NLM; m++) S[n][m] = (T)0;
+    __syncthreads();
+
+    // neighbours inside the angular cutoff: radial sums and angular moments
+    walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+        const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
+        const T r = sqrt_t(x * x + y * y + z * z);
+        const T rinv = (T)1 / r;
+        T f[KC], df[KC];
+        radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+        for (int t = 0; t < NTC; t++)
+#pragma unroll
+            for (int k = 0; k < KC; k++) F[t][k] += (valid && tj == t) ? f[k] : (T)0;
+        radial_basis<T, KC, false>(r, ra_inv, KC, f, df);
+        const T* c = L.coef + ((ti * nt + tj) * NB + NR) * KC;
+        T bl[NLM];
+        blm_values<T, LC>(x * rinv, y * rinv, z * rinv, bl);
+#pragma unroll
+        for (int n = 0; n < NAC; n++) {
+            T c0v[4], c1v[4];
+            ld4(c + n * KC, c0v);
+            ld4(c + n * KC + 4, c1v);
+            T g = (T)0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) g += c0v[k] * f[k];
+#pragma unroll
+            for (int k = 0; k < 4; k++) g += c1v[k] * f[4 + k];
+            g = valid ? g : (T)0;
+#pragma unroll
+            for (int m = 0; m < NLM; m++) S[n][m] += g * bl[m];
+        }
+    });
+    // neighbours between the cutoffs: radial sums only
+    walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+        const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
+        const T r = sqrt_t(x * x + y * y + z * z);
+        T f[KC], df[KC];
+        radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+#pragma unroll
+        for (int t = 0; t < NTC; t++)
+#pragma unroll
+            for (int k = 0; k < KC; k++) F[t][k] += (valid && tj == t) ? f[k] : (T)0;
+    });
+
+    // ---- descriptors (nepBasis.h:174-190) -------------------------------------------------------
+    T q[DC];
+#pragma unroll
+    for (int j = 0; j < DC; j++) q[j] = (T)0;
+#pragma unroll
+    for (int t = 0; t < NTC; t++) {
+        if (t < nt) {
+            const T* c = L.coef + (ti * nt + t) * NB * KC;
+#pragma unroll
+            for (int n = 0; n < NR; n++) {
+                T c0v[4], c1v[4];
+                ld4(c + n * KC, c0v);
+                ld4(c + n * KC + 4, c1v);
+#pragma unroll
+                for (int k = 0; k < 4; k++) q[n] += c0v[k] * F[t][k];
+#pragma unroll
+                for (int k = 0; k < 4; k++) q[n] += c1v[k] * F[t][4 + k];
+            }
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int l = 1; l <= LC; l++) {
+            T acc = (T)0;
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                acc += (T)(mp == 0 ? 1.0 : 2.0) * (T)kC3B[m] * S[n][m] * S[n][m];
+            }
+            q[NR + n * LC + (l - 1)] = acc;
+        }
+
+    // ---- hidden layer (nep.h:415-447) --------------------------------------------------------------
+    T dEdq[DC];
+    T e_site = active ? a.bias[ti] : (T)0;
+    {
+        T qn[DC];
+#pragma unroll
+        for (int j = 0; j < DC; j++) { qn[j] = q[j] * L.qs[j]; dEdq[j] = (T)0; }
+        for (int pn = 0; pn < H; pn++) {
+            const T* wrow = L.w0 + (size_t)(ti * H + pn) * FDP;
+            T wv_[FDP];
+#pragma unroll
+            for (int j = 0; j < FDP; j += 4) {
+                T v[4];
+                ld4(wrow + j, v);
+                wv_[j] = v[0]; wv_[j + 1] = v[1]; wv_[j + 2] = v[2]; wv_[j + 3] = v[3];
+            }
+            T h = L.b0[ti * H + pn];
+#pragma unroll
+            for (int j = 0; j < DC; j++) h += wv_[j] * qn[j];
+            const T t = tanh_t(h);
+            const T w1p = L.w1[ti * H + pn];
+            e_site += active ? w1p * t : (T)0;
+            const T sde = w1p * ((T)1 - t * t);
+#pragma unroll
+            for (int j = 0; j < DC; j++) dEdq[j] += sde * wv_[j];
+        }
+#pragma unroll
+        for (int j = 0; j < DC; j++) dEdq[j] *= L.qs[j];
+    }
+
+    // ---- the atom's record: dE/dS (nep.h:450-466) and the radial coefficients contracted with dE/dq
+    if (active) {
+        T* rp = a.rec + (size_t)atom * REC;
+#pragma unroll
+        for (int n = 0; n < NAC; n++)
+#pragma unroll
+            for (int m0 = 0; m0 < NLM; m0 += 4) {
+                T v[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int m = m0 + u;
+                    const int l = m < 3 ? 1 : m < 8 ? 2 : m < 15 ? 3 : 4;
+                    const int mp = m - (l * l - 1);
+                    v[u] = S[n][m] * dEdq[NR + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+                }
+                st4(rp + n * NLM + m0, v);
+            }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            T cc[KC];
+#pragma unroll
+            for (int k = 0; k < KC; k++) cc[k] = (T)0;
+            if (t < NTC && t < nt) {
+                const T* c = L.coef + (ti * nt + t) * NB * KC;
+#pragma unroll
+                for (int n = 0; n < NR; n++) {
+                    T c0v[4], c1v[4];
+                    ld4(c + n * KC, c0v);
+                    ld4(c + n * KC + 4, c1v);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { cc[k] += dEdq[n] * c0v[k]; cc[4 + k] += dEdq[n] * c1v[k]; }
+                }
+            }
+            T lo[4] = {cc[0], cc[1], cc[2], cc[3]}, hi[4] = {cc[4], cc[5], cc[6], cc[7]};
+            st4(rp + REC_CC + t * KC, lo);
+            st4(rp + REC_CC + t * KC + 4, hi);
+        }
+    }
+
+    // ---- workgroup partial sum of the energy (fp64) -------------------------------------------------
+    const double ew = wave_sum(active ? (double)e_site : 0.0);
+    if (lane == 0) L.red[wv] = ew;
+    __syncthreads();
+    if (tid == 0) {
+        double v = 0.0;
+        for (int w = 0; w < CB / 64; w++) v += L.red[w];
+        a.partial[(size_t)blk * 10] = v;
+    }
+}
+
+// ---- kernel 2: forces and virial by gather ------------------------------------------------------------
+template <typename T, int NTC, int NR>
+__global__ void __launch_bounds__(CB, (sizeof(T) == 4 ? 2 : 1))
+nep_gather_kernel(const GatherArgs<T> a)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int NB = NR + NAC;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int blk = xcd_block(blockIdx.x, gridDim.x);
+    const int p = blk * CB + tid;
+    const int tile = p >> 6;
+    const int nt = a.ntypes;
+    GatherLds<T> L;
+    gather_lds<T>(nt, NTC, NB, smem_raw, L);
+    T* const st = L.stage + (size_t)wv * 64 * STP * 4;
+
+    for (int i = tid; i < nt * nt * NB * KC; i += CB) L.coef[i] = a.coeffs[i];
+
+    int atom, ti, n_outer, n_inner;
+    const bool active = position_header<T>(a, p, atom, ti, n_outer, n_inner);
+    const T rr_inv = (T)1 / a.rr, ra_inv = (T)1 / a.ra;
+    const T* const own = a.rec + (size_t)atom * REC;
+
+    // own adjoints: dE/dS in registers, contracted radial coefficients in LDS (indexed by the
+    // neighbour's species inside the loops)
+    T S[NAC][NLM];
+#pragma unroll
+    for (int n = 0; n < NAC; n++)
+#pragma unroll
+        for (int m0 = 0; m0 < NLM; m0 += 4) {
+            T v[4] = {(T)0, (T)0, (T)0, (T)0};
+            if (active) ld4(own + n * NLM + m0, v);
+#pragma unroll
+            for (int u = 0; u < 4; u++) S[n][m0 + u] = v[u];
+        }
+#pragma unroll
+    for (int t = 0; t < NTC; t++) {
+        T lo[4] = {(T)0, (T)0, (T)0, (T)0}, hi[4] = {(T)0, (T)0, (T)0, (T)0};
+        if (active) { ld4(own + REC_CC + t * KC, lo); ld4(own + REC_CC + t * KC + 4, hi); }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            L.acc[(t * KC + k) * CB + tid] = lo[k];
+            L.acc[(t * KC + 4 + k) * CB + tid] = hi[k];
+        }
+    }
+    __syncthreads();
+
+    T fx = (T)0, fy = (T)0, fz = (T)0;
+    T vir[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vir[i] = (T)0;
+    auto add_pair = [&](bool valid, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
+        gx = valid ? gx : (T)0; gy = valid ? gy : (T)0; gz = valid ? gz : (T)0;
+        fx += gx; fy += gy; fz += gz;
+        vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
+        vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
+        vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
+    };
+    // the neighbour behind an entry: its index (checked; an invalid entry points at the atom
+    // itself, so that every gather stays inside the records) and its species
+    auto neighbour = [&](bool& valid, int bits, int& j, int& tj) __attribute__((always_inline)) {
+        j = bits & CL_INDEX_MASK;
+        if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
+        j = valid ? j : atom;
+        tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
+    };
+
+    // pairs inside the angular cutoff: radial and angular part, both directions
+    walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+        int j, tj;
+        neighbour(valid, bits, j, tj);
+        const T* const rj = a.rec + (size_t)j * REC;
+        const T r = sqrt_t(x * x + y * y + z * z);
+        const T rinv = (T)1 / r;
+        const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+        T f[KC], df[KC];
+        // radial part: (cc_i[tj] + cc_j[ti]) . f'(r)
+        T srad = (T)0;
+        {
+            T lo[4], hi[4];
+            ld4(rj + REC_CC + ti * KC, lo);
+            ld4(rj + REC_CC + ti * KC + 4, hi);
+            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                srad += (L.acc[(tj * KC + k) * CB + tid] + lo[k]) * df[k];
+                srad += (L.acc[(tj * KC + 4 + k) * CB + tid] + hi[k]) * df[4 + k];
+            }
+        }
+        radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+        const T* ci = L.coef + ((ti * nt + tj) * NB + NR) * KC;
+        const T* cj = L.coef + ((tj * nt + ti) * NB + NR) * KC;
+        T A[NLM], Ad[NLM];
+#pragma unroll
+        for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
+#pragma unroll
+        for (int n = 0; n < NAC; n++) {
+            T c0v[4], c1v[4];
+            ld4(ci + n * KC, c0v);
+            ld4(ci + n * KC + 4, c1v);
+            T g = (T)0, dg = (T)0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
+#pragma unroll
+            for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
+#pragma unroll
+            for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
+            // the other direction: atom j's adjoints with its own radial functions, parity (-1)^l
+            ld4(cj + n * KC, c0v);
+            ld4(cj + n * KC + 4, c1v);
+            T gj = (T)0, dgj = (T)0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) { gj += c0v[k] * f[k]; dgj += c0v[k] * df[k]; }
+#pragma unroll
+            for (int k = 0; k < 4; k++) { gj += c1v[k] * f[4 + k]; dgj += c1v[k] * df[4 + k]; }
+#pragma unroll
+            for (int m0 = 0; m0 < NLM; m0 += 4) {
+                T sj[4];
+                ld4(rj + n * NLM + m0, sj);
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int m = m0 + u;
+                    const bool odd = m < 3 || (m >= 8 && m < 15);           // l = 1 or 3
+                    A[m] += sj[u] * (odd ? -gj : gj);
+                    Ad[m] += sj[u] * (odd ? -dgj : dgj);
+                }
+            }
+        }
+        T bl[NLM];
+        blm_values<T, LC>(ux, uy, uz, bl);
+#pragma unroll
+        for (int l = 1; l <= LC; l++)
+#pragma unroll
+            for (int mp = 0; mp < 2 * l + 1; mp++) {
+                const int m = l * l - 1 + mp;
+                srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+            }
+        T wx = (T)0, wy = (T)0, wz = (T)0;
+        blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
+        add_pair(valid, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
+    });
+    // pairs between the cutoffs: radial part only
+    walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+        int j, tj;
+        neighbour(valid, bits, j, tj);
+        const T* const rj = a.rec + (size_t)j * REC;
+        T lo[4], hi[4];
+        ld4(rj + REC_CC + ti * KC, lo);
+        ld4(rj + REC_CC + ti * KC + 4, hi);
+        const T r = sqrt_t(x * x + y * y + z * z);
+        T f[KC], df[KC];
+        radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+        T sr = (T)0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            sr += (L.acc[(tj * KC + k) * CB + tid] + lo[k]) * df[k];
+            sr += (L.acc[(tj * KC + 4 + k) * CB + tid] + hi[k]) * df[4 + k];
+        }
+        sr /= r;
+        add_pair(valid, x, y, z, sr * x, sr * y, sr * z);
+    });
+
+    if (active && a.force) {
+        T* fo = a.force + (size_t)atom * 3;
+        fo[0] = fx; fo[1] = fy; fo[2] = fz;
+    }
+    // every pair was met from both ends: half of the sum is the virial
+    if (a.want_virial) {
+        double vals[9];
+#pragma unroll
+        for (int i = 0; i < 9; i++) vals[i] = active ? 0.5 * (double)vir[i] : 0.0;
+#pragma unroll
+        for (int i = 0; i < 9; i++) {
+            const double v = wave_sum(vals[i]);
+            if (lane == 0) L.red[wv * 9 + i] = v;
+        }
+        __syncthreads();
+        if (tid < 9) {
+            double v = 0.0;
+            for (int w = 0; w < CB / 64; w++) v += L.red[w * 9 + tid];
+            a.partial[(size_t)blk * 10 + 1 + tid] = v;
+        }
+    }
+}
+
+template <typename T, int NTC, int NR>
+int launch_gather(const GatherArgs<T>& a, int nblocks, bool pairs, hipStream_t stream)
+{
+    AdjointLds<T> la;
+    GatherLds<T> lg;
+    const size_t lds_a = adjoint_lds<T>(a.ntypes, a.H, NR + NAC, nullptr, la);
+    const size_t lds_g = gather_lds<T>(a.ntypes, NTC, NR + NAC, nullptr, lg);
+    auto ka = nep_adjoint_kernel<T, NTC, NR>;
+    auto kg = nep_gather_kernel<T, NTC, NR>;
+    if (lds_a > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a));
+    if (lds_g > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kg, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
+    prof_begin("nep_adjoint_kernel", stream);
+    hipLaunchKernelGGL(ka, dim3(nblocks), dim3(CB), lds_a, stream, a);
+    prof_end(stream);
+    if (pairs) {
+        prof_begin("nep_gather_kernel", stream);
+        hipLaunchKernelGGL(kg, dim3(nblocks), dim3(CB), lds_g, stream, a);
+        prof_end(stream);
+    }
+    A2P_HIP_CHECK(hipGetLastError());
+    return A2P_OK;
+}
+
+int ntc_of(int ntypes) { return ntypes <= 1 ? 1 : ntypes == 2 ? 2 : ntypes == 3 ? 3 : 4; }
+
+template <typename T>
+size_t compact_lds_need(int n_r, int H, int ntypes)
+{
+    AdjointLds<T> la;
+    GatherLds<T> lg;
+    return std::max(adjoint_lds<T>(ntypes, H, n_r + NAC, nullptr, la),
+                    gather_lds<T>(ntypes, ntc_of(ntypes), n_r + NAC, nullptr, lg));
+}
+
+bool compact_shape_ok(int K, int n_r, int n_a, int l_max, int H, int ntypes)
+{
+    return K == KC && (n_r == 4 || n_r == 6) && n_a == NAC && l_max == LC && ntypes >= 1 && ntypes <= 4 && H >= 1;
+}
+
+constexpr size_t kLdsLimit = 150 * 1024;
+
+template <typename T>
+int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coeffs, const T* w0, const T* b0,
+                    const T* w1, const T* bias, const T* q_scaler, double rr, double ra, int natoms, int umax,
+                    const int* types, void* compact, T* etot, T* force, T* virial, hipStream_t stream)
+{
+    A2P_REQUIRE(compact_shape_ok(K, n_r, n_a, l_max, H, ntypes), A2P_ERR_INVALID,
+                "nep (compact lists): model shape not covered (chebyshev_size 8, n_radial 4 or 6, n_angular 4, l_max 4, "
+                "at most 4 species); use the padded-list entry points");
+    A2P_REQUIRE(H >= 1, A2P_ERR_INVALID, "nep: num_neurons must be positive");
+    A2P_REQUIRE(compact_supported(natoms, umax), A2P_ERR_INVALID, "nep (compact lists): bad natoms / umax");
+    A2P_REQUIRE(rr > 0 && ra > 0, A2P_ERR_INVALID, "nep: cutoffs must be positive");
+    A2P_REQUIRE(coeffs && w0 && b0 && w1 && bias && q_scaler && types && compact && etot, A2P_ERR_INVALID,
+                "nep (compact lists): null pointer");
+    GatherArgs<T> a;
+    a.H = H; a.ntypes = ntypes;
+    a.coeffs = coeffs; a.w0 = w0; a.b0 = b0; a.w1 = w1; a.bias = bias; a.q_scaler = q_scaler;
+    a.rr = (T)rr; a.ra = (T)ra;
+    a.cv = compact_view<T>(compact, natoms, umax);
+    a.types = types;
+    a.force = force;
+    a.want_virial = virial != nullptr;
+    const int nblocks = ceil_div(a.cv.npad, CB);
+    {
+        const size_t need = compact_lds_need<T>(n_r, H, ntypes);
+        A2P_REQUIRE(need <= kLdsLimit, A2P_ERR_INVALID, "nep (compact lists): %zu bytes of LDS needed (num_neurons %d)",
+                    need, H);
+    }
+    void* ws = nullptr;
+    int rc = ws_get(WS_FLAGS, 64, &ws);
+    if (rc) return rc;
+    a.status = (int*)ws;
+    rc = ws_get(WS_PARTIAL, (size_t)nblocks * 10 * sizeof(double), &ws);
+    if (rc) return rc;
+    a.partial = (double*)ws;
+    rc = ws_get(WS_PAIR_G, (size_t)natoms * REC * sizeof(T), &ws);
+    if (rc) return rc;
+    a.rec = (T*)ws;
+    const bool pairs = force != nullptr || virial != nullptr;
+    auto launch = [&](auto nr) {
+        constexpr int NR = decltype(nr)::value;
+        switch (ntc_of(ntypes)) {
+        case 1: return launch_gather<T, 1, NR>(a, nblocks, pairs, stream);
+        case 2: return launch_gather<T, 2, NR>(a, nblocks, pairs, stream);
+        case 3: return launch_gather<T, 3, NR>(a, nblocks, pairs, stream);
+        default: return launch_gather<T, 4, NR>(a, nblocks, pairs, stream);
+        }
+    };
+    rc = n_r == 4 ? launch(std::integral_constant<int, 4>{}) : launch(std::integral_constant<int, 6>{});
+    if (rc) return rc;
+    return finish_energy_virial<T>(etot, virial, a.partial, 1, nblocks, stream);
+}
+
+}  // namespace
+}  // namespace a2p
+
+extern "C" {
+
+int a2p_nep_efv_compact_supported(int K, int n_r, int n_a, int l_max, int H, int ntypes, int elem_size)
+{
+    if (!a2p::compact_shape_ok(K, n_r, n_a, l_max, H, ntypes)) return 0;
+    if (elem_size == 4) return a2p::compact_lds_need<float>(n_r, H, ntypes) <= a2p::kLdsLimit;
+    if (elem_size == 8) return a2p::compact_lds_need<double>(n_r, H, ntypes) <= a2p::kLdsLimit;
+    return 0;
+}
+
+int a2p_nep_efv_compact_f32(int K, int n_r, int n_a, int l_max, int H, int ntypes, const float* coeffs,
+                            const float* w0, const float* b0, const float* w1, const float* bias,
+                            const float* q_scaler, double rr, double ra, int natoms, int umax, const int* types,
+                            void* compact, float* etot, float* force, float* virial, void* stream)
+{
+    return a2p::nep_efv_compact<float>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra,
+                                       natoms, umax, types, compact, etot, force, virial, (hipStream_t)stream);
+}
+
+int a2p_nep_efv_compact_f64(int K, int n_r, int n_a, int l_max, int H, int ntypes, const double* coeffs,
+                            const double* w0, const double* b0, const double* w1, const double* bias,
+                            const double* q_scaler, double rr, double ra, int natoms, int umax, const int* types,
+                            void* compact, double* etot, double* force, double* virial, void* stream)
+{
+    return a2p::nep_efv_compact<double>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra,
+                                        natoms, umax, types, compact, etot, force, virial, (hipStream_t)stream);
+}
+}

@@ -187,6 +187,58 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
                                 int* incoming, int* max_numneigh, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Device-resident step: compact neighbour lists + NEP E/F/V by gather.  Together the two calls
+ * replace the reference's inference pair  nblist.find_info4mlff(...)  ->  torch.ops.nep.nepToEFVOp(...)
+ * (ai2pot/utils/usepot.py:76-97, ai2pot/models/nep/nep.py:298-357) for ONE periodic structure
+ * without ghosts, when positions stay on the device.  No counterpart of the list format exists in
+ * the reference (its only format is the padded arrays of neighborList.h:532-578).
+ *
+ * a2p_nblist_build_compact_*: the build of a2p_nblist_build_* / a2p_nblist_update_* (sort = 0;
+ * update as there) that ALSO cuts every row into the caller's `compact` buffer of
+ * a2p_nblist_compact_bytes(natoms, umax, sizeof(T)) bytes: atoms in Morton order of their bins,
+ * per atom the neighbours with r <= rcut_outer as 16-byte (fp32) entries [r_j - r_i, index |
+ * species << 28], those with r <= rcut_inner kept apart from the rest (the radial and angular
+ * cutoffs of the model; rcut_inner <= rcut_outer <= rcut).  The five padded outputs are written,
+ * bit-identical to a2p_nblist_build_*, when they are given; pass all five NULL to skip them.
+ * Needs umax % 8 == 0, natoms < 2^28, species < 16, 16-byte aligned firstneigh / rcs.
+ *
+ * a2p_nep_efv_compact_*: energy, forces and virial of the structure from that buffer.  The list
+ * names every pair from both ends, so F_i = sum_j (g_ij - g_ji) is evaluated as a gather over
+ * atom i's own list with atom j's adjoints (nep.h:468-515 scatters the same terms): no atomics,
+ * no per-pair stores, results bit-reproducible.  Model shapes: chebyshev_size 8, n_radial 4 or 6,
+ * n_angular 4, l_max 4, at most 4 species (A2P_ERR_INVALID otherwise: use a2p_nep_efv_*).
+ * types[natoms] are the type indices the list was built with.  etot[1] is required; force[natoms][3]
+ * and virial[9] may be NULL.
+ * ------------------------------------------------------------------------------------------ */
+size_t a2p_nblist_compact_bytes(int natoms, int umax, int elem_size);   /* 0: not available for these sizes */
+
+/* 1 when a2p_nep_efv_compact_* covers the model (shape as above, tables fit in LDS), else 0 */
+int a2p_nep_efv_compact_supported(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
+                                  int ntypes, int elem_size);
+
+int a2p_nblist_build_compact_f32(const float* lattice, const int* types, const float* coords, int natoms,
+                                 double rcut, int umax, int is_cart, const int* pbc, int update, double rcut_outer,
+                                 double rcut_inner, int* ilist, int* numneigh, int* firstneigh, float* rcs,
+                                 int* types_out, void* compact, void* stream);
+
+int a2p_nblist_build_compact_f64(const double* lattice, const int* types, const double* coords, int natoms,
+                                 double rcut, int umax, int is_cart, const int* pbc, int update, double rcut_outer,
+                                 double rcut_inner, int* ilist, int* numneigh, int* firstneigh, double* rcs,
+                                 int* types_out, void* compact, void* stream);
+
+int a2p_nep_efv_compact_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons, int ntypes,
+                            const float* coeffs, const float* w0, const float* b0, const float* w1,
+                            const float* type_bias, const float* q_scaler, double rmax_radial, double rmax_angular,
+                            int natoms, int umax, const int* types, void* compact, float* etot, float* force,
+                            float* virial, void* stream);
+
+int a2p_nep_efv_compact_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons, int ntypes,
+                            const double* coeffs, const double* w0, const double* b0, const double* w1,
+                            const double* type_bias, const double* q_scaler, double rmax_radial, double rmax_angular,
+                            int natoms, int umax, const int* types, void* compact, double* etot, double* force,
+                            double* virial, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Linear Moment Tensor Potential.
  *
  * a2p_mtp_plan_create takes the three HOST tables the reference's mtpParamOp returns

@@ -1,0 +1,205 @@
+"""GPU parity of the device-resident step (compact neighbour lists + NEP E/F/V by gather,
+a2p_nblist_build_compact_* / a2p_nep_efv_compact_*) against the CPU oracle.
+
+Bars as for the scatter path: fp64 within 1e-10 relative, fp32 energies and virials within 1e-5
+relative, fp32 forces within 1e-4 eV/A absolute + 1e-5 relative; padded lists bit-exact; the compact
+lists hold exactly the oracle's pairs with bit-identical relative vectors."""
+import ctypes as c
+
+import numpy as np
+import pytest
+
+from ai2pot_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(out, ref, np_dtype):
+    e, f, v = out
+    er, fr, vr = ref
+    er, fr, vr = np.asarray(er).ravel(), np.asarray(fr).reshape(-1, 3), np.asarray(vr).reshape(9)
+    e, f, v = e.ravel(), f.reshape(-1, 3), v.reshape(9)
+    if np_dtype == np.float64:
+        assert np.allclose(e, er, rtol=1e-10, atol=0)
+        assert np.abs(f - fr).max() <= 1e-10 * max(np.abs(fr).max(), 1e-30)
+        assert np.abs(v - vr).max() <= 1e-10 * max(np.abs(vr).max(), 1e-30)
+    else:
+        assert np.allclose(e, er, rtol=1e-5, atol=0)
+        assert np.all(np.abs(f - fr) <= 1e-4 + 1e-5 * np.abs(fr))
+        assert np.abs(v - vr).max() <= 1e-5 * np.abs(vr).max()
+
+
+def _calc(m, lat, ty, n, np_dtype, umax=200, **kw):
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    dtype = torch.float32 if np_dtype == np.float32 else torch.float64
+    return NepCalculator(m, n, lat, ty, umax=umax, dtype=dtype, device="cuda:0", **kw)
+
+
+def _step(calc, pos, np_dtype):
+    import torch
+    e, f, v = calc.step(torch.from_numpy(pos.astype(np_dtype)).to("cuda:0"))
+    torch.cuda.synchronize()
+    calc.check()
+    return e.cpu().numpy().copy(), f.cpu().numpy().copy(), v.cpu().numpy().copy()
+
+
+def _decode_compact(calc, np_dtype):
+    """Host view of the compact buffer (layout of csrc/compact_list.h): per atom the set of
+    (index, species, x, y, z) of the two classes."""
+    n, U = calc.n, calc.umax
+    elem = 4 if np_dtype == np.float32 else 8
+    npad = (n + 63) // 64 * 64
+    nch = U // 8
+    raw = calc.compact.cpu().numpy()
+    ints = raw[:3 * npad * 4].view(np.int32)
+    order, n_outer, n_inner = ints[:npad], ints[npad:2 * npad], ints[2 * npad:3 * npad]
+    off = (3 * npad * 4 + 255) // 256 * 256
+    ent = raw[off:off + npad * U * 4 * elem].view(np_dtype).reshape(npad // 64, nch, 64, 8, 4)
+    ent = ent.transpose(0, 2, 1, 3, 4).reshape(npad, U, 4)          # [position][slot][4]
+    bits = ent[..., 3].copy().view(np.int32 if elem == 4 else np.int64).astype(np.int64)
+    assert sorted(order[:n].tolist()) == list(range(n))             # a permutation of the atoms
+    outer, inner = {}, {}
+    for p in range(n):
+        a = int(order[p])
+        so = slice(0, n_outer[p])
+        si = slice(U - n_inner[p], U)
+        pack = lambda s: sorted(zip((bits[p, s] & ((1 << 28) - 1)).tolist(), (bits[p, s] >> 28).tolist(),
+                                    ent[p, s, 0].tolist(), ent[p, s, 1].tolist(), ent[p, s, 2].tolist()))
+        outer[a], inner[a] = pack(so), pack(si)
+    return outer, inner
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_random_cell_against_oracle(oracle, np_dtype):
+    """Random packing, 3 species: padded lists bit-exact, compact lists = the oracle's pairs cut at the
+    two cutoffs, E/F/V within the bars."""
+    n = 350
+    lat, pos = synth.random_packed(n, [20.0, 21.0, 22.0], 2.2, 311)
+    ty = synth.rng_randint(312, n, 3)
+    m = synth.nep_model(seed=3301)
+    calc = _calc(m, lat, ty, n, np_dtype, path="gather")
+    assert calc.path == "gather"
+    out = _step(calc, pos, np_dtype)
+    ref = oracle.nblist(lat.astype(np_dtype), ty, pos.astype(np_dtype), 7.0, 200)
+    assert np.array_equal(calc.numneigh.cpu().numpy(), ref[2])
+    assert np.array_equal(calc.firstneigh.cpu().numpy(), ref[3])
+    u = np.uint32 if np_dtype == np.float32 else np.uint64
+    assert np.array_equal(calc.rcs.cpu().numpy().view(u), ref[4].view(u))
+    assert np.array_equal(calc.ilist.cpu().numpy(), np.arange(n)) and np.array_equal(calc.types_out.cpu().numpy(), ty)
+    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
+    # compact lists against the oracle's rows
+    outer, inner = _decode_compact(calc, np_dtype)
+    rows, rcs, nn = np.asarray(ref[3]), np.asarray(ref[4]), np.asarray(ref[2])
+    for a in range(n):
+        r = np.sqrt((rcs[a, :nn[a]].astype(np_dtype) ** 2).sum(1))
+        want_in = sorted((int(rows[a, s]), int(ty[rows[a, s]]), *rcs[a, s].tolist()) for s in range(nn[a]) if r[s] <= 4.0 - 1e-6)
+        want_out = sorted((int(rows[a, s]), int(ty[rows[a, s]]), *rcs[a, s].tolist()) for s in range(nn[a]) if r[s] > 4.0 + 1e-6)
+        border = sum(1 for s in range(nn[a]) if abs(r[s] - 4.0) <= 1e-6)
+        assert len(inner[a]) + len(outer[a]) == nn[a]
+        assert set(want_in) <= set(inner[a]) and set(want_out) <= set(outer[a])
+        assert len(inner[a]) - len(want_in) + len(outer[a]) - len(want_out) == border
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_cell_smaller_than_cutoff(oracle, np_dtype):
+    """A cell of 9 A with a 7 A cutoff: atoms meet their own images and the same neighbour through several
+    images; the gather still pairs every entry with its mirror."""
+    n = 24
+    lat, pos = synth.random_packed(n, [9.0, 9.5, 10.0], 2.2, 321)
+    lat = lat.copy()
+    lat[1, 0] = 1.3                                       # triclinic
+    ty = synth.rng_randint(322, n, 2)
+    m = synth.nep_model(ntypes=2, seed=3302, type_map=(32, 51))
+    calc = _calc(m, lat, ty, n, np_dtype, umax=200, path="gather")
+    out = _step(calc, pos, np_dtype)
+    ref = oracle.nblist(lat.astype(np_dtype), ty, pos.astype(np_dtype), 7.0, 200)
+    assert np.array_equal(calc.firstneigh.cpu().numpy(), ref[3])
+    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
+
+
+@pytest.mark.parametrize("cfg", [dict(ntypes=1, n_r=4, H=30), dict(ntypes=2, n_r=6, H=50), dict(ntypes=4, n_r=4, H=17),
+                                 dict(ntypes=4, n_r=6, H=60)])
+def test_model_shapes(oracle, cfg):
+    """The shapes the gather kernels are instantiated for (n_radial 4 / 6, one to four species), fp64."""
+    n = 160
+    lat, pos = synth.random_packed(n, [15.0, 16.0, 17.0], 2.2, 331)
+    ty = synth.rng_randint(332, n, cfg["ntypes"])
+    m = synth.nep_model(ntypes=cfg["ntypes"], n_radial_basis=cfg["n_r"], num_neurons=cfg["H"], rmax_radial=6.0,
+                        rmax_angular=4.5, seed=3303, type_map=tuple(range(30, 30 + cfg["ntypes"])))
+    calc = _calc(m, lat, ty, n, np.float64, umax=160, path="gather")
+    out = _step(calc, pos, np.float64)
+    ref = oracle.nblist(lat, ty, pos, 6.0, 160)
+    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float64), np.float64)
+
+
+def test_gather_equals_segments_and_is_reproducible(oracle):
+    """fp32, 42,592 atoms (not a multiple of 256): the gather and the segment path agree within the fp32
+    bars, each run of the gather gives the same bits, and skipping the padded arrays changes nothing."""
+    lat, pos = synth.fcc_cell(22, 4.6, 0.15, 341)
+    n = pos.shape[0]
+    ty = synth.rng_randint(342, n, 3)
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0, seed=3304)
+    a = _step(_calc(m, lat, ty, n, np.float32, umax=104, path="gather"), pos, np.float32)
+    b = _step(_calc(m, lat, ty, n, np.float32, umax=104, path="gather"), pos, np.float32)
+    s = _step(_calc(m, lat, ty, n, np.float32, umax=104, path="segments"), pos, np.float32)
+    lean = _calc(m, lat, ty, n, np.float32, umax=104, path="gather", padded=False)
+    assert lean.firstneigh is None
+    d = _step(lean, pos, np.float32)
+    for x, y, z in zip(a, b, d):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+        assert np.array_equal(x.view(np.uint32), z.view(np.uint32))
+    assert np.allclose(a[0], s[0], rtol=2e-6)
+    assert np.all(np.abs(a[1] - s[1]) <= 2e-4 + 2e-5 * np.abs(s[1]))
+    assert np.abs(a[2] - s[2]).max() <= 2e-5 * np.abs(s[2]).max()
+    assert np.abs(a[1].astype(np.float64).sum(0)).max() < 1e-2          # Newton's third law
+    v = a[2].reshape(3, 3)
+    assert np.abs(v - v.T).max() <= 2e-5 * np.abs(v).max()
+
+
+def test_rebuild_in_place(oracle):
+    """Steps on moving coordinates reuse the calculator's buffers (rows updated in place, compact lists
+    rewritten): every step equals a fresh calculator's."""
+    lat, pos = synth.fcc_cell(8, 4.9, 0.15, 351)
+    n = pos.shape[0]
+    ty = synth.rng_randint(352, n, 3)
+    m = synth.nep_model(seed=3305)
+    disp = synth.rng_normal(353, pos.size, 0.0, 0.2).reshape(-1, 3)
+    calc = _calc(m, lat, ty, n, np.float32, path="gather")
+    for k in range(3):
+        p = pos + disp * np.sin(1.3 * k)
+        got = _step(calc, p, np.float32)
+        want = _step(_calc(m, lat, ty, n, np.float32, path="gather"), p, np.float32)
+        for x, y in zip(got, want):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+        ref = oracle.nblist(lat.astype(np.float32), ty, p.astype(np.float32), 7.0, 200)
+        assert np.array_equal(calc.firstneigh.cpu().numpy(), ref[3])
+        assert np.array_equal(calc.rcs.cpu().numpy().view(np.uint32), ref[4].view(np.uint32))
+        _check(got, oracle.nep_efv(m, synth.pack_batch([ref]), np.float32), np.float32)
+
+
+def test_gather_errors(oracle):
+    import torch
+    from ai2pot_amd import _lib
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos = synth.random_packed(100, [14.0, 14.0, 14.0], 2.2, 361)
+    m = synth.nep_model(seed=3306)
+    with pytest.raises(ValueError):                                   # model shape outside the gather kernels
+        NepCalculator(synth.nep_model(l_max=3), 100, lat, np.zeros(100, np.int32), path="gather")
+    with pytest.raises(ValueError):                                   # fp64 tables of 4 x 100 neurons exceed LDS
+        NepCalculator(synth.nep_model(ntypes=4, num_neurons=100, type_map=(1, 2, 3, 4)), 100, lat, np.zeros(100, np.int32),
+                      dtype=torch.float64, path="gather")
+    with pytest.raises(ValueError):                                   # umax not a multiple of 8
+        NepCalculator(m, 100, lat, np.zeros(100, np.int32), umax=100, path="gather")
+    calc = _calc(m, lat, np.full(100, 5, np.int32), 100, np.float32, path="gather")   # species outside the model
+    calc.step(torch.from_numpy(pos.astype(np.float32)).to("cuda:0"))
+    with pytest.raises(_lib.A2PError):
+        calc.check()
+    L = _lib.lib()
+    L.a2p_nblist_compact_bytes.restype = c.c_size_t
+    assert L.a2p_nblist_compact_bytes(c.c_int(100), c.c_int(100), c.c_int(4)) == 0    # umax % 8 != 0
+    assert L.a2p_nblist_compact_bytes(c.c_int(100), c.c_int(104), c.c_int(4)) == 3 * 128 * 4 + 128 * 104 * 16
+    ok = _calc(m, lat, synth.rng_randint(362, 100, 3), 100, np.float32, umax=8, path="gather")   # rows overflow
+    ok.step(torch.from_numpy(pos.astype(np.float32)).to("cuda:0"))
+    with pytest.raises(_lib.A2PError):
+        ok.check()
