@@ -26,12 +26,14 @@ class NepCalculator:
 
     def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
                  sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None, path="auto",
-                 padded=True):
+                 padded=True, reorder_every=64):
         """path: "gather" evaluates forces as a gather over compact lists cut by the list build (common
         model shapes, unsorted rows, umax % 8 == 0); "segments" scatters pair derivatives into reduction
         segments from the padded arrays (any model shape); "auto" takes the gather when it applies.
         padded=False (gather only) skips the padded firstneigh / rcs arrays: the step then produces
-        energy, forces and virial alone."""
+        energy, forces and virial alone.  reorder_every: the gather path processes the atoms along a
+        space-filling curve; the order is a locality hint only (results do not depend on it beyond
+        rounding), so it is recomputed every reorder_every rebuilds and kept in between."""
         self.device = torch.device(device)
         self.dtype = dtype
         self.n = int(natoms)
@@ -91,6 +93,8 @@ class NepCalculator:
             raise ValueError("the gather path does not cover this model shape / list options")
         self.path = "gather" if (path != "segments" and can_gather) else "segments"
         self.padded = bool(padded) or self.path != "gather"
+        self.reorder_every = max(1, int(reorder_every))
+        self._builds = 0
         if self.path == "gather":
             nbytes = L.a2p_nblist_compact_bytes(_c.c_int(n), _c.c_int(U), elem)
             self.compact = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -119,7 +123,8 @@ class NepCalculator:
             rc = self._nbl_compact(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
                                    _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
                                    self.pbc.ctypes.data_as(_c.c_void_p),
-                                   _c.c_int(1 if (self._have_list and self.padded) else 0),
+                                   _c.c_int((1 if (self._have_list and self.padded) else 0) |
+                                            (2 if (self._have_list and self._builds % self.reorder_every) else 0)),
                                    _c.c_double(m["rmax_radial"]), _c.c_double(m["rmax_angular"]),
                                    _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
                                    _vp(self.types_out), _vp(self.compact), stream)
@@ -137,6 +142,7 @@ class NepCalculator:
                     _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
                     _vp(self.types_out), None, stream)
         self._have_list = rc == 0
+        self._builds += 1
         self._places = False
         _lib.check(rc)
         self._places = self.places_from_list

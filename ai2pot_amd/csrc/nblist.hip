@@ -851,6 +851,7 @@ T host_plane_distance(const T* v, const T* n)        // structure.h:818-842, vec
 struct CompactOut {
     void* buffer;
     double split, outer;
+    int keep_order;    // the buffer already holds a processing order from an earlier build: use it
 };
 
 template <typename T>
@@ -1035,6 +1036,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (co) {
         // processing order: atoms sorted by the Morton code of their bin (ties by index: the sort is stable)
         const CompactView<T> cv = compact_view<T>(co->buffer, N, umax);
+        if (!co->keep_order) {
         int maxdim = std::max(g.rdim[0], std::max(g.rdim[1], g.rdim[2]));
         int shift = 0;
         while ((maxdim >> shift) > 1024) shift++;
@@ -1058,6 +1060,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         A2P_HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(tmp_sort, tmp_bytes, (const unsigned*)keys_in, keys_out,
                                                          (const int*)vals_in, cv.order, N, 0, 3 * bits, stream));
         prof_end(stream);
+        }
         ce.order = cv.order;
         ce.entries = cv.entries;
         ce.n_outer = cv.n_outer;
@@ -1214,9 +1217,9 @@ int a2p_nblist_build_compact_f32(const float* lattice, const int* types, const f
                                  double rcut_inner, int* ilist, int* numneigh, int* firstneigh, float* rcs,
                                  int* types_out, void* compact, void* stream)
 {
-    const a2p::CompactOut co{compact, rcut_inner, rcut_outer};
+    const a2p::CompactOut co{compact, rcut_inner, rcut_outer, (update & 2) ? 1 : 0};
     return a2p::nblist_build<float>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
-                                    firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, update ? 1 : 0, nullptr,
+                                    firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, (update & 1) ? 1 : 0, nullptr,
                                     nullptr, &co);
 }
 
@@ -1225,9 +1228,9 @@ int a2p_nblist_build_compact_f64(const double* lattice, const int* types, const 
                                  double rcut_inner, int* ilist, int* numneigh, int* firstneigh, double* rcs,
                                  int* types_out, void* compact, void* stream)
 {
-    const a2p::CompactOut co{compact, rcut_inner, rcut_outer};
+    const a2p::CompactOut co{compact, rcut_inner, rcut_outer, (update & 2) ? 1 : 0};
     return a2p::nblist_build<double>(lattice, types, coords, natoms, rcut, umax, is_cart, pbc, 0, ilist, numneigh,
-                                     firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, update ? 1 : 0, nullptr,
+                                     firstneigh, rcs, types_out, nullptr, (hipStream_t)stream, (update & 1) ? 1 : 0, nullptr,
                                      nullptr, &co);
 }
 }

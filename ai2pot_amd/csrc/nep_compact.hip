@@ -36,8 +36,9 @@ namespace {
 
 constexpr int CB = 256;                 // positions (threads) per workgroup
 constexpr int KC = 8, NAC = 4, LC = 4, NLM = 24, FDP = 24;
-constexpr int REC = 128;                // values per adjoint record
-constexpr int REC_CC = NAC * NLM;       // the contracted radial coefficients follow the 96 dE/dS
+constexpr int REC = NAC * NLM;          // values per adjoint record: dE/dS, 384 bytes in fp32 (three cache lines)
+// the contracted radial coefficients cc[t][k] live in an array of their own, NTC * 8 values per atom:
+// the pairs between the cutoffs gather only these, and a dense array of them stays in L2
 constexpr int STP = CL_CHUNK + 1;       // staged slots per position, padded: 16-byte reads of 8 lanes hit 8 banks
 
 template <typename T>
@@ -47,7 +48,8 @@ struct GatherArgs {
     T rr, ra;
     CompactView<T> cv;
     const int* types;     // [natoms]
-    T* rec;               // [natoms][REC]
+    T* rec;               // [natoms][REC] dE/dS
+    T* rcc;               // [natoms][NTC * KC] radial coefficients contracted with dE/dq
     T* force;             // [natoms][3] or null
     double* partial;      // [nblocks][10]: energy (adjoint kernel), virial (gather kernel)
     int* status;
@@ -361,8 +363,10 @@ nep_adjoint_kernel(const GatherArgs<T> a)
                 }
             }
             T lo[4] = {cc[0], cc[1], cc[2], cc[3]}, hi[4] = {cc[4], cc[5], cc[6], cc[7]};
-            st4(rp + REC_CC + t * KC, lo);
-            st4(rp + REC_CC + t * KC + 4, hi);
+            if (t < NTC) {
+                st4(a.rcc + ((size_t)atom * NTC + t) * KC, lo);
+                st4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi);
+            }
         }
     }
 
@@ -415,7 +419,7 @@ nep_gather_kernel(const GatherArgs<T> a)
 #pragma unroll
     for (int t = 0; t < NTC; t++) {
         T lo[4] = {(T)0, (T)0, (T)0, (T)0}, hi[4] = {(T)0, (T)0, (T)0, (T)0};
-        if (active) { ld4(own + REC_CC + t * KC, lo); ld4(own + REC_CC + t * KC + 4, hi); }
+        if (active) { ld4(a.rcc + ((size_t)atom * NTC + t) * KC, lo); ld4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi); }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             L.acc[(t * KC + k) * CB + tid] = lo[k];
@@ -457,8 +461,8 @@ nep_gather_kernel(const GatherArgs<T> a)
         T srad = (T)0;
         {
             T lo[4], hi[4];
-            ld4(rj + REC_CC + ti * KC, lo);
-            ld4(rj + REC_CC + ti * KC + 4, hi);
+            ld4(a.rcc + ((size_t)j * NTC + ti) * KC, lo);
+            ld4(a.rcc + ((size_t)j * NTC + ti) * KC + 4, hi);
             radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
@@ -522,10 +526,9 @@ nep_gather_kernel(const GatherArgs<T> a)
     walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
         int j, tj;
         neighbour(valid, bits, j, tj);
-        const T* const rj = a.rec + (size_t)j * REC;
         T lo[4], hi[4];
-        ld4(rj + REC_CC + ti * KC, lo);
-        ld4(rj + REC_CC + ti * KC + 4, hi);
+        ld4(a.rcc + ((size_t)j * NTC + ti) * KC, lo);
+        ld4(a.rcc + ((size_t)j * NTC + ti) * KC + 4, hi);
         const T r = sqrt_t(x * x + y * y + z * z);
         T f[KC], df[KC];
         radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
@@ -639,9 +642,10 @@ int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const
     rc = ws_get(WS_PARTIAL, (size_t)nblocks * 10 * sizeof(double), &ws);
     if (rc) return rc;
     a.partial = (double*)ws;
-    rc = ws_get(WS_PAIR_G, (size_t)natoms * REC * sizeof(T), &ws);
+    rc = ws_get(WS_PAIR_G, (size_t)natoms * (REC + ntc_of(ntypes) * KC) * sizeof(T), &ws);
     if (rc) return rc;
     a.rec = (T*)ws;
+    a.rcc = a.rec + (size_t)natoms * REC;
     const bool pairs = force != nullptr || virial != nullptr;
     auto launch = [&](auto nr) {
         constexpr int NR = decltype(nr)::value;
