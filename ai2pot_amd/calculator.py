@@ -91,7 +91,9 @@ class NepCalculator:
             raise ValueError("path must be auto, gather or segments")
         if path == "gather" and not can_gather:
             raise ValueError("the gather path does not cover this model shape / list options")
-        self.path = "gather" if (path != "segments" and can_gather) else "segments"
+        # "auto": the gather kernels give every atom a thread and want tens of thousands of them; small
+        # systems stay with the lane-group kernel of the segment path
+        self.path = "gather" if (can_gather and (path == "gather" or (path == "auto" and self.n >= 32768))) else "segments"
         self.padded = bool(padded) or self.path != "gather"
         self.reorder_every = max(1, int(reorder_every))
         self._builds = 0

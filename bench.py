@@ -38,18 +38,20 @@ def nep_flops_per_atom(nr_mean, na_mean, K=8, n_r=6, n_a=4, D=22, H=50):
             na_mean * (cK + 4 * K * n_a + 210 + 48 * n_a + 432 * n_a) + 144 * n_a + 4 * D * H + 15 * H)
 
 
-def nep_stage_flops_per_atom(nr_mean, K=8):
-    """Staging kernel's share of nep_flops_per_atom: per radial neighbour the distance (14), the
-    basis values (half of c(K)) and their accumulation per species (K)."""
-    return nr_mean * (14 + (14 * K + 24) // 2 + K)
+def nep_efv_bytes_per_atom(nr_mean, s):
+    """E/F/V operator, algorithmic bytes per atom: ilist / numneigh / type (12), the valid part of the
+    row (index + relative vector per neighbour), the neighbour-type gather (4 per neighbour) and the
+    force written (3 s)."""
+    return 12 + nr_mean * (4 + 3 * s) + 4 * nr_mean + 3 * s
 
 
-def nep_stage_bytes_per_atom(nr_mean, s, ntc=3, K=8):
-    """Staging kernel, algorithmic bytes: per pair the relative vector, the neighbour index, its
-    species, the segment counter (read and written by the atomic), and the compact-list entry (vector
-    and place, plus two bits of species); per atom the row header and the summed radial functions
-    with the two list lengths."""
-    return nr_mean * ((3 * s + 4 + 4 + 8) + (4 * s + 0.25)) + 12 + ntc * K * s + 8
+def nbl_bytes_per_atom(nr_mean, s, umax, in_place):
+    """Neighbour list, algorithmic bytes per atom.  Fresh build: position + type in, ilist / numneigh /
+    types and the full padded rows out.  In-place update (the calculator's steady state): a row is
+    written as far as its old or new length reaches, rounded up to four slots."""
+    if in_place:
+        return (3 * s + 4) + 12 + (nr_mean + 2) * (4 + 3 * s)
+    return (3 * s + 4) + 12 + umax * (4 + 3 * s)
 
 
 def mtp_flops_per_atom(nn_mean, K, nmus, kmax, n_basic, n_times, n_scalar):
@@ -131,25 +133,31 @@ def timed_replay(replay, steps, warmup):
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
-# summarised in profiles/nep_md_1048576_hbm_traffic.txt.  Workloads without a counter run report null.
+# summarised in profiles/<workload>_hbm_traffic.txt.  Kernels without a counter run report null.
 MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nep_stage_kernel"): 4.473e6 * 1024,
-    ("nep_md_1048576", "nep_staged_kernel"): 3.190e6 * 1024,
-    ("nep_md_1048576", "nbl_lists"): 1.039e6 * 1024,
 }
 
 
-def roofline_of(kernels, work):
-    """work: {label: (bound, amount per launch, unit, peak, scale, engine)}; picks the label with
-    the largest total time."""
-    cands = [k for k in kernels if k in work]
-    if not cands:
-        return None
-    dom = max(cands, key=lambda k: kernels[k].get("per_step_ms", kernels[k]["total_ms"]))
-    bound, amount, unit, peak, scale, engine = work[dom]
-    achieved = amount / (kernels[dom]["avg_ms"] * 1e-3) / scale
-    return dict(kernel=dom, bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
-                traffic=None, avg_ms=kernels[dom]["avg_ms"], engine=engine)
+def roofline_of(kernels, work, workload=None):
+    """work: {label: (bound, amount per launch, unit, peak, scale, engine)}.  A label may name several
+    kernels joined by '+': they form one operator, whose duration per launch is the sum of the
+    kernels' average durations.  Returns the entry of the label with the largest time (with `traffic`
+    when profiles/ holds a counter run for it) and the list of all entries."""
+    def entry(label):
+        names = label.split("+")
+        if not all(nm in kernels for nm in names):
+            return None
+        bound, amount, unit, peak, scale, engine = work[label]
+        avg_ms = sum(kernels[nm]["avg_ms"] for nm in names)
+        achieved = amount / (avg_ms * 1e-3) / scale
+        traffic = [MEASURED_TRAFFIC.get((workload, nm)) for nm in names]
+        return dict(kernel=label, bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
+                    traffic=sum(traffic) if all(t is not None for t in traffic) else None, avg_ms=avg_ms,
+                    engine=engine, amount_per_launch=amount)
+    entries = [e for e in (entry(l) for l in work) if e is not None]
+    if not entries:
+        return None, []
+    return max(entries, key=lambda e: e["avg_ms"]), entries
 
 
 # ------------------------------------------------------------------------------------------------
@@ -192,7 +200,7 @@ def run_nep_md(args, kind, size, rebuild=True):
         calc.evaluate(stream)
 
     L = _lib.lib()
-    elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    elapsed, kernels = timed(step, args.steps, args.warmup, L, keep=3)
     if args.graph:
         if rebuild:
             sys.exit("bench.py: --graph needs a workload without list rebuild (the build synchronises with the host)")
@@ -207,26 +215,49 @@ def run_nep_md(args, kind, size, rebuild=True):
     r = calc.rcs.norm(dim=2)
     nn_a = float(((r > 0) & (r <= model["rmax_angular"])).sum().item()) / n
     s = 4
+    flops = nep_flops_per_atom(nn_r, nn_a) * n
+    efv_bytes = nep_efv_bytes_per_atom(nn_r, s) * n
+    valu = ("valu", flops, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32")
     work = {
-        "nep_efv_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
-        "nep_stage_kernel": ("hbm", nep_stage_bytes_per_atom(nn_r, s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
-        "nep_staged_kernel": ("mfma", (nep_flops_per_atom(nn_r, nn_a) - nep_stage_flops_per_atom(nn_r)) * n, "TFLOP/s",
-                              PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
-        "nep_group_kernel": ("mfma", nep_flops_per_atom(nn_r, nn_a) * n, "TFLOP/s", PEAK_FP32_TFLOPS, 1e12, "valu_fp32"),
-        # the calculator updates its list in place: a row is written as far as its old or new
-        # length reaches, rounded up to four slots (about two more than its length on average)
-        "nbl_lists": ("hbm", ((3 * s + 4) + 12 + (nn_r + 2) * (4 + 3 * s)) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
-        "reduce_fill": ("hbm", (nn_r * (3 * s + 4) + nn_r * 3 * s) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
+        # the energy / force / virial operator as a whole, against the fp32 vector peak: whichever kernels serve it
+        "nep_adjoint_kernel+nep_gather_kernel": valu,
+        "nep_stage_kernel+nep_staged_kernel+reduce_sum": valu,
+        "nep_group_kernel+reduce_sum": valu,
+        "nep_efv_kernel": valu,
+        "nbl_lists": ("hbm", nbl_bytes_per_atom(nn_r, s, 200, rebuild) * n, "GB/s", PEAK_HBM_GBS, 1e9, "hbm"),
     }
     config = {"workload": args.workload, "natoms": n, "species": 3,
               "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 7.0, "rcut_angular": 4.0,
               "umax": 200, "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
-              "per_step": ("neighbor rebuild + " if rebuild else "") + "descriptors + ANN + force/virial",
-              "launch": "hip graph replay" if args.graph else "eager"}
-    roof = roofline_of(kernels, work)
-    if roof is not None:
-        roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, roof["kernel"]))
-    return n, elapsed, kernels, roof, config, "f32"
+              "per_step": ("neighbor rebuild (padded arrays + compact lists) + " if rebuild else "") +
+                          "descriptors + ANN + force/virial",
+              "path": calc.path, "launch": "hip graph replay" if args.graph else "eager"}
+    roof, entries = roofline_of(kernels, work, args.workload)
+    if roof is not None and roof["bound"] == "valu":
+        # the same operator against the memory roofline (algorithmic bytes of the E/F/V operator)
+        gbs = efv_bytes / (roof["avg_ms"] * 1e-3) / 1e9
+        roof["hbm"] = dict(achieved=gbs, peak=PEAK_HBM_GBS, unit="GB/s", frac=gbs / PEAK_HBM_GBS, amount_per_launch=efv_bytes)
+    extra = {"rooflines": entries}
+    if rebuild and calc.path == "gather" and not args.graph:
+        # the same step without the padded firstneigh / rcs arrays (energy, forces and virial only)
+        lean = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, padded=False)
+        lean.rebuild(coords0, stream)
+
+        def lean_step(k):
+            torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
+            return lean.step(coords)
+        for k in range(args.warmup):
+            lean_step(k)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            lean_step(args.warmup + k)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        lean.check()
+        extra["without_padded_arrays"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
+                                              unit="atom-steps/s")
+    return n, elapsed, kernels, roof, config, "f32", extra
 
 
 def cpu_baseline_nep(sample_reps=32, repeats=2):
@@ -339,9 +370,9 @@ def run_mtp(args, cfg):
         g = GraphedCall(ops.linearMtpToEFVOp, *common, 0.0, 0.0, None, None)
         elapsed = timed_replay(g.replay, args.steps, args.warmup)
     _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
-    work = {label: ("mfma", flops if cfg != 4 else flops - mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s",
+    work = {label: ("valu", flops if cfg != 4 else flops - mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s",
                     PEAK_FP64_TFLOPS, 1e12, "valu_fp64"),
-            "mtp_efv_kernel": ("mfma", mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s", PEAK_FP64_TFLOPS, 1e12,
+            "mtp_efv_kernel": ("valu", mtp_flops_per_atom(nn, *sizes) * natoms, "TFLOP/s", PEAK_FP64_TFLOPS, 1e12,
                                "valu_fp64")}
     config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P,
               "model": "linear MTP level %d K=%d" % ({1: 10, 3: 20, 4: 16}[cfg], m["chebyshev_size"]),
@@ -349,7 +380,8 @@ def run_mtp(args, cfg):
               "per_step": "loss forward + analytic gradient w.r.t. coeffs/linear/bias" if cfg == 4 else
                           "energy + force + virial (list built once, outside the timed region)",
               "launch": "hip graph replay" if args.graph else "eager"}
-    return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f64"
+    roof, entries = roofline_of(kernels, work, args.workload)
+    return natoms, elapsed, kernels, roof, config, "f64", {"rooflines": entries}
 
 
 def run_nep_train(args):
@@ -394,13 +426,14 @@ def run_nep_train(args):
     _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
     # the gradient pass repeats the descriptor work with tangents (x2) and adds the outer products of the
     # hidden layer (4 D H) and the two coefficient-gradient contractions: counted as 2.5 x the E/F/V flops
-    work = {"nep_loss_bwd_kernel": ("mfma", 2.5 * nep_flops_per_atom(nn, nn_a) * natoms, "TFLOP/s", PEAK_FP32_TFLOPS,
+    work = {"nep_loss_bwd_kernel": ("valu", 2.5 * nep_flops_per_atom(nn, nn_a) * natoms, "TFLOP/s", PEAK_FP32_TFLOPS,
                                     1e12, "valu_fp32")}
     config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P, "species": 3,
               "model": "NEP radial+3-body K=8 n_r=6 n_a=4 l_max=4 H=50", "rcut_radial": 6.0, "rcut_angular": 4.0,
               "mean_neighbors_radial": nn, "mean_neighbors_angular": nn_a,
               "per_step": "E/F/V + loss forward + analytic gradient w.r.t. coeffs/w0/b0/w1/bias"}
-    return natoms, elapsed, kernels, roofline_of(kernels, work), config, "f32"
+    roof, entries = roofline_of(kernels, work, args.workload)
+    return natoms, elapsed, kernels, roof, config, "f32", {"rooflines": entries}
 
 
 def cpu_baseline_mtp(cfg):
@@ -467,6 +500,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="nep_md_1048576", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="headline workload only: skip the short runs of the other benchmark configurations")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of the step captured as a HIP graph (workloads without list rebuild)")
     args = ap.parse_args()
@@ -480,7 +515,7 @@ def main():
     if args.workload == "hbm_copy_probe":
         return run_copy_probe(args)
 
-    n, elapsed, kernels, roofline, config, dtype = WORKLOADS[args.workload](args)
+    n, elapsed, kernels, roofline, config, dtype, extra = WORKLOADS[args.workload](args)
     ms_per_step = elapsed * 1e3 / args.steps
     out = {
         "metric": "atom-steps/s (E+F+virial) on 1 MI355X", "value": n * args.steps / elapsed,
@@ -489,6 +524,26 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": config,
         "roofline": roofline, "kernels": kernels,
     }
+    out.update(extra)
+    if args.workload == "nep_md_1048576" and not args.no_other_configs and not args.graph:
+        # the remaining benchmark configurations, after the headline's timed region (so they cannot
+        # perturb it): ms per step and the roofline entry of the kernel that takes the most time
+        import copy
+        import torch
+        others = {}
+        for wl in ("mtp10_efv_216", "nep_efv_4096", "mtp20_efv_8192", "mtp16_train_64x128"):
+            a2 = copy.copy(args)
+            a2.workload, a2.steps, a2.warmup = wl, 50, 5
+            try:
+                n2, el2, k2, roof2, _, dt2, _ = WORKLOADS[wl](a2)
+                others[wl] = dict(natoms=n2, ms_per_step=el2 * 1e3 / a2.steps, value=n2 * a2.steps / el2,
+                                  unit="atom-steps/s", dtype=dt2, steps=a2.steps,
+                                  roofline=None if roof2 is None else
+                                  {k: roof2[k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "avg_ms")})
+            except Exception as ex:
+                others[wl] = {"error": repr(ex)}
+            torch.cuda.synchronize()
+        out["other_configs"] = others
     if not args.no_cpu_baseline:
         try:
             if args.workload == "nep_train_64x128":
