@@ -282,6 +282,19 @@ __device__ __forceinline__ unsigned spread3(unsigned v)      // 10 bits -> every
     return v;
 }
 
+// xs[position] = x[order[position]]: the list kernel then reads its atoms' coordinates without first
+// waiting for the order
+template <typename T>
+__global__ void sorted_coords_kernel(int N, const T* __restrict__ x, const int* __restrict__ order, T* __restrict__ xs)
+{
+    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    if (p >= N) return;
+    const int at = min(max(order[p], 0), N - 1);
+    xs[(size_t)p * 3 + 0] = x[(size_t)at * 3 + 0];
+    xs[(size_t)p * 3 + 1] = x[(size_t)at * 3 + 1];
+    xs[(size_t)p * 3 + 2] = x[(size_t)at * 3 + 2];
+}
+
 template <typename T>
 __global__ void order_keys_kernel(const Grid<T> g, const T* __restrict__ x, int shift, unsigned* __restrict__ keys,
                                   int* __restrict__ vals)
@@ -408,11 +421,12 @@ constexpr int NBL_APW = 2;         // consecutive centre atoms per wavefront
 template <typename T>
 struct CompactEmit {
     const int* order;   // position -> atom
+    const T* xs;        // [natoms][3] Cartesian coordinates in processing order
     T* entries;
     int* n_outer;
     int* n_inner;
     int nch;
-    T split, outer;
+    T split2, outer2;   // squares of the two cutoffs
     int write_rows;     // the padded outputs are wanted as well
 };
 
@@ -470,7 +484,8 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
 #pragma unroll
     for (int a = 0; a < NBL_APW; a++)
 #pragma unroll
-        for (int d = 0; d < 3; d++) cs[a][d] = x[(size_t)atom[a] * 3 + d];
+        for (int d = 0; d < 3; d++)
+            cs[a][d] = COMPACT ? ce.xs[(size_t)min(p0 + a, g.N - 1) * 3 + d] : x[(size_t)atom[a] * 3 + d];
     const int nruns = (2 * g.ext_bins + 1) * (2 * g.ext_bins + 1);
     int start, len;
     column_setup<T>(g, cs[0], lane, offsets, start, len);
@@ -585,22 +600,24 @@ lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ t
         __builtin_amdgcn_wave_barrier();
         const int used = min(cnt, umax);
         int n_outer = 0, n_inner = 0;
+        // slot e of this position sits at  base + (e / 8) * (64 * 8 * 4) + (e % 8) * 4  values
+        T* const base = ce.entries + compact_slot_offset(ce.nch, __builtin_amdgcn_readfirstlane(pos), 0);
         for (int e0 = 0; e0 < used; e0 += 64) {
             const int e = e0 + lane;
             const bool have = e < used;
             const int ee = have ? e : 0;
             const T dx = rb_rcs[ee * 3 + 0], dy = rb_rcs[ee * 3 + 1], dz = rb_rcs[ee * 3 + 2];
             const int bits = rb_first[ee];
-            const T r = sizeof(T) == 4 ? (T)sqrtf((float)(dx * dx + dy * dy + dz * dz)) : (T)sqrt((double)(dx * dx + dy * dy + dz * dz));
-            const bool in_outer = have && r <= ce.outer;
-            const bool is_inner = in_outer && r <= ce.split;
+            const T d2 = dx * dx + dy * dy + dz * dz;
+            const bool in_outer = have && d2 <= ce.outer2;
+            const bool is_inner = in_outer && d2 <= ce.split2;
             const bool is_outer = in_outer && !is_inner;
             const unsigned long long mi = __ballot(is_inner), mo = __ballot(is_outer);
             const unsigned long long below = (1ull << lane) - 1ull;
             int slot = -1;
             if (is_inner) slot = umax - 1 - (n_inner + __popcll(mi & below));
             if (is_outer) slot = n_outer + __popcll(mo & below);
-            if (slot >= 0) entry_store<T>(ce.entries + compact_slot_offset(ce.nch, pos, slot), dx, dy, dz, bits);
+            if (slot >= 0) entry_store<T>(base + (((unsigned)slot >> 3) << 11) + (((unsigned)slot & 7u) << 2), dx, dy, dz, bits);
             n_inner += __popcll(mi);
             n_outer += __popcll(mo);
         }
@@ -919,12 +936,13 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     // workspace A: x[N*3] | partial[nblocks*12] | ext[12]
     const int nblocks = ceil_div(N, NBL_BLOCK);
     void* wsA = nullptr;
-    size_t bytesA = ((size_t)N * 3 + (size_t)nblocks * 12 + 16) * sizeof(T);
+    size_t bytesA = ((size_t)N * 3 * (co ? 2 : 1) + (size_t)nblocks * 12 + 16) * sizeof(T);
     int rc = ws_get(WS_NBL_A, bytesA, &wsA);
     if (rc) return rc;
     T* x = (T*)wsA;
     T* partial = x + (size_t)N * 3;
     T* ext_dev = partial + (size_t)nblocks * 12;
+    T* xs = ext_dev + 16;                               // coordinates in processing order (compact lists)
     void* flags = nullptr;
     rc = ws_get(WS_FLAGS, 64, &flags);
     if (rc) return rc;
@@ -1066,8 +1084,13 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         ce.n_outer = cv.n_outer;
         ce.n_inner = cv.n_inner;
         ce.nch = cv.nch;
-        ce.split = (T)co->split;
-        ce.outer = (T)co->outer;
+        prof_begin("nbl_order", stream);
+        hipLaunchKernelGGL(sorted_coords_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, N, (const T*)x,
+                           (const int*)cv.order, xs);
+        prof_end(stream);
+        ce.xs = xs;
+        ce.split2 = (T)co->split * (T)co->split;
+        ce.outer2 = (T)co->outer * (T)co->outer;
         ce.write_rows = want_rows ? 1 : 0;
     }
     const int list_blocks = ceil_div(N, (NBL_BLOCK / 64) * NBL_APW);
