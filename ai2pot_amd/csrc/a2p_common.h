@@ -58,6 +58,7 @@ enum StatusBits {
     ST_BAD_NEIGHBOR = 1,   // neighbour index outside [0, natoms_pad + nghost)
     ST_BAD_TYPE = 2,       // type index outside [0, ntypes)
     ST_NEIGH_OVERFLOW = 4, // numneigh larger than the row capacity
+    ST_SEG_OVERFLOW = 8,   // more pairs name one atom than its reduction segment holds (a list that is not symmetric)
 };
 
 inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
@@ -136,10 +137,13 @@ int pair_reduce(T* force, const T* pair_g, int B, int P, int U, int nghost, cons
 //                    for EVERY valid pair (zeros where the derivative vanishes), or, without
 //                    ranks, claims  pos = offsets[t] + atomicAdd(&cursor[t], 1)  and may skip pairs;
 //   pair_csr_finish  sums the filled part of every segment onto `force` as above.
-// pair_fixed_begin skips counting: every target owns a segment of fixed capacity seg_cap = U
+// Capacity of the fixed reduction segments: umax unless the calling thread asked for more with
+// a2p_pair_segment_capacity (lists in which an atom is named by more pairs than a row holds).
+int pair_segment_capacity(int U);
+// pair_fixed_begin skips counting: every target owns a segment of fixed capacity seg_cap (umax by default)
 // (a cutoff-built list sends an atom no more pairs than its own row could hold); the producer
 // claims  rank = atomicAdd(&cursor[t], 1),  stores at  pos = t*seg_cap + rank  when rank < seg_cap
-// and otherwise raises ST_NEIGH_OVERFLOW and stores at the spare entry n*seg_cap.
+// and otherwise raises ST_SEG_OVERFLOW and stores at the spare entry n*seg_cap.
 struct PairCsr {
     int* counts;
     int* offsets;

@@ -7,6 +7,8 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 
+#include <cstdlib>
+
 #include "../../../include/ai2pot_hip.h"
 
 namespace a2p_bind {
@@ -84,11 +86,49 @@ inline Batch check_batch(const at::Tensor& binum, const at::Tensor& bilist, cons
     return s;
 }
 
+// Validation switch of an operator library: on (the default), every call ends by reading the device
+// status word, which synchronises the stream; off (set_validate(false), or AI2POT_HIP_VALIDATE=0 in
+// the environment), calls only enqueue work and a caller checks when it chooses to
+// (torch.ops.<lib>.check_status()).  A loop of calls can then run ahead of the device.
+inline bool& validate_flag()
+{
+    static bool on = [] {
+        const char* env = std::getenv("AI2POT_HIP_VALIDATE");
+        return !(env && env[0] == '0');
+    }();
+    return on;
+}
+
 // Errors the reference leaves to a commented-out assert (source/nblist/include/neighborList.h:550)
 // or to out-of-bounds reads; one device status read per call.
 inline void check_device_status(const at::Tensor& t)
 {
-    check_rc(a2p_check_status(current_stream(t)));
+    if (validate_flag()) check_rc(a2p_check_status(current_stream(t)));
+}
+
+// Runs an energy / force / virial (or loss) call and, with validation on, reads the device status.
+// A list that names an atom more often than a row is long (half lists, ghosts collecting the pairs of
+// several rows) overflows the fixed reduction segments of the fast kernels: the status says so and
+// the call is repeated once with segments sized for the list at hand.
+template <class Call>
+inline void run_checked(const at::Tensor& brcs, const at::Tensor& binum, const at::Tensor& bnumneigh,
+                        const at::Tensor& bfirstneigh, int nghost, Call&& call)
+{
+    check_rc(call());
+    if (!validate_flag()) return;
+    void* st = current_stream(brcs);
+    int rc = a2p_check_status(st);
+    if (rc == A2P_ERR_SEGMENT) {
+        int most = 0;
+        check_rc(a2p_pair_incoming_max((int)brcs.size(0), (int)brcs.size(1), (int)brcs.size(2), nghost,
+                                       binum.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                       &most, st));
+        const int old = a2p_pair_segment_capacity(most);
+        rc = call();
+        if (rc == A2P_OK) rc = a2p_check_status(st);
+        a2p_pair_segment_capacity(old);
+    }
+    check_rc(rc);
 }
 
 inline void require_no_zbl(double zbl_rmax)

@@ -167,6 +167,13 @@ variable_list VirialSr::backward(AutogradContext* ctx, variable_list g)
 
 TORCH_LIBRARY(fvt, m)
 {
+    // no counterpart in the reference: the per-call device status check (one stream synchronisation per
+    // call) can be switched off for loops that should run ahead of the device, and asked for explicitly
+    m.def("set_validate", [](bool on) { validate_flag() = on; });
+    m.def("check_status", [](const at::Tensor& any_device_tensor) {
+        DeviceGuard guard(any_device_tensor);
+        check_rc(a2p_check_status(current_stream(any_device_tensor)));
+    });
     m.def("ForceSrOp",
           [](const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
              const at::Tensor& bfirstneigh, int64_t nghost, int64_t umax, const at::Tensor& dei) -> variable_list {

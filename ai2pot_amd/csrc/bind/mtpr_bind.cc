@@ -57,23 +57,25 @@ variable_list mtp_efv(bool want_virial, int64_t K, double scaling, const at::Ten
     at::Tensor v;
     if (want_virial) v = fresh ? at::empty({c.s.B, 9}, opt) : at::zeros({c.s.B, 9}, opt);
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kDouble)
-        rc = a2p_mtp_efv_f64(c.plan.handle, (int)K, scaling, coeffs.data_ptr<double>(), lin.data_ptr<double>(),
-                             bias.data_ptr<double>(), (int)nmus, c.ntypes, q_scaler.data_ptr<double>(), rmax, rmin,
-                             c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                             bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(),
-                             btypes.data_ptr<int>(), e.data_ptr<double>(), f.data_ptr<double>(),
-                             v.defined() ? v.data_ptr<double>() : nullptr, st);
-    else
-        rc = a2p_mtp_efv_f32(c.plan.handle, (int)K, scaling, coeffs.data_ptr<float>(), lin.data_ptr<float>(),
-                             bias.data_ptr<float>(), (int)nmus, c.ntypes, q_scaler.data_ptr<float>(), rmax, rmin,
-                             c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                             bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(),
-                             btypes.data_ptr<int>(), e.data_ptr<float>(), f.data_ptr<float>(),
-                             v.defined() ? v.data_ptr<float>() : nullptr, st);
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kDouble)
+            rc = a2p_mtp_efv_f64(c.plan.handle, (int)K, scaling, coeffs.data_ptr<double>(), lin.data_ptr<double>(),
+                                 bias.data_ptr<double>(), (int)nmus, c.ntypes, q_scaler.data_ptr<double>(), rmax, rmin,
+                                 c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                 bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(),
+                                 btypes.data_ptr<int>(), e.data_ptr<double>(), f.data_ptr<double>(),
+                                 v.defined() ? v.data_ptr<double>() : nullptr, st);
+        else
+            rc = a2p_mtp_efv_f32(c.plan.handle, (int)K, scaling, coeffs.data_ptr<float>(), lin.data_ptr<float>(),
+                                 bias.data_ptr<float>(), (int)nmus, c.ntypes, q_scaler.data_ptr<float>(), rmax, rmin,
+                                 c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                 bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(),
+                                 btypes.data_ptr<int>(), e.data_ptr<float>(), f.data_ptr<float>(),
+                                 v.defined() ? v.data_ptr<float>() : nullptr, st);
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, c.s.nghost, call);
     apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
               e, f, v);
     if (want_virial) return {e, f, v};
@@ -113,26 +115,28 @@ struct LossFunction : public torch::autograd::Function<LossFunction> {
             db = at::zeros({B, bias.numel()}, opt);
         }
         void* st = current_stream(brcs);
-        int rc;
-        if (brcs.scalar_type() == at::kDouble) {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
-            rc = a2p_mtp_loss_f64(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
-                                  (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
-                                  rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                  bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                  btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
-                                  st);
-        } else {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
-            rc = a2p_mtp_loss_f32(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
-                                  (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
-                                  rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                  bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                  btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
-                                  st);
-        }
-        check_rc(rc);
-        check_device_status(brcs);
+        auto call = [&]() -> int {
+            int rc;
+            if (brcs.scalar_type() == at::kDouble) {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+                rc = a2p_mtp_loss_f64(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
+                                      (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
+                                      rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                      bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                      btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
+                                      st);
+            } else {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+                rc = a2p_mtp_loss_f32(c.plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft),
+                                      (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes, p(q_scaler),
+                                      rmax, rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                      bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                      btypes.data_ptr<int>(), p(bloss), p(rmse), p(e), p(f), p(v), p(dc), p(dl), p(db),
+                                      st);
+            }
+            return rc;
+        };
+        run_checked(brcs, binum, bnumneigh, bfirstneigh, 0, call);
         ctx->saved_data["need"] = need;
         if (need) ctx->save_for_backward({dc, dl, db});
         ctx->saved_data["shape_c"] = coeffs.sizes().vec();
@@ -164,22 +168,24 @@ void run_esites(const MtpCtx& c, int64_t K, double scaling, const at::Tensor& co
 {
     a2p_bind::DeviceGuard guard(brcs);
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kDouble) {
-        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
-        rc = a2p_mtp_esites_f64(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
-                                p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
-                                bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
-                                p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
-    } else {
-        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
-        rc = a2p_mtp_esites_f32(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
-                                p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
-                                bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
-                                p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
-    }
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_mtp_esites_f64(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
+                                    p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
+                                    bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                    p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_mtp_esites_f32(c.plan.handle, (int)K, scaling, p(coeffs), p(lin), p(bias), (int)nmus, c.ntypes,
+                                    p(q_scaler), rmax, rmin, c.s.B, c.s.P, c.s.U, c.s.nghost, binum.data_ptr<int>(),
+                                    bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                    p(brcs), btypes.data_ptr<int>(), p(es), p(desc), st);
+        }
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, c.s.nghost, call);
 }
 
 // forward: [e_sites[B, P]]; backward: sum over structures and rows of grad * d e_sites / d theta
@@ -297,22 +303,24 @@ variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at
     a2p_bind::DeviceGuard guard(brcs);
     at::Tensor ec = at::zeros({B, n}, opt), fc = at::zeros({(int64_t)B * P * 3, n}, opt), vc = at::zeros({B * 9, n}, opt);
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kDouble) {
-        auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
-        rc = a2p_mtp_lin_components_f64(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
-                                        rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                        btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
-    } else {
-        auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
-        rc = a2p_mtp_lin_components_f32(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
-                                        rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                        btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
-    }
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+            rc = a2p_mtp_lin_components_f64(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
+                                            rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                            bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                            btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+            rc = a2p_mtp_lin_components_f32(c.plan.handle, (int)K, scaling, p(coeffs), (int)nmus, c.ntypes, p(q_scaler), rmax,
+                                            rmin, B, P, c.s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                            bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                            btypes.data_ptr<int>(), p(ec), p(fc), p(vc), st);
+        }
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, 0, call);
     at::Tensor A = e_w * at::matmul(ec.t(), ec) + f_w * at::matmul(fc.t(), fc) + v_w * at::matmul(vc.t(), vc);
     at::Tensor b = e_w * at::matmul(ec.t(), e_dft.reshape({B})) + f_w * at::matmul(fc.t(), f_dft.reshape({-1})) +
                    v_w * at::matmul(vc.t(), v_dft.reshape({-1}));
@@ -351,6 +359,13 @@ variable_list schmidt_orth(int64_t ntypes, int64_t nmus, int64_t K, const at::Te
 
 TORCH_LIBRARY(mtpr, m)
 {
+    // no counterpart in the reference: the per-call device status check (one stream synchronisation per
+    // call) can be switched off for loops that should run ahead of the device, and asked for explicitly
+    m.def("set_validate", [](bool on) { validate_flag() = on; });
+    m.def("check_status", [](const at::Tensor& any_device_tensor) {
+        DeviceGuard guard(any_device_tensor);
+        check_rc(a2p_check_status(current_stream(any_device_tensor)));
+    });
     m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
     m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
     m.def("linearMtpToEFVOp", [](MTP_EFV_ARGS) -> variable_list { return mtp_efv(true, MTP_EFV_PASS, zbl_rmax, zbl_rmin, zbl_cks, zbl_dks); });

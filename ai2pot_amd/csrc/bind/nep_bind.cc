@@ -61,29 +61,31 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
         if (want_virial) v = fresh ? at::empty({s.B, 9}, opt) : at::zeros({s.B, 9}, opt);
     }
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kFloat) {
-        rc = a2p_nep_efv_f32(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<float>(),
-                             w0.data_ptr<float>(), b0.data_ptr<float>(), w1.data_ptr<float>(),
-                             bias.data_ptr<float>(), q_scaler.data_ptr<float>(), rr, ra, s.B, s.P, s.U, s.nghost,
-                             binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                             bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(), btypes.data_ptr<int>(),
-                             e.defined() ? e.data_ptr<float>() : nullptr, f.defined() ? f.data_ptr<float>() : nullptr,
-                             v.defined() ? v.data_ptr<float>() : nullptr, d.defined() ? d.data_ptr<float>() : nullptr,
-                             st);
-    } else {
-        rc = a2p_nep_efv_f64(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<double>(),
-                             w0.data_ptr<double>(), b0.data_ptr<double>(), w1.data_ptr<double>(),
-                             bias.data_ptr<double>(), q_scaler.data_ptr<double>(), rr, ra, s.B, s.P, s.U, s.nghost,
-                             binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                             bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(), btypes.data_ptr<int>(),
-                             e.defined() ? e.data_ptr<double>() : nullptr,
-                             f.defined() ? f.data_ptr<double>() : nullptr,
-                             v.defined() ? v.data_ptr<double>() : nullptr,
-                             d.defined() ? d.data_ptr<double>() : nullptr, st);
-    }
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kFloat) {
+            rc = a2p_nep_efv_f32(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<float>(),
+                                 w0.data_ptr<float>(), b0.data_ptr<float>(), w1.data_ptr<float>(),
+                                 bias.data_ptr<float>(), q_scaler.data_ptr<float>(), rr, ra, s.B, s.P, s.U, s.nghost,
+                                 binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                 bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(), btypes.data_ptr<int>(),
+                                 e.defined() ? e.data_ptr<float>() : nullptr, f.defined() ? f.data_ptr<float>() : nullptr,
+                                 v.defined() ? v.data_ptr<float>() : nullptr, d.defined() ? d.data_ptr<float>() : nullptr,
+                                 st);
+        } else {
+            rc = a2p_nep_efv_f64(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<double>(),
+                                 w0.data_ptr<double>(), b0.data_ptr<double>(), w1.data_ptr<double>(),
+                                 bias.data_ptr<double>(), q_scaler.data_ptr<double>(), rr, ra, s.B, s.P, s.U, s.nghost,
+                                 binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                 bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(), btypes.data_ptr<int>(),
+                                 e.defined() ? e.data_ptr<double>() : nullptr,
+                                 f.defined() ? f.data_ptr<double>() : nullptr,
+                                 v.defined() ? v.data_ptr<double>() : nullptr,
+                                 d.defined() ? d.data_ptr<double>() : nullptr, st);
+        }
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, s.nghost, call);
     if (want_desc) return {d};
     if (want_virial) return {e, f, v};
     return {e, f};
@@ -125,24 +127,26 @@ struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
             db = at::zeros({B, bias.numel()}, opt);
         }
         void* st = current_stream(brcs);
-        int rc;
-        if (brcs.scalar_type() == at::kDouble) {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
-            rc = a2p_nep_loss_f64(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
-                                  m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
-                                  B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                                  bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
-                                  p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
-        } else {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
-            rc = a2p_nep_loss_f32(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
-                                  m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
-                                  B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                                  bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
-                                  p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
-        }
-        check_rc(rc);
-        check_device_status(brcs);
+        auto call = [&]() -> int {
+            int rc;
+            if (brcs.scalar_type() == at::kDouble) {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+                rc = a2p_nep_loss_f64(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
+                                      m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
+                                      B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                      bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
+                                      p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
+            } else {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+                rc = a2p_nep_loss_f32(e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), m.K, m.n_r, m.n_a,
+                                      m.l_max, m.H, m.ntypes, p(coeffs), p(w0), p(b0), p(w1), p(bias), p(q_scaler), rr, ra,
+                                      B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                      bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(bloss), p(rmse),
+                                      p(e), p(f), p(v), p(dc), p(dw0), p(db0), p(dw1), p(db), st);
+            }
+            return rc;
+        };
+        run_checked(brcs, binum, bnumneigh, bfirstneigh, 0, call);
         ctx->saved_data["need"] = need;
         if (need) ctx->save_for_backward({dc, dw0, db0, dw1, db});
         ctx->saved_data["shape_c"] = coeffs.sizes().vec();
@@ -172,6 +176,13 @@ struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
 
 TORCH_LIBRARY(nep, m)
 {
+    // no counterpart in the reference: the per-call device status check (one stream synchronisation per
+    // call) can be switched off for loops that should run ahead of the device, and asked for explicitly
+    m.def("set_validate", [](bool on) { validate_flag() = on; });
+    m.def("check_status", [](const at::Tensor& any_device_tensor) {
+        DeviceGuard guard(any_device_tensor);
+        check_rc(a2p_check_status(current_stream(any_device_tensor)));
+    });
     m.def("nepToEFOp",
           [](int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const at::Tensor& coeffs, const at::Tensor& w0,
              const at::Tensor& b0, const at::Tensor& w1, const at::Tensor& bias, const at::Tensor& binum,

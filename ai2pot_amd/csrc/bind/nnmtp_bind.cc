@@ -59,24 +59,26 @@ variable_list nnmtp_run(bool want_e, bool want_v, bool want_es, int64_t K, const
     }
     if (want_es) es = at::zeros({s.B, s.P}, opt);
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kDouble) {
-        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
-        rc = a2p_nnmtp_efv_f64(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
-                               p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
-                               binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                               bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
-                               st);
-    } else {
-        auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
-        rc = a2p_nnmtp_efv_f32(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
-                               p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
-                               binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
-                               bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
-                               st);
-    }
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_nnmtp_efv_f64(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                                   p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                                   binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                   bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
+                                   st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_nnmtp_efv_f32(plan.handle, (int)K, H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes,
+                                   p(q_shifter), p(q_scaler), rmax, rmin, s.B, s.P, s.U, s.nghost,
+                                   binum.data_ptr<int>(), bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                   bfirstneigh.data_ptr<int>(), p(brcs), btypes.data_ptr<int>(), p(e), p(f), p(v), p(es),
+                                   st);
+        }
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, s.nghost, call);
     if (want_es) return {es};
     if (want_v) return {e, f, v};
     return {e, f};
@@ -100,22 +102,24 @@ variable_list nnmtp_descriptors(int64_t K, const at::Tensor& coeffs, int64_t n_m
     at::Tensor one = at::ones({plan.n_scalar}, opt), zero = at::zeros({ntypes}, opt);
     at::Tensor desc = at::zeros({s.B, s.P, plan.n_scalar}, opt);
     void* st = current_stream(brcs);
-    int rc;
-    if (brcs.scalar_type() == at::kDouble) {
-        auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
-        rc = a2p_mtp_esites_f64(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
-                                rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                btypes.data_ptr<int>(), nullptr, p(desc), st);
-    } else {
-        auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
-        rc = a2p_mtp_esites_f32(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
-                                rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                btypes.data_ptr<int>(), nullptr, p(desc), st);
-    }
-    check_rc(rc);
-    check_device_status(brcs);
+    auto call = [&]() -> int {
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<double>(); };
+            rc = a2p_mtp_esites_f64(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
+                                    rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                    btypes.data_ptr<int>(), nullptr, p(desc), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.data_ptr<float>(); };
+            rc = a2p_mtp_esites_f32(plan.handle, (int)K, 1.0, p(coeffs), p(one), p(zero), (int)nmus, ntypes, p(one), rmax,
+                                    rmin, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                    btypes.data_ptr<int>(), nullptr, p(desc), st);
+        }
+        return rc;
+    };
+    run_checked(brcs, binum, bnumneigh, bfirstneigh, s.nghost, call);
     return {desc};
 }
 
@@ -237,26 +241,28 @@ struct NNLossFunction : public torch::autograd::Function<NNLossFunction> {
         const char* env = std::getenv("A2P_NNMTP_EXACT_GRADIENT");
         const int exact = env && env[0] == '1';
         void* st = current_stream(brcs);
-        int rc;
-        if (brcs.scalar_type() == at::kDouble) {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
-            rc = a2p_nnmtp_loss_f64(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
-                                    H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
-                                    rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                    btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
-                                    exact, st);
-        } else {
-            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
-            rc = a2p_nnmtp_loss_f32(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
-                                    H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
-                                    rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
-                                    bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
-                                    btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
-                                    exact, st);
-        }
-        check_rc(rc);
-        check_device_status(brcs);
+        auto call = [&]() -> int {
+            int rc;
+            if (brcs.scalar_type() == at::kDouble) {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+                rc = a2p_nnmtp_loss_f64(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
+                                        H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
+                                        rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                        btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
+                                        exact, st);
+            } else {
+                auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+                rc = a2p_nnmtp_loss_f32(plan.handle, e_w, f_w, with_virial ? v_w : 0.0, p(e_dft), p(f_dft), p(v_dft), (int)K,
+                                        H, p(coeffs), p(w0), p(w1), p(bias), (int)nmus, ntypes, p(q_shifter), p(q_scaler),
+                                        rmax, rmin, B, P, s.U, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                        bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), p(brcs),
+                                        btypes.data_ptr<int>(), p(bloss), p(e), p(f), p(v), p(dc), p(d0), p(d1), p(db),
+                                        exact, st);
+            }
+            return rc;
+        };
+        run_checked(brcs, binum, bnumneigh, bfirstneigh, 0, call);
         ctx->saved_data["need"] = need;
         if (need) ctx->save_for_backward({dc, d0, d1, db});
         ctx->saved_data["shape_c"] = coeffs.sizes().vec();
@@ -284,6 +290,13 @@ struct NNLossFunction : public torch::autograd::Function<NNLossFunction> {
 
 TORCH_LIBRARY(nnmtp, m)
 {
+    // no counterpart in the reference: the per-call device status check (one stream synchronisation per
+    // call) can be switched off for loops that should run ahead of the device, and asked for explicitly
+    m.def("set_validate", [](bool on) { validate_flag() = on; });
+    m.def("check_status", [](const at::Tensor& any_device_tensor) {
+        DeviceGuard guard(any_device_tensor);
+        check_rc(a2p_check_status(current_stream(any_device_tensor)));
+    });
     m.def("set_ai2pot_path", [](const std::string& path) { g_ai2pot_path = path; });
     m.def("mtpParamOp", [](int64_t level) -> variable_list { return mtp_param_op(level); });
     m.def("nnMtpToEFVOp", [](NNMTP_ARGS) -> variable_list {

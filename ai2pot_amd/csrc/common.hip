@@ -31,6 +31,7 @@ struct DeviceWs {
 };
 std::mutex g_ws_mutex;
 std::vector<DeviceWs> g_ws;
+unsigned long long g_ws_generation = 0;   // bumped whenever a buffer is freed or replaced
 }  // namespace
 
 int ws_get(int slot, size_t bytes, void** out)
@@ -41,7 +42,10 @@ int ws_get(int slot, size_t bytes, void** out)
     if ((int)g_ws.size() <= dev) g_ws.resize(dev + 1);
     Buf& b = g_ws[dev].slot[slot];
     if (bytes > b.bytes) {
-        if (b.ptr) A2P_HIP_CHECK(hipFree(b.ptr));   // synchronises: no kernel still uses it
+        if (b.ptr) {
+            A2P_HIP_CHECK(hipFree(b.ptr));          // synchronises: no kernel still uses it
+            g_ws_generation++;                      // ... but a captured graph may still name it
+        }
         b.ptr = nullptr;
         b.bytes = 0;
         size_t want = bytes + bytes / 8 + 256;      // head-room so small growth does not realloc
@@ -76,6 +80,7 @@ int ws_release()
         b.ptr = nullptr;
         b.bytes = 0;
     }
+    g_ws_generation++;
     return A2P_OK;
 }
 
@@ -240,6 +245,12 @@ size_t a2p_workspace_bytes(void) { return a2p::ws_bytes(); }
 
 int a2p_workspace_release(void) { return a2p::ws_release(); }
 
+unsigned long long a2p_workspace_generation(void)
+{
+    std::lock_guard<std::mutex> lock(a2p::g_ws_mutex);
+    return a2p::g_ws_generation;
+}
+
 void a2p_profile_enable(int on)
 {
     std::lock_guard<std::mutex> lock(a2p::g_prof_mutex);
@@ -300,6 +311,12 @@ int a2p_check_status(void* stream_)
     rc = a2p::fill_zero(flags, 64, stream);
     if (rc) return rc;
     A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    if (host & a2p::ST_SEG_OVERFLOW) {
+        a2p::set_error("an atom is named by more pairs than its reduction segment holds (the list is not symmetric, or "
+                       "ghosts collect the pairs of several rows): forces of this call are incomplete; call again after "
+                       "a2p_pair_segment_capacity(a2p_pair_incoming_max(...))");
+        return A2P_ERR_SEGMENT;
+    }
     if (host & a2p::ST_NEIGH_OVERFLOW) {
         a2p::set_error("a neighbour count exceeds umax_num_neigh_atoms");
         return A2P_ERR_OVERFLOW;

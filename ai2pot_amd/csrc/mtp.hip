@@ -65,6 +65,7 @@ struct MtpArgs {
     int* seg_cursor;   // reduction segments of fixed capacity U (a2p::PairCsr): entries claimed per target,
     T* seg_g;          // the entries, and the entry that takes what overflows a segment;
     int seg_spare;     // seg_cursor is null when no forces are wanted
+    int seg_cap;       // capacity of a segment
     double* partial;   // [B, P, 10]  energy + virial per atom
     int* status;
     int E;             // table entries per neighbour
@@ -524,8 +525,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                     // is the number of pairs naming the target)
                     const int tg = b * NF + nj;
                     const int rk = atomicAdd(&a.seg_cursor[tg], 1);
-                    T* dst = a.seg_g + (size_t)(rk < a.U ? tg * a.U + rk : a.seg_spare) * 3;
-                    if (rk >= a.U) atomicOr(a.status, ST_NEIGH_OVERFLOW);
+                    T* dst = a.seg_g + (size_t)(rk < a.seg_cap ? tg * a.seg_cap + rk : a.seg_spare) * 3;
+                    if (rk >= a.seg_cap) atomicOr(a.status, ST_SEG_OVERFLOW);
                     dst[0] = gx; dst[1] = gy; dst[2] = gz;
                 }
                 fx += gx; fy += gy; fz += gz;
@@ -1023,7 +1024,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.binum = binum; a.bilist = bilist; a.bnumneigh = bnumneigh; a.bfirstneigh = bfirstneigh;
     a.brcs = brcs; a.btypes = btypes;
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
-    a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.partial = nullptr;
+    a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.seg_cap = 0; a.partial = nullptr;
     a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
     a.nn_exact = 1;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
@@ -1127,6 +1128,7 @@ int mtp_efv(void* handle, int K, double scaling, const T* coeffs, const T* lin, 
         a.seg_cursor = csr.cursor;
         a.seg_g = (T*)csr.seg_g;
         a.seg_spare = csr.n * csr.seg_cap;
+        a.seg_cap = csr.seg_cap;
     } else {
         rc = fill_zero(a.force, force_bytes, stream);
         if (rc) return rc;

@@ -176,7 +176,7 @@ __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& se
                     const int tg = b * NF + nj;
                     const int rk = atomicAdd(&seg.cursor[tg], 1);
                     pos = rk < seg.cap ? tg * seg.cap + rk : seg.spare;
-                    if (rk >= seg.cap) atomicOr(a.status, ST_NEIGH_OVERFLOW);
+                    if (rk >= seg.cap) atomicOr(a.status, ST_SEG_OVERFLOW);
                 }
                 if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
             }

@@ -173,7 +173,7 @@ __device__ __forceinline__ void staged_load(const NepArgs<T>& a, const SegArgs& 
                 }
             }
             pos[it] = rk < seg.cap ? t * seg.cap + rk : seg.spare;
-            if ((unsigned)rk >= (unsigned)seg.cap) { err |= ST_NEIGH_OVERFLOW; pos[it] = seg.spare; }
+            if ((unsigned)rk >= (unsigned)seg.cap) { err |= ST_SEG_OVERFLOW; pos[it] = seg.spare; }
         } else {
             pos[it] = 0;
         }

@@ -347,13 +347,18 @@ int pair_csr_begin(PairCsr* csr, bool with_rank, int B, int P, int U, int nghost
     return exclusive_scan_i32(csr->counts, csr->offsets, n, tiles, stream);
 }
 
+static thread_local int g_seg_capacity = 0;
+
+int pair_segment_capacity(int U) { return g_seg_capacity > U ? g_seg_capacity : U; }
+
 template <typename T>
-int pair_fixed_begin(PairCsr* csr, int B, int P, int U, int nghost, hipStream_t stream, void* also_zero,
+int pair_fixed_begin(PairCsr* csr, int B, int P, int U_rows, int nghost, hipStream_t stream, void* also_zero,
                      size_t also_bytes, int* cursor_ext, bool cursor_final)
 {
+    const int U = pair_segment_capacity(U_rows);
     const long long NT = (long long)B * (P + nghost);
     A2P_REQUIRE(NT * U + 1 < (1ll << 31), A2P_ERR_INVALID,
-                "pair_reduce: (natoms_pad + nghost) * umax exceeds 32-bit pair indexing");
+                "pair_reduce: (natoms_pad + nghost) * segment capacity exceeds 32-bit pair indexing");
     const int n = (int)NT;
     // workspace: cursor[n] | seg_g[(n*U + 1) * 3]   (the last entry takes what overflows)
     size_t bytes = (((size_t)n * sizeof(int) + 255) / 256) * 256;
@@ -439,6 +444,55 @@ template int pair_reduce<double>(double*, const double*, int, int, int, int, con
                                  const int*, hipStream_t);
 
 }  // namespace a2p
+
+// largest number of pairs naming one atom: counts (the histogram of a2p_pair_ranks without the ranks), then the maximum
+__global__ void incoming_max_kernel(const int* __restrict__ v, int n, int* __restrict__ out)
+{
+    __shared__ int sh[4];
+    int m = 0;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) m = max(m, v[i]);
+    m = a2p::wave_max(m);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(out, max(max(sh[0], sh[1]), max(sh[2], sh[3])));
+}
+
+extern "C" int a2p_pair_segment_capacity(int capacity)
+{
+    const int old = a2p::g_seg_capacity;
+    a2p::g_seg_capacity = capacity > 0 ? capacity : 0;
+    return old;
+}
+
+extern "C" int a2p_pair_incoming_max(int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                                     const int* bnumneigh, const int* bfirstneigh, int* max_incoming, void* stream_)
+{
+    using namespace a2p;
+    hipStream_t stream = (hipStream_t)stream_;
+    A2P_REQUIRE(batch >= 0 && natoms_pad >= 0 && umax >= 1 && nghost >= 0, A2P_ERR_INVALID, "pair_incoming_max: bad shape");
+    A2P_REQUIRE(binum && bnumneigh && bfirstneigh && max_incoming, A2P_ERR_INVALID, "pair_incoming_max: null pointer");
+    *max_incoming = 0;
+    if (batch == 0 || natoms_pad == 0) return A2P_OK;
+    const int NF = natoms_pad + nghost;
+    const size_t n = (size_t)batch * NF;
+    void* ws = nullptr;
+    int rc = ws_get(WS_CSR, (n + 64) * sizeof(int), &ws);
+    if (rc) return rc;
+    void* flags = nullptr;
+    rc = ws_get(WS_FLAGS, 64, &flags);
+    if (rc) return rc;
+    int* counts = (int*)ws;
+    rc = fill_zero(counts, (n + 64) * sizeof(int), stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(count_kernel, dim3(ceil_div((long long)batch * natoms_pad * 64, 256)), dim3(256), 0, stream, counts,
+                       (int*)nullptr, batch, natoms_pad, umax, NF, binum, bnumneigh, bfirstneigh, (int*)flags);
+    hipLaunchKernelGGL(incoming_max_kernel, dim3(std::min(ceil_div((long long)n, 256), 1024)), dim3(256), 0, stream,
+                       (const int*)counts, (int)n, counts + n);
+    A2P_HIP_CHECK(hipGetLastError());
+    A2P_HIP_CHECK(hipMemcpyAsync(max_incoming, counts + n, sizeof(int), hipMemcpyDeviceToHost, stream));
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    return A2P_OK;
+}
 
 extern "C" int a2p_pair_ranks(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
                               const int* bfirstneigh, int* rank, int* incoming, void* stream)

@@ -13,9 +13,24 @@ eager warm-up calls made here before the capture).  What a caller has to respect
   place (``tensor.copy_(...)``), keep shapes, dtypes and scalar arguments unchanged;
 * the outputs are overwritten by every replay: consume or clone them before the next one;
 * input checks that read back from the device are skipped (``validate=False`` is forced), so a
-  list that violates the contract is not reported from inside the graph.
+  list that violates the contract is not reported from inside the graph;
+* the graph names the library's per-device workspace by address.  A later call that needs a larger
+  workspace (a bigger system, another ``GraphedCall`` with bigger shapes) or ``a2p_workspace_release``
+  frees those buffers; ``replay`` notices (the library counts such events) and records the call
+  again instead of replaying onto freed memory.  The output tensors are then new objects: use what
+  ``replay`` returns.
 """
+import ctypes
+
 import torch
+
+from . import _lib
+
+
+def _generation():
+    fn = _lib.lib().a2p_workspace_generation
+    fn.restype = ctypes.c_ulonglong
+    return int(fn())
 
 
 class GraphedCall:
@@ -35,11 +50,27 @@ class GraphedCall:
                 op(*args, **kwargs)
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
+        self.recaptures = 0
+        self._capture()
+
+    def _capture(self):
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self.outputs = op(*args, **kwargs)
+            self.outputs = self._op(*self._args, **self._kwargs)
+        self._generation = _generation()
+
+    def valid(self):
+        """False once the workspace the graph names has been freed or replaced."""
+        return _generation() == self._generation
 
     def replay(self):
-        """Runs the recorded call on the current stream and returns the (static) output tensors."""
+        """Runs the recorded call on the current stream and returns the (static) output tensors.  If
+        the library's workspace changed since the capture, the call is first run eagerly (which sizes
+        the workspace again) and recorded anew."""
+        if not self.valid():
+            self._op(*self._args, **self._kwargs)
+            torch.cuda.synchronize(self.device)
+            self._capture()
+            self.recaptures += 1
         self.graph.replay()
         return self.outputs

@@ -52,6 +52,30 @@ def _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost):
     return B, P, U
 
 
+def _status_or_retry(call, B, P, U, nghost, binum, bnumneigh, bfirstneigh, device):
+    """Reads the device status of a call.  The fast kernels give every atom a reduction segment of
+    umax entries, which a list built with one cutoff never exceeds; a list that names an atom more
+    often (half lists, ghosts that collect the pairs of several rows) overflows it.  The status then
+    says so, and the call is repeated once with segments sized for the list at hand."""
+    L = _lib.lib()
+    stream = torch.cuda.current_stream(device).cuda_stream
+    try:
+        _lib.check_status(stream)
+        return
+    except _lib.A2PError as ex:
+        if ex.code != _lib.A2P_ERR_SEGMENT:
+            raise
+    most = _c.c_int(0)
+    _lib.check(L.a2p_pair_incoming_max(_c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(int(nghost)), _ptr(binum),
+                                       _ptr(bnumneigh), _ptr(bfirstneigh), _c.byref(most), _stream(device)))
+    old = L.a2p_pair_segment_capacity(_c.c_int(most.value))
+    try:
+        _lib.check(call())
+        _lib.check_status(stream)
+    finally:
+        L.a2p_pair_segment_capacity(_c.c_int(old))
+
+
 def _validate_batch(binum, bnumneigh, U, P):
     """Checks the reference leaves to asserts or to luck.  One device->host sync."""
     if binum.numel() == 0 or bnumneigh.numel() == 0:
@@ -111,15 +135,15 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
     L = _lib.lib()
     fn = L.a2p_nep_efv_f32 if dtype == torch.float32 else L.a2p_nep_efv_f64
     with torch.cuda.device(device):
-        rc = fn(_c.c_int(chebyshev_size), _c.c_int(n_radial_basis), _c.c_int(n_angular_basis),
+        call = lambda: fn(_c.c_int(chebyshev_size), _c.c_int(n_radial_basis), _c.c_int(n_angular_basis),
                 _c.c_int(l_max), _c.c_int(H), _c.c_int(ntypes), _ptr(coeffs), _ptr(w0), _ptr(b0),
                 _ptr(w1), _ptr(type_bias), _ptr(q_scaler_t), _c.c_double(rmax_radial),
                 _c.c_double(rmax_angular), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost),
                 _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs),
                 _ptr(btypes), _ptr(etot), _ptr(force), _ptr(virial), _ptr(desc), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, nghost, binum, bnumneigh, bfirstneigh, device)
     return etot, force, virial, desc
 
 
@@ -263,7 +287,7 @@ def nep_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
     L = _lib.lib()
     fn = L.a2p_nep_loss_f32 if dtype == torch.float32 else L.a2p_nep_loss_f64
     with torch.cuda.device(device):
-        rc = fn(_c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+        call = lambda: fn(_c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
                 _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_int(n_radial_basis),
                 _c.c_int(n_angular_basis), _c.c_int(l_max), _c.c_int(H), _c.c_int(ntypes), _ptr(coeffs), _ptr(w0),
                 _ptr(b0), _ptr(w1), _ptr(type_bias), _ptr(q_scaler), _c.c_double(rmax_radial),
@@ -272,9 +296,9 @@ def nep_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
                 _ptr(out["energy"]), _ptr(out["force"]), _ptr(out["virial"]), _ptr(out.get("dcoeffs")),
                 _ptr(out.get("dw0")), _ptr(out.get("db0")), _ptr(out.get("dw1")), _ptr(out.get("dbias")),
                 _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, 0, binum, bnumneigh, bfirstneigh, device)
     return out
 
 
@@ -343,6 +367,7 @@ def nepToEFLossOp(e_weight, f_weight, betot_dft, bforce_dft, chebyshev_size, n_r
 # linear MTP  (source/descriptor/mtpr/bind/mtpr_bind.cc:30-457)
 # --------------------------------------------------------------------------------------------
 _plans = {}
+_plans_by_content = {}
 
 
 def set_ai2pot_path(path):
@@ -366,13 +391,16 @@ def mtpParamOp(mtp_level, device="cpu"):
 def _mtp_plan(alpha_moments_count, basic_t, times_t, mapping_t, device):
     """Plan handle for a set of table tensors.  The tables are model constants (registered
     buffers in the reference, ai2pot/models/mtp/linear_mtp.py:63-69): they are read back to
-    the host once and cached by storage address, shape and version."""
+    the host once.  Two caches: by storage address, shape and version of the three tensors (the entry
+    keeps the tensors alive, so an address cannot come back with other contents while it is cached;
+    the oldest entries are dropped first), and by the tables' contents, which owns the plan handles
+    (never destroyed: a captured graph may still name one, and distinct tables are few)."""
     key = (device.index, int(alpha_moments_count),
            basic_t.data_ptr(), tuple(basic_t.shape), basic_t._version,
            times_t.data_ptr(), tuple(times_t.shape), times_t._version,
            mapping_t.data_ptr(), tuple(mapping_t.shape), mapping_t._version)
     if key in _plans:
-        return _plans[key]
+        return _plans[key][:2]
     for name, t in (("alpha_index_basic", basic_t), ("alpha_index_times", times_t),
                     ("alpha_moment_mapping", mapping_t)):
         _req(isinstance(t, torch.Tensor) and t.dtype == torch.int32, "%s must be an int32 tensor" % name)
@@ -382,18 +410,20 @@ def _mtp_plan(alpha_moments_count, basic_t, times_t, mapping_t, device):
     basic = basic_t.detach().cpu().contiguous().numpy()
     times = times_t.detach().cpu().contiguous().numpy().reshape(-1, 4)
     mapping = mapping_t.detach().cpu().contiguous().numpy()
-    handle = _c.c_void_p()
-    with torch.cuda.device(device):
-        rc = _lib.lib().a2p_mtp_plan_create(
-            _c.c_int(int(alpha_moments_count)), _c.c_int(basic.shape[0]), basic.ctypes.data_as(_c.c_void_p),
-            _c.c_int(times.shape[0]), times.ctypes.data_as(_c.c_void_p), _c.c_int(mapping.size),
-            mapping.ctypes.data_as(_c.c_void_p), _c.byref(handle))
-    _lib.check(rc)
-    if len(_plans) > 64:
-        _, old = _plans.popitem()
-        _lib.lib().a2p_mtp_plan_destroy(old[0])
-    _plans[key] = (handle, mapping.size)
-    return _plans[key]
+    content = (device.index, int(alpha_moments_count), basic.shape, basic.tobytes(), times.tobytes(), mapping.tobytes())
+    if content not in _plans_by_content:
+        handle = _c.c_void_p()
+        with torch.cuda.device(device):
+            rc = _lib.lib().a2p_mtp_plan_create(
+                _c.c_int(int(alpha_moments_count)), _c.c_int(basic.shape[0]), basic.ctypes.data_as(_c.c_void_p),
+                _c.c_int(times.shape[0]), times.ctypes.data_as(_c.c_void_p), _c.c_int(mapping.size),
+                mapping.ctypes.data_as(_c.c_void_p), _c.byref(handle))
+        _lib.check(rc)
+        _plans_by_content[content] = (handle, mapping.size)
+    while len(_plans) >= 64:
+        del _plans[next(iter(_plans))]                     # the oldest address entry; its plan stays with its contents
+    _plans[key] = _plans_by_content[content] + ((basic_t, times_t, mapping_t),)
+    return _plans[key][:2]
 
 
 def _mtp_common(coeffs, linear_coeffs, type_bias, alpha_moments_count, alpha_index_basic,
@@ -439,14 +469,14 @@ def _mtp_efv(want_virial, chebyshev_size, scaling, coeffs, linear_coeffs, type_b
     L = _lib.lib()
     fn = L.a2p_mtp_efv_f32 if dtype == torch.float32 else L.a2p_mtp_efv_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
+        call = lambda: fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
                 _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax),
                 _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
                 _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(etot),
                 _ptr(force), _ptr(virial), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, nghost, binum, bnumneigh, bfirstneigh, device)
     _zbl_add(zbl[0], zbl[1], zbl[2], zbl[3], type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
              etot, force, virial, validate)
     return etot, force, virial
@@ -503,7 +533,7 @@ def mtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
     L = _lib.lib()
     fn = L.a2p_mtp_loss_f32 if dtype == torch.float32 else L.a2p_mtp_loss_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+        call = lambda: fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
                 _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_double(scaling),
                 _ptr(coeffs), _ptr(linear_coeffs), _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes),
                 _ptr(q_scaler), _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U),
@@ -511,9 +541,9 @@ def mtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
                 _ptr(out["bloss"]), _ptr(out["rmse"]), _ptr(out["energy"]), _ptr(out["force"]),
                 _ptr(out["virial"]), _ptr(out.get("dcoeffs")), _ptr(out.get("dlinear")),
                 _ptr(out.get("dbias")), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, 0, binum, bnumneigh, bfirstneigh, device)
     return out
 
 
@@ -595,14 +625,14 @@ def _mtp_esites_raw(chebyshev_size, scaling, coeffs, linear_coeffs, type_bias, a
     L = _lib.lib()
     fn = L.a2p_mtp_esites_f32 if dtype == torch.float32 else L.a2p_mtp_esites_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
+        call = lambda: fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _ptr(linear_coeffs),
                 _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax),
                 _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
                 _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(e_sites),
                 _ptr(desc), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, nghost, binum, bnumneigh, bfirstneigh, device)
     return e_sites, desc
 
 
@@ -709,13 +739,13 @@ def mtp_lin_components(chebyshev_size, scaling, coeffs, alpha_moments_count, alp
     L = _lib.lib()
     fn = L.a2p_mtp_lin_components_f32 if dtype == torch.float32 else L.a2p_mtp_lin_components_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _c.c_int(int(nmus)),
+        call = lambda: fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _c.c_int(int(nmus)),
                 _c.c_int(ntypes), _ptr(q_scaler), _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P),
                 _c.c_int(U), _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes),
                 _ptr(ecomp), _ptr(fcomp), _ptr(vcomp), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, 0, binum, bnumneigh, bfirstneigh, device)
     return ecomp, fcomp, vcomp
 
 
@@ -809,14 +839,14 @@ def _nnmtp_call(want, chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_c
     L = _lib.lib()
     fn = L.a2p_nnmtp_efv_f32 if dtype == torch.float32 else L.a2p_nnmtp_efv_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0), _ptr(w1), _ptr(type_bias),
+        call = lambda: fn(plan, _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0), _ptr(w1), _ptr(type_bias),
                 _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_shifter), _ptr(q_scaler), _c.c_double(rmax),
                 _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost), _ptr(binum),
                 _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(etot),
                 _ptr(force), _ptr(virial), _ptr(e_sites), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, nghost, binum, bnumneigh, bfirstneigh, device)
     return etot, force, virial, e_sites
 
 
@@ -975,7 +1005,7 @@ def nnmtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial
     L = _lib.lib()
     fn = L.a2p_nnmtp_loss_f32 if dtype == torch.float32 else L.a2p_nnmtp_loss_f64
     with torch.cuda.device(device):
-        rc = fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
+        call = lambda: fn(plan, _c.c_double(e_weight), _c.c_double(f_weight), _c.c_double(v_weight), _ptr(betot_dft),
                 _ptr(bforce_dft), _ptr(bvirial_dft), _c.c_int(chebyshev_size), _c.c_int(H), _ptr(coeffs), _ptr(w0),
                 _ptr(w1), _ptr(type_bias), _c.c_int(int(nmus)), _c.c_int(ntypes), _ptr(q_shifter), _ptr(q_scaler),
                 _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U), _ptr(binum),
@@ -983,9 +1013,9 @@ def nnmtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial
                 _ptr(out["energy"]), _ptr(out["force"]), _ptr(out["virial"]), _ptr(out.get("dcoeffs")),
                 _ptr(out.get("dw0")), _ptr(out.get("dw1")), _ptr(out.get("dbias")),
                 _c.c_int(1 if exact_gradient else 0), _stream(device))
-        _lib.check(rc)
+        _lib.check(call())
         if validate:
-            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+            _status_or_retry(call, B, P, U, 0, binum, bnumneigh, bfirstneigh, device)
     return out
 
 

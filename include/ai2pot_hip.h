@@ -24,6 +24,7 @@ extern "C" {
 #define A2P_ERR_HIP 2       /* a HIP runtime call failed                                     */
 #define A2P_ERR_OVERFLOW 3  /* a neighbour count exceeds the row capacity umax               */
 #define A2P_ERR_INPUT 4     /* device-side input check failed (bad neighbour / type index)   */
+#define A2P_ERR_SEGMENT 5   /* an atom is named by more pairs than its reduction segment holds */
 
 const char* a2p_last_error(void);
 
@@ -38,11 +39,15 @@ int a2p_abi_version(void);
  * a2p_workspace_release synchronises the device and frees it (the next call allocates again). */
 size_t a2p_workspace_bytes(void);
 int a2p_workspace_release(void);
+/* Counts the times a workspace buffer was freed or replaced by a larger one (any device).  A captured
+ * HIP graph holds raw pointers into the workspace: record the value at capture and replay only while
+ * it is unchanged (a larger call or a2p_workspace_release in between invalidates the graph). */
+unsigned long long a2p_workspace_generation(void);
 
 /* Reads and clears the device status word that kernels set when an input violates the
  * contract (neighbour index outside [0, natoms_pad+nghost), type index outside
- * [0, ntypes), numneigh > umax).  Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT or
- * A2P_ERR_OVERFLOW.  The reference has no such check: it asserts or overflows
+ * [0, ntypes), numneigh > umax, more pairs naming one atom than its reduction segment holds).
+ * Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT, A2P_ERR_OVERFLOW or A2P_ERR_SEGMENT.  The reference has no such check: it asserts or overflows
  * (source/nblist/include/neighborList.h:550, commented-out assert). */
 int a2p_check_status(void* stream);
 
@@ -105,6 +110,21 @@ int a2p_nep_efv_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, 
  * alone.  a2p_pair_ranks fills the two buffers from the list alone. */
 int a2p_pair_ranks(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
                    const int* bfirstneigh, int* rank, int* incoming, void* stream);
+
+/* Reduction segments for lists that are not symmetric (no counterpart in the reference, which adds
+ * forces with atomics, nep.h:498-513).  The fast NEP / MTP kernels store the derivative of every
+ * pair into a segment owned by the neighbour it names, umax entries per atom: a list built with one
+ * cutoff names an atom no more often than its own row is long.  Half lists, or ghosts that collect
+ * the pairs of several rows (LAMMPS domains), can exceed that: the kernels then flag the call
+ * (a2p_check_status returns A2P_ERR_SEGMENT; the forces of that call are incomplete) and the caller
+ * repeats it with larger segments:
+ *   a2p_pair_incoming_max   largest number of pairs naming one atom (HOST int out; synchronises),
+ *   a2p_pair_segment_capacity(c)  segments of max(c, umax) entries for the following calls of the
+ *                           CALLING THREAD (0 = back to umax); returns the previous setting.
+ * The operator libraries and ai2pot_amd.ops do this by themselves unless validation is switched off. */
+int a2p_pair_incoming_max(int batch, int natoms_pad, int umax, int nghost, const int* binum, const int* bnumneigh,
+                          const int* bfirstneigh, int* max_incoming, void* stream);
+int a2p_pair_segment_capacity(int capacity);
 
 int a2p_nep_efv_ranked_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
                            int ntypes, const float* coeffs, const float* w0, const float* b0,

@@ -289,3 +289,60 @@ def test_nep_loss_ops(dropin):
     out2 = torch.ops.nep.nepToEFLossOp(1.0, 0.7, t(labels["energy"]), t(labels["force"]), *sizes,
                                        *[p.detach() for p in params], *tail)
     assert len(out2) == 3 and close(out2[0].cpu().numpy(), g["ef/bloss"])
+
+
+def test_asymmetric_list_names_an_atom_more_often_than_a_row_is_long(oracle, dropin):
+    """A list in which one atom is named by more pairs than umax (here every row names atom 0 in all of
+    its slots, as a half list or a ghost shared by several rows can): the fixed reduction segments of
+    the fast kernels overflow, the status says so, and both operator layers repeat the call with larger
+    segments.  Results equal the oracle's scatter; with validation off the overflow is reported by an
+    explicit status check and by nothing else."""
+    import torch
+    from ai2pot_amd import _lib, ops
+    from test_gpu_nep import _model_to_device, check
+    _, _, _, o = small(oracle, n=120, dtype=np.float64)
+    o = list(o)
+    umax = int(np.asarray(o[2]).max())
+    umax += (-umax) % 4
+    rows = np.asarray(o[3])[:, :umax].copy()
+    rows[rows >= 0] = 0                                    # every pair names atom 0: 120 rows x ~50 pairs > umax
+    o[3] = rows
+    o[4] = np.asarray(o[4])[:, :umax].copy()
+    nb = synth.pack_batch([tuple(o)])
+    assert int((rows == 0).sum()) > umax
+    m = synth.nep_model()
+    md = _model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    z = torch.zeros(36, dtype=torch.float64, device="cuda:0")
+    args = (8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"], d["binum"], d["bilist"],
+            d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], 0, 7.0, 4.0, md["q_scaler"],
+            0.0, 0.0, z, z)
+    ref = oracle.nep_efv(m, nb, np.float64)
+    for fn in (ops.nepToEFVOp, torch.ops.nep.nepToEFVOp):
+        out = [t.cpu().numpy() for t in fn(*args)]
+        check(out, ref, np.float64)
+    # validation off: no exception from the call, the explicit check reports the overflow
+    ops.nepToEFVOp(*args, validate=False)
+    with pytest.raises(_lib.A2PError) as ei:
+        _lib.check_status(torch.cuda.current_stream().cuda_stream)
+    assert ei.value.code == _lib.A2P_ERR_SEGMENT
+    torch.ops.nep.set_validate(False)
+    try:
+        torch.ops.nep.nepToEFVOp(*args)
+        with pytest.raises(RuntimeError):
+            torch.ops.nep.check_status(d["brcs"])
+    finally:
+        torch.ops.nep.set_validate(True)
+    # linear MTP through the same segments
+    tables = mtp_param.mtp_param(10)
+    mm = synth.mtp_model(tables, 3, 8, 7.0, 0.5, 77)
+    f64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64)).to("cuda:0")
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to("cuda:0")
+    margs = (mm["chebyshev_size"], 1.0, f64(mm["coeffs"]), f64(mm["linear_coeffs"]), f64(mm["type_bias"]),
+             mm["alpha_moments_count"], i32(mm["alpha_index_basic"]), i32(mm["alpha_index_times"]),
+             i32(mm["alpha_moment_mapping"]), mm["nmus"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"],
+             d["brcs"], d["btypes"], i32(mm["type_map"]), 0, mm["rmax"], mm["rmin"], f64(mm["q_scaler"]), 0.0, 0.0, z, z)
+    mref = oracle.mtp_efv(mm, nb)
+    for fn in (ops.linearMtpToEFVOp, torch.ops.mtpr.linearMtpToEFVOp):
+        out = [t.cpu().numpy() for t in fn(*margs)]
+        check(out, mref, np.float64)

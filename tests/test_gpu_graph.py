@@ -58,3 +58,34 @@ def test_mtp_graph(oracle, level):
     args = esites_args(m, md, d)
     replay_matches_eager(ops.linearMtpToEFVOp, args, d["brcs"], 3)
     replay_matches_eager(ops.linearMtpToEsitesOp, args, d["brcs"], 1)
+
+
+def test_graph_survives_a_workspace_change(oracle):
+    """A captured graph names the library's workspace by address.  Releasing the workspace (or a later
+    call that needs a larger one) is noticed by the next replay, which records the call again instead of
+    replaying onto freed memory; the result still equals the eager call."""
+    import torch
+    from ai2pot_amd import _lib, ops
+    from ai2pot_amd.graph import GraphedCall
+    from test_gpu_nep import _model_to_device
+    lat, pos = synth.fcc_cell(4, 4.6, 0.15, 63)
+    ty = synth.rng_randint(64, pos.shape[0], 3)
+    nb = synth.pack_batch([oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 6.0, 100)])
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    md = _model_to_device(m, torch.float32)
+    d = to_device(nb, torch.float32)
+    args = (m["chebyshev_size"], m["n_radial_basis"], m["n_angular_basis"], m["l_max"], md["coeffs"], md["w0"],
+            md["b0"], md["w1"], md["type_bias"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"],
+            d["btypes"], md["type_map"], 0, m["rmax_radial"], m["rmax_angular"], md["q_scaler"])
+    g = GraphedCall(ops.nepToEFVOp, *args)
+    want = [t.clone() for t in ops.nepToEFVOp(*args, validate=False)]
+    first = [t.clone() for t in g.replay()]
+    torch.cuda.synchronize()
+    assert g.valid() and g.recaptures == 0
+    _lib.check(_lib.lib().a2p_workspace_release())
+    assert not g.valid()
+    again = g.replay()
+    torch.cuda.synchronize()
+    assert g.valid() and g.recaptures == 1
+    for a, b, c in zip(first, again, want):
+        assert torch.equal(a, c) and torch.equal(b, c)
