@@ -1,7 +1,7 @@
 """Builds the drop-in operator libraries into ai2pot_amd/_lib/ (the directory a reference
 installation calls ai2pot/_lib):
 
-    libnep_bind.so, libmtpr_bind.so, libnnmtp_bind.so, libfvt_sr_op_bind.so   -- TORCH_LIBRARY registrations
+    libnep_bind.so, libmtpr_bind.so, libnnmtp_bind.so, libfvt_sr_op_bind.so, libnblist_bind.so   -- TORCH_LIBRARY registrations
     nblist.<abi>.so                                          -- CPython module `nblist`
 
 They are thin: argument checks plus calls into libai2pot_hip.so (found through an $ORIGIN
@@ -65,8 +65,8 @@ def build_bind(verbose=True):
         raise RuntimeError("build libai2pot_hip.so first (python -m ai2pot_amd.build)")
     os.makedirs(OUT, exist_ok=True)
     jobs = [lambda: _torch_lib("nep_bind"), lambda: _torch_lib("mtpr_bind"), lambda: _torch_lib("nnmtp_bind"),
-            lambda: _torch_lib("fvt_sr_op_bind"), _nblist_module]
-    with ThreadPoolExecutor(max_workers=5) as ex:
+            lambda: _torch_lib("fvt_sr_op_bind"), lambda: _torch_lib("nblist_bind"), _nblist_module]
+    with ThreadPoolExecutor(max_workers=6) as ex:
         outs = [f.result() for f in [ex.submit(j) for j in jobs]]
     if verbose:
         for o in outs:

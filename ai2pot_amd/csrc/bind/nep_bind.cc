@@ -91,6 +91,52 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
     return {e, f};
 }
 
+// Energy, forces and virial of ONE periodic structure from the compact lists cut by
+// torch.ops.nblist.find_info4mlff_compact_ (no counterpart in the reference: its operators take the
+// padded 7-tensor contract only).  The forces are a gather over each atom's own list, without
+// atomics; see include/ai2pot_hip.h, a2p_nep_efv_compact_*.
+variable_list nep_run_compact(int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const at::Tensor& coeffs,
+                              const at::Tensor& w0, const at::Tensor& b0, const at::Tensor& w1, const at::Tensor& bias,
+                              const at::Tensor& types, const at::Tensor& compact, int64_t umax,
+                              const at::Tensor& type_map, double rr, double ra, const at::Tensor& q_scaler)
+{
+    TORCH_CHECK(coeffs.is_cuda() && (coeffs.scalar_type() == at::kFloat || coeffs.scalar_type() == at::kDouble),
+                "coeffs must be a float32 or float64 tensor on a HIP device");
+    NepModel m = check_model(K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, type_map, coeffs);
+    check_device_float(coeffs, q_scaler, "q_scaler");
+    TORCH_CHECK(q_scaler.numel() == m.D, "q_scaler must have ", m.D, " elements");
+    check_device_int(coeffs, types, "types");
+    const int N = (int)types.numel();
+    const bool f32 = coeffs.scalar_type() == at::kFloat;
+    TORCH_CHECK(a2p_nep_efv_compact_supported(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, f32 ? 4 : 8) == 1,
+                "nepToEFVCompactOp covers chebyshev_size 8, n_radial 4 or 6, n_angular 4, l_max 4, at most 4 species; "
+                "use nepToEFVOp for this model");
+    const size_t need = a2p_nblist_compact_bytes(N, (int)umax, f32 ? 4 : 8);
+    TORCH_CHECK(need > 0 && compact.is_cuda() && compact.device() == coeffs.device() && compact.is_contiguous() &&
+                    (size_t)compact.nbytes() >= need,
+                "compact must be the device buffer filled by find_info4mlff_compact_ for these natoms and umax");
+    a2p_bind::DeviceGuard guard(coeffs);
+    auto opt = coeffs.options();
+    at::Tensor e = at::empty({1}, opt), f = at::empty({1, N, 3}, opt), v = at::empty({1, 9}, opt);
+    void* st = current_stream(coeffs);
+    int rc;
+    if (f32)
+        rc = a2p_nep_efv_compact_f32(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<float>(),
+                                     w0.data_ptr<float>(), b0.data_ptr<float>(), w1.data_ptr<float>(),
+                                     bias.data_ptr<float>(), q_scaler.data_ptr<float>(), rr, ra, N, (int)umax,
+                                     types.data_ptr<int>(), compact.data_ptr(), e.data_ptr<float>(),
+                                     f.data_ptr<float>(), v.data_ptr<float>(), st);
+    else
+        rc = a2p_nep_efv_compact_f64(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<double>(),
+                                     w0.data_ptr<double>(), b0.data_ptr<double>(), w1.data_ptr<double>(),
+                                     bias.data_ptr<double>(), q_scaler.data_ptr<double>(), rr, ra, N, (int)umax,
+                                     types.data_ptr<int>(), compact.data_ptr(), e.data_ptr<double>(),
+                                     f.data_ptr<double>(), v.data_ptr<double>(), st);
+    check_rc(rc);
+    check_device_status(coeffs);
+    return {e, f, v};
+}
+
 struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
     static variable_list forward(torch::autograd::AutogradContext* ctx, bool with_virial, double e_w, double f_w,
                                  double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
@@ -176,6 +222,7 @@ struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
 
 TORCH_LIBRARY(nep, m)
 {
+    m.def("nepToEFVCompactOp", &nep_run_compact);
     // no counterpart in the reference: the per-call device status check (one stream synchronisation per
     // call) can be switched off for loops that should run ahead of the device, and asked for explicitly
     m.def("set_validate", [](bool on) { validate_flag() = on; });

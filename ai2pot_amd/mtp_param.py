@@ -6,7 +6,7 @@ src/mtpParamOp.cc:25-63): the tables are data, read either from an ``NN.almtp`` 
 file (same search rule as the reference: ``$AI2POT_PATH/source/descriptor/mtpr/MTP_templates/``
 or ``<package path>/_data/MTP_templates/``) or, when no template directory is available,
 from the compact table archive packaged with this module (``_data/mtp_tables.npz``, levels
-6-22, produced from the same MLIP-3 template files by ``_data/make_mtp_tables.py``).
+6-22, produced from the same MLIP-3 template files by ``tests/golden/make_mtp_tables.py``).
 """
 import os
 import re

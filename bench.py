@@ -178,7 +178,47 @@ def nep_structure(kind, n_or_reps):
     return lattice, pos, types, disp
 
 
-def run_nep_md(args, kind, size, rebuild=True):
+class OpsStepper:
+    """The molecular-dynamics step through registered operators only (torch.ops.nblist.find_info4mlff_compact_
+    + torch.ops.nep.nepToEFVCompactOp from the bind libraries), as a TorchScript model or a C++ host would
+    drive it: no ctypes, no calculator object.  Validation is switched off for the timed loop (no
+    synchronisation per call) and the status word is read once at the end."""
+
+    def __init__(self, model, n, lattice, types, dev, umax=200, reorder_every=64):
+        import torch
+        from ai2pot_amd import bind_build
+        for name in ("libnblist_bind.so", "libnep_bind.so"):
+            path = os.path.join(os.path.dirname(os.path.abspath(bind_build.__file__)), "_lib", name)
+            if not os.path.exists(path):
+                sys.exit("bench.py: %s missing: run python -m ai2pot_amd.build --bind" % path)
+            torch.ops.load_library(path)
+        f = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(dev)
+        self.model_args = (int(model["chebyshev_size"]), int(model["n_radial_basis"]), int(model["n_angular_basis"]),
+                           int(model["l_max"]), f(model["coeffs"]), f(model["w0"]), f(model["b0"]), f(model["w1"]),
+                           f(model["type_bias"]))
+        self.tail = (torch.from_numpy(np.ascontiguousarray(model["type_map"], np.int32)).to(dev),
+                     float(model["rmax_radial"]), float(model["rmax_angular"]), f(model["q_scaler"]))
+        self.rr, self.ra = float(model["rmax_radial"]), float(model["rmax_angular"])
+        self.lattice = torch.from_numpy(np.ascontiguousarray(lattice, np.float32).reshape(3, 3))
+        self.types = torch.from_numpy(np.ascontiguousarray(types, np.int32)).to(dev)
+        self.n, self.umax, self.reorder_every = n, umax, reorder_every
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.rows = [torch.empty(n, **i32), torch.empty(n, **i32), torch.empty((n, umax), **i32),
+                     torch.empty((n, umax, 3), dtype=torch.float32, device=dev), torch.empty(n, **i32)]
+        self.compact = torch.empty(torch.ops.nblist.compact_bytes(n, umax, 4), dtype=torch.uint8, device=dev)
+        self.builds = 0
+        self.build = torch.ops.nblist.find_info4mlff_compact_
+        self.efv = torch.ops.nep.nepToEFVCompactOp
+
+    def step(self, coords):
+        update = (1 if self.builds else 0) | (2 if self.builds % self.reorder_every else 0)
+        self.build(self.lattice, self.types, coords, self.rr, self.umax, True, [True, True, True], self.rr, self.ra,
+                   update, *self.rows, self.compact)
+        self.builds += 1
+        return self.efv(*self.model_args, self.types, self.compact, self.umax, *self.tail)
+
+
+def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     import torch
     from ai2pot_amd import _lib, synth
     from ai2pot_amd.calculator import NepCalculator
@@ -187,6 +227,7 @@ def run_nep_md(args, kind, size, rebuild=True):
     n = pos.shape[0]
     model = synth.nep_model(seed=3006)
     calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev)
+    ops_path = OpsStepper(model, n, lattice, types, dev) if (via_ops or (rebuild and calc.path == "gather")) else None
     coords0 = torch.from_numpy(pos.astype(np.float32)).to(dev)
     disp_t = torch.from_numpy(disp.astype(np.float32)).to(dev)
     coords = torch.empty_like(coords0)
@@ -196,11 +237,24 @@ def run_nep_md(args, kind, size, rebuild=True):
     def step(k):
         if rebuild:     # a small deterministic displacement: every step builds a different list
             torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
-            return calc.step(coords)
+            return ops_path.step(coords) if via_ops else calc.step(coords)
         calc.evaluate(stream)
 
     L = _lib.lib()
+    if via_ops:
+        torch.ops.nblist.set_validate(False)
+        torch.ops.nep.set_validate(False)
     elapsed, kernels = timed(step, args.steps, args.warmup, L, keep=3)
+    if via_ops:
+        last = step(args.warmup + args.steps - 1)
+        ref = calc.step(coords)
+        torch.ops.nblist.check_status(coords)
+        torch.ops.nblist.set_validate(True)
+        torch.ops.nep.set_validate(True)
+        # same kernels; the processing orders of the two drivers may differ, hence rounding-level bars
+        if not (torch.allclose(last[0], ref[0], rtol=1e-5) and torch.allclose(last[1][0], ref[1], rtol=1e-4, atol=1e-4)
+                and torch.allclose(last[2][0], ref[2], rtol=1e-4, atol=1e-2)):
+            sys.exit("bench.py: the operator path and the calculator disagree")
     if args.graph:
         if rebuild:
             sys.exit("bench.py: --graph needs a workload without list rebuild (the build synchronises with the host)")
@@ -231,7 +285,9 @@ def run_nep_md(args, kind, size, rebuild=True):
               "umax": 200, "mean_neighbors_radial": nn_r, "mean_neighbors_angular": nn_a,
               "per_step": ("neighbor rebuild (padded arrays + compact lists) + " if rebuild else "") +
                           "descriptors + ANN + force/virial",
-              "path": calc.path, "launch": "hip graph replay" if args.graph else "eager"}
+              "path": calc.path, "launch": "hip graph replay" if args.graph else "eager",
+              "driver": "torch.ops.nblist.find_info4mlff_compact_ + torch.ops.nep.nepToEFVCompactOp, validation off"
+                        if via_ops else "NepCalculator (ctypes over the C ABI)"}
     roof, entries = roofline_of(kernels, work, args.workload)
     if roof is not None and roof["bound"] == "valu":
         # the same operator against the memory roofline (algorithmic bytes of the E/F/V operator)
@@ -257,6 +313,27 @@ def run_nep_md(args, kind, size, rebuild=True):
         lean.check()
         extra["without_padded_arrays"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
                                               unit="atom-steps/s")
+        if not via_ops:
+            # the same step (padded arrays included) driven through the registered operators alone
+            torch.ops.nblist.set_validate(False)
+            torch.ops.nep.set_validate(False)
+
+            def ops_step(k):
+                torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
+                return ops_path.step(coords)
+            for k in range(args.warmup):
+                ops_step(k)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for k in range(args.steps):
+                ops_step(args.warmup + k)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            torch.ops.nblist.check_status(coords)
+            torch.ops.nblist.set_validate(True)
+            torch.ops.nep.set_validate(True)
+            extra["through_torch_ops"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
+                                              unit="atom-steps/s", vs_calculator=dt / elapsed)
     return n, elapsed, kernels, roof, config, "f32", extra
 
 
@@ -483,6 +560,7 @@ def run_copy_probe(args):
 
 WORKLOADS = {
     "nep_md_1048576": lambda a: run_nep_md(a, "fcc", 64),         # the headline configuration (configs[4] of the benchmark definition)
+    "nep_md_1048576_ops": lambda a: run_nep_md(a, "fcc", 64, via_ops=True),   # the headline step through torch.ops only
     "nep_md_131072": lambda a: run_nep_md(a, "fcc", 32),
     "nep_efv_4096": lambda a: run_nep_md(a, "random", 4096, rebuild=False),   # configs[1]
     "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]

@@ -1,11 +1,11 @@
-"""Pack the MTP contraction tables of levels 6..22 into mtp_tables.npz.
+"""Pack the MTP contraction tables of levels 6..22 into ai2pot_amd/_data/mtp_tables.npz.
 
 The tables are data of MLIP-3 origin (https://gitlab.com/ashapeev/mlip-3), shipped by the
 reference as text templates (source/descriptor/mtpr/MTP_templates/NN.almtp).  This script
 parses those text files with this package's own parser and stores the four integer tables
 of each level; it is run once, by hand, where the template directory exists:
 
-    python ai2pot_amd/_data/make_mtp_tables.py /root/reference/source/descriptor/mtpr/MTP_templates
+    python tests/golden/make_mtp_tables.py /root/reference/source/descriptor/mtpr/MTP_templates
 """
 import os
 import sys
@@ -27,7 +27,7 @@ def main(src):
         out[key + "_mapping"] = t["alpha_moment_mapping"].astype(np.int16)
         print(level, t["alpha_moments_count"], t["alpha_index_basic"].shape,
               t["alpha_index_times"].shape, t["alpha_moment_mapping"].shape, t["nmus"])
-    dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mtp_tables.npz")
+    dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", "ai2pot_amd", "_data", "mtp_tables.npz")
     np.savez_compressed(dst, **out)
     print("wrote", dst, os.path.getsize(dst), "bytes")
 

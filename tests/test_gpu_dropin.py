@@ -20,7 +20,7 @@ LIBDIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))
 @pytest.fixture(scope="module")
 def dropin():
     import torch
-    for name in ("libnep_bind.so", "libmtpr_bind.so", "libnnmtp_bind.so", "libfvt_sr_op_bind.so"):
+    for name in ("libnep_bind.so", "libmtpr_bind.so", "libnnmtp_bind.so", "libfvt_sr_op_bind.so", "libnblist_bind.so"):
         path = os.path.join(LIBDIR, name)
         assert os.path.exists(path), "%s missing: run python -m ai2pot_amd.build --bind" % path
         torch.ops.load_library(path)
@@ -51,6 +51,108 @@ def test_nblist_module(oracle, dropin):
         dropin.find_info4mlff(lat, ty, pos, 7, 200, True, [True, True, True], False)
     with pytest.raises(RuntimeError):
         dropin.find_info4mlff(lat, ty, pos, 7.0, 10, True, [True, True, True], False)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64])
+def test_nblist_op_on_device_tensors(oracle, dropin, np_dtype):
+    """torch.ops.nblist.find_info4mlff: the arguments and seven results of the reference's
+    nblist.find_info4mlff (source/nblist/bind/nblist_bind.cc:35-189) as device tensors, bit-identical
+    to the oracle in both sort modes; the in-place form rewrites an earlier result."""
+    import torch
+    lat, pos, ty, ref = small(oracle, dtype=np_dtype)
+    dev = "cuda:0"
+    tlat = torch.from_numpy(lat.astype(np_dtype))
+    tty = torch.from_numpy(ty.astype(np.int32)).to(dev)
+    tpos = torch.from_numpy(pos.astype(np_dtype)).to(dev)
+    for sort in (False, True):
+        want = oracle.nblist(lat.astype(np_dtype), ty, pos.astype(np_dtype), 7.0, 200, sort=sort)
+        out = torch.ops.nblist.find_info4mlff(tlat, tty, tpos, 7.0, 200, True, [True, True, True], sort)
+        assert len(out) == 7 and all(t.is_cuda for t in out)
+        assert int(out[0]) == want[0] and int(out[6]) == 0
+        for a, b in zip(out[1:6], want[1:6]):
+            assert a.shape == b.shape
+            assert np.array_equal(a.cpu().numpy().view(np.uint8), b.view(np.uint8))
+    # the lattice may live on the device too
+    out_d = torch.ops.nblist.find_info4mlff(tlat.to(dev), tty, tpos, 7.0, 200, True, [True, True, True], False)
+    assert all(torch.equal(a, b) for a, b in zip(out_d, torch.ops.nblist.find_info4mlff(
+        tlat, tty, tpos, 7.0, 200, True, [True, True, True], False)))
+    # in place over an earlier list of other positions
+    lat2, pos2 = synth.random_packed(120, [14.0, 15.0, 13.0], 2.2, 29)
+    bufs = [t.clone() for t in torch.ops.nblist.find_info4mlff(
+        tlat, tty, torch.from_numpy(pos2.astype(np_dtype)).to(dev), 7.0, 200, True, [True, True, True], False)[1:6]]
+    torch.ops.nblist.find_info4mlff_(tlat, tty, tpos, 7.0, 200, True, [True, True, True], False, *bufs, True)
+    nn = ref[2]
+    for a, b in zip(bufs[:2] + bufs[4:], (ref[1], ref[2], ref[5])):
+        assert np.array_equal(a.cpu().numpy(), b)
+    fn, rc = bufs[2].cpu().numpy(), bufs[3].cpu().numpy()
+    for i in range(120):                                   # beyond a row's length the old entries may remain
+        assert np.array_equal(fn[i, :nn[i]], ref[3][i, :nn[i]])
+        assert np.array_equal(rc[i, :nn[i]].view(np.uint8), ref[4][i, :nn[i]].view(np.uint8))
+    with pytest.raises(RuntimeError):                      # umax too small: an error with validation on
+        torch.ops.nblist.find_info4mlff(tlat, tty, tpos, 7.0, 10, True, [True, True, True], False)
+    with pytest.raises(RuntimeError):                      # host coordinates: no CPU path
+        torch.ops.nblist.find_info4mlff(tlat, tty.cpu(), tpos.cpu(), 7.0, 200, True, [True, True, True], False)
+    with pytest.raises(RuntimeError):
+        torch.ops.nblist.find_info4mlff(tlat.double() if np_dtype == np.float32 else tlat.float(), tty, tpos, 7.0,
+                                        200, True, [True, True, True], False)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64])
+def test_compact_ops_match_the_calculator_and_the_oracle(oracle, dropin, np_dtype):
+    """torch.ops.nblist.find_info4mlff_compact_ + torch.ops.nep.nepToEFVCompactOp: the device-resident
+    step through registered operators only.  Same kernels as NepCalculator(path="gather"), so the
+    results are bitwise the calculator's; and within the gather path's bars of the oracle."""
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    from test_gpu_nep import _model_to_device
+    from test_gpu_nep_gather import _check
+    dev = "cuda:0"
+    dtype = torch.float32 if np_dtype == np.float32 else torch.float64
+    lat, pos, ty, nb = small(oracle, dtype=np_dtype)
+    m = synth.nep_model()
+    md = _model_to_device(m, dtype)
+    n, U = 120, 200
+    tlat = torch.from_numpy(lat.astype(np_dtype))
+    tty = torch.from_numpy(ty.astype(np.int32)).to(dev)
+    tpos = torch.from_numpy(pos.astype(np_dtype)).to(dev)
+    nbytes = torch.ops.nblist.compact_bytes(n, U, 4 if np_dtype == np.float32 else 8)
+    assert nbytes > 0 and torch.ops.nblist.compact_bytes(n, 13, 4) == 0
+    compact = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    i32 = dict(dtype=torch.int32, device=dev)
+    rows = [torch.empty(n, **i32), torch.empty(n, **i32), torch.empty((n, U), **i32),
+            torch.empty((n, U, 3), dtype=dtype, device=dev), torch.empty(n, **i32)]
+    model_args = (8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"])
+    tail = (md["type_map"], float(m["rmax_radial"]), float(m["rmax_angular"]), md["q_scaler"])
+    calc = NepCalculator(m, n, lat, ty, umax=U, dtype=dtype, device=dev, path="gather")
+    for with_rows in (True, False):
+        torch.ops.nblist.find_info4mlff_compact_(tlat, tty, tpos, 7.0, U, True, [True, True, True],
+                                                 float(m["rmax_radial"]), float(m["rmax_angular"]), 0,
+                                                 *(rows if with_rows else [None] * 5), compact)
+        e, f, v = torch.ops.nep.nepToEFVCompactOp(*model_args, tty, compact, U, *tail)
+        assert e.shape == (1,) and f.shape == (1, n, 3) and v.shape == (1, 9)
+        ce, cf, cv = calc.step(tpos)
+        calc.check()
+        assert torch.equal(e, ce) and torch.equal(f[0], cf) and torch.equal(v[0], cv)
+    for a, b in zip(rows, nb[1:6]):                        # the padded tensors, bit for bit
+        assert np.array_equal(a.cpu().numpy().view(np.uint8), b.view(np.uint8))
+    ref = oracle.nep_efv(m, synth.pack_batch([nb]), dtype=np_dtype)
+    _check((e.cpu().numpy(), f.cpu().numpy(), v.cpu().numpy()), ref, np_dtype)
+    # validation off: no per-call synchronisation, a flagged call surfaces at check_status
+    torch.ops.nblist.set_validate(False)
+    try:
+        small_compact = torch.empty(torch.ops.nblist.compact_bytes(n, 8, 4 if np_dtype == np.float32 else 8),
+                                    dtype=torch.uint8, device=dev)
+        torch.ops.nblist.find_info4mlff_compact_(tlat, tty, tpos, 7.0, 8, True, [True, True, True], 7.0, 4.0, 0,
+                                                 None, None, None, None, None, small_compact)
+        with pytest.raises(RuntimeError):
+            torch.ops.nblist.check_status(tpos)
+    finally:
+        torch.ops.nblist.set_validate(True)
+    with pytest.raises(RuntimeError):                      # a buffer that is too small is refused on the host
+        torch.ops.nep.nepToEFVCompactOp(*model_args, tty, compact[:1024], U, *tail)
+    with pytest.raises(RuntimeError):                      # padded outputs: all or none
+        torch.ops.nblist.find_info4mlff_compact_(tlat, tty, tpos, 7.0, U, True, [True, True, True], 7.0, 4.0, 0,
+                                                 rows[0], None, None, None, None, compact)
 
 
 def nep_args(oracle, dtype):
