@@ -135,6 +135,9 @@ def timed_replay(replay, steps, warmup):
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/<workload>_hbm_traffic.txt.  Kernels without a counter run report null.
 MEASURED_TRAFFIC = {
+    ("nep_md_1048576", "nbl_lists"): (2.00 * 2.410e5 + 1.691e6) * 1024,
+    ("nep_md_1048576", "nep_adjoint_kernel"): (2.00 * 4.792e5 + 5.464e5) * 1024,
+    ("nep_md_1048576", "nep_gather_kernel"): (2.00 * 2.782e6 + 4.844e4) * 1024,
 }
 
 
@@ -227,7 +230,7 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     n = pos.shape[0]
     model = synth.nep_model(seed=3006)
     calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev)
-    ops_path = OpsStepper(model, n, lattice, types, dev) if (via_ops or (rebuild and calc.path == "gather")) else None
+    ops_path = OpsStepper(model, n, lattice, types, dev) if (via_ops or (rebuild and calc.path == "gather" and not args.no_other_configs)) else None
     coords0 = torch.from_numpy(pos.astype(np.float32)).to(dev)
     disp_t = torch.from_numpy(disp.astype(np.float32)).to(dev)
     coords = torch.empty_like(coords0)
@@ -294,7 +297,7 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
         gbs = efv_bytes / (roof["avg_ms"] * 1e-3) / 1e9
         roof["hbm"] = dict(achieved=gbs, peak=PEAK_HBM_GBS, unit="GB/s", frac=gbs / PEAK_HBM_GBS, amount_per_launch=efv_bytes)
     extra = {"rooflines": entries}
-    if rebuild and calc.path == "gather" and not args.graph:
+    if rebuild and calc.path == "gather" and not args.graph and not args.no_other_configs:
         # the same step without the padded firstneigh / rcs arrays (energy, forces and virial only)
         lean = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, padded=False)
         lean.rebuild(coords0, stream)
@@ -579,7 +582,8 @@ def main():
     ap.add_argument("--workload", default="nep_md_1048576", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true",
-                    help="headline workload only: skip the short runs of the other benchmark configurations")
+                    help="the workload's own timed loop only: skip the short runs of the other benchmark configurations and "
+                         "the variants of the step (without padded arrays, through torch.ops)")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of the step captured as a HIP graph (workloads without list rebuild)")
     args = ap.parse_args()
