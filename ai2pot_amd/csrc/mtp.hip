@@ -12,8 +12,10 @@
 //   products      : level-ordered gather over the host-built plan (mtp_plan.h)
 //   energy        : E_i = bias[t] + sum_s lin[s] M[map[s]] / q_scaler[s]  (linearMtp.h:281-285)
 //   adjoint       : seed + reverse gather                                  (linearMtp.h:292-306)
-//   pair forces   : lane <- (neighbour, a share of the basic moments):
+//   pair forces   : lane <- (neighbour, a share of the monomial rows x^a y^b z^*):
 //                   dE_i/dr_ij = u sum_i adj_i m_i (g' - k g / r) + (1/r) sum_i adj_i g grad_u m_i
+//                   with the adjoints gathered by monomial and z^c by recurrence (pair_walk; three uniform
+//                   LDS reads per monomial instead of ten scattered ones per basic moment)
 //                   -> reduction segments of the neighbours (a2p::PairCsr), summed without float atomics
 // The loss gradient adds the tangent sweep (include/linearMtpLoss.h:371-398), the mixed
 // adjoint (:417-434) and the coefficient-gradient pass (:438-536) in the same structure;
@@ -40,13 +42,18 @@ __host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms)
 {
     return loss ? 2 * n_moms >= 512 : n_moms >= 1024;
 }
-// entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums
+// entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums.
+// In the energy / force / virial kernel the group sums (4 per thread) are written over the table once every
+// thread has finished reading it.
 __host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots)
 {
-    const int a = nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4);
+    int a = loss ? nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4) : nc * E;
+    if (!loss && a < 256 * 4) a = 256 * 4;
     const int b = max_level_slots * (loss ? 2 : 1);
     return a > b ? a : b;
 }
+// the dense adjoint array of the pair-derivative pass takes the place of the moments when it fits
+__host__ __device__ inline bool mtp_dense_in_moments(int nq, int nmp, int n_moms) { return nq * nmp <= n_moms; }
 constexpr int MTP_NGMAX = 16;     // most thread groups that share the basic moments of a chunk
 constexpr int MTP_KMAX = 16;      // radial basis size limit
 constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
@@ -201,19 +208,27 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
             const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
             const int dst = p.f_dst[s];                      // requested with the two words above
             T acc = (T)0, tacc = (T)0;
-            for (int k = 0; k < depth; k += 4) {
-                int2 w[4];
+            // all the slot's words (at most MTP_SLOT_CAP, the depth is shared by the wavefront) are requested
+            // before the first is used: one trip to memory per slot
+            int2 w[MTP_SLOT_CAP];
 #pragma unroll
-                for (int u = 0; u < 4; u++) w[u] = tp[(k + u) * 64];
+            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                if (k < depth) {
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int m0 = w[u].x & 0xffff, m1 = (int)((unsigned)w[u].x >> 16);
-                    const T mult = (T)w[u].y;
-                    const T v0 = M[m0], v1 = M[m1];
-                    acc += mult * v0 * v1;
-                    if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+                    for (int u = 0; u < 4; u++) w[k + u] = tp[(k + u) * 64];
                 }
-            }
+#pragma unroll
+            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                if (k < depth) {
+#pragma unroll
+                    for (int u = k; u < k + 4; u++) {
+                        const int m0 = w[u].x & 0xffff, m1 = (int)((unsigned)w[u].x >> 16);
+                        const T mult = (T)w[u].y;
+                        const T v0 = M[m0], v1 = M[m1];
+                        acc += mult * v0 * v1;
+                        if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+                    }
+                }
             if (multi) {
                 part[s - s0] = acc;
                 if (TANGENT) part2[s - s0] = tacc;
@@ -254,18 +269,24 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
             const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
             const int src = p.r_src[s];
             T acc = (T)0;
-            for (int k = 0; k < depth; k += 4) {
-                int2 w[4];
+            int2 w[MTP_SLOT_CAP];
 #pragma unroll
-                for (int u = 0; u < 4; u++) w[u] = tp[(k + u) * 64];
+            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                if (k < depth) {
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int dst = w[u].x & 0xffff, other = (int)((unsigned)w[u].x >> 16);
-                    const T mult = (T)w[u].y;
-                    acc += X[dst] * mult * M[other];
-                    if (MIXED) acc += mult * A[dst] * Tg[other];
+                    for (int u = 0; u < 4; u++) w[k + u] = tp[(k + u) * 64];
                 }
-            }
+#pragma unroll
+            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                if (k < depth) {
+#pragma unroll
+                    for (int u = k; u < k + 4; u++) {
+                        const int dst = w[u].x & 0xffff, other = (int)((unsigned)w[u].x >> 16);
+                        const T mult = (T)w[u].y;
+                        acc += X[dst] * mult * M[other];
+                        if (MIXED) acc += mult * A[dst] * Tg[other];
+                    }
+                }
             if (multi) part[s - s0] = acc;
             else X[src] += acc;
         }
@@ -299,9 +320,57 @@ __device__ __forceinline__ T block_sum(T v, T* scratch, int tid)
     return t;
 }
 
+// Pair derivatives of one neighbour by a walk over the monomial rows (mtp_plan.h): the lane owns the
+// neighbour whose table row is `t`, takes rows h, h + ng, ... and returns its share of
+//   gs = sum_i adj_i m_i (g' - k g / r),   w = sum_i adj_i g grad_u m_i,
+// with  c_q = sum_mu AD[q][mu] g_mu  and  d_q = sum_mu AD[q][mu] g'_mu  formed once per monomial:
+//   gs += m_q (d_q - k_q c_q / r),  w_x += c_q a x^(a-1) y^b z^c,  w_y += c_q b x^a y^(b-1) z^c,
+//   w_z += c_q c x^a y^b z^(c-1).
+template <typename T, int NMP>
+__device__ __forceinline__ void pair_walk(const T* __restrict__ t, const T* __restrict__ AD, const int* __restrict__ rows,
+                                          int nrows, int h, int ng, int kmax, int nmus, int OX, int OY, int OZ, int OG,
+                                          int ODG, T rinv, T& gs, T& wx, T& wy, T& wz)
+{
+    T g[NMP], dg[NMP];
+#pragma unroll
+    for (int mu = 0; mu < NMP; mu++) {
+        g[mu] = mu < nmus ? t[OG + mu] : (T)0;
+        dg[mu] = mu < nmus ? t[ODG + mu] : (T)0;
+    }
+    const T z = t[OZ + 1];
+    for (int r = h; r < nrows; r += ng) {
+        const int rw = rows[r];
+        const int ea = rw & 255, eb = (rw >> 8) & 255;
+        const int len = kmax - ea - eb + 1;
+        const T xa = t[OX + ea], yb = t[OY + eb];
+        const T xy = xa * yb;
+        const T Wx = (T)ea * t[OX + max(ea - 1, 0)] * yb;
+        const T Wy = (T)eb * xa * t[OY + max(eb - 1, 0)];
+        const T* ad = AD + (size_t)(rw >> 16) * NMP;
+        T zc = (T)1, zcm = (T)0, kf = (T)(ea + eb), cf = (T)0;
+        for (int c = 0; c < len; c++) {
+            T cq = (T)0, dq = (T)0;
+#pragma unroll
+            for (int mu = 0; mu < NMP; mu++) {
+                const T v = ad[mu];
+                cq += v * g[mu];
+                dq += v * dg[mu];
+            }
+            gs += xy * zc * (dq - kf * cq * rinv);
+            const T cz = cq * zc;
+            wx += cz * Wx;
+            wy += cz * Wy;
+            wz += cq * cf * zcm * xy;
+            zcm = zc; zc *= z; kf += (T)1; cf += (T)1;
+            ad += NMP;
+        }
+    }
+}
+
 // NT threads per centre atom: 64 for small tables, 256 when there is enough work per atom
+// (four workgroups of 256 threads fit the LDS of a CU at the larger levels: keep the registers to match)
 template <typename T, bool LOSS, int NT>
-__global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
+__global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_kernel(const MtpArgs<T> a)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const MtpPlanDevice& p = a.p;
@@ -326,7 +395,8 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     // neighbours, when the moments (and, in loss mode, their tangents) are dead: a long enough moment
     // vector lends them its place
     const bool share = mtp_gred_in_moments(LOSS, n_moms);
-    T* gred = share ? M : tab + MTP_NC * E;
+    // energy / force / virial kernel: the group sums are written over the table once it has been read
+    T* gred = LOSS ? (share ? M : tab + MTP_NC * E) : tab;
     T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots);   // loss mode: P[nc][nmus] | Q[nc][nmus]
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
@@ -353,6 +423,12 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
     for (int i = lane; i < n_basic; i += NT)
         bas[i] = (unsigned)p.basic[i * 4] | ((unsigned)p.basic[i * 4 + 1] << 8) |
                  ((unsigned)p.basic[i * 4 + 2] << 16) | ((unsigned)p.basic[i * 4 + 3] << 24);
+    int* rws = (int*)(bas + n_basic);        // monomial rows of the pair-derivative walk
+    int* dpos = rws + p.nrows;               // entry of each basic moment in the dense adjoint array
+    if (!LOSS) {
+        for (int i = lane; i < p.nrows; i += NT) rws[i] = p.rows[i];
+        for (int i = lane; i < n_basic; i += NT) dpos[i] = p.dense_pos[i];
+    }
     for (int q = lane; q < a.ntypes * nmus * K; q += NT) cf[q] = a.coeffs[(size_t)ti * a.ntypes * nmus * K + q];
     for (int i = lane; i < n_moms; i += NT) {
         M[i] = (T)0; A[i] = (T)0;
@@ -465,9 +541,26 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
 
     if (!LOSS) {
         // ---- pair derivatives ------------------------------------------------------------------
+        // The adjoints of the basic moments, gathered by monomial (mtp_plan.h); the moments are dead
+        T* AD = mtp_dense_in_moments(p.nq, p.nmp, n_moms) ? M : nnb + (a.H > 0 ? p.n_scalar + a.H : 0);
+        __syncthreads();
+        if (p.dense_unique) {
+            for (int e = lane; e < p.nq * p.nmp; e += NT) AD[e] = (T)0;
+            __syncthreads();
+            for (int i = lane; i < n_basic; i += NT) AD[dpos[i]] = A[i];
+        } else {
+            for (int e = lane; e < p.nq * p.nmp; e += NT) {
+                const int src = p.dense_src[e];
+                T v = (T)0;
+                if (src >= 0) v = A[src];
+                else if (src == -2)
+                    for (int q = p.dense_off[e]; q < p.dense_off[e + 1]; q++) v += A[p.dense_items[q]];
+                AD[e] = v;
+            }
+        }
         // The row is cut into equal chunks of at most MTP_NC neighbours; within a chunk of nc
-        // neighbours thread = group h * nc + neighbour j, and the groups (as many as fit, at most
-        // MTP_NGMAX) share the basic moments, so a short chunk still keeps the workgroup busy.
+        // neighbours thread = group h * nc + neighbour j, and the groups (as many as fit, at most one
+        // per monomial row) share the rows, so a short chunk still keeps the workgroup busy.
         T fx = (T)0, fy = (T)0, fz = (T)0;
         T vir[9];
 #pragma unroll
@@ -476,31 +569,25 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
         const int csize = nchunks > 0 ? (nn + nchunks - 1) / nchunks : 1;
         for (int c0 = 0; c0 < nn; c0 += csize) {
             const int nc = min(csize, nn - c0);
-            const int ng = min(NT / nc, MTP_NGMAX);
+            const int ng = min(NT / nc, p.nrows);
             const int h = lane / nc, j = lane - h * nc;
             int nj; bool valid; T d[3] = {(T)0, (T)0, (T)0};
             __syncthreads();
             build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
             __syncthreads();
             T gs = (T)0, wx = (T)0, wy = (T)0, wz = (T)0;
+            T ux = (T)0, uy = (T)0, uz = (T)0, rinv = (T)0;
             if (h < ng) {
                 const T* t = tab + j * E;
-                const T rinv = t[OU + 3];
-#pragma unroll 4
-                for (int i = h; i < n_basic; i += ng) {
-                    const unsigned bw = bas[i];
-                    const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
-                    const T adj = A[i];
-                    const T g = t[OG + mu], dg = t[ODG + mu];
-                    const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
-                    const T m = xa * yb * zc;
-                    gs += adj * m * (dg - (T)(ea + eb + ec) * g * rinv);
-                    const T ag = adj * g;
-                    wx += ag * (T)ea * t[OX + max(ea - 1, 0)] * yb * zc;
-                    wy += ag * (T)eb * xa * t[OY + max(eb - 1, 0)] * zc;
-                    wz += ag * (T)ec * xa * yb * t[OZ + max(ec - 1, 0)];
+                ux = t[OU + 0]; uy = t[OU + 1]; uz = t[OU + 2]; rinv = t[OU + 3];
+                switch (p.nmp) {
+                case 2: pair_walk<T, 2>(t, AD, rws, p.nrows, h, ng, kmax, nmus, OX, OY, OZ, OG, ODG, rinv, gs, wx, wy, wz); break;
+                case 4: pair_walk<T, 4>(t, AD, rws, p.nrows, h, ng, kmax, nmus, OX, OY, OZ, OG, ODG, rinv, gs, wx, wy, wz); break;
+                case 6: pair_walk<T, 6>(t, AD, rws, p.nrows, h, ng, kmax, nmus, OX, OY, OZ, OG, ODG, rinv, gs, wx, wy, wz); break;
+                default: pair_walk<T, 8>(t, AD, rws, p.nrows, h, ng, kmax, nmus, OX, OY, OZ, OG, ODG, rinv, gs, wx, wy, wz); break;
                 }
             }
+            __syncthreads();            // every thread has read its table row: the group sums take its place
             // group sums in the order h = 0 .. ng-1
             {
                 T* gr = gred + lane * 4;
@@ -514,11 +601,9 @@ __global__ void __launch_bounds__(NT) mtp_atom_kernel(const MtpArgs<T> a)
                 }
             }
             if (h == 0) {
-                const T* t = tab + j * E;
-                const T rinv = t[OU + 3];
-                T gx = gs * t[OU + 0] + wx * rinv;
-                T gy = gs * t[OU + 1] + wy * rinv;
-                T gz = gs * t[OU + 2] + wz * rinv;
+                T gx = gs * ux + wx * rinv;
+                T gy = gs * uy + wy * rinv;
+                T gz = gs * uz + wz * rinv;
                 if (!valid) { gx = (T)0; gy = (T)0; gz = (T)0; }
                 if (a.seg_cursor && j < nc) {
                     // the pair claims an entry of its target's segment (zeros too: the count of a segment
@@ -913,6 +998,36 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     for (int m = nmus - 1; m >= 0; m--) mu_begin[m] = std::min(mu_begin[m], mu_begin[m + 1]);
     mu_begin[0] = 0;
 
+    // monomial rows and the dense adjoint map of the pair-derivative pass (mtp_plan.h)
+    const int nmp = (nmus + 1) / 2 * 2;
+    std::vector<int> row_base((kmax + 1) * (kmax + 1), -1), rows;
+    int nq = 0;
+    for (int a = 0; a <= kmax; a++)
+        for (int b = 0; a + b <= kmax; b++) {
+            row_base[a * (kmax + 1) + b] = nq;
+            rows.push_back(a | (b << 8) | (nq << 16));
+            nq += kmax - a - b + 1;
+        }
+    A2P_REQUIRE(nq < 32768, A2P_ERR_INVALID, "mtp plan: too many monomials");
+    std::stable_sort(rows.begin(), rows.end(), [&](int x, int y) {
+        return (x & 255) + ((x >> 8) & 255) < (y & 255) + ((y >> 8) & 255);     // longest rows first
+    });
+    std::vector<std::vector<int>> dense_lists((size_t)nq * nmp);
+    for (int i = 0; i < n_basic; i++) {
+        const int* q = basic + i * 4;
+        dense_lists[(size_t)(row_base[q[1] * (kmax + 1) + q[2]] + q[3]) * nmp + q[0]].push_back(i);
+    }
+    std::vector<int> dense_src((size_t)nq * nmp), dense_off((size_t)nq * nmp + 1, 0), dense_items, dense_pos(n_basic);
+    int dense_unique = 1;
+    for (size_t e = 0; e < dense_lists.size(); e++) {
+        dense_src[e] = dense_lists[e].empty() ? -1 : (dense_lists[e].size() == 1 ? dense_lists[e][0] : -2);
+        dense_off[e] = (int)dense_items.size();
+        if (dense_lists[e].size() > 1) dense_unique = 0;
+        for (int i : dense_lists[e]) dense_pos[i] = (int)e;
+        dense_items.insert(dense_items.end(), dense_lists[e].begin(), dense_lists[e].end());
+    }
+    dense_off[dense_lists.size()] = (int)dense_items.size();
+
     // one device block
     struct Seg { const void* src; size_t bytes; size_t off; };
     std::vector<Seg> segs;
@@ -942,6 +1057,11 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     const size_t o_rg = add(R.gbase.data(), sizeof(int) * R.gbase.size());
     const size_t o_rh = add(R.gdepth.data(), sizeof(int) * R.gdepth.size());
     const size_t o_rt = add(R.terms.data(), sizeof(int2) * R.terms.size());
+    const size_t o_rows = add(rows.data(), sizeof(int) * rows.size());
+    const size_t o_dsrc = add(dense_src.data(), sizeof(int) * dense_src.size());
+    const size_t o_doff = add(dense_off.data(), sizeof(int) * dense_off.size());
+    const size_t o_dit = add(dense_items.data(), sizeof(int) * dense_items.size());
+    const size_t o_dpos = add(dense_pos.data(), sizeof(int) * dense_pos.size());
     std::vector<unsigned char> host(total + 16, 0);
     for (auto& s : segs)
         if (s.bytes) std::memcpy(host.data() + s.off, s.src, s.bytes);
@@ -966,6 +1086,10 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.r_gbase = (const int*)(base + o_rg); d.r_gdepth = (const int*)(base + o_rh);
     d.r_terms = (const int2*)(base + o_rt);
     d.max_level_slots = std::max(F.max_slots, R.max_slots);
+    d.nq = nq; d.nmp = nmp; d.nrows = (int)rows.size();
+    d.rows = (const int*)(base + o_rows); d.dense_src = (const int*)(base + o_dsrc);
+    d.dense_off = (const int*)(base + o_doff); d.dense_items = (const int*)(base + o_dit);
+    d.dense_pos = (const int*)(base + o_dpos); d.dense_unique = dense_unique;
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         g_plans.insert(plan);
@@ -1000,6 +1124,7 @@ size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, in
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
     if (H > 0) n += (size_t)p.n_scalar + (loss ? 5 : 1) * (size_t)H;     // network inputs and per-neuron values
+    if (!loss && !mtp_dense_in_moments(p.nq, p.nmp, p.n_moms)) n += (size_t)p.nq * p.nmp;
     return n * sizeof(T) + 64;      // the packed basic-moment table (4 n_basic bytes) follows
 }
 
@@ -1040,7 +1165,8 @@ int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
     auto lds_for = [&](int nc, size_t* main) {
         *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc) + 15) / 16 * 16;
-        return *main + (size_t)a.p.n_basic * sizeof(unsigned);
+        // the packed basic-moment table; energy / force / virial kernel: + the monomial rows and the dense-array map
+        return *main + (LOSS ? (size_t)a.p.n_basic : 2 * (size_t)a.p.n_basic + a.p.nrows) * sizeof(unsigned);
     };
     size_t lds_main = 0;
     int nc_cap = MTP_NC;

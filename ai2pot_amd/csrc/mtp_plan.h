@@ -55,6 +55,18 @@ struct MtpPlanDevice {
     const int* r_gdepth;       // [n_rslots/64]
     const int2* r_terms;
     int max_level_slots;       // most slots of any level (forward or reverse)
+    // Monomial walk of the pair-derivative pass.  The monomials x^a y^b z^c, a + b + c <= kmax, are numbered
+    // q = row_base(a, b) + c; the adjoints of the basic moments are gathered into a dense array
+    // AD[q][nmp] (mu fastest, nmp = nmus rounded up to even, zero where no basic moment has that
+    // (mu, a, b, c)), so that a lane that owns one neighbour can walk a row (a, b), c = 0 .. kmax-a-b,
+    // with z^c by recurrence and the adjoints as uniform reads.
+    int nq, nmp, nrows;
+    const int* rows;           // [nrows] a | b << 8 | row_base << 16, longest rows first
+    const int* dense_pos;      // [n_basic] entry of each basic moment
+    int dense_unique;          // no two basic moments share an entry (the usual case: a plain scatter fills AD)
+    const int* dense_src;      // [nq*nmp] basic moment behind the entry, -1 none, -2 several (dense_off/items)
+    const int* dense_off;      // [nq*nmp+1]
+    const int* dense_items;    // [n_basic] basic moments ordered by dense entry
 };
 
 struct MtpPlan {
