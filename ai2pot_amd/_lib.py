@@ -6,7 +6,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
 
-A2P_OK, A2P_ERR_INVALID, A2P_ERR_HIP, A2P_ERR_OVERFLOW, A2P_ERR_INPUT, A2P_ERR_SEGMENT = 0, 1, 2, 3, 4, 5
+A2P_OK, A2P_ERR_INVALID, A2P_ERR_HIP, A2P_ERR_OVERFLOW, A2P_ERR_INPUT, A2P_ERR_SEGMENT, A2P_ERR_GRID = 0, 1, 2, 3, 4, 5, 6
 
 
 class A2PError(RuntimeError):

@@ -26,14 +26,17 @@ class NepCalculator:
 
     def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
                  sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None, path="auto",
-                 padded=True, reorder_every=64):
+                 padded=True, reorder_every=64, sync_free=False):
         """path: "gather" evaluates forces as a gather over compact lists cut by the list build (common
         model shapes, unsorted rows, umax % 8 == 0); "segments" scatters pair derivatives into reduction
         segments from the padded arrays (any model shape); "auto" takes the gather when it applies.
         padded=False (gather only) skips the padded firstneigh / rcs arrays: the step then produces
         energy, forces and virial alone.  reorder_every: the gather path processes the atoms along a
         space-filling curve; the order is a locality hint only (results do not depend on it beyond
-        rounding), so it is recomputed every reorder_every rebuilds and kept in between."""
+        rounding), so it is recomputed every reorder_every rebuilds and kept in between.
+        sync_free: after the first rebuild (which synchronises), later rebuilds size their bin grid from that build's
+        bound and never wait for the stream (a2p_nblist_sync_free); the step can then be captured into a HIP graph.
+        If the atoms spread beyond the bound, check() raises and the next rebuild synchronises again."""
         self.device = torch.device(device)
         self.dtype = dtype
         self.n = int(natoms)
@@ -96,6 +99,8 @@ class NepCalculator:
         self.path = "gather" if (can_gather and (path == "gather" or (path == "auto" and self.n >= 32768))) else "segments"
         self.padded = bool(padded) or self.path != "gather"
         self.reorder_every = max(1, int(reorder_every))
+        self.sync_free = bool(sync_free)
+        self._resync = False
         self._builds = 0
         if self.path == "gather":
             nbytes = L.a2p_nblist_compact_bytes(_c.c_int(n), _c.c_int(U), elem)
@@ -118,6 +123,14 @@ class NepCalculator:
             self.incoming = torch.empty(self.n, **i32)
 
     def rebuild(self, coords, stream):
+        before = _lib.lib().a2p_nblist_sync_free(_c.c_int(1 if (self.sync_free and not self._resync) else 0))
+        self._resync = False
+        try:
+            self._rebuild(coords, stream)
+        finally:
+            _lib.lib().a2p_nblist_sync_free(_c.c_int(before))
+
+    def _rebuild(self, coords, stream):
         # after the first build the list buffers hold a valid list: later builds write each row
         # only as far as its old or new length reaches
         if self.path == "gather":
@@ -189,4 +202,10 @@ class NepCalculator:
 
     def check(self):
         """Raise if any kernel since the last check flagged a contract violation (synchronises)."""
-        _lib.check_status(torch.cuda.current_stream(self.device).cuda_stream)
+        try:
+            _lib.check_status(torch.cuda.current_stream(self.device).cuda_stream)
+        except _lib.A2PError as ex:
+            if ex.code == _lib.A2P_ERR_GRID:
+                self._resync = True          # the next rebuild reads the extents back and renews the bound
+                self._have_list = False
+            raise

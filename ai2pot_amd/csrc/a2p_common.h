@@ -45,6 +45,7 @@ enum WsSlot {
     WS_MTP,            // MTP per-atom scratch
     WS_FLAGS,          // device-side status words
     WS_MISC,
+    WS_GRID,           // neighbor-list: the bin grid derived on the device (builds without read-back)
     WS_NSLOTS
 };
 // Returns a device pointer valid until the next ws_get on the same slot with a larger size.
@@ -59,6 +60,7 @@ enum StatusBits {
     ST_BAD_TYPE = 2,       // type index outside [0, ntypes)
     ST_NEIGH_OVERFLOW = 4, // numneigh larger than the row capacity
     ST_SEG_OVERFLOW = 8,   // more pairs name one atom than its reduction segment holds (a list that is not symmetric)
+    ST_GRID_BOUND = 16,    // neighbour list built without reading the extents back: the bin box outgrew its bound
 };
 
 inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }

@@ -11,6 +11,7 @@
 //   torch.ops.nblist.find_info4mlff_(... same ..., ilist, numneigh, firstneigh, rcs, types_out, update)
 //       writes into the caller's tensors (update = true: they hold an earlier result, rows are rewritten
 //       only as far as their old or new length reaches)
+//   torch.ops.nblist.set_sync_free(bool)   builds without a host synchronisation (a2p_nblist_sync_free)
 //   torch.ops.nblist.compact_bytes / find_info4mlff_compact_   the build that also cuts the compact
 //       lists torch.ops.nep.nepToEFVCompactOp consumes (include/ai2pot_hip.h: a2p_nblist_build_compact_*)
 // lattice is a 3x3 tensor of the dtype of coords, on the host (preferred) or on the device (copied to the
@@ -146,6 +147,9 @@ TORCH_LIBRARY(nblist, m)
         DeviceGuard guard(any_device_tensor);
         check_rc(a2p_check_status(current_stream(any_device_tensor)));
     });
+    // builds of a structure seen before size their bin grid from that build's bound and never wait for the stream
+    // (include/ai2pot_hip.h: a2p_nblist_sync_free; per host thread); returns the previous setting
+    m.def("set_sync_free", [](bool on) -> bool { return a2p_nblist_sync_free(on ? 1 : 0) != 0; });
     m.def("find_info4mlff",
           [](const at::Tensor& lattice, const at::Tensor& types, const at::Tensor& coords, double rcut, int64_t umax,
              bool is_cart, c10::List<bool> pbc_xyz, bool sort) -> std::vector<at::Tensor> {

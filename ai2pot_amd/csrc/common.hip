@@ -317,6 +317,12 @@ int a2p_check_status(void* stream_)
                        "a2p_pair_segment_capacity(a2p_pair_incoming_max(...))");
         return A2P_ERR_SEGMENT;
     }
+    if (host & a2p::ST_GRID_BOUND) {
+        a2p::set_error("neighbour list: the bin box around the atoms outgrew the bound taken from the last synchronised "
+                       "build (or the coordinates are not finite); the lists of this build are empty: build again "
+                       "after a2p_nblist_sync_free(0)");
+        return A2P_ERR_GRID;
+    }
     if (host & a2p::ST_NEIGH_OVERFLOW) {
         a2p::set_error("a neighbour count exceeds umax_num_neigh_atoms");
         return A2P_ERR_OVERFLOW;

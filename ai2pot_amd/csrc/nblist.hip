@@ -70,6 +70,30 @@ struct Grid {
     T keep_hi[3];     // (the box widened by far more than the rounding of the binning)
 };
 
+// The part of the grid that follows from the extents of the coordinates.  A build that does not read the
+// extents back to the host (a2p_nblist_sync_free) has a one-thread kernel derive it on the device; the other
+// kernels then take these fields from device memory instead of their by-value Grid argument.
+template <typename T>
+struct GridDyn {
+    T mn[3], keep_lo[3], keep_hi[3];
+    int nbin[3], rlo[3], rdim[3];
+    int nregion;
+};
+
+template <typename T>
+__device__ __forceinline__ Grid<T> with_dyn(const Grid<T>& in, const GridDyn<T>* __restrict__ gd)
+{
+    Grid<T> g = in;
+    if (gd) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            g.mn[a] = gd->mn[a]; g.keep_lo[a] = gd->keep_lo[a]; g.keep_hi[a] = gd->keep_hi[a];
+            g.nbin[a] = gd->nbin[a]; g.rlo[a] = gd->rlo[a]; g.rdim[a] = gd->rdim[a];
+        }
+    }
+    return g;
+}
+
 // image coordinate x + b0*ii + b1*jj + b2*kk, left to right (structure.h:659-676)
 template <typename T>
 __device__ __forceinline__ T image_coord(T x, T b0, T b1, T b2, int ii, int jj, int kk)
@@ -174,6 +198,52 @@ __global__ void minmax_finish_kernel(const T* __restrict__ partial, int nblocks,
     if (lane == 0) out[q] = r;
 }
 
+// ---- 1b. bin grid from the extents, on the device (builds that do not read the extents back) ----------
+// The arithmetic of find_pl_info4nblist and of the bin counts (structure.h:1013-1061, binLinkedList.h:685-688) as
+// the host does it in the synchronised build, in T with correctly rounded operations.  The box must fit the
+// bound the host sized its launches and scratch arrays for: otherwise (or if an extent is not finite) the box
+// is made empty, so that no kernel indexes beyond the bound, and ST_GRID_BOUND is raised.
+template <typename T>
+__global__ void grid_setup_kernel(const Grid<T> g, const T* __restrict__ ext, GridDyn<T>* __restrict__ gd, int cap0,
+                                  int cap1, int cap2, int* __restrict__ status)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int cap[3] = {cap0, cap1, cap2};
+    bool ok = true;
+    long long nregion = 1;
+    for (int a = 0; a < 3; a++) {
+        const T lo = ext[a], hi = ext[3 + a];
+        if (!(fabs((double)lo) < 1e300) || !(fabs((double)hi) < 1e300) || !(fabs((double)lo) < 3.0e38) ||
+            !(fabs((double)hi) < 3.0e38))
+            ok = false;
+        const T mn = sub_rn(lo, (T)kMargin);
+        const T mx = add_rn(hi, (T)kMargin);
+        const T pl = sub_rn(mx, mn);
+        const int nbin = (int)ceil(div_rn(pl, g.bin_size));
+        const int cb_lo = (int)floor(div_rn(sub_rn(ext[6 + a], mn), g.bin_size));
+        const int cb_hi = (int)floor(div_rn(sub_rn(ext[9 + a], mn), g.bin_size));
+        const int rlo = max(cb_lo - g.ext_bins, 0);
+        const int rhi = min(cb_hi + g.ext_bins, nbin - 1);
+        int rdim = rhi - rlo + 1;
+        if (rdim <= 0 || rdim > cap[a]) ok = false;
+        const double big = fmax(fabs((double)mn), fabs((double)mx));
+        const double slack = 1.0e-3 * (double)g.bin_size + 1.0e-5 * (big + (double)pl);
+        gd->mn[a] = mn;
+        gd->nbin[a] = nbin;
+        gd->rlo[a] = rlo;
+        gd->rdim[a] = rdim;
+        gd->keep_lo[a] = (T)((double)mn + (double)rlo * (double)g.bin_size - slack);
+        gd->keep_hi[a] = (T)((double)mn + (double)(rlo + rdim) * (double)g.bin_size + slack);
+        nregion *= rdim > 0 ? rdim : 0;
+    }
+    if (!ok) {
+        for (int a = 0; a < 3; a++) { gd->rdim[a] = 0; gd->keep_lo[a] = (T)1; gd->keep_hi[a] = (T)-1; }
+        nregion = 0;
+        atomicOr(status, ST_GRID_BOUND);
+    }
+    gd->nregion = (int)nregion;
+}
+
 // ---- 2 / 4. binning of (atom, image) pairs ---------------------------------------------------
 // Image (i, j, k) of an atom at xp: storage index of its bin inside the box, or -1 when outside.
 template <typename T>
@@ -199,9 +269,10 @@ __device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i,
 // One thread per atom walks its images (x outer, z inner: image m = (i * dim_y + j) * dim_z + k,
 // supercell index m * N + p, structure.h:654-681).
 template <typename T>
-__global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __restrict__ counts,
-                             int* __restrict__ incoming)
+__global__ void count_kernel(const Grid<T> g_in, const T* __restrict__ x, int* __restrict__ counts,
+                             int* __restrict__ incoming, const GridDyn<T>* __restrict__ gd)
 {
+    const Grid<T> g = with_dyn(g_in, gd);
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= g.N) return;
     if (incoming) incoming[p] = 0;                // counted up by the list kernel
@@ -216,9 +287,11 @@ __global__ void count_kernel(const Grid<T> g, const T* __restrict__ x, int* __re
 }
 
 template <typename T>
-__global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ offsets,
-                            int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x)
+__global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict__ offsets,
+                            int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x,
+                            const GridDyn<T>* __restrict__ gd)
 {
+    const Grid<T> g = with_dyn(g_in, gd);
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= g.N) return;
     const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
@@ -244,8 +317,10 @@ __global__ void fill_kernel(const Grid<T> g, const T* __restrict__ x, const int*
 // kernel then never gathers a neighbour's species).
 template <typename T>
 __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* __restrict__ s_idx,
-                               T* __restrict__ s_x, int natoms, const int* __restrict__ types)
+                               T* __restrict__ s_x, int natoms, const int* __restrict__ types,
+                               const GridDyn<T>* __restrict__ gd)
 {
+    if (gd) nbins = gd->nregion;                  // the launch covers the host's bound
     const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (b >= nbins) return;
     const int beg = offsets[b], end = offsets[b + 1];
@@ -296,9 +371,10 @@ __global__ void sorted_coords_kernel(int N, const T* __restrict__ x, const int* 
 }
 
 template <typename T>
-__global__ void order_keys_kernel(const Grid<T> g, const T* __restrict__ x, int shift, unsigned* __restrict__ keys,
-                                  int* __restrict__ vals)
+__global__ void order_keys_kernel(const Grid<T> g_in, const T* __restrict__ x, int shift, unsigned* __restrict__ keys,
+                                  int* __restrict__ vals, const GridDyn<T>* __restrict__ gd)
 {
+    const Grid<T> g = with_dyn(g_in, gd);
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= g.N) return;
     unsigned b[3];
@@ -446,14 +522,15 @@ __device__ __forceinline__ void entry_store<double>(double* p, double x, double 
 
 template <typename T, bool SORT, bool ROWBUF, bool RANK, bool COMPACT = false>
 __global__ void __launch_bounds__(NBL_BLOCK)
-lists_kernel(const Grid<T> g, const T* __restrict__ x, const int* __restrict__ types,
+lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict__ types,
              const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
              int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
              T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
              int* __restrict__ status, int update, int* __restrict__ rank_out, int* __restrict__ incoming,
-             const CompactEmit<T> ce = CompactEmit<T>{})
+             const CompactEmit<T> ce, const GridDyn<T>* __restrict__ gd)
 {
     static_assert(!COMPACT || (ROWBUF && !SORT && !RANK), "compact lists are cut from the row held in LDS");
+    const Grid<T> g = with_dyn(g_in, gd);
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
     __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
@@ -871,6 +948,20 @@ struct CompactOut {
     int keep_order;    // the buffer already holds a processing order from an earlier build: use it
 };
 
+// ---- builds that do not read the extents back (a2p_nblist_sync_free) -----------------------------------
+// The synchronised build remembers, per host thread, the bin box it found for a structure (device, natoms, lattice,
+// cutoff, periodicity).  With the switch on, a later build of the same structure sizes its launches and scratch
+// arrays for that box plus a margin, derives the actual box on the device (grid_setup_kernel) and never waits
+// for the stream; a box that outgrows the bound empties the lists and raises ST_GRID_BOUND.
+struct GridBound {
+    bool valid = false;
+    int device = -1, N = 0, is_cart = 0, pbc[3] = {0, 0, 0};
+    double lattice[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0}, rcut = 0;
+    int rdim[3] = {0, 0, 0};
+};
+thread_local GridBound g_bound;
+thread_local int g_sync_free = 0;
+
 template <typename T>
 int nblist_build(const T* lattice, const int* types, const T* coords, int N, double rcut_in, int umax,
                  int is_cart, const int* pbc, int sort, int* ilist, int* numneigh, int* firstneigh,
@@ -956,39 +1047,69 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_begin("nbl_coords_minmax", stream);
     hipLaunchKernelGGL(minmax_finish_kernel<T>, dim3(1), dim3(12 * 64), 0, stream, partial, nblocks, ext_dev);
     prof_end(stream);
-    T ext[12];
-    A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
-    A2P_HIP_CHECK(hipStreamSynchronize(stream));
-
-    // find_pl_info4nblist + bin counts (structure.h:1013-1061, binLinkedList.h:685-688)
+    // the bin box: read back from the extents, or bounded by the box of the last synchronised build of this structure
+    int device = 0;
+    A2P_HIP_CHECK(hipGetDevice(&device));
+    bool same = g_bound.valid && g_bound.device == device && g_bound.N == N && g_bound.is_cart == is_cart &&
+                g_bound.rcut == (double)g.rcut;
+    for (int a = 0; a < 3 && same; a++) same = g_bound.pbc[a] == (pbc[a] ? 1 : 0);
+    for (int q = 0; q < 9 && same; q++) same = g_bound.lattice[q] == (double)lattice[q];
+    const bool sync_free = g_sync_free && same && !max_nn_host &&
+                           (long long)N * g.nimg * (long long)(sizeof(int) + 3 * sizeof(T)) <= (2ll << 30);
+    GridDyn<T>* gd = nullptr;
     long long nregion = 1;
-    for (int a = 0; a < 3; a++) {
-        A2P_REQUIRE(std::isfinite((double)ext[a]) && std::isfinite((double)ext[3 + a]), A2P_ERR_INVALID,
-                    "nblist: non-finite coordinates");
-        const T mn = ext[a] - (T)kMargin;
-        const T mx = ext[3 + a] + (T)kMargin;
-        const T pl = mx - mn;
-        g.mn[a] = mn;
-        g.nbin[a] = (int)std::ceil(pl / g.bin_size);
-        const int cb_lo = (int)std::floor((ext[6 + a] - mn) / g.bin_size);
-        const int cb_hi = (int)std::floor((ext[9 + a] - mn) / g.bin_size);
-        g.rlo[a] = std::max(cb_lo - g.ext_bins, 0);
-        const int rhi = std::min(cb_hi + g.ext_bins, g.nbin[a] - 1);
-        g.rdim[a] = rhi - g.rlo[a] + 1;
-        A2P_REQUIRE(g.rdim[a] > 0, A2P_ERR_INVALID, "nblist: empty bin box");
-        {
-            // a coordinate c is binned as floor((c - mn) / bin_size) in T: the slack covers the
-            // rounding of that expression and of the two bounds by orders of magnitude
-            const double big = std::max(std::fabs((double)mn), std::fabs((double)mx));
-            const double slack = 1.0e-3 * (double)g.bin_size + 1.0e-5 * (big + (double)pl);
-            g.keep_lo[a] = (T)((double)mn + (double)g.rlo[a] * (double)g.bin_size - slack);
-            g.keep_hi[a] = (T)((double)mn + (double)(g.rlo[a] + g.rdim[a]) * (double)g.bin_size + slack);
+    if (sync_free) {
+        int cap[3];
+        for (int a = 0; a < 3; a++) {
+            cap[a] = g_bound.rdim[a] + std::max(2, g_bound.rdim[a] / 8);
+            g.rdim[a] = cap[a];                         // host copies of the box serve launch and scratch sizes only
+            nregion *= cap[a];
         }
-        nregion *= g.rdim[a];
+        A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID, "nblist: %lld bins around the centre atoms", nregion);
+        void* wsG = nullptr;
+        rc = ws_get(WS_GRID, 256, &wsG);
+        if (rc) return rc;
+        gd = (GridDyn<T>*)wsG;
+        hipLaunchKernelGGL(grid_setup_kernel<T>, dim3(1), dim3(64), 0, stream, g, (const T*)ext_dev, gd, cap[0], cap[1],
+                           cap[2], status);
+    } else {
+        T ext[12];
+        A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
+        A2P_HIP_CHECK(hipStreamSynchronize(stream));
+
+        // find_pl_info4nblist + bin counts (structure.h:1013-1061, binLinkedList.h:685-688)
+        for (int a = 0; a < 3; a++) {
+            A2P_REQUIRE(std::isfinite((double)ext[a]) && std::isfinite((double)ext[3 + a]), A2P_ERR_INVALID,
+                        "nblist: non-finite coordinates");
+            const T mn = ext[a] - (T)kMargin;
+            const T mx = ext[3 + a] + (T)kMargin;
+            const T pl = mx - mn;
+            g.mn[a] = mn;
+            g.nbin[a] = (int)std::ceil(pl / g.bin_size);
+            const int cb_lo = (int)std::floor((ext[6 + a] - mn) / g.bin_size);
+            const int cb_hi = (int)std::floor((ext[9 + a] - mn) / g.bin_size);
+            g.rlo[a] = std::max(cb_lo - g.ext_bins, 0);
+            const int rhi = std::min(cb_hi + g.ext_bins, g.nbin[a] - 1);
+            g.rdim[a] = rhi - g.rlo[a] + 1;
+            A2P_REQUIRE(g.rdim[a] > 0, A2P_ERR_INVALID, "nblist: empty bin box");
+            {
+                // a coordinate c is binned as floor((c - mn) / bin_size) in T: the slack covers the
+                // rounding of that expression and of the two bounds by orders of magnitude
+                const double big = std::max(std::fabs((double)mn), std::fabs((double)mx));
+                const double slack = 1.0e-3 * (double)g.bin_size + 1.0e-5 * (big + (double)pl);
+                g.keep_lo[a] = (T)((double)mn + (double)g.rlo[a] * (double)g.bin_size - slack);
+                g.keep_hi[a] = (T)((double)mn + (double)(g.rlo[a] + g.rdim[a]) * (double)g.bin_size + slack);
+            }
+            nregion *= g.rdim[a];
+        }
+        A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID,
+                    "nblist: %lld bins around the centre atoms; are the coordinates far outside the cell?",
+                    nregion);
+        g_bound.valid = true;
+        g_bound.device = device; g_bound.N = N; g_bound.is_cart = is_cart; g_bound.rcut = (double)g.rcut;
+        for (int a = 0; a < 3; a++) { g_bound.pbc[a] = pbc[a] ? 1 : 0; g_bound.rdim[a] = g.rdim[a]; }
+        for (int q = 0; q < 9; q++) g_bound.lattice[q] = (double)lattice[q];
     }
-    A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID,
-                "nblist: %lld bins around the centre atoms; are the coordinates far outside the cell?",
-                nregion);
     const int nb1 = (int)nregion + 1;
 
     // workspace B: counts[nb1] | offsets[nb1] | cursor[nb1] | scan tmp, then (after the count is
@@ -1006,7 +1127,8 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (rc) return rc;
     const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
     prof_begin("nbl_count", stream);
-    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming);
+    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming,
+                       (const GridDyn<T>*)gd);
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
@@ -1043,12 +1165,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_begin("nbl_fill", stream);
 
     hipLaunchKernelGGL(fill_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
-                       s_idx, s_x);
+                       s_idx, s_x, (const GridDyn<T>*)gd);
 
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
-                       (int)nregion, offsets, s_idx, s_x, g.N, co ? types : (const int*)nullptr);
+                       (int)nregion, offsets, s_idx, s_x, g.N, co ? types : (const int*)nullptr, (const GridDyn<T>*)gd);
     prof_end(stream);
     CompactEmit<T> ce{};
     if (co) {
@@ -1072,7 +1194,8 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         int* vals_in = (int*)((char*)wsD + 2 * key_bytes);
         void* tmp_sort = (char*)wsD + 3 * key_bytes;
         prof_begin("nbl_order", stream);
-        hipLaunchKernelGGL(order_keys_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, shift, keys_in, vals_in);
+        hipLaunchKernelGGL(order_keys_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, shift, keys_in, vals_in,
+                           (const GridDyn<T>*)gd);
         prof_end(stream);
         prof_begin("nbl_order", stream);
         A2P_HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(tmp_sort, tmp_bytes, (const unsigned*)keys_in, keys_out,
@@ -1101,27 +1224,27 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (co)
         hipLaunchKernelGGL((lists_kernel<T, false, true, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds,
                            stream, g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out,
-                           keys, status, update, nullptr, nullptr, ce);
+                           keys, status, update, nullptr, nullptr, ce, (const GridDyn<T>*)gd);
     else if (sort)
         hipLaunchKernelGGL((lists_kernel<T, true, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
-                           status, 0, nullptr, nullptr);
+                           status, 0, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rowbuf && rank)
         hipLaunchKernelGGL((lists_kernel<T, false, true, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
                            g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update, rank, incoming);
+                           status, update, rank, incoming, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rowbuf)
         hipLaunchKernelGGL((lists_kernel<T, false, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
                            g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update, nullptr, nullptr);
+                           status, update, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rank)
         hipLaunchKernelGGL((lists_kernel<T, false, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update, rank, incoming);
+                           status, update, rank, incoming, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else
         hipLaunchKernelGGL((lists_kernel<T, false, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
                            types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
-                           status, update, nullptr, nullptr);
+                           status, update, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     prof_end(stream);
     if (sort) {
         prof_begin("nbl_sort_rows", stream);
@@ -1161,6 +1284,13 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
 }  // namespace a2p
 
 extern "C" {
+
+int a2p_nblist_sync_free(int on)
+{
+    const int before = a2p::g_sync_free;
+    a2p::g_sync_free = on ? 1 : 0;
+    return before;
+}
 
 int a2p_nblist_build_f32(const float* lattice, const int* types, const float* coords, int natoms,
                          double rcut, int umax, int is_cart, const int* pbc, int sort, int* ilist,

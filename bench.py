@@ -229,7 +229,8 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     lattice, pos, types, disp = nep_structure(kind, size)
     n = pos.shape[0]
     model = synth.nep_model(seed=3006)
-    calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev)
+    # rebuilds after the first size their bin grid from the first one's bound: no host synchronisation in the step
+    calc = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, sync_free=rebuild)
     ops_path = OpsStepper(model, n, lattice, types, dev) if (via_ops or (rebuild and calc.path == "gather" and not args.no_other_configs)) else None
     coords0 = torch.from_numpy(pos.astype(np.float32)).to(dev)
     disp_t = torch.from_numpy(disp.astype(np.float32)).to(dev)
@@ -247,11 +248,14 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     if via_ops:
         torch.ops.nblist.set_validate(False)
         torch.ops.nep.set_validate(False)
+        ops_path.step(coords0)                       # a synchronised build first: it sets the bound
+        torch.ops.nblist.set_sync_free(True)
     elapsed, kernels = timed(step, args.steps, args.warmup, L, keep=3)
     if via_ops:
         last = step(args.warmup + args.steps - 1)
         ref = calc.step(coords)
         torch.ops.nblist.check_status(coords)
+        torch.ops.nblist.set_sync_free(False)
         torch.ops.nblist.set_validate(True)
         torch.ops.nep.set_validate(True)
         # same kernels; the processing orders of the two drivers may differ, hence rounding-level bars
@@ -259,12 +263,32 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
                 and torch.allclose(last[2][0], ref[2], rtol=1e-4, atol=1e-2)):
             sys.exit("bench.py: the operator path and the calculator disagree")
     if args.graph:
-        if rebuild:
-            sys.exit("bench.py: --graph needs a workload without list rebuild (the build synchronises with the host)")
+        # the whole step (coordinate update, sync-free rebuild, E/F/V) as one HIP graph
         graph = torch.cuda.CUDAGraph()
+        alpha = torch.zeros((), dtype=torch.float32, device=dev)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                # one call on a capture-capable stream first
+            if rebuild:
+                calc.step(coords)
+            else:
+                calc.evaluate(ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
         with torch.cuda.graph(graph):
-            calc.evaluate(ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
-        elapsed = timed_replay(graph.replay, args.steps, args.warmup)
+            if rebuild:
+                torch.addcmul(coords0, disp_t, alpha, out=coords)
+                calc.step(coords)
+            else:
+                calc.evaluate(ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        state = {"k": 0}
+
+        def replay():
+            if rebuild:
+                alpha.fill_(float(np.sin(0.37 * state["k"])))
+                state["k"] += 1
+            graph.replay()
+        elapsed = timed_replay(replay, args.steps, args.warmup)
     calc.check()
     if not np.isfinite(float(calc.etot.item())):
         sys.exit("bench.py: non-finite energy")
@@ -299,7 +323,8 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     extra = {"rooflines": entries}
     if rebuild and calc.path == "gather" and not args.graph and not args.no_other_configs:
         # the same step without the padded firstneigh / rcs arrays (energy, forces and virial only)
-        lean = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, padded=False)
+        lean = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, padded=False,
+                             sync_free=True)
         lean.rebuild(coords0, stream)
 
         def lean_step(k):
@@ -320,6 +345,8 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
             # the same step (padded arrays included) driven through the registered operators alone
             torch.ops.nblist.set_validate(False)
             torch.ops.nep.set_validate(False)
+            ops_path.step(coords0)                   # a synchronised build first: it sets the bound
+            torch.ops.nblist.set_sync_free(True)
 
             def ops_step(k):
                 torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
@@ -333,6 +360,7 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
             torch.ops.nblist.check_status(coords)
+            torch.ops.nblist.set_sync_free(False)
             torch.ops.nblist.set_validate(True)
             torch.ops.nep.set_validate(True)
             extra["through_torch_ops"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
@@ -566,6 +594,7 @@ WORKLOADS = {
     "nep_md_1048576_ops": lambda a: run_nep_md(a, "fcc", 64, via_ops=True),   # the headline step through torch.ops only
     "nep_md_131072": lambda a: run_nep_md(a, "fcc", 32),
     "nep_efv_4096": lambda a: run_nep_md(a, "random", 4096, rebuild=False),   # configs[1]
+    "nep_md_4096": lambda a: run_nep_md(a, "random", 4096),      # configs[1] as a molecular-dynamics step: with list rebuild
     "mtp10_efv_216": lambda a: run_mtp(a, 1),                     # configs[0]
     "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
     "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]

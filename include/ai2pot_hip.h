@@ -25,6 +25,7 @@ extern "C" {
 #define A2P_ERR_OVERFLOW 3  /* a neighbour count exceeds the row capacity umax               */
 #define A2P_ERR_INPUT 4     /* device-side input check failed (bad neighbour / type index)   */
 #define A2P_ERR_SEGMENT 5   /* an atom is named by more pairs than its reduction segment holds */
+#define A2P_ERR_GRID 6      /* sync-free neighbour-list build: the bin box outgrew the bound of the last synchronised build */
 
 const char* a2p_last_error(void);
 
@@ -47,7 +48,7 @@ unsigned long long a2p_workspace_generation(void);
 /* Reads and clears the device status word that kernels set when an input violates the
  * contract (neighbour index outside [0, natoms_pad+nghost), type index outside
  * [0, ntypes), numneigh > umax, more pairs naming one atom than its reduction segment holds).
- * Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT, A2P_ERR_OVERFLOW or A2P_ERR_SEGMENT.  The reference has no such check: it asserts or overflows
+ * Synchronises `stream`.  Returns A2P_OK, A2P_ERR_INPUT, A2P_ERR_OVERFLOW, A2P_ERR_SEGMENT or A2P_ERR_GRID.  The reference has no such check: it asserts or overflows
  * (source/nblist/include/neighborList.h:550, commented-out assert). */
 int a2p_check_status(void* stream);
 
@@ -234,6 +235,20 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * and virial[9] may be NULL.
  * ------------------------------------------------------------------------------------------ */
 size_t a2p_nblist_compact_bytes(int natoms, int umax, int elem_size);   /* 0: not available for these sizes */
+
+/* Neighbour-list builds without a host synchronisation (no counterpart in the reference, whose list build runs on
+ * the host).  Every a2p_nblist_* build reads twelve coordinate extents back to size its bin grid, which makes the
+ * host wait for the stream once per build and keeps the build out of HIP graphs.  a2p_nblist_sync_free(1) switches
+ * that off for the calling host thread (returns the previous setting): a build of a structure this thread has built
+ * before with the switch off or on (same device, natoms, lattice, cutoff, periodicity, coordinate kind) then sizes
+ * its launches and scratch arrays for the bin box of that synchronised build plus a margin (an eighth, at least two
+ * bins, per axis), derives the actual grid on the device and returns without waiting; results are bit-identical.  If
+ * the atoms have spread beyond that bound (or a coordinate is not finite) the build leaves every list empty and
+ * raises a status bit: a2p_check_status returns A2P_ERR_GRID, and the caller builds again with the switch off, which
+ * also renews the bound.  Builds that ask for max_numneigh, or whose image arrays would exceed 2 GiB, synchronise as
+ * before.  After one eager call in this mode the build can be captured into a HIP graph together with the operators
+ * that consume the list. */
+int a2p_nblist_sync_free(int on);
 
 /* 1 when a2p_nep_efv_compact_* covers the model (shape as above, tables fit in LDS), else 0 */
 int a2p_nep_efv_compact_supported(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,

@@ -89,3 +89,99 @@ def test_graph_survives_a_workspace_change(oracle):
     assert g.valid() and g.recaptures == 1
     for a, b, c in zip(first, again, want):
         assert torch.equal(a, c) and torch.equal(b, c)
+
+
+def _md_inputs(n_reps, seed):
+    lat, pos = synth.fcc_cell(n_reps, 4.6, 0.12, seed)
+    ty = synth.rng_randint(seed + 1, pos.shape[0], 3)
+    disp = synth.rng_normal(seed + 2, pos.size, 0.0, 0.02).reshape(-1, 3)
+    return lat, pos, ty, disp
+
+
+@pytest.mark.parametrize("path", ["segments", "gather"])
+def test_step_with_rebuild_without_host_synchronisation(oracle, path):
+    """Neighbour rebuild + NEP E/F/V with a2p_nblist_sync_free: the bin grid is derived on the device from the
+    bound of the first (synchronised) build.  Lists and results are bitwise those of the synchronised build, and
+    the whole step replays as a HIP graph on new coordinates."""
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos, ty, disp = _md_inputs(6, 71)                       # 864 atoms
+    n = pos.shape[0]
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    dev = "cuda:0"
+    kw = dict(umax=96, dtype=torch.float32, device=dev, path=path)
+    free = NepCalculator(m, n, lat, ty, sync_free=True, **kw)
+    sync = NepCalculator(m, n, lat, ty, **kw)
+    base = torch.from_numpy(pos.astype(np.float32)).to(dev)
+    d = torch.from_numpy(disp.astype(np.float32)).to(dev)
+    coords = base.clone()                                         # the static input of the graph
+    for it, alpha in enumerate((0.0, 1.0, -0.7)):
+        coords.copy_(base + alpha * d)
+        got = [t.clone() for t in free.step(coords)]
+        free.check()
+        want = [t.clone() for t in sync.step(coords)]
+        sync.check()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), "step %d" % it
+        for a, b in ((free.numneigh, sync.numneigh), (free.firstneigh, sync.firstneigh), (free.rcs, sync.rcs)):
+            nn = sync.numneigh.cpu().numpy()
+            fa, fb = a.cpu().numpy(), b.cpu().numpy()
+            if fa.ndim == 1:
+                assert np.array_equal(fa, fb)
+            else:
+                for i in range(0, n, 37):
+                    assert np.array_equal(fa[i, :nn[i]].view(np.uint8), fb[i, :nn[i]].view(np.uint8))
+    # the step as a graph: rebuild and evaluation in one capture, replayed on rewritten coordinates
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        free.step(coords)                                          # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        free.step(coords)
+    for it, alpha in enumerate((0.4, -1.1, 0.9, 0.0)):
+        coords.copy_(base + alpha * d)
+        want = [t.clone() for t in sync.step(coords)]              # eager work between the replays
+        sync.check()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip((free.etot, free.force, free.virial), want):
+            assert torch.equal(a, b), "replay %d" % it
+    free.check()
+
+
+def test_sync_free_build_flags_a_box_that_outgrew_its_bound(oracle):
+    """Atoms that spread far beyond the bin box of the last synchronised build: the sync-free build leaves the
+    lists empty and flags it (no kernel indexes beyond the bound), check() says so, and the next rebuild
+    synchronises again and is right."""
+    import torch
+    from ai2pot_amd import _lib
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos, ty, _ = _md_inputs(5, 81)
+    n = pos.shape[0]
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    dev = "cuda:0"
+    calc = NepCalculator(m, n, lat, ty, umax=96, dtype=torch.float32, device=dev, path="segments", sync_free=True)
+    ref = NepCalculator(m, n, lat, ty, umax=96, dtype=torch.float32, device=dev, path="segments")
+    base = torch.from_numpy(pos.astype(np.float32)).to(dev)
+    calc.step(base)
+    calc.check()
+    far = base.clone()
+    far[::2] += torch.tensor([4.0 * float(lat[0][0]), 0.0, 0.0], device=dev)   # half of the atoms four cells away
+    calc.step(far)
+    with pytest.raises(_lib.A2PError) as err:
+        calc.check()
+    assert err.value.code == _lib.A2P_ERR_GRID
+    got = [t.clone() for t in calc.step(far)]                     # synchronised again, bound renewed
+    calc.check()
+    want = [t.clone() for t in ref.step(far)]
+    ref.check()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    got = [t.clone() for t in calc.step(far)]                     # and sync-free from here on
+    calc.check()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
