@@ -13,8 +13,9 @@
 //     A_lm = sum_n dE_i/dS_{n,lm} g_n^{ij}(r) + (-1)^l sum_n dE_j/dS_{n,lm} g_n^{ji}(r).
 // No per-pair store, no atomics, no reduction pass: two kernels over the atoms.
 //   nep_adjoint_kernel : radial sums and angular moments over the compact lists, descriptors,
-//                        hidden layer, dE/dq, dE/dS; stores a 128-value record per atom
-//                        (96 dE/dS + 4 x 8 contracted radial coefficients) and the energy partials
+//                        hidden layer, dE/dq, dE/dS; stores per atom a 96-value record (dE/dS) and, in a
+//                        dense array of their own, the radial coefficients contracted with dE/dq
+//                        (species x 8 values), and the energy partials
 //   nep_gather_kernel  : walks the lists again, gathers the neighbours' records, forms
 //                        g_ij - g_ji, sums force and virial
 // One thread per atom, 256 per workgroup.  Atoms are processed in the Morton order of the list
