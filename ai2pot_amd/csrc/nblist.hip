@@ -270,12 +270,16 @@ __device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i,
 // supercell index m * N + p, structure.h:654-681).
 template <typename T>
 __global__ void count_kernel(const Grid<T> g_in, const T* __restrict__ x, int* __restrict__ counts,
-                             int* __restrict__ incoming, const GridDyn<T>* __restrict__ gd)
+                             int* __restrict__ incoming, const GridDyn<T>* __restrict__ gd,
+                             const int* __restrict__ types, int* __restrict__ ilist, int* __restrict__ types_out)
 {
     const Grid<T> g = with_dyn(g_in, gd);
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= g.N) return;
     if (incoming) incoming[p] = 0;                // counted up by the list kernel
+    // neighborList.h:548-553: the two outputs that do not depend on the list are written here, in atom order (the
+    // list kernel may process the atoms in another order and would scatter them)
+    if (ilist) { ilist[p] = p; types_out[p] = types[p]; }
     const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
     for (int i = 0; i < g.img_dim[0]; i++)
         for (int j = 0; j < g.img_dim[1]; j++)
@@ -664,11 +668,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         }
     }
     if (lane == 0) {
-        if (rows) {
-            ilist[p] = p;
-            numneigh[p] = cnt;
-            types_out[p] = types[p];
-        }
+        if (rows) numneigh[p] = cnt;             // ilist and types_out: count_kernel
         if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
     }
     if (COMPACT) {
@@ -1128,7 +1128,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
     prof_begin("nbl_count", stream);
     hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming,
-                       (const GridDyn<T>*)gd);
+                       (const GridDyn<T>*)gd, types, want_rows ? ilist : (int*)nullptr, types_out);
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
