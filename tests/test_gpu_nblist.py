@@ -221,3 +221,52 @@ def test_build_with_places(oracle, dt, umax):
         np.add.at(seen, (fi[live], rk[live]), 1)
         assert np.array_equal(seen.sum(1), inc) and seen.max() == 1
 
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("sort", [False, True])
+@pytest.mark.parametrize("pbc", [(True, True, True), (True, False, True)])
+def test_builds_without_host_synchronisation(oracle, dt, sort, pbc):
+    """a2p_nblist_sync_free: after one synchronised build of a structure, later builds derive the bin grid on the
+    device.  Triclinic cell, fractional coordinates, atoms drifting (also out of the cell): every build is
+    bitwise the oracle's, through the C ABI (NumPy front end) and through torch.ops.nblist on device tensors."""
+    import os
+    import torch
+    from ai2pot_amd import _lib
+    L = np.array([[9.0, 0.3, -0.2], [1.1, 8.2, 0.4], [-0.7, 0.9, 10.1]])
+    fr = synth.rng_uniform(27, 3 * 80).reshape(80, 3)
+    ty = synth.rng_randint(28, 80, 3)
+    drift = synth.rng_normal(29, 3 * 80, 0.0, 0.01).reshape(80, 3)
+    lib = _lib.lib()
+    a = gpu_list(L.astype(dt), ty, fr.astype(dt), 5.5, 250, is_cart=False, pbc=pbc, sort=sort)   # sets the bound
+    assert_same(a, oracle.nblist(L.astype(dt), ty, fr.astype(dt), 5.5, 250, is_cart=False, pbc=pbc, sort=sort))
+    from ai2pot_amd import nblist
+    tt0 = torch.from_numpy(ty.astype(np.int32)).to("cuda:0")
+    before = lib.a2p_nblist_sync_free(1)
+    try:
+        for step in range(1, 4):
+            f = (fr + step * drift).astype(dt)
+            # check=False: a build that asks for the largest neighbour count synchronises anyway
+            out = nblist.find_info4mlff_device(L.astype(dt), tt0, torch.from_numpy(f).to("cuda:0"), 5.5, 250, False,
+                                               pbc, sort, check=False)
+            _lib.check_status(torch.cuda.current_stream().cuda_stream)
+            got = tuple(o.cpu().numpy() if hasattr(o, "cpu") else o for o in out)
+            assert_same(got, oracle.nblist(L.astype(dt), ty, f, 5.5, 250, is_cart=False, pbc=pbc, sort=sort))
+    finally:
+        lib.a2p_nblist_sync_free(before)
+    # the same through the registered operator
+    libdir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ai2pot_amd", "_lib")
+    torch.ops.load_library(os.path.join(libdir, "libnblist_bind.so"))
+    tl = torch.from_numpy(L.astype(dt))
+    tt = torch.from_numpy(ty.astype(np.int32)).to("cuda:0")
+    args = (5.5, 250, False, [bool(x) for x in pbc], sort)
+    torch.ops.nblist.find_info4mlff(tl, tt, torch.from_numpy(fr.astype(dt)).to("cuda:0"), *args)
+    was = torch.ops.nblist.set_sync_free(True)
+    try:
+        f = (fr + 2.5 * drift).astype(dt)
+        out = torch.ops.nblist.find_info4mlff(tl, tt, torch.from_numpy(f).to("cuda:0"), *args)
+        want = oracle.nblist(L.astype(dt), ty, f, 5.5, 250, is_cart=False, pbc=pbc, sort=sort)
+        for x, y in zip(out[1:6], want[1:6]):
+            assert np.array_equal(x.cpu().numpy().view(np.uint8), y.view(np.uint8))
+    finally:
+        torch.ops.nblist.set_sync_free(was)
