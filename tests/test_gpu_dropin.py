@@ -448,3 +448,54 @@ def test_asymmetric_list_names_an_atom_more_often_than_a_row_is_long(oracle, dro
     for fn in (ops.linearMtpToEFVOp, torch.ops.mtpr.linearMtpToEFVOp):
         out = [t.cpu().numpy() for t in fn(*margs)]
         check(out, mref, np.float64)
+
+
+def test_bind_libraries_against_the_oracle_at_working_sizes(oracle, dropin):
+    """The registered operators compared with the oracle directly (not through the Python mirror) at sizes where
+    every kernel variant behind them is in play: NEP fp32 at 2,000 atoms (the 8-lanes-per-atom kernel), linear MTP
+    fp64 at level 20 with 4 species (256 threads per atom, monomial walk)."""
+    import torch
+    from test_gpu_nep import _model_to_device
+    from test_gpu_nep_gather import _check
+    from test_gpu_mtp import model_to_device
+    dev = "cuda:0"
+    # NEP through torch.ops.nblist + torch.ops.nep on device tensors
+    n = 2000
+    Lc = (n / 0.033) ** (1.0 / 3.0)
+    lat, pos = synth.random_packed(n, [Lc, Lc, Lc], 2.2, 411)
+    ty = synth.rng_randint(412, n, 3)
+    m = synth.nep_model(seed=413)
+    md = _model_to_device(m, torch.float32)
+    out = torch.ops.nblist.find_info4mlff(torch.from_numpy(lat.astype(np.float32)),
+                                          torch.from_numpy(ty.astype(np.int32)).to(dev),
+                                          torch.from_numpy(pos.astype(np.float32)).to(dev), 7.0, 200, True,
+                                          [True, True, True], False)
+    ref_list = oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 7.0, 200)
+    for a, b in zip(out[1:6], ref_list[1:6]):
+        assert np.array_equal(a.cpu().numpy().view(np.uint8), b.view(np.uint8))
+    z = torch.zeros(36, dtype=torch.float32, device=dev)
+    got = torch.ops.nep.nepToEFVOp(8, 6, 4, 4, md["coeffs"], md["w0"], md["b0"], md["w1"], md["type_bias"],
+                                   out[0], out[1].unsqueeze(0), out[2].unsqueeze(0), out[3].unsqueeze(0),
+                                   out[4].unsqueeze(0), out[5].unsqueeze(0), md["type_map"], 0, 7.0, 4.0,
+                                   md["q_scaler"], 0.0, 0.0, z, z)
+    ref = oracle.nep_efv(m, synth.pack_batch([ref_list]), np.float32)
+    _check(tuple(t.cpu().numpy() for t in got), ref, np.float32)
+    # linear MTP, level 20
+    n = 300
+    lat, pos = synth.random_packed(n, [20.0, 18.0, 16.7], 2.0, 421)
+    ty = synth.rng_randint(422, n, 4)
+    nbl = oracle.nblist(lat, ty, pos, 5.5, 200)
+    nb = synth.pack_batch([nbl])
+    tables = mtp_param.mtp_param(20)
+    mm = synth.mtp_model(tables, 4, 10, 5.5, 1.8, 423, lo=-0.05, hi=0.05)
+    mmd = model_to_device(mm, torch.float64)
+    dv = to_device(nb, torch.float64)
+    z = torch.zeros(64, dtype=torch.float64, device=dev)
+    got = torch.ops.mtpr.linearMtpToEFVOp(10, 1.0, mmd["coeffs"], mmd["linear_coeffs"], mmd["type_bias"],
+                                          int(mm["alpha_moments_count"]), mmd["alpha_index_basic"],
+                                          mmd["alpha_index_times"], mmd["alpha_moment_mapping"], int(mm["nmus"]),
+                                          dv["binum"], dv["bilist"], dv["bnumneigh"], dv["bfirstneigh"], dv["brcs"],
+                                          dv["btypes"], mmd["type_map"], 0, 5.5, 1.8, mmd["q_scaler"], 0.0, 0.0, z, z)
+    ref = oracle.mtp_efv(mm, nb)
+    for a, b in zip(got, ref):
+        assert np.abs(a.cpu().numpy() - b).max() <= 1e-10 * np.abs(b).max()
