@@ -135,11 +135,14 @@ class NepCalculator:
         # only as far as its old or new length reaches
         if self.path == "gather":
             m = self.m
+            # the processing order is never recomputed inside a graph capture (a library sort would be recorded)
+            capturing = torch.cuda.is_current_stream_capturing()
             rc = self._nbl_compact(self.lattice.ctypes.data_as(_c.c_void_p), _vp(self.types), _vp(coords),
                                    _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
                                    self.pbc.ctypes.data_as(_c.c_void_p),
                                    _c.c_int((1 if (self._have_list and self.padded) else 0) |
-                                            (2 if (self._have_list and self._builds % self.reorder_every) else 0)),
+                                            (2 if (self._have_list and (self._builds % self.reorder_every or capturing))
+                                             else 0)),
                                    _c.c_double(m["rmax_radial"]), _c.c_double(m["rmax_angular"]),
                                    _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),
                                    _vp(self.types_out), _vp(self.compact), stream)
