@@ -213,12 +213,11 @@ __global__ void grid_setup_kernel(const Grid<T> g, const T* __restrict__ ext, Gr
     long long nregion = 1;
     for (int a = 0; a < 3; a++) {
         const T lo = ext[a], hi = ext[3 + a];
-        if (!(fabs((double)lo) < 1e300) || !(fabs((double)hi) < 1e300) || !(fabs((double)lo) < 3.0e38) ||
-            !(fabs((double)hi) < 3.0e38))
-            ok = false;
+        if (!(fabs((double)lo) < 1.0e30) || !(fabs((double)hi) < 1.0e30)) ok = false;    // NaN, infinity or absurd
         const T mn = sub_rn(lo, (T)kMargin);
         const T mx = add_rn(hi, (T)kMargin);
         const T pl = sub_rn(mx, mn);
+        if (!((double)pl / (double)g.bin_size < 1.0e9)) ok = false;       // the bin counts below must fit an int
         const int nbin = (int)ceil(div_rn(pl, g.bin_size));
         const int cb_lo = (int)floor(div_rn(sub_rn(ext[6 + a], mn), g.bin_size));
         const int cb_hi = (int)floor(div_rn(sub_rn(ext[9 + a], mn), g.bin_size));
