@@ -116,8 +116,34 @@ bool prof_event(hipEvent_t* e)
 }
 }  // namespace
 
+// The workspace is shared by every call on a device, so work of this library on two streams must not overlap.
+// Every launch passes through prof_begin: when the stream differs from the one the previous launch on this device
+// used, the device is synchronised first (callers that keep to one stream never pay for it).  A stream that is being
+// captured is left alone: a capture keeps to itself, and its replays are ordered by whoever launches them.
+namespace {
+std::mutex g_stream_mutex;
+std::vector<hipStream_t> g_last_stream;
+std::vector<char> g_have_stream;
+
+void order_streams(hipStream_t stream)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_stream_mutex);
+    if ((int)g_last_stream.size() <= dev) { g_last_stream.resize(dev + 1, nullptr); g_have_stream.resize(dev + 1, 0); }
+    if (g_have_stream[dev] && g_last_stream[dev] == stream) return;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) { (void)hipGetLastError(); return; }
+    if (st != hipStreamCaptureStatusNone) return;
+    if (g_have_stream[dev]) (void)hipDeviceSynchronize();
+    g_last_stream[dev] = stream;
+    g_have_stream[dev] = 1;
+}
+}  // namespace
+
 void prof_begin(const char* label, hipStream_t stream)
 {
+    order_streams(stream);
     if (!g_prof_on) return;
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (!g_prof_select.empty() && g_prof_select.find("," + std::string(label) + ",") == std::string::npos) return;

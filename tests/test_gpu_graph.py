@@ -185,3 +185,35 @@ def test_sync_free_build_flags_a_box_that_outgrew_its_bound(oracle):
     calc.check()
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def test_calls_on_two_streams_do_not_overlap(oracle):
+    """The library's workspace is shared by all calls on a device: when the stream changes between calls the library
+    synchronises the device first, so two streams used in turn give the results of the same calls made one after the
+    other on one stream."""
+    import torch
+    from ai2pot_amd import ops
+    from test_gpu_nep import _model_to_device
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0)
+    md = _model_to_device(m, torch.float32)
+    cases = []
+    for reps, seed in ((6, 91), (5, 93)):
+        lat, pos = synth.fcc_cell(reps, 4.6, 0.15, seed)
+        ty = synth.rng_randint(seed + 1, pos.shape[0], 3)
+        nb = synth.pack_batch([oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 6.0, 100)])
+        d = to_device(nb, torch.float32)
+        cases.append((m["chebyshev_size"], m["n_radial_basis"], m["n_angular_basis"], m["l_max"], md["coeffs"], md["w0"],
+                      md["b0"], md["w1"], md["type_bias"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"],
+                      d["brcs"], d["btypes"], md["type_map"], 0, m["rmax_radial"], m["rmax_angular"], md["q_scaler"]))
+    want = [[t.clone() for t in ops.nepToEFVOp(*a, validate=False)] for a in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for it in range(4):
+        got = []
+        for a, s in zip(cases, streams):
+            with torch.cuda.stream(s):
+                got.append(ops.nepToEFVOp(*a, validate=False))      # no synchronisation by the caller in between
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            for x, y in zip(g, w):
+                assert torch.equal(x, y), "round %d" % it
