@@ -34,9 +34,11 @@ int a2p_abi_version(void);
 
 /* The per-device workspace (no counterpart in the reference, whose operators allocate their
  * scratch per call, e.g. source/descriptor/nep/include/nep.h:391-392).  It grows to what the
- * largest call so far needed and is then reused, so calls on ONE device must not overlap in
- * time: issue them on one stream, or order the streams with events.  Different devices are
- * independent.  a2p_workspace_bytes returns what the library holds on the current device;
+ * largest call so far needed and is then reused, so the library's work on ONE device must not
+ * overlap in time.  Calls on one stream never do; when a call arrives on another stream than the
+ * library's previous launch on that device, the library synchronises the device first (a stream
+ * under graph capture is left alone; calls from several host threads at once are not supported).
+ * Different devices are independent.  a2p_workspace_bytes returns what the library holds on the current device;
  * a2p_workspace_release synchronises the device and frees it (the next call allocates again). */
 size_t a2p_workspace_bytes(void);
 int a2p_workspace_release(void);
