@@ -203,3 +203,32 @@ def test_gather_errors(oracle):
     ok.step(torch.from_numpy(pos.astype(np.float32)).to("cuda:0"))
     with pytest.raises(_lib.A2PError):
         ok.check()
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64])
+def test_trajectory_across_reorders_without_host_synchronisation(oracle, np_dtype):
+    """Seven steps of drifting atoms in a slab (one axis not periodic): the processing order is refreshed every third
+    rebuild and kept in between, the rebuilds after the first do not synchronise with the host.  Every step's padded
+    rows are the oracle's bit for bit and E/F/V stay within the bars."""
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos = synth.fcc_cell(7, 4.7, 0.12, 371)
+    n = pos.shape[0]
+    ty = synth.rng_randint(372, n, 3)
+    m = synth.nep_model(rmax_radial=6.0, rmax_angular=4.0, seed=3307)
+    disp = synth.rng_normal(373, pos.size, 0.0, 0.05).reshape(-1, 3)
+    dtype = torch.float32 if np_dtype == np.float32 else torch.float64
+    calc = NepCalculator(m, n, lat, ty, umax=96, dtype=dtype, device="cuda:0", path="gather", pbc=(True, True, False),
+                         reorder_every=3, sync_free=True)
+    for k in range(7):
+        p = pos + k * disp
+        got = _step(calc, p, np_dtype)
+        ref = oracle.nblist(lat.astype(np_dtype), ty, p.astype(np_dtype), 6.0, 96, pbc=(True, True, False))
+        nn = ref[2]
+        assert np.array_equal(calc.numneigh.cpu().numpy(), nn)
+        fn, rc = calc.firstneigh.cpu().numpy(), calc.rcs.cpu().numpy()
+        for i in range(0, n, 11):
+            assert np.array_equal(fn[i, :nn[i]], ref[3][i, :nn[i]]), (k, i)
+            assert np.array_equal(rc[i, :nn[i]].view(np.uint8), ref[4][i, :nn[i]].view(np.uint8)), (k, i)
+            assert (fn[i, nn[i]:] == -1).all() and not rc[i, nn[i]:].any()
+        _check(got, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
