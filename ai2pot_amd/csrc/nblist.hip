@@ -267,20 +267,27 @@ __device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i,
 
 // One thread per atom walks its images (x outer, z inner: image m = (i * dim_y + j) * dim_z + k,
 // supercell index m * N + p, structure.h:654-681).
+// With split > 1 (small structures, where a thread per atom leaves most of the chip idle) a thread takes one
+// x-layer of an atom's images: thread = atom * split + layer, split = img_dim[0].
 template <typename T>
 __global__ void count_kernel(const Grid<T> g_in, const T* __restrict__ x, int* __restrict__ counts,
                              int* __restrict__ incoming, const GridDyn<T>* __restrict__ gd,
-                             const int* __restrict__ types, int* __restrict__ ilist, int* __restrict__ types_out)
+                             const int* __restrict__ types, int* __restrict__ ilist, int* __restrict__ types_out,
+                             int split)
 {
     const Grid<T> g = with_dyn(g_in, gd);
-    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    const int t = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    const int p = split > 1 ? t / split : t;
     if (p >= g.N) return;
-    if (incoming) incoming[p] = 0;                // counted up by the list kernel
-    // neighborList.h:548-553: the two outputs that do not depend on the list are written here, in atom order (the
-    // list kernel may process the atoms in another order and would scatter them)
-    if (ilist) { ilist[p] = p; types_out[p] = types[p]; }
+    const int i0 = split > 1 ? t - p * split : 0, i1 = split > 1 ? i0 + 1 : g.img_dim[0];
+    if (i0 == 0) {
+        if (incoming) incoming[p] = 0;                // counted up by the list kernel
+        // neighborList.h:548-553: the two outputs that do not depend on the list are written here, in atom order (the
+        // list kernel may process the atoms in another order and would scatter them)
+        if (ilist) { ilist[p] = p; types_out[p] = types[p]; }
+    }
     const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
-    for (int i = 0; i < g.img_dim[0]; i++)
+    for (int i = i0; i < i1; i++)
         for (int j = 0; j < g.img_dim[1]; j++)
             for (int k = 0; k < g.img_dim[2]; k++) {
                 T c[3];
@@ -292,14 +299,16 @@ __global__ void count_kernel(const Grid<T> g_in, const T* __restrict__ x, int* _
 template <typename T>
 __global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict__ offsets,
                             int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x,
-                            const GridDyn<T>* __restrict__ gd)
+                            const GridDyn<T>* __restrict__ gd, int split)
 {
     const Grid<T> g = with_dyn(g_in, gd);
-    const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    const int t = blockIdx.x * NBL_BLOCK + threadIdx.x;
+    const int p = split > 1 ? t / split : t;
     if (p >= g.N) return;
+    const int i0 = split > 1 ? t - p * split : 0, i1 = split > 1 ? i0 + 1 : g.img_dim[0];
     const T xp[3] = {x[(size_t)p * 3], x[(size_t)p * 3 + 1], x[(size_t)p * 3 + 2]};
-    int m = 0;
-    for (int i = 0; i < g.img_dim[0]; i++)
+    int m = i0 * g.img_dim[1] * g.img_dim[2];
+    for (int i = i0; i < i1; i++)
         for (int j = 0; j < g.img_dim[1]; j++)
             for (int k = 0; k < g.img_dim[2]; k++, m++) {
                 T c[3];
@@ -1125,9 +1134,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     rc = fill_zero2(counts, (size_t)nb1 * sizeof(int), cursor, (size_t)nb1 * sizeof(int), stream);
     if (rc) return rc;
     const dim3 pair_grid(ceil_div(N, NBL_BLOCK));
+    // binning: a thread per atom, or per x-layer of an atom's images while the structure is small
+    const int split = (N < 65536 && g.img_dim[0] > 1) ? g.img_dim[0] : 1;
+    const dim3 image_grid(ceil_div((long long)N * split, NBL_BLOCK));
     prof_begin("nbl_count", stream);
-    hipLaunchKernelGGL(count_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming,
-                       (const GridDyn<T>*)gd, types, want_rows ? ilist : (int*)nullptr, types_out);
+    hipLaunchKernelGGL(count_kernel<T>, image_grid, dim3(NBL_BLOCK), 0, stream, g, x, counts, incoming,
+                       (const GridDyn<T>*)gd, types, want_rows ? ilist : (int*)nullptr, types_out, split);
     prof_end(stream);
     rc = exclusive_scan_i32(counts, offsets, nb1, tmp, stream);
     if (rc) return rc;
@@ -1163,8 +1175,8 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
 
     prof_begin("nbl_fill", stream);
 
-    hipLaunchKernelGGL(fill_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
-                       s_idx, s_x, (const GridDyn<T>*)gd);
+    hipLaunchKernelGGL(fill_kernel<T>, image_grid, dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
+                       s_idx, s_x, (const GridDyn<T>*)gd, split);
 
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
