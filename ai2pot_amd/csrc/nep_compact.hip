@@ -1,27 +1,26 @@
-// NEP energy / force / virial by gather, for neighbour lists this library built itself
+// NEP energy / force / virial for neighbour lists this library built itself
 // (a2p_nblist_build_compact_*: one periodic structure, no ghosts, every pair listed from both ends).
 //
 // The reference scatters: atom i computes g_ij = dE_i/dr_ij for each neighbour and does
 // F_i += g_ij, F_j -= g_ij (source/descriptor/nep/include/nep.h:468-515).  With a list that holds
-// every pair from both ends the same forces are a gather,
-//     F_i = sum_j (g_ij - g_ji),        V = -1/2 sum_i sum_j (g_ij - g_ji) r_ij^T,
-// and g_ji is a function of the SAME distance vector and of atom j's adjoints: its dE/dq
-// contracted with the radial coefficients, cc_j[t][k] = sum_n dE_j/dq_n c[t_j][t][n][k], and its
-// dE/dS_{n,lm}.  The harmonics have parity (-1)^l, so both directions share the basis functions,
-// the harmonics and their gradients; the second direction only adds the contraction of atom j's
-// adjoints with its own radial functions:
-//     A_lm = sum_n dE_i/dS_{n,lm} g_n^{ij}(r) + (-1)^l sum_n dE_j/dS_{n,lm} g_n^{ji}(r).
-// No per-pair store, no atomics, no reduction pass: two kernels over the atoms.
-//   nep_adjoint_kernel : radial sums and angular moments over the compact lists, descriptors,
-//                        hidden layer, dE/dq, dE/dS; stores per atom a 96-value record (dE/dS) and, in a
-//                        dense array of their own, the radial coefficients contracted with dE/dq
-//                        (species x 8 values), and the energy partials
-//   nep_gather_kernel  : walks the lists again, gathers the neighbours' records, forms
-//                        g_ij - g_ji, sums force and virial
-// One thread per atom, 256 per workgroup.  Atoms are processed in the Morton order of the list
-// build and workgroups are dealt to the XCDs in contiguous runs, so the records a workgroup
-// gathers were written for, and are being gathered by, its neighbours in space and time.  The
-// lists are read in 8 KiB chunks (8 slots of 64 positions), staged through LDS by each wavefront
+// every pair from both ends the same forces are
+//     F_i = sum_j (g_ij - g_ji),        V = - sum_i sum_j g_ij r_ij^T.
+// Two kernels over the atoms, one thread per atom, 256 per workgroup:
+//   nep_adjoint_kernel : radial sums and angular moments over the compact lists, descriptors, hidden layer,
+//                        dE/dq, dE/dS (kept in registers); then the pairs inside the angular cutoff once
+//                        more: g_ij with both parts, summed into F_i and the virial, and handed to atom j
+//                        through a slot array, slots[place][j], the place claimed with an atomic counter
+//                        per target (an atom is named by as many pairs as its own list has entries; places
+//                        beyond the array's depth fall back to atomic adds on a spare force array).
+//                        It also stores, per atom, the radial coefficients contracted with dE/dq,
+//                        cc_i[t][k] = sum_n dE_i/dq_n c[t_i][t][n][k] (species x 8 values).
+//   nep_gather_kernel  : the pairs between the cutoffs, which have a radial part only: g_ij - g_ji is a
+//                        function of the one distance and of cc_i[t_j] + cc_j[t_i], so the neighbour's 32 bytes
+//                        are gathered and nothing is stored per pair; then the slots of the atom are summed
+//                        (in fixed point, so that the result does not depend on which pair got which
+//                        place) and the force is written.
+// Atoms are processed in the Morton order of the list build and workgroups are dealt to the XCDs in contiguous
+// runs.  The lists are read in 8 KiB chunks (8 slots of 64 positions), staged through LDS by each wavefront
 // for itself: global loads are contiguous, LDS reads are one 16-byte entry per lane.
 //
 // Formulas: source/descriptor/nep/include/{nepBasis.h:57-196; nep.h:320-529}.
@@ -37,9 +36,7 @@ namespace {
 
 constexpr int CB = 256;                 // positions (threads) per workgroup
 constexpr int KC = 8, NAC = 4, LC = 4, NLM = 24, FDP = 24;
-constexpr int REC = NAC * NLM;          // values per adjoint record: dE/dS, 384 bytes in fp32 (three cache lines)
-// the contracted radial coefficients cc[t][k] live in an array of their own, NTC * 8 values per atom:
-// the pairs between the cutoffs gather only these, and a dense array of them stays in L2
+constexpr int NSLOT = 32;               // depth of the slot array: places 0 .. NSLOT-1 of every atom
 constexpr int STP = CL_CHUNK + 1;       // staged slots per position, padded: 16-byte reads of 8 lanes hit 8 banks
 
 template <typename T>
@@ -49,10 +46,12 @@ struct GatherArgs {
     T rr, ra;
     CompactView<T> cv;
     const int* types;     // [natoms]
-    T* rec;               // [natoms][REC] dE/dS
     T* rcc;               // [natoms][NTC * KC] radial coefficients contracted with dE/dq
+    T* slots;             // [NSLOT][natoms][4] derivatives handed to the neighbour, by place
+    T* overflow;          // [natoms][3] the same for places >= NSLOT, summed with atomics (zero on entry)
+    int* incoming;        // [natoms] places claimed so far (zero on entry)
     T* force;             // [natoms][3] or null
-    double* partial;      // [nblocks][10]: energy (adjoint kernel), virial (gather kernel)
+    double* partial;      // [nblocks][10]: energy and virial, each workgroup's share
     int* status;
     int want_virial;
 };
@@ -149,36 +148,64 @@ __device__ __forceinline__ bool position_header(const GatherArgs<T>& a, int p, i
     return true;
 }
 
+// Exact, order-independent sum of a few floating-point values: fixed point in 64-bit integers.
+// fp32 values are kept to 2^-40 (a thousandth of the last bit of a 1e-3 eV/A component), fp64 values in two
+// limbs to 2^-84; |x| must stay below 2^22.
+template <typename T>
+struct FixedSum;
+template <>
+struct FixedSum<float> {
+    long long s = 0;
+    __device__ __forceinline__ void add(float x) { s += (long long)((double)x * 0x1p40); }
+    __device__ __forceinline__ double value() const { return (double)s * 0x1p-40; }
+};
+template <>
+struct FixedSum<double> {
+    long long hi = 0, lo = 0;
+    __device__ __forceinline__ void add(double x)
+    {
+        const double v = x * 0x1p32, h = trunc(v);
+        hi += (long long)h;
+        lo += (long long)((v - h) * 0x1p52);
+    }
+    __device__ __forceinline__ double value() const { return (double)hi * 0x1p-32 + (double)lo * 0x1p-84; }
+};
+constexpr double kFixedSumLimit = 4.0e6;
+
 template <typename T>
 struct AdjointLds {
-    T *coef, *w0, *b0, *w1, *qs, *stage;
+    T *coef, *w0, *b0, *w1, *qs, *acc, *stage;
     double* red;
 };
+// The network tables (w0, b0, w1, qs) are dead once the hidden layer is done; the threads' contracted
+// radial coefficients (acc, [NTC * KC][CB]) are laid over them for the second walk.
 template <typename T>
-__host__ __device__ __forceinline__ size_t adjoint_lds(int nt, int H, int nb, unsigned char* base, AdjointLds<T>& L)
+__host__ __device__ __forceinline__ size_t adjoint_lds(int nt, int ntc, int H, int nb, unsigned char* base, AdjointLds<T>& L)
 {
     size_t off = 0;
     L.coef = (T*)(base + off);  off += lds16((size_t)nt * nt * nb * KC * sizeof(T));
+    const size_t tables = off;
+    L.acc = (T*)(base + off);
     L.w0 = (T*)(base + off);    off += lds16((size_t)nt * H * FDP * sizeof(T));
     L.b0 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
     L.w1 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
     L.qs = (T*)(base + off);    off += lds16((size_t)FDP * sizeof(T));
+    const size_t acc_end = tables + lds16((size_t)ntc * KC * CB * sizeof(T));
+    if (off < acc_end) off = acc_end;
     L.stage = (T*)(base + off); off += lds16((size_t)(CB / 64) * 64 * STP * 4 * sizeof(T));
-    L.red = (double*)(base + off); off += lds16((size_t)(CB / 64) * sizeof(double));
+    L.red = (double*)(base + off); off += lds16((size_t)(CB / 64) * 10 * sizeof(double));
     return off;
 }
 
 template <typename T>
 struct GatherLds {
-    T *coef, *acc, *stage;
+    T* stage;
     double* red;
 };
 template <typename T>
-__host__ __device__ __forceinline__ size_t gather_lds(int nt, int ntc, int nb, unsigned char* base, GatherLds<T>& L)
+__host__ __device__ __forceinline__ size_t gather_lds(unsigned char* base, GatherLds<T>& L)
 {
     size_t off = 0;
-    L.coef = (T*)(base + off);  off += lds16((size_t)nt * nt * nb * KC * sizeof(T));
-    L.acc = (T*)(base + off);   off += lds16((size_t)ntc * KC * CB * sizeof(T));
     L.stage = (T*)(base + off); off += lds16((size_t)(CB / 64) * 64 * STP * 4 * sizeof(T));
     L.red = (double*)(base + off); off += lds16((size_t)(CB / 64) * 9 * sizeof(double));
     return off;
@@ -198,7 +225,7 @@ nep_adjoint_kernel(const GatherArgs<T> a)
     const int tile = p >> 6;
     const int nt = a.ntypes, H = a.H;
     AdjointLds<T> L;
-    adjoint_lds<T>(nt, H, NB, smem_raw, L);
+    adjoint_lds<T>(nt, NTC, H, NB, smem_raw, L);
     T* const st = L.stage + (size_t)wv * 64 * STP * 4;
 
     for (int i = tid; i < nt * nt * NB * KC; i += CB) L.coef[i] = a.coeffs[i];
@@ -330,224 +357,232 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         for (int j = 0; j < DC; j++) dEdq[j] *= L.qs[j];
     }
 
-    // ---- the atom's record: dE/dS (nep.h:450-466) and the radial coefficients contracted with dE/dq
-    if (active) {
-        T* rp = a.rec + (size_t)atom * REC;
+    // ---- dE/dS in place of the moments (nep.h:450-466) ----------------------------------------------
 #pragma unroll
-        for (int n = 0; n < NAC; n++)
+    for (int n = 0; n < NAC; n++)
 #pragma unroll
-            for (int m0 = 0; m0 < NLM; m0 += 4) {
-                T v[4];
+        for (int m = 0; m < NLM; m++) {
+            const int l = m < 3 ? 1 : m < 8 ? 2 : m < 15 ? 3 : 4;
+            const int mp = m - (l * l - 1);
+            S[n][m] = S[n][m] * dEdq[NR + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+        }
+    // ---- the radial coefficients contracted with dE/dq: the thread's own copy in LDS (over the network
+    // tables, which every wavefront has finished with), a copy in memory for the neighbours
+    __syncthreads();
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int m = m0 + u;
-                    const int l = m < 3 ? 1 : m < 8 ? 2 : m < 15 ? 3 : 4;
-                    const int mp = m - (l * l - 1);
-                    v[u] = S[n][m] * dEdq[NR + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
-                }
-                st4(rp + n * NLM + m0, v);
+    for (int t = 0; t < NTC; t++) {
+        T cc[KC];
+#pragma unroll
+        for (int k = 0; k < KC; k++) cc[k] = (T)0;
+        if (t < nt) {
+            const T* c = L.coef + (ti * nt + t) * NB * KC;
+#pragma unroll
+            for (int n = 0; n < NR; n++) {
+                T c0v[4], c1v[4];
+                ld4(c + n * KC, c0v);
+                ld4(c + n * KC + 4, c1v);
+#pragma unroll
+                for (int k = 0; k < 4; k++) { cc[k] += dEdq[n] * c0v[k]; cc[4 + k] += dEdq[n] * c1v[k]; }
             }
+        }
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            T cc[KC];
-#pragma unroll
-            for (int k = 0; k < KC; k++) cc[k] = (T)0;
-            if (t < NTC && t < nt) {
-                const T* c = L.coef + (ti * nt + t) * NB * KC;
-#pragma unroll
-                for (int n = 0; n < NR; n++) {
-                    T c0v[4], c1v[4];
-                    ld4(c + n * KC, c0v);
-                    ld4(c + n * KC + 4, c1v);
-#pragma unroll
-                    for (int k = 0; k < 4; k++) { cc[k] += dEdq[n] * c0v[k]; cc[4 + k] += dEdq[n] * c1v[k]; }
-                }
-            }
+        for (int k = 0; k < KC; k++) L.acc[(t * KC + k) * CB + tid] = cc[k];
+        if (active) {
             T lo[4] = {cc[0], cc[1], cc[2], cc[3]}, hi[4] = {cc[4], cc[5], cc[6], cc[7]};
-            if (t < NTC) {
-                st4(a.rcc + ((size_t)atom * NTC + t) * KC, lo);
-                st4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi);
-            }
+            st4(a.rcc + ((size_t)atom * NTC + t) * KC, lo);
+            st4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi);
         }
     }
 
-    // ---- workgroup partial sum of the energy (fp64) -------------------------------------------------
-    const double ew = wave_sum(active ? (double)e_site : 0.0);
-    if (lane == 0) L.red[wv] = ew;
-    __syncthreads();
-    if (tid == 0) {
-        double v = 0.0;
-        for (int w = 0; w < CB / 64; w++) v += L.red[w];
-        a.partial[(size_t)blk * 10] = v;
+    // ---- pairs inside the angular cutoff: g_ij = dE_i/dr_ij, radial and angular part (nep.h:468-515) ----
+    T fx = (T)0, fy = (T)0, fz = (T)0;
+    T vir[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vir[i] = (T)0;
+    if (a.force || a.want_virial) {
+        const bool hand_over = a.force != nullptr;
+        walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+            int j = bits & CL_INDEX_MASK;
+            if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
+            if (!valid) return;
+            const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
+            // the place of this pair among the pairs that name atom j
+            int place = 0;
+            if (hand_over) place = atomicAdd(a.incoming + j, 1);
+            const T r = sqrt_t(x * x + y * y + z * z);
+            const T rinv = (T)1 / r;
+            const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
+            T f[KC], df[KC];
+            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+            T srad = (T)0;
+#pragma unroll
+            for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * CB + tid] * df[k];
+            radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+            const T* ci = L.coef + ((ti * nt + tj) * NB + NR) * KC;
+            T A[NLM], Ad[NLM];
+#pragma unroll
+            for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
+#pragma unroll
+            for (int n = 0; n < NAC; n++) {
+                T c0v[4], c1v[4];
+                ld4(ci + n * KC, c0v);
+                ld4(ci + n * KC + 4, c1v);
+                T g = (T)0, dg = (T)0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
+#pragma unroll
+                for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
+#pragma unroll
+                for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
+            }
+            T bl[NLM];
+            blm_values<T, LC>(ux, uy, uz, bl);
+#pragma unroll
+            for (int l = 1; l <= LC; l++)
+#pragma unroll
+                for (int mp = 0; mp < 2 * l + 1; mp++) {
+                    const int m = l * l - 1 + mp;
+                    srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
+                }
+            T wx = (T)0, wy = (T)0, wz = (T)0;
+            blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
+            const T gx = srad * ux + wx * rinv, gy = srad * uy + wy * rinv, gz = srad * uz + wz * rinv;
+            if (hand_over) {
+                if (place < NSLOT) {
+                    const T g4[4] = {gx, gy, gz, (T)0};
+                    st4(a.slots + ((size_t)place * a.cv.natoms + j) * 4, g4);
+                } else {
+                    atomicAdd(a.overflow + (size_t)j * 3 + 0, gx);
+                    atomicAdd(a.overflow + (size_t)j * 3 + 1, gy);
+                    atomicAdd(a.overflow + (size_t)j * 3 + 2, gz);
+                }
+            }
+            fx += gx; fy += gy; fz += gz;
+            vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
+            vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
+            vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
+        });
+        if (active && a.force) {
+            T* fo = a.force + (size_t)atom * 3;
+            fo[0] = fx; fo[1] = fy; fo[2] = fz;
+        }
+    }
+
+    // ---- workgroup partial sums of the energy and of this kernel's share of the virial (fp64) ----------
+    {
+        double vals[10];
+        vals[0] = active ? (double)e_site : 0.0;
+#pragma unroll
+        for (int i = 0; i < 9; i++) vals[1 + i] = active ? (double)vir[i] : 0.0;
+        const int nv = a.want_virial ? 10 : 1;
+#pragma unroll
+        for (int i = 0; i < 10; i++) {
+            if (i >= nv) break;
+            const double v = wave_sum(vals[i]);
+            if (lane == 0) L.red[wv * 10 + i] = v;
+        }
+        __syncthreads();
+        if (tid < nv) {
+            double v = 0.0;
+            for (int w = 0; w < CB / 64; w++) v += L.red[w * 10 + tid];
+            a.partial[(size_t)blk * 10 + tid] = v;
+        }
     }
 }
 
-// ---- kernel 2: forces and virial by gather ------------------------------------------------------------
-template <typename T, int NTC, int NR>
-__global__ void __launch_bounds__(CB, (sizeof(T) == 4 ? 2 : 1))
+// ---- kernel 2: pairs between the cutoffs by gather, and the slots -----------------------------------------
+template <typename T, int NTC>
+__global__ void __launch_bounds__(CB)
 nep_gather_kernel(const GatherArgs<T> a)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    constexpr int NB = NR + NAC;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int blk = xcd_block(blockIdx.x, gridDim.x);
     const int p = blk * CB + tid;
     const int tile = p >> 6;
     const int nt = a.ntypes;
     GatherLds<T> L;
-    gather_lds<T>(nt, NTC, NB, smem_raw, L);
+    gather_lds<T>(smem_raw, L);
     T* const st = L.stage + (size_t)wv * 64 * STP * 4;
-
-    for (int i = tid; i < nt * nt * NB * KC; i += CB) L.coef[i] = a.coeffs[i];
 
     int atom, ti, n_outer, n_inner;
     const bool active = position_header<T>(a, p, atom, ti, n_outer, n_inner);
-    const T rr_inv = (T)1 / a.rr, ra_inv = (T)1 / a.ra;
-    const T* const own = a.rec + (size_t)atom * REC;
+    const T rr_inv = (T)1 / a.rr;
 
-    // own adjoints: dE/dS in registers, contracted radial coefficients in LDS (indexed by the
-    // neighbour's species inside the loops)
-    T S[NAC][NLM];
-#pragma unroll
-    for (int n = 0; n < NAC; n++)
-#pragma unroll
-        for (int m0 = 0; m0 < NLM; m0 += 4) {
-            T v[4] = {(T)0, (T)0, (T)0, (T)0};
-            if (active) ld4(own + n * NLM + m0, v);
-#pragma unroll
-            for (int u = 0; u < 4; u++) S[n][m0 + u] = v[u];
-        }
-#pragma unroll
-    for (int t = 0; t < NTC; t++) {
+    // own contracted radial coefficients, one array per neighbour species (separate arrays: a select between
+    // them stays a select, where one two-dimensional array would be indexed through scratch memory)
+    T cc0[KC], cc1[KC], cc2[KC], cc3[KC];
+    auto load_cc = [&](int t, T (&c)[KC]) __attribute__((always_inline)) {
         T lo[4] = {(T)0, (T)0, (T)0, (T)0}, hi[4] = {(T)0, (T)0, (T)0, (T)0};
-        if (active) { ld4(a.rcc + ((size_t)atom * NTC + t) * KC, lo); ld4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi); }
+        if (active && t < NTC) { ld4(a.rcc + ((size_t)atom * NTC + t) * KC, lo); ld4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi); }
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            L.acc[(t * KC + k) * CB + tid] = lo[k];
-            L.acc[(t * KC + 4 + k) * CB + tid] = hi[k];
-        }
-    }
-    __syncthreads();
+        for (int k = 0; k < 4; k++) { c[k] = lo[k]; c[4 + k] = hi[k]; }
+    };
+    load_cc(0, cc0); load_cc(1, cc1); load_cc(2, cc2); load_cc(3, cc3);
 
     T fx = (T)0, fy = (T)0, fz = (T)0;
     T vir[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) vir[i] = (T)0;
-    auto add_pair = [&](bool valid, T x, T y, T z, T gx, T gy, T gz) __attribute__((always_inline)) {
-        gx = valid ? gx : (T)0; gy = valid ? gy : (T)0; gz = valid ? gz : (T)0;
-        fx += gx; fy += gy; fz += gz;
-        vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
-        vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
-        vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
-    };
-    // the neighbour behind an entry: its index (checked; an invalid entry points at the atom
-    // itself, so that every gather stays inside the records) and its species
-    auto neighbour = [&](bool& valid, int bits, int& j, int& tj) __attribute__((always_inline)) {
-        j = bits & CL_INDEX_MASK;
-        if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
-        j = valid ? j : atom;
-        tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
-    };
-
-    // pairs inside the angular cutoff: radial and angular part, both directions
-    walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
-        int j, tj;
-        neighbour(valid, bits, j, tj);
-        const T* const rj = a.rec + (size_t)j * REC;
-        const T r = sqrt_t(x * x + y * y + z * z);
-        const T rinv = (T)1 / r;
-        const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
-        T f[KC], df[KC];
-        // radial part: (cc_i[tj] + cc_j[ti]) . f'(r)
-        T srad = (T)0;
-        {
-            T lo[4], hi[4];
-            ld4(a.rcc + ((size_t)j * NTC + ti) * KC, lo);
-            ld4(a.rcc + ((size_t)j * NTC + ti) * KC + 4, hi);
-            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                srad += (L.acc[(tj * KC + k) * CB + tid] + lo[k]) * df[k];
-                srad += (L.acc[(tj * KC + 4 + k) * CB + tid] + hi[k]) * df[4 + k];
-            }
-        }
-        radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
-        const T* ci = L.coef + ((ti * nt + tj) * NB + NR) * KC;
-        const T* cj = L.coef + ((tj * nt + ti) * NB + NR) * KC;
-        T A[NLM], Ad[NLM];
-#pragma unroll
-        for (int m = 0; m < NLM; m++) { A[m] = (T)0; Ad[m] = (T)0; }
-#pragma unroll
-        for (int n = 0; n < NAC; n++) {
-            T c0v[4], c1v[4];
-            ld4(ci + n * KC, c0v);
-            ld4(ci + n * KC + 4, c1v);
-            T g = (T)0, dg = (T)0;
-#pragma unroll
-            for (int k = 0; k < 4; k++) { g += c0v[k] * f[k]; dg += c0v[k] * df[k]; }
-#pragma unroll
-            for (int k = 0; k < 4; k++) { g += c1v[k] * f[4 + k]; dg += c1v[k] * df[4 + k]; }
-#pragma unroll
-            for (int m = 0; m < NLM; m++) { A[m] += S[n][m] * g; Ad[m] += S[n][m] * dg; }
-            // the other direction: atom j's adjoints with its own radial functions, parity (-1)^l
-            ld4(cj + n * KC, c0v);
-            ld4(cj + n * KC + 4, c1v);
-            T gj = (T)0, dgj = (T)0;
-#pragma unroll
-            for (int k = 0; k < 4; k++) { gj += c0v[k] * f[k]; dgj += c0v[k] * df[k]; }
-#pragma unroll
-            for (int k = 0; k < 4; k++) { gj += c1v[k] * f[4 + k]; dgj += c1v[k] * df[4 + k]; }
-#pragma unroll
-            for (int m0 = 0; m0 < NLM; m0 += 4) {
-                T sj[4];
-                ld4(rj + n * NLM + m0, sj);
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int m = m0 + u;
-                    const bool odd = m < 3 || (m >= 8 && m < 15);           // l = 1 or 3
-                    A[m] += sj[u] * (odd ? -gj : gj);
-                    Ad[m] += sj[u] * (odd ? -dgj : dgj);
-                }
-            }
-        }
-        T bl[NLM];
-        blm_values<T, LC>(ux, uy, uz, bl);
-#pragma unroll
-        for (int l = 1; l <= LC; l++)
-#pragma unroll
-            for (int mp = 0; mp < 2 * l + 1; mp++) {
-                const int m = l * l - 1 + mp;
-                srad += (Ad[m] - (T)l * rinv * A[m]) * bl[m];
-            }
-        T wx = (T)0, wy = (T)0, wz = (T)0;
-        blm_grad_dot<T, LC>(ux, uy, uz, A, wx, wy, wz);
-        add_pair(valid, x, y, z, srad * ux + wx * rinv, srad * uy + wy * rinv, srad * uz + wz * rinv);
-    });
-    // pairs between the cutoffs: radial part only
+    // g_ij - g_ji = (cc_i[t_j] + cc_j[t_i]) . f'(r) r_ij / r
     walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
-        int j, tj;
-        neighbour(valid, bits, j, tj);
+        const int j = bits & CL_INDEX_MASK;
+        if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
+        if (!valid) return;                  // lanes past the end of their list issue no loads
+        const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
         T lo[4], hi[4];
         ld4(a.rcc + ((size_t)j * NTC + ti) * KC, lo);
         ld4(a.rcc + ((size_t)j * NTC + ti) * KC + 4, hi);
         const T r = sqrt_t(x * x + y * y + z * z);
         T f[KC], df[KC];
         radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
+        T ck[KC];
+#pragma unroll
+        for (int k = 0; k < KC; k++) {
+            ck[k] = cc0[k];
+            if (NTC > 1) ck[k] = tj == 1 ? cc1[k] : ck[k];
+            if (NTC > 2) ck[k] = tj == 2 ? cc2[k] : ck[k];
+            if (NTC > 3) ck[k] = tj == 3 ? cc3[k] : ck[k];
+        }
         T sr = (T)0;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            sr += (L.acc[(tj * KC + k) * CB + tid] + lo[k]) * df[k];
-            sr += (L.acc[(tj * KC + 4 + k) * CB + tid] + hi[k]) * df[4 + k];
+            sr += (ck[k] + lo[k]) * df[k];
+            sr += (ck[4 + k] + hi[k]) * df[4 + k];
         }
         sr /= r;
-        add_pair(valid, x, y, z, sr * x, sr * y, sr * z);
+        const T gx = sr * x, gy = sr * y, gz = sr * z;
+        fx += gx; fy += gy; fz += gz;
+        vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
+        vir[3] -= gy * x; vir[4] -= gy * y; vir[5] -= gy * z;
+        vir[6] -= gz * x; vir[7] -= gz * y; vir[8] -= gz * z;
     });
 
+    // what the neighbours inside the angular cutoff handed over: F_i -= sum_j g_ji
     if (active && a.force) {
+        const int n = a.incoming[atom];
+        FixedSum<T> sx, sy, sz;
+        bool ok = true;
+        for (int t = 0; t < min(n, NSLOT); t++) {
+            T v[4];
+            ld4(a.slots + ((size_t)t * a.cv.natoms + atom) * 4, v);
+            ok = ok && fabs((double)v[0]) < kFixedSumLimit && fabs((double)v[1]) < kFixedSumLimit &&
+                 fabs((double)v[2]) < kFixedSumLimit;
+            sx.add(v[0]); sy.add(v[1]); sz.add(v[2]);
+        }
+        double ox = 0.0, oy = 0.0, oz = 0.0;
+        if (n > NSLOT) {
+            ox = (double)a.overflow[(size_t)atom * 3 + 0];
+            oy = (double)a.overflow[(size_t)atom * 3 + 1];
+            oz = (double)a.overflow[(size_t)atom * 3 + 2];
+        }
         T* fo = a.force + (size_t)atom * 3;
-        fo[0] = fx; fo[1] = fy; fo[2] = fz;
+        const double nan = __longlong_as_double(0x7ff8000000000000ll);
+        fo[0] = (T)(ok ? (double)fo[0] + (double)fx - sx.value() - ox : nan);
+        fo[1] = (T)(ok ? (double)fo[1] + (double)fy - sy.value() - oy : nan);
+        fo[2] = (T)(ok ? (double)fo[2] + (double)fz - sz.value() - oz : nan);
     }
-    // every pair was met from both ends: half of the sum is the virial
+    // every pair between the cutoffs was met from both ends: half of this sum is their virial
     if (a.want_virial) {
         double vals[9];
 #pragma unroll
@@ -559,7 +594,7 @@ nep_gather_kernel(const GatherArgs<T> a)
         }
         __syncthreads();
         if (tid < 9) {
-            double v = 0.0;
+            double v = a.partial[(size_t)blk * 10 + 1 + tid];      // the adjoint kernel's share
             for (int w = 0; w < CB / 64; w++) v += L.red[w * 9 + tid];
             a.partial[(size_t)blk * 10 + 1 + tid] = v;
         }
@@ -571,10 +606,10 @@ int launch_gather(const GatherArgs<T>& a, int nblocks, bool pairs, hipStream_t s
 {
     AdjointLds<T> la;
     GatherLds<T> lg;
-    const size_t lds_a = adjoint_lds<T>(a.ntypes, a.H, NR + NAC, nullptr, la);
-    const size_t lds_g = gather_lds<T>(a.ntypes, NTC, NR + NAC, nullptr, lg);
+    const size_t lds_a = adjoint_lds<T>(a.ntypes, NTC, a.H, NR + NAC, nullptr, la);
+    const size_t lds_g = gather_lds<T>(nullptr, lg);
     auto ka = nep_adjoint_kernel<T, NTC, NR>;
-    auto kg = nep_gather_kernel<T, NTC, NR>;
+    auto kg = nep_gather_kernel<T, NTC>;
     if (lds_a > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a));
     if (lds_g > 48 * 1024)
@@ -598,8 +633,7 @@ size_t compact_lds_need(int n_r, int H, int ntypes)
 {
     AdjointLds<T> la;
     GatherLds<T> lg;
-    return std::max(adjoint_lds<T>(ntypes, H, n_r + NAC, nullptr, la),
-                    gather_lds<T>(ntypes, ntc_of(ntypes), n_r + NAC, nullptr, lg));
+    return std::max(adjoint_lds<T>(ntypes, ntc_of(ntypes), H, n_r + NAC, nullptr, la), gather_lds<T>(nullptr, lg));
 }
 
 bool compact_shape_ok(int K, int n_r, int n_a, int l_max, int H, int ntypes)
@@ -643,11 +677,20 @@ int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const
     rc = ws_get(WS_PARTIAL, (size_t)nblocks * 10 * sizeof(double), &ws);
     if (rc) return rc;
     a.partial = (double*)ws;
-    rc = ws_get(WS_PAIR_G, (size_t)natoms * (REC + ntc_of(ntypes) * KC) * sizeof(T), &ws);
-    if (rc) return rc;
-    a.rec = (T*)ws;
-    a.rcc = a.rec + (size_t)natoms * REC;
     const bool pairs = force != nullptr || virial != nullptr;
+    // rcc | slots | overflow | incoming; the last two start every call at zero
+    const size_t n_rcc = (size_t)natoms * ntc_of(ntypes) * KC, n_slots = (size_t)NSLOT * natoms * 4;
+    const size_t zero_bytes = (size_t)natoms * (3 * sizeof(T) + sizeof(int));
+    rc = ws_get(WS_PAIR_G, (n_rcc + n_slots) * sizeof(T) + zero_bytes, &ws);
+    if (rc) return rc;
+    a.rcc = (T*)ws;
+    a.slots = a.rcc + n_rcc;
+    a.overflow = a.slots + n_slots;
+    a.incoming = (int*)(a.overflow + (size_t)natoms * 3);
+    if (force) {
+        rc = fill_zero(a.overflow, zero_bytes, stream);
+        if (rc) return rc;
+    }
     auto launch = [&](auto nr) {
         constexpr int NR = decltype(nr)::value;
         switch (ntc_of(ntypes)) {
