@@ -79,6 +79,58 @@ __device__ __forceinline__ void st4(double* p, const double (&v)[4])
 __device__ __forceinline__ int entry_bits(float w) { return __float_as_int(w); }
 __device__ __forceinline__ int entry_bits(double w) { return (int)__double_as_longlong(w); }
 
+// nep_device.h's radial_basis (f_k = 1/2 (T_k(x)+1) fc(r), basis.h:137-158, 300-332, 519-530) for all KC functions
+template <typename T, bool DER>
+__device__ __forceinline__ void radial_functions(T r, T rc_inv, T (&f)[KC], T (&df)[KC])
+{
+    const T t = r * rc_inv;
+    const T xr = t - (T)1;
+    const T x = (T)2 * xr * xr - (T)1, x2 = x + x;
+    T sn, cs;
+    sincospi_t(t, &sn, &cs);
+    const T fc = (T)0.5 * ((T)1 + cs), hfc = (T)0.5 * fc;
+    const T dfc = (T)(-0.5 * 3.14159265358979323846) * sn * rc_inv, hdfc = (T)0.5 * dfc;
+    const T w = hfc * ((T)4 * rc_inv * xr);                  // 1/2 fc dx/dr
+    T t0 = (T)1, t1 = x, d0 = (T)0, d1 = (T)1;
+    f[0] = fc; f[1] = hfc * x + hfc;
+    if (DER) { df[0] = dfc; df[1] = hdfc * x + hdfc + w; }
+#pragma unroll
+    for (int k = 2; k < KC; k++) {
+        const T tv = x2 * t1 - t0;
+        f[k] = hfc * tv + hfc;
+        if (DER) {
+            const T dv = (T)2 * t1 + (x2 * d1 - d0);
+            df[k] = (hdfc * tv + hdfc) + w * dv;
+            d0 = d1; d1 = dv;
+        }
+        t0 = t1; t1 = tv;
+    }
+}
+
+// sum_k a_k f_k'(r) without the functions themselves:
+//   1/2 fc' (sum a_k T_k + sum a_k) + 1/2 fc x' sum a_k T_k'
+template <typename T>
+__device__ __forceinline__ T radial_derivative_dot(T r, T rc_inv, const T (&a)[KC])
+{
+    const T t = r * rc_inv;
+    const T xr = t - (T)1;
+    const T x = (T)2 * xr * xr - (T)1, x2 = x + x;
+    T sn, cs;
+    sincospi_t(t, &sn, &cs);
+    const T hfc = (T)0.25 * ((T)1 + cs);
+    const T hdfc = (T)(-0.25 * 3.14159265358979323846) * sn * rc_inv;
+    T t0 = (T)1, t1 = x, d0 = (T)0, d1 = (T)1;
+    T s0 = a[0] + a[1], st = a[0] + a[1] * x, sd = a[1];
+#pragma unroll
+    for (int k = 2; k < KC; k++) {
+        const T tv = x2 * t1 - t0;
+        const T dv = (T)2 * t1 + (x2 * d1 - d0);
+        s0 += a[k]; st += a[k] * tv; sd += a[k] * dv;
+        t0 = t1; t1 = tv; d0 = d1; d1 = dv;
+    }
+    return hdfc * (st + s0) + hfc * ((T)4 * rc_inv * xr) * sd;
+}
+
 __host__ __device__ __forceinline__ size_t lds16(size_t bytes) { return (bytes + 15) & ~(size_t)15; }
 
 // Workgroups are handed to the 8 XCDs round robin; giving XCD k the k-th contiguous run of blocks
@@ -258,12 +310,14 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         const T r = sqrt_t(x * x + y * y + z * z);
         const T rinv = (T)1 / r;
         T f[KC], df[KC];
-        radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+        radial_functions<T, false>(r, rr_inv, f, df);
 #pragma unroll
-        for (int t = 0; t < NTC; t++)
+        for (int t = 0; t < NTC; t++) {
+            const T mt = (valid && tj == t) ? (T)1 : (T)0;
 #pragma unroll
-            for (int k = 0; k < KC; k++) F[t][k] += (valid && tj == t) ? f[k] : (T)0;
-        radial_basis<T, KC, false>(r, ra_inv, KC, f, df);
+            for (int k = 0; k < KC; k++) F[t][k] += mt * f[k];
+        }
+        radial_functions<T, false>(r, ra_inv, f, df);
         const T* c = L.coef + ((ti * nt + tj) * NB + NR) * KC;
         T bl[NLM];
         blm_values<T, LC>(x * rinv, y * rinv, z * rinv, bl);
@@ -287,11 +341,13 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
         const T r = sqrt_t(x * x + y * y + z * z);
         T f[KC], df[KC];
-        radial_basis<T, KC, false>(r, rr_inv, KC, f, df);
+        radial_functions<T, false>(r, rr_inv, f, df);
 #pragma unroll
-        for (int t = 0; t < NTC; t++)
+        for (int t = 0; t < NTC; t++) {
+            const T mt = (valid && tj == t) ? (T)1 : (T)0;
 #pragma unroll
-            for (int k = 0; k < KC; k++) F[t][k] += (valid && tj == t) ? f[k] : (T)0;
+            for (int k = 0; k < KC; k++) F[t][k] += mt * f[k];
+        }
     });
 
     // ---- descriptors (nepBasis.h:174-190) -------------------------------------------------------
@@ -413,11 +469,14 @@ nep_adjoint_kernel(const GatherArgs<T> a)
             const T rinv = (T)1 / r;
             const T ux = x * rinv, uy = y * rinv, uz = z * rinv;
             T f[KC], df[KC];
-            radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
-            T srad = (T)0;
+            T srad;
+            {
+                T ck[KC];
 #pragma unroll
-            for (int k = 0; k < KC; k++) srad += L.acc[(tj * KC + k) * CB + tid] * df[k];
-            radial_basis<T, KC, true>(r, ra_inv, KC, f, df);
+                for (int k = 0; k < KC; k++) ck[k] = L.acc[(tj * KC + k) * CB + tid];
+                srad = radial_derivative_dot<T>(r, rr_inv, ck);
+            }
+            radial_functions<T, true>(r, ra_inv, f, df);
             const T* ci = L.coef + ((ti * nt + tj) * NB + NR) * KC;
             T A[NLM], Ad[NLM];
 #pragma unroll
@@ -534,8 +593,6 @@ nep_gather_kernel(const GatherArgs<T> a)
         ld4(a.rcc + ((size_t)j * NTC + ti) * KC, lo);
         ld4(a.rcc + ((size_t)j * NTC + ti) * KC + 4, hi);
         const T r = sqrt_t(x * x + y * y + z * z);
-        T f[KC], df[KC];
-        radial_basis<T, KC, true>(r, rr_inv, KC, f, df);
         T ck[KC];
 #pragma unroll
         for (int k = 0; k < KC; k++) {
@@ -544,13 +601,9 @@ nep_gather_kernel(const GatherArgs<T> a)
             if (NTC > 2) ck[k] = tj == 2 ? cc2[k] : ck[k];
             if (NTC > 3) ck[k] = tj == 3 ? cc3[k] : ck[k];
         }
-        T sr = (T)0;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            sr += (ck[k] + lo[k]) * df[k];
-            sr += (ck[4 + k] + hi[k]) * df[4 + k];
-        }
-        sr /= r;
+        for (int k = 0; k < 4; k++) { ck[k] += lo[k]; ck[4 + k] += hi[k]; }
+        const T sr = radial_derivative_dot<T>(r, rr_inv, ck) / r;
         const T gx = sr * x, gy = sr * y, gz = sr * z;
         fx += gx; fy += gy; fz += gz;
         vir[0] -= gx * x; vir[1] -= gx * y; vir[2] -= gx * z;
