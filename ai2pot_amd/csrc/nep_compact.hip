@@ -141,14 +141,17 @@ __device__ __forceinline__ int xcd_block(int w, int nb)
     return k * per + min(k, rem) + (w >> 3);
 }
 
-// One chunk (8 slots of the tile's 64 positions, contiguous in memory) into the wavefront's
-// staging buffer, position-major with STP slots per position.
+// One chunk (8 slots of the tile's 64 positions, contiguous in memory) on its way into the wavefront's
+// staging buffer (position-major with STP slots per position): contiguous loads, then 16-byte LDS stores.
 template <typename T>
-__device__ __forceinline__ void stage_chunk(const T* __restrict__ g, T* __restrict__ st, int lane)
+__device__ __forceinline__ void chunk_load(const T* __restrict__ g, int lane, T (&v)[CL_CHUNK][4])
 {
-    T v[CL_CHUNK][4];
 #pragma unroll
     for (int it = 0; it < CL_CHUNK; it++) ld4(g + (size_t)(it * 64 + lane) * 4, v[it]);
+}
+template <typename T>
+__device__ __forceinline__ void chunk_store(T* __restrict__ st, int lane, const T (&v)[CL_CHUNK][4])
+{
 #pragma unroll
     for (int it = 0; it < CL_CHUNK; it++) {
         const int idx = it * 64 + lane;
@@ -158,24 +161,31 @@ __device__ __forceinline__ void stage_chunk(const T* __restrict__ g, T* __restri
 
 // Walks one of the two lists of the wavefront's 64 positions: chunk after chunk through the staging
 // buffer, every lane making the trips of the longest list; body(valid, x, y, z, bits).  A lane past
-// the end of its own list gets a unit vector and valid = false.
-template <typename T, typename Body>
+// the end of its own list gets a unit vector and valid = false.  With AHEAD the next chunk is requested
+// before the trips of the current one and waits in registers (32 of them) meanwhile.
+template <typename T, bool AHEAD = false, typename Body>
 __device__ __forceinline__ void walk_list(const CompactView<T>& cv, int tile, int lane, T* st, int n, bool inner,
                                           Body&& body)
 {
     const int trips = __builtin_amdgcn_readfirstlane(wave_max(n));
+    T v[CL_CHUNK][4];
+    if (AHEAD && trips > 0)
+        chunk_load<T>(cv.entries + compact_chunk_offset<T>(cv.nch, tile, inner ? cv.nch - 1 : 0), lane, v);
     for (int c = 0; c * CL_CHUNK < trips; c++) {
         const int chunk = inner ? cv.nch - 1 - c : c;
+        if (!AHEAD) chunk_load<T>(cv.entries + compact_chunk_offset<T>(cv.nch, tile, chunk), lane, v);
         __builtin_amdgcn_wave_barrier();
-        stage_chunk<T>(cv.entries + compact_chunk_offset<T>(cv.nch, tile, chunk), st, lane);
+        chunk_store<T>(st, lane, v);
         __builtin_amdgcn_wave_barrier();
+        if (AHEAD && (c + 1) * CL_CHUNK < trips)
+            chunk_load<T>(cv.entries + compact_chunk_offset<T>(cv.nch, tile, inner ? chunk - 1 : chunk + 1), lane, v);
         for (int s = 0; s < CL_CHUNK; s++) {
             const int e = c * CL_CHUNK + s;
             if (e >= trips) break;                               // wave-uniform
-            T v[4];
-            ld4(st + (lane * STP + (inner ? CL_CHUNK - 1 - s : s)) * 4, v);
+            T w[4];
+            ld4(st + (lane * STP + (inner ? CL_CHUNK - 1 - s : s)) * 4, w);
             const bool valid = e < n;
-            body(valid, valid ? v[0] : (T)1, valid ? v[1] : (T)0, valid ? v[2] : (T)0, entry_bits(v[3]));
+            body(valid, valid ? w[0] : (T)1, valid ? w[1] : (T)0, valid ? w[2] : (T)0, entry_bits(w[3]));
         }
     }
 }
@@ -337,7 +347,7 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         }
     });
     // neighbours between the cutoffs: radial sums only
-    walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+    walk_list<T, true>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
         const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
         const T r = sqrt_t(x * x + y * y + z * z);
         T f[KC], df[KC];
@@ -584,7 +594,7 @@ nep_gather_kernel(const GatherArgs<T> a)
 #pragma unroll
     for (int i = 0; i < 9; i++) vir[i] = (T)0;
     // g_ij - g_ji = (cc_i[t_j] + cc_j[t_i]) . f'(r) r_ij / r
-    walk_list<T>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+    walk_list<T, true>(a.cv, tile, lane, st, n_outer, false, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
         const int j = bits & CL_INDEX_MASK;
         if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
         if (!valid) return;                  // lanes past the end of their list issue no loads
