@@ -315,7 +315,7 @@ nep_adjoint_kernel(const GatherArgs<T> a)
     __syncthreads();
 
     // neighbours inside the angular cutoff: radial sums and angular moments
-    walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+    walk_list<T, true>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
         const int tj = min((bits >> CL_TYPE_SHIFT) & 15, nt - 1);
         const T r = sqrt_t(x * x + y * y + z * z);
         const T rinv = (T)1 / r;
@@ -467,7 +467,7 @@ nep_adjoint_kernel(const GatherArgs<T> a)
     for (int i = 0; i < 9; i++) vir[i] = (T)0;
     if (a.force || a.want_virial) {
         const bool hand_over = a.force != nullptr;
-        walk_list<T>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
+        walk_list<T, true>(a.cv, tile, lane, st, n_inner, true, [&](bool valid, T x, T y, T z, int bits) __attribute__((always_inline)) {
             int j = bits & CL_INDEX_MASK;
             if (valid && j >= a.cv.natoms) { atomicOr(a.status, ST_BAD_NEIGHBOR); valid = false; }
             if (!valid) return;
