@@ -545,7 +545,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     const Grid<T> g = with_dyn(g_in, gd);
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
-    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_ENT_CAP];
+    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_APW][NBL_ENT_CAP];
     extern __shared__ __align__(16) unsigned char sh_rows[];
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * NBL_APW;
@@ -576,8 +576,30 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         for (int d = 0; d < 3; d++)
             cs[a][d] = COMPACT ? ce.xs[(size_t)min(p0 + a, g.N - 1) * 3 + d] : x[(size_t)atom[a] * 3 + d];
     const int nruns = (2 * g.ext_bins + 1) * (2 * g.ext_bins + 1);
+    // With at most 32 columns per atom the wave's two atoms are set up side by side, lanes 0-31 and 32-63 (their
+    // halves of sh_start / sh_base, their own flat list); with more, one after the other through the first
+    // flat list, the column runs of the second requested before the candidates of the first are scanned.
+    static_assert(NBL_APW == 2, "two atoms per wavefront");
+    const bool paired = nruns <= 32;              // wave-uniform
     int start, len;
-    column_setup<T>(g, cs[0], lane, offsets, start, len);
+    int totals[NBL_APW] = {0, 0};
+    if (paired) {
+        const int sub = lane >> 5;
+        const T csel[3] = {sub ? cs[1][0] : cs[0][0], sub ? cs[1][1] : cs[0][1], sub ? cs[1][2] : cs[0][2]};
+        column_setup<T>(g, csel, lane & 31, offsets, start, len);
+        if (sub >= np) len = 0;
+        const int incl = wave_inclusive_scan(len);
+        totals[0] = __shfl(incl, 31, 64);
+        totals[1] = __shfl(incl, 63, 64) - totals[0];
+        const int base = incl - len - (sub ? totals[0] : 0);
+        sh_start[wv][lane] = start;
+        sh_base[wv][lane] = base;
+        if ((sub ? totals[1] : totals[0]) <= NBL_ENT_CAP)
+            for (int k = 0; k < len; k++) sh_ent[wv][sub][base + k] = start + k;
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        column_setup<T>(g, cs[0], lane, offsets, start, len);
+    }
 #pragma unroll
     for (int ia = 0; ia < NBL_APW; ia++) {
     if (ia >= np) break;                          // wave-uniform
@@ -586,16 +608,21 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     const bool rows = !COMPACT || ce.write_rows;  // wave-uniform
     const T (&c)[3] = cs[ia];
     int nstart = 0, nlen = 0;
-    if (ia + 1 < NBL_APW && ia + 1 < np) column_setup<T>(g, cs[ia + 1 < NBL_APW ? ia + 1 : ia], lane, offsets, nstart, nlen);
-    const int incl = wave_inclusive_scan(len);
-    const int total = __shfl(incl, 63, 64);
-    const int base = incl - len;
-    sh_start[wv][lane] = start;
-    sh_base[wv][lane] = base;
+    if (!paired) {
+        if (ia + 1 < NBL_APW && ia + 1 < np) column_setup<T>(g, cs[ia + 1 < NBL_APW ? ia + 1 : ia], lane, offsets, nstart, nlen);
+        const int incl = wave_inclusive_scan(len);
+        totals[ia] = __shfl(incl, 63, 64);
+        const int base = incl - len;
+        sh_start[wv][lane] = start;
+        sh_base[wv][lane] = base;
+        if (totals[ia] <= NBL_ENT_CAP)
+            for (int k = 0; k < len; k++) sh_ent[wv][0][base + k] = start + k;
+        __builtin_amdgcn_wave_barrier();
+    }
+    const int total = totals[ia];
     const bool flat = total <= NBL_ENT_CAP;       // wave-uniform
-    if (flat)
-        for (int k = 0; k < len; k++) sh_ent[wv][base + k] = start + k;
-    __builtin_amdgcn_wave_barrier();
+    const int so = paired ? ia * 32 : 0;          // the atom's part of sh_start / sh_base
+    const int* const ents = sh_ent[wv][paired ? ia : 0];
 
     int cnt = 0;
     const size_t rowi = (size_t)p * umax;
@@ -614,15 +641,15 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             if (ci < total) {
                 int ent;
                 if (flat) {
-                    ent = sh_ent[wv][ci];
+                    ent = ents[ci];
                 } else {
                     // last column whose base is <= ci
                     int lo = 0, hi = nruns - 1;
                     while (lo < hi) {
                         const int mid = (lo + hi + 1) >> 1;
-                        if (sh_base[wv][mid] <= ci) lo = mid; else hi = mid - 1;
+                        if (sh_base[wv][so + mid] <= ci) lo = mid; else hi = mid - 1;
                     }
-                    ent = sh_start[wv][lo] + (ci - sh_base[wv][lo]);
+                    ent = sh_start[wv][so + lo] + (ci - sh_base[wv][so + lo]);
                 }
                 sj[u] = s_idx[ent];
                 px[u] = s_x[(size_t)ent * 3 + 0];
