@@ -27,7 +27,8 @@ class NepCalculator:
     def __init__(self, model, natoms, lattice, types, umax=200, rcut=None, pbc=(True, True, True),
                  sort=False, dtype=torch.float32, device="cuda:0", places_from_list=None, path="auto",
                  padded=True, reorder_every=64, sync_free=False):
-        """path: "gather" evaluates forces as a gather over compact lists cut by the list build (common
+        """path: "gather" evaluates energy, forces and virial on compact lists cut by the list build (pairs
+        inside the angular cutoff handed to the neighbour through claimed slots, radial pairs by gather; common
         model shapes, unsorted rows, umax % 8 == 0); "segments" scatters pair derivatives into reduction
         segments from the padded arrays (any model shape); "auto" takes the gather when it applies.
         padded=False (gather only) skips the padded firstneigh / rcs arrays: the step then produces

@@ -210,7 +210,7 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
                                 int* incoming, int* max_numneigh, void* stream);
 
 /* ------------------------------------------------------------------------------------------
- * Device-resident step: compact neighbour lists + NEP E/F/V by gather.  Together the two calls
+ * Device-resident step: compact neighbour lists + NEP E/F/V on them.  Together the two calls
  * replace the reference's inference pair  nblist.find_info4mlff(...)  ->  torch.ops.nep.nepToEFVOp(...)
  * (ai2pot/utils/usepot.py:76-97, ai2pot/models/nep/nep.py:298-357) for ONE periodic structure
  * without ghosts, when positions stay on the device.  No counterpart of the list format exists in
@@ -229,9 +229,16 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * Needs umax % 8 == 0, natoms < 2^28, species < 16, 16-byte aligned firstneigh / rcs.
  *
  * a2p_nep_efv_compact_*: energy, forces and virial of the structure from that buffer.  The list
- * names every pair from both ends, so F_i = sum_j (g_ij - g_ji) is evaluated as a gather over
- * atom i's own list with atom j's adjoints (nep.h:468-515 scatters the same terms): no atomics,
- * no per-pair stores, results bit-reproducible.  Model shapes: chebyshev_size 8, n_radial 4 or 6,
+ * names every pair from both ends, so F_i = sum_j (g_ij - g_ji) (nep.h:468-515 scatters the same terms).
+ * For a pair inside the angular cutoff atom i evaluates g_ij once, adds it to its own force and hands it
+ * to atom j through a 16-byte slot whose place it claims with an integer atomic; atom j sums its slots
+ * in fixed point, so the result does not depend on the order of the claims: bit-reproducible.  For a pair
+ * between the cutoffs g_ij - g_ji is evaluated by both ends from 32 gathered bytes of the other's
+ * adjoints: nothing stored per pair.  The slots (32 per atom, 16 or 32 bytes each) live in the library's
+ * workspace; an atom named by more than 32 pairs inside the angular cutoff receives the rest through
+ * floating-point atomics (summation order, hence the last bits, may then vary between calls).  A pair
+ * derivative of 4e6 or more in magnitude (eV/A) makes the receiving atom's force NaN.
+ * Model shapes: chebyshev_size 8, n_radial 4 or 6,
  * n_angular 4, l_max 4, at most 4 species (A2P_ERR_INVALID otherwise: use a2p_nep_efv_*).
  * types[natoms] are the type indices the list was built with.  etot[1] is required; force[natoms][3]
  * and virial[9] may be NULL.
