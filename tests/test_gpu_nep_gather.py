@@ -1,4 +1,4 @@
-"""GPU parity of the device-resident step (compact neighbour lists + NEP E/F/V by gather,
+"""GPU parity of the device-resident step (compact neighbour lists + NEP E/F/V on them,
 a2p_nblist_build_compact_* / a2p_nep_efv_compact_*) against the CPU oracle.
 
 Bars as for the scatter path: fp64 within 1e-10 relative, fp32 energies and virials within 1e-5
@@ -131,6 +131,23 @@ def test_model_shapes(oracle, cfg):
     out = _step(calc, pos, np.float64)
     ref = oracle.nblist(lat, ty, pos, 6.0, 160)
     _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float64), np.float64)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
+def test_more_pairs_inside_the_angular_cutoff_than_slots(oracle, np_dtype):
+    """Equal cutoffs of 7 A at 0.04 atoms / A^3: every atom is named by about 57 pairs inside the angular cutoff,
+    more than the 32 hand-over slots, so the rest reaches it through the spare force array; also a structure
+    whose atoms have no pair between the cutoffs at all."""
+    n = 300
+    lat, pos = synth.random_packed(n, [19.0, 20.0, 19.5], 2.0, 351)
+    ty = synth.rng_randint(352, n, 3)
+    m = synth.nep_model(rmax_radial=7.0, rmax_angular=7.0, seed=3305)
+    calc = _calc(m, lat, ty, n, np_dtype, umax=136, path="gather")
+    out = _step(calc, pos, np_dtype)
+    ref = oracle.nblist(lat, ty, pos, 7.0, 136)
+    assert ref[2].min() > 32 and ref[2].max() <= 136
+    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
+    assert np.abs(out[1].astype(np.float64).sum(0)).max() < (1e-9 if np_dtype == np.float64 else 1e-2)
 
 
 def test_gather_equals_segments_and_is_reproducible(oracle):
