@@ -265,6 +265,34 @@ __device__ __forceinline__ int locate(const Grid<T>& g, const T (&xp)[3], int i,
     return (bin[0] * g.rdim[1] + bin[1]) * g.rdim[2] + bin[2];
 }
 
+// ---- image records: [x y z index], 4 values of T, the index in the bits of the fourth ------------------
+template <typename T>
+__device__ __forceinline__ void entry_store(T* p, T x, T y, T z, int bits);
+template <>
+__device__ __forceinline__ void entry_store<float>(float* p, float x, float y, float z, int bits)
+{
+    *reinterpret_cast<float4*>(p) = make_float4(x, y, z, __int_as_float(bits));
+}
+template <>
+__device__ __forceinline__ void entry_store<double>(double* p, double x, double y, double z, int bits)
+{
+    *reinterpret_cast<double2*>(p) = make_double2(x, y);
+    *reinterpret_cast<double2*>(p + 2) = make_double2(z, __longlong_as_double((long long)bits));
+}
+
+// the reverse: one 16-byte (fp32) or two 16-byte (fp64) loads
+__device__ __forceinline__ void entry_load(const float* p, float& x, float& y, float& z, int& bits)
+{
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    x = v.x; y = v.y; z = v.z; bits = __float_as_int(v.w);
+}
+__device__ __forceinline__ void entry_load(const double* p, double& x, double& y, double& z, int& bits)
+{
+    const double2 v0 = *reinterpret_cast<const double2*>(p);
+    const double2 v1 = *reinterpret_cast<const double2*>(p + 2);
+    x = v0.x; y = v0.y; z = v1.x; bits = (int)__double_as_longlong(v1.y);
+}
+
 // One thread per atom walks its images (x outer, z inner: image m = (i * dim_y + j) * dim_z + k,
 // supercell index m * N + p, structure.h:654-681).
 // With split > 1 (small structures, where a thread per atom leaves most of the chip idle) a thread takes one
@@ -298,7 +326,7 @@ __global__ void count_kernel(const Grid<T> g_in, const T* __restrict__ x, int* _
 
 template <typename T>
 __global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict__ offsets,
-                            int* __restrict__ cursor, int* __restrict__ s_idx, T* __restrict__ s_x,
+                            int* __restrict__ cursor, T* __restrict__ s_rec,
                             const GridDyn<T>* __restrict__ gd, int split)
 {
     const Grid<T> g = with_dyn(g_in, gd);
@@ -315,10 +343,7 @@ __global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const i
                 const int bin = locate(g, xp, i, j, k, c);
                 if (bin < 0) continue;
                 const int pos = offsets[bin] + atomicAdd(&cursor[bin], 1);
-                s_idx[pos] = m * g.N + p;
-                s_x[(size_t)pos * 3 + 0] = c[0];
-                s_x[(size_t)pos * 3 + 1] = c[1];
-                s_x[(size_t)pos * 3 + 2] = c[2];
+                entry_store<T>(s_rec + (size_t)pos * 4, c[0], c[1], c[2], m * g.N + p);
             }
 }
 
@@ -328,33 +353,34 @@ __global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const i
 // With `types` the species of the atom rides in the bits above CL_TYPE_SHIFT (compact lists: the list
 // kernel then never gathers a neighbour's species).
 template <typename T>
-__global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, int* __restrict__ s_idx,
-                               T* __restrict__ s_x, int natoms, const int* __restrict__ types,
-                               const GridDyn<T>* __restrict__ gd)
+__global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, T* __restrict__ s_rec, int natoms,
+                               const int* __restrict__ types, const GridDyn<T>* __restrict__ gd)
 {
     if (gd) nbins = gd->nregion;                  // the launch covers the host's bound
     const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (b >= nbins) return;
     const int beg = offsets[b], end = offsets[b + 1];
     for (int i = beg + 1; i < end; i++) {
-        const int key = s_idx[i];
-        const T kx = s_x[(size_t)i * 3], ky = s_x[(size_t)i * 3 + 1], kz = s_x[(size_t)i * 3 + 2];
+        T kx, ky, kz;
+        int key;
+        entry_load(s_rec + (size_t)i * 4, kx, ky, kz, key);
         int j = i - 1;
-        while (j >= beg && s_idx[j] < key) {
-            s_idx[j + 1] = s_idx[j];
-            s_x[(size_t)(j + 1) * 3] = s_x[(size_t)j * 3];
-            s_x[(size_t)(j + 1) * 3 + 1] = s_x[(size_t)j * 3 + 1];
-            s_x[(size_t)(j + 1) * 3 + 2] = s_x[(size_t)j * 3 + 2];
+        while (j >= beg) {
+            T x, y, z;
+            int idx;
+            entry_load(s_rec + (size_t)j * 4, x, y, z, idx);
+            if (idx >= key) break;
+            entry_store<T>(s_rec + (size_t)(j + 1) * 4, x, y, z, idx);
             j--;
         }
-        s_idx[j + 1] = key;
-        s_x[(size_t)(j + 1) * 3] = kx;
-        s_x[(size_t)(j + 1) * 3 + 1] = ky;
-        s_x[(size_t)(j + 1) * 3 + 2] = kz;
+        entry_store<T>(s_rec + (size_t)(j + 1) * 4, kx, ky, kz, key);
     }
     for (int i = beg; i < end; i++) {
-        const int at = s_idx[i] % natoms;
-        s_idx[i] = types ? at | ((types[at] & 15) << CL_TYPE_SHIFT) : at;
+        T x, y, z;
+        int idx;
+        entry_load(s_rec + (size_t)i * 4, x, y, z, idx);
+        const int at = idx % natoms;
+        entry_store<T>(s_rec + (size_t)i * 4, x, y, z, types ? at | ((types[at] & 15) << CL_TYPE_SHIFT) : at);
     }
 }
 
@@ -518,24 +544,10 @@ struct CompactEmit {
     int write_rows;     // the padded outputs are wanted as well
 };
 
-template <typename T>
-__device__ __forceinline__ void entry_store(T* p, T x, T y, T z, int bits);
-template <>
-__device__ __forceinline__ void entry_store<float>(float* p, float x, float y, float z, int bits)
-{
-    *reinterpret_cast<float4*>(p) = make_float4(x, y, z, __int_as_float(bits));
-}
-template <>
-__device__ __forceinline__ void entry_store<double>(double* p, double x, double y, double z, int bits)
-{
-    *reinterpret_cast<double2*>(p) = make_double2(x, y);
-    *reinterpret_cast<double2*>(p + 2) = make_double2(z, __longlong_as_double((long long)bits));
-}
-
 template <typename T, bool SORT, bool ROWBUF, bool RANK, bool COMPACT = false>
 __global__ void __launch_bounds__(NBL_BLOCK)
 lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict__ types,
-             const int* __restrict__ offsets, const int* __restrict__ s_idx, const T* __restrict__ s_x,
+             const int* __restrict__ offsets, const T* __restrict__ s_rec,
              int umax, int* __restrict__ ilist, int* __restrict__ numneigh, int* __restrict__ firstneigh,
              T* __restrict__ rcs, int* __restrict__ types_out, T* __restrict__ keys,
              int* __restrict__ status, int update, int* __restrict__ rank_out, int* __restrict__ incoming,
@@ -651,10 +663,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
                     }
                     ent = sh_start[wv][so + lo] + (ci - sh_base[wv][so + lo]);
                 }
-                sj[u] = s_idx[ent];
-                px[u] = s_x[(size_t)ent * 3 + 0];
-                py[u] = s_x[(size_t)ent * 3 + 1];
-                pz[u] = s_x[(size_t)ent * 3 + 2];
+                entry_load(s_rec + (size_t)ent * 4, px[u], py[u], pz[u], sj[u]);
             }
         }
         // RANK: the pair's place among the pairs that name the same neighbour, claimed here so that
@@ -1090,7 +1099,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     for (int a = 0; a < 3 && same; a++) same = g_bound.pbc[a] == (pbc[a] ? 1 : 0);
     for (int q = 0; q < 9 && same; q++) same = g_bound.lattice[q] == (double)lattice[q];
     const bool sync_free = g_sync_free && same && !max_nn_host &&
-                           (long long)N * g.nimg * (long long)(sizeof(int) + 3 * sizeof(T)) <= (2ll << 30);
+                           (long long)N * g.nimg * (long long)(4 * sizeof(T)) <= (2ll << 30);
     GridDyn<T>* gd = nullptr;
     long long nregion = 1;
     if (sync_free) {
@@ -1148,7 +1157,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     const int nb1 = (int)nregion + 1;
 
     // workspace B: counts[nb1] | offsets[nb1] | cursor[nb1] | scan tmp, then (after the count is
-    // known) s_idx[total] | s_x[total*3], and for sort: keys[N*umax] | order[N*umax] | tmp rows
+    // known) the image records s_rec[total][4], and for sort: keys[N*umax] | order[N*umax] | tmp rows
     const int ntmp = scan_tmp_ints(nb1);
     size_t ints = (size_t)nb1 * 3 + ntmp;
     void* wsB = nullptr;
@@ -1174,20 +1183,19 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     // bound stays below 2 GiB the arrays are simply sized for it and the host never learns the count
     // (one synchronisation less per build); beyond, the count is read back.
     long long total = (long long)N * g.nimg;
-    if (total * (long long)(sizeof(int) + 3 * sizeof(T)) > (2ll << 30)) {
+    if (total * (long long)(4 * sizeof(T)) > (2ll << 30)) {
         int counted = 0;
         A2P_HIP_CHECK(hipMemcpyAsync(&counted, offsets + nregion, sizeof(int), hipMemcpyDeviceToHost, stream));
         A2P_HIP_CHECK(hipStreamSynchronize(stream));
         total = counted;
     }
 
-    size_t sorted_bytes = (size_t)total * (sizeof(int) + 3 * sizeof(T)) + 256;
+    size_t sorted_bytes = (size_t)total * 4 * sizeof(T) + 256;
     size_t sort_bytes = sort ? (size_t)N * umax * (2 * sizeof(int) + 4 * sizeof(T)) + 256 : 0;
     void* wsC = nullptr;
     rc = ws_get(WS_MISC, sorted_bytes + sort_bytes, &wsC);
     if (rc) return rc;
-    T* s_x = (T*)wsC;                                   // T first keeps double alignment
-    int* s_idx = (int*)(s_x + (size_t)total * 3);
+    T* s_rec = (T*)wsC;
     char* sort_base = (char*)wsC + (sorted_bytes / 256) * 256;   // 256-byte aligned, inside the slack
     T* tmp_rcs = nullptr;
     T* keys = nullptr;
@@ -1203,12 +1211,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_begin("nbl_fill", stream);
 
     hipLaunchKernelGGL(fill_kernel<T>, image_grid, dim3(NBL_BLOCK), 0, stream, g, x, offsets, cursor,
-                       s_idx, s_x, (const GridDyn<T>*)gd, split);
+                       s_rec, (const GridDyn<T>*)gd, split);
 
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
-                       (int)nregion, offsets, s_idx, s_x, g.N, co ? types : (const int*)nullptr, (const GridDyn<T>*)gd);
+                       (int)nregion, offsets, s_rec, g.N, co ? types : (const int*)nullptr, (const GridDyn<T>*)gd);
     prof_end(stream);
     CompactEmit<T> ce{};
     if (co) {
@@ -1261,27 +1269,27 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                         (uintptr_t)rcs % 16 == 0 && (uintptr_t)rank % 16 == 0;
     if (co)
         hipLaunchKernelGGL((lists_kernel<T, false, true, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds,
-                           stream, g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out,
+                           stream, g, x, types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out,
                            keys, status, update, nullptr, nullptr, ce, (const GridDyn<T>*)gd);
     else if (sort)
         hipLaunchKernelGGL((lists_kernel<T, true, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
-                           types, offsets, s_idx, s_x, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
+                           types, offsets, s_rec, umax, ilist, numneigh, tmp_first, tmp_rcs, types_out, keys,
                            status, 0, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rowbuf && rank)
         hipLaunchKernelGGL((lists_kernel<T, false, true, true>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
-                           g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           g, x, types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
                            status, update, rank, incoming, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rowbuf)
         hipLaunchKernelGGL((lists_kernel<T, false, true, false>), dim3(list_blocks), dim3(NBL_BLOCK), rows_lds, stream,
-                           g, x, types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           g, x, types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
                            status, update, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else if (rank)
         hipLaunchKernelGGL((lists_kernel<T, false, false, true>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
-                           types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
                            status, update, rank, incoming, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     else
         hipLaunchKernelGGL((lists_kernel<T, false, false, false>), dim3(list_blocks), dim3(NBL_BLOCK), 0, stream, g, x,
-                           types, offsets, s_idx, s_x, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
+                           types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
                            status, update, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     prof_end(stream);
     if (sort) {
