@@ -462,13 +462,14 @@ __device__ __forceinline__ void pad_fill(V* __restrict__ row, int beg, int end, 
 // the dz run of a (dx, dy) column is contiguous: lane c owns column c.  A column, or the ends of
 // its dz run, that lies farther from the centre atom than rcut (with a margin for the rounding
 // of the binning) cannot contribute and is left out; the order of what remains is unchanged.
-// The runs are then laid out back to back in LDS as a flat candidate list, which the wave
-// scans 64 candidates at a time; accepted candidates are appended with a ballot prefix.
+// The runs are then laid out back to back as a flat candidate list (in LDS: the column of every
+// candidate, one byte each, next to the columns' starts and bases), which the wave scans 64
+// candidates at a time; accepted candidates are appended with a ballot prefix.
 // With ROWBUF the wave assembles its whole output row (accepted entries, then the -1 / 0 padding)
 // in LDS and writes it with 16-byte stores, one full row of firstneigh and one of rcs; this needs
 // umax % 4 == 0 and 16-byte aligned outputs.
 constexpr int NBL_UNROLL = 4;
-constexpr int NBL_ENT_CAP = 256;   // flat candidate list per wave (entries); longer lists search the runs
+constexpr int NBL_ENT_CAP = 256;   // flat candidate list per atom (entries); longer lists search the runs
 
 template <typename T>
 inline size_t rowbuf_bytes(int umax, bool rank) { return (size_t)umax * (4 + 3 * sizeof(T) + (rank ? 4 : 0)); }
@@ -557,7 +558,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     const Grid<T> g = with_dyn(g_in, gd);
     __shared__ int sh_start[NBL_BLOCK / 64][64];
     __shared__ int sh_base[NBL_BLOCK / 64][64];
-    __shared__ int sh_ent[NBL_BLOCK / 64][NBL_APW][NBL_ENT_CAP];
+    __shared__ unsigned char sh_col[NBL_BLOCK / 64][NBL_APW][NBL_ENT_CAP];   // column of each flat candidate
     extern __shared__ __align__(16) unsigned char sh_rows[];
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * NBL_APW;
@@ -607,7 +608,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         sh_start[wv][lane] = start;
         sh_base[wv][lane] = base;
         if ((sub ? totals[1] : totals[0]) <= NBL_ENT_CAP)
-            for (int k = 0; k < len; k++) sh_ent[wv][sub][base + k] = start + k;
+            for (int k = 0; k < len; k++) sh_col[wv][sub][base + k] = (unsigned char)(lane & 31);
         __builtin_amdgcn_wave_barrier();
     } else {
         column_setup<T>(g, cs[0], lane, offsets, start, len);
@@ -628,13 +629,13 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         sh_start[wv][lane] = start;
         sh_base[wv][lane] = base;
         if (totals[ia] <= NBL_ENT_CAP)
-            for (int k = 0; k < len; k++) sh_ent[wv][0][base + k] = start + k;
+            for (int k = 0; k < len; k++) sh_col[wv][0][base + k] = (unsigned char)lane;
         __builtin_amdgcn_wave_barrier();
     }
     const int total = totals[ia];
     const bool flat = total <= NBL_ENT_CAP;       // wave-uniform
     const int so = paired ? ia * 32 : 0;          // the atom's part of sh_start / sh_base
-    const int* const ents = sh_ent[wv][paired ? ia : 0];
+    const unsigned char* const cols = sh_col[wv][paired ? ia : 0];
 
     int cnt = 0;
     const size_t rowi = (size_t)p * umax;
@@ -653,7 +654,8 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             if (ci < total) {
                 int ent;
                 if (flat) {
-                    ent = ents[ci];
+                    const int col = so + cols[ci];
+                    ent = sh_start[wv][col] + (ci - sh_base[wv][col]);
                 } else {
                     // last column whose base is <= ci
                     int lo = 0, hi = nruns - 1;
