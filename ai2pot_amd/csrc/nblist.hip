@@ -561,7 +561,9 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     __shared__ unsigned char sh_col[NBL_BLOCK / 64][NBL_APW][NBL_ENT_CAP];   // column of each flat candidate
     extern __shared__ __align__(16) unsigned char sh_rows[];
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * NBL_APW;
+    // the wave's first position, in a scalar register: the loads of its atoms' indices and coordinates are then
+    // scalar loads
+    const int p0 = __builtin_amdgcn_readfirstlane((blockIdx.x * (NBL_BLOCK / 64) + wv) * NBL_APW);
     if (p0 >= g.N) return;                        // whole wave leaves together
     const int np = min(NBL_APW, g.N - p0);
     T* rb_rcs = nullptr;
