@@ -139,17 +139,23 @@ __global__ void coords_minmax_kernel(const Grid<T> g, const T* __restrict__ coor
             v[6 + a] = c[a];
             v[9 + a] = c[a];
         }
-        for (int i = 0; i < g.img_dim[0]; i++)
-            for (int j = 0; j < g.img_dim[1]; j++)
-                for (int k = 0; k < g.img_dim[2]; k++) {
+        // Extremes over the atom's images (structure.h:1018-1052 takes them over the whole supercell).  Rounded
+        // multiplication and addition are monotone in each operand, so image_coord is monotone in each image
+        // index, rising or falling with the sign of the lattice component: the extremes sit at the ends of
+        // the index ranges, and two images per axis give the same values as the loop over all of them.
 #pragma unroll
-                    for (int a = 0; a < 3; a++) {
-                        T s = image_coord(c[a], g.b[0][a], g.b[1][a], g.b[2][a], g.img_lo[0] + i,
-                                          g.img_lo[1] + j, g.img_lo[2] + k);
-                        if (s < v[a]) v[a] = s;
-                        if (s > v[3 + a]) v[3 + a] = s;
-                    }
-                }
+        for (int a = 0; a < 3; a++) {
+            int lo[3], hi[3];
+#pragma unroll
+            for (int w = 0; w < 3; w++) {
+                const int first = g.img_lo[w], last = g.img_lo[w] + g.img_dim[w] - 1;
+                const bool rising = g.b[w][a] >= (T)0;
+                lo[w] = rising ? first : last;
+                hi[w] = rising ? last : first;
+            }
+            v[a] = image_coord(c[a], g.b[0][a], g.b[1][a], g.b[2][a], lo[0], lo[1], lo[2]);
+            v[3 + a] = image_coord(c[a], g.b[0][a], g.b[1][a], g.b[2][a], hi[0], hi[1], hi[2]);
+        }
     }
 #pragma unroll
     for (int q = 0; q < 12; q++) {
