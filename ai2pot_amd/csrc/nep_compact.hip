@@ -545,11 +545,11 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         for (int i = 0; i < 9; i++) vals[1 + i] = active ? (double)vir[i] : 0.0;
         const int nv = a.want_virial ? 10 : 1;
 #pragma unroll
-        for (int i = 0; i < 10; i++) {
-            if (i >= nv) break;
-            const double v = wave_sum(vals[i]);
-            if (lane == 0) L.red[wv * 10 + i] = v;
-        }
+        for (int i = 0; i < 10; i++)
+            if (i < nv) {                          // wave-uniform
+                const double v = wave_sum(vals[i]);
+                if (lane == 0) L.red[wv * 10 + i] = v;
+            }
         __syncthreads();
         if (tid < nv) {
             double v = 0.0;
