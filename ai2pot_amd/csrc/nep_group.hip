@@ -172,11 +172,18 @@ __device__ __forceinline__ void load_tile(const NepArgs<T>& a, const SegArgs& se
                 x = p[0]; y = p[1]; z = p[2];
                 tj = types[nj];
                 if (seg.cursor && claim) {
-                    // fixed-capacity segments: the pair claims its entry here (a2p::PairCsr)
+                    // fixed-capacity segments: the pair claims its entry here (a2p::PairCsr), or takes the place
+                    // an earlier call on the same list recorded (no atomic then; the call that claims records)
                     const int tg = b * NF + nj;
-                    const int rk = atomicAdd(&seg.cursor[tg], 1);
-                    pos = rk < seg.cap ? tg * seg.cap + rk : seg.spare;
-                    if (rk >= seg.cap) atomicOr(a.status, ST_SEG_OVERFLOW);
+                    int rk;
+                    if (a.brank && a.ranks_valid) {
+                        rk = a.brank[pr];
+                    } else {
+                        rk = atomicAdd(&seg.cursor[tg], 1);
+                        if (a.brank) a.brank[pr] = rk;
+                    }
+                    pos = (unsigned)rk < (unsigned)seg.cap ? tg * seg.cap + rk : seg.spare;
+                    if ((unsigned)rk >= (unsigned)seg.cap) atomicOr(a.status, ST_SEG_OVERFLOW);
                 }
                 if ((unsigned)tj >= (unsigned)a.ntypes) { atomicOr(a.status, ST_BAD_TYPE); tj = 0; }
             }
@@ -573,7 +580,8 @@ int nep_group_run(const NepArgs<T>& a, size_t lds_bytes, T* etot, T* virial, hip
     int rc;
     if (a.force) {
         rc = pair_fixed_begin<T>(&csr, a.B, a.P, a.U, a.nghost, stream, a.force,
-                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T));
+                                 (size_t)a.B * (a.P + a.nghost) * 3 * sizeof(T), a.bincoming,
+                                 a.bincoming != nullptr && a.ranks_valid != 0);
         if (rc) return rc;
     }
     auto launch = [&](auto nr) {
