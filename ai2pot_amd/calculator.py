@@ -34,7 +34,9 @@ class NepCalculator:
         padded=False (gather only) skips the padded firstneigh / rcs arrays: the step then produces
         energy, forces and virial alone.  reorder_every: the gather path processes the atoms along a
         space-filling curve; the order is a locality hint only (results do not depend on it beyond
-        rounding), so it is recomputed every reorder_every rebuilds and kept in between.
+        rounding), so it is recomputed every reorder_every rebuilds and kept in between; reorder_every=0 processes the
+        atoms in the caller's order (for inputs that are already ordered in space: a crystal written cell by cell, atoms
+        kept sorted by the MD code), which makes the per-atom arrays and the padded rows sequential.
         sync_free: after the first rebuild (which synchronises), later rebuilds size their bin grid from that build's
         bound and never wait for the stream (a2p_nblist_sync_free); the step can then be captured into a HIP graph.
         If the atoms spread beyond the bound, check() raises and the next rebuild synchronises again."""
@@ -99,6 +101,7 @@ class NepCalculator:
         # systems stay with the lane-group kernel of the segment path
         self.path = "gather" if (can_gather and (path == "gather" or (path == "auto" and self.n >= 32768))) else "segments"
         self.padded = bool(padded) or self.path != "gather"
+        self.input_order = int(reorder_every) == 0
         self.reorder_every = max(1, int(reorder_every))
         self.sync_free = bool(sync_free)
         self._resync = False
@@ -106,6 +109,10 @@ class NepCalculator:
         if self.path == "gather":
             nbytes = L.a2p_nblist_compact_bytes(_c.c_int(n), _c.c_int(U), elem)
             self.compact = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            if self.input_order:
+                # the processing order is the first array of the buffer (csrc/compact_list.h): the caller's own
+                # order goes in once and every build is told to keep it
+                self.compact[:4 * n].view(torch.int32).copy_(torch.arange(n, dtype=torch.int32, device=dev))
             self._nbl_compact = L.a2p_nblist_build_compact_f32 if f32 else L.a2p_nblist_build_compact_f64
             self._efv_compact = L.a2p_nep_efv_compact_f32 if f32 else L.a2p_nep_efv_compact_f64
             if not self.padded:
@@ -142,7 +149,8 @@ class NepCalculator:
                                    _c.c_int(self.n), _c.c_double(self.rcut), _c.c_int(self.umax), _c.c_int(1),
                                    self.pbc.ctypes.data_as(_c.c_void_p),
                                    _c.c_int((1 if (self._have_list and self.padded) else 0) |
-                                            (2 if (self._have_list and (self._builds % self.reorder_every or capturing))
+                                            (2 if (self.input_order or
+                                                   (self._have_list and (self._builds % self.reorder_every or capturing)))
                                              else 0)),
                                    _c.c_double(m["rmax_radial"]), _c.c_double(m["rmax_angular"]),
                                    _vp(self.ilist), _vp(self.numneigh), _vp(self.firstneigh), _vp(self.rcs),

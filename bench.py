@@ -341,6 +341,28 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
         lean.check()
         extra["without_padded_arrays"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
                                               unit="atom-steps/s")
+        del lean
+        # the headline step (padded arrays included) with the atoms processed in the order they are given in
+        # instead of along the library's space-filling curve: the synthetic crystal is written cell by cell
+        inorder = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, sync_free=True,
+                                reorder_every=0)
+        inorder.rebuild(coords0, stream)
+
+        def inorder_step(k):
+            torch.add(coords0, disp_t, alpha=float(np.sin(0.37 * k)), out=coords)
+            return inorder.step(coords)
+        for k in range(args.warmup):
+            inorder_step(k)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            inorder_step(args.warmup + k)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        inorder.check()
+        extra["atoms_processed_in_input_order"] = dict(ms_per_step=dt * 1e3 / args.steps, value=n * args.steps / dt,
+                                                       unit="atom-steps/s")
+        del inorder
         if not via_ops:
             # the same step (padded arrays included) driven through the registered operators alone
             torch.ops.nblist.set_validate(False)

@@ -224,7 +224,9 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * cutoffs of the model; rcut_inner <= rcut_outer <= rcut).  update: bit 0 as for a2p_nblist_update_*
  * (the padded outputs hold an earlier result), bit 1 = keep the processing order that an earlier
  * build left in `compact` (it is a locality hint; atoms that moved a little are still well ordered)
- * instead of sorting again.  The five padded outputs are written,
+ * instead of sorting again.  The order is the first array of the buffer, int32[natoms], position ->
+ * atom; a caller whose atoms are already ordered in space may write the identity (or any permutation
+ * of the atoms) there and set bit 1 from the first build on.  The five padded outputs are written,
  * bit-identical to a2p_nblist_build_*, when they are given; pass all five NULL to skip them.
  * Needs umax % 8 == 0, natoms < 2^28, species < 16, 16-byte aligned firstneigh / rcs.
  *

@@ -150,6 +150,24 @@ def test_more_pairs_inside_the_angular_cutoff_than_slots(oracle, np_dtype):
     assert np.abs(out[1].astype(np.float64).sum(0)).max() < (1e-9 if np_dtype == np.float64 else 1e-2)
 
 
+def test_atoms_processed_in_the_callers_order(oracle):
+    """reorder_every=0: the processing order is the caller's (here a random one, the worst case for locality):
+    same lists, same results within the bars, across rebuilds."""
+    n = 500
+    lat, pos = synth.random_packed(n, [23.0, 22.0, 24.0], 2.1, 361)
+    ty = synth.rng_randint(362, n, 3)
+    m = synth.nep_model(seed=3306)
+    calc = _calc(m, lat, ty, n, np.float32, umax=96, path="gather", reorder_every=0)
+    for k in range(3):
+        p = pos + 0.02 * k * np.sin(np.arange(3 * n).reshape(n, 3))
+        out = _step(calc, p, np.float32)
+        ref = oracle.nblist(lat.astype(np.float32), ty, p.astype(np.float32), 7.0, 96)
+        assert np.array_equal(calc.numneigh.cpu().numpy(), ref[2])
+        assert np.array_equal(calc.firstneigh.cpu().numpy(), ref[3])
+        assert np.array_equal(calc.compact[:4 * n].cpu().numpy().view(np.int32), np.arange(n))
+        _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float32), np.float32)
+
+
 def test_gather_equals_segments_and_is_reproducible(oracle):
     """fp32, 42,592 atoms (not a multiple of 256): the gather and the segment path agree within the fp32
     bars, each run of the gather gives the same bits, and skipping the padded arrays changes nothing."""
