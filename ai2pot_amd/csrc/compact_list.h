@@ -23,6 +23,9 @@ constexpr int CL_TILE = 64;            // positions per tile
 constexpr int CL_CHUNK = 8;            // slots per chunk
 constexpr int CL_TYPE_SHIFT = 28;      // bits = index | species << 28
 constexpr int CL_INDEX_MASK = (1 << CL_TYPE_SHIFT) - 1;
+// Inside the list build only: set in the index word of a neighbour that is a periodic image (not the atom in
+// the cell itself); finished entries do not carry it.  Atom indices therefore stay below 2^27.
+constexpr int CL_IMAGE_BIT = 1 << 27;
 
 struct CompactLayout {
     int natoms, umax, npad, nch, ntiles;
@@ -31,7 +34,7 @@ struct CompactLayout {
 
 inline bool compact_supported(int natoms, int umax)
 {
-    return natoms > 0 && natoms <= CL_INDEX_MASK && umax >= CL_CHUNK && umax % CL_CHUNK == 0;
+    return natoms > 0 && natoms < CL_IMAGE_BIT && umax >= CL_CHUNK && umax % CL_CHUNK == 0;
 }
 
 inline CompactLayout compact_layout(int natoms, int umax, size_t elem)

@@ -207,11 +207,12 @@ __global__ void minmax_finish_kernel(const T* __restrict__ partial, int nblocks,
 // ---- 1b. bin grid from the extents, on the device (builds that do not read the extents back) ----------
 // The arithmetic of find_pl_info4nblist and of the bin counts (structure.h:1013-1061, binLinkedList.h:685-688) as
 // the host does it in the synchronised build, in T with correctly rounded operations.  The box must fit the
-// bound the host sized its launches and scratch arrays for: otherwise (or if an extent is not finite) the box
+// bound the host sized its launches and scratch arrays for, and its coordinates the bound the host assumed:
+// otherwise (or if an extent is not finite) the box
 // is made empty, so that no kernel indexes beyond the bound, and ST_GRID_BOUND is raised.
 template <typename T>
 __global__ void grid_setup_kernel(const Grid<T> g, const T* __restrict__ ext, GridDyn<T>* __restrict__ gd, int cap0,
-                                  int cap1, int cap2, int* __restrict__ status)
+                                  int cap1, int cap2, double big_bound, int* __restrict__ status)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     const int cap[3] = {cap0, cap1, cap2};
@@ -239,6 +240,8 @@ __global__ void grid_setup_kernel(const Grid<T> g, const T* __restrict__ ext, Gr
         gd->rdim[a] = rdim;
         gd->keep_lo[a] = (T)((double)mn + (double)rlo * (double)g.bin_size - slack);
         gd->keep_hi[a] = (T)((double)mn + (double)(rlo + rdim) * (double)g.bin_size + slack);
+        // the host sized the symmetry band of the compact lists for coordinates within big_bound
+        if (fmax(fabs((double)gd->keep_lo[a]), fabs((double)gd->keep_hi[a])) > big_bound) ok = false;
         nregion *= rdim > 0 ? rdim : 0;
     }
     if (!ok) {
@@ -356,11 +359,12 @@ __global__ void fill_kernel(const Grid<T> g_in, const T* __restrict__ x, const i
 // ---- 5. order inside a bin: descending supercell index (head insertion, binLinkedList.h:833) -
 // Afterwards only the atom behind a supercell entry matters (neighborList.h:561), so the sorted
 // indices are reduced modulo natoms here, once per entry instead of once per candidate pair.
-// With `types` the species of the atom rides in the bits above CL_TYPE_SHIFT (compact lists: the list
+// With `types` the species of the atom rides in the bits above CL_TYPE_SHIFT and CL_IMAGE_BIT marks the
+// periodic images (compact lists: the list
 // kernel then never gathers a neighbour's species).
 template <typename T>
 __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, T* __restrict__ s_rec, int natoms,
-                               const int* __restrict__ types, const GridDyn<T>* __restrict__ gd)
+                               const int* __restrict__ types, const GridDyn<T>* __restrict__ gd, int central)
 {
     if (gd) nbins = gd->nregion;                  // the launch covers the host's bound
     const int b = blockIdx.x * NBL_BLOCK + threadIdx.x;
@@ -386,7 +390,9 @@ __global__ void binsort_kernel(int nbins, const int* __restrict__ offsets, T* __
         int idx;
         entry_load(s_rec + (size_t)i * 4, x, y, z, idx);
         const int at = idx % natoms;
-        entry_store<T>(s_rec + (size_t)i * 4, x, y, z, types ? at | ((types[at] & 15) << CL_TYPE_SHIFT) : at);
+        // compact lists: the species, and whether this is an image outside the cell (image number != central)
+        entry_store<T>(s_rec + (size_t)i * 4, x, y, z,
+                       types ? at | ((types[at] & 15) << CL_TYPE_SHIFT) | (idx / natoms != central ? CL_IMAGE_BIT : 0) : at);
     }
 }
 
@@ -548,8 +554,49 @@ struct CompactEmit {
     int* n_inner;
     int nch;
     T split2, outer2;   // squares of the two cutoffs
+    T near_band;        // |d^2 - split2| within which the two ends of a pair may disagree about the side
     int write_rows;     // the padded outputs are wanted as well
 };
+// set in n_inner of a position that has an entry close to the inner cutoff, between the list kernel and
+// compact_symmetry_kernel, which clears it
+constexpr int CL_NEAR_FLAG = 1 << 30;
+
+// Squared length of the vector from the atom at c to the image of atom j it sees at c + d, formed so that the two
+// ends of a pair get the same bits: the difference of the two atoms' own coordinates (which changes sign exactly
+// when the ends are swapped) plus the lattice shift of the image (rebuilt from its indices, which also only
+// change sign).  The list's own vector d = image - c does not have this property: the image is rounded at the size
+// of the coordinates, differently for the two ends.  Used to put both entries of a pair on the same side of the
+// inner cutoff of the compact lists.
+template <typename T>
+__device__ T pair_symmetric_d2(const Grid<T>& g, const T* __restrict__ x, const T (&c)[3], T dx, T dy, T dz, int j)
+{
+    const T d[3] = {dx, dy, dz};
+    T e[3], v[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        e[a] = sub_rn(x[(size_t)j * 3 + a], c[a]);
+        v[a] = d[a] - e[a];                       // the image's shift, up to rounding
+    }
+    auto shift = [&](int ii, int jj, int kk, T (&s)[3]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int a = 0; a < 3; a++)
+            s[a] = add_rn(add_rn(mul_rn(g.b[0][a], (T)ii), mul_rn(g.b[1][a], (T)jj)), mul_rn(g.b[2][a], (T)kk));
+    };
+    T best = (T)INFINITY;
+    int bi = 0, bj = 0, bk = 0;
+    for (int ii = g.img_lo[0]; ii < g.img_lo[0] + g.img_dim[0]; ii++)
+        for (int jj = g.img_lo[1]; jj < g.img_lo[1] + g.img_dim[1]; jj++)
+            for (int kk = g.img_lo[2]; kk < g.img_lo[2] + g.img_dim[2]; kk++) {
+                T s[3];
+                shift(ii, jj, kk, s);
+                const T q = (v[0] - s[0]) * (v[0] - s[0]) + (v[1] - s[1]) * (v[1] - s[1]) + (v[2] - s[2]) * (v[2] - s[2]);
+                if (q < best) { best = q; bi = ii; bj = jj; bk = kk; }
+            }
+    T s[3];
+    shift(bi, bj, bk, s);
+    const T w0 = add_rn(e[0], s[0]), w1 = add_rn(e[1], s[1]), w2 = add_rn(e[2], s[2]);
+    return add_rn(add_rn(mul_rn(w0, w0), mul_rn(w1, w1)), mul_rn(w2, w2));
+}
 
 template <typename T, bool SORT, bool ROWBUF, bool RANK, bool COMPACT = false>
 __global__ void __launch_bounds__(NBL_BLOCK)
@@ -621,6 +668,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     } else {
         column_setup<T>(g, cs[0], lane, offsets, start, len);
     }
+    const T near_band = ce.near_band;
 #pragma unroll
     for (int ia = 0; ia < NBL_APW; ia++) {
     if (ia >= np) break;                          // wave-uniform
@@ -657,24 +705,23 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         T px[NBL_UNROLL], py[NBL_UNROLL], pz[NBL_UNROLL];
 #pragma unroll
         for (int u = 0; u < NBL_UNROLL; u++) {
-            const int ci = c0 + u * 64 + lane;
-            sj[u] = 0; px[u] = c[0]; py[u] = c[1]; pz[u] = c[2];
-            if (ci < total) {
-                int ent;
-                if (flat) {
-                    const int col = so + cols[ci];
-                    ent = sh_start[wv][col] + (ci - sh_base[wv][col]);
-                } else {
-                    // last column whose base is <= ci
-                    int lo = 0, hi = nruns - 1;
-                    while (lo < hi) {
-                        const int mid = (lo + hi + 1) >> 1;
-                        if (sh_base[wv][so + mid] <= ci) lo = mid; else hi = mid - 1;
-                    }
-                    ent = sh_start[wv][so + lo] + (ci - sh_base[wv][so + lo]);
+            // no branch around the load: a lane past the end of the list reads the last candidate again and
+            // drops it below, and the loads of the trip's chunks stay back to back
+            const int ci = min(c0 + u * 64 + lane, total - 1);
+            int ent;
+            if (flat) {
+                const int col = so + cols[ci];
+                ent = sh_start[wv][col] + (ci - sh_base[wv][col]);
+            } else {
+                // last column whose base is <= ci
+                int lo = 0, hi = nruns - 1;
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (sh_base[wv][so + mid] <= ci) lo = mid; else hi = mid - 1;
                 }
-                entry_load(s_rec + (size_t)ent * 4, px[u], py[u], pz[u], sj[u]);
+                ent = sh_start[wv][so + lo] + (ci - sh_base[wv][so + lo]);
             }
+            entry_load(s_rec + (size_t)ent * 4, px[u], py[u], pz[u], sj[u]);
         }
         // RANK: the pair's place among the pairs that name the same neighbour, claimed here so that
         // the force kernels need no atomics; the answers are collected after the chunk's last claim
@@ -731,6 +778,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         __builtin_amdgcn_wave_barrier();
         const int used = min(cnt, umax);
         int n_outer = 0, n_inner = 0;
+        T nearest = (T)INFINITY;                  // |d^2 - split^2| of the lane's entry closest to the inner cutoff
         // slot e of this position sits at  base + (e / 8) * (64 * 8 * 4) + (e % 8) * 4  values
         T* const base = ce.entries + compact_slot_offset(ce.nch, __builtin_amdgcn_readfirstlane(pos), 0);
         for (int e0 = 0; e0 < used; e0 += 64) {
@@ -738,10 +786,18 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             const bool have = e < used;
             const int ee = have ? e : 0;
             const T dx = rb_rcs[ee * 3 + 0], dy = rb_rcs[ee * 3 + 1], dz = rb_rcs[ee * 3 + 2];
-            const int bits = rb_first[ee];
+            const int word = rb_first[ee];
+            const int bits = word & ~CL_IMAGE_BIT;
             const T d2 = dx * dx + dy * dy + dz * dz;
             const bool in_outer = have && d2 <= ce.outer2;
             const bool is_inner = in_outer && d2 <= ce.split2;
+            // Both entries of a pair must fall on the same side of the inner cutoff (the force kernels treat the
+            // two classes by different routes), but the two ends see vectors that differ by the rounding of their
+            // images (a pair of atoms in the cell itself has exactly opposite vectors).  A position with an image
+            // inside a band around the cutoff several times wider than that rounding is flagged for
+            // compact_symmetry_kernel, which settles such entries by a squared distance both ends form
+            // bit-identically; outside the band the two ends agree anyway.
+            nearest = fmin(nearest, (in_outer && (word & CL_IMAGE_BIT)) ? fabs(d2 - ce.split2) : nearest);
             const bool is_outer = in_outer && !is_inner;
             const unsigned long long mi = __ballot(is_inner), mo = __ballot(is_outer);
             const unsigned long long below = (1ull << lane) - 1ull;
@@ -752,13 +808,14 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             n_inner += __popcll(mi);
             n_outer += __popcll(mo);
         }
+        const bool any_near = __ballot(nearest <= near_band) != 0ull;
         if (lane == 0) {
             ce.n_outer[pos] = n_outer;
-            ce.n_inner[pos] = n_inner;
+            ce.n_inner[pos] = n_inner | (any_near ? CL_NEAR_FLAG : 0);         // the flag: for compact_symmetry_kernel
         }
         // the padded row lists plain indices
         if (rows)
-            for (int e = lane; e < used; e += 64) rb_first[e] &= CL_INDEX_MASK;
+            for (int e = lane; e < used; e += 64) rb_first[e] &= CL_IMAGE_BIT - 1;
     }
     if (ROWBUF && rows) {
         __builtin_amdgcn_wave_barrier();
@@ -791,6 +848,87 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
     start = nstart;
     len = nlen;
     __builtin_amdgcn_wave_barrier();              // the LDS arrays are reused by the next atom
+    }
+}
+
+// ---- 6b. compact lists: both entries of a pair on the same side of the inner cutoff ---------------------
+// A wavefront looks at the flags of 64 positions and works through the flagged ones, one at a time.  It reads
+// such a position's entries 64 at a time, first the class beyond the cutoff, then the class inside; an entry
+// within the band takes the side its symmetric squared distance gives; entries that stay are written back in
+// order (compacting in place: a write never passes the reads of its own trip), entries that change sides wait
+// in LDS and are appended to their new class at the end.
+template <typename T>
+__global__ void __launch_bounds__(NBL_BLOCK)
+compact_symmetry_kernel(const Grid<T> g_in, const GridDyn<T>* __restrict__ gd, const T* __restrict__ x,
+                        const CompactEmit<T> ce, int umax)
+{
+    extern __shared__ __align__(16) unsigned char sh_move[];     // per wave: umax entries of 4 values
+    const Grid<T> g = with_dyn(g_in, gd);
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T* const mv = (T*)sh_move + (size_t)wv * umax * 4;
+    const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * 64;
+    const int mine = p0 + lane < g.N ? ce.n_inner[p0 + lane] : 0;
+    unsigned long long todo = __ballot((mine & CL_NEAR_FLAG) != 0);
+    if (todo == 0ull) return;                     // whole wave
+    const T band = ce.near_band;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    for (; todo != 0ull; todo &= todo - 1ull) {
+        const int pos = p0 + __builtin_ctzll(todo);
+        const int atom = ce.order[pos];
+        const T c[3] = {x[(size_t)atom * 3], x[(size_t)atom * 3 + 1], x[(size_t)atom * 3 + 2]};
+        const int n_outer = ce.n_outer[pos], n_inner = ce.n_inner[pos] & ~CL_NEAR_FLAG;
+        T* const base = ce.entries + compact_slot_offset(ce.nch, pos, 0);
+        auto slot = [&](int e) __attribute__((always_inline)) {
+            return base + (((unsigned)e >> 3) << 11) + (((unsigned)e & 7u) << 2);
+        };
+        int kept[2] = {0, 0}, moved[2] = {0, 0};   // by the class an entry came from: 0 beyond the cutoff, 1 inside
+        // entries that change sides: those from beyond the cutoff from the front of mv, the others from its back
+#pragma unroll
+        for (int cls = 0; cls < 2; cls++) {
+            const int count = cls ? n_inner : n_outer;
+            for (int e0 = 0; e0 < count; e0 += 64) {
+                const int e = e0 + lane;
+                const bool have = e < count;
+                T dx = (T)0, dy = (T)0, dz = (T)0;
+                int bits = 0;
+                if (have) entry_load(slot(cls ? umax - 1 - e : e), dx, dy, dz, bits);
+                const T d2 = dx * dx + dy * dy + dz * dz;
+                bool inside = cls != 0;
+                if (have && fabs(d2 - ce.split2) <= band)
+                    inside = pair_symmetric_d2<T>(g, x, c, dx, dy, dz, bits & CL_INDEX_MASK) <= ce.split2;
+                const bool stay = have && inside == (cls != 0), go = have && !stay;
+                const unsigned long long ms = __ballot(stay), mg = __ballot(go);
+                if (stay) {
+                    const int k = kept[cls] + __popcll(ms & below);
+                    entry_store<T>(slot(cls ? umax - 1 - k : k), dx, dy, dz, bits);
+                }
+                if (go) {
+                    const int k = moved[cls] + __popcll(mg & below);
+                    entry_store<T>(mv + (size_t)(cls ? umax - 1 - k : k) * 4, dx, dy, dz, bits);
+                }
+                kept[cls] += __popcll(ms);
+                moved[cls] += __popcll(mg);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        // entries that came from beyond the cutoff join the class inside, and the other way round
+        for (int k = lane; k < moved[0]; k += 64) {
+            T dx, dy, dz;
+            int bits;
+            entry_load(mv + (size_t)k * 4, dx, dy, dz, bits);
+            entry_store<T>(slot(umax - 1 - (kept[1] + k)), dx, dy, dz, bits);
+        }
+        for (int k = lane; k < moved[1]; k += 64) {
+            T dx, dy, dz;
+            int bits;
+            entry_load(mv + (size_t)(umax - 1 - k) * 4, dx, dy, dz, bits);
+            entry_store<T>(slot(kept[0] + k), dx, dy, dz, bits);
+        }
+        if (lane == 0) {
+            ce.n_outer[pos] = kept[0] + moved[1];
+            ce.n_inner[pos] = kept[1] + moved[0];
+        }
+        __builtin_amdgcn_wave_barrier();          // mv is reused by the wave's next position
     }
 }
 
@@ -1012,6 +1150,7 @@ struct GridBound {
     int device = -1, N = 0, is_cart = 0, pbc[3] = {0, 0, 0};
     double lattice[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0}, rcut = 0;
     int rdim[3] = {0, 0, 0};
+    double big = 0;    // largest |coordinate| of the box kept by that build
 };
 thread_local GridBound g_bound;
 thread_local int g_sync_free = 0;
@@ -1112,20 +1251,24 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                            (long long)N * g.nimg * (long long)(4 * sizeof(T)) <= (2ll << 30);
     GridDyn<T>* gd = nullptr;
     long long nregion = 1;
+    double big_coord = 0;                               // bound of the coordinates the build keeps
     if (sync_free) {
         int cap[3];
+        int grow = 0;
         for (int a = 0; a < 3; a++) {
             cap[a] = g_bound.rdim[a] + std::max(2, g_bound.rdim[a] / 8);
             g.rdim[a] = cap[a];                         // host copies of the box serve launch and scratch sizes only
             nregion *= cap[a];
+            grow = std::max(grow, cap[a] - g_bound.rdim[a]);
         }
+        big_coord = g_bound.big + (double)(grow + 2) * (double)g.bin_size;   // the box cannot have moved further
         A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID, "nblist: %lld bins around the centre atoms", nregion);
         void* wsG = nullptr;
         rc = ws_get(WS_GRID, 256, &wsG);
         if (rc) return rc;
         gd = (GridDyn<T>*)wsG;
         hipLaunchKernelGGL(grid_setup_kernel<T>, dim3(1), dim3(64), 0, stream, g, (const T*)ext_dev, gd, cap[0], cap[1],
-                           cap[2], status);
+                           cap[2], big_coord, status);
     } else {
         T ext[12];
         A2P_HIP_CHECK(hipMemcpyAsync(ext, ext_dev, sizeof(ext), hipMemcpyDeviceToHost, stream));
@@ -1159,6 +1302,9 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID,
                     "nblist: %lld bins around the centre atoms; are the coordinates far outside the cell?",
                     nregion);
+        for (int a = 0; a < 3; a++)
+            big_coord = std::max(big_coord, std::max(std::fabs((double)g.keep_lo[a]), std::fabs((double)g.keep_hi[a])));
+        g_bound.big = big_coord;
         g_bound.valid = true;
         g_bound.device = device; g_bound.N = N; g_bound.is_cart = is_cart; g_bound.rcut = (double)g.rcut;
         for (int a = 0; a < 3; a++) { g_bound.pbc[a] = pbc[a] ? 1 : 0; g_bound.rdim[a] = g.rdim[a]; }
@@ -1226,7 +1372,8 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     prof_end(stream);
     prof_begin("nbl_binsort", stream);
     hipLaunchKernelGGL(binsort_kernel<T>, dim3(ceil_div(nregion, NBL_BLOCK)), dim3(NBL_BLOCK), 0, stream,
-                       (int)nregion, offsets, s_rec, g.N, co ? types : (const int*)nullptr, (const GridDyn<T>*)gd);
+                       (int)nregion, offsets, s_rec, g.N, co ? types : (const int*)nullptr, (const GridDyn<T>*)gd,
+                       ((-g.img_lo[0]) * g.img_dim[1] + (-g.img_lo[1])) * g.img_dim[2] + (-g.img_lo[2]));
     prof_end(stream);
     CompactEmit<T> ce{};
     if (co) {
@@ -1271,6 +1418,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         ce.split2 = (T)co->split * (T)co->split;
         ce.outer2 = (T)co->outer * (T)co->outer;
         ce.write_rows = want_rows ? 1 : 0;
+        {
+            // the two ends of a pair see vectors that differ by the rounding of their images (three roundings at the
+            // size of the coordinates): the band is 16 such roundings wide
+            const double dr = 16.0 * (sizeof(T) == 4 ? 1.1920929e-7 : 2.220446049250313e-16) * big_coord;
+            ce.near_band = (T)(2.0 * co->split * dr + dr * dr);
+        }
     }
     const int list_blocks = ceil_div(N, (NBL_BLOCK / 64) * NBL_APW);
     prof_begin("nbl_lists", stream);
@@ -1302,6 +1455,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                            types, offsets, s_rec, umax, ilist, numneigh, firstneigh, rcs, types_out, keys,
                            status, update, nullptr, nullptr, CompactEmit<T>{}, (const GridDyn<T>*)gd);
     prof_end(stream);
+    if (co) {
+        prof_begin("nbl_symmetry", stream);
+        hipLaunchKernelGGL(compact_symmetry_kernel<T>, dim3(ceil_div(N, NBL_BLOCK)), dim3(NBL_BLOCK), (size_t)(NBL_BLOCK / 64) * umax * 4 * sizeof(T),
+                           stream, g, (const GridDyn<T>*)gd, (const T*)x, ce, umax);
+        prof_end(stream);
+    }
     if (sort) {
         prof_begin("nbl_sort_rows", stream);
         hipLaunchKernelGGL(sort_rows_kernel<T>, dim3(ceil_div(N, 64)), dim3(64), 0, stream, N, umax, numneigh,

@@ -228,7 +228,7 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * atom; a caller whose atoms are already ordered in space may write the identity (or any permutation
  * of the atoms) there and set bit 1 from the first build on.  The five padded outputs are written,
  * bit-identical to a2p_nblist_build_*, when they are given; pass all five NULL to skip them.
- * Needs umax % 8 == 0, natoms < 2^28, species < 16, 16-byte aligned firstneigh / rcs.
+ * Needs umax % 8 == 0, natoms < 2^27, species < 16, 16-byte aligned firstneigh / rcs.
  *
  * a2p_nep_efv_compact_*: energy, forces and virial of the structure from that buffer.  The list
  * names every pair from both ends, so F_i = sum_j (g_ij - g_ji) (nep.h:468-515 scatters the same terms).
