@@ -168,9 +168,10 @@ def test_atoms_processed_in_the_callers_order(oracle):
         _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float32), np.float32)
 
 
-def test_pairs_across_the_cell_boundary_at_the_angular_cutoff(oracle):
-    """fp32, a 300 A cell: 240 isolated pairs that reach across the periodic boundary at distances within a few
-    1e-4 A of the angular cutoff.  The two ends of such a pair see distance vectors that differ in the last bits
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64])
+def test_pairs_across_the_cell_boundary_at_the_angular_cutoff(oracle, np_dtype):
+    """A 300 A cell: 240 isolated pairs that reach across the periodic boundary at distances within a few
+    roundings of the coordinates of the angular cutoff.  The two ends of such a pair see distance vectors that differ in the last bits
     (their images are rounded at the size of the coordinates), so each end alone could put the pair on a different
     side of the cutoff; the lists must put both entries in the same class, and the forces must match the oracle."""
     L, ra = 300.0, 4.0
@@ -178,7 +179,7 @@ def test_pairs_across_the_cell_boundary_at_the_angular_cutoff(oracle):
     ya = 10.0 + 18.0 * (k % 16)
     za = 10.0 + 18.0 * (k // 16)
     xa = 0.25 + 0.01 * (k % 7)
-    delta = (k - 120) * 4.0e-6
+    delta = (k - 120) * (4.0e-6 if np_dtype == np.float32 else 8.0e-15)
     pos = np.zeros((480, 3))
     pos[0::2] = np.stack([xa, ya, za], 1)
     pos[1::2] = np.stack([L - (ra - xa) + delta, ya + 0.0, za + 0.0], 1)
@@ -186,11 +187,11 @@ def test_pairs_across_the_cell_boundary_at_the_angular_cutoff(oracle):
     lat = np.diag([L, L, L]).astype(np.float64)
     ty = synth.rng_randint(372, n, 3)
     m = synth.nep_model(seed=3307)
-    calc = _calc(m, lat, ty, n, np.float32, umax=16, path="gather")
-    out = _step(calc, pos, np.float32)
-    ref = oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 7.0, 16)
+    calc = _calc(m, lat, ty, n, np_dtype, umax=16, path="gather")
+    out = _step(calc, pos, np_dtype)
+    ref = oracle.nblist(lat.astype(np_dtype), ty, pos.astype(np_dtype), 7.0, 16)
     assert np.array_equal(calc.numneigh.cpu().numpy(), ref[2]) and ref[2].max() == 1
-    outer, inner = _decode_compact(calc, np.float32)
+    outer, inner = _decode_compact(calc, np_dtype)
     n_in = sum(len(inner[a]) for a in range(n))
     assert 0 < n_in < n                                       # the pairs straddle the cutoff
     for a in range(n):
@@ -198,8 +199,8 @@ def test_pairs_across_the_cell_boundary_at_the_angular_cutoff(oracle):
             assert any(e[0] == a for e in inner[j]), (a, j)
         for (j, _, _, _, _) in outer[a]:
             assert any(e[0] == a for e in outer[j]), (a, j)
-    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float32), np.float32)
-    assert np.abs(out[1].astype(np.float64).sum(0)).max() < 1e-4
+    _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
+    assert np.abs(out[1].astype(np.float64).sum(0)).max() < (1e-4 if np_dtype == np.float32 else 1e-12)
 
 
 def test_gather_equals_segments_and_is_reproducible(oracle):
