@@ -4,7 +4,7 @@
 //
 // Atoms are processed in a space-filling order: position p handles atom order[p].  64 consecutive
 // positions form a tile (one wavefront).  A position owns umax entry slots of 4 values each,
-// [x y z bits], bits = neighbour index | neighbour species << 28.  Neighbours beyond the inner
+// [x y z bits], bits = neighbour's position in the processing order | neighbour species << 28.  Neighbours beyond the inner
 // (angular) cutoff fill the slots from 0 upwards, neighbours inside it from umax-1 downwards;
 // neighbours beyond the outer (radial) cutoff are left out.  The slots are stored in chunks of 8:
 //     slot e of position p  ->  entry ((tile * NCH + e / 8) * 64 + p % 64) * 8 + e % 8,   NCH = umax / 8
@@ -21,7 +21,7 @@ namespace a2p {
 
 constexpr int CL_TILE = 64;            // positions per tile
 constexpr int CL_CHUNK = 8;            // slots per chunk
-constexpr int CL_TYPE_SHIFT = 28;      // bits = index | species << 28
+constexpr int CL_TYPE_SHIFT = 28;      // bits = position | species << 28
 constexpr int CL_INDEX_MASK = (1 << CL_TYPE_SHIFT) - 1;
 // Inside the list build only: set in the index word of a neighbour that is a periodic image (not the atom in
 // the cell itself); finished entries do not carry it.  Atom indices therefore stay below 2^27.

@@ -408,13 +408,15 @@ __device__ __forceinline__ unsigned spread3(unsigned v)      // 10 bits -> every
 }
 
 // xs[position] = x[order[position]]: the list kernel then reads its atoms' coordinates without first
-// waiting for the order
+// waiting for the order; and the inverse of the order
 template <typename T>
-__global__ void sorted_coords_kernel(int N, const T* __restrict__ x, const int* __restrict__ order, T* __restrict__ xs)
+__global__ void sorted_coords_kernel(int N, const T* __restrict__ x, const int* __restrict__ order, T* __restrict__ xs,
+                                     int* __restrict__ inv)
 {
     const int p = blockIdx.x * NBL_BLOCK + threadIdx.x;
     if (p >= N) return;
     const int at = min(max(order[p], 0), N - 1);
+    inv[at] = p;                                  // atom -> position: the index the compact entries carry
     xs[(size_t)p * 3 + 0] = x[(size_t)at * 3 + 0];
     xs[(size_t)p * 3 + 1] = x[(size_t)at * 3 + 1];
     xs[(size_t)p * 3 + 2] = x[(size_t)at * 3 + 2];
@@ -549,6 +551,7 @@ template <typename T>
 struct CompactEmit {
     const int* order;   // position -> atom
     const T* xs;        // [natoms][3] Cartesian coordinates in processing order
+    const int* inv;     // [natoms] atom -> position; every value in [0, natoms)
     T* entries;
     int* n_outer;
     int* n_inner;
@@ -772,6 +775,10 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         if (rows) numneigh[p] = cnt;             // ilist and types_out: count_kernel
         if (cnt > umax) atomicOr(status, ST_NEIGH_OVERFLOW);
     }
+    // the first 64 entries of the row: their compact stores wait until the padded row has gone out (below)
+    T first_dx = (T)0, first_dy = (T)0, first_dz = (T)0;
+    int first_bits = 0, first_slot = -1;
+    T* compact_base = nullptr;
     if (COMPACT) {
         // the row's entries, 64 at a time: class by distance, place by ballot prefix, one 16-byte
         // (fp32) store per entry; 8 consecutive slots of a position are contiguous in memory
@@ -781,13 +788,18 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         T nearest = (T)INFINITY;                  // |d^2 - split^2| of the lane's entry closest to the inner cutoff
         // slot e of this position sits at  base + (e / 8) * (64 * 8 * 4) + (e % 8) * 4  values
         T* const base = ce.entries + compact_slot_offset(ce.nch, __builtin_amdgcn_readfirstlane(pos), 0);
+        compact_base = base;
         for (int e0 = 0; e0 < used; e0 += 64) {
             const int e = e0 + lane;
             const bool have = e < used;
             const int ee = have ? e : 0;
             const T dx = rb_rcs[ee * 3 + 0], dy = rb_rcs[ee * 3 + 1], dz = rb_rcs[ee * 3 + 2];
             const int word = rb_first[ee];
-            const int bits = word & ~CL_IMAGE_BIT;
+            // The entry names its neighbour by position in the processing order (what the force kernels index their
+            // per-atom arrays with), the record and the padded row by atom: one gather per entry.  The first 64
+            // entries (most rows have no more) do not wait for the answer here: they are stored after the padded
+            // row.  Every value of the inverse is a valid position (see where it is allocated).
+            const int bits = ce.inv[word & (CL_IMAGE_BIT - 1)] | (word & ~CL_INDEX_MASK);
             const T d2 = dx * dx + dy * dy + dz * dz;
             const bool in_outer = have && d2 <= ce.outer2;
             const bool is_inner = in_outer && d2 <= ce.split2;
@@ -804,7 +816,11 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             int slot = -1;
             if (is_inner) slot = umax - 1 - (n_inner + __popcll(mi & below));
             if (is_outer) slot = n_outer + __popcll(mo & below);
-            if (slot >= 0) entry_store<T>(base + (((unsigned)slot >> 3) << 11) + (((unsigned)slot & 7u) << 2), dx, dy, dz, bits);
+            if (e0 == 0) {                        // wave-uniform
+                first_dx = dx; first_dy = dy; first_dz = dz; first_bits = bits; first_slot = slot;
+            } else if (slot >= 0) {
+                entry_store<T>(base + (((unsigned)slot >> 3) << 11) + (((unsigned)slot & 7u) << 2), dx, dy, dz, bits);
+            }
             n_inner += __popcll(mi);
             n_outer += __popcll(mo);
         }
@@ -845,6 +861,9 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         pad_fill(firstneigh + rowi, first_pad, last_pad, -1, lane);
         pad_fill(rcs + rowi * 3, first_pad * 3, last_pad * 3, (T)0, lane);
     }
+    if (COMPACT && first_slot >= 0)
+        entry_store<T>(compact_base + (((unsigned)first_slot >> 3) << 11) + (((unsigned)first_slot & 7u) << 2), first_dx,
+                       first_dy, first_dz, first_bits);
     start = nstart;
     len = nlen;
     __builtin_amdgcn_wave_barrier();              // the LDS arrays are reused by the next atom
@@ -874,8 +893,7 @@ compact_symmetry_kernel(const Grid<T> g_in, const GridDyn<T>* __restrict__ gd, c
     const unsigned long long below = (1ull << lane) - 1ull;
     for (; todo != 0ull; todo &= todo - 1ull) {
         const int pos = p0 + __builtin_ctzll(todo);
-        const int atom = ce.order[pos];
-        const T c[3] = {x[(size_t)atom * 3], x[(size_t)atom * 3 + 1], x[(size_t)atom * 3 + 2]};
+        const T c[3] = {ce.xs[(size_t)pos * 3], ce.xs[(size_t)pos * 3 + 1], ce.xs[(size_t)pos * 3 + 2]};
         const int n_outer = ce.n_outer[pos], n_inner = ce.n_inner[pos] & ~CL_NEAR_FLAG;
         T* const base = ce.entries + compact_slot_offset(ce.nch, pos, 0);
         auto slot = [&](int e) __attribute__((always_inline)) {
@@ -895,7 +913,7 @@ compact_symmetry_kernel(const Grid<T> g_in, const GridDyn<T>* __restrict__ gd, c
                 const T d2 = dx * dx + dy * dy + dz * dz;
                 bool inside = cls != 0;
                 if (have && fabs(d2 - ce.split2) <= band)
-                    inside = pair_symmetric_d2<T>(g, x, c, dx, dy, dz, bits & CL_INDEX_MASK) <= ce.split2;
+                    inside = pair_symmetric_d2<T>(g, ce.xs, c, dx, dy, dz, bits & CL_INDEX_MASK) <= ce.split2;
                 const bool stay = have && inside == (cls != 0), go = have && !stay;
                 const unsigned long long ms = __ballot(stay), mg = __ballot(go);
                 if (stay) {
@@ -1153,6 +1171,12 @@ struct GridBound {
     double big = 0;    // largest |coordinate| of the box kept by that build
 };
 thread_local GridBound g_bound;
+// where the last inverse of a processing order was written (the workspace is per process, like this record)
+struct InverseAt {
+    const void* ptr = nullptr;
+    int N = 0, device = -1;
+};
+InverseAt g_inverse;
 thread_local int g_sync_free = 0;
 
 template <typename T>
@@ -1220,13 +1244,14 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     // workspace A: x[N*3] | partial[nblocks*12] | ext[12]
     const int nblocks = ceil_div(N, NBL_BLOCK);
     void* wsA = nullptr;
-    size_t bytesA = ((size_t)N * 3 * (co ? 2 : 1) + (size_t)nblocks * 12 + 16) * sizeof(T);
+    size_t bytesA = ((size_t)N * 3 * (co ? 2 : 1) + (size_t)nblocks * 12 + 16) * sizeof(T) + (co ? (size_t)N * sizeof(int) : 0);
     int rc = ws_get(WS_NBL_A, bytesA, &wsA);
     if (rc) return rc;
     T* x = (T*)wsA;
     T* partial = x + (size_t)N * 3;
     T* ext_dev = partial + (size_t)nblocks * 12;
     T* xs = ext_dev + 16;                               // coordinates in processing order (compact lists)
+    int* inv = (int*)(xs + (size_t)N * 3);              // ... and the inverse of the order
     void* flags = nullptr;
     rc = ws_get(WS_FLAGS, 64, &flags);
     if (rc) return rc;
@@ -1243,6 +1268,18 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     // the bin box: read back from the extents, or bounded by the box of the last synchronised build of this structure
     int device = 0;
     A2P_HIP_CHECK(hipGetDevice(&device));
+    {
+        // The list kernel uses values of the inverse unchecked, and an order that is no permutation (the caller may
+        // write the order) leaves some of them unwritten: the array starts from zeros whenever its memory may hold
+        // anything but an earlier inverse for the same number of atoms.
+        if (!co) {
+            g_inverse.ptr = nullptr;                   // this call's own arrays take the place
+        } else if (g_inverse.ptr != (const void*)inv || g_inverse.N != N || g_inverse.device != device) {
+            rc = fill_zero(inv, (size_t)N * sizeof(int), stream);
+            if (rc) return rc;
+            g_inverse.ptr = inv; g_inverse.N = N; g_inverse.device = device;
+        }
+    }
     bool same = g_bound.valid && g_bound.device == device && g_bound.N == N && g_bound.is_cart == is_cart &&
                 g_bound.rcut == (double)g.rcut;
     for (int a = 0; a < 3 && same; a++) same = g_bound.pbc[a] == (pbc[a] ? 1 : 0);
@@ -1412,9 +1449,10 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         ce.nch = cv.nch;
         prof_begin("nbl_order", stream);
         hipLaunchKernelGGL(sorted_coords_kernel<T>, pair_grid, dim3(NBL_BLOCK), 0, stream, N, (const T*)x,
-                           (const int*)cv.order, xs);
+                           (const int*)cv.order, xs, inv);
         prof_end(stream);
         ce.xs = xs;
+        ce.inv = inv;
         ce.split2 = (T)co->split * (T)co->split;
         ce.outer2 = (T)co->outer * (T)co->outer;
         ce.write_rows = want_rows ? 1 : 0;

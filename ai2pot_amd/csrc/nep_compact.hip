@@ -46,6 +46,7 @@ struct GatherArgs {
     T rr, ra;
     CompactView<T> cv;
     const int* types;     // [natoms]
+    // the next four are indexed by position in the processing order, like the index field of the list entries
     T* rcc;               // [natoms][NTC * KC] radial coefficients contracted with dE/dq
     T* slots;             // [NSLOT][natoms][4] derivatives handed to the neighbour, by place
     T* overflow;          // [natoms][3] the same for places >= NSLOT, summed with atomics (zero on entry)
@@ -455,8 +456,8 @@ nep_adjoint_kernel(const GatherArgs<T> a)
         for (int k = 0; k < KC; k++) L.acc[(t * KC + k) * CB + tid] = cc[k];
         if (active) {
             T lo[4] = {cc[0], cc[1], cc[2], cc[3]}, hi[4] = {cc[4], cc[5], cc[6], cc[7]};
-            st4(a.rcc + ((size_t)atom * NTC + t) * KC, lo);
-            st4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi);
+            st4(a.rcc + ((size_t)p * NTC + t) * KC, lo);
+            st4(a.rcc + ((size_t)p * NTC + t) * KC + 4, hi);
         }
     }
 
@@ -583,7 +584,7 @@ nep_gather_kernel(const GatherArgs<T> a)
     T cc0[KC], cc1[KC], cc2[KC], cc3[KC];
     auto load_cc = [&](int t, T (&c)[KC]) __attribute__((always_inline)) {
         T lo[4] = {(T)0, (T)0, (T)0, (T)0}, hi[4] = {(T)0, (T)0, (T)0, (T)0};
-        if (active && t < NTC) { ld4(a.rcc + ((size_t)atom * NTC + t) * KC, lo); ld4(a.rcc + ((size_t)atom * NTC + t) * KC + 4, hi); }
+        if (active && t < NTC) { ld4(a.rcc + ((size_t)p * NTC + t) * KC, lo); ld4(a.rcc + ((size_t)p * NTC + t) * KC + 4, hi); }
 #pragma unroll
         for (int k = 0; k < 4; k++) { c[k] = lo[k]; c[4 + k] = hi[k]; }
     };
@@ -623,21 +624,21 @@ nep_gather_kernel(const GatherArgs<T> a)
 
     // what the neighbours inside the angular cutoff handed over: F_i -= sum_j g_ji
     if (active && a.force) {
-        const int n = a.incoming[atom];
+        const int n = a.incoming[p];
         FixedSum<T> sx, sy, sz;
         bool ok = true;
         for (int t = 0; t < min(n, NSLOT); t++) {
             T v[4];
-            ld4(a.slots + ((size_t)t * a.cv.natoms + atom) * 4, v);
+            ld4(a.slots + ((size_t)t * a.cv.natoms + p) * 4, v);
             ok = ok && fabs((double)v[0]) < kFixedSumLimit && fabs((double)v[1]) < kFixedSumLimit &&
                  fabs((double)v[2]) < kFixedSumLimit;
             sx.add(v[0]); sy.add(v[1]); sz.add(v[2]);
         }
         double ox = 0.0, oy = 0.0, oz = 0.0;
         if (n > NSLOT) {
-            ox = (double)a.overflow[(size_t)atom * 3 + 0];
-            oy = (double)a.overflow[(size_t)atom * 3 + 1];
-            oz = (double)a.overflow[(size_t)atom * 3 + 2];
+            ox = (double)a.overflow[(size_t)p * 3 + 0];
+            oy = (double)a.overflow[(size_t)p * 3 + 1];
+            oz = (double)a.overflow[(size_t)p * 3 + 2];
         }
         T* fo = a.force + (size_t)atom * 3;
         const double nan = __longlong_as_double(0x7ff8000000000000ll);

@@ -219,14 +219,16 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * a2p_nblist_build_compact_*: the build of a2p_nblist_build_* / a2p_nblist_update_* (sort = 0;
  * update as there) that ALSO cuts every row into the caller's `compact` buffer of
  * a2p_nblist_compact_bytes(natoms, umax, sizeof(T)) bytes: atoms in Morton order of their bins,
- * per atom the neighbours with r <= rcut_outer as 16-byte (fp32) entries [r_j - r_i, index |
- * species << 28], those with r <= rcut_inner kept apart from the rest (the radial and angular
+ * per atom the neighbours with r <= rcut_outer as 16-byte (fp32) entries [r_j - r_i, position |
+ * species << 28] (position: the neighbour's place in that order, which is what the force kernels index
+ * their per-atom arrays with), those with r <= rcut_inner kept apart from the rest (the radial and angular
  * cutoffs of the model; rcut_inner <= rcut_outer <= rcut).  update: bit 0 as for a2p_nblist_update_*
  * (the padded outputs hold an earlier result), bit 1 = keep the processing order that an earlier
  * build left in `compact` (it is a locality hint; atoms that moved a little are still well ordered)
  * instead of sorting again.  The order is the first array of the buffer, int32[natoms], position ->
  * atom; a caller whose atoms are already ordered in space may write the identity (or any permutation
- * of the atoms) there and set bit 1 from the first build on.  The five padded outputs are written,
+ * of the atoms) there and set bit 1 from the first build on (an array that is no permutation gives
+ * meaningless lists, inside bounds).  The five padded outputs are written,
  * bit-identical to a2p_nblist_build_*, when they are given; pass all five NULL to skip them.
  * Needs umax % 8 == 0, natoms < 2^27, species < 16, 16-byte aligned firstneigh / rcs.
  *

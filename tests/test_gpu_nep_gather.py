@@ -64,7 +64,8 @@ def _decode_compact(calc, np_dtype):
         a = int(order[p])
         so = slice(0, n_outer[p])
         si = slice(U - n_inner[p], U)
-        pack = lambda s: sorted(zip((bits[p, s] & ((1 << 28) - 1)).tolist(), (bits[p, s] >> 28).tolist(),
+        # an entry names its neighbour by position in the processing order
+        pack = lambda s: sorted(zip(order[bits[p, s] & ((1 << 28) - 1)].tolist(), (bits[p, s] >> 28).tolist(),
                                     ent[p, s, 0].tolist(), ent[p, s, 1].tolist(), ent[p, s, 2].tolist()))
         outer[a], inner[a] = pack(so), pack(si)
     return outer, inner
