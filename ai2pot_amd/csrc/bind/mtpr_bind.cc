@@ -3,8 +3,8 @@
 // set_ai2pot_path, mtpParamOp, linearMtpToEFVOp, linearMtpToEFOp, linearMtpToLossOp,
 // linearMtpToEFLossOp, linearMtpToEsitesOp (autograd to coeffs, linear_coeffs, type_bias only, as
 // src/linearMtpOp.cc:1732-1765, 4002-4027), linearMtpToDescriptorsOp, and the linear-solver
-// operators LinMatrixLinVectorOp and CoeffsSchmidtOrthOp.  The legacy mtpBasisOp is not part of
-// this build.
+// operators LinMatrixLinVectorOp and CoeffsSchmidtOrthOp, and the legacy mtpBasisOp (autograd to coeffs
+// and brcs, src/mtpBasisOp.cc:28-326).
 #include "mtp_bind_common.h"
 
 namespace {
@@ -276,6 +276,72 @@ variable_list mtp_descriptors(int64_t K, double scaling, const at::Tensor& coeff
     return {desc};
 }
 
+// The legacy basis operator (src/mtpBasisOp.cc:28-326): forward = the scalar moments of every row; backward =
+// one adjoint sweep per row from the incoming weights (a2p_mtp_basis_bwd_*), where the reference contracts
+// dense derivative arrays kept from its forward pass (mtpBasis.h:359-394).
+struct BasisFunction : public torch::autograd::Function<BasisFunction> {
+    static variable_list forward(AutogradContext* ctx, const at::Tensor& basic, const at::Tensor& times,
+                                 const at::Tensor& mapping, int64_t n_moms, int64_t nmus, int64_t ntypes, int64_t K,
+                                 double scaling, const at::Tensor& coeffs, const at::Tensor& binum,
+                                 const at::Tensor& bilist, const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh,
+                                 const at::Tensor& brcs, const at::Tensor& btypes, double rmax, double rmin)
+    {
+        at::Tensor type_map = at::zeros({ntypes}, binum.options());     // only its length is used
+        at::Tensor desc = mtp_descriptors(K, scaling, coeffs, n_moms, basic, times, mapping, nmus, binum, bilist,
+                                          bnumneigh, bfirstneigh, brcs.detach(), btypes, type_map, 0, rmax, rmin)[0];
+        ctx->save_for_backward({coeffs, basic, times, mapping, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes});
+        ctx->saved_data["K"] = K;
+        ctx->saved_data["scaling"] = scaling;
+        ctx->saved_data["n_moms"] = n_moms;
+        ctx->saved_data["nmus"] = nmus;
+        ctx->saved_data["ntypes"] = ntypes;
+        ctx->saved_data["rmax"] = rmax;
+        ctx->saved_data["rmin"] = rmin;
+        return {desc};
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads)
+    {
+        variable_list out(17);                   // one slot per forward argument after ctx
+        auto sv = ctx->get_saved_variables();
+        const at::Tensor &coeffs = sv[0], &brcs = sv[8];
+        // needs_input_grad counts the tensor arguments only: coeffs is the fourth, brcs the ninth
+        const bool want_c = ctx->needs_input_grad(3), want_r = ctx->needs_input_grad(8);
+        if (!want_c && !want_r) return out;
+        const int64_t K = ctx->saved_data["K"].toInt(), nmus = ctx->saved_data["nmus"].toInt(),
+                      ntypes = ctx->saved_data["ntypes"].toInt();
+        Batch s = check_batch(sv[4], sv[5], sv[6], sv[7], brcs, sv[9], 0);
+        a2p_bind::DeviceGuard guard(brcs);
+        PlanEntry plan = get_plan(brcs.device().index(), ctx->saved_data["n_moms"].toInt(), sv[1], sv[2], sv[3]);
+        auto opt = brcs.options();
+        at::Tensor g = grads[0].contiguous();
+        TORCH_CHECK(g.dim() == 3 && g.size(0) == s.B && g.size(1) == s.P && g.size(2) == plan.n_scalar,
+                    "grad of the basis values must be [B, P, alpha_scalar_moments]");
+        at::Tensor dr, dc;
+        if (want_r) dr = at::zeros({s.B, s.P, s.U, 3}, opt);
+        if (want_c) dc = at::zeros({s.B, coeffs.numel()}, opt);
+        const double scaling = ctx->saved_data["scaling"].toDouble(), rmax = ctx->saved_data["rmax"].toDouble(),
+                     rmin = ctx->saved_data["rmin"].toDouble();
+        void* st = current_stream(brcs);
+        int rc;
+        if (brcs.scalar_type() == at::kDouble) {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<double>() : nullptr; };
+            rc = a2p_mtp_basis_bwd_f64(plan.handle, (int)K, scaling, p(coeffs), (int)nmus, (int)ntypes, rmax, rmin, s.B,
+                                       s.P, s.U, 0, sv[4].data_ptr<int>(), sv[5].data_ptr<int>(), sv[6].data_ptr<int>(),
+                                       sv[7].data_ptr<int>(), p(brcs), sv[9].data_ptr<int>(), p(g), p(dr), p(dc), st);
+        } else {
+            auto p = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+            rc = a2p_mtp_basis_bwd_f32(plan.handle, (int)K, scaling, p(coeffs), (int)nmus, (int)ntypes, rmax, rmin, s.B,
+                                       s.P, s.U, 0, sv[4].data_ptr<int>(), sv[5].data_ptr<int>(), sv[6].data_ptr<int>(),
+                                       sv[7].data_ptr<int>(), p(brcs), sv[9].data_ptr<int>(), p(g), p(dr), p(dc), st);
+        }
+        check_rc(rc);
+        if (want_c) out[8] = dc.sum(0).reshape(coeffs.sizes());
+        if (want_r) out[13] = dr;
+        return out;
+    }
+};
+
 // normal equations of the linear parameters (linear_mtp_gram_and_cross.h:446-575): components by the
 // library, Gram products by torch's BLAS
 variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at::Tensor& e_dft,
@@ -402,6 +468,19 @@ TORCH_LIBRARY(mtpr, m)
         require_no_zbl(zbl_rmax);
         return EsitesFunction::apply(MTP_EFV_PASS);
     });
+    // mtpr_bind.cc:140-187: num_mus4moms / mus4moms (the radial functions behind each moment, which the reference's
+    // coefficient derivative walks) are not needed here; the first dimension of mus4moms is the number of moments
+    m.def("mtpBasisOp",
+          [](const at::Tensor& basic, const at::Tensor& times, const at::Tensor& mapping, const at::Tensor& num_mus4moms,
+             const at::Tensor& mus4moms, const at::Tensor& nmus, int64_t ntypes, int64_t K, double scaling,
+             const at::Tensor& coeffs, const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+             const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes, int64_t umax,
+             double rmax, double rmin) -> variable_list {
+              TORCH_CHECK(brcs.dim() == 4 && umax == brcs.size(2), "umax_num_neighs does not match brcs");
+              return BasisFunction::apply(basic, times, mapping, mus4moms.size(0), (int64_t)nmus.item<int>(), ntypes, K,
+                                          scaling, coeffs, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, rmax,
+                                          rmin);
+          });
     m.def("linearMtpToDescriptorsOp",
           [](int64_t K, double scaling, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic,
              const at::Tensor& times, const at::Tensor& mapping, int64_t nmus, const at::Tensor& binum,

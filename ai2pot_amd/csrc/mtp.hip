@@ -94,6 +94,10 @@ struct MtpArgs {
     int H;
     const T *w0, *w1, *q_shift;
     int nn_exact;      // loss mode: 1 = complete derivative, 0 = the reference's formulas (see nnmtp_loss)
+    // backward of the legacy basis operator (mtpBasis.h:359-394): the adjoint sweep starts from the caller's
+    // weights of each row's scalar moments instead of a read-out (`lin`, `bias`, `q_scaler` are unused)
+    const T* row_seed; // [B, P, n_scalar], or null
+    T* pair_out;       // [B, P, U, 3] derivative of the row's weighted moments along each pair vector, or null
 };
 
 __device__ __forceinline__ float tanh_t(float x) { return tanhf(x); }
@@ -523,6 +527,8 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
             A[p.mapping[k]] = acc / a.q_scaler[k];
             if (LOSS && a.nn_exact) Bm[p.mapping[k]] = bac / a.q_scaler[k];
         }
+    } else if (a.row_seed) {
+        for (int s = lane; s < p.n_scalar; s += NT) A[p.mapping[s]] = a.row_seed[row * p.n_scalar + s];
     } else {
         for (int s = lane; s < p.n_scalar; s += NT) {
             e_part += a.lin[s] * M[p.mapping[s]] / a.q_scaler[s];
@@ -614,6 +620,10 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
                     if (rk >= a.seg_cap) atomicOr(a.status, ST_SEG_OVERFLOW);
                     dst[0] = gx; dst[1] = gy; dst[2] = gz;
                 }
+                if (a.pair_out) {                 // padded layout of brcs; entries beyond the row stay zero
+                    T* dst = a.pair_out + (row * a.U + c0 + j) * 3;
+                    dst[0] = gx; dst[1] = gy; dst[2] = gz;
+                }
                 fx += gx; fy += gy; fz += gz;
                 vir[0] -= gx * d[0]; vir[1] -= gx * d[1]; vir[2] -= gx * d[2];
                 vir[3] -= gy * d[0]; vir[4] -= gy * d[1]; vir[5] -= gy * d[2];
@@ -624,21 +634,25 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
         fx = wave_sum(fx); fy = wave_sum(fy); fz = wave_sum(fz);
         double e_atom = (double)block_sum<T, NT>(e_part, gred, lane);
         double out[10];
-        out[0] = e_atom + (double)a.bias[ti];
+        out[0] = e_atom + (a.row_seed ? 0.0 : (double)a.bias[ti]);
 #pragma unroll
         for (int q = 0; q < 9; q++) out[1 + q] = (double)wave_sum(vir[q]);
         if (lane == 0) {
-            T* fo = a.force + ((size_t)b * NF + center) * 3;
-            fo[0] = fx; fo[1] = fy; fo[2] = fz;
+            if (a.force) {
+                T* fo = a.force + ((size_t)b * NF + center) * 3;
+                fo[0] = fx; fo[1] = fy; fo[2] = fz;
+            }
+            if (a.partial) {
 #pragma unroll
-            for (int q = 0; q < 10; q++) a.partial[row * 10 + q] = out[q];
+                for (int q = 0; q < 10; q++) a.partial[row * 10 + q] = out[q];
+            }
         }
         return;
     }
 
     // ---- loss gradient ------------------------------------------------------------------------
     if (LOSS) {
-        const T cE = a.cE_per_atom ? a.cE[row] : a.cE[b];
+        const T cE = a.row_seed ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
         // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
         if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
         T* grow = a.gpart + row * a.ngrad;
@@ -666,7 +680,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
             }
             for (int n = lane; n < H; n += NT) grow[nblk + H * S + n] = cE * n_th[n] + n_d1[n] * n_tau[n];
             if (lane == 0) grow[nblk + H * S + H] = cE;
-        } else {
+        } else if (!a.row_seed) {
             // linear coefficients and bias: linearMtpLoss.h:539-554
             for (int s = lane; s < p.n_scalar; s += NT)
                 grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
@@ -1132,14 +1146,14 @@ template <typename T>
 int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coeffs, const T* lin,
               const T* bias, int nmus, int ntypes, const T* q_scaler, double rmax, double rmin, int B, int P,
               int U, int nghost, const int* binum, const int* bilist, const int* bnumneigh,
-              const int* bfirstneigh, const T* brcs, const int* btypes)
+              const int* bfirstneigh, const T* brcs, const int* btypes, bool readout = true)
 {
     A2P_REQUIRE(K >= 1 && K <= MTP_KMAX, A2P_ERR_INVALID, "mtp: chebyshev_size %d outside [1, %d]", K, MTP_KMAX);
     A2P_REQUIRE(nmus == plan->d.nmus, A2P_ERR_INVALID, "mtp: nmus %d does not match the tables (%d)", nmus,
                 plan->d.nmus);
     A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0 && U >= 1 && nghost >= 0, A2P_ERR_INVALID, "mtp: bad shape");
     A2P_REQUIRE(rmax > rmin && rmin >= 0, A2P_ERR_INVALID, "mtp: need 0 <= rmin < rmax");
-    A2P_REQUIRE(coeffs && bias && q_scaler && binum && bilist && bnumneigh && bfirstneigh && brcs &&
+    A2P_REQUIRE(coeffs && (!readout || (bias && q_scaler)) && binum && bilist && bnumneigh && bfirstneigh && brcs &&
                     btypes, A2P_ERR_INVALID, "mtp: null input pointer");
     A2P_REQUIRE((long long)B * P * U < (1ll << 31), A2P_ERR_INVALID, "mtp: batch too large");
     a.p = plan->d;
@@ -1152,6 +1166,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.seg_cap = 0; a.partial = nullptr;
     a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
     a.nn_exact = 1;
+    a.row_seed = nullptr; a.pair_out = nullptr;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
@@ -1449,6 +1464,63 @@ int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T
     return A2P_OK;
 }
 
+// Backward of the legacy basis operator (mtpBasisOp.cc:220-326; mtpBasis.h:359-394 contracts the dense derivative
+// arrays that find_val_der, :107-356, filled in the forward pass): with w = grad_desc[b, ii, :] the weights of
+// the row's scalar moments,  drcs[b, ii, u, :] = sum_s w_s dM_s / d rcs[b, ii, u, :]  and
+// dcoeffs[b, :] = sum_ii sum_s w_s dM_s / d coeffs.  Nothing dense is kept between the passes: the moments are
+// recomputed and the adjoint sweep of the E/F/V kernel (pair derivatives) and of the loss-gradient kernel
+// (coefficient gradient; with zero force and virial residuals its tangent vectors vanish) starts from w.
+template <typename T>
+int mtp_basis_bwd(void* handle, int K, double scaling, const T* coeffs, int nmus, int ntypes, double rmax,
+                  double rmin, int B, int P, int U, int nghost, const int* binum, const int* bilist,
+                  const int* bnumneigh, const int* bfirstneigh, const T* brcs, const int* btypes, const T* grad_desc,
+                  T* drcs, T* dcoeffs, hipStream_t stream)
+{
+    MtpPlan* plan = nullptr;
+    int rc = plan_check(handle, &plan);
+    if (rc) return rc;
+    A2P_REQUIRE(grad_desc && (drcs || dcoeffs), A2P_ERR_INVALID, "mtp basis backward: null pointer");
+    MtpArgs<T> a;
+    rc = fill_args(a, plan, K, scaling, coeffs, (const T*)nullptr, (const T*)nullptr, nmus, ntypes, (const T*)nullptr,
+                   rmax, rmin, B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, false);
+    if (rc) return rc;
+    if (B == 0 || P == 0) return A2P_OK;
+    a.row_seed = grad_desc;
+    if (drcs) {
+        rc = fill_zero(drcs, (size_t)B * P * U * 3 * sizeof(T), stream);
+        if (rc) return rc;
+        MtpArgs<T> e = a;
+        e.E = table_entries<T>(e.p, K, false);
+        e.pair_out = drcs;
+        rc = launch_atoms<T, false>(e, stream);
+        if (rc) return rc;
+    }
+    if (dcoeffs) {
+        const int ncoef = ntypes * ntypes * nmus * K;
+        // workspace: dVs[B*9] | dFs[(B*P + nghost)*3] (both zero) | gpart[B*P*ncoef]
+        const size_t nzero = (size_t)B * 9 + ((size_t)B * P + nghost) * 3;
+        void* ws = nullptr;
+        rc = ws_get(WS_MTP, (nzero + (size_t)B * P * ncoef) * sizeof(T), &ws);
+        if (rc) return rc;
+        T* dVs = (T*)ws;
+        T* dFs = dVs + (size_t)B * 9;
+        T* gpart = (T*)ws + nzero;
+        rc = fill_zero(ws, ((nzero * sizeof(T) + 3) / 4) * 4, stream);
+        if (rc) return rc;
+        MtpArgs<T> g = a;
+        g.E = table_entries<T>(g.p, K, true);
+        g.dFs = dFs; g.dVs = dVs; g.gpart = gpart; g.ngrad = ncoef;
+        rc = launch_atoms<T, true>(g, stream);
+        if (rc) return rc;
+        prof_begin("mtp_grad_reduce", stream);
+        hipLaunchKernelGGL(mtp_grad_reduce_kernel<T>, dim3(ceil_div(ncoef, 256), B), dim3(256), 0, stream, P, ncoef, 0, 0,
+                           binum, gpart, dcoeffs, (T*)nullptr, (T*)nullptr);
+        prof_end(stream);
+        A2P_HIP_CHECK(hipGetLastError());
+    }
+    return A2P_OK;
+}
+
 // Energy, force and virial of every linear parameter taken alone (linear_mtp_gram_and_cross.h:125-374):
 // ecomp[B, n], fcomp[B, P, 3, n], vcomp[B, 9, n] with n = n_scalar + ntypes.  Column s < n_scalar is the
 // E/F/V of the model with linear_coeffs = e_s and no bias (the reference obtains the same numbers by
@@ -1715,5 +1787,21 @@ int a2p_mtp_esites_bwd_f32(void* plan, MTP_MODEL(float), int B, int P, int U, in
 {
     return a2p::mtp_esites_bwd<float>(plan, MTP_MODEL_PASS, B, P, U, nghost, MTP_BATCH_PASS, grad_e_sites, dcoeffs,
                                       dlinear, dbias, (hipStream_t)stream);
+}
+
+int a2p_mtp_basis_bwd_f64(void* plan, int K, double scaling, const double* coeffs, int nmus, int ntypes, double rmax,
+                          double rmin, int B, int P, int U, int nghost, MTP_BATCH(double), const double* grad_desc,
+                          double* drcs, double* dcoeffs, void* stream)
+{
+    return a2p::mtp_basis_bwd<double>(plan, K, scaling, coeffs, nmus, ntypes, rmax, rmin, B, P, U, nghost,
+                                      MTP_BATCH_PASS, grad_desc, drcs, dcoeffs, (hipStream_t)stream);
+}
+
+int a2p_mtp_basis_bwd_f32(void* plan, int K, double scaling, const float* coeffs, int nmus, int ntypes, double rmax,
+                          double rmin, int B, int P, int U, int nghost, MTP_BATCH(float), const float* grad_desc,
+                          float* drcs, float* dcoeffs, void* stream)
+{
+    return a2p::mtp_basis_bwd<float>(plan, K, scaling, coeffs, nmus, ntypes, rmax, rmin, B, P, U, nghost,
+                                     MTP_BATCH_PASS, grad_desc, drcs, dcoeffs, (hipStream_t)stream);
 }
 }

@@ -719,6 +719,89 @@ def linearMtpToDescriptorsOp(chebyshev_size, scaling, coeffs, alpha_moments_coun
     return [desc]
 
 
+def mtp_basis_backward(grad_desc, chebyshev_size, scaling, coeffs, alpha_moments_count, alpha_index_basic,
+                       alpha_index_times, alpha_moment_mapping, nmus, ntypes, binum, bilist, bnumneigh, bfirstneigh,
+                       brcs, btypes, rmax, rmin, want_drcs=True, want_dcoeffs=True, nghost=0):
+    """Backward of the legacy basis operator for the weights grad_desc[B, P, S] of the scalar moments:
+    (drcs[B, P, U, 3], dcoeffs[B, ncoef]) (None where not wanted); mtpBasisOp.cc:220-326, mtpBasis.h:359-394."""
+    _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
+         "brcs must be a tensor on a HIP device: this build has no CPU path")
+    dtype, device = brcs.dtype, brcs.device
+    _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
+    _req(brcs.is_contiguous(), "brcs must be contiguous")
+    _check_float("coeffs", coeffs, dtype, device)
+    _check_float("grad_desc", grad_desc, dtype, device)
+    for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
+                    ("bfirstneigh", bfirstneigh), ("btypes", btypes)):
+        _check_int(name, t, device)
+    nghost, ntypes = int(nghost), int(ntypes)
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost)
+    plan, n_scalar = _mtp_plan(alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping,
+                               device)
+    _req(coeffs.numel() == ntypes * ntypes * int(nmus) * int(chebyshev_size), "coeffs size mismatch")
+    _req(tuple(grad_desc.shape) == (B, P, n_scalar), "grad_desc must have shape [B, P, alpha_scalar_moments]")
+    drcs = torch.zeros((B, P, U, 3), dtype=dtype, device=device) if want_drcs else None
+    dc = torch.zeros((B, coeffs.numel()), dtype=dtype, device=device) if want_dcoeffs else None
+    if not (want_drcs or want_dcoeffs):
+        return None, None
+    L = _lib.lib()
+    fn = L.a2p_mtp_basis_bwd_f32 if dtype == torch.float32 else L.a2p_mtp_basis_bwd_f64
+    with torch.cuda.device(device):
+        rc = fn(plan, _c.c_int(chebyshev_size), _c.c_double(scaling), _ptr(coeffs), _c.c_int(int(nmus)),
+                _c.c_int(ntypes), _c.c_double(rmax), _c.c_double(rmin), _c.c_int(B), _c.c_int(P), _c.c_int(U),
+                _c.c_int(nghost), _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs),
+                _ptr(btypes), _ptr(grad_desc), _ptr(drcs), _ptr(dc), _stream(device))
+        _lib.check(rc)
+    return drcs, dc
+
+
+class _MtpBasis(torch.autograd.Function):
+    """The legacy basis operator with the reference's autograd contract (mtpBasisOp.cc:28-326): the output
+    is the scalar moments of every row; gradients flow to coeffs (summed over structures and atoms) and to
+    brcs.  The reference keeps dM/d rcs [B, P, S, U, 3] and dM/d coeffs [B, P, S, ncoef] from the forward
+    pass; here the backward recomputes the moments and runs one adjoint sweep per row."""
+
+    @staticmethod
+    def forward(ctx, coeffs, brcs, args):
+        (n_moms, basic, times, mapping, nmus, ntypes, K, scaling, binum, bilist, bnumneigh, bfirstneigh, btypes,
+         rmax, rmin, validate) = args
+        dtype, device = brcs.dtype, brcs.device
+        one = torch.ones((int(mapping.numel()),), dtype=dtype, device=device)
+        zero_b = torch.zeros((int(ntypes),), dtype=dtype, device=device)
+        type_map = torch.zeros((int(ntypes),), dtype=torch.int32, device=device)     # only its length is used
+        _, desc = _mtp_esites_raw(K, scaling, coeffs.detach(), one, zero_b, n_moms, basic, times, mapping, nmus,
+                                  binum, bilist, bnumneigh, bfirstneigh, brcs.detach(), btypes, type_map, 0, rmax, rmin,
+                                  one, False, True, validate)
+        ctx.save_for_backward(coeffs, brcs)
+        ctx.args = args
+        return desc
+
+    @staticmethod
+    def backward(ctx, gdesc):
+        coeffs, brcs = ctx.saved_tensors
+        (n_moms, basic, times, mapping, nmus, ntypes, K, scaling, binum, bilist, bnumneigh, bfirstneigh, btypes,
+         rmax, rmin, _) = ctx.args
+        drcs, dc = mtp_basis_backward(gdesc.contiguous(), K, scaling, coeffs.detach(), n_moms, basic, times, mapping,
+                                      nmus, ntypes, binum, bilist, bnumneigh, bfirstneigh, brcs.detach(), btypes, rmax,
+                                      rmin, want_drcs=ctx.needs_input_grad[1], want_dcoeffs=ctx.needs_input_grad[0])
+        return (dc.sum(0).reshape(coeffs.shape) if dc is not None else None, drcs, None)
+
+
+def mtpBasisOp(alpha_index_basic, alpha_index_times, alpha_moment_mapping, num_mus4moms, mus4moms, nmus, ntypes,
+               chebyshev_size, scaling, coeffs, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, umax_num_neighs,
+               rmax, rmin, validate=True):
+    """[mtp_basis_val[B, P, alpha_scalar_moments]]: the scalar moments of every row, differentiable w.r.t.
+    coeffs and brcs; mtpr_bind.cc:140-187 (same argument order).  num_mus4moms / mus4moms (the radial functions
+    behind each moment, which the reference's coefficient derivative walks) are not needed: only the first
+    dimension of mus4moms, the number of moments, is read.  nmus may be a tensor, as in the reference."""
+    nmus = int(nmus.item()) if isinstance(nmus, torch.Tensor) else int(nmus)
+    _req(int(umax_num_neighs) == int(brcs.shape[2]), "umax_num_neighs does not match brcs")
+    args = (int(mus4moms.shape[0]), alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus, int(ntypes),
+            int(chebyshev_size), float(scaling), binum, bilist, bnumneigh, bfirstneigh, btypes, float(rmax),
+            float(rmin), validate)
+    return [_MtpBasis.apply(coeffs, brcs, args)]
+
+
 def mtp_lin_components(chebyshev_size, scaling, coeffs, alpha_moments_count, alpha_index_basic, alpha_index_times,
                        alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
                        rmax, rmin, q_scaler, validate=True):

@@ -393,6 +393,31 @@ int a2p_mtp_esites_bwd_f32(void* plan, int chebyshev_size, double scaling, const
                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Legacy basis operator -- replaces the compute of torch.ops.mtpr.mtpBasisOp, forward and backward
+ * (source/descriptor/mtpr/bind/mtpr_bind.cc:140-187; src/mtpBasisOp.cc:28-218 forward, :220-326 backward;
+ *  include/mtpBasis.h:107-356 MtpBasis::find_val_der, :359-394 find_der_backward).
+ * Forward: the operator's output, the scalar moments M[map[s]] of every row, is what
+ * a2p_mtp_esites_* writes to `descriptors` (e_sites NULL).  The reference's forward also fills two dense
+ * arrays for its backward, dM_s/d rcs [B, P, S, umax, 3] and dM_s/d coeffs [B, P, S, ncoef]; here nothing
+ * is kept between the passes.
+ * a2p_mtp_basis_bwd_*: with w = grad_desc[B, P, S] (the gradient arriving at the forward output),
+ *   drcs[b, ii, u, :] = sum_s w[b, ii, s] dM_s / d rcs[b, ii, u, :]      [B, P, umax, 3], zero beyond each row
+ *   dcoeffs[b, :]     = sum_ii sum_s w[b, ii, s] dM_s / d coeffs          [B, ncoef]
+ * (either may be NULL); the operator's backward sums dcoeffs over the batch (mtpBasis.h:389-393 adds every
+ * structure into one vector).  Rows beyond binum and neighbours beyond rmax contribute nothing.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_mtp_basis_bwd_f64(void* plan, int chebyshev_size, double scaling, const double* coeffs, int nmus,
+                          int ntypes, double rmax, double rmin, int batch, int natoms_pad, int umax, int nghost,
+                          const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
+                          const double* brcs, const int* btypes, const double* grad_desc, double* drcs,
+                          double* dcoeffs, void* stream);
+int a2p_mtp_basis_bwd_f32(void* plan, int chebyshev_size, double scaling, const float* coeffs, int nmus,
+                          int ntypes, double rmax, double rmin, int batch, int natoms_pad, int umax, int nghost,
+                          const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
+                          const float* brcs, const int* btypes, const float* grad_desc, float* drcs,
+                          float* dcoeffs, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * ZBL short-range correction -- the part of every E/F/V operator that its zbl_rmax > 0 argument
  * switches on (source/descriptor/correction/include/zbl.h:262-395 pair formulas;
  *  correction/gpu/include/zbl.cuh:422-620 composition per centre atom;

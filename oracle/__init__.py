@@ -5,7 +5,7 @@ may import this package; the product (``ai2pot_amd``) never does.
 
 Two families of functions with identical NumPy signatures:
 
-* ``nblist``, ``nep_efv``, ``nep_loss``, ``mtp_efv``, ``mtp_loss_step``, ``mtp_esites``, ``mtp_esites_bwd``,
+* ``nblist``, ``nep_efv``, ``nep_loss``, ``mtp_efv``, ``mtp_loss_step``, ``mtp_esites``, ``mtp_esites_bwd``, ``mtp_basis_bwd``,
   ``nnmtp_efv``, ``fvt_force``, ``fvt_virial`` --
   this repository's own C++ restatement of the reference algorithm (``oracle/src``,
   ``liboracle.so``), each function citing the reference file:line it follows;
@@ -396,6 +396,54 @@ def ref_mtp_esites_bwd(model, nb, gout):
 
 def mtp_esites_bwd(model, nb, gout):
     return _mtp_esites_bwd(oracle_lib(), "orc_mtp", model, nb, gout)
+
+
+def ref_mtp_basis(model, nb, w, level, ai2pot_path="/root/reference"):
+    """The legacy basis operator by the reference (MtpBasis::find_val_der + find_der_backward):
+    (val[B, P, S], drcs[B, P, U, 3], dcoeffs[B, ncoef]) for the weights w[B, P, S]; the tables are those of
+    the reference's own MtpParam(level)."""
+    lib = _load("_ref/libref_mtpr.so")
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    S = np.asarray(model["alpha_moment_mapping"]).size
+    ntypes = np.asarray(model["type_map"]).size
+    ncoef = ntypes * ntypes * model["nmus"] * model["chebyshev_size"]
+    coeffs = _c(model["coeffs"], np.float64)
+    w = _c(w, np.float64)
+    assert w.shape == (B, P, S)
+    val, drcs, dc = np.zeros((B, P, S)), np.zeros((B, P, U, 3)), np.zeros((B, ncoef))
+    saved = os.environ.get("AI2POT_PATH")
+    os.environ["AI2POT_PATH"] = ai2pot_path     # the reference reads it with getenv
+    try:
+        lib.ref_mtp_basis_f64.restype = _I
+        rc = lib.ref_mtp_basis_f64(_p(val), _p(drcs), _p(dc), _p(w), _I(level), _I(model["chebyshev_size"]),
+                                   _D(model.get("scaling", 1.0)), _p(coeffs), _I(B), _I(P), _p(binum), _p(bilist),
+                                   _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes), _I(ntypes), _I(U), _I(nghost),
+                                   _D(model["rmax"]), _D(model["rmin"]))
+    finally:
+        if saved is None:
+            del os.environ["AI2POT_PATH"]
+        else:
+            os.environ["AI2POT_PATH"] = saved
+    if rc != 0:
+        raise RuntimeError("reference MtpParam failed for level %d" % level)
+    return val, drcs, dc
+
+
+def mtp_basis_bwd(model, nb, w, want_drcs=True, want_dcoeffs=True):
+    """(drcs[B, P, U, 3], dcoeffs[B, ncoef]) of sum(w * scalar moments), w[B, P, S]: the backward of the legacy
+    basis operator."""
+    margs, k1 = _mtp_model_args(model)
+    largs, k2, (B, P, U, nghost, ntypes) = _mtp_list_args(model, nb)
+    S = np.asarray(model["alpha_moment_mapping"]).size
+    ncoef = ntypes * ntypes * model["nmus"] * model["chebyshev_size"]
+    w = _c(w, np.float64)
+    assert w.shape == (B, P, S)
+    drcs = np.zeros((B, P, U, 3)) if want_drcs else None
+    dc = np.zeros((B, ncoef)) if want_dcoeffs else None
+    fn = oracle_lib().orc_mtp_basis_bwd_f64
+    fn.restype = None
+    fn(_p(drcs) if want_drcs else None, _p(dc) if want_dcoeffs else None, _p(w), *margs, *largs)
+    return drcs, dc
 
 
 def _mtp_lin_system(lib, prefix, model, nb, weights, labels):

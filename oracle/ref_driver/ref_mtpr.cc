@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <string>
 #include "descriptor/mtpr/include/mtpParam.h"
+#include "descriptor/mtpr/include/mtpBasis.h"
 #include "descriptor/mtpr/include/linearMtp_cpu_launcher.h"
 #include "descriptor/mtpr/include/linearMtpLoss_cpu_launcher.h"
 #include "descriptor/mtpr/include/linear_mtp_gram_and_cross.h"
@@ -161,6 +162,45 @@ void ref_mtp_lin_system_f64(double* lin_matrix, double* lin_vector, double e_w, 
         mapping, nmus, B, P, const_cast<int*>(binum), const_cast<int*>(bilist), const_cast<int*>(bnumneigh),
         const_cast<int*>(bfirstneigh), (double(*)[3])const_cast<double*>(brcs), const_cast<int*>(btypes), ntypes,
         const_cast<int*>(type_map), U, nghost, rmax, rmin, const_cast<double*>(q_scaler));
+}
+
+// The legacy basis operator by the reference: MtpBasis::find_val_der (mtpBasis.h:107-356) with both dense
+// derivative arrays, then find_der_backward (:359-394) with the weights w[B, P, n_scalar], per structure as
+// the operator calls them (src/mtpBasisOp.cc:107-140, 277-300).  The tables, including the lists of radial
+// functions behind each moment, are the reference's own (MtpParam of the level).  dcoeffs is kept per
+// structure [B, ncoef] (the operator adds all structures into one vector).  Returns 1 if MtpParam fails.
+int ref_mtp_basis_f64(double* val, double* drcs, double* dcoeffs, const double* w, int level, int K, double scaling,
+                      const double* coeffs, int B, int P, const int* binum, const int* bilist, const int* bnumneigh,
+                      const int* bfirstneigh, const double* brcs, const int* btypes, int ntypes, int U, int nghost,
+                      double rmax, double rmin)
+{
+    try {
+        MtpParam p(level);
+        const int S = p.alpha_scalar_moments();
+        const int ncoef = ntypes * ntypes * p.nmus() * K;
+        std::vector<double> der((size_t)P * S * U * 3), der2c((size_t)P * S * ncoef);
+        std::memset(val, 0, sizeof(double) * (size_t)B * P * S);
+        std::memset(drcs, 0, sizeof(double) * (size_t)B * P * U * 3);
+        std::memset(dcoeffs, 0, sizeof(double) * (size_t)B * ncoef);
+        for (int b = 0; b < B; b++) {
+            std::fill(der.begin(), der.end(), 0.0);
+            std::fill(der2c.begin(), der2c.end(), 0.0);
+            MtpBasis<double>::find_val_der(
+                &val[(size_t)b * P * S], (double(*)[3])der.data(), der2c.data(), true, true, K, scaling,
+                const_cast<double*>(coeffs), p.alpha_moments_count(), p.alpha_index_basic_count(), p.alpha_index_basic(),
+                p.alpha_index_times_count(), p.alpha_index_times(), S, p.alpha_moment_mapping(), p.max_num_mus4mom(),
+                p.num_mus4moms(), p.mus4moms_ptr(), p.nmus(), binum[b], const_cast<int*>(&bilist[(size_t)b * P]),
+                const_cast<int*>(&bnumneigh[(size_t)b * P]), const_cast<int*>(&bfirstneigh[(size_t)b * P * U]),
+                (double(*)[3])const_cast<double*>(&brcs[(size_t)b * P * U * 3]),
+                const_cast<int*>(&btypes[(size_t)b * (P + nghost)]), ntypes, U, rmax, rmin);
+            MtpBasis<double>::find_der_backward(&drcs[(size_t)b * P * U * 3], &dcoeffs[(size_t)b * ncoef], true, true,
+                                                const_cast<double*>(&w[(size_t)b * P * S]), der.data(), der2c.data(), S,
+                                                binum[b], U, ncoef);
+        }
+        return 0;
+    } catch (MtpException& e) {
+        return 1;
+    }
 }
 
 void ref_mtp_schmidt_orth_f64(double* out, int ntypes, int nmus, int K, const double* in)

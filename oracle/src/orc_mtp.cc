@@ -16,6 +16,7 @@
 //
 // Also here, each with its own citations below: site energies / scalar moments and their
 // gradient (pinned by the reference's committed outputs, the sum rule and the linear read-out);
+// the backward of the legacy basis operator (reference outputs, central differences);
 // the normal equations of the linear parameters and the Gram-Schmidt of the radial functions
 // (reference outputs; rebuilt independently from one-hot E/F/V calls); the neural-network MTP
 // (source/descriptor/nnmtp): E/F/V and site energies (reference outputs, finite differences, the
@@ -480,6 +481,109 @@ void orc_nnmtp_esites_bwd_f64(double* dcoeffs, double* dw0, double* dw1, double*
                 else if (p < ncoef + nw0 + nw1) dw1[(size_t)b * nw1 + p - ncoef - nw0] = acc;
                 else dbias[(size_t)b * ntypes + p - ncoef - nw0 - nw1] = acc;
             }
+    }
+}
+
+// Backward of the legacy basis operator (src/mtpBasisOp.cc:220-326): with w[B, P, n_scalar] the gradient arriving
+// at the scalar moments,  drcs[b, ii, u, :] = sum_s w_s dM_s / d rcs[b, ii, u, :]  and, per structure,
+// dcoeffs[b, :] = sum_ii sum_s w_s dM_s / d coeffs  (mtpBasis.h:359-394 contracts the dense derivative arrays that
+// find_val_der fills; the operator adds the structures' coefficient gradients into one vector).
+// The position part restates the reference's forward differentiation (mtpBasis.h:186-245 basic moments,
+// :248-300 products: dense dM[moment][neighbour][3] carried through the product table in file order).  The
+// coefficient part is NOT the reference's mom_ders2coeffs propagation (:255-283): it is forward-mode AD of the
+// scalar moments of efv_one, one coefficient at a time.
+// Pinned by: the compiled reference (oracle/_ref/libref_mtpr.so, MtpBasis::find_val_der + find_der_backward)
+// on the test fixtures; central differences of the scalar moments w.r.t. every pair vector and coefficient.
+void orc_mtp_basis_bwd_f64(double* drcs, double* dcoeffs, const double* w, MTP_MODEL_ARGS, MTP_LIST_ARGS)
+{
+    Tables t{n_moms, n_basic, n_times, n_scalar, nmus, basic, times, mapping};
+    const int ncoef = ntypes * ntypes * nmus * K;
+    int kmax = 0;
+    for (int i = 0; i < n_basic; i++) kmax = std::max(kmax, basic[i * 4 + 1] + basic[i * 4 + 2] + basic[i * 4 + 3]);
+    if (drcs) {
+        std::memset(drcs, 0, sizeof(double) * (size_t)B * P * U * 3);
+#pragma omp parallel
+        {
+            std::vector<double> M(n_moms), dM((size_t)n_moms * U * 3), f(K), df(K), pw((kmax + 1) * 3), rp(kmax + 1),
+                g(nmus), dg(nmus);
+#pragma omp for schedule(dynamic) collapse(2)
+            for (int b = 0; b < B; b++)
+                for (int ii = 0; ii < P; ii++) {
+                    if (ii >= binum[b]) continue;
+                    const size_t row = (size_t)b * P + ii;
+                    const int* types = &btypes[(size_t)b * (P + nghost)];
+                    const int ti = types[bilist[row]], nn = bnumneigh[row];
+                    std::fill(M.begin(), M.end(), 0.0);
+                    std::fill(dM.begin(), dM.end(), 0.0);
+                    for (int jj = 0; jj < nn; jj++) {
+                        const double* v = &brcs[(row * U + jj) * 3];
+                        const double r = std::sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
+                        if (r > rmax) continue;
+                        const int tj = types[bfirstneigh[row * U + jj]];
+                        radial_basis(K, rmax, rmin, scaling, r, f.data(), df.data());
+                        rp[0] = 1; pw[0] = pw[1] = pw[2] = 1;
+                        for (int k = 1; k <= kmax; k++) {
+                            rp[k] = rp[k - 1] * r;
+                            for (int a = 0; a < 3; a++) pw[k * 3 + a] = pw[(k - 1) * 3 + a] * v[a];
+                        }
+                        const double* c = &coeffs[(size_t)(ti * ntypes + tj) * nmus * K];
+                        for (int mu = 0; mu < nmus; mu++) {
+                            g[mu] = 0; dg[mu] = 0;
+                            for (int k = 0; k < K; k++) { g[mu] += c[mu * K + k] * f[k]; dg[mu] += c[mu * K + k] * df[k]; }
+                        }
+                        for (int i = 0; i < n_basic; i++) {
+                            const int* q = &basic[i * 4];
+                            const int k = q[1] + q[2] + q[3];
+                            const double mono = pw[q[1] * 3 + 0] * pw[q[2] * 3 + 1] * pw[q[3] * 3 + 2];
+                            M[i] += g[q[0]] * mono / rp[k];
+                            for (int a = 0; a < 3; a++) {
+                                double dmono = 0;
+                                if (q[1 + a] > 0) {
+                                    int e[3] = {q[1], q[2], q[3]};
+                                    e[a]--;
+                                    dmono = q[1 + a] * pw[e[0] * 3 + 0] * pw[e[1] * 3 + 1] * pw[e[2] * 3 + 2];
+                                }
+                                dM[((size_t)i * U + jj) * 3 + a] =
+                                    (dg[q[0]] * mono / rp[k] - g[q[0]] * k * mono / (rp[k] * r)) * v[a] / r + g[q[0]] * dmono / rp[k];
+                            }
+                        }
+                    }
+                    for (int i = 0; i < n_times; i++) {
+                        const int* q = &times[i * 4];
+                        const double v0 = M[q[0]], v1 = M[q[1]], mult = q[2];
+                        M[q[3]] += mult * v0 * v1;
+                        for (int e = 0; e < nn * 3; e++)
+                            dM[(size_t)q[3] * U * 3 + e] += mult * (dM[(size_t)q[0] * U * 3 + e] * v1 + v0 * dM[(size_t)q[1] * U * 3 + e]);
+                    }
+                    for (int s = 0; s < n_scalar; s++) {
+                        const double ws = w[row * n_scalar + s];
+                        for (int e = 0; e < nn * 3; e++) drcs[row * U * 3 + e] += ws * dM[(size_t)mapping[s] * U * 3 + e];
+                    }
+                }
+        }
+    }
+    if (dcoeffs) {
+#pragma omp parallel
+        {
+            std::vector<Dual> c(ncoef), l(n_scalar, Dual(1.0, 0.0)), bi(ntypes, Dual(0.0, 0.0)), force((size_t)(P + nghost) * 3),
+                virial(9), desc((size_t)P * n_scalar);
+            std::vector<double> ones(n_scalar, 1.0);
+#pragma omp for schedule(dynamic) collapse(2)
+            for (int b = 0; b < B; b++)
+                for (int p = 0; p < ncoef; p++) {
+                    for (int i = 0; i < ncoef; i++) c[i] = Dual(coeffs[i], i == p);
+                    Dual e;
+                    efv_one<Dual>(e, force.data(), virial.data(), K, scaling, c.data(), l.data(), bi.data(), t, binum[b],
+                                  &bilist[(size_t)b * P], &bnumneigh[(size_t)b * P], &bfirstneigh[(size_t)b * P * U],
+                                  &brcs[(size_t)b * P * U * 3], &btypes[(size_t)b * (P + nghost)], ntypes, U, P + nghost,
+                                  rmax, rmin, ones.data(), nullptr, desc.data());
+                    double acc = 0;
+                    for (int ii = 0; ii < binum[b]; ii++)
+                        for (int s = 0; s < n_scalar; s++)
+                            acc += w[((size_t)b * P + ii) * n_scalar + s] * desc[(size_t)ii * n_scalar + s].d;
+                    dcoeffs[(size_t)b * ncoef + p] = acc;
+                }
+        }
     }
 }
 

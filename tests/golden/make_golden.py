@@ -100,6 +100,11 @@ def mtp_cases():
         dc, dl, db = oracle.ref_mtp_esites_bwd(m, nb, synth.rng_normal(4, B * P).reshape(B, P))
         out.update({tag + "/esites": es, tag + "/desc": desc, tag + "/es_dcoeffs": dc,
                     tag + "/es_dlinear": dl, tag + "/es_dbias": db})
+        # legacy basis operator: its output equals the descriptors; the backward for weights w[B, P, S]
+        S = t["alpha_moment_mapping"].size
+        bval, bdrcs, bdc = oracle.ref_mtp_basis(m, nb, synth.rng_normal(5, B * P * S).reshape(B, P, S), level)
+        assert np.allclose(bval, desc, rtol=1e-12, atol=1e-14)
+        out.update({tag + "/basis_drcs": bdrcs[:, :, :int(nb["bnumneigh"].max())], tag + "/basis_dcoeffs": bdc})
         m2 = dict(m)
         m2["q_scaler"] = np.linspace(0.7, 1.4, m["q_scaler"].size)
         A, bv = oracle.ref_mtp_lin_system(m2, nb, (1.0, 0.7, 0.3), labels)

@@ -290,6 +290,21 @@ def test_mtpr_ops(oracle, dropin, tmp_path):
     rc, rl, rb = oracle.mtp_esites_bwd(m, nb, gout)
     assert close(params3[0].grad.cpu().numpy(), rc.sum(0)) and close(params3[1].grad.cpu().numpy(), rl.sum(0))
     assert close(params3[2].grad.cpu().numpy(), rb.sum(0))
+    # the legacy basis operator: the scalar moments, differentiable w.r.t. coeffs and brcs
+    S = int(p[3].numel())
+    w = synth.rng_normal(5, B * P * S).reshape(B, P, S)
+    cb = md["coeffs"].clone().requires_grad_(True)
+    rb_ = dv["brcs"].clone().requires_grad_(True)
+    val = torch.ops.mtpr.mtpBasisOp(p[1].cuda(), p[2].cuda(), p[3].cuda(), p[4].cuda(), p[5].cuda(), p[6], 2, 8, 1.0, cb,
+                                    dv["binum"], dv["bilist"], dv["bnumneigh"], dv["bfirstneigh"], rb_, dv["btypes"],
+                                    int(rb_.shape[2]), 5.0, 1.0)
+    assert len(val) == 1 and close(val[0].detach().cpu().numpy(), desc_ref)
+    (val[0] * t(w)).sum().backward()
+    dr_ref, dc_ref = oracle.mtp_basis_bwd(m, nb, w)
+    assert close(rb_.grad.cpu().numpy(), dr_ref) and close(cb.grad.cpu().numpy().ravel(), dc_ref.sum(0))
+
+
+def test_nnmtp_ops(oracle, dropin, tmp_path):    assert close(params3[2].grad.cpu().numpy(), rb.sum(0))
 
 
 def test_nnmtp_ops(oracle, dropin, tmp_path):

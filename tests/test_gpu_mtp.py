@@ -328,6 +328,87 @@ def test_site_energies_against_golden_and_autograd(oracle):
     assert close(md["type_bias"].grad.cpu().numpy(), g["es_dbias"].sum(0))
 
 
+def basis_args(m, md, d, coeffs, brcs):
+    import torch
+    n_moms = m["alpha_moments_count"]
+    mus4moms = torch.zeros((n_moms, 1), dtype=torch.int32, device="cuda:0")       # only its first dimension is read
+    num_mus4moms = torch.zeros((n_moms,), dtype=torch.int32, device="cuda:0")
+    return (md["alpha_index_basic"], md["alpha_index_times"], md["alpha_moment_mapping"], num_mus4moms, mus4moms,
+            torch.tensor(m["nmus"], dtype=torch.int32), int(md["type_map"].numel()), m["chebyshev_size"], m["scaling"],
+            coeffs, d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], brcs, d["btypes"], int(brcs.shape[2]),
+            m["rmax"], m["rmin"])
+
+
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3), (20, 2)])
+def test_legacy_basis_operator(oracle, level, nt):
+    """mtpBasisOp: forward = the scalar moments; backward for weights w of the moments against the oracle
+    (pinned to the reference's MtpBasis::find_val_der + find_der_backward), with a padded structure and, at
+    level 20, the wide kernel; fp32 to its own tolerance."""
+    import torch
+    from ai2pot_amd import ops
+    m, nb, _ = loss_inputs(oracle, level, nt, sizes=(48, 30), P=52)
+    B, P = nb["bilist"].shape
+    S = m["alpha_moment_mapping"].size
+    w = synth.rng_normal(5, B * P * S).reshape(B, P, S)
+    want_c = level <= 16
+    drcs_ref, dc_ref = oracle.mtp_basis_bwd(m, nb, w, want_dcoeffs=want_c)
+    _, desc_ref = oracle.mtp_esites(m, nb)
+    for dtype, tol in ((torch.float64, 1e-10), (torch.float32, 2e-4)):
+        md = model_to_device(m, dtype)
+        d = to_device(nb, dtype)
+        coeffs = md["coeffs"].clone().requires_grad_(want_c)
+        brcs = d["brcs"].clone().requires_grad_(True)
+        val = ops.mtpBasisOp(*basis_args(m, md, d, coeffs, brcs))[0]
+        assert val.shape == desc_ref.shape and close(val.detach().cpu().numpy(), desc_ref, tol)
+        (val * torch.from_numpy(w).to(dtype).to("cuda:0")).sum().backward()
+        got = brcs.grad.cpu().numpy()
+        assert got.shape == drcs_ref.shape and close(got, drcs_ref, tol)
+        beyond = np.arange(got.shape[2])[None, None, :] >= nb["bnumneigh"][:, :, None]
+        assert np.all(got[beyond] == 0) and np.all(got[1, 30:] == 0)
+        if want_c:
+            assert coeffs.grad.shape == coeffs.shape and close(coeffs.grad.cpu().numpy().ravel(), dc_ref.sum(0), tol)
+    # one gradient only: the other pass is skipped
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    wt = torch.from_numpy(w).to("cuda:0")
+    only_r, none_c = ops.mtp_basis_backward(wt, m["chebyshev_size"], m["scaling"], md["coeffs"], m["alpha_moments_count"],
+                                            md["alpha_index_basic"], md["alpha_index_times"], md["alpha_moment_mapping"],
+                                            m["nmus"], nt, d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"],
+                                            d["brcs"], d["btypes"], m["rmax"], m["rmin"], want_dcoeffs=False)
+    assert none_c is None and close(only_r.cpu().numpy(), drcs_ref)
+
+
+def test_legacy_basis_operator_against_golden(oracle):
+    """Levels 8 and 16 against the committed outputs of the reference's MtpBasis::find_val_der and
+    find_der_backward (dense derivative arrays contracted with the weights)."""
+    import os
+    import torch
+    from ai2pot_amd import ops
+    for level, nt in ((8, 2), (16, 3)):
+        with np.load(os.path.join(os.path.dirname(__file__), "golden", "mtp.npz")) as z:
+            g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+        lat, pos = synth.random_packed(48, [8.5, 9.0, 9.5], 2.0, 21)
+        ty = synth.rng_randint(22, 48, nt)
+        m = synth.mtp_model(mtp_param.mtp_param(level), nt, 8, 5.0, 1.8, 3000 + level)
+        o = oracle.nblist(lat, ty, pos, 5.0, 100)
+        nb = synth.pack_batch([o, o])
+        nb["brcs"][1] *= 1.01
+        B, P = nb["bilist"].shape
+        S = m["alpha_moment_mapping"].size
+        w = synth.rng_normal(5, B * P * S).reshape(B, P, S)
+        md = model_to_device(m, torch.float64)
+        d = to_device(nb, torch.float64)
+        coeffs = md["coeffs"].clone().requires_grad_(True)
+        brcs = d["brcs"].clone().requires_grad_(True)
+        val = ops.mtpBasisOp(*basis_args(m, md, d, coeffs, brcs))[0]
+        assert close(val.detach().cpu().numpy(), g["desc"])
+        (val * torch.from_numpy(w).to("cuda:0")).sum().backward()
+        width = g["basis_drcs"].shape[2]
+        got = brcs.grad.cpu().numpy()
+        assert close(got[:, :, :width], g["basis_drcs"]) and np.all(got[:, :, width:] == 0)
+        assert close(coeffs.grad.cpu().numpy().ravel(), g["basis_dcoeffs"].sum(0))
+
+
 def test_site_energies_with_ghosts(oracle):
     """Rows are the local atoms; neighbours may be ghosts (index >= natoms_pad)."""
     import torch

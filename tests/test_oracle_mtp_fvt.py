@@ -95,6 +95,53 @@ def test_site_energies_and_descriptors(oracle, level, nt):
 
 
 @pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3)])
+def test_legacy_basis_operator_backward(oracle, level, nt):
+    """Backward of mtpBasisOp for weights w of the scalar moments: the committed outputs of the reference's
+    MtpBasis::find_val_der + find_der_backward; then, without it, central differences of the oracle's own
+    scalar moments along pair vectors and coefficients, zeros beyond each row and beyond the cutoff, and
+    linearity in w."""
+    with np.load(os.path.join(HERE, "golden", "mtp.npz")) as z:
+        g = {k.split("/")[1]: z[k] for k in z.files if k.startswith("L%02d/" % level)}
+    m, nb, _ = small_batch(oracle, level, nt)
+    B, P = nb["bilist"].shape
+    U = nb["brcs"].shape[2]
+    S = m["alpha_moment_mapping"].size
+    w = synth.rng_normal(5, B * P * S).reshape(B, P, S)
+    drcs, dc = oracle.mtp_basis_bwd(m, nb, w, want_dcoeffs=level != 16)
+    width = g["basis_drcs"].shape[2]
+    assert np.abs(drcs[:, :, :width] - g["basis_drcs"]).max() <= 1e-11 * np.abs(g["basis_drcs"]).max()
+    assert np.all(drcs[:, :, width:] == 0)
+    if dc is not None:
+        assert np.abs(dc - g["basis_dcoeffs"]).max() <= 1e-11 * np.abs(g["basis_dcoeffs"]).max()
+    # entries beyond a row's neighbour count, and neighbours beyond rmax, get nothing
+    nn = nb["bnumneigh"]
+    beyond = np.arange(U)[None, None, :] >= nn[:, :, None]
+    assert np.all(drcs[beyond] == 0)
+    r = np.linalg.norm(nb["brcs"], axis=-1)
+    assert np.all(drcs[(r > m["rmax"]) & ~beyond] == 0)
+    # central differences of sum(w * desc) along three pair vectors and three coefficients
+    phi = lambda mm, bb: (oracle.mtp_esites(mm, bb)[1] * w).sum((1, 2))
+    h = 1e-6
+    for (b, ii, u, a) in ((0, 0, 0, 0), (1, 17, 3, 2), (0, 40, int(nn[0, 40]) - 1, 1)):
+        if r[b, ii, u] > m["rmax"] - 1e-3:
+            continue
+        p_, m_ = dict(nb), dict(nb)
+        p_["brcs"] = nb["brcs"].copy(); p_["brcs"][b, ii, u, a] += h
+        m_["brcs"] = nb["brcs"].copy(); m_["brcs"][b, ii, u, a] -= h
+        fd = (phi(m, p_)[b] - phi(m, m_)[b]) / (2 * h)
+        assert abs(fd - drcs[b, ii, u, a]) < 1e-6 * max(1.0, abs(fd)), (b, ii, u, a)
+    if dc is not None:
+        for i in (0, 7, m["coeffs"].size - 1):
+            mp, mm = dict(m), dict(m)
+            mp["coeffs"] = m["coeffs"].copy(); mp["coeffs"][i] += h
+            mm["coeffs"] = m["coeffs"].copy(); mm["coeffs"][i] -= h
+            fd = (phi(mp, nb) - phi(mm, nb)) / (2 * h)
+            assert np.abs(fd - dc[:, i]).max() < 1e-6 * max(1.0, np.abs(fd).max())
+    d2, _ = oracle.mtp_basis_bwd(m, nb, -2.5 * w, want_dcoeffs=False)
+    assert np.abs(d2 + 2.5 * drcs).max() <= 1e-13 * np.abs(drcs).max()
+
+
+@pytest.mark.parametrize("level,nt", [(8, 2), (10, 1), (16, 3)])
 def test_linear_system_and_schmidt(oracle, level, nt):
     """Normal equations of the linear parameters and the Gram-Schmidt of the radial functions: the
     reference's committed outputs; then what fixes them without it: column s of the components is
