@@ -373,9 +373,12 @@ __device__ __forceinline__ void pair_walk(const T* __restrict__ t, const T* __re
 
 // NT threads per centre atom: 64 for small tables, 256 when there is enough work per atom
 // (four workgroups of 256 threads fit the LDS of a CU at the larger levels: keep the registers to match)
-template <typename T, bool LOSS, int NT>
+// SEED: the instance of the energy / force / virial kernel that can start its adjoint sweep from per-row weights
+// (row_seed, pair_out); the loss-gradient kernel tests the pointer at run time.
+template <typename T, bool LOSS, int NT, bool SEED = false>
 __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_kernel(const MtpArgs<T> a)
 {
+    const bool seeded = (SEED || LOSS) && a.row_seed != nullptr;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const MtpPlanDevice& p = a.p;
     const int lane = threadIdx.x;     // thread in the workgroup
@@ -527,7 +530,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
             A[p.mapping[k]] = acc / a.q_scaler[k];
             if (LOSS && a.nn_exact) Bm[p.mapping[k]] = bac / a.q_scaler[k];
         }
-    } else if (a.row_seed) {
+    } else if (seeded) {
         for (int s = lane; s < p.n_scalar; s += NT) A[p.mapping[s]] = a.row_seed[row * p.n_scalar + s];
     } else {
         for (int s = lane; s < p.n_scalar; s += NT) {
@@ -620,7 +623,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
                     if (rk >= a.seg_cap) atomicOr(a.status, ST_SEG_OVERFLOW);
                     dst[0] = gx; dst[1] = gy; dst[2] = gz;
                 }
-                if (a.pair_out) {                 // padded layout of brcs; entries beyond the row stay zero
+                if (SEED && a.pair_out) {         // padded layout of brcs; entries beyond the row stay zero
                     T* dst = a.pair_out + (row * a.U + c0 + j) * 3;
                     dst[0] = gx; dst[1] = gy; dst[2] = gz;
                 }
@@ -634,15 +637,15 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
         fx = wave_sum(fx); fy = wave_sum(fy); fz = wave_sum(fz);
         double e_atom = (double)block_sum<T, NT>(e_part, gred, lane);
         double out[10];
-        out[0] = e_atom + (a.row_seed ? 0.0 : (double)a.bias[ti]);
+        out[0] = e_atom + (seeded ? 0.0 : (double)a.bias[ti]);
 #pragma unroll
         for (int q = 0; q < 9; q++) out[1 + q] = (double)wave_sum(vir[q]);
         if (lane == 0) {
-            if (a.force) {
+            if (!SEED || a.force) {
                 T* fo = a.force + ((size_t)b * NF + center) * 3;
                 fo[0] = fx; fo[1] = fy; fo[2] = fz;
             }
-            if (a.partial) {
+            if (!SEED || a.partial) {
 #pragma unroll
                 for (int q = 0; q < 10; q++) a.partial[row * 10 + q] = out[q];
             }
@@ -652,7 +655,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
 
     // ---- loss gradient ------------------------------------------------------------------------
     if (LOSS) {
-        const T cE = a.row_seed ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
+        const T cE = seeded ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
         // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
         if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
         T* grow = a.gpart + row * a.ngrad;
@@ -680,7 +683,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
             }
             for (int n = lane; n < H; n += NT) grow[nblk + H * S + n] = cE * n_th[n] + n_d1[n] * n_tau[n];
             if (lane == 0) grow[nblk + H * S + H] = cE;
-        } else if (!a.row_seed) {
+        } else if (!seeded) {
             // linear coefficients and bias: linearMtpLoss.h:539-554
             for (int s = lane; s < p.n_scalar; s += NT)
                 grow[ncoef + s] = (cE * M[p.mapping[s]] + Tg[p.mapping[s]]) / a.q_scaler[s];
@@ -1175,7 +1178,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     return A2P_OK;
 }
 
-template <typename T, bool LOSS>
+template <typename T, bool LOSS, bool SEED = false>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
     auto lds_for = [&](int nc, size_t* main) {
@@ -1201,7 +1204,7 @@ int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
                 "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
     const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
-    auto kern = wide ? mtp_atom_kernel<T, LOSS, 256> : mtp_atom_kernel<T, LOSS, 64>;
+    auto kern = wide ? mtp_atom_kernel<T, LOSS, 256, SEED> : mtp_atom_kernel<T, LOSS, 64, SEED>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
@@ -1492,7 +1495,7 @@ int mtp_basis_bwd(void* handle, int K, double scaling, const T* coeffs, int nmus
         MtpArgs<T> e = a;
         e.E = table_entries<T>(e.p, K, false);
         e.pair_out = drcs;
-        rc = launch_atoms<T, false>(e, stream);
+        rc = launch_atoms<T, false, true>(e, stream);
         if (rc) return rc;
     }
     if (dcoeffs) {
