@@ -228,6 +228,68 @@ def test_gather_equals_segments_and_is_reproducible(oracle):
     assert np.abs(v - v.T).max() <= 2e-5 * np.abs(v).max()
 
 
+def test_headline_size_properties_and_sampled_atoms(oracle):
+    """The benchmark's configuration itself: 1,048,576 atoms (perturbed fcc, 3 species), fp32, umax 200.  The oracle
+    would need minutes for the whole cell, so the whole-cell checks are properties: two runs give the same bits,
+    the forces sum to zero, the virial is symmetric, and the segment path (another formulation: scatter into
+    reduction segments from the padded rows) agrees within the fp32 bars.  Then the oracle itself on sampled atoms,
+    among them those nearest to the faces of the cell: the rows of the atom and of all its neighbours, taken from
+    the padded arrays of the step, form a small LAMMPS-style domain (the neighbours' other neighbours are ghosts),
+    on which the oracle's force on the atom is complete."""
+    import torch
+    lat, pos = synth.fcc_cell(64, 316.7 / 64.0, 0.15, 1006)
+    n = pos.shape[0]
+    assert n == 1048576
+    ty = synth.rng_randint(2006, n, 3)
+    m = synth.nep_model(seed=3006)
+    calc = _calc(m, lat, ty, n, np.float32, umax=200, path="gather")
+    a = _step(calc, pos, np.float32)
+    b = _step(calc, pos, np.float32)                        # rebuild in place, same coordinates
+    for x, y in zip(a, b):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    f64 = a[1].astype(np.float64)
+    assert np.abs(f64.sum(0)).max() < 5e-2 and np.isfinite(f64).all()
+    v = a[2].reshape(3, 3)
+    assert np.abs(v - v.T).max() <= 2e-5 * np.abs(v).max()
+    # sampled atoms against the oracle, from the rows of this step
+    rng = np.random.RandomState(7)
+    picks = set(int(i) for i in rng.randint(0, n, 6))
+    for ax in range(3):
+        picks.add(int(np.argmin(pos[:, ax])))
+        picks.add(int(np.argmax(pos[:, ax])))
+    U = calc.umax
+    first_d, rcs_d, nn_d = calc.firstneigh.view(n, U), calc.rcs.view(n, U, 3), calc.numneigh
+    for i in sorted(picks):
+        ni = int(nn_d[i])
+        local = [i] + sorted(set(first_d[i, :ni].cpu().numpy().tolist()) - {i})
+        idx = torch.tensor(local, device="cuda:0", dtype=torch.long)
+        nn = nn_d[idx].cpu().numpy()
+        fn = first_d[idx].cpu().numpy()
+        rc = rcs_d[idx].cpu().numpy().astype(np.float64)
+        P = len(local)
+        ids = {g: k for k, g in enumerate(local)}
+        for r in range(P):
+            for g in fn[r, :nn[r]].tolist():
+                if g not in ids:
+                    ids[g] = len(ids)
+        firstm = np.zeros((P, U), np.int32)
+        for r in range(P):
+            firstm[r, :nn[r]] = [ids[g] for g in fn[r, :nn[r]].tolist()]
+        glob = np.array(sorted(ids, key=ids.get))
+        nb = dict(binum=np.array([P], np.int32), bilist=np.arange(P, dtype=np.int32)[None],
+                  bnumneigh=nn.astype(np.int32)[None], bfirstneigh=firstm[None], brcs=rc[None],
+                  btypes=ty[glob].astype(np.int32)[None], nghost=len(ids) - P)
+        _, fr, _ = oracle.nep_efv(m, nb, np.float64)
+        got, want = a[1][i].astype(np.float64), np.asarray(fr).reshape(-1, 3)[0]
+        assert np.all(np.abs(got - want) <= 1e-4 + 1e-5 * np.abs(want)), (i, got, want)
+    del calc
+    torch.cuda.empty_cache()
+    s = _step(_calc(m, lat, ty, n, np.float32, umax=200, path="segments"), pos, np.float32)
+    assert np.allclose(a[0], s[0], rtol=2e-6)
+    assert np.all(np.abs(a[1] - s[1]) <= 2e-4 + 2e-5 * np.abs(s[1]))
+    assert np.abs(a[2] - s[2]).max() <= 2e-5 * np.abs(s[2]).max()
+
+
 def test_rebuild_in_place(oracle):
     """Steps on moving coordinates reuse the calculator's buffers (rows updated in place, compact lists
     rewritten): every step equals a fresh calculator's."""
