@@ -227,8 +227,8 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * build left in `compact` (it is a locality hint; atoms that moved a little are still well ordered)
  * instead of sorting again.  The order is the first array of the buffer, int32[natoms], position ->
  * atom; a caller whose atoms are already ordered in space may write the identity (or any permutation
- * of the atoms) there and set bit 1 from the first build on (an array that is no permutation gives
- * meaningless lists, inside bounds).  The five padded outputs are written,
+ * of the atoms) there and set bit 1 from the first build on.  The array is not checked: it must hold
+ * every index 0 .. natoms-1 once (an index outside that range is an access outside the buffers).  The five padded outputs are written,
  * bit-identical to a2p_nblist_build_*, when they are given; pass all five NULL to skip them.
  * Needs umax % 8 == 0, natoms < 2^27, species < 16, 16-byte aligned firstneigh / rcs.
  *
