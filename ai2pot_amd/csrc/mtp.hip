@@ -33,7 +33,8 @@ namespace a2p {
 namespace {
 
 constexpr int MTP_NC = 32;        // neighbours per chunk (rows of the LDS table); the energy / force / virial
-constexpr int MTP_NC_MAX = 48;    // launch raises it up to MTP_NC_MAX while that costs no workgroup per CU
+constexpr int MTP_NC_MAX = 48;    // the launch picks between MTP_NC_MIN and MTP_NC_MAX rows (launch_atoms)
+constexpr int MTP_NC_MIN = 16;
 
 // The group sums of the last pass over the neighbours (four per thread for the pair derivatives, two
 // for the loss gradient) live in the moment vector (loss mode: moments and tangents) when it is long
@@ -45,11 +46,18 @@ __host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms)
 // entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums.
 // In the energy / force / virial kernel the group sums (4 per thread) are written over the table once every
 // thread has finished reading it.
-__host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots)
+// The adjoints of the energy / force / virial kernel live in this region too, behind the partial sums: they are
+// needed from the end of the forward sweep to the gathering of the dense adjoint array, which is when the
+// neighbour table is not (mtp_adjoint_offset).
+__host__ __device__ inline int mtp_adjoint_offset(int max_level_slots)
+{
+    return ((max_level_slots > 8 ? max_level_slots : 8) + 1) & ~1;     // at least the scratch of a block sum
+}
+__host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots, int nt)
 {
     int a = loss ? nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4) : nc * E;
-    if (!loss && a < 256 * 4) a = 256 * 4;
-    const int b = max_level_slots * (loss ? 2 : 1);
+    if (!loss && a < nt * 4) a = nt * 4;          // four group sums per thread
+    const int b = loss ? max_level_slots * 2 : mtp_adjoint_offset(max_level_slots) + n_moms;
     return a > b ? a : b;
 }
 // the dense adjoint array of the pair-derivative pass takes the place of the moments when it fits
@@ -376,7 +384,7 @@ __device__ __forceinline__ void pair_walk(const T* __restrict__ t, const T* __re
 // SEED: the instance of the energy / force / virial kernel that can start its adjoint sweep from per-row weights
 // (row_seed, pair_out); the loss-gradient kernel tests the pointer at run time.
 template <typename T, bool LOSS, int NT, bool SEED = false>
-__global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_kernel(const MtpArgs<T> a)
+__global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const MtpArgs<T> a)
 {
     const bool seeded = (SEED || LOSS) && a.row_seed != nullptr;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -394,17 +402,18 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
     // moments | (loss mode: their tangents) | adjoints | (loss mode: mixed adjoints)
     T* M = (T*)smem_raw;
     T* Tg = M + n_moms;
-    T* A = Tg + (LOSS ? n_moms : 0);
-    T* Bm = A + n_moms;
+    T* Bm = Tg + (LOSS ? 2 * n_moms : 0);    // loss mode: the adjoints sit between the tangents and the mixed adjoints
     T* cf = Bm + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
     T* tab = cf + a.ntypes * nmus * K;
+    // energy / force / virial kernel: the adjoints share the table's region (behind the sweeps' partial sums)
+    T* A = LOSS ? Tg + n_moms : tab + mtp_adjoint_offset(p.max_level_slots);
     // [256/32][32][4] partial sums of the thread groups.  They are needed only in the last pass over the
     // neighbours, when the moments (and, in loss mode, their tangents) are dead: a long enough moment
     // vector lends them its place
     const bool share = mtp_gred_in_moments(LOSS, n_moms);
     // energy / force / virial kernel: the group sums are written over the table once it has been read
     T* gred = LOSS ? (share ? M : tab + MTP_NC * E) : tab;
-    T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots);   // loss mode: P[nc][nmus] | Q[nc][nmus]
+    T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots, NT);   // loss mode: P[nc][nmus] | Q[nc][nmus]
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
         if (!LOSS && a.partial && lane < 10) a.partial[row * 10 + lane] = 0.0;
@@ -431,15 +440,13 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
         bas[i] = (unsigned)p.basic[i * 4] | ((unsigned)p.basic[i * 4 + 1] << 8) |
                  ((unsigned)p.basic[i * 4 + 2] << 16) | ((unsigned)p.basic[i * 4 + 3] << 24);
     int* rws = (int*)(bas + n_basic);        // monomial rows of the pair-derivative walk
-    int* dpos = rws + p.nrows;               // entry of each basic moment in the dense adjoint array
     if (!LOSS) {
         for (int i = lane; i < p.nrows; i += NT) rws[i] = p.rows[i];
-        for (int i = lane; i < n_basic; i += NT) dpos[i] = p.dense_pos[i];
     }
     for (int q = lane; q < a.ntypes * nmus * K; q += NT) cf[q] = a.coeffs[(size_t)ti * a.ntypes * nmus * K + q];
     for (int i = lane; i < n_moms; i += NT) {
-        M[i] = (T)0; A[i] = (T)0;
-        if (LOSS) { Tg[i] = (T)0; Bm[i] = (T)0; }
+        M[i] = (T)0;
+        if (LOSS) { A[i] = (T)0; Tg[i] = (T)0; Bm[i] = (T)0; }
     }
     __syncthreads();
 
@@ -477,6 +484,10 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
 
     // ---- products, energy, adjoint ------------------------------------------------------------
     sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
+    if (!LOSS) {                              // the table is dead: its place now holds the adjoints
+        for (int i = lane; i < n_moms; i += NT) A[i] = (T)0;
+        __syncthreads();
+    }
     T e_part = (T)0;
     // network buffers (H > 0): inputs q[S]; per neuron w1 tanh', and in loss mode tanh, tanh', tanh'', tau
     T* nnb = LOSS ? pq + 2 * MTP_NC * nmus + MTP_NC + a.ntypes * nmus * K : pq;
@@ -556,7 +567,7 @@ __global__ void __launch_bounds__(NT, (!LOSS && NT == 256 ? 4 : 1)) mtp_atom_ker
         if (p.dense_unique) {
             for (int e = lane; e < p.nq * p.nmp; e += NT) AD[e] = (T)0;
             __syncthreads();
-            for (int i = lane; i < n_basic; i += NT) AD[dpos[i]] = A[i];
+            for (int i = lane; i < n_basic; i += NT) AD[p.dense_pos[i]] = A[i];
         } else {
             for (int e = lane; e < p.nq * p.nmp; e += NT) {
                 const int src = p.dense_src[e];
@@ -1133,11 +1144,11 @@ int table_entries(const MtpPlanDevice& p, int K, bool loss)
 }
 
 template <typename T>
-size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC)
+size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC, int nt)
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
-    const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots);
-    size_t n = (size_t)p.n_moms * (loss ? 4 : 2) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
+    const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots, nt);
+    size_t n = (size_t)p.n_moms * (loss ? 4 : 1) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
     if (H > 0) n += (size_t)p.n_scalar + (loss ? 5 : 1) * (size_t)H;     // network inputs and per-neuron values
@@ -1181,29 +1192,35 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
 template <typename T, bool LOSS, bool SEED = false>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
+    const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
     auto lds_for = [&](int nc, size_t* main) {
-        *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc) + 15) / 16 * 16;
-        // the packed basic-moment table; energy / force / virial kernel: + the monomial rows and the dense-array map
-        return *main + (LOSS ? (size_t)a.p.n_basic : 2 * (size_t)a.p.n_basic + a.p.nrows) * sizeof(unsigned);
+        *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc, wide ? 256 : 64) + 15) / 16 * 16;
+        // the packed basic-moment table; energy / force / virial kernel: + the monomial rows
+        return *main + (LOSS ? (size_t)a.p.n_basic : (size_t)a.p.n_basic + a.p.nrows) * sizeof(unsigned);
     };
     size_t lds_main = 0;
     int nc_cap = MTP_NC;
     size_t lds = lds_for(nc_cap, &lds_main);
-    // A longer table halves the chunks (table builds, barriers) of rows just above MTP_NC neighbours;
-    // taken only while as many workgroups still fit a CU.  The loss kernels keep MTP_NC.
-    if (!LOSS && lds <= 160 * 1024) {
-        const size_t per_cu = 160 * 1024, fit = per_cu / lds;
-        for (int nc = MTP_NC_MAX; nc > MTP_NC; nc -= 8) {
-            size_t m = 0;
+    // Rows of the neighbour table (energy / force / virial kernel; the loss kernels keep MTP_NC): the kernel waits on
+    // dependent LDS reads and barriers, so workgroups per CU count first (level 16: 12 -> 16 workgroups, 0.136 -> 0.122 ms
+    // although rows of more than 20 neighbours then take two chunks), and among the tables that allow as many
+    // workgroups as the registers do (four waves per SIMD), or as the shortest table does, the longest is taken
+    // (level 20: a row of 35 neighbours in one chunk instead of two, 0.45 -> 0.41 ms).
+    if (!LOSS) {
+        // LDS is handed out in pieces of 1280 bytes on this chip
+        auto per_cu = [](size_t l) { return (size_t)(160 * 1024) / ((l + 1279) / 1280 * 1280); };
+        size_t m = 0;
+        const size_t by_registers = wide ? 4 : 16;
+        const size_t want = std::min(by_registers, per_cu(lds_for(MTP_NC_MIN, &m)));
+        for (int nc : {MTP_NC_MAX, 40, 32, 24, 20, MTP_NC_MIN}) {
             const size_t l = lds_for(nc, &m);
-            if (per_cu / l == fit) { nc_cap = nc; lds = l; lds_main = m; break; }
+            if (per_cu(l) >= want || nc == MTP_NC_MIN) { nc_cap = nc; lds = l; lds_main = m; break; }
         }
     }
     const_cast<MtpArgs<T>&>(a).lds_basic_off = (int)lds_main;
     const_cast<MtpArgs<T>&>(a).nc_cap = nc_cap;
     A2P_REQUIRE(lds <= 160 * 1024, A2P_ERR_INVALID,
                 "mtp: %d moments need %zu bytes of LDS per atom; this level is too large", a.p.n_moms, lds);
-    const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
     auto kern = wide ? mtp_atom_kernel<T, LOSS, 256, SEED> : mtp_atom_kernel<T, LOSS, 64, SEED>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
