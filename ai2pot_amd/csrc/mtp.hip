@@ -46,9 +46,10 @@ __host__ __device__ inline bool mtp_gred_in_moments(bool loss, int n_moms)
 // entries of the region that holds the neighbour table (+ group sums) and doubles as the sweeps' partial sums.
 // In the energy / force / virial kernel the group sums (4 per thread) are written over the table once every
 // thread has finished reading it.
-// The adjoints of the energy / force / virial kernel live in this region too, behind the partial sums: they are
-// needed from the end of the forward sweep to the gathering of the dense adjoint array, which is when the
-// neighbour table is not (mtp_adjoint_offset).
+// The adjoints live in this region too, behind the partial sums (mtp_adjoint_offset): they are needed from the end of
+// the forward sweep to the last pass over the neighbours, which is when the neighbour table is not.  That pass needs
+// the adjoints of the basic moments only: the energy / force / virial kernel gathers them into its dense array, the
+// loss kernel copies them behind the region first.
 __host__ __device__ inline int mtp_adjoint_offset(int max_level_slots)
 {
     return ((max_level_slots > 8 ? max_level_slots : 8) + 1) & ~1;     // at least the scratch of a block sum
@@ -57,7 +58,8 @@ __host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_
 {
     int a = loss ? nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4) : nc * E;
     if (!loss && a < nt * 4) a = nt * 4;          // four group sums per thread
-    const int b = loss ? max_level_slots * 2 : mtp_adjoint_offset(max_level_slots) + n_moms;
+    // loss mode: two partial-sum arrays, then the adjoints and the mixed adjoints
+    const int b = loss ? mtp_adjoint_offset(2 * max_level_slots) + 2 * n_moms : mtp_adjoint_offset(max_level_slots) + n_moms;
     return a > b ? a : b;
 }
 // the dense adjoint array of the pair-derivative pass takes the place of the moments when it fits
@@ -399,21 +401,25 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     const int ncoef = a.ntypes * a.ntypes * nmus * K;
 
     const int MTP_NC = a.nc_cap;
-    // moments | (loss mode: their tangents) | adjoints | (loss mode: mixed adjoints)
+    // moments | (loss mode: their tangents) | coefficients | region of the neighbour table
     T* M = (T*)smem_raw;
     T* Tg = M + n_moms;
-    T* Bm = Tg + (LOSS ? 2 * n_moms : 0);    // loss mode: the adjoints sit between the tangents and the mixed adjoints
-    T* cf = Bm + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
+    T* cf = Tg + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
     T* tab = cf + a.ntypes * nmus * K;
-    // energy / force / virial kernel: the adjoints share the table's region (behind the sweeps' partial sums)
-    T* A = LOSS ? Tg + n_moms : tab + mtp_adjoint_offset(p.max_level_slots);
+    // the adjoints (loss mode: and the mixed adjoints) share the table's region, behind the sweeps' partial sums
+    T* A = tab + mtp_adjoint_offset((LOSS ? 2 : 1) * p.max_level_slots);
+    T* Bm = A + n_moms;
     // [256/32][32][4] partial sums of the thread groups.  They are needed only in the last pass over the
     // neighbours, when the moments (and, in loss mode, their tangents) are dead: a long enough moment
     // vector lends them its place
     const bool share = mtp_gred_in_moments(LOSS, n_moms);
     // energy / force / virial kernel: the group sums are written over the table once it has been read
     T* gred = LOSS ? (share ? M : tab + MTP_NC * E) : tab;
-    T* pq = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots, NT);   // loss mode: P[nc][nmus] | Q[nc][nmus]
+    // loss mode, behind the region: adjoints and mixed adjoints of the basic moments (copies for the last pass) |
+    // P[nc][nmus] | Q[nc][nmus] | ...
+    T* Ab = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots, NT);
+    T* Bb = Ab + n_basic;
+    T* pq = LOSS ? Bb + n_basic : Ab;
 
     if (ii >= a.binum[b]) {                  // padded row: contributes nothing
         if (!LOSS && a.partial && lane < 10) a.partial[row * 10 + lane] = 0.0;
@@ -446,7 +452,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     for (int q = lane; q < a.ntypes * nmus * K; q += NT) cf[q] = a.coeffs[(size_t)ti * a.ntypes * nmus * K + q];
     for (int i = lane; i < n_moms; i += NT) {
         M[i] = (T)0;
-        if (LOSS) { A[i] = (T)0; Tg[i] = (T)0; Bm[i] = (T)0; }
+        if (LOSS) Tg[i] = (T)0;
     }
     __syncthreads();
 
@@ -484,10 +490,11 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
 
     // ---- products, energy, adjoint ------------------------------------------------------------
     sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
-    if (!LOSS) {                              // the table is dead: its place now holds the adjoints
-        for (int i = lane; i < n_moms; i += NT) A[i] = (T)0;
-        __syncthreads();
+    for (int i = lane; i < n_moms; i += NT) {    // the table is dead: its place now holds the adjoints
+        A[i] = (T)0;
+        if (LOSS) Bm[i] = (T)0;
     }
+    __syncthreads();
     T e_part = (T)0;
     // network buffers (H > 0): inputs q[S]; per neuron w1 tanh', and in loss mode tanh, tanh', tanh'', tau
     T* nnb = LOSS ? pq + 2 * MTP_NC * nmus + MTP_NC + a.ntypes * nmus * K : pq;
@@ -669,6 +676,8 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
         const T cE = seeded ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
         // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
         if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
+        // the last pass needs the adjoints of the basic moments while the table is back in its region
+        for (int i = lane; i < n_basic; i += NT) { Ab[i] = A[i]; Bb[i] = Bm[i]; }
         T* grow = a.gpart + row * a.ngrad;
         for (int q = lane; q < a.ngrad; q += NT) grow[q] = (T)0;
         __syncthreads();         // other threads overwrite some of these entries below
@@ -730,8 +739,8 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
                         const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
                                      (T)eb * xa * t[OY + max(eb - 1, 0)] * zc * t[OW + 1] +
                                      (T)ec * xa * yb * t[OZ + max(ec - 1, 0)] * t[OW + 2];
-                        const T adj = A[i];
-                        Pv += (cE * adj + Bm[i]) * m + adj * rinv * (gm - (T)(ea + eb + ec) * m * wu);
+                        const T adj = Ab[i];
+                        Pv += (cE * adj + Bb[i]) * m + adj * rinv * (gm - (T)(ea + eb + ec) * m * wu);
                         Qv += adj * m * wu;
                     }
                 }
@@ -1148,7 +1157,8 @@ size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, in
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
     const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots, nt);
-    size_t n = (size_t)p.n_moms * (loss ? 4 : 1) + tabs + (size_t)ntypes * p.nmus * K;   // + the coefficient copy
+    size_t n = (size_t)p.n_moms * (loss ? 2 : 1) + tabs + (loss ? 2 * (size_t)p.n_basic : 0) +
+               (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
     if (loss) n += 2 * (size_t)MTP_NC * p.nmus + MTP_NC + (size_t)ntypes * p.nmus * K;
     if (H > 0) n += (size_t)p.n_scalar + (loss ? 5 : 1) * (size_t)H;     // network inputs and per-neuron values
