@@ -288,6 +288,26 @@ __device__ __forceinline__ void entry_store<double>(double* p, double x, double 
     *reinterpret_cast<double2*>(p) = make_double2(x, y);
     *reinterpret_cast<double2*>(p + 2) = make_double2(z, __longlong_as_double((long long)bits));
 }
+// The same, streamed past the caches (non-temporal): for the compact entries, which are written once and read by other
+// kernels later; ordinary stores of this much data (1.6 GB per build of a million atoms, with the padded rows) cost the
+// list kernel a quarter of its time.
+template <typename T>
+__device__ __forceinline__ void entry_store_stream(T* p, T x, T y, T z, int bits);
+template <>
+__device__ __forceinline__ void entry_store_stream<float>(float* p, float x, float y, float z, int bits)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4 v = {x, y, z, __int_as_float(bits)};
+    __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(p));
+}
+template <>
+__device__ __forceinline__ void entry_store_stream<double>(double* p, double x, double y, double z, int bits)
+{
+    typedef double f64x2 __attribute__((ext_vector_type(2)));
+    const f64x2 lo = {x, y}, hi = {z, __longlong_as_double((long long)bits)};
+    __builtin_nontemporal_store(lo, reinterpret_cast<f64x2*>(p));
+    __builtin_nontemporal_store(hi, reinterpret_cast<f64x2*>(p + 2));
+}
 
 // the reverse: one 16-byte (fp32) or two 16-byte (fp64) loads
 __device__ __forceinline__ void entry_load(const float* p, float& x, float& y, float& z, int& bits)
@@ -819,7 +839,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             if (e0 == 0) {                        // wave-uniform
                 first_dx = dx; first_dy = dy; first_dz = dz; first_bits = bits; first_slot = slot;
             } else if (slot >= 0) {
-                entry_store<T>(base + (((unsigned)slot >> 3) << 11) + (((unsigned)slot & 7u) << 2), dx, dy, dz, bits);
+                entry_store_stream<T>(base + (((unsigned)slot >> 3) << 11) + (((unsigned)slot & 7u) << 2), dx, dy, dz, bits);
             }
             n_inner += __popcll(mi);
             n_outer += __popcll(mo);
@@ -844,11 +864,12 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             rb_rcs[i * 3 + 0] = (T)0; rb_rcs[i * 3 + 1] = (T)0; rb_rcs[i * 3 + 2] = (T)0;
         }
         __builtin_amdgcn_wave_barrier();
-        for (int i = lane; i < live / 4; i += 64) d1[i] = s1[i];
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));    // non-temporal, as the compact entries
+        for (int i = lane; i < live / 4; i += 64) __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&s1[i]), reinterpret_cast<u32x4*>(&d1[i]));
         const uint4* s2 = reinterpret_cast<const uint4*>(rb_rcs);
         uint4* d2 = reinterpret_cast<uint4*>(rcs + rowi * 3);
         const int nv = (int)((size_t)live * 3 * sizeof(T) / 16);
-        for (int i = lane; i < nv; i += 64) d2[i] = s2[i];
+        for (int i = lane; i < nv; i += 64) __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&s2[i]), reinterpret_cast<u32x4*>(&d2[i]));
         if (RANK) {                                                    // slots past the row's end are not defined
             const uint4* s3 = reinterpret_cast<const uint4*>(rb_rank);
             uint4* d3 = reinterpret_cast<uint4*>(rank_out + rowi);
@@ -862,7 +883,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
         pad_fill(rcs + rowi * 3, first_pad * 3, last_pad * 3, (T)0, lane);
     }
     if (COMPACT && first_slot >= 0)
-        entry_store<T>(compact_base + (((unsigned)first_slot >> 3) << 11) + (((unsigned)first_slot & 7u) << 2), first_dx,
+        entry_store_stream<T>(compact_base + (((unsigned)first_slot >> 3) << 11) + (((unsigned)first_slot & 7u) << 2), first_dx,
                        first_dy, first_dz, first_bits);
     start = nstart;
     len = nlen;

@@ -77,6 +77,21 @@ __device__ __forceinline__ void st4(double* p, const double (&v)[4])
     *reinterpret_cast<double2*>(p) = make_double2(v[0], v[1]);
     *reinterpret_cast<double2*>(p + 2) = make_double2(v[2], v[3]);
 }
+// the same past the caches (non-temporal): for the list entries, which a kernel streams through once or twice; with
+// ordinary loads they push the rows that many lanes gather (contracted coefficients, slots) out of the L2
+__device__ __forceinline__ void ld4_stream(const float* p, float (&o)[4])
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void ld4_stream(const double* p, double (&o)[4])
+{
+    typedef double f64x2 __attribute__((ext_vector_type(2)));
+    const f64x2 v0 = __builtin_nontemporal_load(reinterpret_cast<const f64x2*>(p));
+    const f64x2 v1 = __builtin_nontemporal_load(reinterpret_cast<const f64x2*>(p + 2));
+    o[0] = v0.x; o[1] = v0.y; o[2] = v1.x; o[3] = v1.y;
+}
 __device__ __forceinline__ int entry_bits(float w) { return __float_as_int(w); }
 __device__ __forceinline__ int entry_bits(double w) { return (int)__double_as_longlong(w); }
 
@@ -148,7 +163,7 @@ template <typename T>
 __device__ __forceinline__ void chunk_load(const T* __restrict__ g, int lane, T (&v)[CL_CHUNK][4])
 {
 #pragma unroll
-    for (int it = 0; it < CL_CHUNK; it++) ld4(g + (size_t)(it * 64 + lane) * 4, v[it]);
+    for (int it = 0; it < CL_CHUNK; it++) ld4_stream(g + (size_t)(it * 64 + lane) * 4, v[it]);
 }
 template <typename T>
 __device__ __forceinline__ void chunk_store(T* __restrict__ st, int lane, const T (&v)[CL_CHUNK][4])
