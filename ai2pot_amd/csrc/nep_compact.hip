@@ -77,8 +77,8 @@ __device__ __forceinline__ void st4(double* p, const double (&v)[4])
     *reinterpret_cast<double2*>(p) = make_double2(v[0], v[1]);
     *reinterpret_cast<double2*>(p + 2) = make_double2(v[2], v[3]);
 }
-// the same past the caches (non-temporal): for the list entries, which a kernel streams through once or twice; with
-// ordinary loads they push the rows that many lanes gather (contracted coefficients, slots) out of the L2
+// the same past the caches (non-temporal): for the list entries and the filled slots, which a kernel streams through
+// once or twice; with ordinary loads they push the rows that many lanes gather (contracted coefficients) out of the L2
 __device__ __forceinline__ void ld4_stream(const float* p, float (&o)[4])
 {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -644,7 +644,7 @@ nep_gather_kernel(const GatherArgs<T> a)
         bool ok = true;
         for (int t = 0; t < min(n, NSLOT); t++) {
             T v[4];
-            ld4(a.slots + ((size_t)t * a.cv.natoms + p) * 4, v);
+            ld4_stream(a.slots + ((size_t)t * a.cv.natoms + p) * 4, v);        // read once
             ok = ok && fabs((double)v[0]) < kFixedSumLimit && fabs((double)v[1]) < kFixedSumLimit &&
                  fabs((double)v[2]) < kFixedSumLimit;
             sx.add(v[0]); sy.add(v[1]); sz.add(v[2]);
