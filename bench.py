@@ -135,9 +135,9 @@ def timed_replay(replay, steps, warmup):
 # counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
 # summarised in profiles/<workload>_hbm_traffic.txt.  Kernels without a counter run report null.
 MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nbl_lists"): (2.00 * 2.459e5 + 1.645e6) * 1024,
-    ("nep_md_1048576", "nep_adjoint_kernel"): (2.00 * 6.189e5 + 6.653e5) * 1024,
-    ("nep_md_1048576", "nep_gather_kernel"): (2.00 * 7.231e5 + 3.855e4) * 1024,
+    ("nep_md_1048576", "nbl_lists"): (2.00 * 2.082e5 + 1.640e6) * 1024,
+    ("nep_md_1048576", "nep_adjoint_kernel"): (2.00 * 6.065e5 + 6.429e5) * 1024,
+    ("nep_md_1048576", "nep_gather_kernel"): (2.00 * 5.695e5 + 3.582e4) * 1024,
 }
 
 
