@@ -46,11 +46,14 @@ enum WsSlot {
     WS_FLAGS,          // device-side status words
     WS_MISC,
     WS_GRID,           // neighbor-list: the bin grid derived on the device (builds without read-back)
+    WS_NEP_CLAIMS,     // NEP on compact lists: counters of claimed places and spare rows; zero between calls
     WS_NSLOTS
 };
 // Returns a device pointer valid until the next ws_get on the same slot with a larger size.
 // Growth synchronises the device (hipFree); steady-state calls do not allocate.
+// WS_FLAGS and WS_NEP_CLAIMS are zero-filled when they are allocated; their users leave them zero.
 int ws_get(int slot, size_t bytes, void** out);
+int ws_drop(int slot); // synchronises the device and frees one buffer of the current device (its contents are suspect)
 size_t ws_bytes();     // held on the current device
 int ws_release();      // synchronises the device, frees the current device's buffers
 
@@ -71,6 +74,9 @@ inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 // totals.  Disabled (the default) it costs one branch.
 void prof_begin(const char* label, hipStream_t stream);
 void prof_end(hipStream_t stream);
+// Orders this library's work across streams of a device (device synchronisation when the stream changes; a stream
+// under capture is left alone).  prof_begin calls it; entry points that launch without prof_begin call it first.
+int enter_stream(hipStream_t stream);
 struct ProfScope {
     hipStream_t s;
     ProfScope(const char* label, hipStream_t stream) : s(stream) { prof_begin(label, stream); }

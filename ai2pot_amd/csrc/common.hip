@@ -51,9 +51,26 @@ int ws_get(int slot, size_t bytes, void** out)
         size_t want = bytes + bytes / 8 + 256;      // head-room so small growth does not realloc
         A2P_HIP_CHECK(hipMalloc(&b.ptr, want));
         b.bytes = want;
-        if (slot == WS_FLAGS) A2P_HIP_CHECK(hipMemset(b.ptr, 0, want));
+        if (slot == WS_FLAGS || slot == WS_NEP_CLAIMS) A2P_HIP_CHECK(hipMemset(b.ptr, 0, want));
     }
     *out = b.ptr;
+    return A2P_OK;
+}
+
+int ws_drop(int slot)
+{
+    int dev = 0;
+    A2P_HIP_CHECK(hipGetDevice(&dev));
+    A2P_HIP_CHECK(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if ((int)g_ws.size() <= dev) return A2P_OK;
+    Buf& b = g_ws[dev].slot[slot];
+    if (b.ptr) {
+        A2P_HIP_CHECK(hipFree(b.ptr));
+        g_ws_generation++;
+    }
+    b.ptr = nullptr;
+    b.bytes = 0;
     return A2P_OK;
 }
 
@@ -117,33 +134,36 @@ bool prof_event(hipEvent_t* e)
 }  // namespace
 
 // The workspace is shared by every call on a device, so work of this library on two streams must not overlap.
-// Every launch passes through prof_begin: when the stream differs from the one the previous launch on this device
-// used, the device is synchronised first (callers that keep to one stream never pay for it).  A stream that is being
-// captured is left alone: a capture keeps to itself, and its replays are ordered by whoever launches them.
+// Every launch passes through prof_begin, which calls enter_stream: when the stream differs from the one the
+// previous launch on this device used, the device is synchronised first (callers that keep to one stream never
+// pay for it).  Entry points whose launches are not bracketed by prof_begin call enter_stream themselves.  A
+// stream that is being captured is left alone: a capture keeps to itself, and its replays are ordered by whoever
+// launches them.
 namespace {
 std::mutex g_stream_mutex;
 std::vector<hipStream_t> g_last_stream;
 std::vector<char> g_have_stream;
+}  // namespace
 
-void order_streams(hipStream_t stream)
+int enter_stream(hipStream_t stream)
 {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return;
+    A2P_HIP_CHECK(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_stream_mutex);
     if ((int)g_last_stream.size() <= dev) { g_last_stream.resize(dev + 1, nullptr); g_have_stream.resize(dev + 1, 0); }
-    if (g_have_stream[dev] && g_last_stream[dev] == stream) return;
+    if (g_have_stream[dev] && g_last_stream[dev] == stream) return A2P_OK;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &st) != hipSuccess) { (void)hipGetLastError(); return; }
-    if (st != hipStreamCaptureStatusNone) return;
-    if (g_have_stream[dev]) (void)hipDeviceSynchronize();
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) { (void)hipGetLastError(); return A2P_OK; }
+    if (st != hipStreamCaptureStatusNone) return A2P_OK;
+    if (g_have_stream[dev]) A2P_HIP_CHECK(hipDeviceSynchronize());
     g_last_stream[dev] = stream;
     g_have_stream[dev] = 1;
+    return A2P_OK;
 }
-}  // namespace
 
 void prof_begin(const char* label, hipStream_t stream)
 {
-    order_streams(stream);
+    (void)enter_stream(stream);        // a failed synchronisation stays pending and fails the call's own check
     if (!g_prof_on) return;
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (!g_prof_select.empty() && g_prof_select.find("," + std::string(label) + ",") == std::string::npos) return;

@@ -252,6 +252,8 @@ int virial_fwd_noalloc(int B, int P, int U, const int* bnumneigh, const float* r
     double* partial = nullptr;
     rc = scratch_address(&partial);
     if (rc) return rc;
+    rc = enter_stream(stream);          // the scratch is shared by every stream of the device
+    if (rc) return rc;
     // every row below batch * nlocal is written by the first kernel before the second reads it, so
     // what an earlier call left in the buffer never shows; nlocal == 0 leaves nothing to sum (zeros)
     if (P > 0) {

@@ -571,7 +571,7 @@ template <typename T>
 struct CompactEmit {
     const int* order;   // position -> atom
     const T* xs;        // [natoms][3] Cartesian coordinates in processing order
-    const int* inv;     // [natoms] atom -> position; every value in [0, natoms)
+    const int* inv;     // [natoms] atom -> position (for an order that is no permutation: leftovers in places)
     T* entries;
     int* n_outer;
     int* n_inner;
@@ -595,6 +595,7 @@ __device__ T pair_symmetric_d2(const Grid<T>& g, const T* __restrict__ x, const 
 {
     const T d[3] = {dx, dy, dz};
     T e[3], v[3];
+    j = min(max(j, 0), g.N - 1);                     // positions come from the inverse of a caller-writable order
 #pragma unroll
     for (int a = 0; a < 3; a++) {
         e[a] = sub_rn(x[(size_t)j * 3 + a], c[a]);
@@ -659,7 +660,9 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
 #pragma unroll
     for (int a = 0; a < NBL_APW; a++) {
         const int q = min(p0 + a, g.N - 1);
-        atom[a] = COMPACT ? ce.order[q] : q;
+        // the caller may write the order: an index outside the structure must not reach an address
+        // (compact_symmetry_kernel reports it)
+        atom[a] = COMPACT ? min(max(ce.order[q], 0), g.N - 1) : q;
     }
 #pragma unroll
     for (int a = 0; a < NBL_APW; a++)
@@ -818,7 +821,8 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
             // The entry names its neighbour by position in the processing order (what the force kernels index their
             // per-atom arrays with), the record and the padded row by atom: one gather per entry.  The first 64
             // entries (most rows have no more) do not wait for the answer here: they are stored after the padded
-            // row.  Every value of the inverse is a valid position (see where it is allocated).
+            // row.  A value of the inverse is a valid position unless the order is no permutation, which
+            // compact_symmetry_kernel reports; the consumers of the entries check the index they find.
             const int bits = ce.inv[word & (CL_IMAGE_BIT - 1)] | (word & ~CL_INDEX_MASK);
             const T d2 = dx * dx + dy * dy + dz * dz;
             const bool in_outer = have && d2 <= ce.outer2;
@@ -900,7 +904,7 @@ lists_kernel(const Grid<T> g_in, const T* __restrict__ x, const int* __restrict_
 template <typename T>
 __global__ void __launch_bounds__(NBL_BLOCK)
 compact_symmetry_kernel(const Grid<T> g_in, const GridDyn<T>* __restrict__ gd, const T* __restrict__ x,
-                        const CompactEmit<T> ce, int umax)
+                        const CompactEmit<T> ce, int umax, int* __restrict__ status)
 {
     extern __shared__ __align__(16) unsigned char sh_move[];     // per wave: umax entries of 4 values
     const Grid<T> g = with_dyn(g_in, gd);
@@ -908,6 +912,12 @@ compact_symmetry_kernel(const Grid<T> g_in, const GridDyn<T>* __restrict__ gd, c
     T* const mv = (T*)sh_move + (size_t)wv * umax * 4;
     const int p0 = (blockIdx.x * (NBL_BLOCK / 64) + wv) * 64;
     const int mine = p0 + lane < g.N ? ce.n_inner[p0 + lane] : 0;
+    // The processing order must name every atom once: an index outside the structure (clamped where it is used) or
+    // an atom named twice (then some atom has no row, and the inverse of the order holds leftovers) is reported.
+    if (p0 + lane < g.N) {
+        const int at = ce.order[p0 + lane];
+        if ((unsigned)at >= (unsigned)g.N || ce.inv[at] != p0 + lane) atomicOr(status, ST_BAD_NEIGHBOR);
+    }
     unsigned long long todo = __ballot((mine & CL_NEAR_FLAG) != 0);
     if (todo == 0ull) return;                     // whole wave
     const T band = ce.near_band;
@@ -1191,13 +1201,9 @@ struct GridBound {
     int rdim[3] = {0, 0, 0};
     double big = 0;    // largest |coordinate| of the box kept by that build
 };
-thread_local GridBound g_bound;
-// where the last inverse of a processing order was written (the workspace is per process, like this record)
-struct InverseAt {
-    const void* ptr = nullptr;
-    int N = 0, device = -1;
-};
-InverseAt g_inverse;
+// a few structures per host thread (two calculators used in turn keep both of their bounds), oldest replaced first
+constexpr size_t kMaxBounds = 8;
+thread_local std::vector<GridBound> g_bounds;
 thread_local int g_sync_free = 0;
 
 template <typename T>
@@ -1289,22 +1295,14 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     // the bin box: read back from the extents, or bounded by the box of the last synchronised build of this structure
     int device = 0;
     A2P_HIP_CHECK(hipGetDevice(&device));
-    {
-        // The list kernel uses values of the inverse unchecked, and an order that is no permutation (the caller may
-        // write the order) leaves some of them unwritten: the array starts from zeros whenever its memory may hold
-        // anything but an earlier inverse for the same number of atoms.
-        if (!co) {
-            g_inverse.ptr = nullptr;                   // this call's own arrays take the place
-        } else if (g_inverse.ptr != (const void*)inv || g_inverse.N != N || g_inverse.device != device) {
-            rc = fill_zero(inv, (size_t)N * sizeof(int), stream);
-            if (rc) return rc;
-            g_inverse.ptr = inv; g_inverse.N = N; g_inverse.device = device;
-        }
+    const GridBound* bound = nullptr;
+    for (const GridBound& gb : g_bounds) {
+        bool same = gb.valid && gb.device == device && gb.N == N && gb.is_cart == is_cart && gb.rcut == (double)g.rcut;
+        for (int a = 0; a < 3 && same; a++) same = gb.pbc[a] == (pbc[a] ? 1 : 0);
+        for (int q = 0; q < 9 && same; q++) same = gb.lattice[q] == (double)lattice[q];
+        if (same) { bound = &gb; break; }
     }
-    bool same = g_bound.valid && g_bound.device == device && g_bound.N == N && g_bound.is_cart == is_cart &&
-                g_bound.rcut == (double)g.rcut;
-    for (int a = 0; a < 3 && same; a++) same = g_bound.pbc[a] == (pbc[a] ? 1 : 0);
-    for (int q = 0; q < 9 && same; q++) same = g_bound.lattice[q] == (double)lattice[q];
+    const bool same = bound != nullptr;
     const bool sync_free = g_sync_free && same && !max_nn_host &&
                            (long long)N * g.nimg * (long long)(4 * sizeof(T)) <= (2ll << 30);
     GridDyn<T>* gd = nullptr;
@@ -1314,12 +1312,12 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
         int cap[3];
         int grow = 0;
         for (int a = 0; a < 3; a++) {
-            cap[a] = g_bound.rdim[a] + std::max(2, g_bound.rdim[a] / 8);
+            cap[a] = bound->rdim[a] + std::max(2, bound->rdim[a] / 8);
             g.rdim[a] = cap[a];                         // host copies of the box serve launch and scratch sizes only
             nregion *= cap[a];
-            grow = std::max(grow, cap[a] - g_bound.rdim[a]);
+            grow = std::max(grow, cap[a] - bound->rdim[a]);
         }
-        big_coord = g_bound.big + (double)(grow + 2) * (double)g.bin_size;   // the box cannot have moved further
+        big_coord = bound->big + (double)(grow + 2) * (double)g.bin_size;   // the box cannot have moved further
         A2P_REQUIRE(nregion < (1ll << 30), A2P_ERR_INVALID, "nblist: %lld bins around the centre atoms", nregion);
         void* wsG = nullptr;
         rc = ws_get(WS_GRID, 256, &wsG);
@@ -1362,11 +1360,18 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
                     nregion);
         for (int a = 0; a < 3; a++)
             big_coord = std::max(big_coord, std::max(std::fabs((double)g.keep_lo[a]), std::fabs((double)g.keep_hi[a])));
-        g_bound.big = big_coord;
-        g_bound.valid = true;
-        g_bound.device = device; g_bound.N = N; g_bound.is_cart = is_cart; g_bound.rcut = (double)g.rcut;
-        for (int a = 0; a < 3; a++) { g_bound.pbc[a] = pbc[a] ? 1 : 0; g_bound.rdim[a] = g.rdim[a]; }
-        for (int q = 0; q < 9; q++) g_bound.lattice[q] = (double)lattice[q];
+        GridBound nb;
+        nb.big = big_coord;
+        nb.valid = true;
+        nb.device = device; nb.N = N; nb.is_cart = is_cart; nb.rcut = (double)g.rcut;
+        for (int a = 0; a < 3; a++) { nb.pbc[a] = pbc[a] ? 1 : 0; nb.rdim[a] = g.rdim[a]; }
+        for (int q = 0; q < 9; q++) nb.lattice[q] = (double)lattice[q];
+        if (bound) {
+            g_bounds[bound - g_bounds.data()] = nb;
+        } else {
+            if (g_bounds.size() >= kMaxBounds) g_bounds.erase(g_bounds.begin());
+            g_bounds.push_back(nb);
+        }
     }
     const int nb1 = (int)nregion + 1;
 
@@ -1517,7 +1522,7 @@ int nblist_build(const T* lattice, const int* types, const T* coords, int N, dou
     if (co) {
         prof_begin("nbl_symmetry", stream);
         hipLaunchKernelGGL(compact_symmetry_kernel<T>, dim3(ceil_div(N, NBL_BLOCK)), dim3(NBL_BLOCK), (size_t)(NBL_BLOCK / 64) * umax * 4 * sizeof(T),
-                           stream, g, (const GridDyn<T>*)gd, (const T*)x, ce, umax);
+                           stream, g, (const GridDyn<T>*)gd, (const T*)x, ce, umax, status);
         prof_end(stream);
     }
     if (sort) {

@@ -11,7 +11,8 @@
 //                        more: g_ij with both parts, summed into F_i and the virial, and handed to atom j
 //                        through a slot array, slots[place][j], the place claimed with an atomic counter
 //                        per target (an atom is named by as many pairs as its own list has entries; places
-//                        beyond the array's depth fall back to atomic adds on a spare force array).
+//                        beyond the array's depth are added to a spare row of 64-bit integers in the fixed
+//                        point of the slot sums, so the result does not depend on their order either).
 //                        It also stores, per atom, the radial coefficients contracted with dE/dq,
 //                        cc_i[t][k] = sum_n dE_i/dq_n c[t_i][t][n][k] (species x 8 values).
 //   nep_gather_kernel  : the pairs between the cutoffs, which have a radial part only: g_ij - g_ji is a
@@ -49,8 +50,10 @@ struct GatherArgs {
     // the next four are indexed by position in the processing order, like the index field of the list entries
     T* rcc;               // [natoms][NTC * KC] radial coefficients contracted with dE/dq
     T* slots;             // [NSLOT][natoms][4] derivatives handed to the neighbour, by place
-    T* overflow;          // [natoms][3] the same for places >= NSLOT, summed with atomics (zero on entry)
-    int* incoming;        // [natoms] places claimed so far (zero on entry)
+    // the next two live in a workspace slot that is zero when a call starts: nep_gather_kernel clears what it read
+    unsigned long long* overflow;   // [natoms][OverflowRow<T>::WORDS] the same for places >= NSLOT: fixed-point sums
+    int* incoming;        // [natoms] places claimed so far
+    double overflow_limit; // largest magnitude a spare row accepts per value (sums of umax values must fit)
     T* force;             // [natoms][3] or null
     double* partial;      // [nblocks][10]: energy and virial, each workgroup's share
     int* status;
@@ -228,7 +231,8 @@ __device__ __forceinline__ bool position_header(const GatherArgs<T>& a, int p, i
 
 // Exact, order-independent sum of a few floating-point values: fixed point in 64-bit integers.
 // fp32 values are kept to 2^-40 (a thousandth of the last bit of a 1e-3 eV/A component), fp64 values in two
-// limbs to 2^-84; |x| must stay below 2^22.
+// limbs to 2^-84.  The magnitudes summed into one FixedSum must stay below 2^21 IN TOTAL (kFixedSumLimit): the
+// callers track the sum of magnitudes and give NaN beyond it.
 template <typename T>
 struct FixedSum;
 template <>
@@ -248,7 +252,42 @@ struct FixedSum<double> {
     }
     __device__ __forceinline__ double value() const { return (double)hi * 0x1p-32 + (double)lo * 0x1p-84; }
 };
-constexpr double kFixedSumLimit = 4.0e6;
+constexpr double kFixedSumLimit = 0x1p21;
+
+// The spare row of an atom: the same fixed point, added to with 64-bit integer atomics (order-independent).
+// Word BAD counts values that were not finite or too large to convert; the reader then gives NaN.
+template <typename T>
+struct OverflowRow;
+template <>
+struct OverflowRow<float> {
+    static constexpr int WORDS = 4, BAD = 3;
+    static __device__ __forceinline__ void add(unsigned long long* row, int c, float x)
+    {
+        atomicAdd(row + c, (unsigned long long)(long long)((double)x * 0x1p40));
+    }
+    static __device__ __forceinline__ void take(unsigned long long* row, int c, FixedSum<float>& s)
+    {
+        s.s += (long long)row[c];
+        row[c] = 0ull;
+    }
+};
+template <>
+struct OverflowRow<double> {
+    static constexpr int WORDS = 8, BAD = 6;
+    static __device__ __forceinline__ void add(unsigned long long* row, int c, double x)
+    {
+        const double v = x * 0x1p32, h = trunc(v);
+        atomicAdd(row + 2 * c, (unsigned long long)(long long)h);
+        atomicAdd(row + 2 * c + 1, (unsigned long long)(long long)((v - h) * 0x1p52));
+    }
+    static __device__ __forceinline__ void take(unsigned long long* row, int c, FixedSum<double>& s)
+    {
+        s.hi += (long long)row[2 * c];
+        s.lo += (long long)row[2 * c + 1];
+        row[2 * c] = 0ull;
+        row[2 * c + 1] = 0ull;
+    }
+};
 
 template <typename T>
 struct AdjointLds {
@@ -537,9 +576,16 @@ nep_adjoint_kernel(const GatherArgs<T> a)
                     const T g4[4] = {gx, gy, gz, (T)0};
                     st4(a.slots + ((size_t)place * a.cv.natoms + j) * 4, g4);
                 } else {
-                    atomicAdd(a.overflow + (size_t)j * 3 + 0, gx);
-                    atomicAdd(a.overflow + (size_t)j * 3 + 1, gy);
-                    atomicAdd(a.overflow + (size_t)j * 3 + 2, gz);
+                    unsigned long long* row = a.overflow + (size_t)j * OverflowRow<T>::WORDS;
+                    // (a comparison with NaN is false)
+                    if (fabs((double)gx) < a.overflow_limit && fabs((double)gy) < a.overflow_limit &&
+                        fabs((double)gz) < a.overflow_limit) {
+                        OverflowRow<T>::add(row, 0, gx);
+                        OverflowRow<T>::add(row, 1, gy);
+                        OverflowRow<T>::add(row, 2, gz);
+                    } else {
+                        atomicAdd(row + OverflowRow<T>::BAD, 1ull);
+                    }
                 }
             }
             fx += gx; fy += gy; fz += gz;
@@ -638,28 +684,33 @@ nep_gather_kernel(const GatherArgs<T> a)
     });
 
     // what the neighbours inside the angular cutoff handed over: F_i -= sum_j g_ji
-    if (active && a.force) {
+    if (p < a.cv.natoms && a.force) {
         const int n = a.incoming[p];
+        a.incoming[p] = 0;                                  // the next call finds the counters at zero
         FixedSum<T> sx, sy, sz;
-        bool ok = true;
+        double mag = 0.0;                                   // NaN or inf in a slot makes this NaN or inf
         for (int t = 0; t < min(n, NSLOT); t++) {
             T v[4];
             ld4_stream(a.slots + ((size_t)t * a.cv.natoms + p) * 4, v);        // read once
-            ok = ok && fabs((double)v[0]) < kFixedSumLimit && fabs((double)v[1]) < kFixedSumLimit &&
-                 fabs((double)v[2]) < kFixedSumLimit;
+            mag += fabs((double)v[0]) + fabs((double)v[1]) + fabs((double)v[2]);
             sx.add(v[0]); sy.add(v[1]); sz.add(v[2]);
         }
-        double ox = 0.0, oy = 0.0, oz = 0.0;
+        bool ok = mag < kFixedSumLimit;
         if (n > NSLOT) {
-            ox = (double)a.overflow[(size_t)p * 3 + 0];
-            oy = (double)a.overflow[(size_t)p * 3 + 1];
-            oz = (double)a.overflow[(size_t)p * 3 + 2];
+            unsigned long long* row = a.overflow + (size_t)p * OverflowRow<T>::WORDS;
+            ok = ok && row[OverflowRow<T>::BAD] == 0ull;
+            row[OverflowRow<T>::BAD] = 0ull;
+            OverflowRow<T>::take(row, 0, sx);
+            OverflowRow<T>::take(row, 1, sy);
+            OverflowRow<T>::take(row, 2, sz);
         }
-        T* fo = a.force + (size_t)atom * 3;
-        const double nan = __longlong_as_double(0x7ff8000000000000ll);
-        fo[0] = (T)(ok ? (double)fo[0] + (double)fx - sx.value() - ox : nan);
-        fo[1] = (T)(ok ? (double)fo[1] + (double)fy - sy.value() - oy : nan);
-        fo[2] = (T)(ok ? (double)fo[2] + (double)fz - sz.value() - oz : nan);
+        if (active) {
+            T* fo = a.force + (size_t)atom * 3;
+            const double nan = __longlong_as_double(0x7ff8000000000000ll);
+            fo[0] = (T)(ok ? (double)fo[0] + (double)fx - sx.value() : nan);
+            fo[1] = (T)(ok ? (double)fo[1] + (double)fy - sy.value() : nan);
+            fo[2] = (T)(ok ? (double)fo[2] + (double)fz - sz.value() : nan);
+        }
     }
     // every pair between the cutoffs was met from both ends: half of this sum is their virial
     if (a.want_virial) {
@@ -757,19 +808,18 @@ int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const
     if (rc) return rc;
     a.partial = (double*)ws;
     const bool pairs = force != nullptr || virial != nullptr;
-    // rcc | slots | overflow | incoming; the last two start every call at zero
     const size_t n_rcc = (size_t)natoms * ntc_of(ntypes) * KC, n_slots = (size_t)NSLOT * natoms * 4;
-    const size_t zero_bytes = (size_t)natoms * (3 * sizeof(T) + sizeof(int));
-    rc = ws_get(WS_PAIR_G, (n_rcc + n_slots) * sizeof(T) + zero_bytes, &ws);
+    rc = ws_get(WS_PAIR_G, (n_rcc + n_slots) * sizeof(T), &ws);
     if (rc) return rc;
     a.rcc = (T*)ws;
     a.slots = a.rcc + n_rcc;
-    a.overflow = a.slots + n_slots;
-    a.incoming = (int*)(a.overflow + (size_t)natoms * 3);
-    if (force) {
-        rc = fill_zero(a.overflow, zero_bytes, stream);
-        if (rc) return rc;
-    }
+    // spare rows | counters of claimed places: zero when allocated, and nep_gather_kernel leaves them zero
+    const size_t ovf_bytes = (size_t)natoms * OverflowRow<T>::WORDS * sizeof(unsigned long long);
+    rc = ws_get(WS_NEP_CLAIMS, ovf_bytes + (size_t)natoms * sizeof(int), &ws);
+    if (rc) return rc;
+    a.overflow = (unsigned long long*)ws;
+    a.incoming = (int*)((unsigned char*)ws + ovf_bytes);
+    a.overflow_limit = kFixedSumLimit / (double)umax;       // umax values of that size still sum below 2^21
     auto launch = [&](auto nr) {
         constexpr int NR = decltype(nr)::value;
         switch (ntc_of(ntypes)) {
@@ -780,7 +830,10 @@ int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const
         }
     };
     rc = n_r == 4 ? launch(std::integral_constant<int, 4>{}) : launch(std::integral_constant<int, 6>{});
-    if (rc) return rc;
+    if (rc) {
+        (void)ws_drop(WS_NEP_CLAIMS);       // a launch that failed may have left counters behind
+        return rc;
+    }
     return finish_energy_virial<T>(etot, virial, a.partial, 1, nblocks, stream);
 }
 

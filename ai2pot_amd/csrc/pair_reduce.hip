@@ -473,10 +473,12 @@ extern "C" int a2p_pair_incoming_max(int batch, int natoms_pad, int umax, int ng
     A2P_REQUIRE(binum && bnumneigh && bfirstneigh && max_incoming, A2P_ERR_INVALID, "pair_incoming_max: null pointer");
     *max_incoming = 0;
     if (batch == 0 || natoms_pad == 0) return A2P_OK;
+    int rc = enter_stream(stream);
+    if (rc) return rc;
     const int NF = natoms_pad + nghost;
     const size_t n = (size_t)batch * NF;
     void* ws = nullptr;
-    int rc = ws_get(WS_CSR, (n + 64) * sizeof(int), &ws);
+    rc = ws_get(WS_CSR, (n + 64) * sizeof(int), &ws);
     if (rc) return rc;
     void* flags = nullptr;
     rc = ws_get(WS_FLAGS, 64, &flags);

@@ -239,9 +239,12 @@ int a2p_nblist_build_ranked_f64(const double* lattice, const int* types, const d
  * in fixed point, so the result does not depend on the order of the claims: bit-reproducible.  For a pair
  * between the cutoffs g_ij - g_ji is evaluated by both ends from 32 gathered bytes of the other's
  * adjoints: nothing stored per pair.  The slots (32 per atom, 16 or 32 bytes each) live in the library's
- * workspace; an atom named by more than 32 pairs inside the angular cutoff receives the rest through
- * floating-point atomics (summation order, hence the last bits, may then vary between calls).  A pair
- * derivative of 4e6 or more in magnitude (eV/A) makes the receiving atom's force NaN.
+ * workspace; an atom named by more than 32 pairs inside the angular cutoff receives the rest through a
+ * spare row of 64-bit integers in the same fixed point, added to with integer atomics: bit-reproducible as
+ * well.  The fixed point holds sums of magnitudes below 2^21 eV/A: when the magnitudes handed to one atom
+ * through its slots add up to more, or one value sent to a spare row reaches 2^21 / umax, that atom's
+ * force is NaN.  The counters of claimed places and the spare rows are zero between calls (the second
+ * kernel clears what it read), so a call launches no fill kernel.
  * Model shapes: chebyshev_size 8, n_radial 4 or 6,
  * n_angular 4, l_max 4, at most 4 species (A2P_ERR_INVALID otherwise: use a2p_nep_efv_*).
  * types[natoms] are the type indices the list was built with.  etot[1] is required; force[natoms][3]

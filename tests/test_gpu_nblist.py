@@ -158,6 +158,40 @@ def test_config5_recipe_reduced(oracle):
     assert np.array_equal(counts, numneigh)
 
 
+def test_config5_full_size_bit_exact(oracle):
+    """The benchmark's own structure (1,048,576 atoms, L = 316.7 A, fp32, umax 200, unsorted) against the oracle on
+    the host, every row: numneigh, firstneigh with its order, rcs bit for bit, the -1 / 0 padding included -- through
+    the NumPy entry point (a fresh build) and through the device-resident step the benchmark times (compact build
+    with padded rows, processing order along the space-filling curve; an in-place rebuild on top of the first)."""
+    import torch
+    from ai2pot_amd.calculator import NepCalculator
+    lat, pos = synth.fcc_cell(64, 316.7 / 64.0, 0.15, 1006)
+    n = pos.shape[0]
+    assert n == 1048576
+    types = synth.rng_randint(2006, n, 3)
+    lat32, pos32 = lat.astype(np.float32), pos.astype(np.float32)
+    b = oracle.nblist(lat32, types, pos32, 7.0, 200)
+    a = gpu_list(lat32, types, pos32, 7.0, 200)
+    assert_same(a, b)
+    del a
+    calc = NepCalculator(synth.nep_model(seed=3006), n, lat, types, umax=200, dtype=torch.float32, device="cuda:0",
+                         path="gather")
+    x = torch.from_numpy(pos32).to("cuda:0")
+    calc.firstneigh.fill_(-7)
+    calc.rcs.fill_(float("nan"))
+    for build in range(2):                  # a build into buffers full of garbage, then a rebuild in place
+        calc.step(x)
+        torch.cuda.synchronize()
+        calc.check()
+        assert np.array_equal(calc.numneigh.cpu().numpy(), b[2])
+        first = calc.firstneigh.cpu().numpy()
+        bad = np.nonzero((first != b[3]).any(axis=1))[0]
+        assert bad.size == 0, "build %d: firstneigh (order, padding) differs in rows %s" % (build, bad[:10])
+        del first
+        assert np.array_equal(calc.rcs.cpu().numpy().view(np.uint32), b[4].view(np.uint32)), "rcs not bitwise identical"
+        assert np.array_equal(calc.ilist.cpu().numpy(), b[1]) and np.array_equal(calc.types_out.cpu().numpy(), b[5])
+
+
 def test_overflow_and_type_errors(oracle):
     lat, types, frac = synth.mos2_fixture()
     with pytest.raises(RuntimeError):

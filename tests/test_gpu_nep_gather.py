@@ -137,8 +137,10 @@ def test_model_shapes(oracle, cfg):
 @pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
 def test_more_pairs_inside_the_angular_cutoff_than_slots(oracle, np_dtype):
     """Equal cutoffs of 7 A at 0.04 atoms / A^3: every atom is named by about 57 pairs inside the angular cutoff,
-    more than the 32 hand-over slots, so the rest reaches it through the spare force array; also a structure
-    whose atoms have no pair between the cutoffs at all."""
+    more than the 32 hand-over slots, so the rest reaches it through the spare rows (integer atomics in the fixed
+    point of the slot sums): values against the oracle, and three evaluations bit for bit equal (which pair gets
+    which place, and the order of the atomic additions, differ from run to run).  Also a structure whose atoms
+    have no pair between the cutoffs at all."""
     n = 300
     lat, pos = synth.random_packed(n, [19.0, 20.0, 19.5], 2.0, 351)
     ty = synth.rng_randint(352, n, 3)
@@ -149,6 +151,18 @@ def test_more_pairs_inside_the_angular_cutoff_than_slots(oracle, np_dtype):
     assert ref[2].min() > 32 and ref[2].max() <= 136
     _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np_dtype), np_dtype)
     assert np.abs(out[1].astype(np.float64).sum(0)).max() < (1e-9 if np_dtype == np.float64 else 1e-2)
+    for _ in range(2):
+        again = _step(calc, pos, np_dtype)
+        for x, y in zip(out, again):
+            assert np.array_equal(np.ascontiguousarray(x).view(np.uint8), np.ascontiguousarray(y).view(np.uint8))
+    # a smaller structure next, on the same workspace: the counters and spare rows it finds must be clean
+    n2 = 120
+    lat2, pos2 = synth.random_packed(n2, [14.5, 14.0, 15.0], 2.0, 353)
+    ty2 = synth.rng_randint(354, n2, 3)
+    calc2 = _calc(m, lat2, ty2, n2, np_dtype, umax=136, path="gather")
+    out2 = _step(calc2, pos2, np_dtype)
+    ref2 = oracle.nblist(lat2, ty2, pos2, 7.0, 136)
+    _check(out2, oracle.nep_efv(m, synth.pack_batch([ref2]), np_dtype), np_dtype)
 
 
 def test_atoms_processed_in_the_callers_order(oracle):
@@ -336,6 +350,35 @@ def test_gather_errors(oracle):
     ok.step(torch.from_numpy(pos.astype(np.float32)).to("cuda:0"))
     with pytest.raises(_lib.A2PError):
         ok.check()
+
+
+def test_order_written_by_the_caller_is_checked(oracle):
+    """The processing order at the head of the compact buffer may be written by the caller.  An index outside the
+    structure, or an atom named twice, is reported by the status check (the index is clamped where it is used,
+    so no kernel touches memory outside the buffers); a valid order written afterwards works again."""
+    import torch
+    from ai2pot_amd import _lib
+    n = 200
+    lat, pos = synth.random_packed(n, [17.0, 16.0, 18.0], 2.2, 381)
+    ty = synth.rng_randint(382, n, 3)
+    m = synth.nep_model(seed=3308)
+    x = torch.from_numpy(pos.astype(np.float32)).to("cuda:0")
+    ref = oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 7.0, 96)
+    want = oracle.nep_efv(m, synth.pack_batch([ref]), np.float32)
+    for bad in ([n + 5, 3], [-7, 3], [1 << 30, 3], [11, 11], None):
+        calc = _calc(m, lat, ty, n, np.float32, umax=96, path="gather", reorder_every=0)
+        order = calc.compact[:4 * n].view(torch.int32)
+        if bad is not None:
+            order[7] = bad[0]
+            order[9] = bad[1]
+        e, f, v = calc.step(x)
+        torch.cuda.synchronize()
+        if bad is None:
+            calc.check()
+            _check((e.cpu().numpy(), f.cpu().numpy(), v.cpu().numpy()), want, np.float32)
+        else:
+            with pytest.raises(_lib.A2PError):
+                calc.check()
 
 
 @pytest.mark.parametrize("np_dtype", [np.float32, np.float64])
