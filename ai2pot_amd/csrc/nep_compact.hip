@@ -29,6 +29,8 @@
 #include "compact_list.h"
 #include "nep_device.h"
 
+#include <cstdlib>
+#include <string>
 #include <type_traits>
 
 namespace a2p {
@@ -291,19 +293,25 @@ struct OverflowRow<double> {
 
 template <typename T>
 struct AdjointLds {
-    T *coef, *w0, *b0, *w1, *qs, *acc, *stage;
+    T *coef, *w0, *w0t, *b0, *w1, *qs, *acc, *stage;
     double* red;
 };
+constexpr int HM_HP = 64;               // neurons of the zero-padded tables of the matrix-core hidden layer
+constexpr int HM_HPT = 68;              // row length of the transposed table: 16 lanes reading 16 rows hit 16 bank groups
 // The network tables (w0, b0, w1, qs) are dead once the hidden layer is done; the threads' contracted
 // radial coefficients (acc, [NTC * KC][CB]) are laid over them for the second walk.
+// hm: tables of the matrix-core hidden layer: H padded to HM_HP neurons with zeros, and a transposed copy of w0
 template <typename T>
-__host__ __device__ __forceinline__ size_t adjoint_lds(int nt, int ntc, int H, int nb, unsigned char* base, AdjointLds<T>& L)
+__host__ __device__ __forceinline__ size_t adjoint_lds(int nt, int ntc, int H, int nb, unsigned char* base, AdjointLds<T>& L,
+                                                       bool hm = false)
 {
     size_t off = 0;
     L.coef = (T*)(base + off);  off += lds16((size_t)nt * nt * nb * KC * sizeof(T));
     const size_t tables = off;
+    if (hm) H = HM_HP;
     L.acc = (T*)(base + off);
     L.w0 = (T*)(base + off);    off += lds16((size_t)nt * H * FDP * sizeof(T));
+    L.w0t = (T*)(base + off);   if (hm) off += lds16((size_t)nt * HM_HPT * FDP * sizeof(T));
     L.b0 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
     L.w1 = (T*)(base + off);    off += lds16((size_t)nt * H * sizeof(T));
     L.qs = (T*)(base + off);    off += lds16((size_t)FDP * sizeof(T));
@@ -328,8 +336,150 @@ __host__ __device__ __forceinline__ size_t gather_lds(unsigned char* base, Gathe
     return off;
 }
 
+// ---- the hidden layer of a wavefront's 64 atoms on the matrix cores (fp32) ----------------------------
+// The weights depend on the atom's species, so the wavefront first groups its atoms by species: every lane gets a
+// row in a table of scaled descriptors in LDS (the wavefront's own staging buffer, idle between the walks; no
+// workgroup barrier is involved), each species' rows padded to a multiple of 16: at most 96 rows for up to three
+// species.  Then, tile by tile (16 rows of one species), with v_mfma_f32_16x16x4f32 (D[i][j] += sum_k A[i][k] B[k][j];
+// lane l holds A[l%16][l/16], B[l/16][l%16] and D[4 (l/16) + v][l%16] in register v):
+//   layer 1, transposed:  H^T[n][r] = sum_k W0[n][k] Q[r][k]   (A = weights, B = descriptors), four tiles of 16
+//            neurons; on the accumulators: + b0, tanh, the energy terms w1 tanh, and G = w1 (1 - tanh^2);
+//   layer 2:              dE/dq[r][j] = sum_n G[r][n] W0[n][j]: the accumulators of layer 1 are already laid out
+//            as the A operand of this product (lane l holds row r = l%16 and, in register v of neuron tile n0,
+//            neuron n0 + 4 (l/16) + v), so the sum over the neurons simply runs in that order and G never leaves
+//            the registers; B = W0[n0 + 4 (l/16) + v][j0 + l%16].
+// dE/dq and the energy go back into the table row, and every lane reads its row.  Neurons beyond H and
+// descriptors beyond DC are zero weights.  Reference arithmetic: nep.h:415-447.
+constexpr int kHiddenDefault = 0;                 // vector ALUs unless measured otherwise
+constexpr int HM_TILE = 16, HM_NT = 4;            // rows per tile; neuron tiles (H <= 64)
+constexpr int HM_STRIDE = FDP;                    // floats per table row: DC descriptors, [FDP-1] the energy
+constexpr int HM_ROWS = 64 * STP * 4 / HM_STRIDE; // rows the staging buffer of a wavefront holds (96)
+constexpr int HM_NTC_MAX = 3;                     // 64 atoms of up to three species fit: 64 + 3 * 15 -> 96 rows
+static_assert(HM_ROWS >= ((64 + HM_NTC_MAX * (HM_TILE - 1)) / HM_TILE) * HM_TILE, "staging buffer too small");
+
+typedef float hm_f4 __attribute__((ext_vector_type(4)));
+
+template <int NTC, int DC>
+__device__ __forceinline__ void hidden_layer_mfma(const AdjointLds<float>& L, float* Q, int H, int ti, int lane,
+                                                  float (&qn)[FDP], float& e_net)
+{
+    static_assert(DC < FDP, "the last column of a row carries the energy");
+    static_assert(NTC <= HM_NTC_MAX, "too many species for the wavefront's table");
+    // -- rows: species by species, inside a species by lane; ends[t] = end of species t's (padded) rows
+    int row = 0, nrows = 0;
+    int ends[NTC];
+#pragma unroll
+    for (int t = 0; t < NTC; t++) {
+        const unsigned long long m = __ballot(ti == t);
+        if (ti == t) row = nrows + __popcll(m & ((1ull << lane) - 1ull));
+        nrows += (__popcll(m) + HM_TILE - 1) & ~(HM_TILE - 1);
+        ends[t] = nrows;
+    }
+    __builtin_amdgcn_wave_barrier();
+    {
+        // rows that pad a species to a multiple of 16 are never read back; their contents only need to exist
+        float* qr = Q + (size_t)row * HM_STRIDE;
+#pragma unroll
+        for (int j = 0; j < FDP; j += 4) *reinterpret_cast<float4*>(qr + j) = make_float4(qn[j], qn[j + 1], qn[j + 2], qn[j + 3]);
+    }
+    __builtin_amdgcn_wave_barrier();
+    const int c = lane & 15, g = lane >> 4;
+    for (int row0 = 0; row0 < nrows; row0 += HM_TILE) {
+        int t = 0;                                 // species of the tile
+#pragma unroll
+        for (int s2 = 0; s2 + 1 < NTC; s2++) t += row0 >= ends[s2] ? 1 : 0;
+        // layer 1; the sum over the descriptors runs in the order k = 6 g + kk, so that a lane's six values are
+        // neighbours in memory: B = Q[row0 + c][6 g + kk], A = W0[n][6 g + kk]
+        float qb[FDP / 4];
+        {
+            const float* qr = Q + (size_t)(row0 + c) * HM_STRIDE + 6 * g;
+#pragma unroll
+            for (int kk = 0; kk < FDP / 4; kk += 2) {
+                const float2 v = *reinterpret_cast<const float2*>(qr + kk);
+                qb[kk] = v.x; qb[kk + 1] = v.y;
+            }
+        }
+        hm_f4 acc[HM_NT];
+#pragma unroll
+        for (int nt_ = 0; nt_ < HM_NT; nt_++) {
+            acc[nt_] = hm_f4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (nt_ * HM_TILE < H) {                       // wave-uniform
+                const float* wr = L.w0 + ((size_t)t * HM_HP + nt_ * HM_TILE + c) * FDP + 6 * g;
+#pragma unroll
+                for (int kk = 0; kk < FDP / 4; kk += 2) {
+                    const float2 wa = *reinterpret_cast<const float2*>(wr + kk);
+                    acc[nt_] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa.x, qb[kk], acc[nt_], 0, 0, 0);
+                    acc[nt_] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa.y, qb[kk + 1], acc[nt_], 0, 0, 0);
+                }
+            }
+        }
+        // on the accumulators: lane (c, g), register v of tile nt_ = neuron nt_ * 16 + 4 g + v of row row0 + c
+        float e = 0.0f;
+#pragma unroll
+        for (int nt_ = 0; nt_ < HM_NT; nt_++) {
+            const float4 b0v = *reinterpret_cast<const float4*>(L.b0 + t * HM_HP + nt_ * HM_TILE + 4 * g);
+            const float4 w1v = *reinterpret_cast<const float4*>(L.w1 + t * HM_HP + nt_ * HM_TILE + 4 * g);
+            const float b0a[4] = {b0v.x, b0v.y, b0v.z, b0v.w}, w1a[4] = {w1v.x, w1v.y, w1v.z, w1v.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                if (nt_ * HM_TILE + v < H) {               // wave-uniform: some lane has a neuron here
+                    const float th = tanh_t(acc[nt_][v] + b0a[v]);
+                    e += w1a[v] * th;
+                    acc[nt_][v] = w1a[v] * (1.0f - th * th);
+                } else {
+                    acc[nt_][v] = 0.0f;
+                }
+            }
+        }
+        e += __shfl_xor(e, 16, 64);
+        e += __shfl_xor(e, 32, 64);
+        // layer 2: two tiles of 16 descriptors (j0 = 0, 16); B = W0^T[j0 + c][nt_ * 16 + 4 g + v], four neighbours
+        // in the transposed table (columns beyond the table read its last, all-zero row)
+        hm_f4 out[2] = {hm_f4{0.0f, 0.0f, 0.0f, 0.0f}, hm_f4{0.0f, 0.0f, 0.0f, 0.0f}};
+        const float* wt0 = L.w0t + ((size_t)t * FDP + c) * HM_HPT + 4 * g;
+        const float* wt1 = L.w0t + ((size_t)t * FDP + min(16 + c, FDP - 1)) * HM_HPT + 4 * g;
+#pragma unroll
+        for (int nt_ = 0; nt_ < HM_NT; nt_++) {
+            if (nt_ * HM_TILE < H) {                       // wave-uniform
+                const float4 u0 = *reinterpret_cast<const float4*>(wt0 + nt_ * HM_TILE);
+                const float4 u1 = *reinterpret_cast<const float4*>(wt1 + nt_ * HM_TILE);
+                const float b0a[4] = {u0.x, u0.y, u0.z, u0.w}, b1a[4] = {u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    if (nt_ * HM_TILE + v < H) {           // wave-uniform
+                        out[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[nt_][v], b0a[v], out[0], 0, 0, 0);
+                        out[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[nt_][v], b1a[v], out[1], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // back into the rows (the tile's descriptors have been read): register v = row row0 + 4 g + v, column j0 + c
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            float* qr = Q + (size_t)(row0 + 4 * g + v) * HM_STRIDE;
+            qr[c] = out[0][v];
+            if (16 + c < FDP - 1) qr[16 + c] = out[1][v];
+        }
+        if (g == 0) Q[(size_t)(row0 + c) * HM_STRIDE + FDP - 1] = e;
+    }
+    __builtin_amdgcn_wave_barrier();
+    {
+        const float* qr = Q + (size_t)row * HM_STRIDE;
+#pragma unroll
+        for (int j = 0; j < FDP; j += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(qr + j);
+            qn[j] = v.x; qn[j + 1] = v.y; qn[j + 2] = v.z; qn[j + 3] = v.w;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();               // the staging buffer goes back to the walks
+    e_net = qn[FDP - 1];
+}
+
 // ---- kernel 1: descriptors, hidden layer, adjoints -------------------------------------------------
-template <typename T, int NTC, int NR>
+// HM: the hidden layer of each wavefront's 64 atoms runs on the matrix cores (fp32, at most 64 neurons and three
+// species): see hidden_layer_mfma
+template <typename T, int NTC, int NR, bool HM = false>
 __global__ void __launch_bounds__(CB, (sizeof(T) == 4 ? 2 : 1))
 nep_adjoint_kernel(const GatherArgs<T> a)
 {
@@ -342,15 +492,30 @@ nep_adjoint_kernel(const GatherArgs<T> a)
     const int tile = p >> 6;
     const int nt = a.ntypes, H = a.H;
     AdjointLds<T> L;
-    adjoint_lds<T>(nt, NTC, H, NB, smem_raw, L);
+    adjoint_lds<T>(nt, NTC, H, NB, smem_raw, L, HM);
     T* const st = L.stage + (size_t)wv * 64 * STP * 4;
 
     for (int i = tid; i < nt * nt * NB * KC; i += CB) L.coef[i] = a.coeffs[i];
-    for (int i = tid; i < nt * H * FDP; i += CB) {
-        const int r = i / FDP, j = i - r * FDP;
-        L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
+    if constexpr (HM) {
+        // [species][HM_HP neurons][FDP] and its transpose [species][FDP][HM_HPT], zeros beyond H and DC
+        for (int i = tid; i < nt * HM_HP * FDP; i += CB) {
+            const int r = i / FDP, j = i - r * FDP, t = r / HM_HP, n = r - t * HM_HP;
+            const T v = (n < H && j < DC) ? a.w0[((size_t)t * H + n) * DC + j] : (T)0;
+            L.w0[i] = v;
+            L.w0t[((size_t)t * FDP + j) * HM_HPT + n] = v;
+        }
+        for (int i = tid; i < nt * HM_HP; i += CB) {
+            const int t = i / HM_HP, n = i - t * HM_HP;
+            L.b0[i] = n < H ? a.b0[t * H + n] : (T)0;
+            L.w1[i] = n < H ? a.w1[t * H + n] : (T)0;
+        }
+    } else {
+        for (int i = tid; i < nt * H * FDP; i += CB) {
+            const int r = i / FDP, j = i - r * FDP;
+            L.w0[i] = j < DC ? a.w0[(size_t)r * DC + j] : (T)0;
+        }
+        for (int i = tid; i < nt * H; i += CB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
     }
-    for (int i = tid; i < nt * H; i += CB) { L.b0[i] = a.b0[i]; L.w1[i] = a.w1[i]; }
     if (tid < FDP) L.qs[tid] = tid < DC ? (T)1 / a.q_scaler[tid] : (T)0;
 
     int atom, ti, n_outer, n_inner;
@@ -451,7 +616,17 @@ nep_adjoint_kernel(const GatherArgs<T> a)
     // ---- hidden layer (nep.h:415-447) --------------------------------------------------------------
     T dEdq[DC];
     T e_site = active ? a.bias[ti] : (T)0;
-    {
+    if constexpr (HM) {
+        static_assert(std::is_same<T, float>::value, "the matrix-core hidden layer is fp32");
+        float qn[FDP];
+#pragma unroll
+        for (int j = 0; j < FDP; j++) qn[j] = j < DC ? q[j] * L.qs[j] : 0.0f;
+        float e_net = 0.0f;
+        hidden_layer_mfma<NTC, DC>(L, st, H, ti, lane, qn, e_net);
+        e_site += active ? e_net : 0.0f;
+#pragma unroll
+        for (int j = 0; j < DC; j++) dEdq[j] = qn[j] * L.qs[j];
+    } else {
         T qn[DC];
 #pragma unroll
         for (int j = 0; j < DC; j++) { qn[j] = q[j] * L.qs[j]; dEdq[j] = (T)0; }
@@ -731,14 +906,36 @@ nep_gather_kernel(const GatherArgs<T> a)
     }
 }
 
+// Which unit runs the hidden layer: 0 vector ALUs (one thread per atom), 1 matrix cores (fp32, at most 64
+// neurons).  AI2POT_NEP_HIDDEN=valu|mfma overrides the default; a2p_nep_hidden_layer_unit sets it at run time.
+int g_hidden_unit = -1;
+int hidden_unit()
+{
+    if (g_hidden_unit < 0) {
+        const char* e = getenv("AI2POT_NEP_HIDDEN");
+        g_hidden_unit = (e && std::string(e) == "mfma") ? 1 : (e && std::string(e) == "valu") ? 0 : kHiddenDefault;
+    }
+    return g_hidden_unit;
+}
+
+template <typename T, int NTC, int NR>
+auto adjoint_kernel_for(bool mfma)
+{
+    if constexpr (std::is_same<T, float>::value && NTC <= HM_NTC_MAX) {
+        if (mfma) return nep_adjoint_kernel<T, NTC, NR, true>;
+    }
+    return nep_adjoint_kernel<T, NTC, NR, false>;
+}
+
 template <typename T, int NTC, int NR>
 int launch_gather(const GatherArgs<T>& a, int nblocks, bool pairs, hipStream_t stream)
 {
     AdjointLds<T> la;
     GatherLds<T> lg;
-    const size_t lds_a = adjoint_lds<T>(a.ntypes, NTC, a.H, NR + NAC, nullptr, la);
+    const bool mfma = std::is_same<T, float>::value && NTC <= HM_NTC_MAX && hidden_unit() == 1 && a.H <= HM_NT * HM_TILE;
+    const size_t lds_a = adjoint_lds<T>(a.ntypes, NTC, a.H, NR + NAC, nullptr, la, mfma);
     const size_t lds_g = gather_lds<T>(nullptr, lg);
-    auto ka = nep_adjoint_kernel<T, NTC, NR>;
+    auto ka = adjoint_kernel_for<T, NTC, NR>(mfma);
     auto kg = nep_gather_kernel<T, NTC>;
     if (lds_a > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a));
@@ -841,6 +1038,13 @@ int nep_efv_compact(int K, int n_r, int n_a, int l_max, int H, int ntypes, const
 }  // namespace a2p
 
 extern "C" {
+
+int a2p_nep_hidden_layer_unit(int unit)
+{
+    const int before = a2p::hidden_unit();
+    if (unit == 0 || unit == 1) a2p::g_hidden_unit = unit;
+    return before;
+}
 
 int a2p_nep_efv_compact_supported(int K, int n_r, int n_a, int l_max, int H, int ntypes, int elem_size)
 {

@@ -266,6 +266,14 @@ size_t a2p_nblist_compact_bytes(int natoms, int umax, int elem_size);   /* 0: no
  * that consume the list. */
 int a2p_nblist_sync_free(int on);
 
+/* Which unit evaluates the per-species network (nep.h:415-447) inside a2p_nep_efv_compact_f32: 0 = the vector
+ * ALUs, one thread per atom; 1 = the matrix cores (v_mfma_f32_16x16x4f32): the 64 atoms of a wavefront are grouped
+ * by species in LDS and both layers run as [16 x 24] x [24 x 64] and [16 x 64] x [64 x 24] products per tile of 16
+ * atoms, fp32 in and out (num_neurons <= 64, at most three species; larger models and fp64 stay on the vector
+ * ALUs).  Returns the previous setting; any other argument only queries.  The environment variable
+ * AI2POT_NEP_HIDDEN=valu|mfma sets the initial value.  Process-wide. */
+int a2p_nep_hidden_layer_unit(int unit);
+
 /* 1 when a2p_nep_efv_compact_* covers the model (shape as above, tables fit in LDS), else 0 */
 int a2p_nep_efv_compact_supported(int chebyshev_size, int n_radial, int n_angular, int l_max, int num_neurons,
                                   int ntypes, int elem_size);

@@ -134,6 +134,41 @@ def test_model_shapes(oracle, cfg):
     _check(out, oracle.nep_efv(m, synth.pack_batch([ref]), np.float64), np.float64)
 
 
+@pytest.mark.parametrize("cfg", [dict(ntypes=3, n_r=6, H=50, n=700), dict(ntypes=1, n_r=4, H=30, n=300),
+                                 dict(ntypes=4, n_r=6, H=64, n=521), dict(ntypes=2, n_r=4, H=7, n=130),
+                                 dict(ntypes=3, n_r=6, H=100, n=200)])
+def test_hidden_layer_on_the_matrix_cores(oracle, cfg):
+    """a2p_nep_hidden_layer_unit(1): the per-species network of the workgroup's atoms as matrix products (fp32,
+    species grouped in LDS, neuron counts that fill the 16-wide tiles unevenly, wavefronts with fewer than 64
+    atoms, a scaled q_scaler; 100 neurons and four species stay on the vector ALUs).  Bars as for every fp32 result; the two units
+    agree far inside them."""
+    from ai2pot_amd import _lib
+    n = cfg["n"]
+    side = (n / 0.035) ** (1.0 / 3.0)
+    lat, pos = synth.random_packed(n, [side, side * 1.05, side * 0.95], 2.2, 341)
+    ty = synth.rng_randint(342, n, cfg["ntypes"])
+    m = synth.nep_model(ntypes=cfg["ntypes"], n_radial_basis=cfg["n_r"], num_neurons=cfg["H"], seed=3304,
+                        type_map=tuple(range(30, 30 + cfg["ntypes"])))
+    D = cfg["n_r"] + 16
+    m["q_scaler"] = 0.6 + 0.07 * np.arange(D)
+    ref = oracle.nblist(lat.astype(np.float32), ty, pos.astype(np.float32), 7.0, 96)
+    want = oracle.nep_efv(m, synth.pack_batch([ref]), np.float32)
+    L = _lib.lib()
+    before = L.a2p_nep_hidden_layer_unit(c.c_int(-1))
+    outs = {}
+    try:
+        for unit in (1, 0):
+            L.a2p_nep_hidden_layer_unit(c.c_int(unit))
+            assert L.a2p_nep_hidden_layer_unit(c.c_int(-1)) == unit
+            calc = _calc(m, lat, ty, n, np.float32, umax=96, path="gather")
+            outs[unit] = _step(calc, pos, np.float32)
+            _check(outs[unit], want, np.float32)
+    finally:
+        L.a2p_nep_hidden_layer_unit(c.c_int(before))
+    assert np.abs(outs[0][1] - outs[1][1]).max() <= 2e-5 * max(1.0, np.abs(outs[0][1]).max())
+    assert abs(outs[0][0][0] - outs[1][0][0]) <= 2e-6 * abs(outs[0][0][0])
+
+
 @pytest.mark.parametrize("np_dtype", [np.float64, np.float32])
 def test_more_pairs_inside_the_angular_cutoff_than_slots(oracle, np_dtype):
     """Equal cutoffs of 7 A at 0.04 atoms / A^3: every atom is named by about 57 pairs inside the angular cutoff,
