@@ -131,12 +131,6 @@ inline void run_checked(const at::Tensor& brcs, const at::Tensor& binum, const a
     check_rc(rc);
 }
 
-inline void require_no_zbl(double zbl_rmax)
-{
-    TORCH_CHECK(zbl_rmax == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
-                                 "and the loss operators only; this operator needs zbl_rmax == 0");
-}
-
 // Adds the ZBL pair repulsion onto a model's E/F/V when zbl_rmax > 0, as the reference's operators
 // do on the device (correction/gpu/include/zbl.cuh:422-620); v may be undefined.
 inline void apply_zbl(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, const at::Tensor& dks,
@@ -168,6 +162,42 @@ inline void apply_zbl(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, c
     }
     check_rc(rc);
     check_device_status(brcs);
+}
+
+// Per-row ZBL energies [B, P] of the site-energy operators (GroupZBL::correct_e_sites, zbl.h:625-685): half of
+// every pair energy of the row's centre atom; undefined when zbl_rmax == 0.  The reference's CPU operators add the
+// term and then assign the rows (linearMtp.h:598), which loses it; here the rows keep it.
+inline at::Tensor zbl_esites(double zbl_rmax, double zbl_rmin, const at::Tensor& cks, const at::Tensor& dks,
+                             const at::Tensor& type_map, const at::Tensor& binum, const at::Tensor& bilist,
+                             const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
+                             const at::Tensor& btypes, int64_t nghost)
+{
+    if (zbl_rmax == 0.0) return at::Tensor();
+    const int ntypes = (int)type_map.numel();
+    check_device_float(brcs, cks, "zbl_cks");
+    check_device_float(brcs, dks, "zbl_dks");
+    TORCH_CHECK(cks.numel() == (int64_t)ntypes * ntypes * 4 && dks.numel() == (int64_t)ntypes * ntypes * 4,
+                "zbl_cks and zbl_dks must have ntypes * ntypes * 4 elements");
+    TORCH_CHECK(brcs.dim() == 4, "brcs must have shape [B, P, U, 3]");
+    at::Tensor tm = type_map.to(brcs.device(), at::kInt).contiguous();
+    DeviceGuard guard(brcs);
+    const int B = (int)brcs.size(0), P = (int)brcs.size(1), U = (int)brcs.size(2);
+    at::Tensor out = at::zeros({B, P}, brcs.options());
+    void* st = current_stream(brcs);
+    int rc;
+    if (brcs.scalar_type() == at::kDouble)
+        rc = a2p_zbl_esites_f64(zbl_rmax, zbl_rmin, cks.data_ptr<double>(), dks.data_ptr<double>(), ntypes,
+                                tm.data_ptr<int>(), B, P, U, (int)nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(),
+                                btypes.data_ptr<int>(), out.data_ptr<double>(), st);
+    else
+        rc = a2p_zbl_esites_f32(zbl_rmax, zbl_rmin, cks.data_ptr<float>(), dks.data_ptr<float>(), ntypes,
+                                tm.data_ptr<int>(), B, P, U, (int)nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(), brcs.data_ptr<float>(),
+                                btypes.data_ptr<int>(), out.data_ptr<float>(), st);
+    check_rc(rc);
+    check_device_status(brcs);
+    return out;
 }
 
 // Labels of a loss operator with the ZBL pair repulsion taken out.  The correction does not depend

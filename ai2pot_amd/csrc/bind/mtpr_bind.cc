@@ -456,8 +456,9 @@ TORCH_LIBRARY(mtpr, m)
     m.def("LinMatrixLinVectorOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,
              const at::Tensor& v_dft, MTP_EFV_ARGS) -> variable_list {
-              require_no_zbl(zbl_rmax);
-              return lin_matrix_lin_vector(e_w, f_w, v_w, e_dft, f_dft, v_dft, K, scaling, coeffs, n_moms, basic, times,
+              // labels minus the ZBL energy, forces and virial (src/linear_mtp_gram_and_cross_op.cc:309-338)
+              auto lab = zbl_shift_labels(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost, e_dft, f_dft, v_dft);
+              return lin_matrix_lin_vector(e_w, f_w, v_w, lab.e, lab.f, lab.v, K, scaling, coeffs, n_moms, basic, times,
                                            mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
                                            nghost, rmax, rmin, q_scaler);
           });
@@ -465,8 +466,10 @@ TORCH_LIBRARY(mtpr, m)
         return schmidt_orth(ntypes, nmus, K, coeffs);
     });
     m.def("linearMtpToEsitesOp", [](MTP_EFV_ARGS) -> variable_list {
-        require_no_zbl(zbl_rmax);
-        return EsitesFunction::apply(MTP_EFV_PASS);
+        variable_list out = EsitesFunction::apply(MTP_EFV_PASS);
+        at::Tensor zb = zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+        if (zb.defined()) out[0] = out[0] + zb;
+        return out;
     });
     // mtpr_bind.cc:140-187: num_mus4moms / mus4moms (the radial functions behind each moment, which the reference's
     // coefficient derivative walks) are not needed here; the first dimension of mus4moms is the number of moments

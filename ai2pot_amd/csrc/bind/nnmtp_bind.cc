@@ -312,8 +312,10 @@ TORCH_LIBRARY(nnmtp, m)
         return out;
     });
     m.def("nnMtpToEsitesOp", [](NNMTP_ARGS) -> variable_list {
-        require_no_zbl(zbl_rmax);
-        return NNEsitesFunction::apply(NNMTP_PASS);
+        variable_list out = NNEsitesFunction::apply(NNMTP_PASS);
+        at::Tensor zb = zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
+        if (zb.defined()) out[0] = out[0] + zb;
+        return out;
     });
     m.def("nnMtpToDescriptorsOp",
           [](int64_t K, const at::Tensor& coeffs, int64_t n_moms, const at::Tensor& basic, const at::Tensor& times,

@@ -5,6 +5,8 @@
 //   every ordered pair (i, j) of the list with r <= rmax gives  0.5 E_pair  to the energy,
 //   dE_pair/dr * r_vec / r  to the force of the CENTRE atom i only (the pair (j, i) of a full list
 //   supplies the other half; ghosts receive nothing), and  -0.5 r_a dE_pair/dr r_b / r  to the virial.
+// The site-energy operators take the per-row sums of the 0.5 E_pair terms instead (GroupZBL::correct_e_sites,
+// zbl.h:625-685).
 // One thread per row; the force is written by its row's thread alone, energy and virial leave
 // each workgroup as fp64 partial sums that a second kernel adds onto the outputs in block order.
 #include "a2p_common.h"
@@ -30,7 +32,7 @@ zbl_kernel(int B, int P, int U, int nghost, const int* __restrict__ binum, const
            const int* __restrict__ bnumneigh, const int* __restrict__ bfirstneigh, const T* __restrict__ brcs,
            const int* __restrict__ btypes, int ntypes, const int* __restrict__ type_map, T rmax, T rmin,
            const T* __restrict__ cks, const T* __restrict__ dks, T* __restrict__ force,
-           double* __restrict__ partial, int nblocks, int* __restrict__ status)
+           double* __restrict__ partial, int nblocks, int* __restrict__ status, T* __restrict__ e_sites)
 {
     __shared__ double red[ZB / 64][10];
     const int b = blockIdx.y, ii = blockIdx.x * ZB + threadIdx.x;
@@ -93,6 +95,7 @@ zbl_kernel(int B, int P, int U, int nghost, const int* __restrict__ binum, const
             T* fo = force + ((size_t)b * NF + center) * 3;
             fo[0] += f[0]; fo[1] += f[1]; fo[2] += f[2];
         }
+        if (e_sites) e_sites[row] += e;                     // GroupZBL::correct_e_sites, zbl.h:625-685
         acc[0] = (double)e;
 #pragma unroll
         for (int q = 0; q < 9; q++) acc[1 + q] = (double)v[q];
@@ -126,13 +129,14 @@ __global__ void zbl_add_kernel(const double* __restrict__ partial, int nblocks, 
 template <typename T>
 int zbl_correct(double rmax, double rmin, const T* cks, const T* dks, int ntypes, const int* type_map, int B, int P,
                 int U, int nghost, const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
-                const T* brcs, const int* btypes, T* etot, T* force, T* virial, hipStream_t stream)
+                const T* brcs, const int* btypes, T* etot, T* force, T* virial, hipStream_t stream,
+                T* e_sites = nullptr)
 {
     A2P_REQUIRE(rmax > rmin && rmin >= 0, A2P_ERR_INVALID, "zbl: need 0 <= zbl_rmin < zbl_rmax");
     A2P_REQUIRE(cks && dks && type_map && binum && bilist && bnumneigh && bfirstneigh && brcs && btypes,
                 A2P_ERR_INVALID, "zbl: null input pointer");
     A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0 && U >= 1 && nghost >= 0, A2P_ERR_INVALID, "zbl: bad shape");
-    if (B == 0 || P == 0 || (!etot && !force && !virial)) return A2P_OK;
+    if (B == 0 || P == 0 || (!etot && !force && !virial && !e_sites)) return A2P_OK;
     const int nblocks = ceil_div(P, ZB);
     void* ws = nullptr;
     int rc = ws_get(WS_FLAGS, 64, &ws);
@@ -144,8 +148,9 @@ int zbl_correct(double rmax, double rmin, const T* cks, const T* dks, int ntypes
     prof_begin("zbl_kernel", stream);
     hipLaunchKernelGGL(zbl_kernel<T>, dim3(nblocks, B), dim3(ZB), 0, stream, B, P, U, nghost, binum, bilist,
                        bnumneigh, bfirstneigh, brcs, btypes, ntypes, type_map, (T)rmax, (T)rmin, cks, dks, force,
-                       partial, nblocks, status);
-    hipLaunchKernelGGL(zbl_add_kernel<T>, dim3(B), dim3(64), 0, stream, partial, nblocks, etot, virial);
+                       partial, nblocks, status, e_sites);
+    if (etot || virial)
+        hipLaunchKernelGGL(zbl_add_kernel<T>, dim3(B), dim3(64), 0, stream, partial, nblocks, etot, virial);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     return A2P_OK;
@@ -172,5 +177,25 @@ int a2p_zbl_correct_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, 
     return a2p::zbl_correct<float>(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, ntypes, type_map, B, P, U, nghost, binum,
                                    bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial,
                                    (hipStream_t)stream);
+}
+int a2p_zbl_esites_f64(double zbl_rmax, double zbl_rmin, const double* zbl_cks, const double* zbl_dks, int ntypes,
+                       const int* type_map, int B, int P, int U, int nghost, const int* binum, const int* bilist,
+                       const int* bnumneigh, const int* bfirstneigh, const double* brcs, const int* btypes,
+                       double* be_sites, void* stream)
+{
+    A2P_REQUIRE(be_sites, A2P_ERR_INVALID, "zbl: null be_sites");
+    return a2p::zbl_correct<double>(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, ntypes, type_map, B, P, U, nghost, binum,
+                                    bilist, bnumneigh, bfirstneigh, brcs, btypes, nullptr, nullptr, nullptr,
+                                    (hipStream_t)stream, be_sites);
+}
+int a2p_zbl_esites_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, const float* zbl_dks, int ntypes,
+                       const int* type_map, int B, int P, int U, int nghost, const int* binum, const int* bilist,
+                       const int* bnumneigh, const int* bfirstneigh, const float* brcs, const int* btypes,
+                       float* be_sites, void* stream)
+{
+    A2P_REQUIRE(be_sites, A2P_ERR_INVALID, "zbl: null be_sites");
+    return a2p::zbl_correct<float>(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, ntypes, type_map, B, P, U, nghost, binum,
+                                   bilist, bnumneigh, bfirstneigh, brcs, btypes, nullptr, nullptr, nullptr,
+                                   (hipStream_t)stream, be_sites);
 }
 }

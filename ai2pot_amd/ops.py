@@ -147,9 +147,33 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
     return etot, force, virial, desc
 
 
-def _no_zbl(zbl_rmax):
-    _req(float(zbl_rmax) == 0.0, "the ZBL correction (zbl_rmax > 0) is implemented for the energy / force / virial "
-                                 "and the loss operators only; this operator needs zbl_rmax == 0")
+def _zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
+                nghost, validate):
+    """Per-row ZBL energies [B, P] (half of every pair energy of the row's centre atom;
+    GroupZBL::correct_e_sites, correction/include/zbl.h:625-685), or None when zbl_rmax == 0.  The site-energy
+    operators add them to the model's rows, so that the rows sum to the energy of the E/F/V operators.  Parity
+    unpinned by a run of the reference's operator: its CPU code adds the term first and then assigns the rows
+    (linearMtp.h:598), which loses it; the term itself is pinned to correct_e_sites through the oracle."""
+    if float(zbl_rmax) == 0.0:
+        return None
+    dtype, device = brcs.dtype, brcs.device
+    ntypes = int(type_map.numel())
+    for name, t in (("zbl_cks", zbl_cks), ("zbl_dks", zbl_dks)):
+        _check_float(name, t, dtype, device)
+        _req(t.numel() == ntypes * ntypes * 4, "%s must have ntypes*ntypes*4 = %d elements" % (name, ntypes * ntypes * 4))
+    tm = type_map.to(device=device, dtype=torch.int32).contiguous()
+    B, P, U = _batch_shapes(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, int(nghost))
+    out = torch.zeros((B, P), dtype=dtype, device=device)
+    L = _lib.lib()
+    fn = L.a2p_zbl_esites_f32 if dtype == torch.float32 else L.a2p_zbl_esites_f64
+    with torch.cuda.device(device):
+        rc = fn(_c.c_double(zbl_rmax), _c.c_double(zbl_rmin), _ptr(zbl_cks), _ptr(zbl_dks), _c.c_int(ntypes), _ptr(tm),
+                _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(int(nghost)), _ptr(binum), _ptr(bilist),
+                _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs), _ptr(btypes), _ptr(out), _stream(device))
+        _lib.check(rc)
+        if validate:
+            _lib.check_status(torch.cuda.current_stream(device).cuda_stream)
+    return out
 
 
 def _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
@@ -695,12 +719,14 @@ def linearMtpToEsitesOp(chebyshev_size, scaling, coeffs, linear_coeffs, type_bia
                         bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_scaler,
                         zbl_rmax=0.0, zbl_rmin=0.0, zbl_cks=None, zbl_dks=None, validate=True):
     """[e_sites[B, P]] in row order (zero beyond binum), differentiable w.r.t. coeffs, linear_coeffs
-    and type_bias; mtpr_bind.cc:458-518."""
-    _no_zbl(zbl_rmax)
+    and type_bias; mtpr_bind.cc:458-518.  zbl_rmax > 0 adds each row's half pair energies (_zbl_esites)."""
     args = (chebyshev_size, scaling, alpha_moments_count, alpha_index_basic, alpha_index_times,
             alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
             rmax, rmin, q_scaler, validate)
-    return [_LinearMtpToEsites.apply(coeffs, linear_coeffs, type_bias, args)]
+    es = _LinearMtpToEsites.apply(coeffs, linear_coeffs, type_bias, args)
+    zb = _zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                     btypes, nghost, validate)
+    return [es if zb is None else es + zb]
 
 
 def linearMtpToDescriptorsOp(chebyshev_size, scaling, coeffs, alpha_moments_count, alpha_index_basic,
@@ -840,10 +866,13 @@ def LinMatrixLinVectorOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bv
     """[lin_matrix[n, n], lin_vector[n]]: the normal equations of the linear parameters
     (linear_coeffs / q_scaler, then type_bias) for fixed radial coefficients; mtpr_bind.cc:57-131,
     linear_mtp_gram_and_cross.h:446-575.  linear_coeffs and type_bias do not enter, as in the
-    reference; no gradient."""
-    _no_zbl(zbl_rmax)
+    reference; no gradient.  zbl_rmax > 0: the labels enter with the ZBL energy, forces and virial taken out
+    (src/linear_mtp_gram_and_cross_op.cc:309-338)."""
     _req(int(nghost) == 0, "LinMatrixLinVectorOp requires nghost == 0: the reference's force components "
                            "have natoms_pad rows")
+    betot_dft, bforce_dft, bvirial_dft = _zbl_shift_labels(
+        zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost,
+        betot_dft, bforce_dft, bvirial_dft, validate)
     ecomp, fcomp, vcomp = mtp_lin_components(chebyshev_size, scaling, coeffs.detach(), alpha_moments_count,
                                              alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
                                              binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, rmax,
@@ -1024,12 +1053,14 @@ def nnMtpToEsitesOp(chebyshev_size, coeffs, w0, w1, type_bias, alpha_moments_cou
                     btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler, zbl_rmax=0.0, zbl_rmin=0.0,
                     zbl_cks=None, zbl_dks=None, validate=True):
     """[e_sites[B, P]] in row order, differentiable w.r.t. coeffs, w0, w1, type_bias;
-    nnmtp_bind.cc:370-430."""
-    _no_zbl(zbl_rmax)
+    nnmtp_bind.cc:370-430.  zbl_rmax > 0 adds each row's half pair energies (_zbl_esites)."""
     args = (chebyshev_size, alpha_moments_count, alpha_index_basic, alpha_index_times, alpha_moment_mapping, nmus,
             binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax, rmin, q_shifter, q_scaler,
             validate)
-    return [_NNMtpToEsites.apply(coeffs, w0, w1, type_bias, args)]
+    es = _NNMtpToEsites.apply(coeffs, w0, w1, type_bias, args)
+    zb = _zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
+                     btypes, nghost, validate)
+    return [es if zb is None else es + zb]
 
 
 def nnMtpToDescriptorsOp(chebyshev_size, coeffs, alpha_moments_count, alpha_index_basic, alpha_index_times,

@@ -447,6 +447,19 @@ int a2p_zbl_correct_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, 
                         const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
                         const int* bilist, const int* bnumneigh, const int* bfirstneigh, const float* brcs,
                         const int* btypes, float* etot, float* force, float* virial, void* stream);
+/* The same correction for the site-energy operators (GroupZBL::correct_e_sites, zbl.h:625-685, called by
+ * src/linearMtpOp.cc:3662-3683 and the NN-MTP twin): ADDS to be_sites[B, natoms_pad] the row's sum of 0.5 E_pair
+ * over its pairs with r <= zbl_rmax.  The reference's CPU operators call it BEFORE find_e_sites, which then assigns
+ * its rows (linearMtp.h:598), so their output does not contain the term; here it is added to the model's rows, so
+ * that the site energies sum to the energy the E/F/V operators give. */
+int a2p_zbl_esites_f64(double zbl_rmax, double zbl_rmin, const double* zbl_cks, const double* zbl_dks, int ntypes,
+                       const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                       const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                       const int* btypes, double* be_sites, void* stream);
+int a2p_zbl_esites_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, const float* zbl_dks, int ntypes,
+                       const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                       const int* bilist, const int* bnumneigh, const int* bfirstneigh, const float* brcs,
+                       const int* btypes, float* be_sites, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Linear solver support of the linear MTP -- replaces the compute of torch.ops.mtpr.LinMatrixLinVectorOp

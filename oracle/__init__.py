@@ -623,6 +623,28 @@ def zbl_correct(zbl, nb, type_map, efv=None):
     return _zbl(oracle_lib(), "orc_zbl_correct_f64", zbl, nb, type_map, efv)
 
 
+def _zbl_esites(lib, name, zbl, nb, type_map):
+    binum, bilist, bnumneigh, bfirst, brcs, btypes, nghost, B, P, U = _batch(nb, np.float64)
+    type_map = _c(type_map, np.int32)
+    cks, dks = _c(zbl["cks"], np.float64), _c(zbl["dks"], np.float64)
+    nt = type_map.size
+    es = np.zeros((B, P))
+    fn = getattr(lib, name)
+    fn.restype = None
+    fn(_p(es), _D(zbl["rmax"]), _D(zbl["rmin"]), _p(cks), _p(dks), _I(nt), _p(type_map), _I(B), _I(P), _I(U),
+       _I(nghost), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes))
+    return es
+
+
+def ref_zbl_esites(zbl, nb, type_map):
+    """Per-row ZBL energies [B, P] by the reference's GroupZBL::correct_e_sites."""
+    return _zbl_esites(_load("_ref/libref_zbl.so"), "ref_zbl_esites_f64", zbl, nb, type_map)
+
+
+def zbl_esites(zbl, nb, type_map):
+    return _zbl_esites(oracle_lib(), "orc_zbl_esites_f64", zbl, nb, type_map)
+
+
 # ----------------------------------------------------------------------------------------
 # fvt (single structure, fp64)
 # ----------------------------------------------------------------------------------------

@@ -37,3 +37,19 @@ extern "C" void ref_zbl_correct_f64(double* betot, double* bforce, double* bviri
             }
         }
 }
+
+// GroupZBL::correct_e_sites (zbl.h:625-685) itself, structure by structure
+extern "C" void ref_zbl_esites_f64(double* be_sites, double rmax, double rmin, const double* cks, const double* dks,
+                                   int ntypes, const int* type_map, int B, int P, int U, int nghost, const int* binum,
+                                   const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                                   const int* btypes)
+{
+    const int NF = P + nghost;
+    GroupZBL<double> gz(ntypes, const_cast<int*>(type_map), const_cast<int*>(type_map), rmax, rmin,
+                        const_cast<double*>(cks), const_cast<double*>(dks));
+    for (int b = 0; b < B; b++)
+        gz.correct_e_sites(be_sites + (size_t)b * P, binum[b], const_cast<int*>(bilist + (size_t)b * P),
+                           const_cast<int*>(bnumneigh + (size_t)b * P), const_cast<int*>(bfirstneigh + (size_t)b * P * U),
+                           (double (*)[3])const_cast<double*>(brcs + (size_t)b * P * U * 3),
+                           const_cast<int*>(btypes + (size_t)b * NF), ntypes, const_cast<int*>(type_map), U, nghost);
+}

@@ -56,3 +56,39 @@ extern "C" void orc_zbl_correct_f64(double* betot, double* bforce, double* bviri
             }
         }
 }
+
+// Per-row ZBL energies added onto be_sites[B, P]: half of every pair energy of the row's centre atom
+// (GroupZBL::correct_e_sites, zbl.h:625-685).  Pinned by that member function itself, compiled from the
+// reference's header (oracle/_ref/libref_zbl.so), and by the sum rule against orc_zbl_correct_f64's energy.
+extern "C" void orc_zbl_esites_f64(double* be_sites, double rmax, double rmin, const double* cks, const double* dks,
+                                   int ntypes, const int* type_map, int B, int P, int U, int nghost, const int* binum,
+                                   const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                                   const int* btypes)
+{
+    const double kc = 14.399645;                                                // zbl.h:34
+    const int NF = P + nghost;
+    for (int b = 0; b < B; b++)
+        for (int ii = 0; ii < binum[b]; ii++) {
+            const size_t row = (size_t)b * P + ii;
+            const int ci = bilist[row], ti = btypes[(size_t)b * NF + ci];
+            const double Zi = type_map[ti];
+            for (int jj = 0; jj < bnumneigh[row]; jj++) {
+                const double* v = &brcs[(row * U + jj) * 3];
+                const double r = std::sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
+                if (r > rmax) continue;                                         // zbl.h:677-678
+                const int tj = btypes[(size_t)b * NF + bfirstneigh[row * U + jj]];
+                const double Zj = type_map[tj];
+                const double* ck = &cks[(size_t)(ti * ntypes + tj) * 4];
+                const double* dk = &dks[(size_t)(ti * ntypes + tj) * 4];
+                const double a = 0.46848 / (std::pow(Zi, 0.23) + std::pow(Zj, 0.23));
+                double phi = 0;
+                for (int k = 0; k < 4; k++) phi += ck[k] * std::exp(-dk[k] * r / a);
+                double sw = 1;
+                if (r >= rmin) {
+                    const double u = (r - rmin) / (rmax - rmin);
+                    sw = u * u * u * (-6 * u * u + 15 * u - 10) + 1;
+                }
+                be_sites[row] += 0.5 * kc * Zi * Zj / r * phi * sw;             // zbl.h:331-339, 680
+            }
+        }
+}

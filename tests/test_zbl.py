@@ -32,6 +32,21 @@ def test_oracle_against_reference_pair_functions(oracle):
     assert np.abs(a[1]).max() > 1.0                         # the correction is active in this cell
 
 
+def test_oracle_site_energies_against_the_reference(oracle):
+    """Per-row ZBL energies: the restatement against the reference's own GroupZBL::correct_e_sites (zbl.h:625-685,
+    compiled from its header), a padded batch of two structures; and the sum rule against the energy."""
+    lat, pos, ty = close_cell(oracle)
+    lat2, pos2, ty2 = close_cell(oracle, n=41, seed=9)
+    nb = synth.pack_batch([oracle.nblist(lat, ty, pos, 4.0, 200), oracle.nblist(lat2, ty2, pos2, 4.0, 200)])
+    a = oracle.zbl_esites(ZBL, nb, TYPE_MAP)
+    assert a.shape == nb["bilist"].shape and np.all(a[1, 41:] == 0) and a.min() >= 0 and a.max() > 1.0
+    assert np.abs(a.sum(1) - oracle.zbl_correct(ZBL, nb, TYPE_MAP)[0]).max() <= 1e-12 * a.sum(1).max()
+    if not oracle.ref_available("zbl"):
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    b = oracle.ref_zbl_esites(ZBL, nb, TYPE_MAP)
+    assert np.abs(a - b).max() <= 1e-12 * np.abs(b).max()
+
+
 def test_force_and_virial_are_derivatives_of_the_energy(oracle):
     lat, pos, ty = close_cell(oracle)
 
@@ -133,9 +148,13 @@ def test_gpu_kernel_and_operators(oracle, np_dtype):
     got = ops.nnMtpToEFVOp(*nnargs, *zargs)
     want = oracle.zbl_correct(ZBL, nbq, TYPE_MAP, [x.cpu().numpy() for x in base])
     assert all(close(g, w) for g, w in zip(got, want))
-    # operators without an E/F/V output keep refusing the correction
-    with pytest.raises(RuntimeError):
-        ops.linearMtpToEsitesOp(*margs, *zargs)
+    # site energies: the model's rows plus each row's half pair energies; they sum to the corrected energy
+    zs = oracle.zbl_esites(ZBL, nbq, TYPE_MAP)
+    for fn, args, efv in ((ops.linearMtpToEsitesOp, margs, ops.linearMtpToEFVOp), (ops.nnMtpToEsitesOp, nnargs, ops.nnMtpToEFVOp)):
+        plain = fn(*args, 0.0, 0.0, None, None)[0]
+        with_zbl = fn(*args, *zargs)[0]
+        assert close(with_zbl, plain.cpu().numpy() + zs)
+        assert close(with_zbl.sum(1), efv(*args, *zargs)[0].cpu().numpy())
 
 
 @pytest.mark.gpu
@@ -227,9 +246,30 @@ def test_gpu_loss_operators_with_zbl(oracle):
             assert close(a, b)
         plain = fn(*w, *lab, 8, 6, 4, 4, *params, *ntl, *off)
         assert not close(cpu(plain[0]), rb[0])               # the correction changed the loss
-    # operators without an E/F/V output keep refusing the correction
-    with pytest.raises(RuntimeError):
-        ops.linearMtpToEsitesOp(8, 1.0, mmd["coeffs"], mmd["linear_coeffs"], mmd["type_bias"], *tail)
+    # the normal equations of the linear parameters: labels enter with the correction taken out
+    Ar, br = oracle.mtp_lin_system(mm, nb, w, shifted)
+    for fn in (ops.LinMatrixLinVectorOp, torch.ops.mtpr.LinMatrixLinVectorOp):
+        A, bv = fn(*w, *lab, 8, 1.0, mmd["coeffs"], mmd["linear_coeffs"], mmd["type_bias"], *tail)
+        assert close(cpu(A), Ar) and close(cpu(bv), br)
+    A0, b0 = ops.LinMatrixLinVectorOp(*w, *lab, 8, 1.0, mmd["coeffs"], mmd["linear_coeffs"], mmd["type_bias"],
+                                      *tail[:-4], 0.0, 0.0, None, None)
+    assert close(cpu(A0), Ar) and not close(cpu(b0), br)      # the matrix does not see the labels, the vector does
+    # site energies through the bind libraries, and their gradients (the correction has no parameters)
+    zs = oracle.zbl_esites(ZBL, nb, TYPE_MAP)
+    gs = t(synth.rng_normal(35, B * P).reshape(B, P))
+    for fn, params, args in ((torch.ops.mtpr.linearMtpToEsitesOp, (mmd["coeffs"], mmd["linear_coeffs"], mmd["type_bias"]),
+                              lambda ps, z: (8, 1.0, *ps, *tail[:-4], *z)),
+                             (torch.ops.nnmtp.nnMtpToEsitesOp, (mnd["coeffs"], mnd["w0"], mnd["w1"], mnd["type_bias"]),
+                              lambda ps, z: (8, *ps, *ntail[:-4], *z))):
+        res = {}
+        for key, z in (("zbl", zargs), ("plain", (0.0, 0.0, zargs[2] * 0, zargs[3] * 0))):
+            ps = [q.detach().clone().requires_grad_(True) for q in params]
+            es = fn(*args(ps, z))[0]
+            (es * gs).sum().backward()
+            res[key] = (cpu(es), [cpu(q.grad) for q in ps])
+        assert close(res["zbl"][0], res["plain"][0] + zs)
+        for ga, gb in zip(res["zbl"][1], res["plain"][1]):
+            assert np.array_equal(ga, gb)
 
 
 @pytest.mark.gpu
