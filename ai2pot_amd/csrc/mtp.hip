@@ -209,18 +209,32 @@ __device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, const T
     }
 }
 
+// Sum over the pieces of a list (mtp_plan.h): the pieces sit in neighbouring lanes of one wavefront, `rem` is the
+// number of pieces behind the lane's own in its list; after `steps` doubling steps the lane of a list's first piece
+// holds the list's sum (pieces in a fixed tree order).  All 64 lanes take part.
+template <typename T>
+__device__ __forceinline__ T piece_sum(T v, int rem, int steps)
+{
+    for (int k = 0; k < steps; k++) {
+        const int d = 1 << k;
+        const T o = __shfl_down(v, d, 64);
+        v += rem >= d ? o : (T)0;
+    }
+    return v;
+}
+
 // forward products: M[dst] = sum mult M[m0] M[m1]; with TANGENT also the product rule on Tg.
-// `part` (and `part2` with TANGENT) hold one partial sum per slot of the current level.
 template <typename T, bool TANGENT, int NT>
-__device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, T* part, T* part2, int tid)
+__device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, int tid)
 {
     for (int l = 0; l < p.n_levels; l++) {
-        const int s0 = p.f_level[l], s1 = p.f_lend[l];
-        const bool multi = p.f_multi[l] != 0;
+        const int s0 = p.f_level[l], s1 = p.f_level[l + 1];     // whole groups of 64 slots: every lane of a wave walks one
+        const int steps = p.f_multi[l];
         for (int s = s0 + tid; s < s1; s += NT) {
             const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group, a multiple of 4
             const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
             const int dst = p.f_dst[s];                      // requested with the two words above
+            const int rem = steps ? p.f_rem[s] : 0;
             T acc = (T)0, tacc = (T)0;
             // all the slot's words (at most MTP_SLOT_CAP, the depth is shared by the wavefront) are requested
             // before the first is used: one trip to memory per slot
@@ -243,45 +257,32 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
                         if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
                     }
                 }
-            if (multi) {
-                part[s - s0] = acc;
-                if (TANGENT) part2[s - s0] = tacc;
-            } else {
+            if (steps) {
+                acc = piece_sum(acc, rem, steps);
+                if (TANGENT) tacc = piece_sum(tacc, rem, steps);
+            }
+            if (dst >= 0) {                                  // the first piece of a list
                 M[dst] = acc;
                 if (TANGENT) Tg[dst] = tacc;
             }
         }
         __syncthreads();
-        if (multi) {
-            for (int s = s0 + tid; s < s1; s += NT) {
-                const int np = p.f_lead[s];
-                if (np == 0) continue;
-                T acc = (T)0, tacc = (T)0;
-                for (int q = 0; q < np; q++) {
-                    acc += part[s - s0 + q];
-                    if (TANGENT) tacc += part2[s - s0 + q];
-                }
-                const int dst = p.f_dst[s];
-                M[dst] = acc;
-                if (TANGENT) Tg[dst] = tacc;
-            }
-            __syncthreads();
-        }
     }
 }
 
 // reverse gather: X[m] += sum mult (X[dst] M[other] (+ A[dst] Tg[other] when MIXED))
 template <typename T, bool MIXED, int NT>
 __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M, T* X, const T* A,
-                                              const T* Tg, T* part, int tid)
+                                              const T* Tg, int tid)
 {
     for (int l = p.n_levels - 1; l >= 0; l--) {
-        const int s0 = p.r_level[l], s1 = p.r_lend[l];
-        const bool multi = p.r_multi[l] != 0;
+        const int s0 = p.r_level[l], s1 = p.r_level[l + 1];
+        const int steps = p.r_multi[l];
         for (int s = s0 + tid; s < s1; s += NT) {
             const int depth = p.r_gdepth[s >> 6];
             const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
             const int src = p.r_src[s];
+            const int rem = steps ? p.r_rem[s] : 0;
             T acc = (T)0;
             int2 w[MTP_SLOT_CAP];
 #pragma unroll
@@ -301,21 +302,10 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
                         if (MIXED) acc += mult * A[dst] * Tg[other];
                     }
                 }
-            if (multi) part[s - s0] = acc;
-            else X[src] += acc;
+            if (steps) acc = piece_sum(acc, rem, steps);
+            if (src >= 0) X[src] += acc;
         }
         __syncthreads();
-        if (multi) {
-            for (int s = s0 + tid; s < s1; s += NT) {
-                const int np = p.r_lead[s];
-                if (np == 0) continue;
-                const int m = p.r_src[s];
-                T acc = X[m];
-                for (int q = 0; q < np; q++) acc += part[s - s0 + q];
-                X[m] = acc;
-            }
-            __syncthreads();
-        }
     }
 }
 
@@ -489,7 +479,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     }
 
     // ---- products, energy, adjoint ------------------------------------------------------------
-    sweep_forward<T, LOSS, NT>(p, M, Tg, tab, tab + p.max_level_slots, lane);
+    sweep_forward<T, LOSS, NT>(p, M, Tg, lane);
     for (int i = lane; i < n_moms; i += NT) {    // the table is dead: its place now holds the adjoints
         A[i] = (T)0;
         if (LOSS) Bm[i] = (T)0;
@@ -564,7 +554,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
         if (a.energy_only) return;
     }
     __syncthreads();
-    sweep_reverse<T, false, NT>(p, M, A, nullptr, nullptr, tab, lane);
+    sweep_reverse<T, false, NT>(p, M, A, nullptr, nullptr, lane);
 
     if (!LOSS) {
         // ---- pair derivatives ------------------------------------------------------------------
@@ -675,7 +665,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     if (LOSS) {
         const T cE = seeded ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
         // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
-        if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, tab, lane);
+        if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, lane);
         // the last pass needs the adjoints of the basic moments while the table is back in its region
         for (int i = lane; i < n_basic; i += NT) { Ab[i] = A[i]; Bb[i] = Bm[i]; }
         T* grow = a.gpart + row * a.ngrad;
@@ -960,9 +950,10 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     A2P_REQUIRE(n_moms < 65536, A2P_ERR_INVALID, "mtp plan: more than 65535 moments");
     // Interleaved gather lists (see mtp_plan.h).  `lists[m]` holds the packed terms of moment m.
     struct Ell {
-        std::vector<int> level, lend, multi, slot, lead, gbase, gdepth;
+        std::vector<int> level, lend, multi, slot, lead, gbase, gdepth;   // multi: doubling steps; lead: pieces behind
         std::vector<int2> terms;
         int max_slots = 0;
+        bool too_long = false;
     };
     auto build_ell = [&](const std::vector<std::vector<int2>>& lists, const std::vector<std::vector<int>>& by_level) {
         Ell e;
@@ -972,18 +963,24 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
             std::vector<int> ms = members;
             std::stable_sort(ms.begin(), ms.end(),
                              [&](int x, int y) { return lists[x].size() > lists[y].size(); });
-            // slots of the level: (moment, first term, term count), pieces of a list adjacent
-            struct Piece { int m, t0, n, lead; };
+            // slots of the level: (list, first term, term count, pieces behind this one); the pieces of a list are
+            // adjacent and stay inside one group of 64 slots (one wavefront adds them up with shuffles)
+            struct Piece { int m, t0, n, rem; };
             std::vector<Piece> pieces;
-            int multi = 0;
+            int most = 1;
             for (int m : ms) {
                 const int n = (int)lists[m].size();
                 const int np = (n + MTP_SLOT_CAP - 1) / MTP_SLOT_CAP;
-                if (np > 1) multi = 1;
+                if (np > 64) { e.too_long = true; continue; }
+                most = std::max(most, np);
+                if ((int)(pieces.size() % 64) + np > 64)
+                    while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
                 for (int q = 0; q < np; q++)
-                    pieces.push_back({m, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, n - q * MTP_SLOT_CAP), q == 0 ? np : 0});
+                    pieces.push_back({m, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, n - q * MTP_SLOT_CAP), np - 1 - q});
             }
-            e.multi.push_back(multi);
+            int steps = 0;
+            while ((1 << steps) < most) steps++;
+            e.multi.push_back(steps);
             for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
                 const size_t g1 = std::min(pieces.size(), g0 + 64);
                 int depth = 0;
@@ -996,8 +993,8 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
                     const Piece& pc = pieces[q];
                     for (int k = 0; k < pc.n; k++)
                         e.terms[e.gbase.back() + (size_t)k * 64 + (q - g0)] = lists[pc.m][pc.t0 + k];
-                    e.slot.push_back(pc.m);
-                    e.lead.push_back(pc.lead);
+                    e.slot.push_back(pc.t0 == 0 ? pc.m : -1);      // the first piece of a list names the moment
+                    e.lead.push_back(pc.rem);
                 }
             }
             e.lend.push_back((int)e.slot.size());
@@ -1030,6 +1027,8 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     for (int m = 0; m < n_moms; m++)
         if (level[m] < n_levels && !rl[m].empty()) r_by[level[m]].push_back(m);
     const Ell F = build_ell(fl, f_by), R = build_ell(rl, r_by);
+    A2P_REQUIRE(!F.too_long && !R.too_long, A2P_ERR_INVALID,
+                "mtp plan: a moment takes part in more than %d products; this level is too large", 64 * MTP_SLOT_CAP);
     std::vector<int> mu_begin(nmus + 1, n_basic);
     for (int i = n_basic - 1; i >= 0; i--) mu_begin[basic[i * 4]] = i;
     for (int m = nmus - 1; m >= 0; m--) mu_begin[m] = std::min(mu_begin[m], mu_begin[m + 1]);
@@ -1114,15 +1113,15 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.mapping = (const int*)(base + o_map);
     d.f_level = (const int*)(base + o_fl); d.f_lend = (const int*)(base + o_fe);
     d.f_multi = (const int*)(base + o_fx);
-    d.f_dst = (const int*)(base + o_fd); d.f_lead = (const int*)(base + o_fc);
+    d.f_dst = (const int*)(base + o_fd); d.f_rem = (const int*)(base + o_fc);
     d.f_gbase = (const int*)(base + o_fg); d.f_gdepth = (const int*)(base + o_fh);
     d.f_terms = (const int2*)(base + o_ft);
     d.r_level = (const int*)(base + o_rl); d.r_lend = (const int*)(base + o_re);
     d.r_multi = (const int*)(base + o_rx);
-    d.r_src = (const int*)(base + o_rs); d.r_lead = (const int*)(base + o_rc);
+    d.r_src = (const int*)(base + o_rs); d.r_rem = (const int*)(base + o_rc);
     d.r_gbase = (const int*)(base + o_rg); d.r_gdepth = (const int*)(base + o_rh);
     d.r_terms = (const int2*)(base + o_rt);
-    d.max_level_slots = std::max(F.max_slots, R.max_slots);
+    d.max_level_slots = 0;       // the sweeps keep no partial sums in LDS
     d.nq = nq; d.nmp = nmp; d.nrows = (int)rows.size();
     d.rows = (const int*)(base + o_rows); d.dense_src = (const int*)(base + o_dsrc);
     d.dense_off = (const int*)(base + o_doff); d.dense_items = (const int*)(base + o_dit);

@@ -29,18 +29,19 @@ struct MtpPlanDevice {
     const int* mu_begin;       // [nmus+1]     basics are grouped by mu: run of each mu
     const int* mapping;        // [n_scalar]
     // forward gather.  A slot holds up to MTP_SLOT_CAP terms of one destination moment; a longer
-    // list is cut into consecutive slots (pieces) whose partial sums are added in slot order, so
-    // that no lane walks a long list alone.  Slots are grouped 64 at a time; level l covers slots
-    // [f_level[l], f_lend[l]) and starts at a multiple of 64.  The terms of a group are stored
+    // list is cut into consecutive slots (pieces), so that no lane walks a long list alone; the pieces of a
+    // list lie in one group of 64 slots and the wavefront that walks the group adds their partial sums with
+    // shuffles (f_multi[l] doubling steps).  Slots are grouped 64 at a time; level l covers slots
+    // [f_level[l], f_level[l+1]) (whole groups; [f_level[l], f_lend[l]) without the padding slots).  The terms of a group are stored
     // interleaved and padded with zero terms to the group's depth (a multiple of four): term k of slot s is
     // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
     // a group read consecutive words and share the trip count.  A term packs x = m0 | m1 << 16,
     // y = multiplicity.
     const int* f_level;        // [n_levels+1]
     const int* f_lend;         // [n_levels+1]
-    const int* f_multi;        // [n_levels]   1 when the level has a list cut into pieces
-    const int* f_dst;          // [n_fslots]   destination (-1 in padding slots)
-    const int* f_lead;         // [n_fslots]   number of pieces if the slot is the first of its list, else 0
+    const int* f_multi;        // [n_levels]   doubling steps that add up the longest list's pieces (0: no list is cut)
+    const int* f_dst;          // [n_fslots]   destination in the first piece of a list (-1 elsewhere and in padding)
+    const int* f_rem;          // [n_fslots]   pieces of the same list behind this one
     const int* f_gbase;        // [n_fslots/64]
     const int* f_gdepth;       // [n_fslots/64]
     const int2* f_terms;
@@ -50,7 +51,7 @@ struct MtpPlanDevice {
     const int* r_lend;         // [n_levels+1]
     const int* r_multi;        // [n_levels]
     const int* r_src;          // [n_rslots]
-    const int* r_lead;         // [n_rslots]
+    const int* r_rem;          // [n_rslots]
     const int* r_gbase;        // [n_rslots/64]
     const int* r_gdepth;       // [n_rslots/64]
     const int2* r_terms;
