@@ -18,7 +18,7 @@ struct NepModel {
 
 NepModel check_model(int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const at::Tensor& coeffs,
                      const at::Tensor& w0, const at::Tensor& b0, const at::Tensor& w1, const at::Tensor& bias,
-                     const at::Tensor& type_map, const at::Tensor& brcs)
+                     const at::Tensor& type_map, const at::Tensor& brcs, int64_t l4 = 0, int64_t l5 = 0)
 {
     NepModel m;
     m.K = (int)K; m.n_r = (int)n_r; m.n_a = (int)n_a; m.l_max = (int)l_max;
@@ -31,7 +31,9 @@ NepModel check_model(int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, const a
     check_device_float(brcs, w1, "w1");
     check_device_float(brcs, bias, "type_bias");
     m.H = (int)(w1.numel() / m.ntypes);
-    m.D = l_max == 0 ? m.n_r : m.n_r + m.n_a * m.l_max;
+    TORCH_CHECK((l4 == 0 || l4 == 2) && (l5 == 0 || l5 == 1) && l_max >= l4 && l_max >= l5,
+                "l_4body must be 0 or 2, l_5body 0 or 1, and l_max at least as large");
+    m.D = l_max == 0 ? m.n_r : m.n_r + m.n_a * (m.l_max + (l4 ? 1 : 0) + (l5 ? 1 : 0));
     TORCH_CHECK(m.H > 0 && w0.numel() == (int64_t)m.ntypes * m.H * m.D, "w0 must have ntypes*H*D elements");
     TORCH_CHECK(b0.numel() == (int64_t)m.ntypes * m.H && bias.numel() == m.ntypes, "b0 / type_bias size mismatch");
     TORCH_CHECK(coeffs.numel() == (int64_t)m.ntypes * m.ntypes * (m.n_r + m.n_a) * m.K, "coeffs size mismatch");
@@ -43,10 +45,10 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
                       const at::Tensor& bias, const at::Tensor& binum, const at::Tensor& bilist,
                       const at::Tensor& bnumneigh, const at::Tensor& bfirstneigh, const at::Tensor& brcs,
                       const at::Tensor& btypes, const at::Tensor& type_map, int64_t nghost, double rr, double ra,
-                      const at::Tensor& q_scaler)
+                      const at::Tensor& q_scaler, int64_t l4 = 0, int64_t l5 = 0)
 {
     Batch s = check_batch(binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, nghost);
-    NepModel m = check_model(K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, type_map, brcs);
+    NepModel m = check_model(K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, type_map, brcs, l4, l5);
     check_device_float(brcs, q_scaler, "q_scaler");
     TORCH_CHECK(q_scaler.numel() == m.D, "q_scaler must have ", m.D, " elements");
     a2p_bind::DeviceGuard guard(brcs);
@@ -63,7 +65,24 @@ variable_list nep_run(bool want_virial, bool want_desc, int64_t K, int64_t n_r, 
     void* st = current_stream(brcs);
     auto call = [&]() -> int {
         int rc;
-        if (brcs.scalar_type() == at::kFloat) {
+        if (l4 || l5) {        // the extension with four- / five-body invariants: its own entry points
+            if (brcs.scalar_type() == at::kFloat)
+                rc = a2p_nep_efv_manybody_f32(m.K, m.n_r, m.n_a, m.l_max, (int)l4, (int)l5, m.H, m.ntypes,
+                                              coeffs.data_ptr<float>(), w0.data_ptr<float>(), b0.data_ptr<float>(),
+                                              w1.data_ptr<float>(), bias.data_ptr<float>(), q_scaler.data_ptr<float>(), rr,
+                                              ra, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(), bilist.data_ptr<int>(),
+                                              bnumneigh.data_ptr<int>(), bfirstneigh.data_ptr<int>(),
+                                              brcs.data_ptr<float>(), btypes.data_ptr<int>(), e.data_ptr<float>(),
+                                              f.data_ptr<float>(), v.data_ptr<float>(), nullptr, st);
+            else
+                rc = a2p_nep_efv_manybody_f64(m.K, m.n_r, m.n_a, m.l_max, (int)l4, (int)l5, m.H, m.ntypes,
+                                              coeffs.data_ptr<double>(), w0.data_ptr<double>(), b0.data_ptr<double>(),
+                                              w1.data_ptr<double>(), bias.data_ptr<double>(), q_scaler.data_ptr<double>(),
+                                              rr, ra, s.B, s.P, s.U, s.nghost, binum.data_ptr<int>(),
+                                              bilist.data_ptr<int>(), bnumneigh.data_ptr<int>(),
+                                              bfirstneigh.data_ptr<int>(), brcs.data_ptr<double>(), btypes.data_ptr<int>(),
+                                              e.data_ptr<double>(), f.data_ptr<double>(), v.data_ptr<double>(), nullptr, st);
+        } else if (brcs.scalar_type() == at::kFloat) {
             rc = a2p_nep_efv_f32(m.K, m.n_r, m.n_a, m.l_max, m.H, m.ntypes, coeffs.data_ptr<float>(),
                                  w0.data_ptr<float>(), b0.data_ptr<float>(), w1.data_ptr<float>(),
                                  bias.data_ptr<float>(), q_scaler.data_ptr<float>(), rr, ra, s.B, s.P, s.U, s.nghost,
@@ -255,6 +274,18 @@ TORCH_LIBRARY(nep, m)
               apply_zbl(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs,
                         btypes, nghost, out[0], out[1], out[2]);
               return out;
+          });
+    // EXTENSION, no counterpart in the reference (parity unpinned): nepToEFVOp with one four-body (l_4body = 2) and /
+    // or one five-body (l_5body = 1) invariant per angular channel; see include/ai2pot_hip.h, a2p_nep_efv_manybody_*
+    m.def("nepToEFVManyBodyOp",
+          [](int64_t K, int64_t n_r, int64_t n_a, int64_t l_max, int64_t l_4body, int64_t l_5body,
+             const at::Tensor& coeffs, const at::Tensor& w0, const at::Tensor& b0, const at::Tensor& w1,
+             const at::Tensor& bias, const at::Tensor& binum, const at::Tensor& bilist, const at::Tensor& bnumneigh,
+             const at::Tensor& bfirstneigh, const at::Tensor& brcs, const at::Tensor& btypes,
+             const at::Tensor& type_map, int64_t nghost, double rr, double ra,
+             const at::Tensor& q_scaler) -> variable_list {
+              return nep_run(true, false, K, n_r, n_a, l_max, coeffs, w0, b0, w1, bias, binum, bilist, bnumneigh,
+                             bfirstneigh, brcs, btypes, type_map, nghost, rr, ra, q_scaler, l_4body, l_5body);
           });
     m.def("nepToLossOp",
           [](double e_w, double f_w, double v_w, const at::Tensor& e_dft, const at::Tensor& f_dft,

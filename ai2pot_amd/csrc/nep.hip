@@ -31,12 +31,18 @@ constexpr int NEP_BLOCK = 128;
 // KC, NRC, NAC, LC: compile-time capacities; the runtime sizes in `a` must not exceed them.
 // EXACT: the runtime sizes equal the capacities and the network weights are in LDS (fast
 // path: every loop bound and descriptor slot is a compile-time constant).
-template <typename T, int KC, int NRC, int NAC, int LC, bool EXACT>
+// MB: the extension with one four-body (from the l = 2 moments) and / or one five-body (l = 1) invariant per angular
+// channel (a.mb4, a.mb5; weights of source/descriptor/ace/include/nep_descriptor.h:43-54, whose routines for them
+// are declared and never defined: there is no reference result for these descriptors).  Descriptor order per
+// channel: l = 1 .. l_max, then the four-body, then the five-body entry.
+template <typename T, int KC, int NRC, int NAC, int LC, bool EXACT, bool MB = false>
 __global__ void __launch_bounds__(NEP_BLOCK)
 nep_efv_kernel(const NepArgs<T> a)
 {
+    static_assert(!(MB && EXACT), "the many-body extension runs with runtime sizes");
     constexpr int NLM = LC * LC + 2 * LC;
-    constexpr int DC = NRC + NAC * LC;
+    constexpr int LCX = LC + (MB ? 2 : 0);       // descriptor slots per angular channel
+    constexpr int DC = NRC + NAC * LCX;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tid = threadIdx.x;
     const int b = blockIdx.y;
@@ -171,17 +177,39 @@ nep_efv_kernel(const NepArgs<T> a)
                     const int m = l * l - 1 + mp;
                     acc += (T)(mp == 0 ? 1.0 : 2.0) * (T)kC3B[m] * S[n][m] * S[n][m];
                 }
-                q[NRC + n * LC + (l - 1)] = acc;
+                q[NRC + n * LCX + (l - 1)] = acc;
             }
         }
+    if (MB) {
+        // q_4b from s[3..7] (l = 2), q_5b from s[0..2] (l = 1)
+#pragma unroll
+        for (int n = 0; n < NAC; n++) {
+            if (n < n_a) {
+                const T* s = S[n];
+                if (LC >= 2 && a.mb4)
+                    q[NRC + n * LCX + LC] = (T)kC4B[0] * s[3] * s[3] * s[3] + (T)kC4B[1] * s[3] * (s[4] * s[4] + s[5] * s[5]) +
+                                            (T)kC4B[2] * s[3] * (s[6] * s[6] + s[7] * s[7]) +
+                                            (T)kC4B[3] * s[6] * (s[5] * s[5] - s[4] * s[4]) + (T)kC4B[4] * s[4] * s[5] * s[7];
+                if (a.mb5) {
+                    const T p0 = s[0] * s[0], p1 = s[1] * s[1] + s[2] * s[2];
+                    q[NRC + n * LCX + LC + 1] = (T)kC5B[0] * p0 * p0 + (T)kC5B[1] * p0 * p1 + (T)kC5B[2] * p1 * p1;
+                }
+            }
+        }
+    }
 
     // Static slot j of q[] holds the descriptor whose index in the reference's runtime order
     // (n_r radial, then n*l_max + l-1) is kmap(j); -1 marks a slot the runtime sizes leave unused.
     auto kmap = [&](int j) -> int {
         if (EXACT) return j;
         if (j < NRC) return (j < n_r) ? j : -1;
-        const int n = (j - NRC) / LC, l = (j - NRC) % LC;
-        return (n < n_a && l < l_max) ? n_r + n * l_max + l : -1;
+        const int n = (j - NRC) / LCX, l = (j - NRC) % LCX;
+        if (!MB) return (n < n_a && l < l_max) ? n_r + n * l_max + l : -1;
+        const int num_l = l_max + a.mb4 + a.mb5;
+        if (n >= n_a) return -1;
+        if (l < LC) return l < l_max ? n_r + n * num_l + l : -1;
+        if (l == LC) return a.mb4 ? n_r + n * num_l + l_max : -1;
+        return a.mb5 ? n_r + n * num_l + l_max + a.mb4 : -1;
     };
 
     if (active && a.desc) {
@@ -233,14 +261,38 @@ nep_efv_kernel(const NepArgs<T> a)
     }
     // dE/dS (nep.h:450-466), overwriting S
 #pragma unroll
-    for (int n = 0; n < NAC; n++)
+    for (int n = 0; n < NAC; n++) {
+        T extra[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) extra[k] = (T)0;
+        if (MB && n < n_a) {
+            const T* s = S[n];
+            if (LC >= 2 && a.mb4) {
+                const T w = dEdq[NRC + n * LCX + LC];
+                extra[3] = w * ((T)3 * (T)kC4B[0] * s[3] * s[3] + (T)kC4B[1] * (s[4] * s[4] + s[5] * s[5]) +
+                                (T)kC4B[2] * (s[6] * s[6] + s[7] * s[7]));
+                extra[4] = w * ((T)2 * (T)kC4B[1] * s[3] * s[4] - (T)2 * (T)kC4B[3] * s[6] * s[4] + (T)kC4B[4] * s[5] * s[7]);
+                extra[5] = w * ((T)2 * (T)kC4B[1] * s[3] * s[5] + (T)2 * (T)kC4B[3] * s[6] * s[5] + (T)kC4B[4] * s[4] * s[7]);
+                extra[6] = w * ((T)2 * (T)kC4B[2] * s[3] * s[6] + (T)kC4B[3] * (s[5] * s[5] - s[4] * s[4]));
+                extra[7] = w * ((T)2 * (T)kC4B[2] * s[3] * s[7] + (T)kC4B[4] * s[4] * s[5]);
+            }
+            if (a.mb5) {
+                const T w = dEdq[NRC + n * LCX + LC + 1];
+                const T p0 = s[0] * s[0], p1 = s[1] * s[1] + s[2] * s[2];
+                extra[0] = w * ((T)4 * (T)kC5B[0] * p0 * s[0] + (T)2 * (T)kC5B[1] * s[0] * p1);
+                extra[1] = w * ((T)2 * (T)kC5B[1] * p0 * s[1] + (T)4 * (T)kC5B[2] * p1 * s[1]);
+                extra[2] = w * ((T)2 * (T)kC5B[1] * p0 * s[2] + (T)4 * (T)kC5B[2] * p1 * s[2]);
+            }
+        }
 #pragma unroll
         for (int l = 1; l <= LC; l++)
 #pragma unroll
             for (int mp = 0; mp < 2 * l + 1; mp++) {
                 const int m = l * l - 1 + mp;
-                S[n][m] *= dEdq[NRC + n * LC + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+                S[n][m] *= dEdq[NRC + n * LCX + (l - 1)] * (T)(mp == 0 ? 2.0 : 4.0) * (T)kC3B[m];
+                if (MB && m < 8) S[n][m] += extra[m];
             }
+    }
 
     // ---- sweeps 3 and 4: pair derivatives ----------------------------------------------------
     T fx = (T)0, fy = (T)0, fz = (T)0;
@@ -373,10 +425,10 @@ size_t nep_lds_bytes(const NepArgs<T>& a)
     return std::max(bytes, (size_t)(NEP_BLOCK / 64) * 10 * sizeof(double));
 }
 
-template <typename T, int KC, int NRC, int NAC, int LC, bool EXACT>
+template <typename T, int KC, int NRC, int NAC, int LC, bool EXACT, bool MB = false>
 int launch(const NepArgs<T>& a, size_t lds, hipStream_t stream)
 {
-    auto kern = nep_efv_kernel<T, KC, NRC, NAC, LC, EXACT>;
+    auto kern = nep_efv_kernel<T, KC, NRC, NAC, LC, EXACT, MB>;
     if (lds > 48 * 1024)
         A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds));
@@ -392,8 +444,11 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
             const T* b0, const T* w1, const T* bias, const T* q_scaler, double rr, double ra, int B,
             int P, int U, int nghost, const int* binum, const int* bilist, const int* bnumneigh,
             const int* bfirstneigh, const T* brcs, const int* btypes, T* etot, T* force, T* virial,
-            T* desc, hipStream_t stream, int* brank = nullptr, int* bincoming = nullptr, int ranks_valid = 0)
+            T* desc, hipStream_t stream, int* brank = nullptr, int* bincoming = nullptr, int ranks_valid = 0,
+            int mb4 = 0, int mb5 = 0)
 {
+    A2P_REQUIRE((mb4 == 0 || l_max >= 2) && (mb5 == 0 || l_max >= 1) && (mb4 | mb5 | 1) == 1, A2P_ERR_INVALID,
+                "nep: the four-body term needs l_max >= 2, the five-body term l_max >= 1");
     A2P_REQUIRE((brank == nullptr) == (bincoming == nullptr), A2P_ERR_INVALID,
                 "nep: pair ranks and incoming counts come together");
     A2P_REQUIRE(K >= 1 && K <= 16, A2P_ERR_INVALID, "nep: chebyshev_size %d outside [1, 16]", K);
@@ -412,7 +467,8 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
 
     NepArgs<T> a;
     a.K = K; a.n_r = n_r; a.n_a = n_a; a.l_max = l_max; a.H = H; a.ntypes = ntypes;
-    a.D = (l_max == 0) ? n_r : n_r + n_a * l_max;     // nep_utilities.h:39-49
+    a.mb4 = mb4; a.mb5 = mb5;
+    a.D = (l_max == 0) ? n_r : n_r + n_a * (l_max + mb4 + mb5);     // nep_utilities.h:39-49
     a.coeffs = coeffs; a.w0 = w0; a.b0 = b0; a.w1 = w1; a.bias = bias; a.q_scaler = q_scaler;
     a.rr = (T)rr; a.ra = (T)ra;
     a.B = B; a.P = P; a.U = U; a.nghost = nghost; a.nblocks = ceil_div(P, NEP_BLOCK);
@@ -432,7 +488,7 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
     a.force = force;
     a.pair_g = nullptr;
     size_t lds_staged = 0;
-    const bool staged = nep_staged_supported<T>(a, &lds_staged);
+    const bool staged = !(mb4 || mb5) && nep_staged_supported<T>(a, &lds_staged);
     if (staged) a.nblocks = nep_staged_nblocks(P);
     size_t lds_group = 0;
     // fewer staged workgroups than half the compute units: the system is small, spread it wider
@@ -467,7 +523,10 @@ int nep_efv(int K, int n_r, int n_a, int l_max, int H, int ntypes, const T* coef
             rc = fill_zero(a.force, force_bytes, stream);
             if (rc) return rc;
         }
-        if (K <= 8 && n_r <= 6 && n_a <= 4 && l_max <= 3)
+        if (mb4 || mb5)
+            rc = (K <= 8 && n_r <= 6 && n_a <= 4) ? launch<T, 8, 6, 4, 4, false, true>(a, lds, stream)
+                                                  : launch<T, 16, 12, 8, 4, false, true>(a, lds, stream);
+        else if (K <= 8 && n_r <= 6 && n_a <= 4 && l_max <= 3)
             rc = launch<T, 8, 6, 4, 3, false>(a, lds, stream);
         else if (K <= 8 && n_r <= 6 && n_a <= 4)
             rc = launch<T, 8, 6, 4, 4, false>(a, lds, stream);
@@ -535,5 +594,34 @@ int a2p_nep_efv_ranked_f64(int K, int n_r, int n_a, int l_max, int H, int ntypes
     return a2p::nep_efv<double>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra,
                                 B, P, U, nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot,
                                 force, virial, desc, (hipStream_t)stream, brank, bincoming, ranks_valid);
+}
+
+/* extension: four- / five-body invariants (l_4body 0 or 2, l_5body 0 or 1); no counterpart in the reference */
+int a2p_nep_efv_manybody_f32(int K, int n_r, int n_a, int l_max, int l_4body, int l_5body, int H, int ntypes,
+                             const float* coeffs, const float* w0, const float* b0, const float* w1, const float* bias,
+                             const float* q_scaler, double rr, double ra, int B, int P, int U, int nghost,
+                             const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
+                             const float* brcs, const int* btypes, float* etot, float* force, float* virial,
+                             float* desc, void* stream)
+{
+    A2P_REQUIRE((l_4body == 0 || l_4body == 2) && (l_5body == 0 || l_5body == 1), A2P_ERR_INVALID,
+                "nep: l_4body must be 0 or 2, l_5body 0 or 1");
+    return a2p::nep_efv<float>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra, B, P, U,
+                               nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, desc,
+                               (hipStream_t)stream, nullptr, nullptr, 0, l_4body ? 1 : 0, l_5body ? 1 : 0);
+}
+
+int a2p_nep_efv_manybody_f64(int K, int n_r, int n_a, int l_max, int l_4body, int l_5body, int H, int ntypes,
+                             const double* coeffs, const double* w0, const double* b0, const double* w1,
+                             const double* bias, const double* q_scaler, double rr, double ra, int B, int P, int U,
+                             int nghost, const int* binum, const int* bilist, const int* bnumneigh,
+                             const int* bfirstneigh, const double* brcs, const int* btypes, double* etot, double* force,
+                             double* virial, double* desc, void* stream)
+{
+    A2P_REQUIRE((l_4body == 0 || l_4body == 2) && (l_5body == 0 || l_5body == 1), A2P_ERR_INVALID,
+                "nep: l_4body must be 0 or 2, l_5body 0 or 1");
+    return a2p::nep_efv<double>(K, n_r, n_a, l_max, H, ntypes, coeffs, w0, b0, w1, bias, q_scaler, rr, ra, B, P, U,
+                                nghost, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, etot, force, virial, desc,
+                                (hipStream_t)stream, nullptr, nullptr, 0, l_4body ? 1 : 0, l_5body ? 1 : 0);
 }
 }

@@ -18,6 +18,12 @@ __device__ constexpr double kC3B[24] = {
     0.223811638722978, 0.223811638722978f, 0.111905819361489f, 0.111905819361489f,
     1.566681471060845, 1.566681471060845f, 0.195835183882606f, 0.195835183882606f};
 
+// weights of the four- and five-body invariants of the extension (source/descriptor/ace/include/nep_descriptor.h:43-54;
+// the reference never evaluates them)
+__device__ constexpr double kC4B[5] = {-0.007499480826664, -0.134990654879954, 0.067495327439977, 0.404971964639861,
+                                       -0.809943929279723};
+__device__ constexpr double kC5B[3] = {0.026596810706114, 0.053193621412227, 0.026596810706114};
+
 template <typename T>
 struct NepArgs {
     int K, n_r, n_a, l_max, H, ntypes, D;
@@ -41,6 +47,7 @@ struct NepArgs {
     int* brank;
     int* bincoming;
     int ranks_valid;
+    int mb4 = 0, mb5 = 0;   // extension (generic kernel only): four- / five-body invariant per angular channel
 };
 
 __device__ __forceinline__ void sincospi_t(float x, float* s, float* c) { sincospif(x, s, c); }

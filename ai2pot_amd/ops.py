@@ -90,12 +90,14 @@ def _validate_batch(binum, bnumneigh, U, P):
 # --------------------------------------------------------------------------------------------
 def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs,
               w0, b0, w1, type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map,
-              nghost, rmax_radial, rmax_angular, q_scaler, validate=True):
+              nghost, rmax_radial, rmax_angular, q_scaler, validate=True, l_4body=0, l_5body=0):
     _req(isinstance(brcs, torch.Tensor) and brcs.is_cuda,
          "brcs must be a tensor on a HIP device: this build has no CPU path")
     dtype, device = brcs.dtype, brcs.device
     _req(dtype in (torch.float32, torch.float64), "brcs must be float32 or float64")
     _req(brcs.is_contiguous(), "brcs must be contiguous")
+    many_body = bool(l_4body or l_5body)
+    _req(l_4body in (0, 2) and l_5body in (0, 1), "l_4body must be 0 or 2, l_5body 0 or 1")
     for name, t in (("coeffs", coeffs), ("w0", w0), ("b0", b0), ("w1", w1), ("type_bias", type_bias)):
         _check_float(name, t, dtype, device)
     for name, t in (("binum", binum), ("bilist", bilist), ("bnumneigh", bnumneigh),
@@ -107,7 +109,9 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
     _req(ntypes > 0, "type_map is empty")
     _req(0 <= l_max <= 4, "l_max must be in [0, 4]")     # nep.py:50 / nep_utilities.h:46
     H = w1.numel() // ntypes
-    D = n_radial_basis + n_angular_basis * l_max if l_max > 0 else n_radial_basis
+    num_l = l_max + (1 if l_4body else 0) + (1 if l_5body else 0)
+    _req(not many_body or l_max >= max(l_4body, l_5body), "the four-body term needs l_max >= 2, the five-body term l_max >= 1")
+    D = n_radial_basis + n_angular_basis * num_l if l_max > 0 else n_radial_basis
     _req(w0.numel() == ntypes * H * D, "w0 has %d elements, expected ntypes*H*D = %d"
          % (w0.numel(), ntypes * H * D))
     _req(b0.numel() == ntypes * H and type_bias.numel() == ntypes, "b0 / type_bias size mismatch")
@@ -133,10 +137,15 @@ def _nep_call(want_virial, want_desc, chebyshev_size, n_radial_basis, n_angular_
         if want_virial:
             virial = new((B, 9), dtype=dtype, device=device)
     L = _lib.lib()
-    fn = L.a2p_nep_efv_f32 if dtype == torch.float32 else L.a2p_nep_efv_f64
+    if many_body:
+        fn = L.a2p_nep_efv_manybody_f32 if dtype == torch.float32 else L.a2p_nep_efv_manybody_f64
+        lead = (_c.c_int(l_max), _c.c_int(l_4body), _c.c_int(l_5body))
+    else:
+        fn = L.a2p_nep_efv_f32 if dtype == torch.float32 else L.a2p_nep_efv_f64
+        lead = (_c.c_int(l_max),)
     with torch.cuda.device(device):
         call = lambda: fn(_c.c_int(chebyshev_size), _c.c_int(n_radial_basis), _c.c_int(n_angular_basis),
-                _c.c_int(l_max), _c.c_int(H), _c.c_int(ntypes), _ptr(coeffs), _ptr(w0), _ptr(b0),
+                *lead, _c.c_int(H), _c.c_int(ntypes), _ptr(coeffs), _ptr(w0), _ptr(b0),
                 _ptr(w1), _ptr(type_bias), _ptr(q_scaler_t), _c.c_double(rmax_radial),
                 _c.c_double(rmax_angular), _c.c_int(B), _c.c_int(P), _c.c_int(U), _c.c_int(nghost),
                 _ptr(binum), _ptr(bilist), _ptr(bnumneigh), _ptr(bfirstneigh), _ptr(brcs),
@@ -236,6 +245,32 @@ def nepToEFVOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w
                            type_map, nghost, rmax_radial, rmax_angular, q_scaler, validate)
     _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
              nghost, e, f, v, validate)
+    return [e, f, v]
+
+
+def nepToEFVManyBodyOp(chebyshev_size, n_radial_basis, n_angular_basis, l_max, l_4body, l_5body, coeffs, w0, b0, w1,
+                       type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost, rmax_radial,
+                       rmax_angular, q_scaler, want_descriptors=False, validate=True):
+    """EXTENSION, no counterpart in the reference (PARITY UNPINNED): nepToEFVOp with one four-body invariant (from
+    the l = 2 moments, l_4body = 2) and / or one five-body invariant (l = 1, l_5body = 1) per angular channel, the
+    descriptors of a channel ordered l = 1 .. l_max, four-body, five-body, so D = n_radial + n_angular * (l_max +
+    [l_4body > 0] + [l_5body > 0]) sets the shapes of w0 and q_scaler.  The reference's operators have radial and
+    three-body terms only (nep_bind.cc:81-105); its unfinished draft holds the weights
+    (source/descriptor/ace/include/nep_descriptor.h:43-54) and no code that uses them.  Checked by rotation
+    invariance, finite differences and the reduction to nepToEFVOp.  Returns [E, F, V], or [descriptors] with
+    want_descriptors."""
+    if want_descriptors:
+        ntypes = int(type_map.numel())
+        D = n_radial_basis + n_angular_basis * (l_max + (1 if l_4body else 0) + (1 if l_5body else 0))
+        z = lambda *sh: torch.zeros(sh, dtype=brcs.dtype, device=brcs.device)
+        _, _, _, d = _nep_call(False, True, chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs,
+                               z(ntypes * D), z(ntypes), z(ntypes), z(ntypes), binum, bilist, bnumneigh, bfirstneigh,
+                               brcs, btypes, type_map, nghost, rmax_radial, rmax_angular, None, validate,
+                               l_4body=l_4body, l_5body=l_5body)
+        return [d]
+    e, f, v, _ = _nep_call(True, False, chebyshev_size, n_radial_basis, n_angular_basis, l_max, coeffs, w0, b0, w1,
+                           type_bias, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, nghost,
+                           rmax_radial, rmax_angular, q_scaler, validate, l_4body=l_4body, l_5body=l_5body)
     return [e, f, v]
 
 

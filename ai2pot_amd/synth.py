@@ -140,10 +140,13 @@ def fcc_cell(reps, a, sigma, seed):
 # ----------------------------------------------------------------------------------------
 def nep_model(ntypes=3, n_radial_basis=6, n_angular_basis=4, l_max=4, chebyshev_size=8,
               num_neurons=50, rmax_radial=7.0, rmax_angular=4.0, seed=3002, sigma=0.1,
-              type_map=(32, 51, 52)):
-    D = n_radial_basis + n_angular_basis * l_max
+              type_map=(32, 51, 52), l_4body=0, l_5body=0):
+    """l_4body = 2 / l_5body = 1 add one four-body / five-body invariant per angular channel (an extension: the
+    reference's operators have no such descriptors)."""
+    D = n_radial_basis + n_angular_basis * (l_max + (1 if l_4body else 0) + (1 if l_5body else 0))
     ncoef = ntypes * ntypes * (n_radial_basis + n_angular_basis) * chebyshev_size
-    return dict(chebyshev_size=chebyshev_size, n_radial_basis=n_radial_basis,
+    extra = dict(l_4body=l_4body, l_5body=l_5body) if (l_4body or l_5body) else {}
+    return dict(extra, chebyshev_size=chebyshev_size, n_radial_basis=n_radial_basis,
                 n_angular_basis=n_angular_basis, l_max=l_max, rmax_radial=rmax_radial,
                 rmax_angular=rmax_angular,
                 coeffs=rng_normal(seed, ncoef, 0, sigma),

@@ -131,14 +131,45 @@ def timed_replay(replay, steps, warmup):
     return time.perf_counter() - t0
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
-# counters read for a plain copy of known size (2.00 for FETCH_SIZE, 1.00 for WRITE_SIZE); the runs are
-# summarised in profiles/<workload>_hbm_traffic.txt.  Kernels without a counter run report null.
-MEASURED_TRAFFIC = {
-    ("nep_md_1048576", "nbl_lists"): (2.00 * 2.082e5 + 1.640e6) * 1024,
-    ("nep_md_1048576", "nep_adjoint_kernel"): (2.00 * 6.065e5 + 6.429e5) * 1024,
-    ("nep_md_1048576", "nep_gather_kernel"): (2.00 * 5.695e5 + 3.582e4) * 1024,
-}
+# Counter figures come from the rocprofv3 summaries under profiles/: a line
+#     @data <workload> <kernel> fetch_kib=<FETCH_SIZE> write_kib=<WRITE_SIZE> flops_executed=<flops per launch>
+# holds, per launch of one kernel, the raw FETCH_SIZE / WRITE_SIZE readings (KiB; scaled here by what the same
+# counters read for a plain copy of known size: 2.00 and 1.00, `bench.py --workload hbm_copy_probe`) and the
+# floating-point operations the kernel executed (2 x FMA + MUL + ADD instructions x 64 lanes).  Kernels without
+# such a line report null.
+FETCH_SCALE, WRITE_SCALE = 2.00, 1.00
+_PROFILE_DATA = None
+
+
+def profile_data():
+    global _PROFILE_DATA
+    if _PROFILE_DATA is None:
+        _PROFILE_DATA = {}
+        root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+        for name in sorted(os.listdir(root)) if os.path.isdir(root) else []:
+            if not name.endswith(".txt"):
+                continue
+            with open(os.path.join(root, name)) as f:
+                for line in f:
+                    if not line.startswith("@data "):
+                        continue
+                    parts = line.split()
+                    rec = _PROFILE_DATA.setdefault((parts[1], parts[2]), {})
+                    for kv in parts[3:]:
+                        k, v = kv.split("=")
+                        rec[k] = float(v)
+    return _PROFILE_DATA
+
+
+def measured_traffic(workload, kernel):
+    rec = profile_data().get((workload, kernel), {})
+    if "fetch_kib" not in rec or "write_kib" not in rec:
+        return None
+    return (FETCH_SCALE * rec["fetch_kib"] + WRITE_SCALE * rec["write_kib"]) * 1024.0
+
+
+def executed_flops(workload, kernel):
+    return profile_data().get((workload, kernel), {}).get("flops_executed")
 
 
 def roofline_of(kernels, work, workload=None):
@@ -153,10 +184,20 @@ def roofline_of(kernels, work, workload=None):
         bound, amount, unit, peak, scale, engine = work[label]
         avg_ms = sum(kernels[nm]["avg_ms"] for nm in names)
         achieved = amount / (avg_ms * 1e-3) / scale
-        traffic = [MEASURED_TRAFFIC.get((workload, nm)) for nm in names]
-        return dict(kernel=label, bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
-                    traffic=sum(traffic) if all(t is not None for t in traffic) else None, avg_ms=avg_ms,
-                    engine=engine, amount_per_launch=amount)
+        traffic = [measured_traffic(workload, nm) for nm in names]
+        e = dict(kernel=label, bound=bound, achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
+                 traffic=sum(traffic) if all(t is not None for t in traffic) else None, avg_ms=avg_ms,
+                 engine=engine, amount_per_launch=amount)
+        if bound == "valu":
+            # what the kernels executed (counter run under profiles/) beside the algorithmic count above
+            ex = [executed_flops(workload, nm) for nm in names]
+            if all(x is not None for x in ex):
+                e["executed"] = sum(ex) / (avg_ms * 1e-3) / scale
+                e["executed_frac"] = e["executed"] / peak
+                e["executed_per_launch"] = sum(ex)
+            else:
+                e["executed"] = None
+        return e
     entries = [e for e in (entry(l) for l in work) if e is not None]
     if not entries:
         return None, []
@@ -292,6 +333,27 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
     calc.check()
     if not np.isfinite(float(calc.etot.item())):
         sys.exit("bench.py: non-finite energy")
+    order_refresh = None
+    if rebuild and calc.path == "gather" and not via_ops:
+        # The processing order of the atoms (a locality hint) is renewed every calc.reorder_every rebuilds: the timed
+        # region holds such a rebuild whenever it spans a multiple of that count.  Its cost, measured on its own:
+        def rebuild_ms(refresh, reps=6):
+            best = None
+            for _ in range(reps):
+                calc._builds = calc.reorder_every if refresh else 1
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                calc.rebuild(coords, stream)
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) * 1e3
+                best = dt if best is None else min(best, dt)
+            return best
+        kept, fresh = rebuild_ms(False), rebuild_ms(True)
+        first, last = args.warmup + 1, args.warmup + args.steps        # the calculator's build counter in the timed region
+        inside = last // calc.reorder_every - (first - 1) // calc.reorder_every
+        order_refresh = dict(reorder_every=calc.reorder_every, rebuild_ms_order_kept=kept, rebuild_ms_order_renewed=fresh,
+                             amortised_ms_per_step=(fresh - kept) / calc.reorder_every,
+                             renewals_inside_timed_region=inside)
     nn_r = float(calc.numneigh.float().mean().item())
     r = calc.rcs.norm(dim=2)
     nn_a = float(((r > 0) & (r <= model["rmax_angular"])).sum().item()) / n
@@ -321,6 +383,9 @@ def run_nep_md(args, kind, size, rebuild=True, via_ops=False):
         gbs = efv_bytes / (roof["avg_ms"] * 1e-3) / 1e9
         roof["hbm"] = dict(achieved=gbs, peak=PEAK_HBM_GBS, unit="GB/s", frac=gbs / PEAK_HBM_GBS, amount_per_launch=efv_bytes)
     extra = {"rooflines": entries}
+    if order_refresh is not None:
+        extra["order_refresh"] = order_refresh
+        config["reorder_every"] = calc.reorder_every
     if rebuild and calc.path == "gather" and not args.graph and not args.no_other_configs:
         # the same step without the padded firstneigh / rcs arrays (energy, forces and virial only)
         lean = NepCalculator(model, n, lattice, types, umax=200, dtype=torch.float32, device=dev, padded=False,
@@ -664,7 +729,7 @@ def main():
         import copy
         import torch
         others = {}
-        for wl in ("mtp10_efv_216", "nep_efv_4096", "mtp20_efv_8192", "mtp16_train_64x128"):
+        for wl in ("mtp10_efv_216", "nep_efv_4096", "mtp20_efv_8192", "mtp16_train_64x128", "nep_train_64x128"):
             a2 = copy.copy(args)
             a2.workload, a2.steps, a2.warmup = wl, 50, 5
             try:
@@ -672,7 +737,8 @@ def main():
                 others[wl] = dict(natoms=n2, ms_per_step=el2 * 1e3 / a2.steps, value=n2 * a2.steps / el2,
                                   unit="atom-steps/s", dtype=dt2, steps=a2.steps,
                                   roofline=None if roof2 is None else
-                                  {k: roof2[k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "avg_ms")})
+                                  {k: roof2.get(k) for k in ("kernel", "bound", "achieved", "peak", "unit", "frac",
+                                                             "avg_ms", "traffic", "executed", "executed_frac")})
             except Exception as ex:
                 others[wl] = {"error": repr(ex)}
             torch.cuda.synchronize()

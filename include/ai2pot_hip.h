@@ -429,6 +429,33 @@ int a2p_mtp_basis_bwd_f32(void* plan, int chebyshev_size, double scaling, const 
                           float* dcoeffs, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * EXTENSION without a counterpart in the reference -- NEP energy / force / virial with four- and five-body
+ * descriptors.  The reference's operators have radial and three-body descriptors only
+ * (source/descriptor/nep/bind/nep_bind.cc:81-105, include/nep_utilities.h:39-49); its unfinished draft
+ * source/descriptor/ace/include/nep_descriptor.h holds the weights C4B / C5B (:43-54) and declares
+ * accum_4b_descriptor_one / accum_5b_descriptor_one (:109-111) without defining them.  PARITY UNPINNED: there is
+ * no reference result to compare with; the entry points are checked by rotation invariance, finite differences of
+ * the energy and the reduction to a2p_nep_efv_* when both terms are off.
+ * Arguments as a2p_nep_efv_*, plus l_4body (0 or 2: one invariant per angular channel, cubic in its l = 2 moments)
+ * and l_5body (0 or 1: one invariant, quartic in its l = 1 moments).  Descriptors of a channel are ordered
+ * l = 1 .. l_max, four-body, five-body: D = n_radial + n_angular * (l_max + [l_4body > 0] + [l_5body > 0]), which
+ * is the row length of w0 and q_scaler and of desc.
+ * ------------------------------------------------------------------------------------------ */
+int a2p_nep_efv_manybody_f32(int chebyshev_size, int n_radial, int n_angular, int l_max, int l_4body, int l_5body,
+                             int num_neurons, int ntypes, const float* coeffs, const float* w0, const float* b0,
+                             const float* w1, const float* type_bias, const float* q_scaler, double rmax_radial,
+                             double rmax_angular, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                             const int* bilist, const int* bnumneigh, const int* bfirstneigh, const float* brcs,
+                             const int* btypes, float* etot, float* force, float* virial, float* desc, void* stream);
+int a2p_nep_efv_manybody_f64(int chebyshev_size, int n_radial, int n_angular, int l_max, int l_4body, int l_5body,
+                             int num_neurons, int ntypes, const double* coeffs, const double* w0, const double* b0,
+                             const double* w1, const double* type_bias, const double* q_scaler, double rmax_radial,
+                             double rmax_angular, int batch, int natoms_pad, int umax, int nghost, const int* binum,
+                             const int* bilist, const int* bnumneigh, const int* bfirstneigh, const double* brcs,
+                             const int* btypes, double* etot, double* force, double* virial, double* desc,
+                             void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * ZBL short-range correction -- the part of every E/F/V operator that its zbl_rmax > 0 argument
  * switches on (source/descriptor/correction/include/zbl.h:262-395 pair formulas;
  *  correction/gpu/include/zbl.cuh:422-620 composition per centre atom;

@@ -137,14 +137,25 @@ def _nep_efv(lib, prefix, model, nb, dtype):
     e = np.zeros(B, dt)
     f = np.zeros((B, P + nghost, 3), dt)
     v = np.zeros((B, 9), dt)
-    fn = getattr(lib, "%s_efv_%s" % (prefix, suffix))
+    mb = _many_body(model)
+    fn = getattr(lib, "%s_efv_%s%s" % (prefix, "mb_" if mb else "", suffix))
     fn.restype = None
     fn(_p(e), _p(f), _p(v), _I(model["chebyshev_size"]), _I(model["n_radial_basis"]),
        _I(model["n_angular_basis"]), _I(model["l_max"]), _I(H), _p(coeffs), _p(w0), _p(b0), _p(w1),
        _p(bias), _I(B), _I(P), _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs),
        _p(btypes), _I(ntypes), _p(type_map), _I(U), _I(nghost), _D(model["rmax_radial"]),
-       _D(model["rmax_angular"]), _p(q_scaler))
+       _D(model["rmax_angular"]), _p(q_scaler), *mb)
     return e, f, v
+
+
+def _many_body(model):
+    """() for the reference's model; (_I(mb4), _I(mb5)) for the extension with a four-body (l_4body = 2) and / or a
+    five-body (l_5body = 1) invariant per angular channel (restatement only: the reference has no such terms)."""
+    l4, l5 = int(model.get("l_4body", 0)), int(model.get("l_5body", 0))
+    if not (l4 or l5):
+        return ()
+    assert l4 in (0, 2) and l5 in (0, 1) and model["l_max"] >= max(l4, l5)
+    return (_I(1 if l4 else 0), _I(1 if l5 else 0))
 
 
 def _nep_desc(lib, prefix, model, nb, dtype):
@@ -155,13 +166,14 @@ def _nep_desc(lib, prefix, model, nb, dtype):
     coeffs = _c(model["coeffs"], dt)
     type_map = _c(model["type_map"], np.int32)
     n_r, n_a, l_max = model["n_radial_basis"], model["n_angular_basis"], model["l_max"]
-    D = n_r + n_a * l_max
+    mb = _many_body(model)
+    D = n_r + n_a * (l_max + sum(x.value for x in mb))
     d = np.zeros((B, P, D), dt)
-    fn = getattr(lib, "%s_desc_%s" % (prefix, suffix))
+    fn = getattr(lib, "%s_desc_%s%s" % (prefix, "mb_" if mb else "", suffix))
     fn.restype = None
     fn(_p(d), _I(model["chebyshev_size"]), _I(n_r), _I(n_a), _I(l_max), _p(coeffs), _I(B), _I(P),
        _p(binum), _p(bilist), _p(bnumneigh), _p(bfirst), _p(brcs), _p(btypes), _I(type_map.size),
-       _p(type_map), _I(U), _I(nghost), _D(model["rmax_radial"]), _D(model["rmax_angular"]))
+       _p(type_map), _I(U), _I(nghost), _D(model["rmax_radial"]), _D(model["rmax_angular"]), *mb)
     return d
 
 

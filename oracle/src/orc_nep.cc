@@ -27,6 +27,15 @@ const double C3B[24] = {
     0.223811638722978, 0.223811638722978f, 0.111905819361489f, 0.111905819361489f,
     1.566681471060845, 1.566681471060845f, 0.195835183882606f, 0.195835183882606f};
 
+// Four- and five-body weights: the constants of the reference's unfinished draft
+// (source/descriptor/ace/include/nep_descriptor.h:43-54; its accum_4b_descriptor_one / accum_5b_descriptor_one are
+// declared at :109-111 and never defined).  The invariants they weight are restated below from the published NEP
+// formulation; PARITY UNPINNED: no reference code evaluates them.  Pinned instead by rotation invariance,
+// finite differences and the reduction to the three-body model (tests/test_oracle_nep_manybody.py).
+const double C4B[5] = {-0.007499480826664, -0.134990654879954, 0.067495327439977, 0.404971964639861,
+                       -0.809943929279723};
+const double C5B[3] = {0.026596810706114, 0.053193621412227, 0.026596810706114};
+
 // Un-normalised real solid harmonics b_lm (nep_utilities.h:110-203) as polynomials
 // sum_t c_t x^a y^b z^c r^(2d), listed per flat index l*l-1+mp.
 struct Term { double c; int a, b, c_, d; };
@@ -121,9 +130,36 @@ struct Model {
     int K, n_r, n_a, l_max, H, ntypes;
     const double *coeffs, *w0, *b0, *w1, *bias, *q_scaler;
     double rr, ra;
-    int D() const { return l_max == 0 ? n_r : n_r + n_a * l_max; }
+    int mb4 = 0, mb5 = 0;       // extension: a four-body (l = 2) and a five-body (l = 1) invariant per angular channel
+    int num_l() const { return l_max + mb4 + mb5; }
+    int D() const { return l_max == 0 ? n_r : n_r + n_a * num_l(); }
     int nlm() const { return l_max * l_max + 2 * l_max; }
 };
+
+// q_4b(s) of the l = 2 moments s[3..7] and q_5b(s) of the l = 1 moments s[0..2] of one channel, with gradients
+inline double q4b_of(const double* s, double* d)
+{
+    const double s3 = s[3], s4 = s[4], s5 = s[5], s6 = s[6], s7 = s[7];
+    if (d) {
+        d[3] = 3 * C4B[0] * s3 * s3 + C4B[1] * (s4 * s4 + s5 * s5) + C4B[2] * (s6 * s6 + s7 * s7);
+        d[4] = 2 * C4B[1] * s3 * s4 - 2 * C4B[3] * s6 * s4 + C4B[4] * s5 * s7;
+        d[5] = 2 * C4B[1] * s3 * s5 + 2 * C4B[3] * s6 * s5 + C4B[4] * s4 * s7;
+        d[6] = 2 * C4B[2] * s3 * s6 + C4B[3] * (s5 * s5 - s4 * s4);
+        d[7] = 2 * C4B[2] * s3 * s7 + C4B[4] * s4 * s5;
+    }
+    return C4B[0] * s3 * s3 * s3 + C4B[1] * s3 * (s4 * s4 + s5 * s5) + C4B[2] * s3 * (s6 * s6 + s7 * s7) +
+           C4B[3] * s6 * (s5 * s5 - s4 * s4) + C4B[4] * s4 * s5 * s7;
+}
+inline double q5b_of(const double* s, double* d)
+{
+    const double a = s[0] * s[0], b = s[1] * s[1] + s[2] * s[2];
+    if (d) {
+        d[0] = 4 * C5B[0] * a * s[0] + 2 * C5B[1] * s[0] * b;
+        d[1] = 2 * C5B[1] * a * s[1] + 4 * C5B[2] * b * s[1];
+        d[2] = 2 * C5B[1] * a * s[2] + 4 * C5B[2] * b * s[2];
+    }
+    return C5B[0] * a * a + C5B[1] * a * b + C5B[2] * b * b;
+}
 
 // One centre atom: descriptors q[D], moments S[n_a*nlm] (nepBasis.h:57-196).
 void descriptors_of(const Model& m, int ti, int nn, const int* first, const double* rcs,
@@ -159,8 +195,12 @@ void descriptors_of(const Model& m, int ti, int nn, const int* first, const doub
         for (int l = 1; l <= m.l_max; l++)
             for (int mp = 0; mp < 2 * l + 1; mp++) {
                 double s = S[n * nlm + l * l - 1 + mp];
-                q[m.n_r + n * m.l_max + (l - 1)] += (mp == 0 ? 1 : 2) * C3B[l * l - 1 + mp] * s * s;
+                q[m.n_r + n * m.num_l() + (l - 1)] += (mp == 0 ? 1 : 2) * C3B[l * l - 1 + mp] * s * s;
             }
+    for (int n = 0; n < m.n_a && m.l_max > 0; n++) {
+        if (m.mb4) q[m.n_r + n * m.num_l() + m.l_max] = q4b_of(&S[n * nlm], nullptr);
+        if (m.mb5) q[m.n_r + n * m.num_l() + m.l_max + m.mb4] = q5b_of(&S[n * nlm], nullptr);
+    }
 }
 
 template <typename T>
@@ -194,9 +234,20 @@ void efv_one(const Model& m, double& etot, double* force, double* virial, int in
             for (int l = 1; l <= m.l_max; l++)
                 for (int mp = 0; mp < 2 * l + 1; mp++) {
                     int is = n * nlm + l * l - 1 + mp;
-                    dEdS[is] = dEdq[m.n_r + n * m.l_max + l - 1] * (mp == 0 ? 1 : 2) * 2 *
+                    dEdS[is] = dEdq[m.n_r + n * m.num_l() + l - 1] * (mp == 0 ? 1 : 2) * 2 *
                                C3B[l * l - 1 + mp] * S[is];
                 }
+        for (int n = 0; n < m.n_a && m.l_max > 0; n++) {
+            double d[8];
+            if (m.mb4) {
+                q4b_of(&S[n * nlm], d);
+                for (int k = 3; k < 8; k++) dEdS[n * nlm + k] += dEdq[m.n_r + n * m.num_l() + m.l_max] * d[k];
+            }
+            if (m.mb5) {
+                q5b_of(&S[n * nlm], d);
+                for (int k = 0; k < 3; k++) dEdS[n * nlm + k] += dEdq[m.n_r + n * m.num_l() + m.l_max + m.mb4] * d[k];
+            }
+        }
         // pair derivatives and scatter, nep.h:468-515
         for (int jj = 0; jj < nn; jj++) {
             const double* v = &rcs[jj * 3];
@@ -245,9 +296,10 @@ template <typename T>
 void efv(T* betot, T* bforce, T* bvirial, int K, int n_r, int n_a, int l_max, int H, const T* coeffs,
          const T* w0, const T* b0, const T* w1, const T* bias, int B, int P, const int* binum,
          const int* bilist, const int* bnumneigh, const int* bfirstneigh, const T* brcs,
-         const int* btypes, int ntypes, int U, int nghost, double rr, double ra, const T* q_scaler)
+         const int* btypes, int ntypes, int U, int nghost, double rr, double ra, const T* q_scaler, int mb4 = 0,
+         int mb5 = 0)
 {
-    const int D = l_max == 0 ? n_r : n_r + n_a * l_max;
+    const int D = l_max == 0 ? n_r : n_r + n_a * (l_max + mb4 + mb5);
     auto up = [](const T* p, size_t n) { return std::vector<double>(p, p + n); };
     std::vector<double> c = up(coeffs, (size_t)ntypes * ntypes * (n_r + n_a) * K),
                         W0 = up(w0, (size_t)ntypes * H * D), B0 = up(b0, (size_t)ntypes * H),
@@ -255,6 +307,7 @@ void efv(T* betot, T* bforce, T* bvirial, int K, int n_r, int n_a, int l_max, in
     // cutoffs are rounded to T first, as the reference's launcher receives them in T
     Model m{K, n_r, n_a, l_max, H, ntypes, c.data(), W0.data(), B0.data(), W1.data(), bi.data(),
             qs.data(), (double)(T)rr, (double)(T)ra};
+    m.mb4 = mb4; m.mb5 = mb5;
     for (int b = 0; b < B; b++) {
         double e = 0, v[9] = {0};
         std::vector<double> f((size_t)(P + nghost) * 3, 0.0);
@@ -270,12 +323,13 @@ void efv(T* betot, T* bforce, T* bvirial, int K, int n_r, int n_a, int l_max, in
 template <typename T>
 void desc(T* bdesc, int K, int n_r, int n_a, int l_max, const T* coeffs, int B, int P,
           const int* binum, const int* bilist, const int* bnumneigh, const int* bfirstneigh,
-          const T* brcs, const int* btypes, int ntypes, int U, double rr, double ra)
+          const T* brcs, const int* btypes, int ntypes, int U, double rr, double ra, int mb4 = 0, int mb5 = 0)
 {
-    const int D = l_max == 0 ? n_r : n_r + n_a * l_max;
+    const int D = l_max == 0 ? n_r : n_r + n_a * (l_max + mb4 + mb5);
     std::vector<double> c(coeffs, coeffs + (size_t)ntypes * ntypes * (n_r + n_a) * K);
     Model m{K, n_r, n_a, l_max, 0, ntypes, c.data(), nullptr, nullptr, nullptr, nullptr, nullptr,
             (double)(T)rr, (double)(T)ra};
+    m.mb4 = mb4; m.mb5 = mb5;
     std::vector<double> q(D), S(n_a * m.nlm() + 1), rcs((size_t)U * 3);
     for (int b = 0; b < B; b++)
         for (int ii = 0; ii < binum[b]; ii++) {
@@ -314,4 +368,9 @@ void orc_nep_efv_f32(ARGS_EFV(float)) { efv<float>(PASS_EFV); }
 void orc_nep_efv_f64(ARGS_EFV(double)) { efv<double>(PASS_EFV); }
 void orc_nep_desc_f32(ARGS_DESC(float)) { desc<float>(PASS_DESC); }
 void orc_nep_desc_f64(ARGS_DESC(double)) { desc<double>(PASS_DESC); }
+// the extension with four- and five-body invariants (mb4, mb5 = 0 or 1); parity unpinned, see C4B above
+void orc_nep_efv_mb_f32(ARGS_EFV(float), int mb4, int mb5) { efv<float>(PASS_EFV, mb4, mb5); }
+void orc_nep_efv_mb_f64(ARGS_EFV(double), int mb4, int mb5) { efv<double>(PASS_EFV, mb4, mb5); }
+void orc_nep_desc_mb_f32(ARGS_DESC(float), int mb4, int mb5) { desc<float>(PASS_DESC, mb4, mb5); }
+void orc_nep_desc_mb_f64(ARGS_DESC(double), int mb4, int mb5) { desc<double>(PASS_DESC, mb4, mb5); }
 }
