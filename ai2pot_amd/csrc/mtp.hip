@@ -99,6 +99,8 @@ struct MtpArgs {
     T* desc;           // [B, P, n_scalar] scalar moments, or null
     int energy_only;   // stop after the energy: no adjoint, no pair derivatives
     int cE_per_atom;   // loss-gradient mode: cE is indexed per row (weights of the site energies)
+    int no_tangent;    // loss-gradient mode: the force and virial residuals are zero (site-energy and basis backward),
+                       // so the tangents and mixed adjoints vanish: their sweeps and terms are left out
     // neural-network read-out (source/descriptor/nnmtp/include/nnMtp.h:470-507) when H > 0:
     // e_i = bias + sum_p w1[t,p] tanh(sum_k w0[t,p,k] (M_k - q_shift[k]) / q_scaler[k]); `lin` is unused
     int H;
@@ -379,6 +381,7 @@ template <typename T, bool LOSS, int NT, bool SEED = false>
 __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const MtpArgs<T> a)
 {
     const bool seeded = (SEED || LOSS) && a.row_seed != nullptr;
+    const bool no_tan = LOSS && a.no_tangent != 0;      // uniform over the launch
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const MtpPlanDevice& p = a.p;
     const int lane = threadIdx.x;     // thread in the workgroup
@@ -464,7 +467,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
                 const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
                 const T m = xa * yb * zc;
                 acc += g * m;
-                if (LOSS) {
+                if (LOSS && !no_tan) {
                     const T dg = t[ODG + mu], rinv = t[OU + 3], wu = t[OW + 3];
                     const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
                                  (T)eb * xa * t[OY + max(eb - 1, 0)] * zc * t[OW + 1] +
@@ -479,7 +482,8 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     }
 
     // ---- products, energy, adjoint ------------------------------------------------------------
-    sweep_forward<T, LOSS, NT>(p, M, Tg, lane);
+    if (LOSS && !no_tan) sweep_forward<T, LOSS, NT>(p, M, Tg, lane);
+    else sweep_forward<T, false, NT>(p, M, Tg, lane);
     for (int i = lane; i < n_moms; i += NT) {    // the table is dead: its place now holds the adjoints
         A[i] = (T)0;
         if (LOSS) Bm[i] = (T)0;
@@ -665,7 +669,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     if (LOSS) {
         const T cE = seeded ? (T)1 : (a.cE_per_atom ? a.cE[row] : a.cE[b]);
         // linearMtpLoss.h:417-434; the reference's network backward has no such term (Bm stays zero)
-        if (a.H == 0 || a.nn_exact) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, lane);
+        if (!no_tan && (a.H == 0 || a.nn_exact)) sweep_reverse<T, true, NT>(p, M, Bm, A, Tg, lane);
         // the last pass needs the adjoints of the basic moments while the table is back in its region
         for (int i = lane; i < n_basic; i += NT) { Ab[i] = A[i]; Bb[i] = Bm[i]; }
         T* grow = a.gpart + row * a.ngrad;
@@ -726,10 +730,14 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
                         const int ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
                         const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
                         const T m = xa * yb * zc;
+                        const T adj = Ab[i];
+                        if (no_tan) {                 // w = 0: only the energy term is left
+                            Pv += cE * adj * m;
+                            continue;
+                        }
                         const T gm = (T)ea * t[OX + max(ea - 1, 0)] * yb * zc * t[OW + 0] +
                                      (T)eb * xa * t[OY + max(eb - 1, 0)] * zc * t[OW + 1] +
                                      (T)ec * xa * yb * t[OZ + max(ec - 1, 0)] * t[OW + 2];
-                        const T adj = Ab[i];
                         Pv += (cE * adj + Bb[i]) * m + adj * rinv * (gm - (T)(ea + eb + ec) * m * wu);
                         Qv += adj * m * wu;
                     }
@@ -1187,7 +1195,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.brcs = brcs; a.btypes = btypes;
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
     a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.seg_cap = 0; a.partial = nullptr;
-    a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0;
+    a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0; a.no_tangent = 0;
     a.nn_exact = 1;
     a.row_seed = nullptr; a.pair_out = nullptr;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
@@ -1482,7 +1490,7 @@ int mtp_esites_bwd(void* handle, int K, double scaling, const T* coeffs, const T
     rc = fill_zero(ws, ((nzero * sizeof(T) + 3) / 4) * 4, stream);
     if (rc) return rc;
     a.E = table_entries<T>(a.p, K, true);
-    a.cE = gout; a.cE_per_atom = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = ngrad;
+    a.cE = gout; a.cE_per_atom = 1; a.no_tangent = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = ngrad;
     rc = launch_atoms<T, true>(a, stream);
     if (rc) return rc;
     prof_begin("mtp_grad_reduce", stream);
@@ -1538,7 +1546,7 @@ int mtp_basis_bwd(void* handle, int K, double scaling, const T* coeffs, int nmus
         if (rc) return rc;
         MtpArgs<T> g = a;
         g.E = table_entries<T>(g.p, K, true);
-        g.dFs = dFs; g.dVs = dVs; g.gpart = gpart; g.ngrad = ncoef;
+        g.dFs = dFs; g.dVs = dVs; g.gpart = gpart; g.ngrad = ncoef; g.no_tangent = 1;
         rc = launch_atoms<T, true>(g, stream);
         if (rc) return rc;
         prof_begin("mtp_grad_reduce", stream);
@@ -1650,7 +1658,7 @@ int nnmtp_esites_bwd(void* handle, int K, const MtpNet<T>& net, const T* coeffs,
     rc = fill_zero(ws, ((nzero * sizeof(T) + 3) / 4) * 4, stream);
     if (rc) return rc;
     a.E = table_entries<T>(a.p, K, true);
-    a.cE = gout; a.cE_per_atom = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = nrow;
+    a.cE = gout; a.cE_per_atom = 1; a.no_tangent = 1; a.dFs = dFs; a.dVs = dVs; a.gpart = gpart; a.ngrad = nrow;
     rc = launch_atoms<T, true>(a, stream);
     if (rc) return rc;
     prof_begin("mtp_grad_reduce", stream);

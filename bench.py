@@ -631,6 +631,41 @@ def run_nep_train(args):
     return natoms, elapsed, kernels, roof, config, "f32", {"rooflines": entries}
 
 
+def run_mtp_solver(args):
+    """The normal equations of the linear parameters (LinMatrixLinVectorOp) on configuration 4's structures, level
+    16: one energy / force / virial pass per scalar moment (92) plus three Gram products by the BLAS."""
+    import torch
+    from ai2pot_amd import _lib, ops, synth
+    dev = torch.device("cuda:0")
+    m, nb, tables = mtp_setup(4)
+    f64 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float64)).to(dev)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(dev)
+    md = {k: f64(m[k]) for k in ("coeffs", "linear_coeffs", "type_bias", "q_scaler")}
+    tb = {k: i32(m[k]) for k in ("alpha_index_basic", "alpha_index_times", "alpha_moment_mapping", "type_map")}
+    d = {k: i32(nb[k]) for k in ("binum", "bilist", "bnumneigh", "bfirstneigh", "btypes")}
+    d["brcs"] = f64(nb["brcs"])
+    B, P = nb["bilist"].shape
+    natoms = int(nb["binum"].sum())
+    lab = (f64(synth.rng_normal(4005, B * P, -4.0, 0.2).reshape(B, P).sum(1)),
+           f64(synth.rng_normal(4006, B * P * 3, 0.0, 1.0).reshape(B, P, 3)),
+           f64(synth.rng_normal(4007, B * 9, 0.0, 0.5).reshape(B, 9)))
+
+    def step(k):
+        ops.LinMatrixLinVectorOp(1.0, 1.0, 1.0, lab[0], lab[1], lab[2], m["chebyshev_size"], 1.0, md["coeffs"],
+                                 md["linear_coeffs"], md["type_bias"], m["alpha_moments_count"], tb["alpha_index_basic"],
+                                 tb["alpha_index_times"], tb["alpha_moment_mapping"], m["nmus"], d["binum"], d["bilist"],
+                                 d["bnumneigh"], d["bfirstneigh"], d["brcs"], d["btypes"], tb["type_map"], 0, m["rmax"],
+                                 m["rmin"], md["q_scaler"], 0.0, 0.0, None, None, validate=False)
+    L = _lib.lib()
+    elapsed, kernels = timed(step, args.steps, args.warmup, L)
+    _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
+    config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P,
+              "model": "linear MTP level 16 K=%d" % m["chebyshev_size"], "species": int(m["type_map"].size),
+              "per_step": "normal equations of the linear parameters: %d E/F/V passes + Gram products"
+                          % int(m["alpha_moment_mapping"].size)}
+    return natoms, elapsed, kernels, None, config, "f64", {}
+
+
 def cpu_baseline_mtp(cfg):
     import oracle
     from ai2pot_amd import synth
@@ -686,6 +721,7 @@ WORKLOADS = {
     "mtp20_efv_8192": lambda a: run_mtp(a, 3),                    # configs[2]
     "mtp16_train_64x128": lambda a: run_mtp(a, 4),                # configs[3]
     "nep_train_64x128": run_nep_train,                            # NEP counterpart of configs[3] (not one of the benchmark configurations)
+    "mtp16_solver_64x128": run_mtp_solver,                        # linear-solver operator on configs[3]'s structures (extra)
     "hbm_copy_probe": None,                                       # counter calibration, not a workload of the path
 }
 
@@ -729,9 +765,10 @@ def main():
         import copy
         import torch
         others = {}
-        for wl in ("mtp10_efv_216", "nep_efv_4096", "mtp20_efv_8192", "mtp16_train_64x128", "nep_train_64x128"):
+        for wl in ("mtp10_efv_216", "nep_efv_4096", "mtp20_efv_8192", "mtp16_train_64x128", "nep_train_64x128",
+                   "mtp16_solver_64x128"):
             a2 = copy.copy(args)
-            a2.workload, a2.steps, a2.warmup = wl, 50, 5
+            a2.workload, a2.steps, a2.warmup = wl, (5 if "solver" in wl else 50), (1 if "solver" in wl else 5)
             try:
                 n2, el2, k2, roof2, _, dt2, _ = WORKLOADS[wl](a2)
                 others[wl] = dict(natoms=n2, ms_per_step=el2 * 1e3 / a2.steps, value=n2 * a2.steps / el2,
@@ -745,7 +782,7 @@ def main():
         out["other_configs"] = others
     if not args.no_cpu_baseline:
         try:
-            if args.workload == "nep_train_64x128":
+            if args.workload in ("nep_train_64x128", "mtp16_solver_64x128"):
                 out["cpu_baseline"] = {"note": "no CPU baseline leg for this extra workload"}
             elif args.workload.startswith("nep"):
                 out["cpu_baseline"] = cpu_baseline_nep()
