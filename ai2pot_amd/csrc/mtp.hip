@@ -225,6 +225,14 @@ __device__ __forceinline__ T piece_sum(T v, int rem, int steps)
     return v;
 }
 
+// A plan term names its two moments by byte offsets into an array of doubles (index * 8): no shift between the
+// word and the LDS address in fp64.
+template <typename T>
+__device__ __forceinline__ T plan_entry(const T* base, unsigned off)
+{
+    return *(const T*)((const char*)base + (sizeof(T) == 8 ? off : off >> 1));
+}
+
 // forward products: M[dst] = sum mult M[m0] M[m1]; with TANGENT also the product rule on Tg.
 template <typename T, bool TANGENT, int NT>
 __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* Tg, int tid)
@@ -252,11 +260,11 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
                 if (k < depth) {
 #pragma unroll
                     for (int u = k; u < k + 4; u++) {
-                        const int m0 = w[u].x & 0xffff, m1 = (int)((unsigned)w[u].x >> 16);
+                        const unsigned m0 = (unsigned)w[u].x & 0xffffu, m1 = (unsigned)w[u].x >> 16;
                         const T mult = (T)w[u].y;
-                        const T v0 = M[m0], v1 = M[m1];
+                        const T v0 = plan_entry(M, m0), v1 = plan_entry(M, m1);
                         acc += mult * v0 * v1;
-                        if (TANGENT) tacc += Tg[m0] * mult * v1 + Tg[m1] * mult * v0;
+                        if (TANGENT) tacc += plan_entry(Tg, m0) * mult * v1 + plan_entry(Tg, m1) * mult * v0;
                     }
                 }
             if (steps) {
@@ -298,10 +306,10 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
                 if (k < depth) {
 #pragma unroll
                     for (int u = k; u < k + 4; u++) {
-                        const int dst = w[u].x & 0xffff, other = (int)((unsigned)w[u].x >> 16);
+                        const unsigned dst = (unsigned)w[u].x & 0xffffu, other = (unsigned)w[u].x >> 16;
                         const T mult = (T)w[u].y;
-                        acc += X[dst] * mult * M[other];
-                        if (MIXED) acc += mult * A[dst] * Tg[other];
+                        acc += plan_entry(X, dst) * mult * plan_entry(M, other);
+                        if (MIXED) acc += mult * plan_entry(A, dst) * plan_entry(Tg, other);
                     }
                 }
             if (steps) acc = piece_sum(acc, rem, steps);
@@ -955,7 +963,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
         A2P_REQUIRE(!seen[mapping[s]], A2P_ERR_INVALID, "mtp plan: alpha_moment_mapping repeats a moment");
         seen[mapping[s]] = 1;
     }
-    A2P_REQUIRE(n_moms < 65536, A2P_ERR_INVALID, "mtp plan: more than 65535 moments");
+    A2P_REQUIRE(n_moms < 8192, A2P_ERR_INVALID, "mtp plan: more than 8191 moments");    // 16-bit byte offsets
     // Interleaved gather lists (see mtp_plan.h).  `lists[m]` holds the packed terms of moment m.
     struct Ell {
         std::vector<int> level, lend, multi, slot, lead, gbase, gdepth;   // multi: doubling steps; lead: pieces behind
@@ -1021,7 +1029,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     std::vector<std::vector<int2>> fl(n_moms), rl(n_moms);
     for (int e = 0; e < n_times; e++) {
         const int* q = times + e * 4;
-        fl[q[3]].push_back(make_int2(q[0] | (q[1] << 16), q[2]));
+        fl[q[3]].push_back(make_int2((q[0] * 8) | ((q[1] * 8) << 16), q[2]));
     }
     std::vector<std::vector<int>> f_by(n_levels), r_by(n_levels);
     for (int m = n_basic; m < n_moms; m++)
@@ -1029,8 +1037,8 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     // reverse: terms per source in reverse file order
     for (int e = n_times - 1; e >= 0; e--) {
         const int* q = times + e * 4;
-        rl[q[1]].push_back(make_int2(q[3] | (q[0] << 16), q[2]));     // adj[m1] += adj[dst] mult M[m0]
-        rl[q[0]].push_back(make_int2(q[3] | (q[1] << 16), q[2]));     // adj[m0] += adj[dst] mult M[m1]
+        rl[q[1]].push_back(make_int2((q[3] * 8) | ((q[0] * 8) << 16), q[2]));     // adj[m1] += adj[dst] mult M[m0]
+        rl[q[0]].push_back(make_int2((q[3] * 8) | ((q[1] * 8) << 16), q[2]));     // adj[m0] += adj[dst] mult M[m1]
     }
     for (int m = 0; m < n_moms; m++)
         if (level[m] < n_levels && !rl[m].empty()) r_by[level[m]].push_back(m);

@@ -35,8 +35,8 @@ struct MtpPlanDevice {
     // [f_level[l], f_level[l+1]) (whole groups; [f_level[l], f_lend[l]) without the padding slots).  The terms of a group are stored
     // interleaved and padded with zero terms to the group's depth (a multiple of four): term k of slot s is
     // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
-    // a group read consecutive words and share the trip count.  A term packs x = m0 | m1 << 16,
-    // y = multiplicity.
+    // a group read consecutive words and share the trip count.  A term packs x = 8 m0 | 8 m1 << 16 (byte offsets
+    // into an array of doubles), y = multiplicity.
     const int* f_level;        // [n_levels+1]
     const int* f_lend;         // [n_levels+1]
     const int* f_multi;        // [n_levels]   doubling steps that add up the longest list's pieces (0: no list is cut)
@@ -46,7 +46,7 @@ struct MtpPlanDevice {
     const int* f_gdepth;       // [n_fslots/64]
     const int2* f_terms;
     // reverse gather, same layout: sources by level (index l = level of the SOURCE moment),
-    // processed from the last level to level 0; a term packs x = dst | other << 16, y = mult
+    // processed from the last level to level 0; a term packs x = 8 dst | 8 other << 16, y = mult
     const int* r_level;        // [n_levels+1]
     const int* r_lend;         // [n_levels+1]
     const int* r_multi;        // [n_levels]
