@@ -342,6 +342,21 @@ struct BasisFunction : public torch::autograd::Function<BasisFunction> {
     }
 };
 
+// X^T X [n, n] and X^T y [n] of a tall matrix X [N, n]: the rows are cut into up to 64 blocks whose products run
+// as one batched GEMM and are added afterwards (a single GEMM with n of about a hundred and N in the tens of
+// thousands occupies one tile of the chip: 0.66 ms against 0.03 ms for 24576 x 95 in fp64)
+std::pair<at::Tensor, at::Tensor> gram(const at::Tensor& X, const at::Tensor& y)
+{
+    const int64_t N = X.size(0), n = X.size(1);
+    at::Tensor R = at::cat({X, y.reshape({N, 1})}, 1);
+    const int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(64, N / 256));
+    const int64_t k = N / chunks, head = k * chunks;
+    at::Tensor G = at::bmm(X.narrow(0, 0, head).reshape({chunks, k, n}).transpose(1, 2),
+                           R.narrow(0, 0, head).reshape({chunks, k, n + 1})).sum(0);
+    if (head < N) G = G + at::matmul(X.narrow(0, head, N - head).t(), R.narrow(0, head, N - head));
+    return {G.narrow(1, 0, n), G.select(1, n)};
+}
+
 // normal equations of the linear parameters (linear_mtp_gram_and_cross.h:446-575): components by the
 // library, Gram products by torch's BLAS
 variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at::Tensor& e_dft,
@@ -367,7 +382,8 @@ variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at
     TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
                 "label tensors must have shapes [B], [B, P, 3], [B, 9]");
     a2p_bind::DeviceGuard guard(brcs);
-    at::Tensor ec = at::zeros({B, n}, opt), fc = at::zeros({(int64_t)B * P * 3, n}, opt), vc = at::zeros({B * 9, n}, opt);
+    // (the library writes every element)
+    at::Tensor ec = at::empty({B, n}, opt), fc = at::empty({(int64_t)B * P * 3, n}, opt), vc = at::empty({B * 9, n}, opt);
     void* st = current_stream(brcs);
     auto call = [&]() -> int {
         int rc;
@@ -387,10 +403,10 @@ variable_list lin_matrix_lin_vector(double e_w, double f_w, double v_w, const at
         return rc;
     };
     run_checked(brcs, binum, bnumneigh, bfirstneigh, 0, call);
-    at::Tensor A = e_w * at::matmul(ec.t(), ec) + f_w * at::matmul(fc.t(), fc) + v_w * at::matmul(vc.t(), vc);
-    at::Tensor b = e_w * at::matmul(ec.t(), e_dft.reshape({B})) + f_w * at::matmul(fc.t(), f_dft.reshape({-1})) +
-                   v_w * at::matmul(vc.t(), v_dft.reshape({-1}));
-    return {A, b};
+    auto ge = gram(ec, e_dft.reshape({B})), gf = gram(fc, f_dft.reshape({-1})), gv = gram(vc, v_dft.reshape({-1}));
+    at::Tensor A = e_w * ge.first + f_w * gf.first + v_w * gv.first;
+    at::Tensor b = e_w * ge.second + f_w * gf.second + v_w * gv.second;
+    return {A.contiguous(), b.contiguous()};
 }
 
 variable_list schmidt_orth(int64_t ntypes, int64_t nmus, int64_t K, const at::Tensor& coeffs)

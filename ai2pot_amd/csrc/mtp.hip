@@ -25,9 +25,11 @@
 #include "loss_kernels.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <set>
+#include <string>
 
 namespace a2p {
 namespace {
@@ -872,7 +874,7 @@ lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, in
                            const int* __restrict__ btypes)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < S) eye[(size_t)i * S + i] = (T)1;
+    if (eye && i < S) eye[(size_t)i * S + i] = (T)1;
     if (i < B * ntypes) {
         const int b = i / ntypes, t = i - b * ntypes;
         int cnt = 0;
@@ -882,6 +884,281 @@ lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, in
         }
         ecomp[(size_t)b * (S + ntypes) + S + t] = (T)cnt;
     }
+}
+
+// ---- linear-solver components, all scalar moments in one pass ------------------------------------------------
+// Column s of the components is the E/F/V of the read-out e_s / q_scaler[s].  Its adjoint is non-zero on the
+// ancestors of scalar moment s only (15 of 350 moments on average at level 16, 25 of 1352 at level 20), so the adjoints
+// of all columns together are one reverse gather over the nodes (scalar moment, ancestor) of the plan, about as
+// long as one ordinary reverse sweep, and a pair derivative sums over the basic ancestors of its column only.
+// The kernel computes the moments once per atom, runs that gather, and writes the pair derivatives of every column
+// to pb[pair][3][slots]; the kernels below add them up per atom (own pairs minus the pairs that name the atom, the
+// latter in the fixed order of a sorted list) and per structure.
+template <typename T>
+struct CompArgs {
+    T* pb;                  // [pairs, 3, x_slots]
+    const int* pair_off;    // [rows + 1] first pair of each row
+    const int* nnc;         // [rows] checked neighbour count of each row (0 for rows that are not evaluated)
+    T* desc;                // [rows, n_scalar] scalar moments
+    T* rowpart;             // [rows, 12, x_slots] per row and column: sum of the pair derivatives (3), virial (9)
+    int nc_cap, lds_basic_off;
+};
+
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, const CompArgs<T> c)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const MtpPlanDevice& p = a.p;
+    const int lane = threadIdx.x;
+    const int ii = blockIdx.x, b = blockIdx.y;
+    const int NF = a.P;
+    const size_t row = (size_t)b * a.P + ii;
+    const int n_moms = p.n_moms, n_basic = p.n_basic, nmus = p.nmus, kmax = p.kmax, K = a.K, E = a.E;
+    const int OX = 0, OY = kmax + 1, OZ = 2 * (kmax + 1), OG = 3 * (kmax + 1), ODG = OG + nmus, OU = ODG + nmus;
+    const int S = p.n_scalar;
+    // moments | node adjoints (+ the zero entry) | coefficients | neighbour table
+    T* M = (T*)smem_raw;
+    T* X = M + n_moms;
+    T* cf = X + ((p.x_nodes + 2) & ~1);
+    T* tab = cf + a.ntypes * nmus * K;
+    unsigned* bas = (unsigned*)(smem_raw + c.lds_basic_off);
+    const int nn = c.nnc[row];
+    if (ii >= a.binum[b] || nn == 0) {                       // padded or refused row (k_rows flags the reasons)
+        for (int s = lane; s < S; s += NT) c.desc[row * S + s] = (T)0;
+        for (int q = lane; q < 12 * p.x_slots; q += NT) c.rowpart[row * 12 * p.x_slots + q] = (T)0;
+        return;
+    }
+    int center = a.bilist[row];
+    if ((unsigned)center >= (unsigned)NF) center = 0;
+    const int* types = a.btypes + (size_t)b * NF;
+    int ti = types[center];
+    if ((unsigned)ti >= (unsigned)a.ntypes) ti = 0;
+    const int* first = a.bfirstneigh + row * a.U;
+    const T* rcs = a.brcs + row * a.U * 3;
+    for (int i = lane; i < n_basic; i += NT)
+        bas[i] = (unsigned)p.basic[i * 4] | ((unsigned)p.basic[i * 4 + 1] << 8) |
+                 ((unsigned)p.basic[i * 4 + 2] << 16) | ((unsigned)p.basic[i * 4 + 3] << 24);
+    for (int q = lane; q < a.ntypes * nmus * K; q += NT) cf[q] = a.coeffs[(size_t)ti * a.ntypes * nmus * K + q];
+    for (int i = lane; i < n_moms; i += NT) M[i] = (T)0;
+    for (int i = lane; i <= p.x_nodes; i += NT) X[i] = (T)0;
+    __syncthreads();
+
+    // basic moments (as in mtp_atom_kernel)
+    const int MTP_NC = c.nc_cap;
+    const int nchunks = (nn + MTP_NC - 1) / MTP_NC;
+    const int chunk = nchunks > 0 ? (nn + nchunks - 1) / nchunks : 1;
+    for (int c0 = 0; c0 < nn; c0 += chunk) {
+        const int nc = min(chunk, nn - c0);
+        int nj; bool valid; T d[3];
+        build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
+        __syncthreads();
+        for (int i = lane; i < n_basic; i += NT) {
+            const unsigned bw = bas[i];
+            const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
+            T acc = (T)0;
+            for (int j = 0; j < nc; j++) {
+                const T* t = tab + j * E;
+                acc += t[OG + mu] * (t[OX + ea] * t[OY + eb] * t[OZ + ec]);
+            }
+            M[i] += acc;
+        }
+        __syncthreads();
+    }
+    sweep_forward<T, false, NT>(p, M, (T*)nullptr, lane);
+    for (int s = lane; s < S; s += NT) {
+        c.desc[row * S + s] = M[p.mapping[s]];
+        X[p.x_root[s]] = (T)1 / a.q_scaler[s];
+    }
+    __syncthreads();
+    {
+        MtpPlanDevice px = p;              // the reverse gather over the nodes
+        px.r_level = p.x_level; px.r_multi = p.x_multi; px.r_src = p.x_src; px.r_rem = p.x_rem;
+        px.r_gbase = p.x_gbase; px.r_gdepth = p.x_gdepth; px.r_terms = p.x_terms;
+        sweep_reverse<T, false, NT>(px, M, X, (const T*)nullptr, (const T*)nullptr, lane);
+    }
+
+    // Pair derivatives.  A wavefront takes a neighbour j: its lanes first form, for every basic moment, the vector
+    //   D_b = d(g_mu x^a y^b z^c)/dr_j = m (g' - k g / r) u + g / r grad_u m
+    // from the neighbour's table row into the wavefront's own LDS buffer; then a lane owns a column and sums
+    // adj * D_b over the column's basic ancestors (three reads and three FMAs per ancestor).  The own-row sums of the
+    // columns (force of the centre, virial) are kept per lane and added over the wavefronts at the end.
+    const int ngroups = p.x_slots >> 6;
+    const int l64 = lane & 63, wv = lane >> 6;
+    T* D = tab + (size_t)c.nc_cap * E + (size_t)wv * n_basic * 3;
+    for (int c0 = 0; c0 < nn; c0 += chunk) {
+        const int nc = min(chunk, nn - c0);
+        if (nchunks > 1) {                                  // (a single chunk's table is still in place)
+            int nj; bool valid; T d[3];
+            __syncthreads();
+            build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
+            __syncthreads();
+        }
+        for (int j = wv; j < nc; j += NT / 64) {
+            const T* t = tab + j * E;
+            const T ux = t[OU + 0], uy = t[OU + 1], uz = t[OU + 2], rinv = t[OU + 3];
+            __builtin_amdgcn_wave_barrier();               // the last neighbour's sums have read D
+            for (int i = l64; i < n_basic; i += 64) {
+                const unsigned bw = bas[i];
+                const int mu = bw & 255, ea = (bw >> 8) & 255, eb = (bw >> 16) & 255, ec = bw >> 24;
+                const T gm = t[OG + mu], dg = t[ODG + mu];
+                const T xa = t[OX + ea], yb = t[OY + eb], zc = t[OZ + ec];
+                const T gs = xa * yb * zc * (dg - (T)(ea + eb + ec) * gm * rinv);
+                const T gr = gm * rinv;
+                D[i * 3 + 0] = gs * ux + gr * ((T)ea * t[OX + max(ea - 1, 0)] * yb * zc);
+                D[i * 3 + 1] = gs * uy + gr * ((T)eb * xa * t[OY + max(eb - 1, 0)] * zc);
+                D[i * 3 + 2] = gs * uz + gr * ((T)ec * xa * yb * t[OZ + max(ec - 1, 0)]);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            for (int g = 0; g < ngroups; g++) {
+                const int depth = p.x_bdepth[g];
+                const int* wp = p.x_bwords + p.x_bbase[g] + l64;
+                T gx = (T)0, gy = (T)0, gz = (T)0;
+                for (int k = 0; k < depth; k++) {
+                    const unsigned w = (unsigned)wp[k * 64];
+                    const T adj = X[w & 0xffffu];
+                    const T* dv = D + (w >> 16) * 3;
+                    gx += adj * dv[0]; gy += adj * dv[1]; gz += adj * dv[2];
+                }
+                T* dst = c.pb + ((size_t)(c.pair_off[row] + c0 + j) * 3) * p.x_slots + g * 64 + l64;
+                dst[0] = gx;
+                dst[(size_t)p.x_slots] = gy;
+                dst[2 * (size_t)p.x_slots] = gz;
+            }
+        }
+    }
+    // own-row sums of every column (force of the centre, virial), in neighbour order, from the pair derivatives this
+    // workgroup has just written: rowpart[row][12][slots]
+    __syncthreads();
+    for (int q = lane; q < p.x_slots; q += NT) {
+        T f[3] = {(T)0, (T)0, (T)0}, v[9];
+#pragma unroll
+        for (int i = 0; i < 9; i++) v[i] = (T)0;
+        const T* g = c.pb + (size_t)c.pair_off[row] * 3 * p.x_slots + q;
+        for (int j = 0; j < nn; j++) {
+            const T gx = g[0], gy = g[p.x_slots], gz = g[2 * (size_t)p.x_slots];
+            const T dx = rcs[j * 3], dy = rcs[j * 3 + 1], dz = rcs[j * 3 + 2];
+            f[0] += gx; f[1] += gy; f[2] += gz;
+            v[0] -= gx * dx; v[1] -= gx * dy; v[2] -= gx * dz;
+            v[3] -= gy * dx; v[4] -= gy * dy; v[5] -= gy * dz;
+            v[6] -= gz * dx; v[7] -= gz * dy; v[8] -= gz * dz;
+            g += 3 * (size_t)p.x_slots;
+        }
+        T* o = c.rowpart + row * 12 * p.x_slots + q;
+#pragma unroll
+        for (int i = 0; i < 3; i++) o[(size_t)i * p.x_slots] = f[i];
+#pragma unroll
+        for (int i = 0; i < 9; i++) o[(size_t)(3 + i) * p.x_slots] = v[i];
+    }
+}
+
+// rows that the components kernel evaluates, with the checks of mtp_atom_kernel; row_of1[b, atom] = 1 + the row whose
+// centre the atom is
+__global__ void __launch_bounds__(256)
+comp_rows_kernel(int B, int P, int U, int ntypes, const int* __restrict__ binum, const int* __restrict__ bilist,
+                 const int* __restrict__ bnumneigh, const int* __restrict__ btypes, int* __restrict__ nnc,
+                 int* __restrict__ row_of1, int* __restrict__ status)
+{
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row > B * P) return;
+    if (row == B * P) { nnc[row] = 0; return; }
+    const int b = row / P, ii = row - b * P;
+    int nn = 0;
+    if (ii < binum[b]) {
+        nn = bnumneigh[row];
+        if (nn > U) { atomicOr(status, ST_NEIGH_OVERFLOW); nn = U; }
+        if (nn < 0) nn = 0;
+        const int center = bilist[row];
+        if ((unsigned)center >= (unsigned)P) { atomicOr(status, ST_BAD_NEIGHBOR); nn = 0; }
+        else {
+            if ((unsigned)btypes[(size_t)b * P + center] >= (unsigned)ntypes) { atomicOr(status, ST_BAD_TYPE); nn = 0; }
+            row_of1[(size_t)b * P + center] = row + 1;
+        }
+    }
+    nnc[row] = nn;
+}
+
+// the pairs that name each atom: counted, then listed (comp_incoming_fill), then put in order (comp_incoming_sort)
+__global__ void __launch_bounds__(256)
+comp_incoming_kernel(int B, int P, int U, const int* __restrict__ nnc, const int* __restrict__ pair_off,
+                     const int* __restrict__ bfirstneigh, int* __restrict__ cnt, const int* __restrict__ ioff,
+                     int* __restrict__ inc)
+{
+    const long long q = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= (long long)B * P * U) return;
+    const int row = (int)(q / U), j = (int)(q - (long long)row * U);
+    if (j >= nnc[row]) return;
+    const int nj = bfirstneigh[q];
+    if ((unsigned)nj >= (unsigned)P) return;             // flagged by the components kernel's table
+    const int tg = (row / P) * P + nj;
+    const int place = atomicAdd(cnt + tg, 1);
+    if (inc) inc[ioff[tg] + place] = pair_off[row] + j;
+}
+
+__global__ void __launch_bounds__(256)
+comp_incoming_sort_kernel(int n, const int* __restrict__ ioff, int* __restrict__ inc)
+{
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    int* v = inc + ioff[t];
+    const int m = ioff[t + 1] - ioff[t];
+    for (int i = 1; i < m; i++) {
+        const int x = v[i];
+        int k = i - 1;
+        while (k >= 0 && v[k] > x) { v[k + 1] = v[k]; k--; }
+        v[k + 1] = x;
+    }
+}
+
+// force column of every atom: its own row's sum minus the pairs that name it, in the order of the sorted list
+template <typename T>
+__global__ void __launch_bounds__(64)
+comp_force_kernel(int slots, int n, const int* __restrict__ seed, const int* __restrict__ row_of1,
+                  const int* __restrict__ ioff, const int* __restrict__ inc, const T* __restrict__ pb,
+                  const T* __restrict__ rowpart, T* __restrict__ fcomp)
+{
+    const int t = blockIdx.x, q = blockIdx.y * 64 + threadIdx.x;
+    const int s = seed[q];
+    T f[3] = {(T)0, (T)0, (T)0};
+    const int r1 = row_of1[t];
+    if (r1 > 0) {
+        const T* o = rowpart + (size_t)(r1 - 1) * 12 * slots + q;
+#pragma unroll
+        for (int i = 0; i < 3; i++) f[i] = o[(size_t)i * slots];
+    }
+    for (int k = ioff[t]; k < ioff[t + 1]; k++) {
+        const T* g = pb + (size_t)inc[k] * 3 * slots + q;
+        f[0] -= g[0]; f[1] -= g[slots]; f[2] -= g[2 * (size_t)slots];
+    }
+    if (s < 0) return;
+#pragma unroll
+    for (int i = 0; i < 3; i++) fcomp[((size_t)t * 3 + i) * n + s] = f[i];
+}
+
+// energy and virial columns per structure: sums over the rows in row order
+template <typename T>
+__global__ void __launch_bounds__(64)
+comp_structure_kernel(int slots, int n, int S, int P, const int* __restrict__ seed, const int* __restrict__ binum,
+                      const T* __restrict__ q_scaler, const T* __restrict__ desc, const T* __restrict__ rowpart,
+                      T* __restrict__ ecomp, T* __restrict__ vcomp)
+{
+    const int b = blockIdx.x, q = blockIdx.y * 64 + threadIdx.x;
+    const int s = seed[q];
+    if (s < 0) return;
+    T e = (T)0, v[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) v[i] = (T)0;
+    for (int ii = 0; ii < binum[b]; ii++) {
+        const size_t row = (size_t)b * P + ii;
+        e += desc[row * S + s];
+        const T* o = rowpart + row * 12 * slots + q;
+#pragma unroll
+        for (int i = 0; i < 9; i++) v[i] += o[(size_t)(3 + i) * slots];
+    }
+    ecomp[(size_t)b * n + s] = e / q_scaler[s];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vcomp[((size_t)b * 9 + i) * n + s] = v[i];
 }
 
 // Gram-Schmidt over the nmus radial functions, each the vector of its ntypes^2 * K coefficients
@@ -1080,6 +1357,71 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     }
     dense_off[dense_lists.size()] = (int)dense_items.size();
 
+    // nodes (scalar moment, ancestor) and their reverse gather (mtp_plan.h)
+    std::vector<int> x_root(n_scalar, 0), x_seed, x_bbase, x_bdepth, x_bwords;
+    std::vector<std::vector<int2>> xl;
+    std::vector<std::vector<int>> x_by(n_levels);
+    std::vector<std::vector<int>> seed_basic(n_scalar);
+    int x_nodes = 0;
+    {
+        std::vector<std::vector<int>> terms_of(n_moms);
+        for (int e = 0; e < n_times; e++) terms_of[times[e * 4 + 3]].push_back(e);
+        std::vector<int> node_of(n_moms, -1), anc, stack;
+        for (int s = 0; s < n_scalar; s++) {
+            anc.clear();
+            stack.assign(1, mapping[s]);
+            while (!stack.empty()) {
+                const int m = stack.back();
+                stack.pop_back();
+                if (node_of[m] >= 0) continue;
+                node_of[m] = x_nodes++;
+                xl.emplace_back();
+                anc.push_back(m);
+                for (int e : terms_of[m]) { stack.push_back(times[e * 4]); stack.push_back(times[e * 4 + 1]); }
+            }
+            x_root[s] = node_of[mapping[s]];
+            for (int e = n_times - 1; e >= 0; e--) {          // reverse file order, as in the reverse gather above
+                const int* q = times + e * 4;
+                if (node_of[q[3]] < 0) continue;
+                const int nd = node_of[q[3]];
+                if (nd * 8 >= 65536) continue;                   // (too many nodes: refused below)
+                xl[node_of[q[1]]].push_back(make_int2((nd * 8) | ((q[0] * 8) << 16), q[2]));
+                xl[node_of[q[0]]].push_back(make_int2((nd * 8) | ((q[1] * 8) << 16), q[2]));
+            }
+            for (int m : anc) {
+                if (level[m] < n_levels && !xl[node_of[m]].empty()) x_by[level[m]].push_back(node_of[m]);
+                if (m < n_basic) seed_basic[s].push_back(node_of[m] | (m << 16));
+            }
+            for (int m : anc) node_of[m] = -1;
+        }
+    }
+    const bool x_ok = x_nodes < 8191 && n_basic < 32768;      // node x_nodes (a zero) must have a 16-bit byte offset too
+    if (!x_ok) { xl.assign(1, {}); for (auto& v : x_by) v.clear(); }
+    const Ell X = build_ell(xl, x_by);
+    A2P_REQUIRE(!X.too_long, A2P_ERR_INVALID, "mtp plan: a moment takes part in more than %d products", 64 * MTP_SLOT_CAP);
+    if (x_ok) {
+        std::vector<int> by_len(n_scalar);
+        for (int s = 0; s < n_scalar; s++) by_len[s] = s;
+        std::stable_sort(by_len.begin(), by_len.end(),
+                         [&](int x, int y) { return seed_basic[x].size() > seed_basic[y].size(); });
+        x_seed = by_len;
+        while (x_seed.size() % 64) x_seed.push_back(-1);
+        for (size_t g0 = 0; g0 < x_seed.size(); g0 += 64) {
+            size_t depth = 0;
+            for (size_t q = g0; q < g0 + 64; q++)
+                if (x_seed[q] >= 0) depth = std::max(depth, seed_basic[x_seed[q]].size());
+            x_bbase.push_back((int)x_bwords.size());
+            x_bdepth.push_back((int)depth);
+            x_bwords.resize(x_bwords.size() + depth * 64, x_nodes);       // node x_nodes, basic moment 0
+            for (size_t q = g0; q < g0 + 64; q++)
+                if (x_seed[q] >= 0)
+                    for (size_t k = 0; k < seed_basic[x_seed[q]].size(); k++)
+                        x_bwords[x_bbase.back() + k * 64 + (q - g0)] = seed_basic[x_seed[q]][k];
+        }
+    }
+    if (x_seed.empty()) { x_seed.push_back(-1); x_bbase.push_back(0); x_bdepth.push_back(0); }
+    if (x_bwords.empty()) x_bwords.push_back(0);
+
     // one device block
     struct Seg { const void* src; size_t bytes; size_t off; };
     std::vector<Seg> segs;
@@ -1114,6 +1456,18 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     const size_t o_doff = add(dense_off.data(), sizeof(int) * dense_off.size());
     const size_t o_dit = add(dense_items.data(), sizeof(int) * dense_items.size());
     const size_t o_dpos = add(dense_pos.data(), sizeof(int) * dense_pos.size());
+    const size_t o_xroot = add(x_root.data(), sizeof(int) * x_root.size());
+    const size_t o_xseed = add(x_seed.data(), sizeof(int) * x_seed.size());
+    const size_t o_xl = add(X.level.data(), sizeof(int) * X.level.size());
+    const size_t o_xx = add(X.multi.data(), sizeof(int) * X.multi.size());
+    const size_t o_xs = add(X.slot.data(), sizeof(int) * X.slot.size());
+    const size_t o_xc = add(X.lead.data(), sizeof(int) * X.lead.size());
+    const size_t o_xg = add(X.gbase.data(), sizeof(int) * X.gbase.size());
+    const size_t o_xh = add(X.gdepth.data(), sizeof(int) * X.gdepth.size());
+    const size_t o_xt = add(X.terms.data(), sizeof(int2) * X.terms.size());
+    const size_t o_xbb = add(x_bbase.data(), sizeof(int) * x_bbase.size());
+    const size_t o_xbd = add(x_bdepth.data(), sizeof(int) * x_bdepth.size());
+    const size_t o_xbw = add(x_bwords.data(), sizeof(int) * x_bwords.size());
     std::vector<unsigned char> host(total + 16, 0);
     for (auto& s : segs)
         if (s.bytes) std::memcpy(host.data() + s.off, s.src, s.bytes);
@@ -1142,6 +1496,15 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.rows = (const int*)(base + o_rows); d.dense_src = (const int*)(base + o_dsrc);
     d.dense_off = (const int*)(base + o_doff); d.dense_items = (const int*)(base + o_dit);
     d.dense_pos = (const int*)(base + o_dpos); d.dense_unique = dense_unique;
+    d.x_nodes = x_ok ? x_nodes : 0;
+    d.x_slots = x_ok ? (int)x_seed.size() : 0;
+    d.x_root = (const int*)(base + o_xroot); d.x_seed = (const int*)(base + o_xseed);
+    d.x_level = (const int*)(base + o_xl); d.x_multi = (const int*)(base + o_xx);
+    d.x_src = (const int*)(base + o_xs); d.x_rem = (const int*)(base + o_xc);
+    d.x_gbase = (const int*)(base + o_xg); d.x_gdepth = (const int*)(base + o_xh);
+    d.x_terms = (const int2*)(base + o_xt);
+    d.x_bbase = (const int*)(base + o_xbb); d.x_bdepth = (const int*)(base + o_xbd);
+    d.x_bwords = (const int*)(base + o_xbw);
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         g_plans.insert(plan);
@@ -1566,12 +1929,99 @@ int mtp_basis_bwd(void* handle, int K, double scaling, const T* coeffs, int nmus
     return A2P_OK;
 }
 
+// Which route a2p_mtp_lin_components_* takes: 1 = all columns in one pass over the atoms (when the plan has the node
+// graph and it fits in LDS), 0 = one E/F/V pass per column.  AI2POT_MTP_COMPONENTS=passes|nodes sets the initial value,
+// a2p_mtp_components_route changes it at run time.
+int g_components_route = -1;
+int components_route()
+{
+    if (g_components_route < 0) {
+        const char* e = getenv("AI2POT_MTP_COMPONENTS");
+        g_components_route = (e && std::string(e) == "passes") ? 0 : 1;
+    }
+    return g_components_route;
+}
+
+template <typename T>
+int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecomp, T* fcomp, T* vcomp, size_t lds,
+                             int lds_basic_off, int nc_cap, hipStream_t stream)
+{
+    const int B = a.B, P = a.P, U = a.U;
+    const int rows = B * P, slots = a.p.x_slots;
+    // integer scratch: nnc[rows+1] | pair_off[rows+1] | cnt[rows+1] | ioff[rows+1] | row_of1[rows] | scan tmp
+    const int ntmp = scan_tmp_ints(rows + 1);
+    void* wsI = nullptr;
+    int rc = ws_get(WS_CSR, ((size_t)(rows + 1) * 4 + rows + ntmp) * sizeof(int), &wsI);
+    if (rc) return rc;
+    int* nnc = (int*)wsI;
+    int* pair_off = nnc + rows + 1;
+    int* cnt = pair_off + rows + 1;
+    int* ioff = cnt + rows + 1;
+    int* row_of1 = ioff + rows + 1;
+    int* tmp = row_of1 + rows;
+    rc = fill_zero2(cnt, (size_t)(rows + 1) * sizeof(int), row_of1, (size_t)rows * sizeof(int), stream);
+    if (rc) return rc;
+    prof_begin("mtp_components_lists", stream);
+    hipLaunchKernelGGL(comp_rows_kernel, dim3(ceil_div(rows + 1, 256)), dim3(256), 0, stream, B, P, U, a.ntypes, a.binum,
+                       a.bilist, a.bnumneigh, a.btypes, nnc, row_of1, a.status);
+    prof_end(stream);
+    rc = exclusive_scan_i32(nnc, pair_off, rows + 1, tmp, stream);
+    if (rc) return rc;
+    int npairs = 0;                         // sizes the pair buffer: one read-back per call
+    A2P_HIP_CHECK(hipMemcpyAsync(&npairs, pair_off + rows, sizeof(int), hipMemcpyDeviceToHost, stream));
+    A2P_HIP_CHECK(hipStreamSynchronize(stream));
+    if (npairs < 0) npairs = 0;
+    // pair derivatives | row sums | scalar moments | list of the pairs that name each atom
+    const size_t n_pb = (size_t)std::max(npairs, 1) * 3 * slots, n_rp = (size_t)rows * 12 * slots, n_desc = (size_t)rows * S;
+    void* wsT = nullptr;
+    rc = ws_get(WS_MTP, (n_pb + n_rp + n_desc) * sizeof(T) + ((size_t)npairs + 1) * sizeof(int), &wsT);
+    if (rc) return rc;
+    T* pb = (T*)wsT;
+    T* rowpart = pb + n_pb;
+    T* desc = rowpart + n_rp;
+    int* inc = (int*)(desc + n_desc);
+    const long long nslots = (long long)rows * U;
+    prof_begin("mtp_components_lists", stream);
+    hipLaunchKernelGGL(comp_incoming_kernel, dim3(ceil_div(nslots, 256)), dim3(256), 0, stream, B, P, U, (const int*)nnc,
+                       (const int*)pair_off, a.bfirstneigh, cnt, (const int*)nullptr, (int*)nullptr);
+    prof_end(stream);
+    rc = exclusive_scan_i32(cnt, ioff, rows + 1, tmp, stream);
+    if (rc) return rc;
+    rc = fill_zero(cnt, (size_t)(rows + 1) * sizeof(int), stream);
+    if (rc) return rc;
+    prof_begin("mtp_components_lists", stream);
+    hipLaunchKernelGGL(comp_incoming_kernel, dim3(ceil_div(nslots, 256)), dim3(256), 0, stream, B, P, U, (const int*)nnc,
+                       (const int*)pair_off, a.bfirstneigh, cnt, (const int*)ioff, inc);
+    hipLaunchKernelGGL(comp_incoming_sort_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, stream, rows, (const int*)ioff,
+                       inc);
+    prof_end(stream);
+
+    CompArgs<T> c;
+    c.pb = pb; c.pair_off = pair_off; c.nnc = nnc; c.desc = desc; c.rowpart = rowpart; c.nc_cap = nc_cap;
+    c.lds_basic_off = lds_basic_off;
+    auto kern = mtp_components_kernel<T, 256>;
+    if (lds > 48 * 1024)
+        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    prof_begin("mtp_components_kernel", stream);
+    hipLaunchKernelGGL(kern, dim3(P, B), dim3(256), lds, stream, a, c);
+    prof_end(stream);
+    prof_begin("mtp_components_sums", stream);
+    hipLaunchKernelGGL(comp_force_kernel<T>, dim3(rows, slots / 64), dim3(64), 0, stream, slots, n, a.p.x_seed,
+                       (const int*)row_of1, (const int*)ioff, (const int*)inc, (const T*)pb, (const T*)rowpart, fcomp);
+    hipLaunchKernelGGL(comp_structure_kernel<T>, dim3(B, slots / 64), dim3(64), 0, stream, slots, n, S, P, a.p.x_seed,
+                       a.binum, a.q_scaler, (const T*)desc, (const T*)rowpart, ecomp, vcomp);
+    prof_end(stream);
+    A2P_HIP_CHECK(hipGetLastError());
+    (void)plan;
+    return A2P_OK;
+}
+
 // Energy, force and virial of every linear parameter taken alone (linear_mtp_gram_and_cross.h:125-374):
 // ecomp[B, n], fcomp[B, P, 3, n], vcomp[B, 9, n] with n = n_scalar + ntypes.  Column s < n_scalar is the
 // E/F/V of the model with linear_coeffs = e_s and no bias (the reference obtains the same numbers by
 // differentiating each scalar moment along every pair displacement); column n_scalar + t counts the
-// atoms of species t in the energy and is zero in force and virial.  One E/F/V pass per scalar
-// moment: simple and exact, at the price of recomputing the moments n_scalar times.
+// atoms of species t in the energy and is zero in force and virial.  All columns come from one pass over the
+// atoms (mtp_components_kernel); levels whose node graph is too large take one E/F/V pass per scalar moment.
 template <typename T>
 int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int nmus, int ntypes,
                        const T* q_scaler, double rmax, double rmin, int B, int P, int U, const int* binum,
@@ -1585,6 +2035,42 @@ int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int
     A2P_REQUIRE(ntypes >= 1 && B >= 0 && P >= 0, A2P_ERR_INVALID, "mtp components: bad shape");
     const int S = plan->d.n_scalar, n = S + ntypes;
     if (B == 0 || P == 0) return A2P_OK;
+    rc = fill_zero(ecomp, (size_t)B * n * sizeof(T), stream);
+    if (rc) return rc;
+    rc = fill_zero(fcomp, (size_t)B * P * 3 * n * sizeof(T), stream);
+    if (rc) return rc;
+    rc = fill_zero(vcomp, (size_t)B * 9 * n * sizeof(T), stream);
+    if (rc) return rc;
+    if (components_route() == 1 && plan->d.x_nodes > 0) {
+        MtpArgs<T> a;
+        rc = fill_args(a, plan, K, scaling, coeffs, (const T*)nullptr, (const T*)nullptr, nmus, ntypes, q_scaler, rmax,
+                       rmin, B, P, U, 0, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, false);
+        if (rc) return rc;
+        A2P_REQUIRE(q_scaler, A2P_ERR_INVALID, "mtp components: null q_scaler");
+        a.E = table_entries<T>(a.p, K, false);
+        // LDS: moments | node adjoints | coefficients | table of nc rows; then the packed basic moments
+        auto lds_for = [&](int nc, size_t* main) {
+            // (behind the table: a buffer of 3 n_basic values per wavefront)
+            const size_t region = (size_t)nc * a.E + (size_t)4 * a.p.n_basic * 3;
+            const size_t vals = (size_t)a.p.n_moms + ((a.p.x_nodes + 2) & ~1) + (size_t)ntypes * nmus * K + region;
+            *main = (vals * sizeof(T) + 15) / 16 * 16;
+            return *main + (size_t)a.p.n_basic * sizeof(unsigned);
+        };
+        auto per_cu = [](size_t l) { return (size_t)(160 * 1024) / ((l + 1279) / 1280 * 1280); };
+        size_t m = 0;
+        const size_t want = per_cu(lds_for(MTP_NC_MIN, &m));
+        if (want >= 1) {
+            int nc_cap = MTP_NC_MIN;
+            for (int nc : {MTP_NC_MAX, 40, 32, 24, 20, MTP_NC_MIN})
+                if (per_cu(lds_for(nc, &m)) >= std::min<size_t>(want, 8)) { nc_cap = nc; break; }
+            const size_t lds = lds_for(nc_cap, &m);
+            hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(B * ntypes, 256)), dim3(256), 0, stream,
+                               (T*)nullptr, S, ecomp, B, P, P, ntypes, binum, bilist, btypes);
+            A2P_HIP_CHECK(hipGetLastError());
+            return mtp_lin_components_nodes<T>(plan, a, S, n, ecomp, fcomp, vcomp, lds, (int)m, nc_cap, stream);
+        }
+    }
+    // one E/F/V pass per scalar moment with a one-hot read-out
     // workspace: eye[S*S] | zero bias[ntypes] | etot[B] | force[B*P*3] | virial[B*9]
     const size_t nT = (size_t)S * S + ntypes + B + (size_t)B * P * 3 + (size_t)B * 9;
     void* ws = nullptr;
@@ -1596,12 +2082,6 @@ int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int
     T* force = etot + B;
     T* virial = force + (size_t)B * P * 3;
     rc = fill_zero(ws, (((size_t)S * S + ntypes) * sizeof(T) + 3) / 4 * 4, stream);
-    if (rc) return rc;
-    rc = fill_zero(ecomp, (size_t)B * n * sizeof(T), stream);
-    if (rc) return rc;
-    rc = fill_zero(fcomp, (size_t)B * P * 3 * n * sizeof(T), stream);
-    if (rc) return rc;
-    rc = fill_zero(vcomp, (size_t)B * 9 * n * sizeof(T), stream);
     if (rc) return rc;
     hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(std::max(S, B * ntypes), 256)), dim3(256), 0,
                        stream, eye, S, ecomp, B, P, P, ntypes, binum, bilist, btypes);
@@ -1691,6 +2171,13 @@ int a2p_mtp_plan_create(int n_moms, int n_basic, const int* basic, int n_times, 
     if (rc) return rc;
     *plan = p;
     return A2P_OK;
+}
+
+int a2p_mtp_components_route(int route)
+{
+    const int before = a2p::components_route();
+    if (route == 0 || route == 1) a2p::g_components_route = route;
+    return before;
 }
 
 int a2p_mtp_plan_destroy(void* handle)

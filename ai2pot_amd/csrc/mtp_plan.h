@@ -68,6 +68,27 @@ struct MtpPlanDevice {
     const int* dense_src;      // [nq*nmp] basic moment behind the entry, -1 none, -2 several (dense_off/items)
     const int* dense_off;      // [nq*nmp+1]
     const int* dense_items;    // [n_basic] basic moments ordered by dense entry
+    // The one-hot adjoints of all scalar moments at once (linear-solver components).  A node (s, m) is moment m as an
+    // ancestor of scalar moment s: mapping[s] itself, or a factor of a product among its ancestors.  The adjoint
+    // sweeps of all read-outs e_s together are one reverse gather over the nodes, laid out like the reverse gather
+    // above (a term packs x = 8 node(dst) | 8 other << 16 with `other` a moment, y = mult; x_src names the node).
+    // Scalar moments are dealt to slots sorted by their number of basic ancestors, 64 slots a group; the basic
+    // ancestors of a group's slots are stored interleaved and padded to the group's depth with node x_nodes, whose
+    // adjoint is always zero: word k of slot q is x_bwords[x_bbase[q >> 6] + k * 64 + (q & 63)] = node | basic << 16.
+    // x_nodes = 0: the level has too many nodes for 16-bit offsets (the components are then computed pass by pass).
+    int x_nodes, x_slots;
+    const int* x_root;         // [n_scalar] node (s, mapping[s])
+    const int* x_seed;         // [x_slots]  scalar moment of the slot, -1 in padding
+    const int* x_level;        // [n_levels+1]
+    const int* x_multi;        // [n_levels]
+    const int* x_src;          // [n_xslots]
+    const int* x_rem;          // [n_xslots]
+    const int* x_gbase;        // [n_xslots/64]
+    const int* x_gdepth;       // [n_xslots/64]
+    const int2* x_terms;
+    const int* x_bbase;        // [x_slots/64]
+    const int* x_bdepth;       // [x_slots/64]
+    const int* x_bwords;
 };
 
 struct MtpPlan {

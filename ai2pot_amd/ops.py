@@ -878,7 +878,7 @@ def mtp_lin_components(chebyshev_size, scaling, coeffs, alpha_moments_count, alp
         alpha_moment_mapping, nmus, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, type_map, 0, q_scaler,
         chebyshev_size, validate)
     n = n_scalar + ntypes
-    z = lambda *sh: torch.zeros(sh, dtype=dtype, device=device)
+    z = lambda *sh: torch.empty(sh, dtype=dtype, device=device)       # the library writes every element
     ecomp, fcomp, vcomp = z(B, n), z(B, P, 3, n), z(B, 9, n)
     L = _lib.lib()
     fn = L.a2p_mtp_lin_components_f32 if dtype == torch.float32 else L.a2p_mtp_lin_components_f64
@@ -891,6 +891,21 @@ def mtp_lin_components(chebyshev_size, scaling, coeffs, alpha_moments_count, alp
         if validate:
             _status_or_retry(call, B, P, U, 0, binum, bnumneigh, bfirstneigh, device)
     return ecomp, fcomp, vcomp
+
+
+def _gram(X, y):
+    """X^T X [n, n] and X^T y [n] of a tall matrix X [N, n].  The rows are cut into up to 64 blocks whose products run as
+    one batched GEMM and are added afterwards: a single GEMM with n of about a hundred and N in the tens of thousands
+    occupies one tile of the chip (0.66 ms against 0.03 ms for 24576 x 95 in fp64)."""
+    N, n = X.shape
+    R = torch.cat([X, y.reshape(N, 1)], dim=1)
+    chunks = max(1, min(64, N // 256))
+    k = N // chunks
+    head = k * chunks
+    G = torch.bmm(X[:head].reshape(chunks, k, n).transpose(1, 2), R[:head].reshape(chunks, k, n + 1)).sum(0)
+    if head < N:
+        G = G + X[head:].t() @ R[head:]
+    return G[:, :n], G[:, n]
 
 
 def LinMatrixLinVectorOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_dft, chebyshev_size, scaling,
@@ -920,10 +935,11 @@ def LinMatrixLinVectorOp(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bv
         _req(t.numel() == numel, "%s has %d elements, expected %d" % (name, t.numel(), numel))
     F = fcomp.reshape(B * P * 3, n)          # rows of padded atoms are zero
     V = vcomp.reshape(B * 9, n)
-    lin_matrix = e_weight * (ecomp.t() @ ecomp) + f_weight * (F.t() @ F) + v_weight * (V.t() @ V)
-    lin_vector = (e_weight * (ecomp.t() @ betot_dft.reshape(B)) + f_weight * (F.t() @ bforce_dft.reshape(-1)) +
-                  v_weight * (V.t() @ bvirial_dft.reshape(-1)))
-    return [lin_matrix, lin_vector]
+    (ae, be), (af, bf), (av, bv) = (_gram(ecomp, betot_dft.reshape(B)), _gram(F, bforce_dft.reshape(-1)),
+                                    _gram(V, bvirial_dft.reshape(-1)))
+    lin_matrix = e_weight * ae + f_weight * af + v_weight * av
+    lin_vector = e_weight * be + f_weight * bf + v_weight * bv
+    return [lin_matrix.contiguous(), lin_vector.contiguous()]
 
 
 def CoeffsSchmidtOrthOp(ntypes, nmus, chebyshev_size, coeffs):

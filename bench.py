@@ -633,7 +633,7 @@ def run_nep_train(args):
 
 def run_mtp_solver(args):
     """The normal equations of the linear parameters (LinMatrixLinVectorOp) on configuration 4's structures, level
-    16: one energy / force / virial pass per scalar moment (92) plus three Gram products by the BLAS."""
+    16: the components of all 92 scalar moments from one pass over the atoms, plus three Gram products by the BLAS."""
     import torch
     from ai2pot_amd import _lib, ops, synth
     dev = torch.device("cuda:0")
@@ -661,7 +661,7 @@ def run_mtp_solver(args):
     _lib.check_status(torch.cuda.current_stream(dev).cuda_stream)
     config = {"workload": args.workload, "natoms": natoms, "structures": B, "natoms_pad": P,
               "model": "linear MTP level 16 K=%d" % m["chebyshev_size"], "species": int(m["type_map"].size),
-              "per_step": "normal equations of the linear parameters: %d E/F/V passes + Gram products"
+              "per_step": "normal equations of the linear parameters: components of %d scalar moments + Gram products"
                           % int(m["alpha_moment_mapping"].size)}
     return natoms, elapsed, kernels, None, config, "f64", {}
 

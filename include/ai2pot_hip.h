@@ -500,6 +500,13 @@ int a2p_zbl_esites_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, c
  *   lin_matrix = sum_b e_w E_b^T E_b + f_w F_b^T F_b + v_w V_b^T V_b,   lin_vector = the same against the residuals,
  * are plain GEMMs over these arrays and are left to the caller's BLAS (the bind library uses torch's).
  * nghost is 0, as the reference's force_components has natoms_pad rows.
+ * All columns come from one pass over the atoms: the adjoint of column s is non-zero on the ancestors of scalar
+ * moment s only, so the adjoints of all columns together are one gather about as long as an ordinary adjoint sweep
+ * (the reference differentiates every moment along every pair displacement instead).  The call reads one integer back
+ * (the number of pairs, to size its pair buffer).  Levels with more than 8190 (scalar moment, ancestor) pairs, and
+ * a2p_mtp_components_route(0), take one energy / force / virial pass per scalar moment; both routes agree to rounding.
+ * a2p_mtp_components_route returns the previous setting (1 = one pass, the default; 0 = pass per column); any other
+ * argument only queries.  The environment variable AI2POT_MTP_COMPONENTS=nodes|passes sets the initial value.
  * a2p_mtp_schmidt_orth_*: Gram-Schmidt over the nmus radial functions, each the vector of its
  * ntypes^2 * chebyshev_size coefficients; orth_coeffs must not alias coeffs.
  * ------------------------------------------------------------------------------------------ */
@@ -513,6 +520,7 @@ int a2p_mtp_lin_components_f32(void* plan, int chebyshev_size, double scaling, c
                                int natoms_pad, int umax, const int* binum, const int* bilist, const int* bnumneigh,
                                const int* bfirstneigh, const float* brcs, const int* btypes, float* ecomp,
                                float* fcomp, float* vcomp, void* stream);
+int a2p_mtp_components_route(int route);
 int a2p_mtp_schmidt_orth_f64(int ntypes, int nmus, int chebyshev_size, const double* coeffs, double* orth_coeffs,
                              void* stream);
 int a2p_mtp_schmidt_orth_f32(int ntypes, int nmus, int chebyshev_size, const float* coeffs, float* orth_coeffs,

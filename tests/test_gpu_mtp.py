@@ -450,6 +450,45 @@ def test_linear_system(oracle, level, nt):
     assert close(A.cpu().numpy(), Ar) and close(b.cpu().numpy(), br)
 
 
+@pytest.mark.parametrize("level,nt,U", [(10, 1, None), (16, 3, None), (20, 2, None), (16, 2, 8)])
+def test_components_in_one_pass_equal_a_pass_per_column(oracle, level, nt, U):
+    """The components of the linear system, all columns from one pass over the atoms (the adjoints of all scalar
+    moments as one gather over their ancestors), against one energy / force / virial pass per column: a padded batch
+    with rows in a permuted order (rows of 30-odd neighbours take two chunks of the table at level 16), and (U = 8) lists
+    cut short, in which most pairs have no counterpart from the other end."""
+    import torch
+    from ai2pot_amd import _lib, ops
+    m, nb, _ = loss_inputs(oracle, level, nt, sizes=(30, 41) if level == 20 else (48, 30, 37))
+    if U is not None:                                    # keep the first U neighbours of every row
+        nb = dict(nb)
+        nb["bnumneigh"] = np.minimum(nb["bnumneigh"], U)
+    B, P = nb["bilist"].shape
+    perm = np.argsort(synth.rng_normal(9, P))            # rows of a structure in another order than its atoms
+    for b in range(B):
+        n = int(nb["binum"][b])
+        order = perm[perm < n]
+        for k in ("bilist", "bnumneigh", "bfirstneigh", "brcs"):
+            nb[k][b, :n] = nb[k][b, order]
+    md = model_to_device(m, torch.float64)
+    d = to_device(nb, torch.float64)
+    args = (m["chebyshev_size"], m["scaling"], md["coeffs"], m["alpha_moments_count"], md["alpha_index_basic"],
+            md["alpha_index_times"], md["alpha_moment_mapping"], m["nmus"], d["binum"], d["bilist"], d["bnumneigh"],
+            d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], m["rmax"], m["rmin"], md["q_scaler"])
+    L = _lib.lib()
+    before = L.a2p_mtp_components_route(1)
+    try:
+        one = [t.cpu().numpy() for t in ops.mtp_lin_components(*args)]
+        again = [t.cpu().numpy() for t in ops.mtp_lin_components(*args)]
+        L.a2p_mtp_components_route(0)
+        per_column = [t.cpu().numpy() for t in ops.mtp_lin_components(*args)]
+    finally:
+        L.a2p_mtp_components_route(before)
+    for a, b, c in zip(one, per_column, again):
+        assert np.abs(b).max() > 0
+        assert close(a, b)
+        assert np.array_equal(a, c)                      # bit-reproducible
+
+
 def test_linear_system_and_schmidt_against_golden(oracle):
     """Level 16 against the committed outputs of the reference's CPU launcher and of its Gram-Schmidt."""
     import os
