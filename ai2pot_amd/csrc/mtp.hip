@@ -896,11 +896,11 @@ lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, in
 // latter in the fixed order of a sorted list) and per structure.
 template <typename T>
 struct CompArgs {
-    T* pb;                  // [pairs, 3, x_slots]
+    T* pb;                  // [pairs, 3, n_scalar]
     const int* pair_off;    // [rows + 1] first pair of each row
     const int* nnc;         // [rows] checked neighbour count of each row (0 for rows that are not evaluated)
     T* desc;                // [rows, n_scalar] scalar moments
-    T* rowpart;             // [rows, 12, x_slots] per row and column: sum of the pair derivatives (3), virial (9)
+    T* rowpart;             // [rows, 12, n_scalar] per row and column: sum of the pair derivatives (3), virial (9)
     int nc_cap, lds_basic_off;
 };
 
@@ -925,7 +925,7 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
     const int nn = c.nnc[row];
     if (ii >= a.binum[b] || nn == 0) {                       // padded or refused row (k_rows flags the reasons)
         for (int s = lane; s < S; s += NT) c.desc[row * S + s] = (T)0;
-        for (int q = lane; q < 12 * p.x_slots; q += NT) c.rowpart[row * 12 * p.x_slots + q] = (T)0;
+        for (int q = lane; q < 12 * S; q += NT) c.rowpart[row * 12 * S + q] = (T)0;
         return;
     }
     int center = a.bilist[row];
@@ -1012,8 +1012,9 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             for (int g = 0; g < ngroups; g++) {
-                const int depth = p.x_bdepth[g];
+                const int depth = p.x_bdepth[g], steps = p.x_bsteps[g];
                 const int* wp = p.x_bwords + p.x_bbase[g] + l64;
+                const int col = p.x_seed[g * 64 + l64];
                 T gx = (T)0, gy = (T)0, gz = (T)0;
                 for (int k = 0; k < depth; k++) {
                     const unsigned w = (unsigned)wp[k * 64];
@@ -1021,35 +1022,41 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
                     const T* dv = D + (w >> 16) * 3;
                     gx += adj * dv[0]; gy += adj * dv[1]; gz += adj * dv[2];
                 }
-                T* dst = c.pb + ((size_t)(c.pair_off[row] + c0 + j) * 3) * p.x_slots + g * 64 + l64;
-                dst[0] = gx;
-                dst[(size_t)p.x_slots] = gy;
-                dst[2 * (size_t)p.x_slots] = gz;
+                if (steps) {                                // a long list's pieces sit in neighbouring lanes
+                    const int rem = p.x_brem[g * 64 + l64];
+                    gx = piece_sum(gx, rem, steps); gy = piece_sum(gy, rem, steps); gz = piece_sum(gz, rem, steps);
+                }
+                if (col >= 0) {
+                    T* dst = c.pb + ((size_t)(c.pair_off[row] + c0 + j) * 3) * S + col;
+                    dst[0] = gx;
+                    dst[S] = gy;
+                    dst[2 * S] = gz;
+                }
             }
         }
     }
     // own-row sums of every column (force of the centre, virial), in neighbour order, from the pair derivatives this
-    // workgroup has just written: rowpart[row][12][slots]
+    // workgroup has just written: rowpart[row][12][S]
     __syncthreads();
-    for (int q = lane; q < p.x_slots; q += NT) {
+    for (int q = lane; q < S; q += NT) {
         T f[3] = {(T)0, (T)0, (T)0}, v[9];
 #pragma unroll
         for (int i = 0; i < 9; i++) v[i] = (T)0;
-        const T* g = c.pb + (size_t)c.pair_off[row] * 3 * p.x_slots + q;
+        const T* g = c.pb + (size_t)c.pair_off[row] * 3 * S + q;
         for (int j = 0; j < nn; j++) {
-            const T gx = g[0], gy = g[p.x_slots], gz = g[2 * (size_t)p.x_slots];
+            const T gx = g[0], gy = g[S], gz = g[2 * S];
             const T dx = rcs[j * 3], dy = rcs[j * 3 + 1], dz = rcs[j * 3 + 2];
             f[0] += gx; f[1] += gy; f[2] += gz;
             v[0] -= gx * dx; v[1] -= gx * dy; v[2] -= gx * dz;
             v[3] -= gy * dx; v[4] -= gy * dy; v[5] -= gy * dz;
             v[6] -= gz * dx; v[7] -= gz * dy; v[8] -= gz * dz;
-            g += 3 * (size_t)p.x_slots;
+            g += 3 * (size_t)S;
         }
-        T* o = c.rowpart + row * 12 * p.x_slots + q;
+        T* o = c.rowpart + row * 12 * S + q;
 #pragma unroll
-        for (int i = 0; i < 3; i++) o[(size_t)i * p.x_slots] = f[i];
+        for (int i = 0; i < 3; i++) o[(size_t)i * S] = f[i];
 #pragma unroll
-        for (int i = 0; i < 9; i++) o[(size_t)(3 + i) * p.x_slots] = v[i];
+        for (int i = 0; i < 9; i++) o[(size_t)(3 + i) * S] = v[i];
     }
 }
 
@@ -1114,24 +1121,23 @@ comp_incoming_sort_kernel(int n, const int* __restrict__ ioff, int* __restrict__
 // force column of every atom: its own row's sum minus the pairs that name it, in the order of the sorted list
 template <typename T>
 __global__ void __launch_bounds__(64)
-comp_force_kernel(int slots, int n, const int* __restrict__ seed, const int* __restrict__ row_of1,
-                  const int* __restrict__ ioff, const int* __restrict__ inc, const T* __restrict__ pb,
-                  const T* __restrict__ rowpart, T* __restrict__ fcomp)
+comp_force_kernel(int S, int n, const int* __restrict__ row_of1, const int* __restrict__ ioff,
+                  const int* __restrict__ inc, const T* __restrict__ pb, const T* __restrict__ rowpart,
+                  T* __restrict__ fcomp)
 {
-    const int t = blockIdx.x, q = blockIdx.y * 64 + threadIdx.x;
-    const int s = seed[q];
+    const int t = blockIdx.x, s = blockIdx.y * 64 + threadIdx.x;
+    if (s >= S) return;
     T f[3] = {(T)0, (T)0, (T)0};
     const int r1 = row_of1[t];
     if (r1 > 0) {
-        const T* o = rowpart + (size_t)(r1 - 1) * 12 * slots + q;
+        const T* o = rowpart + (size_t)(r1 - 1) * 12 * S + s;
 #pragma unroll
-        for (int i = 0; i < 3; i++) f[i] = o[(size_t)i * slots];
+        for (int i = 0; i < 3; i++) f[i] = o[(size_t)i * S];
     }
     for (int k = ioff[t]; k < ioff[t + 1]; k++) {
-        const T* g = pb + (size_t)inc[k] * 3 * slots + q;
-        f[0] -= g[0]; f[1] -= g[slots]; f[2] -= g[2 * (size_t)slots];
+        const T* g = pb + (size_t)inc[k] * 3 * S + s;
+        f[0] -= g[0]; f[1] -= g[S]; f[2] -= g[2 * S];
     }
-    if (s < 0) return;
 #pragma unroll
     for (int i = 0; i < 3; i++) fcomp[((size_t)t * 3 + i) * n + s] = f[i];
 }
@@ -1139,22 +1145,21 @@ comp_force_kernel(int slots, int n, const int* __restrict__ seed, const int* __r
 // energy and virial columns per structure: sums over the rows in row order
 template <typename T>
 __global__ void __launch_bounds__(64)
-comp_structure_kernel(int slots, int n, int S, int P, const int* __restrict__ seed, const int* __restrict__ binum,
-                      const T* __restrict__ q_scaler, const T* __restrict__ desc, const T* __restrict__ rowpart,
-                      T* __restrict__ ecomp, T* __restrict__ vcomp)
+comp_structure_kernel(int n, int S, int P, const int* __restrict__ binum, const T* __restrict__ q_scaler,
+                      const T* __restrict__ desc, const T* __restrict__ rowpart, T* __restrict__ ecomp,
+                      T* __restrict__ vcomp)
 {
-    const int b = blockIdx.x, q = blockIdx.y * 64 + threadIdx.x;
-    const int s = seed[q];
-    if (s < 0) return;
+    const int b = blockIdx.x, s = blockIdx.y * 64 + threadIdx.x;
+    if (s >= S) return;
     T e = (T)0, v[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) v[i] = (T)0;
     for (int ii = 0; ii < binum[b]; ii++) {
         const size_t row = (size_t)b * P + ii;
         e += desc[row * S + s];
-        const T* o = rowpart + row * 12 * slots + q;
+        const T* o = rowpart + row * 12 * S + s;
 #pragma unroll
-        for (int i = 0; i < 9; i++) v[i] += o[(size_t)(3 + i) * slots];
+        for (int i = 0; i < 9; i++) v[i] += o[(size_t)(3 + i) * S];
     }
     ecomp[(size_t)b * n + s] = e / q_scaler[s];
 #pragma unroll
@@ -1395,31 +1400,49 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
             for (int m : anc) node_of[m] = -1;
         }
     }
-    const bool x_ok = x_nodes < 8191 && n_basic < 32768;      // node x_nodes (a zero) must have a 16-bit byte offset too
+    const bool x_ok = x_nodes < 8191 && n_basic < 64 * MTP_SLOT_CAP;      // node x_nodes (a zero) must have a 16-bit byte offset too
     if (!x_ok) { xl.assign(1, {}); for (auto& v : x_by) v.clear(); }
     const Ell X = build_ell(xl, x_by);
     A2P_REQUIRE(!X.too_long, A2P_ERR_INVALID, "mtp plan: a moment takes part in more than %d products", 64 * MTP_SLOT_CAP);
+    std::vector<int> x_brem, x_bsteps;
     if (x_ok) {
         std::vector<int> by_len(n_scalar);
         for (int s = 0; s < n_scalar; s++) by_len[s] = s;
         std::stable_sort(by_len.begin(), by_len.end(),
                          [&](int x, int y) { return seed_basic[x].size() > seed_basic[y].size(); });
-        x_seed = by_len;
-        while (x_seed.size() % 64) x_seed.push_back(-1);
-        for (size_t g0 = 0; g0 < x_seed.size(); g0 += 64) {
-            size_t depth = 0;
-            for (size_t q = g0; q < g0 + 64; q++)
-                if (x_seed[q] >= 0) depth = std::max(depth, seed_basic[x_seed[q]].size());
+        struct Piece { int s, t0, n, rem; };
+        std::vector<Piece> pieces;
+        for (int s : by_len) {
+            const int len = (int)seed_basic[s].size();
+            const int np = std::max(1, (len + MTP_SLOT_CAP - 1) / MTP_SLOT_CAP);      // (np <= 64: n_basic < 64 * cap is checked above)
+            if ((int)(pieces.size() % 64) + np > 64)
+                while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
+            for (int q = 0; q < np; q++)
+                pieces.push_back({s, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, len - q * MTP_SLOT_CAP), np - 1 - q});
+        }
+        while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
+        for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
+            int depth = 0, most = 1;
+            for (size_t q = g0; q < g0 + 64; q++) {
+                depth = std::max(depth, pieces[q].n);
+                most = std::max(most, pieces[q].rem + 1);
+            }
+            int steps = 0;
+            while ((1 << steps) < most) steps++;
             x_bbase.push_back((int)x_bwords.size());
-            x_bdepth.push_back((int)depth);
-            x_bwords.resize(x_bwords.size() + depth * 64, x_nodes);       // node x_nodes, basic moment 0
-            for (size_t q = g0; q < g0 + 64; q++)
-                if (x_seed[q] >= 0)
-                    for (size_t k = 0; k < seed_basic[x_seed[q]].size(); k++)
-                        x_bwords[x_bbase.back() + k * 64 + (q - g0)] = seed_basic[x_seed[q]][k];
+            x_bdepth.push_back(depth);
+            x_bsteps.push_back(steps);
+            x_bwords.resize(x_bwords.size() + (size_t)depth * 64, x_nodes);       // node x_nodes, basic moment 0
+            for (size_t q = g0; q < g0 + 64; q++) {
+                const Piece& pc = pieces[q];
+                for (int k = 0; k < pc.n; k++)
+                    x_bwords[x_bbase.back() + (size_t)k * 64 + (q - g0)] = seed_basic[pc.s][pc.t0 + k];
+                x_seed.push_back(pc.s >= 0 && pc.t0 == 0 ? pc.s : -1);
+                x_brem.push_back(pc.rem);
+            }
         }
     }
-    if (x_seed.empty()) { x_seed.push_back(-1); x_bbase.push_back(0); x_bdepth.push_back(0); }
+    if (x_seed.empty()) { x_seed.push_back(-1); x_brem.push_back(0); x_bbase.push_back(0); x_bdepth.push_back(0); x_bsteps.push_back(0); }
     if (x_bwords.empty()) x_bwords.push_back(0);
 
     // one device block
@@ -1467,6 +1490,8 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     const size_t o_xt = add(X.terms.data(), sizeof(int2) * X.terms.size());
     const size_t o_xbb = add(x_bbase.data(), sizeof(int) * x_bbase.size());
     const size_t o_xbd = add(x_bdepth.data(), sizeof(int) * x_bdepth.size());
+    const size_t o_xbs = add(x_bsteps.data(), sizeof(int) * x_bsteps.size());
+    const size_t o_xbr = add(x_brem.data(), sizeof(int) * x_brem.size());
     const size_t o_xbw = add(x_bwords.data(), sizeof(int) * x_bwords.size());
     std::vector<unsigned char> host(total + 16, 0);
     for (auto& s : segs)
@@ -1505,6 +1530,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.x_terms = (const int2*)(base + o_xt);
     d.x_bbase = (const int*)(base + o_xbb); d.x_bdepth = (const int*)(base + o_xbd);
     d.x_bwords = (const int*)(base + o_xbw);
+    d.x_bsteps = (const int*)(base + o_xbs); d.x_brem = (const int*)(base + o_xbr);
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         g_plans.insert(plan);
@@ -1947,7 +1973,7 @@ int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecom
                              int lds_basic_off, int nc_cap, hipStream_t stream)
 {
     const int B = a.B, P = a.P, U = a.U;
-    const int rows = B * P, slots = a.p.x_slots;
+    const int rows = B * P;
     // integer scratch: nnc[rows+1] | pair_off[rows+1] | cnt[rows+1] | ioff[rows+1] | row_of1[rows] | scan tmp
     const int ntmp = scan_tmp_ints(rows + 1);
     void* wsI = nullptr;
@@ -1972,7 +1998,7 @@ int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecom
     A2P_HIP_CHECK(hipStreamSynchronize(stream));
     if (npairs < 0) npairs = 0;
     // pair derivatives | row sums | scalar moments | list of the pairs that name each atom
-    const size_t n_pb = (size_t)std::max(npairs, 1) * 3 * slots, n_rp = (size_t)rows * 12 * slots, n_desc = (size_t)rows * S;
+    const size_t n_pb = (size_t)std::max(npairs, 1) * 3 * S, n_rp = (size_t)rows * 12 * S, n_desc = (size_t)rows * S;
     void* wsT = nullptr;
     rc = ws_get(WS_MTP, (n_pb + n_rp + n_desc) * sizeof(T) + ((size_t)npairs + 1) * sizeof(int), &wsT);
     if (rc) return rc;
@@ -2006,10 +2032,10 @@ int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecom
     hipLaunchKernelGGL(kern, dim3(P, B), dim3(256), lds, stream, a, c);
     prof_end(stream);
     prof_begin("mtp_components_sums", stream);
-    hipLaunchKernelGGL(comp_force_kernel<T>, dim3(rows, slots / 64), dim3(64), 0, stream, slots, n, a.p.x_seed,
-                       (const int*)row_of1, (const int*)ioff, (const int*)inc, (const T*)pb, (const T*)rowpart, fcomp);
-    hipLaunchKernelGGL(comp_structure_kernel<T>, dim3(B, slots / 64), dim3(64), 0, stream, slots, n, S, P, a.p.x_seed,
-                       a.binum, a.q_scaler, (const T*)desc, (const T*)rowpart, ecomp, vcomp);
+    hipLaunchKernelGGL(comp_force_kernel<T>, dim3(rows, ceil_div(S, 64)), dim3(64), 0, stream, S, n, (const int*)row_of1,
+                       (const int*)ioff, (const int*)inc, (const T*)pb, (const T*)rowpart, fcomp);
+    hipLaunchKernelGGL(comp_structure_kernel<T>, dim3(B, ceil_div(S, 64)), dim3(64), 0, stream, n, S, P, a.binum,
+                       a.q_scaler, (const T*)desc, (const T*)rowpart, ecomp, vcomp);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
     (void)plan;

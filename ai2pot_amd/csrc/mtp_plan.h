@@ -72,13 +72,16 @@ struct MtpPlanDevice {
     // ancestor of scalar moment s: mapping[s] itself, or a factor of a product among its ancestors.  The adjoint
     // sweeps of all read-outs e_s together are one reverse gather over the nodes, laid out like the reverse gather
     // above (a term packs x = 8 node(dst) | 8 other << 16 with `other` a moment, y = mult; x_src names the node).
-    // Scalar moments are dealt to slots sorted by their number of basic ancestors, 64 slots a group; the basic
-    // ancestors of a group's slots are stored interleaved and padded to the group's depth with node x_nodes, whose
-    // adjoint is always zero: word k of slot q is x_bwords[x_bbase[q >> 6] + k * 64 + (q & 63)] = node | basic << 16.
+    // The basic ancestors of a scalar moment form a list of words node | basic << 16; lists are sorted by length, cut into
+    // pieces of at most MTP_SLOT_CAP words, and dealt to slots, 64 slots a group, the pieces of a list in neighbouring
+    // slots of one group (the wavefront adds their sums with shuffles, x_bsteps doubling steps).  A group's words are
+    // stored interleaved and padded to the group's depth with node x_nodes, whose adjoint is always zero: word k of
+    // slot q is x_bwords[x_bbase[q >> 6] + k * 64 + (q & 63)].
     // x_nodes = 0: the level has too many nodes for 16-bit offsets (the components are then computed pass by pass).
     int x_nodes, x_slots;
     const int* x_root;         // [n_scalar] node (s, mapping[s])
-    const int* x_seed;         // [x_slots]  scalar moment of the slot, -1 in padding
+    const int* x_seed;         // [x_slots]  scalar moment, in the slot of its list's first piece; -1 elsewhere
+    const int* x_brem;         // [x_slots]  pieces of the same list behind this one
     const int* x_level;        // [n_levels+1]
     const int* x_multi;        // [n_levels]
     const int* x_src;          // [n_xslots]
@@ -88,6 +91,7 @@ struct MtpPlanDevice {
     const int2* x_terms;
     const int* x_bbase;        // [x_slots/64]
     const int* x_bdepth;       // [x_slots/64]
+    const int* x_bsteps;       // [x_slots/64]
     const int* x_bwords;
 };
 
