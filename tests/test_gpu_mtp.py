@@ -489,6 +489,35 @@ def test_components_in_one_pass_equal_a_pass_per_column(oracle, level, nt, U):
         assert np.array_equal(a, c)                      # bit-reproducible
 
 
+def test_components_flag_bad_lists(oracle):
+    """The one-pass components check their lists like the energy / force / virial kernel: a neighbour index or a type
+    outside its range, or a row longer than umax, is skipped on the device and reported; nothing is read or written
+    out of bounds, and a good call afterwards is right."""
+    import torch
+    from ai2pot_amd import _lib, ops
+    m, nb, _ = loss_inputs(oracle, 10, 2, sizes=(30, 24))
+    md = model_to_device(m, torch.float64)
+
+    def run(lists):
+        d = to_device(lists, torch.float64)
+        return ops.mtp_lin_components(m["chebyshev_size"], m["scaling"], md["coeffs"], m["alpha_moments_count"],
+                                      md["alpha_index_basic"], md["alpha_index_times"], md["alpha_moment_mapping"],
+                                      m["nmus"], d["binum"], d["bilist"], d["bnumneigh"], d["bfirstneigh"], d["brcs"],
+                                      d["btypes"], md["type_map"], m["rmax"], m["rmin"], md["q_scaler"])
+    good = [t.cpu().numpy() for t in run(nb)]
+    P = nb["bilist"].shape[1]
+    for key, where, value in (("bfirstneigh", (0, 3, 1), P + 5), ("bfirstneigh", (1, 0, 0), -7),
+                              ("btypes", (0, 2), 9), ("bilist", (1, 4), P + 1),
+                              ("bnumneigh", (0, 1), nb["bfirstneigh"].shape[2] + 3)):
+        bad = {k: (v.copy() if hasattr(v, "copy") else v) for k, v in nb.items()}
+        bad[key][where] = value
+        with pytest.raises((_lib.A2PError, RuntimeError)):      # (the row length is checked on the host first)
+            run(bad)
+    again = [t.cpu().numpy() for t in run(nb)]
+    for a, b in zip(good, again):
+        assert np.array_equal(a, b)
+
+
 def test_linear_system_and_schmidt_against_golden(oracle):
     """Level 16 against the committed outputs of the reference's CPU launcher and of its Gram-Schmidt."""
     import os
