@@ -69,6 +69,7 @@ __host__ __device__ inline bool mtp_dense_in_moments(int nq, int nmp, int n_moms
 constexpr int MTP_NGMAX = 16;     // most thread groups that share the basic moments of a chunk
 constexpr int MTP_KMAX = 16;      // radial basis size limit
 constexpr int MTP_NMUS_MAX = 8;   // radial function count limit
+constexpr int MTP_NODE_CAP = 4094; // most (scalar moment, ancestor) nodes of one launch of the components kernel
 
 template <typename T>
 struct MtpArgs {
@@ -866,26 +867,6 @@ column_store_kernel(T* __restrict__ dst, const T* __restrict__ src, long long n,
     if (i < n) dst[i * ncols + col] = src[i];
 }
 
-// eye[s * S + s] = 1 (the matrix is zero-filled before); counts[b, S + t] = atoms of species t
-template <typename T>
-__global__ void __launch_bounds__(256)
-lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, int B, int P, int NF, int ntypes,
-                           const int* __restrict__ binum, const int* __restrict__ bilist,
-                           const int* __restrict__ btypes)
-{
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (eye && i < S) eye[(size_t)i * S + i] = (T)1;
-    if (i < B * ntypes) {
-        const int b = i / ntypes, t = i - b * ntypes;
-        int cnt = 0;
-        for (int ii = 0; ii < binum[b]; ii++) {
-            const int c = bilist[(size_t)b * P + ii];
-            if ((unsigned)c < (unsigned)NF && btypes[(size_t)b * NF + c] == t) cnt++;
-        }
-        ecomp[(size_t)b * (S + ntypes) + S + t] = (T)cnt;
-    }
-}
-
 // ---- linear-solver components, all scalar moments in one pass ------------------------------------------------
 // Column s of the components is the E/F/V of the read-out e_s / q_scaler[s].  Its adjoint is non-zero on the
 // ancestors of scalar moment s only (15 of 350 moments on average at level 16, 25 of 1352 at level 20), so the adjoints
@@ -967,7 +948,7 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
     sweep_forward<T, false, NT>(p, M, (T*)nullptr, lane);
     for (int s = lane; s < S; s += NT) {
         c.desc[row * S + s] = M[p.mapping[s]];
-        X[p.x_root[s]] = (T)1 / a.q_scaler[s];
+        if (p.x_root[s] >= 0) X[p.x_root[s]] = (T)1 / a.q_scaler[s];       // (the columns of this launch)
     }
     __syncthreads();
     {
@@ -1039,6 +1020,7 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
     // workgroup has just written: rowpart[row][12][S]
     __syncthreads();
     for (int q = lane; q < S; q += NT) {
+        if (p.x_root[q] < 0) continue;                      // a column of another launch
         T f[3] = {(T)0, (T)0, (T)0}, v[9];
 #pragma unroll
         for (int i = 0; i < 9; i++) v[i] = (T)0;
@@ -1142,28 +1124,81 @@ comp_force_kernel(int S, int n, const int* __restrict__ row_of1, const int* __re
     for (int i = 0; i < 3; i++) fcomp[((size_t)t * 3 + i) * n + s] = f[i];
 }
 
-// energy and virial columns per structure: sums over the rows in row order
+// energy and virial columns per structure: sums over the rows in row order, in two steps (blocks of COMP_ROWS rows,
+// then the blocks); part[B][nblocks][10][S]
+constexpr int COMP_ROWS = 32;
+
 template <typename T>
 __global__ void __launch_bounds__(64)
-comp_structure_kernel(int n, int S, int P, const int* __restrict__ binum, const T* __restrict__ q_scaler,
-                      const T* __restrict__ desc, const T* __restrict__ rowpart, T* __restrict__ ecomp,
-                      T* __restrict__ vcomp)
+comp_structure_blocks_kernel(int S, int P, int nblocks, const int* __restrict__ binum, const T* __restrict__ desc,
+                             const T* __restrict__ rowpart, T* __restrict__ part)
 {
-    const int b = blockIdx.x, s = blockIdx.y * 64 + threadIdx.x;
+    const int b = blockIdx.x, s = blockIdx.y * 64 + threadIdx.x, blk = blockIdx.z;
     if (s >= S) return;
     T e = (T)0, v[9];
 #pragma unroll
     for (int i = 0; i < 9; i++) v[i] = (T)0;
-    for (int ii = 0; ii < binum[b]; ii++) {
+    const int i1 = min(binum[b], (blk + 1) * COMP_ROWS);
+    for (int ii = blk * COMP_ROWS; ii < i1; ii++) {
         const size_t row = (size_t)b * P + ii;
         e += desc[row * S + s];
         const T* o = rowpart + row * 12 * S + s;
 #pragma unroll
         for (int i = 0; i < 9; i++) v[i] += o[(size_t)(3 + i) * S];
     }
-    ecomp[(size_t)b * n + s] = e / q_scaler[s];
+    T* o = part + ((size_t)b * nblocks + blk) * 10 * S + s;
+    o[0] = e;
 #pragma unroll
-    for (int i = 0; i < 9; i++) vcomp[((size_t)b * 9 + i) * n + s] = v[i];
+    for (int i = 0; i < 9; i++) o[(size_t)(1 + i) * S] = v[i];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+comp_structure_kernel(int n, int S, int nblocks, const T* __restrict__ q_scaler, const T* __restrict__ part,
+                      T* __restrict__ ecomp, T* __restrict__ vcomp)
+{
+    const int b = blockIdx.x, s = blockIdx.y * 64 + threadIdx.x;
+    if (s >= S) return;
+    T acc[10];
+#pragma unroll
+    for (int i = 0; i < 10; i++) acc[i] = (T)0;
+    for (int blk = 0; blk < nblocks; blk++) {
+        const T* o = part + ((size_t)b * nblocks + blk) * 10 * S + s;
+#pragma unroll
+        for (int i = 0; i < 10; i++) acc[i] += o[(size_t)i * S];
+    }
+    ecomp[(size_t)b * n + s] = acc[0] / q_scaler[s];
+#pragma unroll
+    for (int i = 0; i < 9; i++) vcomp[((size_t)b * 9 + i) * n + s] = acc[1 + i];
+}
+
+// counts[b, t] += 1 for every evaluated row whose centre has species t (integer atomics: exact in any order)
+__global__ void __launch_bounds__(256)
+species_count_kernel(int B, int P, int ntypes, const int* __restrict__ binum, const int* __restrict__ bilist,
+                     const int* __restrict__ btypes, int* __restrict__ counts)
+{
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= B * P) return;
+    const int b = row / P, ii = row - b * P;
+    if (ii >= binum[b]) return;
+    const int c = bilist[row];
+    if ((unsigned)c >= (unsigned)P) return;
+    const int t = btypes[(size_t)b * P + c];
+    if ((unsigned)t < (unsigned)ntypes) atomicAdd(counts + b * ntypes + t, 1);
+}
+
+// eye[s * S + s] = 1 (the matrix is zero-filled before, may be null); ecomp[b, S + t] = counts[b, t]
+template <typename T>
+__global__ void __launch_bounds__(256)
+lin_components_init_kernel(T* __restrict__ eye, int S, T* __restrict__ ecomp, int B, int ntypes,
+                           const int* __restrict__ counts)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (eye && i < S) eye[(size_t)i * S + i] = (T)1;
+    if (i < B * ntypes) {
+        const int b = i / ntypes, t = i - b * ntypes;
+        ecomp[(size_t)b * (S + ntypes) + S + t] = (T)counts[i];
+    }
 }
 
 // Gram-Schmidt over the nmus radial functions, each the vector of its ntypes^2 * K coefficients
@@ -1362,88 +1397,111 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     }
     dense_off[dense_lists.size()] = (int)dense_items.size();
 
-    // nodes (scalar moment, ancestor) and their reverse gather (mtp_plan.h)
-    std::vector<int> x_root(n_scalar, 0), x_seed, x_bbase, x_bdepth, x_bwords;
-    std::vector<std::vector<int2>> xl;
-    std::vector<std::vector<int>> x_by(n_levels);
-    std::vector<std::vector<int>> seed_basic(n_scalar);
-    int x_nodes = 0;
-    {
+    // nodes (scalar moment, ancestor) and their reverse gather (mtp_plan.h), for batches of scalar moments whose node
+    // adjoints fit MTP_NODE_CAP entries of LDS
+    struct XHost {
+        std::vector<int> root, seed, brem, bsteps, bbase, bdepth, bwords;
+        Ell ell;
+        int nodes = 0;
+    };
+    std::vector<XHost> xhosts;
+    if (n_basic < 64 * MTP_SLOT_CAP) {
         std::vector<std::vector<int>> terms_of(n_moms);
         for (int e = 0; e < n_times; e++) terms_of[times[e * 4 + 3]].push_back(e);
         std::vector<int> node_of(n_moms, -1), anc, stack;
-        for (int s = 0; s < n_scalar; s++) {
+        auto ancestors = [&](int s, int first_node) {          // fills anc and node_of; returns the number of nodes
             anc.clear();
             stack.assign(1, mapping[s]);
+            int nd = first_node;
             while (!stack.empty()) {
                 const int m = stack.back();
                 stack.pop_back();
                 if (node_of[m] >= 0) continue;
-                node_of[m] = x_nodes++;
-                xl.emplace_back();
+                node_of[m] = nd++;
                 anc.push_back(m);
                 for (int e : terms_of[m]) { stack.push_back(times[e * 4]); stack.push_back(times[e * 4 + 1]); }
             }
-            x_root[s] = node_of[mapping[s]];
-            for (int e = n_times - 1; e >= 0; e--) {          // reverse file order, as in the reverse gather above
-                const int* q = times + e * 4;
-                if (node_of[q[3]] < 0) continue;
-                const int nd = node_of[q[3]];
-                if (nd * 8 >= 65536) continue;                   // (too many nodes: refused below)
-                xl[node_of[q[1]]].push_back(make_int2((nd * 8) | ((q[0] * 8) << 16), q[2]));
-                xl[node_of[q[0]]].push_back(make_int2((nd * 8) | ((q[1] * 8) << 16), q[2]));
-            }
-            for (int m : anc) {
-                if (level[m] < n_levels && !xl[node_of[m]].empty()) x_by[level[m]].push_back(node_of[m]);
-                if (m < n_basic) seed_basic[s].push_back(node_of[m] | (m << 16));
-            }
+            return nd - first_node;
+        };
+        // batches: scalar moments in table order, as many as fit
+        std::vector<std::vector<int>> batches(1);
+        int in_batch = 0;
+        bool fits = true;
+        for (int s = 0; s < n_scalar; s++) {
+            const int cnt = ancestors(s, 0);
             for (int m : anc) node_of[m] = -1;
+            if (cnt > MTP_NODE_CAP) fits = false;
+            if (in_batch + cnt > MTP_NODE_CAP) { batches.emplace_back(); in_batch = 0; }
+            batches.back().push_back(s);
+            in_batch += cnt;
+        }
+        if (!fits) batches.clear();
+        for (const auto& seeds : batches) {
+            xhosts.emplace_back();
+            XHost& h = xhosts.back();
+            h.root.assign(n_scalar, -1);
+            std::vector<std::vector<int2>> xl;
+            std::vector<std::vector<int>> x_by(n_levels);
+            std::vector<std::vector<int>> seed_basic(n_scalar);
+            for (int s : seeds) {
+                const int cnt = ancestors(s, h.nodes);
+                h.nodes += cnt;
+                xl.resize(h.nodes);
+                h.root[s] = node_of[mapping[s]];
+                for (int e = n_times - 1; e >= 0; e--) {          // reverse file order, as in the reverse gather above
+                    const int* q = times + e * 4;
+                    if (node_of[q[3]] < 0) continue;
+                    const int nd = node_of[q[3]];
+                    xl[node_of[q[1]]].push_back(make_int2((nd * 8) | ((q[0] * 8) << 16), q[2]));
+                    xl[node_of[q[0]]].push_back(make_int2((nd * 8) | ((q[1] * 8) << 16), q[2]));
+                }
+                for (int m : anc) {
+                    if (level[m] < n_levels && !xl[node_of[m]].empty()) x_by[level[m]].push_back(node_of[m]);
+                    if (m < n_basic) seed_basic[s].push_back(node_of[m] | (m << 16));
+                }
+                for (int m : anc) node_of[m] = -1;
+            }
+            if (xl.empty()) xl.emplace_back();
+            h.ell = build_ell(xl, x_by);
+            A2P_REQUIRE(!h.ell.too_long, A2P_ERR_INVALID, "mtp plan: a moment takes part in more than %d products",
+                        64 * MTP_SLOT_CAP);
+            std::vector<int> by_len = seeds;
+            std::stable_sort(by_len.begin(), by_len.end(),
+                             [&](int x, int y) { return seed_basic[x].size() > seed_basic[y].size(); });
+            struct Piece { int s, t0, n, rem; };
+            std::vector<Piece> pieces;
+            for (int s : by_len) {
+                const int len = (int)seed_basic[s].size();
+                const int np = std::max(1, (len + MTP_SLOT_CAP - 1) / MTP_SLOT_CAP);      // <= 64: n_basic < 64 * cap
+                if ((int)(pieces.size() % 64) + np > 64)
+                    while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
+                for (int q = 0; q < np; q++)
+                    pieces.push_back({s, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, len - q * MTP_SLOT_CAP), np - 1 - q});
+            }
+            while (pieces.empty() || pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
+            for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
+                int depth = 0, most = 1;
+                for (size_t q = g0; q < g0 + 64; q++) {
+                    depth = std::max(depth, pieces[q].n);
+                    most = std::max(most, pieces[q].rem + 1);
+                }
+                int steps = 0;
+                while ((1 << steps) < most) steps++;
+                h.bbase.push_back((int)h.bwords.size());
+                h.bdepth.push_back(depth);
+                h.bsteps.push_back(steps);
+                h.bwords.resize(h.bwords.size() + (size_t)depth * 64, h.nodes);       // node `nodes` (a zero), basic moment 0
+                for (size_t q = g0; q < g0 + 64; q++) {
+                    const Piece& pc = pieces[q];
+                    for (int k = 0; k < pc.n; k++)
+                        h.bwords[h.bbase.back() + (size_t)k * 64 + (q - g0)] = seed_basic[pc.s][pc.t0 + k];
+                    h.seed.push_back(pc.s >= 0 && pc.t0 == 0 ? pc.s : -1);
+                    h.brem.push_back(pc.rem);
+                }
+            }
+            if (h.bwords.empty()) h.bwords.push_back(0);
         }
     }
-    const bool x_ok = x_nodes < 8191 && n_basic < 64 * MTP_SLOT_CAP;      // node x_nodes (a zero) must have a 16-bit byte offset too
-    if (!x_ok) { xl.assign(1, {}); for (auto& v : x_by) v.clear(); }
-    const Ell X = build_ell(xl, x_by);
-    A2P_REQUIRE(!X.too_long, A2P_ERR_INVALID, "mtp plan: a moment takes part in more than %d products", 64 * MTP_SLOT_CAP);
-    std::vector<int> x_brem, x_bsteps;
-    if (x_ok) {
-        std::vector<int> by_len(n_scalar);
-        for (int s = 0; s < n_scalar; s++) by_len[s] = s;
-        std::stable_sort(by_len.begin(), by_len.end(),
-                         [&](int x, int y) { return seed_basic[x].size() > seed_basic[y].size(); });
-        struct Piece { int s, t0, n, rem; };
-        std::vector<Piece> pieces;
-        for (int s : by_len) {
-            const int len = (int)seed_basic[s].size();
-            const int np = std::max(1, (len + MTP_SLOT_CAP - 1) / MTP_SLOT_CAP);      // (np <= 64: n_basic < 64 * cap is checked above)
-            if ((int)(pieces.size() % 64) + np > 64)
-                while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
-            for (int q = 0; q < np; q++)
-                pieces.push_back({s, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, len - q * MTP_SLOT_CAP), np - 1 - q});
-        }
-        while (pieces.size() % 64) pieces.push_back({-1, 0, 0, 0});
-        for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
-            int depth = 0, most = 1;
-            for (size_t q = g0; q < g0 + 64; q++) {
-                depth = std::max(depth, pieces[q].n);
-                most = std::max(most, pieces[q].rem + 1);
-            }
-            int steps = 0;
-            while ((1 << steps) < most) steps++;
-            x_bbase.push_back((int)x_bwords.size());
-            x_bdepth.push_back(depth);
-            x_bsteps.push_back(steps);
-            x_bwords.resize(x_bwords.size() + (size_t)depth * 64, x_nodes);       // node x_nodes, basic moment 0
-            for (size_t q = g0; q < g0 + 64; q++) {
-                const Piece& pc = pieces[q];
-                for (int k = 0; k < pc.n; k++)
-                    x_bwords[x_bbase.back() + (size_t)k * 64 + (q - g0)] = seed_basic[pc.s][pc.t0 + k];
-                x_seed.push_back(pc.s >= 0 && pc.t0 == 0 ? pc.s : -1);
-                x_brem.push_back(pc.rem);
-            }
-        }
-    }
-    if (x_seed.empty()) { x_seed.push_back(-1); x_brem.push_back(0); x_bbase.push_back(0); x_bdepth.push_back(0); x_bsteps.push_back(0); }
-    if (x_bwords.empty()) x_bwords.push_back(0);
 
     // one device block
     struct Seg { const void* src; size_t bytes; size_t off; };
@@ -1479,20 +1537,26 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     const size_t o_doff = add(dense_off.data(), sizeof(int) * dense_off.size());
     const size_t o_dit = add(dense_items.data(), sizeof(int) * dense_items.size());
     const size_t o_dpos = add(dense_pos.data(), sizeof(int) * dense_pos.size());
-    const size_t o_xroot = add(x_root.data(), sizeof(int) * x_root.size());
-    const size_t o_xseed = add(x_seed.data(), sizeof(int) * x_seed.size());
-    const size_t o_xl = add(X.level.data(), sizeof(int) * X.level.size());
-    const size_t o_xx = add(X.multi.data(), sizeof(int) * X.multi.size());
-    const size_t o_xs = add(X.slot.data(), sizeof(int) * X.slot.size());
-    const size_t o_xc = add(X.lead.data(), sizeof(int) * X.lead.size());
-    const size_t o_xg = add(X.gbase.data(), sizeof(int) * X.gbase.size());
-    const size_t o_xh = add(X.gdepth.data(), sizeof(int) * X.gdepth.size());
-    const size_t o_xt = add(X.terms.data(), sizeof(int2) * X.terms.size());
-    const size_t o_xbb = add(x_bbase.data(), sizeof(int) * x_bbase.size());
-    const size_t o_xbd = add(x_bdepth.data(), sizeof(int) * x_bdepth.size());
-    const size_t o_xbs = add(x_bsteps.data(), sizeof(int) * x_bsteps.size());
-    const size_t o_xbr = add(x_brem.data(), sizeof(int) * x_brem.size());
-    const size_t o_xbw = add(x_bwords.data(), sizeof(int) * x_bwords.size());
+    struct XOff { size_t root, seed, level, multi, src, rem, gbase, gdepth, terms, bbase, bdepth, bsteps, brem, bwords; };
+    std::vector<XOff> xoffs;
+    for (const XHost& h : xhosts) {
+        XOff o;
+        o.root = add(h.root.data(), sizeof(int) * h.root.size());
+        o.seed = add(h.seed.data(), sizeof(int) * h.seed.size());
+        o.level = add(h.ell.level.data(), sizeof(int) * h.ell.level.size());
+        o.multi = add(h.ell.multi.data(), sizeof(int) * h.ell.multi.size());
+        o.src = add(h.ell.slot.data(), sizeof(int) * h.ell.slot.size());
+        o.rem = add(h.ell.lead.data(), sizeof(int) * h.ell.lead.size());
+        o.gbase = add(h.ell.gbase.data(), sizeof(int) * h.ell.gbase.size());
+        o.gdepth = add(h.ell.gdepth.data(), sizeof(int) * h.ell.gdepth.size());
+        o.terms = add(h.ell.terms.data(), sizeof(int2) * h.ell.terms.size());
+        o.bbase = add(h.bbase.data(), sizeof(int) * h.bbase.size());
+        o.bdepth = add(h.bdepth.data(), sizeof(int) * h.bdepth.size());
+        o.bsteps = add(h.bsteps.data(), sizeof(int) * h.bsteps.size());
+        o.brem = add(h.brem.data(), sizeof(int) * h.brem.size());
+        o.bwords = add(h.bwords.data(), sizeof(int) * h.bwords.size());
+        xoffs.push_back(o);
+    }
     std::vector<unsigned char> host(total + 16, 0);
     for (auto& s : segs)
         if (s.bytes) std::memcpy(host.data() + s.off, s.src, s.bytes);
@@ -1521,16 +1585,21 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
     d.rows = (const int*)(base + o_rows); d.dense_src = (const int*)(base + o_dsrc);
     d.dense_off = (const int*)(base + o_doff); d.dense_items = (const int*)(base + o_dit);
     d.dense_pos = (const int*)(base + o_dpos); d.dense_unique = dense_unique;
-    d.x_nodes = x_ok ? x_nodes : 0;
-    d.x_slots = x_ok ? (int)x_seed.size() : 0;
-    d.x_root = (const int*)(base + o_xroot); d.x_seed = (const int*)(base + o_xseed);
-    d.x_level = (const int*)(base + o_xl); d.x_multi = (const int*)(base + o_xx);
-    d.x_src = (const int*)(base + o_xs); d.x_rem = (const int*)(base + o_xc);
-    d.x_gbase = (const int*)(base + o_xg); d.x_gdepth = (const int*)(base + o_xh);
-    d.x_terms = (const int2*)(base + o_xt);
-    d.x_bbase = (const int*)(base + o_xbb); d.x_bdepth = (const int*)(base + o_xbd);
-    d.x_bwords = (const int*)(base + o_xbw);
-    d.x_bsteps = (const int*)(base + o_xbs); d.x_brem = (const int*)(base + o_xbr);
+    d.x_nodes = 0; d.x_slots = 0;                // set per batch by the components call (MtpPlan::xbatches)
+    for (size_t i = 0; i < xhosts.size(); i++) {
+        const XOff& o = xoffs[i];
+        MtpXBatch xb;
+        xb.nodes = xhosts[i].nodes; xb.slots = (int)xhosts[i].seed.size();
+        xb.root = (const int*)(base + o.root); xb.seed = (const int*)(base + o.seed);
+        xb.level = (const int*)(base + o.level); xb.multi = (const int*)(base + o.multi);
+        xb.src = (const int*)(base + o.src); xb.rem = (const int*)(base + o.rem);
+        xb.gbase = (const int*)(base + o.gbase); xb.gdepth = (const int*)(base + o.gdepth);
+        xb.terms = (const int2*)(base + o.terms);
+        xb.bbase = (const int*)(base + o.bbase); xb.bdepth = (const int*)(base + o.bdepth);
+        xb.bsteps = (const int*)(base + o.bsteps); xb.brem = (const int*)(base + o.brem);
+        xb.bwords = (const int*)(base + o.bwords);
+        plan->xbatches.push_back(xb);
+    }
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         g_plans.insert(plan);
@@ -1969,8 +2038,8 @@ int components_route()
 }
 
 template <typename T>
-int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecomp, T* fcomp, T* vcomp, size_t lds,
-                             int lds_basic_off, int nc_cap, hipStream_t stream)
+int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecomp, T* fcomp, T* vcomp,
+                             hipStream_t stream)
 {
     const int B = a.B, P = a.P, U = a.U;
     const int rows = B * P;
@@ -2023,22 +2092,51 @@ int mtp_lin_components_nodes(MtpPlan* plan, MtpArgs<T>& a, int S, int n, T* ecom
     prof_end(stream);
 
     CompArgs<T> c;
-    c.pb = pb; c.pair_off = pair_off; c.nnc = nnc; c.desc = desc; c.rowpart = rowpart; c.nc_cap = nc_cap;
-    c.lds_basic_off = lds_basic_off;
+    c.pb = pb; c.pair_off = pair_off; c.nnc = nnc; c.desc = desc; c.rowpart = rowpart;
     auto kern = mtp_components_kernel<T, 256>;
-    if (lds > 48 * 1024)
-        A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    prof_begin("mtp_components_kernel", stream);
-    hipLaunchKernelGGL(kern, dim3(P, B), dim3(256), lds, stream, a, c);
-    prof_end(stream);
+    for (const MtpXBatch& xb : plan->xbatches) {
+        MtpPlanDevice& p = a.p;
+        p.x_nodes = xb.nodes; p.x_slots = xb.slots; p.x_root = xb.root; p.x_seed = xb.seed;
+        p.x_level = xb.level; p.x_multi = xb.multi; p.x_src = xb.src; p.x_rem = xb.rem;
+        p.x_gbase = xb.gbase; p.x_gdepth = xb.gdepth; p.x_terms = xb.terms;
+        p.x_bbase = xb.bbase; p.x_bdepth = xb.bdepth; p.x_bsteps = xb.bsteps; p.x_brem = xb.brem; p.x_bwords = xb.bwords;
+        // LDS: moments | node adjoints | coefficients | table of nc rows | 3 n_basic values per wavefront; then the
+        // packed basic moments.  Workgroups per CU count first, then the longest table that still allows them.
+        auto lds_for = [&](int nc, size_t* main) {
+            const size_t vals = (size_t)p.n_moms + ((p.x_nodes + 2) & ~1) + (size_t)a.ntypes * p.nmus * a.K +
+                                (size_t)nc * a.E + (size_t)4 * p.n_basic * 3;
+            *main = (vals * sizeof(T) + 15) / 16 * 16;
+            return *main + (size_t)p.n_basic * sizeof(unsigned);
+        };
+        auto per_cu = [](size_t l) { return (size_t)(160 * 1024) / ((l + 1279) / 1280 * 1280); };
+        size_t m = 0;
+        const size_t want = std::min<size_t>(per_cu(lds_for(MTP_NC_MIN, &m)), 8);
+        A2P_REQUIRE(want >= 1, A2P_ERR_INVALID, "mtp components: %d moments need %zu bytes of LDS per atom", p.n_moms,
+                    lds_for(MTP_NC_MIN, &m));
+        int nc_cap = MTP_NC_MIN;
+        for (int nc : {MTP_NC_MAX, 40, 32, 24, 20, MTP_NC_MIN})
+            if (per_cu(lds_for(nc, &m)) >= want) { nc_cap = nc; break; }
+        const size_t lds = lds_for(nc_cap, &m);
+        c.nc_cap = nc_cap; c.lds_basic_off = (int)m;
+        if (lds > 48 * 1024)
+            A2P_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        prof_begin("mtp_components_kernel", stream);
+        hipLaunchKernelGGL(kern, dim3(P, B), dim3(256), lds, stream, a, c);
+        prof_end(stream);
+    }
     prof_begin("mtp_components_sums", stream);
     hipLaunchKernelGGL(comp_force_kernel<T>, dim3(rows, ceil_div(S, 64)), dim3(64), 0, stream, S, n, (const int*)row_of1,
                        (const int*)ioff, (const int*)inc, (const T*)pb, (const T*)rowpart, fcomp);
-    hipLaunchKernelGGL(comp_structure_kernel<T>, dim3(B, ceil_div(S, 64)), dim3(64), 0, stream, n, S, P, a.binum,
-                       a.q_scaler, (const T*)desc, (const T*)rowpart, ecomp, vcomp);
+    const int nblocks = ceil_div(P, COMP_ROWS);
+    void* wsP = nullptr;
+    rc = ws_get(WS_MISC, (size_t)B * nblocks * 10 * S * sizeof(T), &wsP);
+    if (rc) return rc;
+    hipLaunchKernelGGL(comp_structure_blocks_kernel<T>, dim3(B, ceil_div(S, 64), nblocks), dim3(64), 0, stream, S, P,
+                       nblocks, a.binum, (const T*)desc, (const T*)rowpart, (T*)wsP);
+    hipLaunchKernelGGL(comp_structure_kernel<T>, dim3(B, ceil_div(S, 64)), dim3(64), 0, stream, n, S, nblocks, a.q_scaler,
+                       (const T*)wsP, ecomp, vcomp);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());
-    (void)plan;
     return A2P_OK;
 }
 
@@ -2067,34 +2165,27 @@ int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int
     if (rc) return rc;
     rc = fill_zero(vcomp, (size_t)B * 9 * n * sizeof(T), stream);
     if (rc) return rc;
-    if (components_route() == 1 && plan->d.x_nodes > 0) {
+    // atoms of each species per structure (the bias columns of the energy)
+    void* wsC = nullptr;
+    rc = ws_get(WS_PARTIAL, (size_t)B * ntypes * sizeof(int), &wsC);
+    if (rc) return rc;
+    int* counts = (int*)wsC;
+    rc = fill_zero(counts, (size_t)B * ntypes * sizeof(int), stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(species_count_kernel, dim3(ceil_div(B * P, 256)), dim3(256), 0, stream, B, P, ntypes, binum, bilist,
+                       btypes, counts);
+    A2P_HIP_CHECK(hipGetLastError());
+    if (components_route() == 1 && !plan->xbatches.empty()) {
         MtpArgs<T> a;
         rc = fill_args(a, plan, K, scaling, coeffs, (const T*)nullptr, (const T*)nullptr, nmus, ntypes, q_scaler, rmax,
                        rmin, B, P, U, 0, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes, false);
         if (rc) return rc;
         A2P_REQUIRE(q_scaler, A2P_ERR_INVALID, "mtp components: null q_scaler");
         a.E = table_entries<T>(a.p, K, false);
-        // LDS: moments | node adjoints | coefficients | table of nc rows; then the packed basic moments
-        auto lds_for = [&](int nc, size_t* main) {
-            // (behind the table: a buffer of 3 n_basic values per wavefront)
-            const size_t region = (size_t)nc * a.E + (size_t)4 * a.p.n_basic * 3;
-            const size_t vals = (size_t)a.p.n_moms + ((a.p.x_nodes + 2) & ~1) + (size_t)ntypes * nmus * K + region;
-            *main = (vals * sizeof(T) + 15) / 16 * 16;
-            return *main + (size_t)a.p.n_basic * sizeof(unsigned);
-        };
-        auto per_cu = [](size_t l) { return (size_t)(160 * 1024) / ((l + 1279) / 1280 * 1280); };
-        size_t m = 0;
-        const size_t want = per_cu(lds_for(MTP_NC_MIN, &m));
-        if (want >= 1) {
-            int nc_cap = MTP_NC_MIN;
-            for (int nc : {MTP_NC_MAX, 40, 32, 24, 20, MTP_NC_MIN})
-                if (per_cu(lds_for(nc, &m)) >= std::min<size_t>(want, 8)) { nc_cap = nc; break; }
-            const size_t lds = lds_for(nc_cap, &m);
-            hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(B * ntypes, 256)), dim3(256), 0, stream,
-                               (T*)nullptr, S, ecomp, B, P, P, ntypes, binum, bilist, btypes);
-            A2P_HIP_CHECK(hipGetLastError());
-            return mtp_lin_components_nodes<T>(plan, a, S, n, ecomp, fcomp, vcomp, lds, (int)m, nc_cap, stream);
-        }
+        hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(B * ntypes, 256)), dim3(256), 0, stream,
+                           (T*)nullptr, S, ecomp, B, ntypes, (const int*)counts);
+        A2P_HIP_CHECK(hipGetLastError());
+        return mtp_lin_components_nodes<T>(plan, a, S, n, ecomp, fcomp, vcomp, stream);
     }
     // one E/F/V pass per scalar moment with a one-hot read-out
     // workspace: eye[S*S] | zero bias[ntypes] | etot[B] | force[B*P*3] | virial[B*9]
@@ -2110,7 +2201,7 @@ int mtp_lin_components(void* handle, int K, double scaling, const T* coeffs, int
     rc = fill_zero(ws, (((size_t)S * S + ntypes) * sizeof(T) + 3) / 4 * 4, stream);
     if (rc) return rc;
     hipLaunchKernelGGL(lin_components_init_kernel<T>, dim3(ceil_div(std::max(S, B * ntypes), 256)), dim3(256), 0,
-                       stream, eye, S, ecomp, B, P, P, ntypes, binum, bilist, btypes);
+                       stream, eye, S, ecomp, B, ntypes, (const int*)counts);
     A2P_HIP_CHECK(hipGetLastError());
     for (int s = 0; s < S; s++) {
         // force / virial go to WS_MISC, which mtp_efv does not touch when a force pointer is given

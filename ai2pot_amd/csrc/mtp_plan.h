@@ -77,7 +77,8 @@ struct MtpPlanDevice {
     // slots of one group (the wavefront adds their sums with shuffles, x_bsteps doubling steps).  A group's words are
     // stored interleaved and padded to the group's depth with node x_nodes, whose adjoint is always zero: word k of
     // slot q is x_bwords[x_bbase[q >> 6] + k * 64 + (q & 63)].
-    // x_nodes = 0: the level has too many nodes for 16-bit offsets (the components are then computed pass by pass).
+    // The scalar moments are dealt to batches whose nodes fit the kernel's LDS budget (MtpPlan::xbatches); the fields
+    // below are those of the batch a launch works on (x_root is -1 for the scalar moments of other batches).
     int x_nodes, x_slots;
     const int* x_root;         // [n_scalar] node (s, mapping[s])
     const int* x_seed;         // [x_slots]  scalar moment, in the slot of its list's first piece; -1 elsewhere
@@ -95,8 +96,17 @@ struct MtpPlanDevice {
     const int* x_bwords;
 };
 
+// one batch of scalar moments of the components kernel: the x_ fields of MtpPlanDevice
+struct MtpXBatch {
+    int nodes, slots;
+    const int *root, *seed, *level, *multi, *src, *rem, *gbase, *gdepth;
+    const int2* terms;
+    const int *bbase, *bdepth, *bsteps, *brem, *bwords;
+};
+
 struct MtpPlan {
     MtpPlanDevice d;
+    std::vector<MtpXBatch> xbatches;   // empty: a scalar moment has too many ancestors (components pass by pass)
     void* device_block = nullptr;   // one allocation holding all arrays
     int device = 0;
 };

@@ -450,7 +450,7 @@ def test_linear_system(oracle, level, nt):
     assert close(A.cpu().numpy(), Ar) and close(b.cpu().numpy(), br)
 
 
-@pytest.mark.parametrize("level,nt,U", [(10, 1, None), (16, 3, None), (20, 2, None), (16, 2, 8)])
+@pytest.mark.parametrize("level,nt,U", [(10, 1, None), (16, 3, None), (20, 2, None), (22, 2, None), (16, 2, 8)])
 def test_components_in_one_pass_equal_a_pass_per_column(oracle, level, nt, U):
     """The components of the linear system, all columns from one pass over the atoms (the adjoints of all scalar
     moments as one gather over their ancestors), against one energy / force / virial pass per column: a padded batch
@@ -458,7 +458,7 @@ def test_components_in_one_pass_equal_a_pass_per_column(oracle, level, nt, U):
     cut short, in which most pairs have no counterpart from the other end."""
     import torch
     from ai2pot_amd import _lib, ops
-    m, nb, _ = loss_inputs(oracle, level, nt, sizes=(30, 41) if level == 20 else (48, 30, 37))
+    m, nb, _ = loss_inputs(oracle, level, nt, sizes=(30, 41) if level >= 20 else (48, 30, 37))
     if U is not None:                                    # keep the first U neighbours of every row
         nb = dict(nb)
         nb["bnumneigh"] = np.minimum(nb["bnumneigh"], U)
