@@ -997,12 +997,25 @@ __global__ void __launch_bounds__(NT) mtp_components_kernel(const MtpArgs<T> a, 
                 const int* wp = p.x_bwords + p.x_bbase[g] + l64;
                 const int col = p.x_seed[g * 64 + l64];
                 T gx = (T)0, gy = (T)0, gz = (T)0;
-                for (int k = 0; k < depth; k++) {
-                    const unsigned w = (unsigned)wp[k * 64];
-                    const T adj = X[w & 0xffffu];
-                    const T* dv = D + (w >> 16) * 3;
-                    gx += adj * dv[0]; gy += adj * dv[1]; gz += adj * dv[2];
-                }
+                // all words of the slot (at most MTP_SLOT_CAP; the depth is a multiple of four and shared by the
+                // wavefront) are requested before the first is used
+                int w[MTP_SLOT_CAP];
+#pragma unroll
+                for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                    if (k < depth) {
+#pragma unroll
+                        for (int u = 0; u < 4; u++) w[k + u] = wp[(k + u) * 64];
+                    }
+#pragma unroll
+                for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+                    if (k < depth) {
+#pragma unroll
+                        for (int u = k; u < k + 4; u++) {
+                            const T adj = X[(unsigned)w[u] & 0xffffu];
+                            const T* dv = D + ((unsigned)w[u] >> 16) * 3;
+                            gx += adj * dv[0]; gy += adj * dv[1]; gz += adj * dv[2];
+                        }
+                    }
                 if (steps) {                                // a long list's pieces sit in neighbouring lanes
                     const int rem = p.x_brem[g * 64 + l64];
                     gx = piece_sum(gx, rem, steps); gy = piece_sum(gy, rem, steps); gz = piece_sum(gz, rem, steps);
@@ -1487,6 +1500,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
                 }
                 int steps = 0;
                 while ((1 << steps) < most) steps++;
+                depth = (depth + 3) / 4 * 4;            // the kernel fetches four words at a time
                 h.bbase.push_back((int)h.bwords.size());
                 h.bdepth.push_back(depth);
                 h.bsteps.push_back(steps);

@@ -503,7 +503,9 @@ int a2p_zbl_esites_f32(double zbl_rmax, double zbl_rmin, const float* zbl_cks, c
  * All columns come from one pass over the atoms: the adjoint of column s is non-zero on the ancestors of scalar
  * moment s only, so the adjoints of all columns together are one gather about as long as an ordinary adjoint sweep
  * (the reference differentiates every moment along every pair displacement instead).  The call reads one integer back
- * (the number of pairs, to size its pair buffer).  a2p_mtp_components_route(0) switches to one energy / force / virial
+ * (the number of pairs, to size its pair buffer: pairs * 3 * n_scalar values in the library's workspace, 0.4 GB for
+ * 8192 atoms of 21 neighbours at level 16, 2 GB for 8192 atoms of 35 neighbours at level 20), so it cannot be captured in
+ * a HIP graph.  a2p_mtp_components_route(0) switches to one energy / force / virial
  * pass per scalar moment; both routes agree to rounding.
  * a2p_mtp_components_route returns the previous setting (1 = one pass, the default; 0 = pass per column); any other
  * argument only queries.  The environment variable AI2POT_MTP_COMPONENTS=nodes|passes sets the initial value.
