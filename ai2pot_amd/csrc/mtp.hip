@@ -835,7 +835,7 @@ nnmtp_grad_reduce_kernel(int P, int NF, int nblk, int HS, int H, int ntypes, con
     if (q >= nrow) return;
     const int inum = binum[b];
     T acc = (T)0;
-    // eight rows in flight; the rows of other species add zero, the order of the sum is the atom order
+    // eight rows in flight; the rows of other species are skipped, the order of the sum is the atom order
     for (int i0 = 0; i0 < inum; i0 += 8) {
         int c[8], ty[8];
         T v[8];
@@ -848,9 +848,12 @@ nnmtp_grad_reduce_kernel(int P, int NF, int nblk, int HS, int H, int ntypes, con
             if (!ok) ty[u] = -1;
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = gpart[((size_t)b * P + min(i0 + u, inum - 1)) * nrow + q];
+        for (int u = 0; u < 8; u++) {            // (a row of another species is not read)
+            v[u] = (T)0;
+            if (ty[u] == t) v[u] = gpart[((size_t)b * P + min(i0 + u, inum - 1)) * nrow + q];
+        }
 #pragma unroll
-        for (int u = 0; u < 8; u++) acc += ty[u] == t ? v[u] : (T)0;
+        for (int u = 0; u < 8; u++) acc += v[u];
     }
     if (q < nblk) { if (dcoeffs) dcoeffs[((size_t)b * ntypes + t) * nblk + q] = acc; }
     else if (q < nblk + HS) { if (dw0) dw0[((size_t)b * ntypes + t) * HS + q - nblk] = acc; }

@@ -329,7 +329,8 @@ __global__ void __launch_bounds__(LNT) nep_loss_grad_kernel(const NepLossArgs<T>
 }
 
 // Full-layout gradients of one structure: element e of the layout belongs to centre species t(e)
-// and position q(e) of the per-atom row; sum the rows of the atoms of that species in atom order.
+// and position q(e) of the per-atom row; sum the rows of the atoms of that species (four runs of rows in atom order,
+// then the runs).
 template <typename T>
 __global__ void __launch_bounds__(256)
 nep_grad_reduce_kernel(NepLossArgs<T> a, T* __restrict__ dcoeffs, T* __restrict__ dw0, T* __restrict__ db0,
@@ -340,36 +341,48 @@ nep_grad_reduce_kernel(NepLossArgs<T> a, T* __restrict__ dcoeffs, T* __restrict_
     const int ncl = nt * nb * K;
     const int n_c = nt * ncl, n_w0 = nt * H * D, n_h = nt * H;
     const int total = n_c + n_w0 + 2 * n_h + nt;
-    const int e = blockIdx.x * 256 + threadIdx.x;
-    if (e >= total) return;
-    int t, q;
-    T* out;
-    if (e < n_c) { t = e / ncl; q = e - t * ncl; out = dcoeffs ? dcoeffs + (size_t)b * n_c + e : nullptr; }
-    else if (e < n_c + n_w0) { const int r = e - n_c; t = r / (H * D); q = ncl + r - t * H * D; out = dw0 ? dw0 + (size_t)b * n_w0 + r : nullptr; }
-    else if (e < n_c + n_w0 + n_h) { const int r = e - n_c - n_w0; t = r / H; q = ncl + H * D + r - t * H; out = db0 ? db0 + (size_t)b * n_h + r : nullptr; }
-    else if (e < n_c + n_w0 + 2 * n_h) { const int r = e - n_c - n_w0 - n_h; t = r / H; q = ncl + H * D + H + r - t * H; out = dw1 ? dw1 + (size_t)b * n_h + r : nullptr; }
-    else { t = e - n_c - n_w0 - 2 * n_h; q = a.nrow - 1; out = dbias ? dbias + (size_t)b * nt + t : nullptr; }
-    if (!out) return;
-    const int inum = a.binum[b];
-    T acc = (T)0;
-    // eight rows in flight; the rows of other species add zero, the order of the sum is the atom order
-    for (int i0 = 0; i0 < inum; i0 += 8) {
-        int c[8], ty[8];
-        T v[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) c[u] = a.bilist[(size_t)b * a.P + min(i0 + u, inum - 1)];
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const bool ok = i0 + u < inum && (unsigned)c[u] < (unsigned)a.P;
-            ty[u] = a.btypes[(size_t)b * a.P + (ok ? c[u] : 0)];
-            if (!ok) ty[u] = -1;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = a.gpart[((size_t)b * a.P + min(i0 + u, inum - 1)) * a.nrow + q];
-#pragma unroll
-        for (int u = 0; u < 8; u++) acc += ty[u] == t ? v[u] : (T)0;
+    // 64 elements per workgroup, the rows of the structure in four runs (one per wavefront) whose sums are added in
+    // run order: the chain of dependent loads per row (centre, species, entry) is a quarter as long
+    __shared__ T red[4][64];
+    const int e = blockIdx.x * 64 + (threadIdx.x & 63), part = threadIdx.x >> 6;
+    int t = 0, q = 0;
+    T* out = nullptr;
+    if (e < total) {
+        if (e < n_c) { t = e / ncl; q = e - t * ncl; out = dcoeffs ? dcoeffs + (size_t)b * n_c + e : nullptr; }
+        else if (e < n_c + n_w0) { const int r = e - n_c; t = r / (H * D); q = ncl + r - t * H * D; out = dw0 ? dw0 + (size_t)b * n_w0 + r : nullptr; }
+        else if (e < n_c + n_w0 + n_h) { const int r = e - n_c - n_w0; t = r / H; q = ncl + H * D + r - t * H; out = db0 ? db0 + (size_t)b * n_h + r : nullptr; }
+        else if (e < n_c + n_w0 + 2 * n_h) { const int r = e - n_c - n_w0 - n_h; t = r / H; q = ncl + H * D + H + r - t * H; out = dw1 ? dw1 + (size_t)b * n_h + r : nullptr; }
+        else { t = e - n_c - n_w0 - 2 * n_h; q = a.nrow - 1; out = dbias ? dbias + (size_t)b * nt + t : nullptr; }
     }
-    *out = acc;
+    const int inum = a.binum[b];
+    const int run = ((inum + 3) / 4 + 7) / 8 * 8;
+    const int i_end = min(inum, (part + 1) * run);
+    T acc = (T)0;
+    if (out) {
+        // eight rows in flight; the rows of other species are skipped, the order of the sum is the atom order
+        for (int i0 = part * run; i0 < i_end; i0 += 8) {
+            int c[8], ty[8];
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) c[u] = a.bilist[(size_t)b * a.P + min(i0 + u, i_end - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const bool ok = i0 + u < i_end && (unsigned)c[u] < (unsigned)a.P;
+                ty[u] = a.btypes[(size_t)b * a.P + (ok ? c[u] : 0)];
+                if (!ok) ty[u] = -1;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {        // (a row of another species is not read: its lanes are masked off)
+                v[u] = (T)0;
+                if (ty[u] == t) v[u] = a.gpart[((size_t)b * a.P + min(i0 + u, i_end - 1)) * a.nrow + q];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc += v[u];
+        }
+    }
+    red[part][threadIdx.x & 63] = acc;
+    __syncthreads();
+    if (part == 0 && out) *out = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
 }
 
 inline int efv_call(int K, int n_r, int n_a, int l_max, int H, int ntypes, const float* c, const float* w0,
@@ -449,7 +462,7 @@ int nep_loss(double e_w, double f_w, double v_w, const T* e_dft, const T* f_dft,
     prof_end(stream);
     const int total = ntypes * ntypes * (n_r + n_a) * K + ntypes * H * a.D + 2 * ntypes * H + ntypes;
     prof_begin("nep_grad_reduce", stream);
-    hipLaunchKernelGGL(nep_grad_reduce_kernel<T>, dim3(ceil_div(total, 256), B), dim3(256), 0, stream, a, dcoeffs, dw0,
+    hipLaunchKernelGGL(nep_grad_reduce_kernel<T>, dim3(ceil_div(total, 64), B), dim3(256), 0, stream, a, dcoeffs, dw0,
                        db0, dw1, dbias);
     prof_end(stream);
     A2P_HIP_CHECK(hipGetLastError());

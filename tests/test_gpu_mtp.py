@@ -489,6 +489,24 @@ def test_components_in_one_pass_equal_a_pass_per_column(oracle, level, nt, U):
         assert np.array_equal(a, c)                      # bit-reproducible
 
 
+def test_components_in_single_precision(oracle):
+    """The fp32 instance of the one-pass components against the fp64 one (the plan's byte offsets are halved for
+    4-byte moments)."""
+    import torch
+    from ai2pot_amd import ops
+    m, nb, _ = loss_inputs(oracle, 12, 2, sizes=(30, 24))
+    out = {}
+    for dt in (torch.float64, torch.float32):
+        md = model_to_device(m, dt)
+        d = to_device(nb, dt)
+        out[dt] = [t.double().cpu().numpy() for t in ops.mtp_lin_components(
+            m["chebyshev_size"], m["scaling"], md["coeffs"], m["alpha_moments_count"], md["alpha_index_basic"],
+            md["alpha_index_times"], md["alpha_moment_mapping"], m["nmus"], d["binum"], d["bilist"], d["bnumneigh"],
+            d["bfirstneigh"], d["brcs"], d["btypes"], md["type_map"], m["rmax"], m["rmin"], md["q_scaler"])]
+    for a, b in zip(out[torch.float32], out[torch.float64]):
+        assert close(a, b, 2e-4)
+
+
 def test_components_flag_bad_lists(oracle):
     """The one-pass components check their lists like the energy / force / virial kernel: a neighbour index or a type
     outside its range, or a row longer than umax, is skipped on the device and reported; nothing is read or written
