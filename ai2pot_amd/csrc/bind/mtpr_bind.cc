@@ -107,12 +107,13 @@ struct LossFunction : public torch::autograd::Function<LossFunction> {
         TORCH_CHECK(e_dft.numel() == B && f_dft.numel() == (int64_t)B * P * 3 && v_dft.numel() == (int64_t)B * 9,
                     "label tensors must have shapes [B], [B, P, 3], [B, 9]");
         const bool need = coeffs.requires_grad() || lin.requires_grad() || bias.requires_grad();
-        at::Tensor bloss = at::zeros({B}, opt), rmse = at::zeros({3}, opt), e = at::zeros({B}, opt),
-                   f = at::zeros({B, P, 3}, opt), v = at::zeros({B, 9}, opt), dc, dl, db;
+        // the library writes every element of these outputs when the batch is not empty
+        auto out = [&](at::IntArrayRef shape) { return B > 0 && P > 0 ? at::empty(shape, opt) : at::zeros(shape, opt); };
+        at::Tensor bloss = out({B}), rmse = out({3}), e = out({B}), f = out({B, P, 3}), v = out({B, 9}), dc, dl, db;
         if (need) {
-            dc = at::zeros({B, coeffs.numel()}, opt);
-            dl = at::zeros({B, lin.numel()}, opt);
-            db = at::zeros({B, bias.numel()}, opt);
+            dc = out({B, coeffs.numel()});
+            dl = out({B, lin.numel()});
+            db = out({B, bias.numel()});
         }
         void* st = current_stream(brcs);
         auto call = [&]() -> int {

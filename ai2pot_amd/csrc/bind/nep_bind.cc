@@ -182,14 +182,15 @@ struct NepLossFunction : public torch::autograd::Function<NepLossFunction> {
                     "label tensors must have shapes [B], [B, P, 3], [B, 9]");
         const bool need = coeffs.requires_grad() || w0.requires_grad() || b0.requires_grad() ||
                           w1.requires_grad() || bias.requires_grad();
-        at::Tensor bloss = at::zeros({B}, opt), rmse = at::zeros({3}, opt), e = at::zeros({B}, opt),
-                   f = at::zeros({B, P, 3}, opt), v = at::zeros({B, 9}, opt), dc, dw0, db0, dw1, db;
+        // the library writes every element of these outputs when the batch is not empty
+        auto out = [&](at::IntArrayRef shape) { return B > 0 && P > 0 ? at::empty(shape, opt) : at::zeros(shape, opt); };
+        at::Tensor bloss = out({B}), rmse = out({3}), e = out({B}), f = out({B, P, 3}), v = out({B, 9}), dc, dw0, db0, dw1, db;
         if (need) {
-            dc = at::zeros({B, coeffs.numel()}, opt);
-            dw0 = at::zeros({B, w0.numel()}, opt);
-            db0 = at::zeros({B, b0.numel()}, opt);
-            dw1 = at::zeros({B, w1.numel()}, opt);
-            db = at::zeros({B, bias.numel()}, opt);
+            dc = out({B, coeffs.numel()});
+            dw0 = out({B, w0.numel()});
+            db0 = out({B, b0.numel()});
+            dw1 = out({B, w1.numel()});
+            db = out({B, bias.numel()});
         }
         void* st = current_stream(brcs);
         auto call = [&]() -> int {

@@ -6,6 +6,7 @@ source/fvt/bind/fvt_sr_op_bind.cc).  Tensors are torch tensors on a HIP device; 
 provides memory and the current stream, the compute is the C ABI of libai2pot_hip.so.
 """
 import ctypes
+import os
 
 import torch
 
@@ -20,6 +21,17 @@ def _ptr(t):
 
 def _stream(device):
     return _c.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _new_output(shape, dtype, device, written):
+    """An output tensor of an operator whose library call writes every element (written = the batch is not empty):
+    uninitialised memory, no fill kernel per output per call.  AI2POT_POISON_OUTPUTS=1 fills it with NaN instead, so
+    that an element the library leaves out shows."""
+    if not written:
+        return torch.zeros(shape, dtype=dtype, device=device)
+    if os.environ.get("AI2POT_POISON_OUTPUTS") == "1":
+        return torch.full(shape, float("nan"), dtype=dtype, device=device)
+    return torch.empty(shape, dtype=dtype, device=device)
 
 
 def _req(cond, msg):
@@ -338,7 +350,7 @@ def nep_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
         _req(t.numel() == n_expected, "%s has %d elements, expected %d" % (name, t.numel(), n_expected))
     if validate:
         _validate_batch(binum, bnumneigh, U, P)
-    z = lambda *s_: torch.zeros(s_, dtype=dtype, device=device)
+    z = lambda *s_: _new_output(s_, dtype, device, B * P > 0)
     out = dict(bloss=z(B), rmse=z(3), energy=z(B), force=z(B, P, 3), virial=z(B, 9))
     if want_grad:
         out.update(dcoeffs=z(B, coeffs.numel()), dw0=z(B, w0.numel()), db0=z(B, b0.numel()),
@@ -585,7 +597,7 @@ def mtp_loss_step(e_weight, f_weight, v_weight, betot_dft, bforce_dft, bvirial_d
             n_expected *= s_
         _req(t.numel() == n_expected, "%s must have shape %s" % (name, shape))
     ncoef = coeffs.numel()
-    z = lambda *s: torch.zeros(s, dtype=dtype, device=device)
+    z = lambda *s: _new_output(s, dtype, device, B * P > 0)
     out = dict(bloss=z(B), rmse=z(3), energy=z(B), force=z(B, P, 3), virial=z(B, 9))
     if want_grad:
         out.update(dcoeffs=z(B, ncoef), dlinear=z(B, n_scalar), dbias=z(B, ntypes))
