@@ -56,12 +56,21 @@ __host__ __device__ inline int mtp_adjoint_offset(int max_level_slots)
 {
     return ((max_level_slots > 8 ? max_level_slots : 8) + 1) & ~1;     // at least the scratch of a block sum
 }
-__host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots, int nt)
+// keep (energy / force / virial kernel, when the LDS allows it without costing a workgroup per CU): the adjoints lie
+// behind the table instead of inside it, so that a row of one chunk finds its table still in place in the last pass.
+__host__ __device__ inline int mtp_table_entries(int nc, int E, bool loss, int n_moms, int nt)
 {
     int a = loss ? nc * E + (mtp_gred_in_moments(loss, n_moms) ? 0 : (256 / 32) * 32 * 4) : nc * E;
     if (!loss && a < nt * 4) a = nt * 4;          // four group sums per thread
+    return (a + 1) & ~1;
+}
+__host__ __device__ inline int mtp_table_region(int nc, int E, bool loss, int n_moms, int max_level_slots, int nt,
+                                                bool keep = false)
+{
+    const int a = mtp_table_entries(nc, E, loss, n_moms, nt);
     // loss mode: two partial-sum arrays, then the adjoints and the mixed adjoints
     const int b = loss ? mtp_adjoint_offset(2 * max_level_slots) + 2 * n_moms : mtp_adjoint_offset(max_level_slots) + n_moms;
+    if (keep) return a + n_moms;
     return a > b ? a : b;
 }
 // the dense adjoint array of the pair-derivative pass takes the place of the moments when it fits
@@ -97,6 +106,7 @@ struct MtpArgs {
     int ngrad;
     int lds_basic_off;  // byte offset of the packed basic-moment table in LDS
     int nc_cap;         // rows of the LDS neighbour table: a row is processed in chunks of at most nc_cap
+    int keep_table;     // energy / force / virial kernel: the adjoints lie behind the table (mtp_table_region)
     // site-energy / descriptor mode (linearMtp.h:514-611, 821-890)
     T* e_sites;        // [B, P] per-row energies, or null
     T* desc;           // [B, P, n_scalar] scalar moments, or null
@@ -132,7 +142,7 @@ __device__ __forceinline__ double sqrt_t(double x) { return sqrt(x); }
 template <typename T, bool LOSS, int NT>
 __device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, const T* cf, int lane, int nc, int c0,
                                             const T* rcs, const int* first, const int* types, int center,
-                                            int b, int NF, int* nj_out, bool* valid_out, T* d_out)
+                                            int b, int NF, int* nj_out, bool* valid_out, T* d_out, bool fill = true)
 {
     const int kmax = a.p.kmax, nmus = a.p.nmus, K = a.K;
     const int OG = 3 * (kmax + 1), ODG = OG + nmus, OU = ODG + nmus, OW = OU + 4, OF = OW + 4, ODF = OF + K;
@@ -148,8 +158,8 @@ __device__ __forceinline__ void build_table(const MtpArgs<T>& a, T* tab, const T
         *nj_out = nj;
         *valid_out = !(sqrt_t(x * x + y * y + z * z) > a.rmax);      // mtpBasis.h:457, linearMtp.h:316
     }
-    const int ntask = nc * (nmus + 3);
-    for (int task = lane; task < ntask; task += NT) {
+    const int ntask = fill ? nc * (nmus + 3) : 0;          // fill = false: the table is in place, only the lanes' own
+    for (int task = lane; task < ntask; task += NT) {      // neighbours are returned
         const int role = task / nc, j = task - role * nc;
         const int jj = c0 + j;
         const T x = rcs[jj * 3 + 0], y = rcs[jj * 3 + 1], z = rcs[jj * 3 + 2];
@@ -411,7 +421,8 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     T* cf = Tg + (LOSS ? n_moms : 0);        // coefficients of the centre species: [ntypes][nmus][K]
     T* tab = cf + a.ntypes * nmus * K;
     // the adjoints (loss mode: and the mixed adjoints) share the table's region, behind the sweeps' partial sums
-    T* A = tab + mtp_adjoint_offset((LOSS ? 2 : 1) * p.max_level_slots);
+    const bool keep = !LOSS && a.keep_table != 0;       // uniform over the launch
+    T* A = tab + (keep ? mtp_table_entries(MTP_NC, E, LOSS, n_moms, NT) : mtp_adjoint_offset((LOSS ? 2 : 1) * p.max_level_slots));
     T* Bm = A + n_moms;
     // [256/32][32][4] partial sums of the thread groups.  They are needed only in the last pass over the
     // neighbours, when the moments (and, in loss mode, their tangents) are dead: a long enough moment
@@ -421,7 +432,7 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
     T* gred = LOSS ? (share ? M : tab + MTP_NC * E) : tab;
     // loss mode, behind the region: adjoints and mixed adjoints of the basic moments (copies for the last pass) |
     // P[nc][nmus] | Q[nc][nmus] | ...
-    T* Ab = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots, NT);
+    T* Ab = tab + mtp_table_region(MTP_NC, E, LOSS, n_moms, p.max_level_slots, NT, keep);
     T* Bb = Ab + n_basic;
     T* pq = LOSS ? Bb + n_basic : Ab;
 
@@ -605,7 +616,9 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
             const int h = lane / nc, j = lane - h * nc;
             int nj; bool valid; T d[3] = {(T)0, (T)0, (T)0};
             __syncthreads();
-            build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d);
+            // (a row of one chunk finds the table of the first pass still in place when the adjoints lie behind it)
+            build_table<T, false, NT>(a, tab, cf, lane, nc, c0, rcs, first, types, center, b, NF, &nj, &valid, d,
+                                      !(keep && nchunks == 1));
             __syncthreads();
             T gs = (T)0, wx = (T)0, wy = (T)0, wz = (T)0;
             T ux = (T)0, uy = (T)0, uz = (T)0, rinv = (T)0;
@@ -1643,10 +1656,11 @@ int table_entries(const MtpPlanDevice& p, int K, bool loss)
 }
 
 template <typename T>
-size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC, int nt)
+size_t lds_bytes(const MtpPlanDevice& p, int E, bool loss, int ntypes, int K, int H, int MTP_NC, int nt,
+                 bool keep = false)
 {
     // the neighbour table and the group sums double as the sweeps' partial-sum arrays
-    const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots, nt);
+    const size_t tabs = (size_t)mtp_table_region(MTP_NC, E, loss, p.n_moms, p.max_level_slots, nt, keep);
     size_t n = (size_t)p.n_moms * (loss ? 2 : 1) + tabs + (loss ? 2 * (size_t)p.n_basic : 0) +
                (size_t)ntypes * p.nmus * K;   // + the coefficient copy
     // loss mode: P, Q, the neighbour types and the per-atom coefficient-gradient block
@@ -1678,7 +1692,7 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     a.brcs = brcs; a.btypes = btypes;
     a.cE = nullptr; a.dFs = nullptr; a.dVs = nullptr; a.gpart = nullptr; a.ngrad = 0;
     a.force = nullptr; a.seg_cursor = nullptr; a.seg_g = nullptr; a.seg_spare = 0; a.seg_cap = 0; a.partial = nullptr;
-    a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0; a.no_tangent = 0;
+    a.e_sites = nullptr; a.desc = nullptr; a.energy_only = 0; a.cE_per_atom = 0; a.no_tangent = 0; a.keep_table = 0;
     a.nn_exact = 1;
     a.row_seed = nullptr; a.pair_out = nullptr;
     a.H = 0; a.w0 = nullptr; a.w1 = nullptr; a.q_shift = nullptr;
@@ -1689,12 +1703,18 @@ int fill_args(MtpArgs<T>& a, MtpPlan* plan, int K, double scaling, const T* coef
     return A2P_OK;
 }
 
+int g_keep_table = 1;      // (measurement switch: AI2POT_MTP_KEEP_TABLE=0)
+
 template <typename T, bool LOSS, bool SEED = false>
 int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
 {
+    {
+        static const char* e = getenv("AI2POT_MTP_KEEP_TABLE");
+        if (e) g_keep_table = e[0] != '0';
+    }
     const bool wide = a.p.n_moms >= (LOSS ? 300 : 1000);   // enough work per atom to keep 256 threads busy
-    auto lds_for = [&](int nc, size_t* main) {
-        *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc, wide ? 256 : 64) + 15) / 16 * 16;
+    auto lds_for = [&](int nc, size_t* main, bool keep = false) {
+        *main = (lds_bytes<T>(a.p, a.E, LOSS, a.ntypes, a.K, a.H, nc, wide ? 256 : 64, keep) + 15) / 16 * 16;
         // the packed basic-moment table; energy / force / virial kernel: + the monomial rows
         return *main + (LOSS ? (size_t)a.p.n_basic : (size_t)a.p.n_basic + a.p.nrows) * sizeof(unsigned);
     };
@@ -1716,6 +1736,17 @@ int launch_atoms(const MtpArgs<T>& a, hipStream_t stream)
             const size_t l = lds_for(nc, &m);
             if (per_cu(l) >= want || nc == MTP_NC_MIN) { nc_cap = nc; lds = l; lds_main = m; break; }
         }
+        // The table kept through the sweeps (adjoints behind it) saves a row of one chunk its second table build: taken
+        // when a table of at least 32 rows fits that way at the same number of workgroups per CU (level 20: 0.387 ->
+        // 0.368 ms, level 10: 0.026 -> 0.023 ms; at level 16 the sixteen workgroups per CU count for more).  Not in the
+        // modes that use the table's place as scratch between the sweeps (site energies, descriptors).
+        int keep = 0;
+        if (!a.e_sites && !a.desc && !a.energy_only && g_keep_table)
+            for (int nc : {MTP_NC_MAX, 40, 32}) {
+                const size_t l = lds_for(nc, &m, true);
+                if (per_cu(l) >= want) { keep = 1; nc_cap = nc; lds = l; lds_main = m; break; }
+            }
+        const_cast<MtpArgs<T>&>(a).keep_table = keep;
     }
     const_cast<MtpArgs<T>&>(a).lds_basic_off = (int)lds_main;
     const_cast<MtpArgs<T>&>(a).nc_cap = nc_cap;
