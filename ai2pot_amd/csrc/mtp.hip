@@ -669,9 +669,10 @@ __global__ void __launch_bounds__(NT, (!LOSS ? 4 : 1)) mtp_atom_kernel(const Mtp
                 vir[6] -= gz * d[0]; vir[7] -= gz * d[1]; vir[8] -= gz * d[2];
             }
         }
-        // only the threads of group 0 (inside wave 0) hold force and virial terms
+        // only the threads of group 0 (inside wave 0) hold force and virial terms: the other wavefronts are done
+        const double e_atom = (double)block_sum<T, NT>(e_part, gred, lane);
+        if (lane >= 64) return;
         fx = wave_sum(fx); fy = wave_sum(fy); fz = wave_sum(fz);
-        double e_atom = (double)block_sum<T, NT>(e_part, gred, lane);
         double out[10];
         out[0] = e_atom + (seeded ? 0.0 : (double)a.bias[ti]);
 #pragma unroll
