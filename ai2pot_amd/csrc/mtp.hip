@@ -252,8 +252,8 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
 {
     for (int l = 0; l < p.n_levels; l++) {
         const int s0 = p.f_level[l], s1 = p.f_level[l + 1];     // whole groups of 64 slots: every lane of a wave walks one
-        const int steps = p.f_multi[l];
         for (int s = s0 + tid; s < s1; s += NT) {
+            const int steps = p.f_multi[s >> 6];             // of the group: only groups with cut lists pay for the sums
             const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group, a multiple of 4
             const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
             const int dst = p.f_dst[s];                      // requested with the two words above
@@ -300,8 +300,8 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
 {
     for (int l = p.n_levels - 1; l >= 0; l--) {
         const int s0 = p.r_level[l], s1 = p.r_level[l + 1];
-        const int steps = p.r_multi[l];
         for (int s = s0 + tid; s < s1; s += NT) {
+            const int steps = p.r_multi[s >> 6];
             const int depth = p.r_gdepth[s >> 6];
             const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
             const int src = p.r_src[s];
@@ -1341,13 +1341,17 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
                 for (int q = 0; q < np; q++)
                     pieces.push_back({m, q * MTP_SLOT_CAP, std::min(MTP_SLOT_CAP, n - q * MTP_SLOT_CAP), np - 1 - q});
             }
-            int steps = 0;
-            while ((1 << steps) < most) steps++;
-            e.multi.push_back(steps);
+            (void)most;
             for (size_t g0 = 0; g0 < pieces.size(); g0 += 64) {
                 const size_t g1 = std::min(pieces.size(), g0 + 64);
-                int depth = 0;
-                for (size_t q = g0; q < g1; q++) depth = std::max(depth, pieces[q].n);
+                int depth = 0, longest = 1;
+                for (size_t q = g0; q < g1; q++) {
+                    depth = std::max(depth, pieces[q].n);
+                    longest = std::max(longest, pieces[q].rem + 1);
+                }
+                int steps = 0;                      // doubling steps that add up the pieces of this group's lists
+                while ((1 << steps) < longest) steps++;
+                e.multi.push_back(steps);
                 depth = (depth + 3) / 4 * 4;        // the kernels fetch four terms at a time
                 e.gbase.push_back((int)e.terms.size());
                 e.gdepth.push_back(depth);
@@ -1366,9 +1370,8 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
         }
         e.level.push_back((int)e.slot.size());
         e.lend.push_back((int)e.slot.size());
-        e.multi.push_back(0);
         if (e.terms.empty()) e.terms.push_back(make_int2(0, 0));
-        if (e.gbase.empty()) { e.gbase.push_back(0); e.gdepth.push_back(0); }
+        if (e.gbase.empty()) { e.gbase.push_back(0); e.gdepth.push_back(0); e.multi.push_back(0); }
         if (e.slot.empty()) { e.slot.push_back(-1); e.lead.push_back(0); }
         return e;
     };

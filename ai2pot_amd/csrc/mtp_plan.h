@@ -31,7 +31,7 @@ struct MtpPlanDevice {
     // forward gather.  A slot holds up to MTP_SLOT_CAP terms of one destination moment; a longer
     // list is cut into consecutive slots (pieces), so that no lane walks a long list alone; the pieces of a
     // list lie in one group of 64 slots and the wavefront that walks the group adds their partial sums with
-    // shuffles (f_multi[l] doubling steps).  Slots are grouped 64 at a time; level l covers slots
+    // shuffles (f_multi[group] doubling steps: lists are sorted by length, so only a level's first groups hold cut lists).  Slots are grouped 64 at a time; level l covers slots
     // [f_level[l], f_level[l+1]) (whole groups; [f_level[l], f_lend[l]) without the padding slots).  The terms of a group are stored
     // interleaved and padded with zero terms to the group's depth (a multiple of four): term k of slot s is
     // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
@@ -39,7 +39,7 @@ struct MtpPlanDevice {
     // into an array of doubles), y = multiplicity.
     const int* f_level;        // [n_levels+1]
     const int* f_lend;         // [n_levels+1]
-    const int* f_multi;        // [n_levels]   doubling steps that add up the longest list's pieces (0: no list is cut)
+    const int* f_multi;        // [n_fslots/64] doubling steps that add up the pieces of the group's longest list (0: none is cut)
     const int* f_dst;          // [n_fslots]   destination in the first piece of a list (-1 elsewhere and in padding)
     const int* f_rem;          // [n_fslots]   pieces of the same list behind this one
     const int* f_gbase;        // [n_fslots/64]
@@ -49,7 +49,7 @@ struct MtpPlanDevice {
     // processed from the last level to level 0; a term packs x = 8 dst | 8 other << 16, y = mult
     const int* r_level;        // [n_levels+1]
     const int* r_lend;         // [n_levels+1]
-    const int* r_multi;        // [n_levels]
+    const int* r_multi;        // [n_rslots/64]
     const int* r_src;          // [n_rslots]
     const int* r_rem;          // [n_rslots]
     const int* r_gbase;        // [n_rslots/64]
@@ -84,7 +84,7 @@ struct MtpPlanDevice {
     const int* x_seed;         // [x_slots]  scalar moment, in the slot of its list's first piece; -1 elsewhere
     const int* x_brem;         // [x_slots]  pieces of the same list behind this one
     const int* x_level;        // [n_levels+1]
-    const int* x_multi;        // [n_levels]
+    const int* x_multi;        // [n_xslots/64]
     const int* x_src;          // [n_xslots]
     const int* x_rem;          // [n_xslots]
     const int* x_gbase;        // [n_xslots/64]
