@@ -253,9 +253,10 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
     for (int l = 0; l < p.n_levels; l++) {
         const int s0 = p.f_level[l], s1 = p.f_level[l + 1];     // whole groups of 64 slots: every lane of a wave walks one
         for (int s = s0 + tid; s < s1; s += NT) {
-            const int steps = p.f_multi[s >> 6];             // of the group: only groups with cut lists pay for the sums
-            const int depth = p.f_gdepth[s >> 6];            // shared by the 64 lanes of the group, a multiple of 4
-            const int2* tp = p.f_terms + p.f_gbase[s >> 6] + (s & 63);
+            const int grp = __builtin_amdgcn_readfirstlane(s >> 6);     // the wavefront's group: scalar loads below
+            const int steps = p.f_multi[grp];                // of the group: only groups with cut lists pay for the sums
+            const int depth = p.f_gdepth[grp];               // shared by the 64 lanes of the group, a multiple of 4
+            const int2* tp = p.f_terms + p.f_gbase[grp] + (s & 63);
             const int dst = p.f_dst[s];                      // requested with the two words above
             const int rem = steps ? p.f_rem[s] : 0;
             T acc = (T)0, tacc = (T)0;
@@ -301,9 +302,10 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
     for (int l = p.n_levels - 1; l >= 0; l--) {
         const int s0 = p.r_level[l], s1 = p.r_level[l + 1];
         for (int s = s0 + tid; s < s1; s += NT) {
-            const int steps = p.r_multi[s >> 6];
-            const int depth = p.r_gdepth[s >> 6];
-            const int2* tp = p.r_terms + p.r_gbase[s >> 6] + (s & 63);
+            const int grp = __builtin_amdgcn_readfirstlane(s >> 6);
+            const int steps = p.r_multi[grp];
+            const int depth = p.r_gdepth[grp];
+            const int2* tp = p.r_terms + p.r_gbase[grp] + (s & 63);
             const int src = p.r_src[s];
             const int rem = steps ? p.r_rem[s] : 0;
             T acc = (T)0;
