@@ -255,7 +255,7 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
         for (int s = s0 + tid; s < s1; s += NT) {
             const int grp = __builtin_amdgcn_readfirstlane(s >> 6);     // the wavefront's group: scalar loads below
             const int steps = p.f_multi[grp];                // of the group: only groups with cut lists pay for the sums
-            const int depth = p.f_gdepth[grp];               // shared by the 64 lanes of the group, a multiple of 4
+            const int depth = p.f_gdepth[grp];               // shared by the 64 lanes of the group, a multiple of MTP_DEPTH_STEP
             const int2* tp = p.f_terms + p.f_gbase[grp] + (s & 63);
             const int dst = p.f_dst[s];                      // requested with the two words above
             const int rem = steps ? p.f_rem[s] : 0;
@@ -264,16 +264,16 @@ __device__ __forceinline__ void sweep_forward(const MtpPlanDevice& p, T* M, T* T
             // before the first is used: one trip to memory per slot
             int2 w[MTP_SLOT_CAP];
 #pragma unroll
-            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+            for (int k = 0; k < MTP_SLOT_CAP; k += MTP_DEPTH_STEP)
                 if (k < depth) {
 #pragma unroll
-                    for (int u = 0; u < 4; u++) w[k + u] = tp[(k + u) * 64];
+                    for (int u = 0; u < MTP_DEPTH_STEP; u++) w[k + u] = tp[(k + u) * 64];
                 }
 #pragma unroll
-            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+            for (int k = 0; k < MTP_SLOT_CAP; k += MTP_DEPTH_STEP)
                 if (k < depth) {
 #pragma unroll
-                    for (int u = k; u < k + 4; u++) {
+                    for (int u = k; u < k + MTP_DEPTH_STEP; u++) {
                         const unsigned m0 = (unsigned)w[u].x & 0xffffu, m1 = (unsigned)w[u].x >> 16;
                         const T mult = (T)w[u].y;
                         const T v0 = plan_entry(M, m0), v1 = plan_entry(M, m1);
@@ -311,16 +311,16 @@ __device__ __forceinline__ void sweep_reverse(const MtpPlanDevice& p, const T* M
             T acc = (T)0;
             int2 w[MTP_SLOT_CAP];
 #pragma unroll
-            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+            for (int k = 0; k < MTP_SLOT_CAP; k += MTP_DEPTH_STEP)
                 if (k < depth) {
 #pragma unroll
-                    for (int u = 0; u < 4; u++) w[k + u] = tp[(k + u) * 64];
+                    for (int u = 0; u < MTP_DEPTH_STEP; u++) w[k + u] = tp[(k + u) * 64];
                 }
 #pragma unroll
-            for (int k = 0; k < MTP_SLOT_CAP; k += 4)
+            for (int k = 0; k < MTP_SLOT_CAP; k += MTP_DEPTH_STEP)
                 if (k < depth) {
 #pragma unroll
-                    for (int u = k; u < k + 4; u++) {
+                    for (int u = k; u < k + MTP_DEPTH_STEP; u++) {
                         const unsigned dst = (unsigned)w[u].x & 0xffffu, other = (unsigned)w[u].x >> 16;
                         const T mult = (T)w[u].y;
                         acc += plan_entry(X, dst) * mult * plan_entry(M, other);
@@ -1354,7 +1354,7 @@ int plan_create(int n_moms, int n_basic, const int* basic, int n_times, const in
                 int steps = 0;                      // doubling steps that add up the pieces of this group's lists
                 while ((1 << steps) < longest) steps++;
                 e.multi.push_back(steps);
-                depth = (depth + 3) / 4 * 4;        // the kernels fetch four terms at a time
+                depth = (depth + MTP_DEPTH_STEP - 1) / MTP_DEPTH_STEP * MTP_DEPTH_STEP;    // the sweeps fetch that many terms at a time
                 e.gbase.push_back((int)e.terms.size());
                 e.gdepth.push_back(depth);
                 e.terms.resize(e.terms.size() + (size_t)depth * 64, make_int2(0, 0));

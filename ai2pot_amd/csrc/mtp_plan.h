@@ -19,6 +19,8 @@
 namespace a2p {
 
 constexpr int MTP_SLOT_CAP = 16;
+// The sweeps fetch the words of a slot MTP_DEPTH_STEP at a time; the depth of a group of slots is a multiple of it.
+constexpr int MTP_DEPTH_STEP = 2;
 
 struct MtpPlanDevice {
     // sizes
@@ -33,7 +35,7 @@ struct MtpPlanDevice {
     // list lie in one group of 64 slots and the wavefront that walks the group adds their partial sums with
     // shuffles (f_multi[group] doubling steps: lists are sorted by length, so only a level's first groups hold cut lists).  Slots are grouped 64 at a time; level l covers slots
     // [f_level[l], f_level[l+1]) (whole groups; [f_level[l], f_lend[l]) without the padding slots).  The terms of a group are stored
-    // interleaved and padded with zero terms to the group's depth (a multiple of four): term k of slot s is
+    // interleaved and padded with zero terms to the group's depth (a multiple of MTP_DEPTH_STEP): term k of slot s is
     // f_terms[f_gbase[s >> 6] + k * 64 + (s & 63)], k < f_gdepth[s >> 6], so the 64 lanes that walk
     // a group read consecutive words and share the trip count.  A term packs x = 8 m0 | 8 m1 << 16 (byte offsets
     // into an array of doubles), y = multiplicity.
