@@ -138,3 +138,82 @@ def test_staged_rows_never_load_past_the_arrays():
                         pr = row * U + (slot if have else 0)
                         assert 0 <= pr < B * P * U
                         assert row // P == b                            # never another structure's row
+
+
+# Positional argument types of the operators the reference registers (i = int, f = float, T = Tensor, s = str), read
+# off its TORCH_LIBRARY blocks; the number is the line of the m.def in
+# source/descriptor/{nep,mtpr,nnmtp}/bind/*_bind.cc and source/fvt/bind/fvt_sr_op_bind.cc.
+REFERENCE_SCHEMAS = {
+    ("nep", "nepToEFOp"): ("iiiiTTTTTTTTTTTTiffTffTT", 25),
+    ("nep", "nepToEFVOp"): ("iiiiTTTTTTTTTTTTiffTffTT", 80),
+    ("nep", "nepToEFLossOp"): ("ffTTiiiiTTTTTTTTTTTTiffTffTT", 135),
+    ("nep", "nepToLossOp"): ("fffTTTiiiiTTTTTTTTTTTTiffTffTT", 204),
+    ("nep", "nepToDescriptorsOp"): ("iiiiTTTTTTTTiff", 277),
+    ("mtpr", "set_ai2pot_path"): ("s", 31),
+    ("mtpr", "CoeffsSchmidtOrthOp"): ("iiiT", 38),
+    ("mtpr", "LinMatrixLinVectorOp"): ("fffTTTifTTTiTTTiTTTTTTTiffTffTT", 57),
+    ("mtpr", "mtpParamOp"): ("i", 131),
+    ("mtpr", "mtpBasisOp"): ("TTTTTTiifTTTTTTTiff", 140),
+    ("mtpr", "linearMtpToLossOp"): ("fffTTTifTTTiTTTiTTTTTTTiffTffTT", 189),
+    ("mtpr", "linearMtpToEFLossOp"): ("ffTTifTTTiTTTiTTTTTTTiffTffTT", 263),
+    ("mtpr", "linearMtpToEFVOp"): ("ifTTTiTTTiTTTTTTTiffTffTT", 333),
+    ("mtpr", "linearMtpToEFOp"): ("ifTTTiTTTiTTTTTTTiffTffTT", 396),
+    ("mtpr", "linearMtpToEsitesOp"): ("ifTTTiTTTiTTTTTTTiffTffTT", 459),
+    ("mtpr", "linearMtpToDescriptorsOp"): ("ifTiTTTiTTTTTTTiff", 521),
+    ("nnmtp", "set_ai2pot_path"): ("s", 27),
+    ("nnmtp", "mtpParamOp"): ("i", 34),
+    ("nnmtp", "nnMtpToEFLossOp"): ("ffTTiTTTTiTTTiTTTTTTTiffTTffTT", 43),
+    ("nnmtp", "nnMtpToLossOp"): ("fffTTTiTTTTiTTTiTTTTTTTiffTTffTT", 116),
+    ("nnmtp", "nnMtpToEFOp"): ("iTTTTiTTTiTTTTTTTiffTTffTT", 193),
+    ("nnmtp", "nnMtpToEFVOp"): ("iTTTTiTTTiTTTTTTTiffTTffTT", 258),
+    ("nnmtp", "nnMtpToDescriptorsOp"): ("iTiTTTiTTTTTTTiff", 323),
+    ("nnmtp", "nnMtpToEsitesOp"): ("iTTTTiTTTiTTTTTTTiffTTffTT", 370),
+    ("fvt", "ForceSrOp"): ("TTTTiiT", 10),
+    ("fvt", "VirialSrOp"): ("TTiT", 32),
+}
+
+
+def test_bind_libraries_register_the_reference_operators():
+    """The operator libraries load without a GPU and register every operator of the reference under its name with
+    its positional argument types (what TorchScript-exported models and ai2pot/fromcc bind to)."""
+    import glob
+    import torch
+    import ai2pot_amd
+    libdir = os.path.join(os.path.dirname(os.path.abspath(ai2pot_amd.__file__)), "_lib")
+    libs = sorted(glob.glob(os.path.join(libdir, "lib*_bind.so")))
+    assert {os.path.basename(p) for p in libs} >= {"libnep_bind.so", "libmtpr_bind.so", "libnnmtp_bind.so",
+                                                   "libfvt_sr_op_bind.so", "libnblist_bind.so"}
+    for p in libs:
+        torch.ops.load_library(p)
+    code = {"int": "i", "float": "f", "Tensor": "T", "str": "s", "Optional[Tensor]": "T"}
+    for (ns, name), (want, _) in REFERENCE_SCHEMAS.items():
+        op = getattr(getattr(torch.ops, ns), name)
+        schema = op.default._schema
+        got = "".join(code.get(str(a.type), "?") for a in schema.arguments)
+        assert got == want, (ns, name, got, want)
+
+
+def test_nblist_module_checks_its_arguments_like_the_reference():
+    """The CPython module `nblist` (source/nblist/bind/nblist_bind.cc:46-69): eight positional arguments, a
+    TypeError for an argument of the wrong kind, raised before any device work."""
+    import importlib
+    import sys
+    import ai2pot_amd
+    libdir = os.path.join(os.path.dirname(os.path.abspath(ai2pot_amd.__file__)), "_lib")
+    sys.path.insert(0, libdir)
+    try:
+        mod = importlib.import_module("nblist")
+    finally:
+        sys.path.remove(libdir)
+    assert hasattr(mod, "find_info4mlff")
+    lat = np.eye(3) * 10.0
+    ty = np.zeros(2, np.int32)
+    pos = np.zeros((2, 3))
+    good = [lat, ty, pos, 5.0, 20, True, [True, True, True], False]
+    for i, bad in [(0, [1.0]), (1, [0, 0]), (2, "x"), (3, 5), (4, 20.0), (5, 1), (6, (True, True, True)), (7, 0)]:
+        args = list(good)
+        args[i] = bad
+        with pytest.raises(TypeError):
+            mod.find_info4mlff(*args)
+    with pytest.raises(TypeError):
+        mod.find_info4mlff(*good[:7])
