@@ -200,7 +200,11 @@ def _zbl_esites(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, b
 def _zbl_add(zbl_rmax, zbl_rmin, zbl_cks, zbl_dks, type_map, binum, bilist, bnumneigh, bfirstneigh, brcs, btypes,
              nghost, etot, force, virial, validate):
     """Adds the ZBL pair repulsion onto a model's E/F/V when zbl_rmax > 0, as the reference's
-    operators do on the device (correction/gpu/include/zbl.cuh:422-620; e.g. nepOp.cc:1086-1110)."""
+    operators do on the device (correction/gpu/include/zbl.cuh:422-620; e.g. nepOp.cc:1086-1110).
+    The pair formulas are pinned to the reference's PairZBL member functions; the composition per centre
+    atom (halves of the pair energy, force on the centre only) is PARITY UNPINNED by a run of the reference:
+    its CPU GroupZBL::correct_efv has the force and virial calls commented out, so only the device source
+    can be followed."""
     if float(zbl_rmax) == 0.0:
         return
     dtype, device = brcs.dtype, brcs.device

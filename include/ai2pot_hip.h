@@ -465,6 +465,9 @@ int a2p_nep_efv_manybody_f64(int chebyshev_size, int n_radial, int n_angular, in
  * the centre atom only (a full list supplies the other half; ghosts receive nothing), and
  * -0.5 r_a dE_pair/dr r_b / r to the virial.  zbl_cks / zbl_dks: [ntypes, ntypes, 4] (device);
  * type_map: atomic numbers [ntypes] (device int32).
+ * Parity: the pair formulas equal the reference's PairZBL member functions; the composition per centre atom
+ * follows the reference's device source only (its CPU correct_efv has the force and virial calls commented
+ * out): PARITY UNPINNED by a run of the reference.
  * ------------------------------------------------------------------------------------------ */
 int a2p_zbl_correct_f64(double zbl_rmax, double zbl_rmin, const double* zbl_cks, const double* zbl_dks, int ntypes,
                         const int* type_map, int batch, int natoms_pad, int umax, int nghost, const int* binum,
