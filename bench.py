@@ -741,7 +741,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
-                 "(no collectives or sharding in this round)" % args.gpus)
+                 "(the path has no collectives or sharding)" % args.gpus)
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
